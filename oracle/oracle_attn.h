@@ -1,0 +1,150 @@
+/*
+ * CPU oracle for the KV-cache attention path of metallic-foundry.
+ *
+ * THIS IS TEST INFRASTRUCTURE, NOT PRODUCT CODE. It restates the reference's
+ * arithmetic (Metal kernels + Rust host helpers) in scalar C so the HIP library
+ * can be checked against it. Only the test-suite, the smoke check and the
+ * benchmark's cpu_baseline leg may link or load it.
+ *
+ * All tensors are IEEE binary16 stored as uint16_t; all arithmetic is f32 with
+ * round-to-nearest-even conversions, no FMA contraction (build with
+ * -ffp-contract=off).
+ *
+ * Citations are paths under /root/reference/crates/metallic-foundry/.
+ *
+ * Parity status per function (what pins it is listed in tests/test_oracle_*.py):
+ *   orc_f16_*                 pinned: exhaustive against numpy.float16
+ *   orc_rope_tables           pinned: closed forms + float64 library cos/sin
+ *   orc_rope_neox             pinned: transcription of tests/rope.rs:31-63 + rotation invariants
+ *   orc_kv_prep_fused (neox)  pinned: equals legacy chain (tests/kv_prep_fused.rs contract)
+ *   orc_kv_prep_fused (normal pairing, NoPE-layer rule)
+ *                             PARITY UNPINNED by any reference test (source only,
+ *                             src/metals/kv_prep/kv_prep_fused.metal:57,66-73); pinned here only by
+ *                             invariants (de-interleave permutation identity, NoPE == plain copy)
+ *   orc_kv_rearrange / orc_kv_cache_write* / orc_kv_cache_read / orc_repeat_kv_heads
+ *                             pinned: brute-force index maps of the reference's CPU helpers
+ *   orc_sdpa_decode / orc_sdpa_prefill (MHA)
+ *                             pinned: closed-form known-answer inputs of tests/sdpa_oob_repro.rs and
+ *                             tests/sdpa_head_stride_misaligned.rs against float64 library softmax
+ *   GQA head map in orc_sdpa_* PARITY UNPINNED by any reference numeric test (source only,
+ *                             flash_decode.metal:129-132); pinned by GQA == MHA on repeat_kv_heads-expanded K/V
+ *   orc_splitk_merge          pinned: independence of split count, brute force
+ *   orc_paged_*               no reference counterpart; pinned by gather(paged) == contiguous
+ *   orc_sage_*                PARITY UNPINNED: the reference holds only a prose sketch (docs/SAGE.md);
+ *                             pinned by softmax shift identity and error vs f16 SDPA
+ */
+#ifndef ORACLE_ATTN_H
+#define ORACLE_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint16_t orc_f16;
+
+/* KvPrepFusedParams, 13 x u32 in the reference's field order (src/metals/kv_prep/mod.rs:79-114). */
+typedef struct {
+    uint32_t d_model, kv_dim, head_dim, n_heads, n_kv_heads, group_size, seq_len, position_offset,
+        max_seq_len, total_elements, rope_mode /*0 neox, 1 normal*/, layer_idx, no_rope_layer_step;
+} orc_kv_prep_params;
+
+float orc_f16_to_f32(orc_f16 h);
+orc_f16 orc_f32_to_f16(float f);
+void orc_f16_to_f32_n(const orc_f16 *src, float *dst, size_t n);
+void orc_f32_to_f16_n(const float *src, orc_f16 *dst, size_t n);
+
+/* src/model/executor.rs:1981-2006 */
+void orc_rope_tables(float rope_base, uint32_t head_dim, uint32_t pos_begin, uint32_t pos_end,
+                     const float *freq_factors /*nullable, head_dim/2*/, orc_f16 *cos_out, orc_f16 *sin_out);
+
+/* src/metals/rope/rope.metal:28-75 == tests/rope.rs:31-63 */
+void orc_rope_neox(const orc_f16 *input, orc_f16 *output, const orc_f16 *cos_t, const orc_f16 *sin_t,
+                   uint32_t dim, uint32_t seq_len, uint32_t position_offset, size_t total_elements);
+
+/* src/metals/kv_rearrange/kv_rearrange.metal:10-47 */
+void orc_kv_rearrange(const orc_f16 *input, orc_f16 *output, uint32_t kv_dim, uint32_t row_stride,
+                      uint32_t kv_head_dim, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                      uint32_t seq, size_t total_elements);
+
+/* src/metals/kv_cache_write/kv_cache_write.metal:6-30 == tests/kv_cache.rs:14-32 */
+void orc_kv_cache_write(orc_f16 *cache, const orc_f16 *input, uint32_t n_kv_heads, uint32_t head_dim,
+                        uint32_t input_seq_len, uint32_t position_offset, uint32_t max_seq_len);
+/* src/metals/kv_cache_write/kv_cache_write_repeat.metal:9-40 */
+void orc_kv_cache_write_repeat(orc_f16 *cache, const orc_f16 *input, uint32_t n_kv_heads, uint32_t n_heads,
+                               uint32_t group_size, uint32_t head_dim, uint32_t input_seq_len,
+                               uint32_t position_offset, uint32_t max_seq_len);
+/* src/metals/kv_cache_write/kv_cache_read.metal:7-29 == tests/kv_cache.rs:34-46 */
+void orc_kv_cache_read(const orc_f16 *cache, orc_f16 *out, uint32_t n_kv_heads, uint32_t head_dim,
+                       uint32_t seq_len, uint32_t max_seq_len);
+/* src/metals/repeat_kv_heads/repeat_kv_heads.metal:11-44 */
+void orc_repeat_kv_heads(const orc_f16 *input, orc_f16 *output, uint32_t group_size, uint32_t batch,
+                         uint32_t n_kv_heads, uint32_t n_heads, uint32_t seq, uint32_t head_dim,
+                         uint32_t cache_stride);
+
+/* src/metals/kv_prep/kv_prep_fused.metal:26-123 */
+void orc_kv_prep_fused(const orc_f16 *q_in, const orc_f16 *k_in, const orc_f16 *v_in, orc_f16 *q_rot,
+                       orc_f16 *k_cache, orc_f16 *v_cache, const orc_f16 *cos_t, const orc_f16 *sin_t,
+                       const orc_kv_prep_params *p);
+
+/* Decode SDPA, M = 1, blockwise online softmax (src/metals/flashattention/flash_decode.metal:107-144,324-490).
+ * q: [n_heads, head_dim]; k, v: [n_kv_heads, capacity, head_dim]; out: [n_heads * head_dim].
+ * block_keys = WARPS * KEYS_PER_WARP of the emulated variant (any value >= 1 gives the same result up to
+ * f32 rounding). tg_out_half != 0 rounds the per-warp partial outputs to f16 as the reference's
+ * TG_OUT_HALF variants do (flash_decode.metal:431), with `warps` partial sums per block. */
+void orc_sdpa_decode(const orc_f16 *q, const orc_f16 *k, const orc_f16 *v, orc_f16 *out, uint32_t n_heads,
+                     uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t kv_len, float scale,
+                     uint32_t block_keys, uint32_t warps, int tg_out_half, int n_threads);
+
+/* Prefill SDPA, M >= 1 (src/metals/flashattention/flash_prefill.metal:93-446, 985-1021): 32-key tiles,
+ * causal limit = row + query_offset, finalise with inv_l = 0 when l is not finite or <= 1e-6.
+ * Element strides as in SdpaPrefillParams (src/metals/flashattention/stages.rs:240-275); batch = 1.
+ * causal == 0 disables the mask (the reference routes that case to its materialized path,
+ * src/metals/sdpa/step.rs:442-447; the arithmetic definition is the same softmax(QK^T)V). */
+void orc_sdpa_prefill(const orc_f16 *q, const orc_f16 *k, const orc_f16 *v, orc_f16 *out, uint32_t n_heads,
+                      uint32_t group_size, uint32_t head_dim, uint32_t q_len, uint32_t kv_len,
+                      uint32_t query_offset, int causal, float scale, uint64_t q_stride_h, uint64_t q_stride_m,
+                      uint64_t k_stride_h, uint64_t stride_k_s, uint64_t v_stride_h, uint64_t stride_v_s,
+                      uint64_t out_stride_h, uint64_t out_stride_m, uint32_t tile_keys, int n_threads);
+
+/* Split-K partial pass + merge (flash_prefill.metal:452-457, 592-617, 843-888) for one query row of one head.
+ * Writes un-normalised acc[split][head_dim], m[split], l[split]. */
+void orc_sdpa_row_partials(const orc_f16 *q_row, const orc_f16 *k_head, const orc_f16 *v_head, uint32_t head_dim,
+                           uint64_t stride_k_s, uint64_t stride_v_s, uint32_t kv_len, uint32_t causal_limit,
+                           float scale, uint32_t split_k, uint32_t tile_keys, float *acc, float *m, float *l);
+void orc_splitk_merge(const float *acc, const float *m, const float *l, uint32_t split_k, uint32_t head_dim,
+                      orc_f16 *out_row);
+
+/* Paged cache (no reference counterpart). Pool layout [n_blocks, n_kv_heads, block_size, head_dim];
+ * logical row `pos` of a sequence lives in physical block block_table[pos / block_size], slot pos % block_size. */
+void orc_paged_gather(const orc_f16 *pool, const int32_t *block_table, uint32_t n_kv_heads, uint32_t block_size,
+                      uint32_t head_dim, uint32_t seq_len, uint32_t out_capacity, orc_f16 *out /*[n_kv_heads,out_capacity,head_dim]*/);
+void orc_paged_scatter(orc_f16 *pool, const int32_t *block_table, uint32_t n_kv_heads, uint32_t block_size,
+                       uint32_t head_dim, uint32_t pos_begin, uint32_t pos_end, uint32_t in_capacity,
+                       const orc_f16 *in /*[n_kv_heads,in_capacity,head_dim]*/);
+
+/* Sage-style int8 Q/K (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170).
+ * K smoothing: subtract per-(head, channel) mean over the sequence (f32), quantise per block of
+ * `block` tokens with scale = max|.|/127 stored as f16; Q quantised per head with one f32 scale. */
+void orc_sage_k_mean(const orc_f16 *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim, uint32_t kv_len,
+                     float *mean /*[n_kv_heads, head_dim]*/);
+void orc_sage_quantize_k(const orc_f16 *k, const float *mean, uint32_t n_kv_heads, uint32_t capacity,
+                         uint32_t head_dim, uint32_t kv_len, uint32_t block, int8_t *k_q /*[n_kv_heads,capacity,head_dim]*/,
+                         orc_f16 *k_scale /*[n_kv_heads, ceil(capacity/block)]*/);
+void orc_sage_quantize_q(const orc_f16 *q, uint32_t n_heads, uint32_t head_dim, int8_t *q_q, float *q_scale);
+void orc_sage_decode(const int8_t *q_q, const float *q_scale, const int8_t *k_q, const orc_f16 *k_scale,
+                     const orc_f16 *v, orc_f16 *out, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                     uint32_t capacity, uint32_t kv_len, uint32_t block, float scale, int n_threads);
+
+/* LCG of the reference's attention tests (tests/flashattention_decode_parity.rs:15-30):
+ * state = state*1664525 + 1013904223; u = (state >> 9) / 2^23; value = f16((2u-1)*scale). */
+void orc_lcg_fill_f16(uint32_t *state, orc_f16 *dst, size_t n, float scale);
+
+int orc_max_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,263 @@
+"""ctypes loader for the CPU oracle (oracle/liboracle_attn.so). Test infrastructure only.
+
+The oracle takes IEEE binary16 tensors as uint16 buffers; the wrappers here accept and return
+numpy float16 arrays.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_ORACLE_DIR = os.path.join(_ROOT, "oracle")
+_SO = os.path.join(_ORACLE_DIR, "liboracle_attn.so")
+
+u16p = C.POINTER(C.c_uint16)
+f32p = C.POINTER(C.c_float)
+i8p = C.POINTER(C.c_int8)
+i32p = C.POINTER(C.c_int32)
+
+
+class KvPrepParams(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in (
+        "d_model", "kv_dim", "head_dim", "n_heads", "n_kv_heads", "group_size", "seq_len", "position_offset",
+        "max_seq_len", "total_elements", "rope_mode", "layer_idx", "no_rope_layer_step")]
+
+
+def build():
+    subprocess.check_call(["make", "-s", "-C", _ORACLE_DIR, "liboracle_attn.so"])
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = C.CDLL(_SO)
+        L.orc_f16_to_f32.restype = C.c_float
+        L.orc_f16_to_f32.argtypes = [C.c_uint16]
+        L.orc_f32_to_f16.restype = C.c_uint16
+        L.orc_f32_to_f16.argtypes = [C.c_float]
+        L.orc_max_threads.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def _p(a, t):
+    return a.ctypes.data_as(t)
+
+
+def _h(a):
+    a = np.ascontiguousarray(a)
+    assert a.dtype == np.float16, a.dtype
+    return a
+
+
+def f16_to_f32_n(h):
+    h = np.ascontiguousarray(h, dtype=np.uint16)
+    out = np.empty(h.shape, np.float32)
+    lib().orc_f16_to_f32_n(_p(h, u16p), _p(out, f32p), C.c_size_t(h.size))
+    return out
+
+
+def f32_to_f16_n(f):
+    f = np.ascontiguousarray(f, dtype=np.float32)
+    out = np.empty(f.shape, np.uint16)
+    lib().orc_f32_to_f16_n(_p(f, f32p), _p(out, u16p), C.c_size_t(f.size))
+    return out
+
+
+def rope_tables(base, head_dim, n_pos, freq_factors=None, pos_begin=0):
+    half = head_dim // 2
+    cos = np.empty((n_pos - pos_begin, half), np.float16)
+    sin = np.empty((n_pos - pos_begin, half), np.float16)
+    ff = None
+    if freq_factors is not None:
+        ff = np.ascontiguousarray(freq_factors, dtype=np.float32)
+    lib().orc_rope_tables(C.c_float(base), C.c_uint32(head_dim), C.c_uint32(pos_begin), C.c_uint32(n_pos),
+                          _p(ff, f32p) if ff is not None else None, _p(cos, u16p), _p(sin, u16p))
+    return cos, sin
+
+
+def rope_neox(x, cos, sin, dim, seq_len, position_offset):
+    x = _h(x)
+    out = np.empty_like(x)
+    lib().orc_rope_neox(_p(x, u16p), _p(out, u16p), _p(_h(cos), u16p), _p(_h(sin), u16p), C.c_uint32(dim),
+                        C.c_uint32(seq_len), C.c_uint32(position_offset), C.c_size_t(x.size))
+    return out
+
+
+def kv_rearrange(x, n_heads, n_kv_heads, head_dim, seq, batch=1):
+    """[batch*seq, n_kv_heads*head_dim] -> [batch*n_heads, seq, head_dim] (GQA map h -> h/group)."""
+    x = _h(x)
+    kv_dim = n_kv_heads * head_dim
+    out = np.zeros((batch * n_heads, seq, head_dim), np.float16)
+    lib().orc_kv_rearrange(_p(x, u16p), _p(out, u16p), C.c_uint32(kv_dim), C.c_uint32(kv_dim), C.c_uint32(head_dim),
+                           C.c_uint32(n_heads), C.c_uint32(n_kv_heads), C.c_uint32(head_dim), C.c_uint32(seq),
+                           C.c_size_t(out.size))
+    return out
+
+
+def kv_cache_write(cache, x, n_kv_heads, head_dim, input_seq_len, position_offset, max_seq_len):
+    assert cache.dtype == np.float16 and cache.flags.c_contiguous
+    lib().orc_kv_cache_write(_p(cache, u16p), _p(_h(x), u16p), C.c_uint32(n_kv_heads), C.c_uint32(head_dim),
+                             C.c_uint32(input_seq_len), C.c_uint32(position_offset), C.c_uint32(max_seq_len))
+
+
+def kv_cache_write_repeat(cache, x, n_kv_heads, n_heads, head_dim, input_seq_len, position_offset, max_seq_len):
+    assert cache.dtype == np.float16 and cache.flags.c_contiguous
+    lib().orc_kv_cache_write_repeat(_p(cache, u16p), _p(_h(x), u16p), C.c_uint32(n_kv_heads), C.c_uint32(n_heads),
+                                    C.c_uint32(n_heads // n_kv_heads), C.c_uint32(head_dim),
+                                    C.c_uint32(input_seq_len), C.c_uint32(position_offset), C.c_uint32(max_seq_len))
+
+
+def kv_cache_read(cache, n_kv_heads, head_dim, seq_len, max_seq_len):
+    out = np.empty((n_kv_heads, seq_len, head_dim), np.float16)
+    lib().orc_kv_cache_read(_p(_h(cache), u16p), _p(out, u16p), C.c_uint32(n_kv_heads), C.c_uint32(head_dim),
+                            C.c_uint32(seq_len), C.c_uint32(max_seq_len))
+    return out
+
+
+def repeat_kv_heads(x, n_kv_heads, n_heads, seq, head_dim, cache_stride, batch=1):
+    out = np.empty((batch * n_heads, seq, head_dim), np.float16)
+    lib().orc_repeat_kv_heads(_p(_h(x), u16p), _p(out, u16p), C.c_uint32(n_heads // n_kv_heads), C.c_uint32(batch),
+                              C.c_uint32(n_kv_heads), C.c_uint32(n_heads), C.c_uint32(seq), C.c_uint32(head_dim),
+                              C.c_uint32(cache_stride))
+    return out
+
+
+def make_params(n_heads, n_kv_heads, head_dim, seq_len, position_offset, max_seq_len, rope_mode=0, layer_idx=0,
+                no_rope_layer_step=0):
+    return KvPrepParams(n_heads * head_dim, n_kv_heads * head_dim, head_dim, n_heads, n_kv_heads,
+                        n_heads // n_kv_heads, seq_len, position_offset, max_seq_len,
+                        n_heads * seq_len * head_dim, rope_mode, layer_idx, no_rope_layer_step)
+
+
+def kv_prep_fused(q, k, v, k_cache, v_cache, cos, sin, params):
+    """Appends into k_cache / v_cache in place and returns q_rot [n_heads, seq_len, head_dim]."""
+    q_rot = np.empty((params.n_heads, params.seq_len, params.head_dim), np.float16)
+    assert k_cache.dtype == np.float16 and k_cache.flags.c_contiguous
+    assert v_cache.dtype == np.float16 and v_cache.flags.c_contiguous
+    lib().orc_kv_prep_fused(_p(_h(q), u16p), _p(_h(k), u16p), _p(_h(v), u16p), _p(q_rot, u16p), _p(k_cache, u16p),
+                            _p(v_cache, u16p), _p(_h(cos), u16p), _p(_h(sin), u16p), C.byref(params))
+    return q_rot
+
+
+def sdpa_decode(q, k, v, n_heads, n_kv_heads, head_dim, capacity, kv_len, scale=None, block_keys=256, warps=16,
+                tg_out_half=False, n_threads=1):
+    if scale is None:
+        scale = np.float32(1.0) / np.sqrt(np.float32(head_dim))
+    out = np.empty((n_heads * head_dim,), np.float16)
+    lib().orc_sdpa_decode(_p(_h(q), u16p), _p(_h(k), u16p), _p(_h(v), u16p), _p(out, u16p), C.c_uint32(n_heads),
+                          C.c_uint32(n_kv_heads), C.c_uint32(head_dim), C.c_uint32(capacity), C.c_uint32(kv_len),
+                          C.c_float(scale), C.c_uint32(block_keys), C.c_uint32(warps), C.c_int(int(tg_out_half)),
+                          C.c_int(n_threads))
+    return out
+
+
+def sdpa_prefill(q, k, v, n_heads, n_kv_heads, head_dim, q_len, kv_len, query_offset, capacity, causal=True,
+                 q_layout="head_major", out_layout="token_major", scale=None, tile_keys=32, n_threads=1):
+    """q: head-major [H, q_len, D] or token-major [q_len, H*D]; K/V [Hkv, capacity, D]; out token-major
+    [q_len, H*D] (the reference's attn_out layout) or head-major [H, q_len, D]."""
+    if scale is None:
+        scale = np.float32(1.0) / np.sqrt(np.float32(head_dim))
+    D = head_dim
+    if q_layout == "head_major":
+        qsh, qsm = q_len * D, D
+    else:
+        qsh, qsm = D, n_heads * D
+    if out_layout == "token_major":
+        out = np.zeros((q_len, n_heads * D), np.float16)
+        osh, osm = D, n_heads * D
+    else:
+        out = np.zeros((n_heads, q_len, D), np.float16)
+        osh, osm = q_len * D, D
+    u64 = C.c_uint64
+    lib().orc_sdpa_prefill(_p(_h(q), u16p), _p(_h(k), u16p), _p(_h(v), u16p), _p(out, u16p), C.c_uint32(n_heads),
+                           C.c_uint32(n_heads // n_kv_heads), C.c_uint32(D), C.c_uint32(q_len), C.c_uint32(kv_len),
+                           C.c_uint32(query_offset), C.c_int(int(causal)), C.c_float(scale), u64(qsh), u64(qsm),
+                           u64(capacity * D), u64(D), u64(capacity * D), u64(D), u64(osh), u64(osm),
+                           C.c_uint32(tile_keys), C.c_int(n_threads))
+    return out
+
+
+def sdpa_row_splitk(q_row, k_head, v_head, head_dim, kv_len, causal_limit, split_k, tile_keys=32, scale=None):
+    if scale is None:
+        scale = np.float32(1.0) / np.sqrt(np.float32(head_dim))
+    acc = np.zeros((split_k, head_dim), np.float32)
+    m = np.zeros((split_k,), np.float32)
+    l = np.zeros((split_k,), np.float32)
+    lib().orc_sdpa_row_partials(_p(_h(q_row), u16p), _p(_h(k_head), u16p), _p(_h(v_head), u16p), C.c_uint32(head_dim),
+                                C.c_uint64(head_dim), C.c_uint64(head_dim), C.c_uint32(kv_len),
+                                C.c_uint32(causal_limit), C.c_float(scale), C.c_uint32(split_k), C.c_uint32(tile_keys),
+                                _p(acc, f32p), _p(m, f32p), _p(l, f32p))
+    out = np.empty((head_dim,), np.float16)
+    lib().orc_splitk_merge(_p(acc, f32p), _p(m, f32p), _p(l, f32p), C.c_uint32(split_k), C.c_uint32(head_dim),
+                           _p(out, u16p))
+    return out, acc, m, l
+
+
+def paged_gather(pool, block_table, n_kv_heads, block_size, head_dim, seq_len, out_capacity=None):
+    if out_capacity is None:
+        out_capacity = seq_len
+    out = np.zeros((n_kv_heads, out_capacity, head_dim), np.float16)
+    bt = np.ascontiguousarray(block_table, dtype=np.int32)
+    lib().orc_paged_gather(_p(_h(pool), u16p), _p(bt, i32p), C.c_uint32(n_kv_heads), C.c_uint32(block_size),
+                           C.c_uint32(head_dim), C.c_uint32(seq_len), C.c_uint32(out_capacity), _p(out, u16p))
+    return out
+
+
+def paged_scatter(pool, block_table, n_kv_heads, block_size, head_dim, pos_begin, pos_end, src):
+    assert pool.dtype == np.float16 and pool.flags.c_contiguous
+    bt = np.ascontiguousarray(block_table, dtype=np.int32)
+    src = _h(src)
+    lib().orc_paged_scatter(_p(pool, u16p), _p(bt, i32p), C.c_uint32(n_kv_heads), C.c_uint32(block_size),
+                            C.c_uint32(head_dim), C.c_uint32(pos_begin), C.c_uint32(pos_end),
+                            C.c_uint32(src.shape[1]), _p(src, u16p))
+
+
+def sage_k_mean(k, n_kv_heads, capacity, head_dim, kv_len):
+    mean = np.zeros((n_kv_heads, head_dim), np.float32)
+    lib().orc_sage_k_mean(_p(_h(k), u16p), C.c_uint32(n_kv_heads), C.c_uint32(capacity), C.c_uint32(head_dim),
+                          C.c_uint32(kv_len), _p(mean, f32p))
+    return mean
+
+
+def sage_quantize_k(k, mean, n_kv_heads, capacity, head_dim, kv_len, block=32):
+    kq = np.zeros((n_kv_heads, capacity, head_dim), np.int8)
+    ks = np.zeros((n_kv_heads, (capacity + block - 1) // block), np.float16)
+    mean = np.ascontiguousarray(mean, dtype=np.float32)
+    lib().orc_sage_quantize_k(_p(_h(k), u16p), _p(mean, f32p), C.c_uint32(n_kv_heads), C.c_uint32(capacity),
+                              C.c_uint32(head_dim), C.c_uint32(kv_len), C.c_uint32(block), _p(kq, i8p), _p(ks, u16p))
+    return kq, ks
+
+
+def sage_quantize_q(q, n_heads, head_dim):
+    qq = np.zeros((n_heads, head_dim), np.int8)
+    qs = np.zeros((n_heads,), np.float32)
+    lib().orc_sage_quantize_q(_p(_h(q), u16p), C.c_uint32(n_heads), C.c_uint32(head_dim), _p(qq, i8p), _p(qs, f32p))
+    return qq, qs
+
+
+def sage_decode(qq, qs, kq, ks, v, n_heads, n_kv_heads, head_dim, capacity, kv_len, block=32, scale=None,
+                n_threads=1):
+    if scale is None:
+        scale = np.float32(1.0) / np.sqrt(np.float32(head_dim))
+    out = np.empty((n_heads * head_dim,), np.float16)
+    lib().orc_sage_decode(_p(np.ascontiguousarray(qq), i8p), _p(np.ascontiguousarray(qs), f32p),
+                          _p(np.ascontiguousarray(kq), i8p), _p(_h(ks), u16p), _p(_h(v), u16p), _p(out, u16p),
+                          C.c_uint32(n_heads), C.c_uint32(n_kv_heads), C.c_uint32(head_dim), C.c_uint32(capacity),
+                          C.c_uint32(kv_len), C.c_uint32(block), C.c_float(scale), C.c_int(n_threads))
+    return out
+
+
+def lcg_fill_f16(state, n, scale):
+    """Returns (array, new_state): the reference tests' LCG stream."""
+    st = C.c_uint32(state)
+    out = np.empty((n,), np.float16)
+    lib().orc_lcg_fill_f16(C.byref(st), _p(out, u16p), C.c_size_t(n), C.c_float(scale))
+    return out, st.value

@@ -1,0 +1,458 @@
+"""Pins the CPU oracle (oracle/oracle_attn.c) without a GPU.
+
+Each check is independent of the oracle's own formulae: exhaustive comparison with numpy's binary16,
+closed forms, float64 library softmax / complex rotation, index brute force, the reference tests' own
+closed-form known-answer inputs (tests/golden/known_answer_sdpa.npz) and algebraic invariants.
+Reference citations are paths under /root/reference/crates/metallic-foundry/.
+"""
+import os
+
+import numpy as np
+import pytest
+
+import orc
+import refmath as rm
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+rng_global = np.random.default_rng(0xF0DD)
+
+
+def h16(a):
+    return np.asarray(a, dtype=np.float32).astype(np.float16)
+
+
+# ----------------------------------------------------------------------------- f16 conversions
+
+def test_f16_to_f32_exhaustive():
+    bits = np.arange(65536, dtype=np.uint16)
+    got = orc.f16_to_f32_n(bits)
+    want = bits.view(np.float16).astype(np.float32)
+    assert np.array_equal(got.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.all(np.isnan(got[np.isnan(want)]))
+
+
+def test_f32_to_f16_rne_against_numpy():
+    rng = np.random.default_rng(1)
+    # random bit patterns, midpoints between adjacent halves, subnormal and overflow boundaries
+    rand = rng.integers(0, 2 ** 32, size=2_000_000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    halves = np.arange(0, 0x7c00, dtype=np.uint16).view(np.float16).astype(np.float64)
+    mids = ((halves[:-1] + halves[1:]) / 2).astype(np.float32)  # exact ties
+    near = np.concatenate([np.nextafter(mids, np.float32(np.inf)), np.nextafter(mids, np.float32(-np.inf))])
+    edge = np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 65536.0, 1e30, np.inf, -np.inf, 2.0 ** -24, 2.0 ** -25,
+                     np.nextafter(np.float32(2.0 ** -25), np.float32(1)), 2.0 ** -26, 5.96e-8, 6.1e-5], np.float32)
+    x = np.concatenate([rand, mids, -mids, near, edge, -edge])
+    x = x[~np.isnan(x)]
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    got = orc.f32_to_f16_n(x)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, (x[bad[:5]], got[bad[:5]], want[bad[:5]])
+    assert np.isnan(np.array([orc.lib().orc_f32_to_f16(float("nan"))], np.uint16).view(np.float16))[0]
+
+
+# ----------------------------------------------------------------------------- RoPE tables (src/model/executor.rs:1981-2006)
+
+@pytest.mark.parametrize("base,D,P", [(1e6, 64, 1100), (5e5, 128, 8500), (1e4, 128, 64)])
+def test_rope_tables_closed_forms(base, D, P):
+    cos, sin = orc.rope_tables(base, D, P)
+    assert cos.shape == (P, D // 2)
+    assert np.all(cos[0] == np.float16(1)) and np.all(sin[0] == np.float16(0))
+    # column 0: exponent 0 -> inv_freq 1 -> angle = p exactly (p < 2^24)
+    p = np.arange(P, dtype=np.float64)
+    assert np.all(np.abs(cos[:, 0].astype(np.float64) - np.cos(p)) <= 0.5 * rm.f16_ulp(np.cos(p)) + 1e-7)
+    assert np.all(np.abs(sin[:, 0].astype(np.float64) - np.sin(p)) <= 0.5 * rm.f16_ulp(np.sin(p)) + 1e-7)
+    # all columns against float64 cos/sin of the f32 angle
+    i = np.arange(D // 2)
+    inv = (np.float32(1) / np.power(np.float32(base), (2 * i).astype(np.float32) / np.float32(D))).astype(np.float32)
+    ang = (p.astype(np.float32)[:, None] * inv[None, :]).astype(np.float32).astype(np.float64)
+    # a few f32 ulp of slack on inv_freq (libm powf vs numpy power) scale with the angle
+    slack = 4e-7 * np.abs(ang) + 0.5 * 2.0 ** -11 + 1e-6
+    assert np.all(np.abs(cos.astype(np.float64) - np.cos(ang)) <= slack)
+    assert np.all(np.abs(sin.astype(np.float64) - np.sin(ang)) <= slack)
+    # cos^2 + sin^2 = 1 within f16 rounding
+    assert np.all(np.abs(cos.astype(np.float64) ** 2 + sin.astype(np.float64) ** 2 - 1) < 2e-3)
+
+
+def test_rope_tables_freq_factors_and_window():
+    ff = np.linspace(1.0, 8.0, 32).astype(np.float32)
+    c_all, s_all = orc.rope_tables(5e5, 64, 300, ff)
+    c_win, s_win = orc.rope_tables(5e5, 64, 300, ff, pos_begin=200)
+    assert np.array_equal(c_all[200:], c_win) and np.array_equal(s_all[200:], s_win)
+    c_one, _ = orc.rope_tables(5e5, 64, 300, np.ones(32, np.float32))
+    c_none, _ = orc.rope_tables(5e5, 64, 300)
+    assert np.array_equal(c_one, c_none)
+    # dividing inv_freq by f == evaluating the unscaled column at angle/f
+    i = np.arange(32)
+    inv = 1.0 / np.power(5e5, 2 * i / 64.0) / ff
+    ang = np.arange(300)[:, None] * inv[None, :]
+    assert np.max(np.abs(c_all.astype(np.float64) - np.cos(ang))) < 1e-3
+
+
+# ----------------------------------------------------------------------------- NeoX RoPE (tests/rope.rs:31-63)
+
+@pytest.mark.parametrize("dim,seq,rows,off", [(64, 1, 1, 0), (64, 16, 16, 0), (128, 8, 32, 0), (256, 4, 8, 0),
+                                              (64, 1, 14, 1024), (128, 7, 21, 5), (64, 128, 128, 0), (2, 4, 4, 1)])
+def test_rope_neox_is_complex_rotation(dim, seq, rows, off):
+    rng = np.random.default_rng(dim * 131 + seq)
+    x = h16(rng.uniform(-1, 1, size=(rows, dim)))
+    cos, sin = orc.rope_tables(10000.0, dim, seq + off)
+    got = orc.rope_neox(x, cos, sin, dim, seq, off)
+    pos = (np.arange(rows) % seq) + off
+    want = rm.rope_rotate_f64(x, cos, sin, pos, "neox")
+    err = np.abs(got.astype(np.float64) - want)
+    assert np.all(err <= 0.5 * rm.f16_ulp(want) + 2e-7)  # f32 products/sum then one RNE to f16
+
+
+def test_rope_neox_invariants():
+    rng = np.random.default_rng(7)
+    dim, seq = 64, 9
+    x = h16(rng.normal(size=(seq, dim)))
+    cos, sin = orc.rope_tables(1e6, dim, seq)
+    y = orc.rope_neox(x, cos, sin, dim, seq, 0)
+    assert np.array_equal(y[0], x[0])  # position 0: cos 1, sin 0
+    nx = x.astype(np.float64)[:, :32] ** 2 + x.astype(np.float64)[:, 32:] ** 2
+    ny = y.astype(np.float64)[:, :32] ** 2 + y.astype(np.float64)[:, 32:] ** 2
+    assert np.all(np.abs(nx - ny) <= 4e-3 * (1 + nx))  # table cos^2+sin^2 != 1 exactly in f16
+    back = orc.rope_neox(y, cos, (-sin.astype(np.float32)).astype(np.float16), dim, seq, 0)
+    assert np.max(np.abs(back.astype(np.float32) - x.astype(np.float32))) < 6e-3
+    ident = orc.rope_neox(x, np.ones_like(cos), np.zeros_like(sin), dim, seq, 0)
+    assert np.array_equal(ident, x)  # tests/sdpa_v2_parity.rs:153-155 identity tables
+
+
+# ----------------------------------------------------------------------------- index maps of the legacy chain
+
+def test_kv_rearrange_brute_force():
+    # tests/kv_rearrange.rs:33-68: out[b*H + h, s, d] = in[b*seq + s, (h / G)*D + d]
+    H, Hkv, D, S, B = 6, 2, 8, 5, 2
+    x = h16(np.arange(B * S * Hkv * D).reshape(B * S, Hkv * D) % 2048)
+    got = orc.kv_rearrange(x, H, Hkv, D, S, batch=B)
+    for b in range(B):
+        for h in range(H):
+            for s in range(S):
+                assert np.array_equal(got[b * H + h, s], x[b * S + s, (h // 3) * D:(h // 3 + 1) * D])
+
+
+def test_kv_cache_write_read_brute_force():
+    Hkv, D, S, off, cap = 3, 4, 5, 7, 16
+    x = h16(np.arange(Hkv * S * D).reshape(Hkv, S, D))
+    cache = np.zeros((Hkv, cap, D), np.float16)
+    orc.kv_cache_write(cache, x, Hkv, D, S, off, cap)
+    want = np.zeros_like(cache)
+    want[:, off:off + S] = x
+    assert np.array_equal(cache, want)
+    assert np.array_equal(orc.kv_cache_read(cache, Hkv, D, off + S, cap), want[:, :off + S])
+
+
+def test_kv_cache_write_repeat_and_repeat_kv_heads():
+    # tests/kv_cache_write_repeat_kv_heads.rs:57-70 and tests/repeat_kv_heads.rs:32-61
+    Hkv, H, D, S, off, cap = 2, 6, 4, 3, 2, 8
+    x = h16(np.arange(Hkv * S * D).reshape(Hkv, S, D) + 1)
+    cache = np.zeros((H, cap, D), np.float16)
+    orc.kv_cache_write_repeat(cache, x, Hkv, H, D, S, off, cap)
+    for h in range(H):
+        assert np.array_equal(cache[h, off:off + S], x[h // 3])
+        assert not cache[h, :off].any() and not cache[h, off + S:].any()
+    compact = np.zeros((Hkv, cap, D), np.float16)
+    orc.kv_cache_write(compact, x, Hkv, D, S, off, cap)
+    rep = orc.repeat_kv_heads(compact, Hkv, H, off + S, D, cap)
+    assert np.array_equal(rep, cache[:, :off + S])
+
+
+# ----------------------------------------------------------------------------- fused kv_prep
+
+def _chain_reference(q, k, v, H, Hkv, D, S, off, cap, cos, sin):
+    """The un-fused chain the reference's parity test compares against (tests/kv_prep_fused.rs:60-200):
+    rearrange -> NeoX rope -> compact cache write."""
+    q_r = orc.kv_rearrange(q, H, H, D, S)
+    q_rot = orc.rope_neox(q_r, cos, sin, D, S, off)
+    k_r = orc.kv_rearrange(k, Hkv, Hkv, D, S)
+    k_rot = orc.rope_neox(k_r, cos, sin, D, S, off)
+    v_r = orc.kv_rearrange(v, Hkv, Hkv, D, S)
+    kc = np.zeros((Hkv, cap, D), np.float16)
+    vc = np.zeros((Hkv, cap, D), np.float16)
+    orc.kv_cache_write(kc, k_rot, Hkv, D, S, off, cap)
+    orc.kv_cache_write(vc, v_r, Hkv, D, S, off, cap)
+    return q_rot, kc, vc
+
+
+@pytest.mark.parametrize("S,off,cap,H,Hkv,D", [(1, 5, 16, 14, 2, 64), (4, 0, 16, 14, 2, 64), (2, 0, 64, 32, 8, 128),
+                                               (3, 9, 12, 24, 8, 128), (1, 1024, 1152, 14, 2, 64)])
+def test_kv_prep_fused_neox_equals_chain_bitwise(S, off, cap, H, Hkv, D):
+    rng = np.random.default_rng(S * 1000 + off)
+    q = h16(rng.uniform(-1, 1, (S, H * D)))
+    k = h16(rng.uniform(-1, 1, (S, Hkv * D)))
+    v = h16(rng.uniform(-1, 1, (S, Hkv * D)))
+    cos, sin = orc.rope_tables(10000.0, D, cap)
+    q_ref, kc_ref, vc_ref = _chain_reference(q, k, v, H, Hkv, D, S, off, cap, cos, sin)
+    kc = np.zeros((Hkv, cap, D), np.float16)
+    vc = np.zeros((Hkv, cap, D), np.float16)
+    q_rot = orc.kv_prep_fused(q, k, v, kc, vc, cos, sin, orc.make_params(H, Hkv, D, S, off, cap, rope_mode=0))
+    assert np.array_equal(q_rot.view(np.uint16), q_ref.view(np.uint16))
+    assert np.array_equal(kc.view(np.uint16), kc_ref.view(np.uint16))  # tests/kv_prep_fused.rs:239-244
+    assert np.array_equal(vc.view(np.uint16), vc_ref.view(np.uint16))
+    assert not kc[:, :off].any() and not kc[:, off + S:].any()  # untouched slots stay zero
+
+
+def _deinterleave(x, D):
+    """Per head: even dims first, then odd dims."""
+    shp = x.shape
+    xx = x.reshape(shp[0], -1, D)
+    return np.concatenate([xx[..., 0::2], xx[..., 1::2]], axis=-1).reshape(shp)
+
+
+def _interleave(x, D):
+    shp = x.shape
+    xx = x.reshape(-1, D)
+    out = np.empty_like(xx)
+    out[:, 0::2], out[:, 1::2] = xx[:, :D // 2], xx[:, D // 2:]
+    return out.reshape(shp)
+
+
+@pytest.mark.parametrize("S,off,cap,H,Hkv,D", [(1, 5, 16, 14, 2, 64), (5, 3, 16, 24, 8, 128)])
+def test_kv_prep_fused_normal_is_neox_under_deinterleave(S, off, cap, H, Hkv, D):
+    """`normal` pairing (kv_prep_fused.metal:66-73) has no reference test; pinned by
+    normal(x) == interleave(neox(deinterleave(x))) and by the complex-rotation closed form."""
+    rng = np.random.default_rng(99 + S)
+    q = h16(rng.normal(size=(S, H * D)))
+    k = h16(rng.normal(size=(S, Hkv * D)))
+    v = h16(rng.normal(size=(S, Hkv * D)))
+    cos, sin = orc.rope_tables(5e5, D, cap)
+    kc_n, vc_n = np.zeros((Hkv, cap, D), np.float16), np.zeros((Hkv, cap, D), np.float16)
+    q_n = orc.kv_prep_fused(q, k, v, kc_n, vc_n, cos, sin, orc.make_params(H, Hkv, D, S, off, cap, rope_mode=1))
+    kc_x, vc_x = np.zeros((Hkv, cap, D), np.float16), np.zeros((Hkv, cap, D), np.float16)
+    q_x = orc.kv_prep_fused(_deinterleave(q, D), _deinterleave(k, D), v, kc_x, vc_x, cos, sin,
+                            orc.make_params(H, Hkv, D, S, off, cap, rope_mode=0))
+    assert np.array_equal(q_n.view(np.uint16), _interleave(q_x, D).view(np.uint16))
+    assert np.array_equal(kc_n.view(np.uint16), _interleave(kc_x, D).view(np.uint16))
+    assert np.array_equal(vc_n.view(np.uint16), vc_x.view(np.uint16))
+    # closed form
+    pos = np.arange(S) + off
+    q_tm = q.reshape(S, H, D)
+    want = rm.rope_rotate_f64(q_tm, cos, sin, pos[:, None], "normal").transpose(1, 0, 2)
+    assert np.all(np.abs(q_n.astype(np.float64) - want) <= 0.5 * rm.f16_ulp(want) + 4e-7)
+
+
+def test_kv_prep_fused_nope_layer_rule():
+    """apply_rope = step == 0 or (layer+1) % step != 0 (kv_prep_fused.metal:57); SmolLM3 uses step 4."""
+    S, off, cap, H, Hkv, D = 2, 3, 8, 16, 4, 128
+    rng = np.random.default_rng(5)
+    q, k, v = (h16(rng.normal(size=(S, n * D))) for n in (H, Hkv, Hkv))
+    cos, sin = orc.rope_tables(5e6, D, cap)
+    plain_q = orc.kv_rearrange(q, H, H, D, S)
+    plain_k = np.zeros((Hkv, cap, D), np.float16)
+    orc.kv_cache_write(plain_k, orc.kv_rearrange(k, Hkv, Hkv, D, S), Hkv, D, S, off, cap)
+    roped = None
+    for layer in range(8):
+        kc, vc = np.zeros((Hkv, cap, D), np.float16), np.zeros((Hkv, cap, D), np.float16)
+        q_rot = orc.kv_prep_fused(q, k, v, kc, vc, cos, sin,
+                                  orc.make_params(H, Hkv, D, S, off, cap, rope_mode=1, layer_idx=layer,
+                                                  no_rope_layer_step=4))
+        if layer in (3, 7):
+            assert np.array_equal(q_rot, plain_q) and np.array_equal(kc, plain_k)
+        else:
+            assert not np.array_equal(q_rot, plain_q)
+            if roped is None:
+                roped = (q_rot.copy(), kc.copy())
+            assert np.array_equal(q_rot, roped[0]) and np.array_equal(kc, roped[1])
+    kc0, vc0 = np.zeros((Hkv, cap, D), np.float16), np.zeros((Hkv, cap, D), np.float16)
+    q0 = orc.kv_prep_fused(q, k, v, kc0, vc0, cos, sin, orc.make_params(H, Hkv, D, S, off, cap, rope_mode=1,
+                                                                        layer_idx=3, no_rope_layer_step=0))
+    assert np.array_equal(q0, roped[0])  # step 0 disables the rule
+
+
+# ----------------------------------------------------------------------------- SDPA decode
+
+def test_sdpa_known_answer_decode_fixture():
+    g = np.load(os.path.join(GOLD, "known_answer_sdpa.npz"))
+    q, k, v, want = g["oob_m1_q"], g["oob_m1_k"], g["oob_m1_v"], g["oob_m1_expected_f64"]
+    H, M, D = q.shape
+    N = k.shape[1]
+    got = orc.sdpa_decode(q.reshape(H, D), k, v, H, H, D, N, N).reshape(H, D).astype(np.float64)
+    assert np.all(np.abs(got - want[:, 0]) <= 0.5 * rm.f16_ulp(want[:, 0]) + 2e-6 * np.abs(want[:, 0]) + 1e-8)
+
+
+def test_sdpa_known_answer_prefill_fixture_noncausal():
+    g = np.load(os.path.join(GOLD, "known_answer_sdpa.npz"))
+    q, k, v, want = (g["misaligned_m17_" + n] for n in ("q", "k", "v", "expected_f64"))
+    H, M, D = q.shape
+    N = k.shape[1]
+    got = orc.sdpa_prefill(q, k, v, H, H, D, M, N, 0, N, causal=False)  # token-major [M, H*D]
+    got = got.reshape(M, H, D).transpose(1, 0, 2).astype(np.float64)
+    assert np.all(np.abs(got - want) <= 0.5 * rm.f16_ulp(want) + 4e-6 * np.abs(want) + 1e-8)
+
+
+def test_lcg_stream_matches_integer_recurrence():
+    # tests/flashattention_decode_parity.rs:15-30, recomputed with Python integers
+    st = 1
+    want = []
+    for _ in range(64):
+        st = (st * 1664525 + 1013904223) % (1 << 32)
+        want.append(np.float32(np.float32(st >> 9) * np.float32(1.0 / (1 << 23)) * np.float32(2) - np.float32(1))
+                    * np.float32(0.25))
+    got, new_state = orc.lcg_fill_f16(1, 64, 0.25)
+    assert new_state == st
+    assert np.array_equal(got, np.array(want, np.float32).astype(np.float16))
+
+
+@pytest.mark.parametrize("seed,H,D,N", [(1, 14, 64, 128), (7, 14, 64, 257), (42, 8, 128, 300)])
+def test_sdpa_decode_reference_test_inputs_vs_f64(seed, H, D, N):
+    """The reference's decode parity inputs (LCG, +-0.25), MHA cache [H, N, D]
+    (tests/flashattention_decode_parity.rs:117-200); expected from float64 softmax."""
+    st = seed
+    q, st = orc.lcg_fill_f16(st, H * D, 0.25)
+    k, st = orc.lcg_fill_f16(st, H * N * D, 0.25)
+    v, st = orc.lcg_fill_f16(st, H * N * D, 0.25)
+    k, v = k.reshape(H, N, D), v.reshape(H, N, D)
+    want = rm.gqa_decode_f64(q, k, v, H, H, D, N)
+    for block, warps in [(512, 16), (128, 8), (1, 1), (37, 5)]:
+        got = orc.sdpa_decode(q, k, v, H, H, D, N, N, block_keys=block, warps=warps).reshape(H, D)
+        assert np.max(np.abs(got.astype(np.float64) - want)) < 2.5e-4  # half an f16 ulp at |x| < 0.25 + f32 noise
+    got_h = orc.sdpa_decode(q, k, v, H, H, D, N, N, block_keys=256, warps=16, tg_out_half=True).reshape(H, D)
+    assert np.max(np.abs(got_h.astype(np.float64) - want)) < 3e-3  # f16 partials: the reference's looser variant
+
+
+def test_sdpa_decode_invariants():
+    rng = np.random.default_rng(3)
+    H, Hkv, D, cap, N = 6, 2, 64, 40, 33
+    q = h16(rng.normal(size=(H, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    k_same = np.broadcast_to(h16(rng.normal(size=(Hkv, 1, D))), (Hkv, cap, D)).copy()
+    out = orc.sdpa_decode(q, k_same, v, H, Hkv, D, cap, N).reshape(H, D)
+    for h in range(H):  # equal keys -> uniform weights -> mean of V
+        want = v[h // 3, :N].astype(np.float64).mean(axis=0)
+        assert np.max(np.abs(out[h].astype(np.float64) - want)) < 1e-3
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    out1 = orc.sdpa_decode(q, k, v, H, Hkv, D, cap, 1).reshape(H, D)
+    for h in range(H):  # a single key -> V[0]
+        assert np.array_equal(out1[h], v[h // 3, 0])
+    # rows beyond kv_len are never read
+    k2, v2 = k.copy(), v.copy()
+    k2[:, N:], v2[:, N:] = np.float16(np.nan), np.float16(np.nan)
+    a = orc.sdpa_decode(q, k, v, H, Hkv, D, cap, N)
+    b = orc.sdpa_decode(q, k2, v2, H, Hkv, D, cap, N)
+    assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("H,Hkv,D,N", [(14, 2, 64, 100), (24, 8, 128, 70), (16, 2, 128, 65), (16, 4, 128, 40)])
+def test_sdpa_gqa_equals_mha_on_expanded_cache(H, Hkv, D, N):
+    """GQA head map (flash_decode.metal:129-132) has no reference numeric test; pinned by
+    GQA(compact) == MHA(repeat_kv_heads(compact)) and by float64 per-head attention."""
+    rng = np.random.default_rng(H + N)
+    cap = N + 5
+    q = h16(rng.normal(size=(H, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    got = orc.sdpa_decode(q, k, v, H, Hkv, D, cap, N)
+    k_exp = orc.repeat_kv_heads(k, Hkv, H, cap, D, cap)
+    v_exp = orc.repeat_kv_heads(v, Hkv, H, cap, D, cap)
+    mha = orc.sdpa_decode(q, k_exp, v_exp, H, H, D, cap, N)
+    assert np.array_equal(got, mha)
+    want = rm.gqa_decode_f64(q, k, v, H, Hkv, D, N)
+    assert np.max(np.abs(got.reshape(H, D).astype(np.float64) - want)) < 1.5e-3
+
+
+# ----------------------------------------------------------------------------- SDPA prefill
+
+@pytest.mark.parametrize("M,prefix", [(1, 0), (2, 0), (7, 0), (16, 0), (17, 5), (26, 0), (31, 100), (32, 0), (33, 64)])
+def test_sdpa_prefill_causal_vs_f64_and_decode(M, prefix):
+    """m values of tests/flashattention_prefill_parity.rs:143-183; causal limit = row + query_offset
+    (flash_prefill.metal:176-199)."""
+    H, Hkv, D = 4, 2, 64
+    N = prefix + M
+    cap = N + 3
+    rng = np.random.default_rng(M * 7 + prefix)
+    q = h16(rng.normal(size=(H, M, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    got = orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, prefix, cap, causal=True, out_layout="head_major")
+    want = rm.gqa_prefill_f64(q, k, v, H, Hkv, D, N, prefix, causal=True)
+    assert np.max(np.abs(got.astype(np.float64) - want)) < 2e-3
+    tm = orc.sdpa_prefill(q.transpose(1, 0, 2).reshape(M, H * D).copy(), k, v, H, Hkv, D, M, N, prefix, cap,
+                          causal=True, q_layout="token_major", out_layout="token_major")
+    assert np.array_equal(tm.reshape(M, H, D).transpose(1, 0, 2), got)  # layouts only move data
+    for r in (0, M - 1):  # prefill row r == decode at kv_len = offset + r + 1
+        dec = orc.sdpa_decode(q[:, r].copy(), k, v, H, Hkv, D, cap, prefix + r + 1, block_keys=32, warps=1)
+        assert np.max(np.abs(dec.reshape(H, D).astype(np.float32) - got[:, r].astype(np.float32))) <= 1e-3
+    if prefix == 0:
+        for h in range(H):  # first row sees only key 0
+            assert np.array_equal(got[h, 0], v[h // 2, 0])
+
+
+def test_splitk_merge_independent_of_split_count():
+    """flash_prefill.metal:452-457,843-888, including empty splits (l_s <= 0 is skipped)."""
+    D, N = 64, 150
+    rng = np.random.default_rng(11)
+    q = h16(rng.normal(size=(D,)))
+    k = h16(rng.normal(size=(N, D)))
+    v = h16(rng.normal(size=(N, D)))
+    want = rm.attn_f64(q[None], k[:101], v[:101], 1 / np.sqrt(D))[0]
+    base = None
+    for S in (1, 2, 3, 4, 8, 16):
+        out, acc, m, l = orc.sdpa_row_splitk(q, k, v, D, N, 100, S)  # causal limit 100 -> later splits are empty
+        assert np.max(np.abs(out.astype(np.float64) - want)) < 1e-3
+        if S >= 8:
+            assert np.any(l == 0) and np.all(m[l == 0] == np.float32(-1e30))
+        if base is None:
+            base = out
+        assert np.max(np.abs(out.astype(np.float32) - base.astype(np.float32))) <= 1e-3
+    tiny, _, m1, l1 = orc.sdpa_row_splitk(q, k, v, D, 5, 4, 8)  # more splits than tiles
+    assert np.max(np.abs(tiny.astype(np.float64) - rm.attn_f64(q[None], k[:5], v[:5], 1 / np.sqrt(D))[0])) < 1e-3
+
+
+# ----------------------------------------------------------------------------- paged cache
+
+def test_paged_gather_scatter_roundtrip_with_permutation():
+    rng = np.random.default_rng(21)
+    Hkv, D, bs, N = 2, 16, 16, 75
+    n_blocks = 9
+    perm = rng.permutation(n_blocks)[: (N + bs - 1) // bs].astype(np.int32)
+    contiguous = h16(rng.normal(size=(Hkv, N, D)))
+    pool = np.full((n_blocks, Hkv, bs, D), np.float16(-7), np.float16)
+    orc.paged_scatter(pool, perm, Hkv, bs, D, 0, N, contiguous)
+    assert np.array_equal(orc.paged_gather(pool, perm, Hkv, bs, D, N), contiguous)
+    # brute force: slot of (h, pos)
+    for h, pos in [(0, 0), (1, 17), (0, 74), (1, 63)]:
+        assert np.array_equal(pool[perm[pos // bs], h, pos % bs], contiguous[h, pos])
+    untouched = np.setdiff1d(np.arange(n_blocks), perm)
+    assert np.all(pool[untouched] == np.float16(-7))
+
+
+# ----------------------------------------------------------------------------- Sage-style int8 Q/K
+
+def test_sage_quantizer_and_decode():
+    rng = np.random.default_rng(31)
+    H, Hkv, D, N = 8, 2, 128, 200
+    cap = 224
+    k = rng.normal(size=(Hkv, cap, D))
+    k += rng.normal(size=(Hkv, 1, D)) * 3  # channel bias that smoothing removes
+    out_mask = rng.random(size=k.shape) < 0.01
+    k = h16(np.where(out_mask, 8.0 * np.sign(k), k))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    q = h16(rng.normal(size=(H, D)))
+    mean = orc.sage_k_mean(k, Hkv, cap, D, N)
+    assert np.max(np.abs(mean - k[:, :N].astype(np.float64).mean(axis=1))) < 1e-5
+    kq, ks = orc.sage_quantize_k(k, mean, Hkv, cap, D, N)
+    ksf = ks.astype(np.float64)
+    centred = k[:, :N].astype(np.float32) - mean[:, None, :]
+    deq = kq[:, :N].astype(np.float64) * np.repeat(ksf, 32, axis=1)[:, :N, None]
+    # |x - dequant| <= scale/2 except where the f16-rounded scale clips the block maximum
+    assert np.all(np.abs(deq - centred) <= 0.5 * np.repeat(ksf, 32, axis=1)[:, :N, None] * 1.002 + 1e-6 +
+                  127 * np.abs(np.repeat(ksf, 32, axis=1)[:, :N, None] * 2.0 ** -11))
+    assert np.all(np.abs(kq) <= 127) and not kq[:, N:].any()
+    qq, qs = orc.sage_quantize_q(q, H, D)
+    assert np.all(np.abs(qq.astype(np.float64) * qs[:, None] - q.astype(np.float64)) <= 0.5 * qs[:, None] + 1e-7)
+    # mean smoothing leaves softmax unchanged: softmax(q (K - mu)^T) == softmax(q K^T)
+    s1 = q[0].astype(np.float64) @ k[0, :N].astype(np.float64).T
+    s2 = q[0].astype(np.float64) @ (k[0, :N].astype(np.float64) - mean[0].astype(np.float64)).T
+    from scipy.special import softmax
+    assert np.max(np.abs(softmax(s1) - softmax(s2))) < 1e-12
+    got = orc.sage_decode(qq, qs, kq, ks, v, H, Hkv, D, cap, N).reshape(H, D).astype(np.float64)
+    # against the int8 model evaluated in float64
+    for h in range(H):
+        s = (qq[h].astype(np.float64) @ kq[h // 4, :N].astype(np.float64).T) * qs[h] * \
+            np.repeat(ksf[h // 4], 32)[:N] / np.sqrt(D)
+        want = softmax(s) @ v[h // 4, :N].astype(np.float64)
+        assert np.max(np.abs(got[h] - want)) < 1e-3
+    # and the quantisation error against f16 SDPA on the unquantised tensors stays small
+    full = rm.gqa_decode_f64(q, k, v, H, Hkv, D, N)
+    assert np.max(np.abs(got - full)) < 5e-2
