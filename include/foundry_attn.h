@@ -1,0 +1,299 @@
+/*
+ * foundry_attn.h - C ABI of libfoundry_attn.so: the KV-cache attention path of metallic-foundry
+ * (fused RoPE + KV-cache append, flash decode, flash prefill, Sage-style int8 decode) for AMD MI355X
+ * (gfx950), written in HIP.
+ *
+ * This header is the single source of truth for the boundary. Every entry point names the reference
+ * interface it stands in for; paths are relative to crates/metallic-foundry/ of cchance27/test-burn.
+ *
+ * Conventions
+ *  - Every function returns fa_status (0 = ok). On failure a human-readable message is kept per thread
+ *    and returned by fa_last_error_string(). The library never aborts and never silently skips work on
+ *    an unsupported shape: what the reference's kernels guard with an early `return`
+ *    (src/metals/flashattention/flash_decode.metal:343-351) is a host-side error here.
+ *  - All device work is enqueued on the context's single HIP stream in program order and the call
+ *    returns immediately (the reference enqueues on one Metal queue with a buffer barrier after every
+ *    dispatch, src/types/mod.rs:577-580). fa_synchronize() waits for completion.
+ *  - One context per thread; a context is not thread-safe (Foundry is used through &mut,
+ *    src/lib.rs:44-53).
+ *  - The caller owns every tensor buffer. The library owns only a grow-only scratch workspace inside
+ *    the context (split-K partials), the counterpart of the reference's pooled split-K scratch
+ *    (src/metals/flashattention/step.rs:927-929).
+ *  - Tensors are f16 (IEEE binary16) unless stated; strides are in elements, offsets in bytes, exactly
+ *    as in TensorArg (src/types/mod.rs:339-347).
+ */
+#ifndef FOUNDRY_ATTN_H
+#define FOUNDRY_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---------------------------------------------------------------------------------------------
+ * Errors: the variants of MetalError that this path raises (src/error.rs:22-75).
+ * ------------------------------------------------------------------------------------------- */
+typedef enum fa_status {
+    FA_OK = 0,
+    FA_ERR_DEVICE_NOT_FOUND = 1,        /* MetalError::DeviceNotFound */
+    FA_ERR_NULL_POINTER = 2,            /* MetalError::NullPointer */
+    FA_ERR_INVALID_SHAPE = 3,           /* MetalError::InvalidShape(String) */
+    FA_ERR_OUT_OF_MEMORY = 4,           /* MetalError::OutOfMemory */
+    FA_ERR_OPERATION_NOT_SUPPORTED = 5, /* MetalError::OperationNotSupported(String) */
+    FA_ERR_INVALID_OPERATION = 6,       /* MetalError::InvalidOperation(String) */
+    FA_ERR_UNSUPPORTED_DTYPE = 7,       /* MetalError::UnsupportedDtype */
+    FA_ERR_OPERATION_FAILED = 8,        /* MetalError::OperationFailed(String) - HIP runtime failures land here */
+    FA_ERR_INPUT_NOT_FOUND = 9          /* MetalError::InputNotFound(String) - a required tensor has no buffer */
+} fa_status;
+
+const char *fa_status_name(fa_status s);
+/* Message of the last failing call on this thread ("" if none). Valid until the next failing call. */
+const char *fa_last_error_string(void);
+
+/* Dtype, same order as metallic-sdk's enum (crates/metallic-sdk/src/tensor.rs:7-30). */
+typedef enum fa_dtype {
+    FA_DTYPE_F32 = 0, FA_DTYPE_F16 = 1, FA_DTYPE_BF16 = 2,
+    FA_DTYPE_I8 = 15, FA_DTYPE_I16 = 16, FA_DTYPE_I32 = 17, FA_DTYPE_U8 = 18, FA_DTYPE_U16 = 19,
+    FA_DTYPE_U32 = 20, FA_DTYPE_F64 = 21
+} fa_dtype;
+
+/* TensorArg (src/types/mod.rs:339-347): buffer + byte offset + dtype + dims + element strides. */
+typedef struct fa_tensor_arg {
+    void *buffer;      /* device pointer; NULL = "no buffer" -> FA_ERR_INPUT_NOT_FOUND */
+    size_t offset;     /* bytes */
+    uint32_t dtype;    /* fa_dtype */
+    uint32_t rank;     /* 0..4 */
+    size_t dims[4];
+    size_t strides[4]; /* elements */
+} fa_tensor_arg;
+
+/* ---------------------------------------------------------------------------------------------
+ * Context = Foundry (src/lib.rs:44-188): device + queue + capture state.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct fa_ctx fa_ctx;
+typedef struct fa_graph fa_graph;
+
+/* Foundry::new (src/lib.rs:57-61). Creates a stream on `device` and a 64 MiB scratch workspace. */
+fa_status fa_ctx_create(int device, fa_ctx **out);
+fa_status fa_ctx_destroy(fa_ctx *ctx);
+/* Foundry::synchronize (src/lib.rs:175-188). */
+fa_status fa_synchronize(fa_ctx *ctx);
+/* The context's hipStream_t, for callers that enqueue their own work between the ops. */
+void *fa_ctx_stream(fa_ctx *ctx);
+/* Grows the scratch workspace to at least `bytes`. Must be called outside a capture; ops that need
+ * more scratch than is reserved while capturing fail with FA_ERR_OPERATION_FAILED. */
+fa_status fa_ctx_reserve_workspace(fa_ctx *ctx, size_t bytes);
+
+/* Foundry::start_capture / end_capture (src/lib.rs:94-164). The reference batches dispatches into one
+ * command buffer and commits it once; here the ops enqueued between the two calls are recorded into a
+ * HIP graph that can be replayed with fa_graph_launch (nothing runs until then). Ops whose position
+ * comes from device memory (the *_dyn and paged entry points) make the recorded graph valid for every
+ * later decode step without patching. */
+fa_status fa_start_capture(fa_ctx *ctx);
+fa_status fa_end_capture(fa_ctx *ctx, fa_graph **out);
+fa_status fa_graph_launch(fa_ctx *ctx, fa_graph *graph);
+fa_status fa_graph_destroy(fa_graph *graph);
+int fa_is_capturing(fa_ctx *ctx); /* Foundry::is_capturing (src/lib.rs:308) */
+
+/* Per-kernel timing, the counterpart of METALLIC_FOUNDRY_PER_KERNEL_PROFILING (src/lib.rs:214-222,
+ * src/instrument.rs:97-124): while enabled every dispatch is bracketed by two HIP events on the
+ * context's stream (not allowed while capturing). fa_profile_query synchronises, then reports
+ * launches and summed device milliseconds for kernels whose name starts with `kernel_prefix`. */
+fa_status fa_profile_enable(fa_ctx *ctx, int on);
+fa_status fa_profile_reset(fa_ctx *ctx);
+fa_status fa_profile_query(fa_ctx *ctx, const char *kernel_prefix, uint64_t *launches, double *total_ms);
+
+/* Device memory, the executor's buffer management (src/model/executor.rs:2286-2328, src/lib.rs:317-377).
+ * fa_upload/fa_download are synchronous with respect to the context's stream. */
+fa_status fa_device_alloc(fa_ctx *ctx, size_t bytes, void **out);
+fa_status fa_device_free(fa_ctx *ctx, void *ptr);
+fa_status fa_upload(fa_ctx *ctx, void *dst, size_t dst_offset, const void *src_host, size_t bytes);
+fa_status fa_download(fa_ctx *ctx, void *dst_host, const void *src, size_t src_offset, size_t bytes);
+fa_status fa_device_memset(fa_ctx *ctx, void *dst, int value, size_t bytes);
+/* Foundry::blit_copy (src/lib.rs:317-336), asynchronous on the stream. */
+fa_status fa_device_copy(fa_ctx *ctx, void *dst, size_t dst_offset, const void *src, size_t src_offset, size_t bytes);
+/* values[i] += delta for i < n, on the stream: advances device-side positions / sequence lengths. */
+fa_status fa_u32_add(fa_ctx *ctx, uint32_t *d_values, uint32_t n, uint32_t delta);
+
+/* ---------------------------------------------------------------------------------------------
+ * RoPE tables, host side: ensure_rope_capacity_named (src/model/executor.rs:1977-2029).
+ * inv_freq[i] = 1/powf(base, 2i/D) (/ freq_factors[i]); angle = p*inv_freq; cos/sin in f32 -> f16.
+ * Fills rows [pos_begin, pos_end) of [*, head_dim/2] host buffers (row 0 of the output = pos_begin).
+ * ------------------------------------------------------------------------------------------- */
+fa_status fa_rope_tables_f16(float rope_base, uint32_t head_dim, uint32_t pos_begin, uint32_t pos_end,
+                             const float *freq_factors /* nullable, head_dim/2 */, uint16_t *cos_out_host,
+                             uint16_t *sin_out_host);
+
+/* ---------------------------------------------------------------------------------------------
+ * KvPrepFused: fused RoPE(Q) + RoPE(K) + head-major rearrange + KV-cache append.
+ * ------------------------------------------------------------------------------------------- */
+
+/* KvPrepFusedParamsResolved: 13 x u32 in the reference's order (src/metals/kv_prep/mod.rs:79-114). */
+typedef struct fa_kv_prep_fused_params {
+    uint32_t d_model;            /* n_heads * head_dim */
+    uint32_t kv_dim;             /* n_kv_heads * head_dim */
+    uint32_t head_dim;           /* even */
+    uint32_t n_heads;
+    uint32_t n_kv_heads;
+    uint32_t group_size;         /* n_heads / n_kv_heads */
+    uint32_t seq_len;            /* tokens in this call */
+    uint32_t position_offset;    /* first cache / RoPE-table row */
+    uint32_t max_seq_len;        /* cache capacity (row stride of a head) */
+    uint32_t total_elements;     /* n_heads * seq_len * head_dim */
+    uint32_t rope_mode;          /* 0 = neox (pair i with i + D/2), 1 = normal (pair 2i with 2i+1) */
+    uint32_t layer_idx;          /* 0-based */
+    uint32_t no_rope_layer_step; /* >0: skip RoPE when (layer_idx + 1) % step == 0 */
+} fa_kv_prep_fused_params;
+
+#define FA_ROPE_MODE_NEOX 0u
+#define FA_ROPE_MODE_NORMAL 1u
+
+/* The KvPrepFused kernel (src/metals/kv_prep/mod.rs:157-182, kv_prep_fused.metal:26-123), as dispatched by
+ * CompiledKvPrepFusedStep::execute (src/metals/kv_prep/step.rs:92-130).
+ *   q [seq_len, d_model], k/v [seq_len, kv_dim] token-major; q_rot [n_heads, seq_len, head_dim] packed;
+ *   k_cache/v_cache [n_kv_heads, max_seq_len, head_dim]; cos/sin [>= position_offset+seq_len, head_dim/2].
+ * Errors: missing buffer -> INPUT_NOT_FOUND; non-f16 -> UNSUPPORTED_DTYPE; odd head_dim, n_heads not a
+ * multiple of n_kv_heads, inconsistent derived fields -> INVALID_SHAPE; position_offset + seq_len >
+ * max_seq_len -> INVALID_OPERATION. */
+fa_status fa_kv_prep_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                           const fa_tensor_arg *q_rot, const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
+                           const fa_tensor_arg *cos, const fa_tensor_arg *sin, const fa_kv_prep_fused_params *params);
+
+/* Same op with the position read from device memory at execution time: row = *d_position_offset + s
+ * (params->position_offset is ignored). The reference re-encodes the scalar every step
+ * (src/types/mod.rs:553-559); a recorded HIP graph cannot, so the scalar lives on the device. Rows that
+ * would land at or beyond max_seq_len are not written. */
+fa_status fa_kv_prep_fused_dyn(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                               const fa_tensor_arg *q_rot, const fa_tensor_arg *k_cache,
+                               const fa_tensor_arg *v_cache, const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                               const fa_kv_prep_fused_params *params, const uint32_t *d_position_offset);
+
+/* ---------------------------------------------------------------------------------------------
+ * FlashAttention: the DSL op (src/metals/sdpa/step.rs:21-38) and its router (:160-503).
+ * ------------------------------------------------------------------------------------------- */
+
+/* CompiledFlashAttentionStep::execute. Arguments are FlashAttentionStep's fields after
+ * DynamicValue::resolve. K/V are the head-major cache [n_kv_heads, capacity, head_dim] (rank 3) or
+ * [batch, n_kv_heads, capacity, head_dim] (rank 4, batch must be 1).
+ *   m <= 1 : decode. q is q_rot, read as head-major [n_heads, 1, head_dim] whatever its metadata says
+ *            (src/metals/flashattention/step.rs:1005-1020); out is [n_heads*head_dim]. All kv_seq_len
+ *            keys are attended (the reference takes this path when !causal or query_offset+1 == kv_seq_len).
+ *   m  > 1 : prefill. Q / out layouts are inferred from dims+strides by the reference's rules
+ *            (src/metals/flashattention/step.rs:648-756), including "token-major metadata, head-major
+ *            contents" for q. Mask: key j visible to row r iff !causal or j <= query_offset + r.
+ * Differences from the reference, by design: there is no materialized fallback; the cases the reference
+ * routes to it (non-causal prefill, causal offset mismatch, src/metals/sdpa/step.rs:442-502) run on the
+ * same flash kernels with the mask above, and keep the GQA head map the fallback lacks.
+ * Errors: kv_head_major == 0 -> OPERATION_NOT_SUPPORTED (src/metals/sdpa/step.rs:193-197); head_dim not in
+ * {64,128} -> OPERATION_NOT_SUPPORTED (src/metals/flashattention/step.rs:616-627,986-991); unsupported
+ * layout -> OPERATION_NOT_SUPPORTED; kv_seq_len == 0 or > capacity -> INVALID_SHAPE. */
+fa_status fa_flash_attention(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                             const fa_tensor_arg *output, int causal, uint32_t query_offset, uint32_t n_heads,
+                             uint32_t head_dim, uint32_t kv_seq_len, uint32_t m, int kv_head_major);
+
+/* Decode with kv_seq_len = *d_position + kv_len_add read on the device (see fa_kv_prep_fused_dyn).
+ * kv_len_bound >= every kv_seq_len the recorded call will see (sizes the launch grid); a length that
+ * exceeds it or the cache capacity is clamped. */
+fa_status fa_flash_decode_dyn(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                              const fa_tensor_arg *output, uint32_t n_heads, uint32_t head_dim,
+                              const uint32_t *d_position, uint32_t kv_len_add, uint32_t kv_len_bound);
+
+/* Tuning override, the counterpart of FlashDecodeVariant + METALLIC_FA_DECODE_* (src/metals/flashattention/
+ * variants.rs:36-140). keys_per_split: context partition per workgroup (multiple of 64; 0 = auto).
+ * merge: 0 = merged by the last workgroup to finish (one launch), 1 = separate merge kernel.
+ * Environment: FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT, FOUNDRY_ATTN_DECODE_MERGE (read at fa_ctx_create). */
+typedef struct fa_decode_variant {
+    uint32_t keys_per_split;
+    uint32_t merge;
+} fa_decode_variant;
+fa_status fa_set_decode_variant(fa_ctx *ctx, const fa_decode_variant *variant);
+
+/* ---------------------------------------------------------------------------------------------
+ * Paged KV cache (no counterpart in the reference, whose cache is contiguous per layer and batch 1:
+ * models/llama.json:301-330). Contract: gathering a sequence's blocks in block-table order yields,
+ * byte for byte, the contiguous cache the reference would hold after the same appends.
+ *   pools        [n_blocks, n_kv_heads, block_size, head_dim] f16 (one pool pair per layer)
+ *   block_table  [n_seqs, max_blocks_per_seq] i32 physical block ids (device memory)
+ *   seq_lens     [n_seqs] u32 tokens currently stored per sequence (device memory)
+ * ------------------------------------------------------------------------------------------- */
+typedef struct fa_paged_kv {
+    void *k_pool;
+    void *v_pool;
+    const int32_t *block_table;
+    const uint32_t *seq_lens;
+    uint32_t n_blocks;
+    uint32_t n_kv_heads;
+    uint32_t block_size; /* multiple of 16 */
+    uint32_t head_dim;   /* 64 or 128 */
+    uint32_t n_seqs;
+    uint32_t max_blocks_per_seq;
+} fa_paged_kv;
+
+/* KvPrepFused into a paged cache, one sequence (`seq_index`), params->seq_len tokens at rows
+ * params->position_offset.. (params->max_seq_len is ignored; capacity = max_blocks_per_seq*block_size).
+ * q_rot is [n_heads, seq_len, head_dim] as in fa_kv_prep_fused. Does not modify seq_lens. */
+fa_status fa_kv_prep_fused_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                 const fa_tensor_arg *v, const fa_tensor_arg *q_rot, const fa_paged_kv *cache,
+                                 uint32_t seq_index, const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                 const fa_kv_prep_fused_params *params);
+
+/* Batched decode append: one new token for each of cache->n_seqs sequences. Token b comes from row b of
+ * q/k/v ([n_seqs, d_model] / [n_seqs, kv_dim]) and lands at row seq_lens[b] of sequence b (read on the
+ * device). q_rot is [n_seqs, n_heads, head_dim]. params->seq_len must equal n_seqs. Does not modify
+ * seq_lens (advance them with fa_u32_add after the layer loop). */
+fa_status fa_kv_prep_decode_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                  const fa_tensor_arg *v, const fa_tensor_arg *q_rot, const fa_paged_kv *cache,
+                                  const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                  const fa_kv_prep_fused_params *params);
+
+/* Batched ragged flash decode over a paged cache: sequence b attends rows [0, seq_lens[b] + kv_len_add).
+ * q [n_seqs, n_heads, head_dim], out [n_seqs, n_heads*head_dim]. kv_len_bound as in fa_flash_decode_dyn. */
+fa_status fa_flash_decode_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_paged_kv *cache,
+                                const fa_tensor_arg *output, uint32_t n_heads, uint32_t kv_len_add,
+                                uint32_t kv_len_bound);
+
+/* Causal flash prefill for one sequence reading K/V through the block table. q is head-major
+ * [n_heads, m, head_dim]; out token-major [m, n_heads*head_dim]. Mask as in fa_flash_attention. */
+fa_status fa_flash_prefill_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_paged_kv *cache, uint32_t seq_index,
+                                 const fa_tensor_arg *output, int causal, uint32_t query_offset, uint32_t n_heads,
+                                 uint32_t kv_seq_len, uint32_t m);
+
+/* Copies rows [0, seq_len) of one sequence out of the pools into contiguous [n_kv_heads, out_capacity,
+ * head_dim] buffers (the layout of the reference's cache; also the paged form of the executor's
+ * per-head prefix snapshot, src/model/executor.rs:1136-1350). */
+fa_status fa_paged_gather(fa_ctx *ctx, const fa_paged_kv *cache, uint32_t seq_index, uint32_t seq_len,
+                          void *k_out, void *v_out, uint32_t out_capacity);
+
+/* ---------------------------------------------------------------------------------------------
+ * SageAttention-style int8 Q/K decode (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170 - prose only in
+ * the reference). K is mean-smoothed over the sequence per (kv head, channel), then quantised per block
+ * of 32 tokens: scale = max|k - mean| / 127 stored as f16, k_q = rint((k - mean)/scale) in [-127,127].
+ * Q is quantised per head with one f32 scale. V stays f16.
+ * ------------------------------------------------------------------------------------------- */
+#define FA_SAGE_BLOCK 32u
+/* mean [n_kv_heads, head_dim] f32 over rows [0, kv_len) of k [n_kv_heads, capacity, head_dim]. */
+fa_status fa_sage_k_mean(fa_ctx *ctx, const void *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim,
+                         uint32_t kv_len, float *mean_out);
+/* Quantises rows [row_begin, row_end) (row_begin a multiple of 32) into k_q [n_kv_heads, capacity, head_dim]
+ * i8 and k_scale [n_kv_heads, ceil(capacity/32)] f16. */
+fa_status fa_sage_quantize_k(fa_ctx *ctx, const void *k, const float *mean, uint32_t n_kv_heads, uint32_t capacity,
+                             uint32_t head_dim, uint32_t row_begin, uint32_t row_end, void *k_q, void *k_scale);
+/* q [n_heads, head_dim] f16 -> q_q i8 + q_scale [n_heads] f32. */
+fa_status fa_sage_quantize_q(fa_ctx *ctx, const void *q, uint32_t n_heads, uint32_t head_dim, void *q_q,
+                             float *q_scale);
+/* out [n_heads*head_dim] f16 = softmax(scale * q_scale*k_scale * (q_q . k_q)) V over kv_len keys. */
+fa_status fa_sage_decode(fa_ctx *ctx, const void *q_q, const float *q_scale, const void *k_q, const void *k_scale,
+                         const void *v, void *out, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
+                         uint32_t capacity, uint32_t kv_len);
+
+/* Library / device facts for harnesses. */
+const char *fa_version(void);
+fa_status fa_device_info(fa_ctx *ctx, char *name_out, size_t name_cap, uint32_t *compute_units,
+                         uint64_t *global_mem_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FOUNDRY_ATTN_H */

@@ -1,0 +1,53 @@
+"""Builds libfoundry_attn.so (HIP, gfx950 only) next to this file.
+
+    python test-burn_amd/build.py            # incremental: recompiles sources newer than their objects
+    python test-burn_amd/build.py --force    # recompile everything
+
+hipcc cross-compiles without a GPU. Packed-FP32 code generation is disabled for all device code.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
+LIB = os.path.join(HERE, "libfoundry_attn.so")
+SOURCES = ["fa_api.hip", "fa_kvprep.hip", "fa_decode.hip", "fa_prefill.hip", "fa_sage.hip"]
+HEADERS = [os.path.join(CSRC, "fa_internal.h"), os.path.join(HERE, "..", "include", "foundry_attn.h")]
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Wall", "-Wno-unused-function",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _stale(src, obj):
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    return any(os.path.getmtime(p) > t for p in [src] + HEADERS)
+
+
+def _compile(name, force):
+    src = os.path.join(CSRC, name)
+    obj = os.path.join(OBJ, name.replace(".hip", ".o"))
+    if force or _stale(src, obj):
+        subprocess.check_call([HIPCC] + FLAGS + ["-c", src, "-o", obj])
+        return True
+    return False
+
+
+def build(force=False, verbose=True):
+    os.makedirs(OBJ, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
+        changed = list(ex.map(lambda n: _compile(n, force), SOURCES))
+    objs = [os.path.join(OBJ, n.replace(".hip", ".o")) for n in SOURCES]
+    if any(changed) or not os.path.exists(LIB):
+        subprocess.check_call([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs)
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build(force="--force" in sys.argv)

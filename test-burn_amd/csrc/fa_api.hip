@@ -1,0 +1,923 @@
+// Host side of libfoundry_attn: context, errors, argument validation, layout inference and routing.
+// Mirrors, for the attention path only, Foundry (crates/metallic-foundry/src/lib.rs:44-305) and the two
+// compiled steps CompiledKvPrepFusedStep (src/metals/kv_prep/step.rs:92-130) and
+// CompiledFlashAttentionStep (src/metals/sdpa/step.rs:160-503, src/metals/flashattention/step.rs:614-1086).
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+
+#include "fa_internal.h"
+
+// ------------------------------------------------------------------------------------------------ errors
+
+static thread_local char g_err[1024] = "";
+
+fa_status fa_fail(fa_status s, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return s;
+}
+
+extern "C" const char *fa_last_error_string(void) { return g_err; }
+
+extern "C" const char *fa_status_name(fa_status s) {
+    switch (s) {
+        case FA_OK: return "Ok";
+        case FA_ERR_DEVICE_NOT_FOUND: return "DeviceNotFound";
+        case FA_ERR_NULL_POINTER: return "NullPointer";
+        case FA_ERR_INVALID_SHAPE: return "InvalidShape";
+        case FA_ERR_OUT_OF_MEMORY: return "OutOfMemory";
+        case FA_ERR_OPERATION_NOT_SUPPORTED: return "OperationNotSupported";
+        case FA_ERR_INVALID_OPERATION: return "InvalidOperation";
+        case FA_ERR_UNSUPPORTED_DTYPE: return "UnsupportedDtype";
+        case FA_ERR_OPERATION_FAILED: return "OperationFailed";
+        case FA_ERR_INPUT_NOT_FOUND: return "InputNotFound";
+    }
+    return "Unknown";
+}
+
+extern "C" const char *fa_version(void) { return "foundry_attn 0.1 (gfx950)"; }
+
+// ------------------------------------------------------------------------------------------------ profiling scope
+
+FaLaunchScope::FaLaunchScope(fa_ctx *c, const char *n) : ctx(c), name(n) {
+    if (!ctx->profiling || ctx->capturing) return;
+    auto get = [&]() -> hipEvent_t {
+        if (!ctx->event_pool.empty()) {
+            hipEvent_t e = ctx->event_pool.back();
+            ctx->event_pool.pop_back();
+            return e;
+        }
+        hipEvent_t e = nullptr;
+        if (hipEventCreate(&e) != hipSuccess) return nullptr;
+        return e;
+    };
+    start = get();
+    stop = get();
+    if (start) (void)hipEventRecord(start, ctx->stream);
+}
+
+fa_status FaLaunchScope::finish() {
+    hipError_t e = hipGetLastError();
+    if (start && stop) {
+        (void)hipEventRecord(stop, ctx->stream);
+        ctx->prof.push_back({name, start, stop});
+    }
+    if (e != hipSuccess) return fa_fail(FA_ERR_OPERATION_FAILED, "launch of %s failed: %s", name, hipGetErrorString(e));
+    return FA_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ context
+
+#define FA_NEED(p, what)                                                        \
+    do {                                                                        \
+        if (!(p)) return fa_fail(FA_ERR_NULL_POINTER, "%s is null", what);     \
+    } while (0)
+
+static uint32_t env_u32(const char *key, uint32_t dflt) {
+    const char *s = getenv(key);
+    if (!s || !*s) return dflt;
+    char *end = nullptr;
+    unsigned long v = strtoul(s, &end, 10);
+    return (end && *end == 0) ? (uint32_t)v : dflt;
+}
+
+extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
+    FA_NEED(out, "out");
+    *out = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0 || device < 0 || device >= n)
+        return fa_fail(FA_ERR_DEVICE_NOT_FOUND, "Device not found (device %d of %d)", device, n);
+    FA_HIP(hipSetDevice(device));
+    fa_ctx *ctx = new fa_ctx();
+    ctx->device = device;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess) ctx->n_cus = prop.multiProcessorCount;
+    hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        delete ctx;
+        return fa_fail(FA_ERR_OPERATION_FAILED, "hipStreamCreate failed: %s", hipGetErrorString(e));
+    }
+    ctx->decode_variant.keys_per_split = env_u32("FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT", 0);
+    ctx->decode_variant.merge = env_u32("FOUNDRY_ATTN_DECODE_MERGE", 0);
+    fa_status s = fa_ensure_workspace(ctx, (size_t)64 << 20);
+    if (s == FA_OK) s = fa_ensure_counters(ctx, 4096);
+    if (s != FA_OK) {
+        fa_ctx_destroy(ctx);
+        return s;
+    }
+    *out = ctx;
+    return FA_OK;
+}
+
+extern "C" fa_status fa_ctx_destroy(fa_ctx *ctx) {
+    if (!ctx) return FA_OK;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    for (auto &r : ctx->prof) {
+        (void)hipEventDestroy(r.start);
+        (void)hipEventDestroy(r.stop);
+    }
+    for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
+    if (ctx->workspace) (void)hipFree(ctx->workspace);
+    if (ctx->counters) (void)hipFree(ctx->counters);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return FA_OK;
+}
+
+extern "C" void *fa_ctx_stream(fa_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+extern "C" fa_status fa_synchronize(fa_ctx *ctx) {
+    FA_NEED(ctx, "ctx");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "cannot synchronize while a capture is active");
+    FA_HIP(hipStreamSynchronize(ctx->stream));
+    return FA_OK;
+}
+
+fa_status fa_ensure_workspace(fa_ctx *ctx, size_t bytes) {
+    if (bytes <= ctx->workspace_bytes) return FA_OK;
+    if (ctx->capturing)
+        return fa_fail(FA_ERR_OPERATION_FAILED,
+                       "scratch workspace of %zu bytes needed during capture but only %zu reserved; call "
+                       "fa_ctx_reserve_workspace before fa_start_capture",
+                       bytes, ctx->workspace_bytes);
+    FA_HIP(hipStreamSynchronize(ctx->stream));
+    if (ctx->workspace) FA_HIP(hipFree(ctx->workspace));
+    ctx->workspace = nullptr;
+    ctx->workspace_bytes = 0;
+    size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+    FA_HIP(hipMalloc(&ctx->workspace, want));
+    ctx->workspace_bytes = want;
+    return FA_OK;
+}
+
+fa_status fa_ensure_counters(fa_ctx *ctx, uint32_t n) {
+    if (n <= ctx->n_counters) return FA_OK;
+    if (ctx->capturing)
+        return fa_fail(FA_ERR_OPERATION_FAILED, "%u split counters needed during capture but only %u exist", n,
+                       ctx->n_counters);
+    FA_HIP(hipStreamSynchronize(ctx->stream));
+    if (ctx->counters) FA_HIP(hipFree(ctx->counters));
+    ctx->counters = nullptr;
+    ctx->n_counters = 0;
+    uint32_t want = (n + 4095u) & ~4095u;
+    FA_HIP(hipMalloc((void **)&ctx->counters, (size_t)want * sizeof(uint32_t)));
+    FA_HIP(hipMemset(ctx->counters, 0, (size_t)want * sizeof(uint32_t)));
+    ctx->n_counters = want;
+    return FA_OK;
+}
+
+extern "C" fa_status fa_ctx_reserve_workspace(fa_ctx *ctx, size_t bytes) {
+    FA_NEED(ctx, "ctx");
+    return fa_ensure_workspace(ctx, bytes);
+}
+
+extern "C" fa_status fa_set_decode_variant(fa_ctx *ctx, const fa_decode_variant *v) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(v, "variant");
+    if (v->keys_per_split % 64 != 0)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "decode keys_per_split must be a multiple of 64 (or 0), got %u",
+                       v->keys_per_split);
+    if (v->merge > 1) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "decode merge must be 0 or 1, got %u", v->merge);
+    ctx->decode_variant = *v;
+    return FA_OK;
+}
+
+// capture ---------------------------------------------------------------------------------------
+
+extern "C" int fa_is_capturing(fa_ctx *ctx) { return ctx && ctx->capturing ? 1 : 0; }
+
+extern "C" fa_status fa_start_capture(fa_ctx *ctx) {
+    FA_NEED(ctx, "ctx");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "Capture already active");
+    if (ctx->profiling) return fa_fail(FA_ERR_OPERATION_FAILED, "per-kernel profiling cannot be combined with capture");
+    FA_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    ctx->capturing = true;
+    return FA_OK;
+}
+
+extern "C" fa_status fa_end_capture(fa_ctx *ctx, fa_graph **out) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(out, "out");
+    *out = nullptr;
+    if (!ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "No active capture");
+    ctx->capturing = false;
+    hipGraph_t g = nullptr;
+    FA_HIP(hipStreamEndCapture(ctx->stream, &g));
+    hipGraphExec_t ex = nullptr;
+    hipError_t e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(g);
+        return fa_fail(FA_ERR_OPERATION_FAILED, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    }
+    fa_graph *gr = new fa_graph();
+    gr->graph = g;
+    gr->exec = ex;
+    *out = gr;
+    return FA_OK;
+}
+
+extern "C" fa_status fa_graph_launch(fa_ctx *ctx, fa_graph *graph) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(graph, "graph");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "cannot launch a graph while a capture is active");
+    FA_HIP(hipGraphLaunch(graph->exec, ctx->stream));
+    return FA_OK;
+}
+
+extern "C" fa_status fa_graph_destroy(fa_graph *graph) {
+    if (!graph) return FA_OK;
+    if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+    if (graph->graph) (void)hipGraphDestroy(graph->graph);
+    delete graph;
+    return FA_OK;
+}
+
+// profiling -------------------------------------------------------------------------------------
+
+static void prof_recycle(fa_ctx *ctx) {
+    for (auto &r : ctx->prof) {
+        ctx->event_pool.push_back(r.start);
+        ctx->event_pool.push_back(r.stop);
+    }
+    ctx->prof.clear();
+}
+
+extern "C" fa_status fa_profile_enable(fa_ctx *ctx, int on) {
+    FA_NEED(ctx, "ctx");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "per-kernel profiling cannot be combined with capture");
+    ctx->profiling = on != 0;
+    return FA_OK;
+}
+
+extern "C" fa_status fa_profile_reset(fa_ctx *ctx) {
+    FA_NEED(ctx, "ctx");
+    FA_HIP(hipStreamSynchronize(ctx->stream));
+    prof_recycle(ctx);
+    return FA_OK;
+}
+
+extern "C" fa_status fa_profile_query(fa_ctx *ctx, const char *prefix, uint64_t *launches, double *total_ms) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(prefix, "kernel_prefix");
+    FA_HIP(hipStreamSynchronize(ctx->stream));
+    uint64_t n = 0;
+    double ms = 0.0;
+    const size_t plen = strlen(prefix);
+    for (auto &r : ctx->prof) {
+        if (strncmp(r.name, prefix, plen) != 0) continue;
+        float t = 0.0f;
+        FA_HIP(hipEventElapsedTime(&t, r.start, r.stop));
+        ms += t;
+        ++n;
+    }
+    if (launches) *launches = n;
+    if (total_ms) *total_ms = ms;
+    return FA_OK;
+}
+
+// memory ----------------------------------------------------------------------------------------
+
+extern "C" fa_status fa_device_alloc(fa_ctx *ctx, size_t bytes, void **out) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(out, "out");
+    *out = nullptr;
+    if (bytes == 0) bytes = 16;
+    hipError_t e = hipMalloc(out, bytes);
+    if (e != hipSuccess) return fa_fail(FA_ERR_OUT_OF_MEMORY, "Buffer creation failed with size %zu: %s", bytes, hipGetErrorString(e));
+    return FA_OK;
+}
+
+extern "C" fa_status fa_device_free(fa_ctx *ctx, void *ptr) {
+    FA_NEED(ctx, "ctx");
+    if (!ptr) return FA_OK;
+    FA_HIP(hipStreamSynchronize(ctx->stream));
+    FA_HIP(hipFree(ptr));
+    return FA_OK;
+}
+
+extern "C" fa_status fa_upload(fa_ctx *ctx, void *dst, size_t dst_offset, const void *src_host, size_t bytes) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(dst, "dst");
+    FA_NEED(src_host, "src_host");
+    if (bytes == 0) return FA_OK;
+    FA_HIP(hipMemcpyAsync((char *)dst + dst_offset, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    FA_HIP(hipStreamSynchronize(ctx->stream));
+    return FA_OK;
+}
+
+extern "C" fa_status fa_download(fa_ctx *ctx, void *dst_host, const void *src, size_t src_offset, size_t bytes) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(dst_host, "dst_host");
+    FA_NEED(src, "src");
+    if (bytes == 0) return FA_OK;
+    FA_HIP(hipMemcpyAsync(dst_host, (const char *)src + src_offset, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    FA_HIP(hipStreamSynchronize(ctx->stream));
+    return FA_OK;
+}
+
+extern "C" fa_status fa_device_memset(fa_ctx *ctx, void *dst, int value, size_t bytes) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(dst, "dst");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "fa_device_memset is not recordable; clear buffers before the capture");
+    if (bytes == 0) return FA_OK;
+    FA_HIP(hipMemsetAsync(dst, value, bytes, ctx->stream));
+    return FA_OK;
+}
+
+extern "C" fa_status fa_device_copy(fa_ctx *ctx, void *dst, size_t dst_offset, const void *src, size_t src_offset,
+                                    size_t bytes) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(dst, "dst");
+    FA_NEED(src, "src");
+    if (bytes == 0) return FA_OK;
+    FA_HIP(hipMemcpyAsync((char *)dst + dst_offset, (const char *)src + src_offset, bytes, hipMemcpyDeviceToDevice,
+                          ctx->stream));
+    return FA_OK;
+}
+
+extern "C" fa_status fa_u32_add(fa_ctx *ctx, uint32_t *d_values, uint32_t n, uint32_t delta) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(d_values, "d_values");
+    return fa_launch_u32_add(ctx, d_values, n, delta);
+}
+
+extern "C" fa_status fa_device_info(fa_ctx *ctx, char *name_out, size_t name_cap, uint32_t *compute_units,
+                                    uint64_t *global_mem_bytes) {
+    FA_NEED(ctx, "ctx");
+    hipDeviceProp_t prop;
+    FA_HIP(hipGetDeviceProperties(&prop, ctx->device));
+    if (name_out && name_cap) {
+        snprintf(name_out, name_cap, "%s (%s)", prop.name, prop.gcnArchName);
+    }
+    if (compute_units) *compute_units = (uint32_t)prop.multiProcessorCount;
+    if (global_mem_bytes) *global_mem_bytes = (uint64_t)prop.totalGlobalMem;
+    return FA_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ RoPE tables
+
+// f32 -> f16, IEEE round-to-nearest-even (what half::f16::from_f32 does on the reference's host side).
+static uint16_t f32_to_f16_rne(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    x &= 0x7fffffffu;
+    if (x >= 0x7f800000u) return (uint16_t)(sign | 0x7c00u | ((x & 0x007fffffu) ? 0x0200u : 0u));
+    if (x >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);
+    if (x < 0x33000001u) return (uint16_t)sign;
+    const int e = (int)(x >> 23) - 127;
+    uint32_t man = (x & 0x007fffffu) | 0x00800000u;
+    uint32_t shift = 13, base = 0;
+    if (e < -14) {
+        shift = (uint32_t)(-1 - e);
+    } else {
+        base = (uint32_t)(e + 15) << 10;
+        man &= 0x007fffffu;
+    }
+    uint32_t r = base + (man >> shift);
+    const uint32_t rem = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (r & 1u))) ++r;
+    return (uint16_t)(sign | r);
+}
+
+extern "C" fa_status fa_rope_tables_f16(float rope_base, uint32_t head_dim, uint32_t pos_begin, uint32_t pos_end,
+                                        const float *freq_factors, uint16_t *cos_out, uint16_t *sin_out) {
+    FA_NEED(cos_out, "cos_out_host");
+    FA_NEED(sin_out, "sin_out_host");
+    if (head_dim == 0 || head_dim % 2 != 0) return fa_fail(FA_ERR_INVALID_SHAPE, "head_dim must be even, got %u", head_dim);
+    if (pos_end < pos_begin) return fa_fail(FA_ERR_INVALID_SHAPE, "pos_end %u < pos_begin %u", pos_end, pos_begin);
+    const uint32_t dim_half = head_dim / 2;
+    std::vector<float> inv(dim_half);
+    for (uint32_t i = 0; i < dim_half; ++i) {
+        const float exponent = (float)(2 * i) / (float)head_dim;
+        float f = 1.0f / powf(rope_base, exponent);
+        if (freq_factors) f /= freq_factors[i];
+        inv[i] = f;
+    }
+    for (uint32_t p = pos_begin; p < pos_end; ++p)
+        for (uint32_t i = 0; i < dim_half; ++i) {
+            const float angle = (float)p * inv[i];
+            const size_t idx = (size_t)(p - pos_begin) * dim_half + i;
+            cos_out[idx] = f32_to_f16_rne(cosf(angle));
+            sin_out[idx] = f32_to_f16_rne(sinf(angle));
+        }
+    return FA_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ tensor helpers
+
+static size_t numel(const fa_tensor_arg *t) {
+    if (t->rank == 0) return 0;  // unknown extent: metadata-free buffer
+    size_t n = 1;
+    for (uint32_t i = 0; i < t->rank; ++i) n *= t->dims[i];
+    return n;
+}
+
+static fa_status check_tensor(const fa_tensor_arg *t, const char *name, fa_dtype want, size_t need_elems, int align) {
+    if (!t) return fa_fail(FA_ERR_NULL_POINTER, "tensor argument '%s' is null", name);
+    if (!t->buffer) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: %s", name);
+    if (t->rank > 4) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %s has rank %u > 4", name, t->rank);
+    if (t->dtype != (uint32_t)want)
+        return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "Unsupported dtype %u for %s (expected %u)", t->dtype, name, (unsigned)want);
+    if (t->rank > 0 && numel(t) < need_elems)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %s holds %zu elements, %zu needed", name, numel(t), need_elems);
+    if (align > 1 && (((uintptr_t)t->buffer + t->offset) % (size_t)align) != 0)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "%s must be %d-byte aligned (buffer + offset)", name, align);
+    return FA_OK;
+}
+
+template <typename T>
+static T *tptr(const fa_tensor_arg *t) {
+    return reinterpret_cast<T *>((char *)t->buffer + t->offset);
+}
+
+// ------------------------------------------------------------------------------------------------ KvPrepFused
+
+static fa_status check_kv_prep_params(const fa_kv_prep_fused_params *p) {
+    FA_NEED(p, "params");
+    if (p->head_dim == 0 || p->head_dim % 2 != 0)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: head_dim must be even for RoPE, got %u", p->head_dim);
+    if (p->n_heads == 0 || p->n_kv_heads == 0 || p->n_heads % p->n_kv_heads != 0)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_heads %u must be a multiple of n_kv_heads %u", p->n_heads,
+                       p->n_kv_heads);
+    if (p->group_size != p->n_heads / p->n_kv_heads)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: group_size %u != n_heads/n_kv_heads %u", p->group_size,
+                       p->n_heads / p->n_kv_heads);
+    if (p->d_model != p->n_heads * p->head_dim || p->kv_dim != p->n_kv_heads * p->head_dim)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: d_model %u / kv_dim %u inconsistent with heads x head_dim",
+                       p->d_model, p->kv_dim);
+    if ((uint64_t)p->total_elements != (uint64_t)p->n_heads * p->seq_len * p->head_dim)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: total_elements %u != n_heads*seq_len*head_dim", p->total_elements);
+    if (p->rope_mode > 1) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "rope_mode must be 0 (neox) or 1 (normal), got %u", p->rope_mode);
+    return FA_OK;
+}
+
+static fa_status kv_prep_common(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                                const fa_tensor_arg *q_rot, const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                const fa_kv_prep_fused_params *p, KvPrepLaunch &L) {
+    FA_NEED(ctx, "ctx");
+    FA_TRY(check_kv_prep_params(p));
+    const int al = p->head_dim % 16 == 0 ? 16 : 2;
+    const size_t nq = (size_t)p->seq_len * p->d_model, nkv = (size_t)p->seq_len * p->kv_dim;
+    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, nq, al));
+    FA_TRY(check_tensor(k, "k", FA_DTYPE_F16, nkv, al));
+    FA_TRY(check_tensor(v, "v", FA_DTYPE_F16, nkv, al));
+    FA_TRY(check_tensor(q_rot, "q_rot", FA_DTYPE_F16, nq, al));
+    FA_TRY(check_tensor(cos, "cos", FA_DTYPE_F16, 0, al));
+    FA_TRY(check_tensor(sin, "sin", FA_DTYPE_F16, 0, al));
+    const uint32_t half = p->head_dim / 2;
+    size_t rows = numel(cos) / half;
+    const size_t rows_s = numel(sin) / half;
+    if (rows_s < rows) rows = rows_s;
+    if (cos->rank == 0 || sin->rank == 0) rows = 0xffffffffu;  // metadata-free tables: trust the caller
+    if (rows == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: empty RoPE tables");
+    L.q = tptr<const __half>(q), L.k = tptr<const __half>(k), L.v = tptr<const __half>(v);
+    L.q_rot = tptr<__half>(q_rot);
+    L.cos_t = tptr<const __half>(cos), L.sin_t = tptr<const __half>(sin);
+    L.p = *p;
+    L.d_position = nullptr, L.block_table = nullptr, L.seq_lens = nullptr;
+    L.bt_stride = 0, L.block_size = 1;
+    L.table_rows = (uint32_t)(rows > 0xffffffffu ? 0xffffffffu : rows);
+    return FA_OK;
+}
+
+static fa_status kv_prep_contig(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                                const fa_tensor_arg *q_rot, const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
+                                const fa_tensor_arg *cos, const fa_tensor_arg *sin, const fa_kv_prep_fused_params *p,
+                                const uint32_t *d_pos) {
+    KvPrepLaunch L;
+    FA_TRY(kv_prep_common(ctx, q, k, v, q_rot, cos, sin, p, L));
+    const int al = p->head_dim % 16 == 0 ? 16 : 2;
+    const size_t ncache = (size_t)p->n_kv_heads * p->max_seq_len * p->head_dim;
+    FA_TRY(check_tensor(k_cache, "k_cache", FA_DTYPE_F16, ncache, al));
+    FA_TRY(check_tensor(v_cache, "v_cache", FA_DTYPE_F16, ncache, al));
+    if (!d_pos) {
+        if ((uint64_t)p->position_offset + p->seq_len > p->max_seq_len)
+            return fa_fail(FA_ERR_INVALID_OPERATION, "Invalid operation: position_offset %u + seq_len %u exceeds max_seq_len %u",
+                           p->position_offset, p->seq_len, p->max_seq_len);
+        if ((uint64_t)p->position_offset + p->seq_len > L.table_rows)
+            return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: RoPE tables hold %u rows, %u needed", L.table_rows,
+                           p->position_offset + p->seq_len);
+    }
+    L.k_cache = tptr<__half>(k_cache), L.v_cache = tptr<__half>(v_cache);
+    L.mode = 0;
+    L.d_position = d_pos;
+    L.capacity = p->max_seq_len;
+    return fa_launch_kv_prep(ctx, L);
+}
+
+extern "C" fa_status fa_kv_prep_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                      const fa_tensor_arg *v, const fa_tensor_arg *q_rot, const fa_tensor_arg *k_cache,
+                                      const fa_tensor_arg *v_cache, const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                      const fa_kv_prep_fused_params *params) {
+    return kv_prep_contig(ctx, q, k, v, q_rot, k_cache, v_cache, cos, sin, params, nullptr);
+}
+
+extern "C" fa_status fa_kv_prep_fused_dyn(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                          const fa_tensor_arg *v, const fa_tensor_arg *q_rot,
+                                          const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
+                                          const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                          const fa_kv_prep_fused_params *params, const uint32_t *d_position_offset) {
+    FA_NEED(d_position_offset, "d_position_offset");
+    return kv_prep_contig(ctx, q, k, v, q_rot, k_cache, v_cache, cos, sin, params, d_position_offset);
+}
+
+static fa_status check_paged(const fa_paged_kv *c) {
+    FA_NEED(c, "cache");
+    if (!c->k_pool || !c->v_pool) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: paged k_pool / v_pool");
+    if (!c->block_table) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: block_table");
+    if (c->block_size == 0 || c->block_size % 16 != 0)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "paged block_size must be a multiple of 16, got %u", c->block_size);
+    if (!(c->head_dim == 64 || c->head_dim == 128))
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "paged cache supports head_dim=64 or 128, got %u", c->head_dim);
+    if (c->n_seqs == 0 || c->max_blocks_per_seq == 0 || c->n_kv_heads == 0 || c->n_blocks == 0)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: empty paged cache descriptor");
+    if ((((uintptr_t)c->k_pool) | ((uintptr_t)c->v_pool)) % 16 != 0)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "paged pools must be 16-byte aligned");
+    return FA_OK;
+}
+
+extern "C" fa_status fa_kv_prep_fused_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                            const fa_tensor_arg *v, const fa_tensor_arg *q_rot, const fa_paged_kv *cache,
+                                            uint32_t seq_index, const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                            const fa_kv_prep_fused_params *p) {
+    KvPrepLaunch L;
+    FA_TRY(check_paged(cache));
+    FA_TRY(kv_prep_common(ctx, q, k, v, q_rot, cos, sin, p, L));
+    if (p->head_dim != cache->head_dim || p->n_kv_heads != cache->n_kv_heads)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: params (Hkv %u, D %u) do not match the paged cache (Hkv %u, D %u)",
+                       p->n_kv_heads, p->head_dim, cache->n_kv_heads, cache->head_dim);
+    if (seq_index >= cache->n_seqs) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: seq_index %u >= n_seqs %u", seq_index, cache->n_seqs);
+    const uint64_t cap = (uint64_t)cache->max_blocks_per_seq * cache->block_size;
+    if ((uint64_t)p->position_offset + p->seq_len > cap)
+        return fa_fail(FA_ERR_INVALID_OPERATION, "Invalid operation: position_offset %u + seq_len %u exceeds paged capacity %llu",
+                       p->position_offset, p->seq_len, (unsigned long long)cap);
+    if ((uint64_t)p->position_offset + p->seq_len > L.table_rows)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: RoPE tables hold %u rows, %u needed", L.table_rows,
+                       p->position_offset + p->seq_len);
+    L.k_cache = (__half *)cache->k_pool, L.v_cache = (__half *)cache->v_pool;
+    L.mode = 1;
+    L.block_table = cache->block_table + (size_t)seq_index * cache->max_blocks_per_seq;
+    L.bt_stride = cache->max_blocks_per_seq, L.block_size = cache->block_size;
+    L.capacity = (uint32_t)cap;
+    return fa_launch_kv_prep(ctx, L);
+}
+
+extern "C" fa_status fa_kv_prep_decode_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                             const fa_tensor_arg *v, const fa_tensor_arg *q_rot,
+                                             const fa_paged_kv *cache, const fa_tensor_arg *cos,
+                                             const fa_tensor_arg *sin, const fa_kv_prep_fused_params *p) {
+    KvPrepLaunch L;
+    FA_TRY(check_paged(cache));
+    FA_TRY(kv_prep_common(ctx, q, k, v, q_rot, cos, sin, p, L));
+    if (!cache->seq_lens) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: seq_lens");
+    if (p->head_dim != cache->head_dim || p->n_kv_heads != cache->n_kv_heads)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: params (Hkv %u, D %u) do not match the paged cache (Hkv %u, D %u)",
+                       p->n_kv_heads, p->head_dim, cache->n_kv_heads, cache->head_dim);
+    if (p->seq_len != cache->n_seqs)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: batched decode append needs seq_len == n_seqs (%u != %u)",
+                       p->seq_len, cache->n_seqs);
+    L.k_cache = (__half *)cache->k_pool, L.v_cache = (__half *)cache->v_pool;
+    L.mode = 2;
+    L.block_table = cache->block_table, L.seq_lens = cache->seq_lens;
+    L.bt_stride = cache->max_blocks_per_seq, L.block_size = cache->block_size;
+    L.capacity = cache->max_blocks_per_seq * cache->block_size;
+    return fa_launch_kv_prep(ctx, L);
+}
+
+extern "C" fa_status fa_paged_gather(fa_ctx *ctx, const fa_paged_kv *cache, uint32_t seq_index, uint32_t seq_len,
+                                     void *k_out, void *v_out, uint32_t out_capacity) {
+    FA_NEED(ctx, "ctx");
+    FA_TRY(check_paged(cache));
+    FA_NEED(k_out, "k_out");
+    FA_NEED(v_out, "v_out");
+    if (seq_index >= cache->n_seqs) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: seq_index %u >= n_seqs %u", seq_index, cache->n_seqs);
+    if (seq_len > out_capacity || (uint64_t)seq_len > (uint64_t)cache->max_blocks_per_seq * cache->block_size)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: seq_len %u exceeds out_capacity %u or the block table", seq_len, out_capacity);
+    return fa_launch_paged_gather(ctx, cache, seq_index, seq_len, k_out, v_out, out_capacity);
+}
+
+// ------------------------------------------------------------------------------------------------ FlashAttention
+
+struct KvLayout {
+    uint32_t n_kv_heads, capacity;
+    uint64_t stride_h;
+};
+
+// K/V are head-major caches: rank 3 [Hkv, cap, D] or rank 4 [1, Hkv, cap, D]
+// (infer_n_kv_heads, src/metals/flashattention/step.rs:430-446; strides :797-831).
+static fa_status kv_layout(const fa_tensor_arg *t, const char *name, uint32_t head_dim, KvLayout &o) {
+    if (t->rank != 3 && t->rank != 4)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "%s must be a head-major cache of rank 3 or 4, got rank %u", name, t->rank);
+    const uint32_t r = t->rank;
+    if (r == 4 && t->dims[0] != 1)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "%s: batch %zu != 1 (this path assumes batch = 1)", name, t->dims[0]);
+    if (t->dims[r - 1] != head_dim)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %s last dim %zu != head_dim %u", name, t->dims[r - 1], head_dim);
+    if (t->strides[r - 1] != 1 || t->strides[r - 2] != head_dim)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "%s rows must be contiguous with row stride == head_dim (strides %zu,%zu)",
+                       name, t->strides[r - 2], t->strides[r - 1]);
+    o.n_kv_heads = (uint32_t)t->dims[r - 3];
+    o.capacity = (uint32_t)t->dims[r - 2];
+    o.stride_h = t->strides[r - 3];
+    if (o.n_kv_heads == 0 || o.capacity == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %s is empty", name);
+    return FA_OK;
+}
+
+static bool dims_eq(const fa_tensor_arg *t, uint32_t rank) { return t->rank == rank; }
+
+// Q layout inference for prefill (src/metals/flashattention/step.rs:648-719).
+static fa_status infer_q_layout(const fa_tensor_arg *q, uint32_t n_heads, uint32_t head_dim, uint32_t q_len,
+                                uint64_t &sh, uint64_t &sm) {
+    const size_t H = n_heads, D = head_dim, dm = (size_t)n_heads * head_dim, M = q_len;
+    const size_t *d = q->dims, *s = q->strides;
+    if (q->rank >= 1 && s[q->rank - 1] != 1)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill requires contiguous last dim for q");
+    // token-major metadata [1, M_cap, d_model] but head-major packed contents written by KvPrepFused
+    if (dims_eq(q, 3) && d[0] == 1 && d[2] == dm) {
+        sh = (uint64_t)M * D, sm = D;
+        return FA_OK;
+    }
+    if (dims_eq(q, 3) && d[0] == H && d[1] >= M && d[2] == D) { sh = s[0], sm = s[1]; return FA_OK; }
+    if (dims_eq(q, 4) && d[1] == H && d[2] >= M && d[3] == D) {
+        if (d[0] != 1) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill dispatches with batch = 1, q batch is %zu", d[0]);
+        sh = s[1], sm = s[2];
+        return FA_OK;
+    }
+    if (dims_eq(q, 2) && d[0] >= M && d[1] == dm) { sh = D, sm = s[0]; return FA_OK; }
+    if (dims_eq(q, 3) && d[1] >= M && d[2] == dm) {
+        if (d[0] != 1) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill dispatches with batch = 1, q batch is %zu", d[0]);
+        sh = D, sm = s[1];
+        return FA_OK;
+    }
+    if (dims_eq(q, 3) && d[0] >= M && d[1] == H && d[2] == D) { sh = s[1], sm = s[0]; return FA_OK; }
+    if (dims_eq(q, 4) && d[1] >= M && d[2] == H && d[3] == D) {
+        if (d[0] != 1) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill dispatches with batch = 1, q batch is %zu", d[0]);
+        sh = s[2], sm = s[1];
+        return FA_OK;
+    }
+    return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED,
+                   "Prefill Q layout unsupported: rank %u dims [%zu,%zu,%zu,%zu] (expected head-major [H,M>=q_len,D] or "
+                   "token-major [M>=q_len,d_model]/[M>=q_len,H,D])",
+                   q->rank, d[0], d[1], d[2], d[3]);
+}
+
+// Output layout inference for prefill (src/metals/flashattention/step.rs:722-756).
+static fa_status infer_out_layout(const fa_tensor_arg *o, uint32_t n_heads, uint32_t head_dim, uint32_t q_len,
+                                  uint64_t &sh, uint64_t &sm) {
+    const size_t H = n_heads, D = head_dim, dm = (size_t)n_heads * head_dim, M = q_len;
+    const size_t *d = o->dims, *s = o->strides;
+    if (o->rank >= 1 && s[o->rank - 1] != 1)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill requires contiguous last dim for output");
+    if (dims_eq(o, 2) && d[0] >= M && d[1] == dm) { sh = D, sm = s[0]; return FA_OK; }
+    if (dims_eq(o, 3) && d[1] >= M && d[2] == dm) {
+        if (d[0] != 1) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill dispatches with batch = 1, output batch is %zu", d[0]);
+        sh = D, sm = s[1];
+        return FA_OK;
+    }
+    if (dims_eq(o, 3) && d[0] >= M && d[1] == H && d[2] == D) { sh = s[1], sm = s[0]; return FA_OK; }
+    if (dims_eq(o, 4) && d[1] >= M && d[2] == H && d[3] == D) {
+        if (d[0] != 1) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill dispatches with batch = 1, output batch is %zu", d[0]);
+        sh = s[2], sm = s[1];
+        return FA_OK;
+    }
+    if (dims_eq(o, 3) && d[0] == H && d[1] >= M && d[2] == D) { sh = s[0], sm = s[1]; return FA_OK; }
+    if (dims_eq(o, 4) && d[1] == H && d[2] >= M && d[3] == D) {
+        if (d[0] != 1) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill dispatches with batch = 1, output batch is %zu", d[0]);
+        sh = s[1], sm = s[2];
+        return FA_OK;
+    }
+    return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill output layout unsupported: rank %u dims [%zu,%zu,%zu,%zu]", o->rank,
+                   d[0], d[1], d[2], d[3]);
+}
+
+static fa_status decode_common(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                               const fa_tensor_arg *output, uint32_t n_heads, uint32_t head_dim, DecodeLaunch &L) {
+    FA_NEED(ctx, "ctx");
+    if (head_dim != 64 && head_dim != 128)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Flash Decode only supports head_dim=64 or 128, got %u", head_dim);
+    if (n_heads == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_heads is 0");
+    const size_t dm = (size_t)n_heads * head_dim;
+    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, dm, 16));
+    FA_TRY(check_tensor(k, "k", FA_DTYPE_F16, 0, 16));
+    FA_TRY(check_tensor(v, "v", FA_DTYPE_F16, 0, 16));
+    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, dm, 2));
+    KvLayout kl, vl;
+    FA_TRY(kv_layout(k, "k", head_dim, kl));
+    FA_TRY(kv_layout(v, "v", head_dim, vl));
+    if (kl.n_kv_heads != vl.n_kv_heads || kl.capacity != vl.capacity)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: k [%u,%u] and v [%u,%u] caches differ", kl.n_kv_heads, kl.capacity,
+                       vl.n_kv_heads, vl.capacity);
+    if (n_heads % kl.n_kv_heads != 0)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_heads %u not a multiple of the cache's %u kv heads", n_heads, kl.n_kv_heads);
+    memset(&L, 0, sizeof(L));
+    L.q = tptr<const void>(q), L.k = tptr<const void>(k), L.v = tptr<const __half>(v), L.out = tptr<__half>(output);
+    // q_rot is head-major packed over q_seq_len = 1 whatever its metadata says (step.rs:1005-1020)
+    L.q_stride_b = dm, L.q_stride_h = head_dim;
+    L.k_stride_b = 0, L.k_stride_h = kl.stride_h, L.v_stride_b = 0, L.v_stride_h = vl.stride_h;
+    L.out_stride_b = dm, L.out_stride_h = head_dim;
+    L.n_heads = n_heads, L.n_kv_heads = kl.n_kv_heads, L.head_dim = head_dim, L.batch = 1;
+    L.capacity = kl.capacity;
+    L.scale = 1.0f / sqrtf((float)head_dim);  // step.rs:1042
+    L.paged = false;
+    return FA_OK;
+}
+
+extern "C" fa_status fa_flash_attention(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                        const fa_tensor_arg *v, const fa_tensor_arg *output, int causal,
+                                        uint32_t query_offset, uint32_t n_heads, uint32_t head_dim, uint32_t kv_seq_len,
+                                        uint32_t m, int kv_head_major) {
+    FA_NEED(ctx, "ctx");
+    if (!kv_head_major)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FlashAttention only supports kv_head_major=true for now");
+    if (m == 0) m = 1;  // m_raw.max(1), sdpa/step.rs:180
+    if (m == 1) {
+        DecodeLaunch L;
+        FA_TRY(decode_common(ctx, q, k, v, output, n_heads, head_dim, L));
+        if (kv_seq_len == 0 || kv_seq_len > L.capacity)
+            return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_seq_len %u outside (0, capacity %u]", kv_seq_len, L.capacity);
+        // keys visible to the single query row: all of them, or j <= query_offset under a causal mask
+        uint32_t vis = kv_seq_len;
+        if (causal && (uint64_t)query_offset + 1 < kv_seq_len) vis = query_offset + 1;
+        L.kv_len = vis, L.kv_len_bound = vis, L.d_len = nullptr;
+        return fa_launch_decode(ctx, L);
+    }
+    if (head_dim != 64 && head_dim != 128)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill only supports head_dim=64 or 128, got %u", head_dim);
+    if (n_heads == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_heads is 0");
+    const size_t need = (size_t)m * n_heads * head_dim;
+    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, need, 16));
+    FA_TRY(check_tensor(k, "k", FA_DTYPE_F16, 0, 16));
+    FA_TRY(check_tensor(v, "v", FA_DTYPE_F16, 0, 16));
+    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, need, 8));
+    KvLayout kl, vl;
+    FA_TRY(kv_layout(k, "k", head_dim, kl));
+    FA_TRY(kv_layout(v, "v", head_dim, vl));
+    if (kl.n_kv_heads != vl.n_kv_heads || kl.capacity != vl.capacity)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: k and v caches differ");
+    if (n_heads % kl.n_kv_heads != 0)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_heads %u not a multiple of the cache's %u kv heads", n_heads, kl.n_kv_heads);
+    if (kv_seq_len == 0 || kv_seq_len > kl.capacity)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_seq_len %u outside (0, capacity %u]", kv_seq_len, kl.capacity);
+    PrefillLaunch P;
+    memset(&P, 0, sizeof(P));
+    FA_TRY(infer_q_layout(q, n_heads, head_dim, m, P.q_stride_h, P.q_stride_m));
+    FA_TRY(infer_out_layout(output, n_heads, head_dim, m, P.out_stride_h, P.out_stride_m));
+    if (P.q_stride_h % 8 != 0 || P.q_stride_m % 8 != 0 || P.out_stride_h % 4 != 0 || P.out_stride_m % 4 != 0)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill needs q strides that are multiples of 8 and output strides multiples of 4");
+    P.q = tptr<const __half>(q), P.k = tptr<const __half>(k), P.v = tptr<const __half>(v), P.out = tptr<__half>(output);
+    P.k_stride_h = kl.stride_h, P.v_stride_h = vl.stride_h;
+    P.n_heads = n_heads, P.group_size = n_heads / kl.n_kv_heads, P.head_dim = head_dim;
+    P.q_len = m, P.kv_len = kv_seq_len, P.query_offset = query_offset, P.causal = causal;
+    P.scale = 1.0f / sqrtf((float)head_dim);
+    P.paged = false, P.n_kv_heads = kl.n_kv_heads;
+    return fa_launch_prefill(ctx, P);
+}
+
+extern "C" fa_status fa_flash_decode_dyn(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                         const fa_tensor_arg *v, const fa_tensor_arg *output, uint32_t n_heads,
+                                         uint32_t head_dim, const uint32_t *d_position, uint32_t kv_len_add,
+                                         uint32_t kv_len_bound) {
+    FA_NEED(d_position, "d_position");
+    DecodeLaunch L;
+    FA_TRY(decode_common(ctx, q, k, v, output, n_heads, head_dim, L));
+    if (kv_len_bound == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_len_bound is 0");
+    L.d_len = d_position, L.d_len_stride = 0, L.kv_len_add = kv_len_add;
+    L.kv_len_bound = kv_len_bound < L.capacity ? kv_len_bound : L.capacity;
+    return fa_launch_decode(ctx, L);
+}
+
+extern "C" fa_status fa_flash_decode_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_paged_kv *cache,
+                                           const fa_tensor_arg *output, uint32_t n_heads, uint32_t kv_len_add,
+                                           uint32_t kv_len_bound) {
+    FA_NEED(ctx, "ctx");
+    FA_TRY(check_paged(cache));
+    if (!cache->seq_lens) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: seq_lens");
+    if (n_heads == 0 || n_heads % cache->n_kv_heads != 0)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_heads %u not a multiple of n_kv_heads %u", n_heads, cache->n_kv_heads);
+    const size_t need = (size_t)cache->n_seqs * n_heads * cache->head_dim;
+    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, need, 16));
+    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, need, 2));
+    if (kv_len_bound == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_len_bound is 0");
+    DecodeLaunch L;
+    memset(&L, 0, sizeof(L));
+    const size_t dm = (size_t)n_heads * cache->head_dim;
+    L.q = tptr<const void>(q), L.k = cache->k_pool, L.v = (const __half *)cache->v_pool, L.out = tptr<__half>(output);
+    L.q_stride_b = dm, L.q_stride_h = cache->head_dim, L.out_stride_b = dm, L.out_stride_h = cache->head_dim;
+    L.n_heads = n_heads, L.n_kv_heads = cache->n_kv_heads, L.head_dim = cache->head_dim, L.batch = cache->n_seqs;
+    L.d_len = cache->seq_lens, L.d_len_stride = 1, L.kv_len_add = kv_len_add;
+    L.capacity = cache->max_blocks_per_seq * cache->block_size;
+    L.kv_len_bound = kv_len_bound < L.capacity ? kv_len_bound : L.capacity;
+    L.scale = 1.0f / sqrtf((float)cache->head_dim);
+    L.paged = true, L.block_table = cache->block_table, L.bt_stride = cache->max_blocks_per_seq;
+    L.block_size = cache->block_size;
+    return fa_launch_decode(ctx, L);
+}
+
+extern "C" fa_status fa_flash_prefill_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_paged_kv *cache,
+                                            uint32_t seq_index, const fa_tensor_arg *output, int causal,
+                                            uint32_t query_offset, uint32_t n_heads, uint32_t kv_seq_len, uint32_t m) {
+    FA_NEED(ctx, "ctx");
+    FA_TRY(check_paged(cache));
+    if (seq_index >= cache->n_seqs) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: seq_index %u >= n_seqs %u", seq_index, cache->n_seqs);
+    if (n_heads == 0 || n_heads % cache->n_kv_heads != 0)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_heads %u not a multiple of n_kv_heads %u", n_heads, cache->n_kv_heads);
+    if (m == 0) return FA_OK;
+    const uint64_t cap = (uint64_t)cache->max_blocks_per_seq * cache->block_size;
+    if (kv_seq_len == 0 || kv_seq_len > cap)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_seq_len %u outside (0, capacity %llu]", kv_seq_len, (unsigned long long)cap);
+    const uint32_t D = cache->head_dim;
+    const size_t need = (size_t)m * n_heads * D;
+    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, need, 16));
+    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, need, 8));
+    PrefillLaunch P;
+    memset(&P, 0, sizeof(P));
+    P.q = tptr<const __half>(q), P.k = (const __half *)cache->k_pool, P.v = (const __half *)cache->v_pool;
+    P.out = tptr<__half>(output);
+    P.q_stride_h = (uint64_t)m * D, P.q_stride_m = D;          // head-major [H, m, D]
+    P.out_stride_h = D, P.out_stride_m = (uint64_t)n_heads * D; // token-major [m, H*D]
+    P.n_heads = n_heads, P.group_size = n_heads / cache->n_kv_heads, P.head_dim = D;
+    P.q_len = m, P.kv_len = kv_seq_len, P.query_offset = query_offset, P.causal = causal;
+    P.scale = 1.0f / sqrtf((float)D);
+    P.paged = true, P.block_table = cache->block_table + (size_t)seq_index * cache->max_blocks_per_seq;
+    P.block_size = cache->block_size, P.n_kv_heads = cache->n_kv_heads;
+    return fa_launch_prefill(ctx, P);
+}
+
+// ------------------------------------------------------------------------------------------------ Sage int8
+
+static fa_status sage_dims(uint32_t head_dim) {
+    if (head_dim != 64 && head_dim != 128)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Sage decode supports head_dim=64 or 128, got %u", head_dim);
+    return FA_OK;
+}
+
+extern "C" fa_status fa_sage_k_mean(fa_ctx *ctx, const void *k, uint32_t n_kv_heads, uint32_t capacity,
+                                    uint32_t head_dim, uint32_t kv_len, float *mean_out) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(k, "k");
+    FA_NEED(mean_out, "mean_out");
+    FA_TRY(sage_dims(head_dim));
+    if (kv_len > capacity || n_kv_heads == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_len %u > capacity %u", kv_len, capacity);
+    return fa_launch_sage_k_mean(ctx, k, n_kv_heads, capacity, head_dim, kv_len, mean_out);
+}
+
+extern "C" fa_status fa_sage_quantize_k(fa_ctx *ctx, const void *k, const float *mean, uint32_t n_kv_heads,
+                                        uint32_t capacity, uint32_t head_dim, uint32_t row_begin, uint32_t row_end,
+                                        void *k_q, void *k_scale) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(k, "k");
+    FA_NEED(mean, "mean");
+    FA_NEED(k_q, "k_q");
+    FA_NEED(k_scale, "k_scale");
+    FA_TRY(sage_dims(head_dim));
+    if (row_begin % FA_SAGE_BLOCK != 0)
+        return fa_fail(FA_ERR_INVALID_OPERATION, "Invalid operation: row_begin %u is not a multiple of %u", row_begin, FA_SAGE_BLOCK);
+    if (row_end > capacity || row_begin > row_end)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: rows [%u,%u) outside capacity %u", row_begin, row_end, capacity);
+    return fa_launch_sage_quantize_k(ctx, k, mean, n_kv_heads, capacity, head_dim, row_begin, row_end, k_q, k_scale);
+}
+
+extern "C" fa_status fa_sage_quantize_q(fa_ctx *ctx, const void *q, uint32_t n_heads, uint32_t head_dim, void *q_q,
+                                        float *q_scale) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(q, "q");
+    FA_NEED(q_q, "q_q");
+    FA_NEED(q_scale, "q_scale");
+    FA_TRY(sage_dims(head_dim));
+    return fa_launch_sage_quantize_q(ctx, q, n_heads, head_dim, q_q, q_scale);
+}
+
+extern "C" fa_status fa_sage_decode(fa_ctx *ctx, const void *q_q, const float *q_scale, const void *k_q,
+                                    const void *k_scale, const void *v, void *out, uint32_t n_heads,
+                                    uint32_t n_kv_heads, uint32_t head_dim, uint32_t capacity, uint32_t kv_len) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(q_q, "q_q");
+    FA_NEED(q_scale, "q_scale");
+    FA_NEED(k_q, "k_q");
+    FA_NEED(k_scale, "k_scale");
+    FA_NEED(v, "v");
+    FA_NEED(out, "out");
+    FA_TRY(sage_dims(head_dim));
+    if (n_kv_heads == 0 || n_heads % n_kv_heads != 0)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_heads %u not a multiple of n_kv_heads %u", n_heads, n_kv_heads);
+    if (kv_len == 0 || kv_len > capacity)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_len %u outside (0, capacity %u]", kv_len, capacity);
+    if ((((uintptr_t)q_q) | ((uintptr_t)k_q)) % 8 != 0 || ((uintptr_t)v) % 16 != 0)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Sage decode needs 8-byte aligned int8 tensors and 16-byte aligned v");
+    DecodeLaunch L;
+    memset(&L, 0, sizeof(L));
+    const size_t dm = (size_t)n_heads * head_dim;
+    L.q = q_q, L.k = k_q, L.v = (const __half *)v, L.out = (__half *)out;
+    L.q_stride_b = dm, L.q_stride_h = head_dim, L.out_stride_b = dm, L.out_stride_h = head_dim;
+    L.k_stride_h = (uint64_t)capacity * head_dim, L.v_stride_h = (uint64_t)capacity * head_dim;
+    L.n_heads = n_heads, L.n_kv_heads = n_kv_heads, L.head_dim = head_dim, L.batch = 1;
+    L.kv_len = kv_len, L.kv_len_bound = kv_len, L.capacity = capacity;
+    L.scale = 1.0f / sqrtf((float)head_dim);
+    L.q_scale = q_scale, L.k_scale = (const __half *)k_scale, L.ks_stride = ceil_div_u32(capacity, FA_SAGE_BLOCK);
+    return fa_launch_decode(ctx, L);
+}

@@ -1,0 +1,141 @@
+// Internal declarations shared by the host API and the kernel translation units of libfoundry_attn.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "../../include/foundry_attn.h"
+
+struct fa_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+struct FaProfileRec {
+    const char *name;
+    hipEvent_t start, stop;
+};
+
+struct fa_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool capturing = false;
+    // grow-only scratch for split-K partials
+    void *workspace = nullptr;
+    size_t workspace_bytes = 0;
+    // per-(sequence, kv head) arrival counters for the in-kernel split merge; always zero between launches
+    uint32_t *counters = nullptr;
+    uint32_t n_counters = 0;
+    fa_decode_variant decode_variant{0, 0};
+    // per-kernel profiling
+    bool profiling = false;
+    std::vector<FaProfileRec> prof;
+    std::vector<hipEvent_t> event_pool;
+    int n_cus = 0;
+};
+
+// Error plumbing --------------------------------------------------------------------------------
+fa_status fa_fail(fa_status s, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define FA_HIP(expr)                                                                                       \
+    do {                                                                                                   \
+        hipError_t _e = (expr);                                                                            \
+        if (_e != hipSuccess)                                                                              \
+            return fa_fail(_e == hipErrorOutOfMemory ? FA_ERR_OUT_OF_MEMORY : FA_ERR_OPERATION_FAILED,     \
+                           "%s failed: %s", #expr, hipGetErrorString(_e));                                 \
+    } while (0)
+
+#define FA_TRY(expr)                    \
+    do {                                \
+        fa_status _s = (expr);          \
+        if (_s != FA_OK) return _s;     \
+    } while (0)
+
+// Brackets a kernel launch with events when profiling; checks the launch result.
+struct FaLaunchScope {
+    fa_ctx *ctx;
+    const char *name;
+    hipEvent_t start = nullptr, stop = nullptr;
+    FaLaunchScope(fa_ctx *c, const char *n);
+    fa_status finish();
+};
+
+static inline uint32_t ceil_div_u32(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
+
+// Kernel launchers (defined in the kernel translation units) -------------------------------------
+
+struct KvPrepLaunch {
+    const __half *q, *k, *v;
+    __half *q_rot, *k_cache, *v_cache;
+    const __half *cos_t, *sin_t;
+    fa_kv_prep_fused_params p;
+    const uint32_t *d_position;  // nullable: device-side position for mode 0/1
+    // mode: 0 contiguous cache, 1 paged one sequence, 2 paged batched decode (one token per sequence)
+    int mode;
+    const int32_t *block_table;  // row of the sequence (mode 1) or whole table (mode 2)
+    const uint32_t *seq_lens;    // mode 2
+    uint32_t bt_stride;          // max_blocks_per_seq
+    uint32_t block_size;
+    uint32_t capacity;           // rows addressable through the cache (contiguous: max_seq_len)
+    uint32_t table_rows;         // rows available in cos/sin
+};
+fa_status fa_launch_kv_prep(fa_ctx *ctx, const KvPrepLaunch &a);
+
+struct DecodeLaunch {
+    const void *q;  // [batch][n_heads][D] via strides
+    const void *k;
+    const __half *v;
+    __half *out;
+    uint64_t q_stride_b, q_stride_h, k_stride_b, k_stride_h, v_stride_b, v_stride_h, out_stride_b, out_stride_h;
+    uint32_t n_heads, n_kv_heads, head_dim, batch;
+    uint32_t kv_len;             // static length (used when d_len == nullptr)
+    const uint32_t *d_len;       // nullable: per-batch device lengths
+    uint32_t d_len_stride;       // 0 = one shared scalar, 1 = per sequence
+    uint32_t kv_len_add;
+    uint32_t kv_len_bound;       // sizes the grid
+    uint32_t capacity;           // clamp
+    float scale;
+    // paged
+    bool paged;
+    const int32_t *block_table;
+    uint32_t bt_stride, block_size;
+    // Sage-style int8 Q/K (q and k are int8 when q_scale != nullptr)
+    const float *q_scale;
+    const __half *k_scale;
+    uint32_t ks_stride;
+};
+fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &a);
+
+struct PrefillLaunch {
+    const __half *q, *k, *v;
+    __half *out;
+    uint64_t q_stride_h, q_stride_m, k_stride_h, v_stride_h, out_stride_h, out_stride_m;
+    uint32_t n_heads, group_size, head_dim, q_len, kv_len, query_offset;
+    int causal;
+    float scale;
+    bool paged;
+    const int32_t *block_table;
+    uint32_t block_size, n_kv_heads;
+};
+fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &a);
+
+fa_status fa_launch_u32_add(fa_ctx *ctx, uint32_t *vals, uint32_t n, uint32_t delta);
+fa_status fa_launch_paged_gather(fa_ctx *ctx, const fa_paged_kv *c, uint32_t seq_index, uint32_t seq_len, void *k_out,
+                                 void *v_out, uint32_t out_capacity);
+
+fa_status fa_launch_sage_k_mean(fa_ctx *ctx, const void *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim,
+                                uint32_t kv_len, float *mean_out);
+fa_status fa_launch_sage_quantize_k(fa_ctx *ctx, const void *k, const float *mean, uint32_t n_kv_heads,
+                                    uint32_t capacity, uint32_t head_dim, uint32_t row_begin, uint32_t row_end,
+                                    void *k_q, void *k_scale);
+fa_status fa_launch_sage_quantize_q(fa_ctx *ctx, const void *q, uint32_t n_heads, uint32_t head_dim, void *q_q,
+                                    float *q_scale);
+
+fa_status fa_ensure_workspace(fa_ctx *ctx, size_t bytes);
+fa_status fa_ensure_counters(fa_ctx *ctx, uint32_t n);

@@ -1,0 +1,69 @@
+"""No-GPU checks of the C ABI: the library loads, exports every symbol the header declares, its host-only
+entry points work, and errors follow the documented convention."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import foundry_attn as fa
+import orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "foundry_attn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = fa.load()
+    names = _declared_symbols()
+    assert len(names) >= 35
+    for n in names:
+        assert hasattr(lib, n), "symbol %s declared in foundry_attn.h is not exported" % n
+    # and the binding declares a prototype for each of them
+    assert set(names) == set(fa.PROTOTYPES), set(names) ^ set(fa.PROTOTYPES)
+
+
+def test_struct_layouts_match_the_reference_abi():
+    # KvPrepFusedParamsResolved is 13 x u32 = 52 bytes (src/metals/kv_prep/mod.rs:79-114)
+    assert C.sizeof(fa.KvPrepFusedParams) == 52
+    assert [f[0] for f in fa.KvPrepFusedParams._fields_] == [
+        "d_model", "kv_dim", "head_dim", "n_heads", "n_kv_heads", "group_size", "seq_len", "position_offset",
+        "max_seq_len", "total_elements", "rope_mode", "layer_idx", "no_rope_layer_step"]
+    assert C.sizeof(fa.TensorArg) == 8 + 8 + 4 + 4 + 32 + 32
+
+
+def test_status_names():
+    lib = fa.load()
+    for code, name in fa.STATUS_NAMES.items():
+        assert lib.fa_status_name(code).decode() == name
+    assert lib.fa_version().decode().startswith("foundry_attn")
+
+
+@pytest.mark.parametrize("base,D,P,ff", [(1e6, 64, 1100, False), (5e5, 128, 8500, False), (5e6, 128, 300, True)])
+def test_host_rope_tables_equal_oracle(base, D, P, ff):
+    factors = np.linspace(1, 4, D // 2).astype(np.float32) if ff else None
+    cos, sin = fa.rope_tables(base, D, P, factors)
+    ocos, osin = orc.rope_tables(base, D, P, factors)
+    assert np.array_equal(cos.view(np.uint16), ocos.view(np.uint16))
+    assert np.array_equal(sin.view(np.uint16), osin.view(np.uint16))
+    wc, ws = fa.rope_tables(base, D, P, factors, pos_begin=P - 10)
+    assert np.array_equal(wc, cos[P - 10:]) and np.array_equal(ws, sin[P - 10:])
+
+
+def test_host_errors_without_a_device():
+    lib = fa.load()
+    with pytest.raises(fa.FoundryError) as e:
+        fa.rope_tables(1e4, 63, 4)
+    assert e.value.variant == "InvalidShape"
+    assert lib.fa_ctx_create(0, None) == 2  # NullPointer
+    h = C.c_void_p()
+    st = lib.fa_ctx_create(4096, C.byref(h))  # no such device anywhere
+    assert st == 1 and "Device not found" in lib.fa_last_error_string().decode()
+    assert lib.fa_synchronize(None) == 2
+    assert lib.fa_graph_destroy(None) == 0 and lib.fa_ctx_destroy(None) == 0

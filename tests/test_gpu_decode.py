@@ -1,0 +1,196 @@
+"""GPU parity: flash decode (fa_flash_attention with m = 1, fa_flash_decode_dyn) against the CPU oracle.
+Tolerance: max-abs <= 2e-3 on f16 outputs with f32 accumulation (N(0,1) inputs)."""
+import os
+
+import numpy as np
+import pytest
+
+import foundry_attn as fa
+import orc
+import refmath as rm
+from gpu_util import announce, bits, ctx, h16, max_abs
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def gpu_decode(q, k, v, H, D, N, causal=True, query_offset=None, q_arg_dims=None):
+    f = ctx()
+    Hkv, cap = k.shape[0], k.shape[1]
+    dq, dk, dv, do = f.array(q), f.array(k), f.array(v), f.zeros((1, H * D))
+    qa = dq.arg(q_arg_dims) if q_arg_dims else dq.arg((1, H * D))
+    f.flash_attention(qa, dk.arg(), dv.arg(), do.arg(), causal, N - 1 if query_offset is None else query_offset, H, D,
+                      N, 1)
+    f.synchronize()
+    out = do.download().reshape(H, D)
+    for b in (dq, dk, dv, do):
+        b.free()
+    return out
+
+
+@pytest.mark.parametrize("H,Hkv,D,N,cap", [
+    (14, 2, 64, 1025, 1152),    # BASELINE config 1 (Qwen2.5-0.5B shape)
+    (24, 8, 128, 8193, 8448),   # BASELINE config 2 (Llama-3.2-3B shape, one layer)
+    (16, 2, 128, 3000, 3008),   # Qwen2.5-3B shape
+    (16, 4, 128, 5000, 5120),   # SmolLM3 shape
+    (32, 8, 128, 777, 1024),
+    (8, 8, 64, 130, 130), (2, 1, 128, 64, 64), (12, 2, 64, 333, 400), (10, 2, 128, 100, 128), (16, 1, 64, 70, 96),
+])
+def test_decode_vs_oracle(H, Hkv, D, N, cap):
+    announce("decode", H, Hkv, D, N, cap)
+    rng = np.random.default_rng(H * 1000 + N)
+    q = h16(rng.normal(size=(H, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    got = gpu_decode(q, k, v, H, D, N)
+    want = orc.sdpa_decode(q, k, v, H, Hkv, D, cap, N, n_threads=8).reshape(H, D)
+    assert max_abs(got, want) <= TOL
+    assert max_abs(got, rm.gqa_decode_f64(q, k, v, H, Hkv, D, N)) <= TOL
+
+
+@pytest.mark.parametrize("N", [1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 257, 1000])
+@pytest.mark.parametrize("D,H,Hkv", [(64, 14, 2), (128, 6, 2)])
+def test_decode_ragged_lengths_and_splits(N, D, H, Hkv):
+    announce("decode ragged", N, D)
+    f = ctx()
+    rng = np.random.default_rng(N)
+    cap = 1024
+    q = h16(rng.normal(size=(H, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    k[:, N:], v[:, N:] = np.float16(np.nan), np.float16(np.nan)  # rows past kv_len must never contribute
+    want = orc.sdpa_decode(q, k, v, H, Hkv, D, cap, N).reshape(H, D)
+    try:
+        for kps, merge in [(0, 0), (64, 0), (64, 1), (128, 0), (1024, 1)]:
+            f.set_decode_variant(kps, merge)
+            got = gpu_decode(q, k, v, H, D, N)
+            assert np.all(np.isfinite(got)), (kps, merge)
+            assert max_abs(got, want) <= TOL, (kps, merge)
+    finally:
+        f.set_decode_variant(0, 0)
+
+
+def test_decode_known_answer_fixture():
+    announce("decode known-answer fixture")
+    g = np.load(os.path.join(GOLD, "known_answer_sdpa.npz"))
+    q, k, v, want = g["oob_m1_q"], g["oob_m1_k"], g["oob_m1_v"], g["oob_m1_expected_f64"]
+    H, _, D = q.shape
+    N = k.shape[1]
+    got = gpu_decode(q.reshape(H, D), k, v, H, D, N, causal=False, query_offset=0)
+    assert np.all(np.abs(got.astype(np.float64) - want[:, 0]) <= rm.f16_ulp(want[:, 0]) + 1e-6)
+
+
+@pytest.mark.parametrize("seed,H,D,N", [(1, 14, 64, 128), (7, 14, 64, 257), (42, 8, 128, 300)])
+def test_decode_reference_lcg_inputs(seed, H, D, N):
+    """Inputs of tests/flashattention_decode_parity.rs (LCG, MHA cache); the reference accepts 6e-2 there."""
+    announce("decode lcg", seed)
+    st = seed
+    q, st = orc.lcg_fill_f16(st, H * D, 0.25)
+    k, st = orc.lcg_fill_f16(st, H * N * D, 0.25)
+    v, st = orc.lcg_fill_f16(st, H * N * D, 0.25)
+    k, v = k.reshape(H, N, D), v.reshape(H, N, D)
+    got = gpu_decode(q.reshape(H, D), k, v, H, D, N, q_arg_dims=(1, H * D))
+    assert max_abs(got, rm.gqa_decode_f64(q, k, v, H, H, D, N)) <= 5e-4
+
+
+def test_decode_group_sizes_and_invariants():
+    announce("decode group sizes")
+    rng = np.random.default_rng(5)
+    D, N, cap = 128, 200, 256
+    for G in (1, 2, 3, 4, 5, 6, 7, 8, 12, 16):
+        Hkv = 2
+        H = G * Hkv
+        q = h16(rng.normal(size=(H, D)))
+        k = h16(rng.normal(size=(Hkv, cap, D)))
+        v = h16(rng.normal(size=(Hkv, cap, D)))
+        got = gpu_decode(q, k, v, H, D, N)
+        assert max_abs(got, orc.sdpa_decode(q, k, v, H, Hkv, D, cap, N).reshape(H, D)) <= TOL, G
+        # GQA(compact) == MHA(expanded)
+        ke = orc.repeat_kv_heads(k, Hkv, H, cap, D, cap)
+        ve = orc.repeat_kv_heads(v, Hkv, H, cap, D, cap)
+        assert max_abs(got, gpu_decode(q, ke, ve, H, D, N)) <= 1e-3, G
+    # equal keys -> mean of V ; single key -> V[0]
+    H, Hkv = 6, 2
+    q = h16(rng.normal(size=(H, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    ks = np.broadcast_to(h16(rng.normal(size=(Hkv, 1, D))), (Hkv, cap, D)).copy()
+    got = gpu_decode(q, ks, v, H, D, N)
+    for h in range(H):
+        assert max_abs(got[h], v[h // 3, :N].astype(np.float64).mean(0)) <= 1e-3
+    got1 = gpu_decode(q, ks, v, H, D, 1)
+    for h in range(H):
+        assert np.array_equal(bits(got1[h]), bits(v[h // 3, 0]))
+
+
+def test_decode_causal_offset_and_rank4_cache():
+    """m = 1 with query_offset + 1 < kv_seq_len (the reference routes this to its materialized path,
+    src/metals/sdpa/step.rs:268-290): only keys j <= query_offset are visible."""
+    announce("decode causal offset")
+    f = ctx()
+    rng = np.random.default_rng(9)
+    H, Hkv, D, N, cap = 8, 2, 64, 90, 96
+    q = h16(rng.normal(size=(H, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    got = gpu_decode(q, k, v, H, D, N, causal=True, query_offset=40)
+    assert max_abs(got, orc.sdpa_decode(q, k, v, H, Hkv, D, cap, 41).reshape(H, D)) <= TOL
+    got = gpu_decode(q, k, v, H, D, N, causal=False, query_offset=40)
+    assert max_abs(got, orc.sdpa_decode(q, k, v, H, Hkv, D, cap, N).reshape(H, D)) <= TOL
+    dq, dk, dv, do = f.array(q), f.array(k), f.array(v), f.zeros((H * D,))
+    f.flash_attention(dq.arg((H * D,)), dk.arg((1, Hkv, cap, D)), dv.arg((1, Hkv, cap, D)), do.arg(), True, N - 1, H, D,
+                      N, 1)
+    f.synchronize()
+    assert max_abs(do.download().reshape(H, D), orc.sdpa_decode(q, k, v, H, Hkv, D, cap, N).reshape(H, D)) <= TOL
+
+
+def test_decode_device_position_matches_static():
+    announce("decode dyn")
+    f = ctx()
+    rng = np.random.default_rng(11)
+    H, Hkv, D, cap = 24, 8, 128, 1024
+    q = h16(rng.normal(size=(H, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    dq, dk, dv, do = f.array(q), f.array(k), f.array(v), f.zeros((1, H * D))
+    dpos = f.array(np.array([0], np.uint32))
+    for pos in (0, 63, 64, 500, 1023):
+        dpos.upload(np.array([pos], np.uint32))
+        f.flash_decode_dyn(dq.arg(), dk.arg(), dv.arg(), do.arg(), H, D, dpos, 1, cap)
+        f.synchronize()
+        got = do.download().reshape(H, D)
+        assert max_abs(got, orc.sdpa_decode(q, k, v, H, Hkv, D, cap, pos + 1).reshape(H, D)) <= TOL, pos
+    # a bound smaller than the device length clamps instead of reading past it
+    dpos.upload(np.array([900], np.uint32))
+    f.flash_decode_dyn(dq.arg(), dk.arg(), dv.arg(), do.arg(), H, D, dpos, 1, 256)
+    f.synchronize()
+    assert max_abs(do.download().reshape(H, D), orc.sdpa_decode(q, k, v, H, Hkv, D, cap, 256).reshape(H, D)) <= TOL
+
+
+def test_decode_errors():
+    announce("decode errors")
+    f = ctx()
+    H, Hkv, cap = 4, 2, 32
+    for D, variant in [(96, "OperationNotSupported"), (32, "OperationNotSupported")]:
+        dq, dk, dv, do = f.zeros((1, H * D)), f.zeros((Hkv, cap, D)), f.zeros((Hkv, cap, D)), f.zeros((1, H * D))
+        with pytest.raises(fa.FoundryError) as e:
+            f.flash_attention(dq.arg(), dk.arg(), dv.arg(), do.arg(), True, 0, H, D, 1, 1)
+        assert e.value.variant == variant and "head_dim" in str(e.value)
+    D = 64
+    dq, dk, dv, do = f.zeros((1, H * D)), f.zeros((Hkv, cap, D)), f.zeros((Hkv, cap, D)), f.zeros((1, H * D))
+    with pytest.raises(fa.FoundryError) as e:
+        f.flash_attention(dq.arg(), dk.arg(), dv.arg(), do.arg(), True, 0, H, D, 1, 1, kv_head_major=False)
+    assert e.value.variant == "OperationNotSupported" and "kv_head_major" in str(e.value)
+    with pytest.raises(fa.FoundryError) as e:
+        f.flash_attention(dq.arg(), dk.arg(), dv.arg(), do.arg(), True, 0, H, D, cap + 1, 1)
+    assert e.value.variant == "InvalidShape"
+    with pytest.raises(fa.FoundryError) as e:
+        f.flash_attention(dq.arg(), dk.arg(), dv.arg(), do.arg(), True, 0, H, D, 0, 1)
+    assert e.value.variant == "InvalidShape"
+    with pytest.raises(fa.FoundryError) as e:
+        f.flash_attention(dq.arg(), dk.arg((Hkv, cap, D), (cap * D * 2, 2 * D, 1)), dv.arg(), do.arg(), True, 0, H, D, 4, 1)
+    assert e.value.variant == "OperationNotSupported"
+    with pytest.raises(fa.FoundryError) as e:
+        f.set_decode_variant(100, 0)
+    assert e.value.variant == "OperationNotSupported"
+    f.synchronize()
