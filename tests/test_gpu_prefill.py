@@ -1,0 +1,172 @@
+"""GPU parity: causal flash prefill on MFMA (fa_flash_attention with m > 1, fa_flash_prefill_paged) against the
+CPU oracle. Tolerance: max-abs <= 2e-3 (f32 accumulation; probabilities are rounded to f16 for the PV MFMA)."""
+import os
+
+import numpy as np
+import pytest
+
+import foundry_attn as fa
+import orc
+import refmath as rm
+from gpu_util import announce, bits, ctx, h16, max_abs
+
+pytestmark = pytest.mark.gpu
+TOL = 2e-3
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def gpu_prefill(q_hm, k, v, H, D, M, N, offset, causal=True, q_layout="head_major", out_layout="token_major"):
+    f = ctx()
+    if q_layout == "head_major":
+        dq = f.array(q_hm)
+        qa = dq.arg((H, M, D))
+    elif q_layout == "token_meta_head_contents":  # [1, M_cap, d_model] metadata over head-major packed contents
+        cap_m = M + 5
+        buf = np.zeros((cap_m * H * D,), np.float16)
+        buf[:H * M * D] = q_hm.reshape(-1)
+        dq = f.array(buf)
+        qa = dq.arg((1, cap_m, H * D))
+    else:  # token-major [M, H, D] with explicit head dim
+        dq = f.array(np.ascontiguousarray(q_hm.transpose(1, 0, 2)))
+        qa = dq.arg((M, H, D))
+    dk, dv = f.array(k), f.array(v)
+    if out_layout == "token_major":
+        do = f.zeros((M, H * D))
+        oa = do.arg()
+    else:
+        do = f.zeros((H, M, D))
+        oa = do.arg()
+    f.flash_attention(qa, dk.arg(), dv.arg(), oa, causal, offset, H, D, N, M)
+    f.synchronize()
+    out = do.download()
+    for b in (dq, dk, dv, do):
+        b.free()
+    if out_layout == "token_major":
+        out = out.reshape(M, H, D).transpose(1, 0, 2)
+    return out
+
+
+@pytest.mark.parametrize("M,prefix", [(2, 0), (7, 0), (16, 0), (17, 5), (26, 0), (31, 100), (32, 0), (33, 64),
+                                      (128, 0), (129, 31), (200, 1000), (257, 0)])
+@pytest.mark.parametrize("D,H,Hkv", [(64, 14, 2), (128, 6, 2)])
+def test_prefill_causal_vs_oracle(M, prefix, D, H, Hkv):
+    announce("prefill", M, prefix, D)
+    rng = np.random.default_rng(M * 31 + prefix)
+    N = prefix + M
+    cap = N + 7
+    q = h16(rng.normal(size=(H, M, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    k[:, N:], v[:, N:] = np.float16(np.nan), np.float16(np.nan)
+    want = orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, prefix, cap, causal=True, out_layout="head_major", n_threads=8)
+    got = gpu_prefill(q, k, v, H, D, M, N, prefix)
+    assert np.all(np.isfinite(got))
+    assert max_abs(got, want) <= TOL
+    assert max_abs(got, rm.gqa_prefill_f64(q, k, v, H, Hkv, D, N, prefix)) <= TOL
+
+
+def test_prefill_layouts_and_noncausal():
+    announce("prefill layouts")
+    rng = np.random.default_rng(2)
+    H, Hkv, D, M, prefix = 8, 2, 128, 45, 19
+    N, cap = M + prefix, 80
+    q = h16(rng.normal(size=(H, M, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    want = orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, prefix, cap, causal=True, out_layout="head_major")
+    base = gpu_prefill(q, k, v, H, D, M, N, prefix)
+    assert max_abs(base, want) <= TOL
+    for ql in ("token_meta_head_contents", "token_major_hd"):
+        for ol in ("token_major", "head_major"):
+            got = gpu_prefill(q, k, v, H, D, M, N, prefix, q_layout=ql, out_layout=ol)
+            assert np.array_equal(bits(got), bits(base)), (ql, ol)  # layouts only move data
+    # non-causal and causal-offset-mismatch cases run on the same kernel (no materialized fallback)
+    nc = gpu_prefill(q, k, v, H, D, M, N, 0, causal=False)
+    assert max_abs(nc, orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, 0, cap, causal=False, out_layout="head_major")) <= TOL
+    off = gpu_prefill(q, k, v, H, D, M, N, 3, causal=True)  # query_offset + m != kv_seq_len
+    assert max_abs(off, orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, 3, cap, causal=True, out_layout="head_major")) <= TOL
+
+
+def test_prefill_known_answer_fixture_noncausal():
+    announce("prefill fixture")
+    g = np.load(os.path.join(GOLD, "known_answer_sdpa.npz"))
+    q, k, v, want = (g["misaligned_m17_" + n] for n in ("q", "k", "v", "expected_f64"))
+    H, M, D = q.shape
+    N = k.shape[1]
+    got = gpu_prefill(q, k, v, H, D, M, N, 0, causal=False)
+    assert np.all(np.abs(got.astype(np.float64) - want) <= rm.f16_ulp(want) + 2e-4 * np.abs(want) + 1e-6)
+
+
+def test_prefill_rows_equal_decode_and_first_row():
+    announce("prefill rows == decode")
+    f = ctx()
+    rng = np.random.default_rng(4)
+    H, Hkv, D, M = 6, 2, 64, 70
+    cap = M
+    q = h16(rng.normal(size=(H, M, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    got = gpu_prefill(q, k, v, H, D, M, M, 0)
+    for h in range(H):
+        assert np.array_equal(bits(got[h, 0]), bits(v[h // 3, 0]))
+    for r in (1, 33, 69):
+        dq, dk, dv, do = f.array(q[:, r].copy()), f.array(k), f.array(v), f.zeros((1, H * D))
+        f.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), do.arg(), True, r, H, D, r + 1, 1)
+        f.synchronize()
+        assert max_abs(do.download().reshape(H, D), got[:, r]) <= 1.5e-3
+
+
+def test_prefill_llama_shape_full_size_from_paged_cache():
+    """BASELINE config 4: 2048-token prompt, H24/Hkv8/D128, RoPE theta 5e5 on positions 0..2047, all rows
+    appended into an empty paged cache, causal flash attention reading through the block table."""
+    announce("prefill C4 full size")
+    f = ctx()
+    rng = np.random.default_rng(0xF0DD + 4)
+    H, Hkv, D, M, bs = 24, 8, 128, 2048, 16
+    n_blocks = M // bs + 4
+    bt = rng.permutation(n_blocks)[:M // bs].astype(np.int32)[None, :]
+    q, k, v = (h16(rng.normal(size=(M, n * D))) for n in (H, Hkv, Hkv))
+    cos, sin = fa.rope_tables(5e5, D, M)
+    dkp, dvp = f.zeros((n_blocks, Hkv, bs, D)), f.zeros((n_blocks, Hkv, bs, D))
+    dbt = f.array(bt)
+    desc = fa.paged_kv(dkp, dvp, dbt, None, n_blocks, Hkv, bs, D, 1, M // bs)
+    dq, dk, dv, dqr, dout = f.array(q), f.array(k), f.array(v), f.zeros((H, M, D)), f.zeros((M, H * D))
+    dcos, dsin = f.array(cos), f.array(sin)
+    f.kv_prep_fused_paged(dq.arg(), dk.arg(), dv.arg(), dqr.arg(), desc, 0, dcos.arg(), dsin.arg(),
+                          fa.KvPrepFusedParams.make(H, Hkv, D, M, 0, 0, fa.ROPE_NORMAL))
+    f.flash_prefill_paged(dqr.arg(), desc, 0, dout.arg(), True, 0, H, M, M)
+    f.synchronize()
+    kc, vc = np.zeros((Hkv, M, D), np.float16), np.zeros((Hkv, M, D), np.float16)
+    qr = orc.kv_prep_fused(q, k, v, kc, vc, cos, sin, orc.make_params(H, Hkv, D, M, 0, M, rope_mode=1))
+    assert np.array_equal(bits(dqr.download()), bits(qr))
+    assert np.array_equal(bits(orc.paged_gather(dkp.download(), bt[0], Hkv, bs, D, M)), bits(kc))
+    assert np.array_equal(bits(orc.paged_gather(dvp.download(), bt[0], Hkv, bs, D, M)), bits(vc))
+    want = orc.sdpa_prefill(qr, kc, vc, H, Hkv, D, M, M, 0, M, causal=True, n_threads=16)  # token-major
+    got = dout.download()
+    assert max_abs(got, want) <= TOL
+    # the contiguous entry point on the gathered cache gives the same bits
+    dkc, dvc, dout2 = f.array(kc), f.array(vc), f.zeros((M, H * D))
+    f.flash_attention(dqr.arg((1, M, H * D)), dkc.arg(), dvc.arg(), dout2.arg(), True, 0, H, D, M, M)
+    f.synchronize()
+    assert np.array_equal(bits(dout2.download()), bits(got))
+
+
+def test_prefill_errors():
+    announce("prefill errors")
+    f = ctx()
+    H, Hkv, D, M, cap = 4, 2, 64, 8, 16
+    dq, dk, dv, do = f.zeros((H, M, D)), f.zeros((Hkv, cap, D)), f.zeros((Hkv, cap, D)), f.zeros((M, H * D))
+    f.flash_attention(dq.arg(), dk.arg(), dv.arg(), do.arg(), True, 0, H, D, M, M)
+    with pytest.raises(fa.FoundryError) as e:
+        f.flash_attention(dq.arg((H, M, 96)), dk.arg(), dv.arg(), do.arg(), True, 0, H, 96, M, M)
+    assert e.value.variant == "OperationNotSupported" and "64 or 128" in str(e.value)
+    with pytest.raises(fa.FoundryError) as e:
+        f.flash_attention(dq.arg((M * H * D,)), dk.arg(), dv.arg(), do.arg(), True, 0, H, D, M, M)
+    assert e.value.variant == "OperationNotSupported" and "layout" in str(e.value)
+    with pytest.raises(fa.FoundryError) as e:
+        f.flash_attention(dq.arg(), dk.arg(), dv.arg(), do.arg((H * M * D,)), True, 0, H, D, M, M)
+    assert e.value.variant == "OperationNotSupported"
+    with pytest.raises(fa.FoundryError) as e:
+        f.flash_attention(dq.arg(), dk.arg(), dv.arg(), do.arg(), True, 0, H, D, cap + 1, M)
+    assert e.value.variant == "InvalidShape"
+    f.synchronize()
