@@ -200,6 +200,20 @@ fa_status fa_flash_decode_dyn(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tens
                               const fa_tensor_arg *output, uint32_t n_heads, uint32_t head_dim,
                               const uint32_t *d_position, uint32_t kv_len_add, uint32_t kv_len_bound);
 
+/* One decode step of one layer in ONE launch: KvPrepFused with seq_len = 1 followed by FlashAttention with
+ * m = 1, i.e. what the model graph runs per layer per token (models/llama.json:529-565), fused the way the
+ * reference fuses RoPE into decode in RopeFlashDecodeStep (src/metals/flashattention/step.rs:16-306).
+ * q/k/v are the raw projections of the new token ([1, d_model] / [1, kv_dim]); the token is rotated, appended at
+ * row P of the caches and attended together with rows [0, P), where P = *d_position if d_position != NULL,
+ * else params->position_offset. Results are bit-identical to calling the two ops one after the other: the cache
+ * rows and q_rot carry the same bits, and the attention reads the same f16 values. q_rot may have a NULL buffer
+ * (then it is not written). kv_len_bound >= P + 1 as in fa_flash_decode_dyn. params->seq_len must be 1. */
+fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                               const fa_tensor_arg *q_rot, const fa_tensor_arg *k_cache,
+                               const fa_tensor_arg *v_cache, const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                               const fa_tensor_arg *output, const fa_kv_prep_fused_params *params,
+                               const uint32_t *d_position, uint32_t kv_len_bound);
+
 /* Tuning override, the counterpart of FlashDecodeVariant + METALLIC_FA_DECODE_* (src/metals/flashattention/
  * variants.rs:36-140). keys_per_split: context partition per workgroup (multiple of 64; 0 = auto).
  * merge: 0 = merged by the last workgroup to finish (one launch), 1 = separate merge kernel.
@@ -253,6 +267,15 @@ fa_status fa_kv_prep_decode_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_
 fa_status fa_flash_decode_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_paged_kv *cache,
                                 const fa_tensor_arg *output, uint32_t n_heads, uint32_t kv_len_add,
                                 uint32_t kv_len_bound);
+
+/* fa_kv_prep_decode_paged + fa_flash_decode_paged in one launch (see fa_decode_step_fused): sequence b's new
+ * token (row b of q/k/v) is rotated at position seq_lens[b], appended there and attended with the rows before
+ * it. q_rot [n_seqs, n_heads, head_dim] may have a NULL buffer. Does not modify seq_lens. */
+fa_status fa_decode_step_fused_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                     const fa_tensor_arg *v, const fa_tensor_arg *q_rot, const fa_paged_kv *cache,
+                                     const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                     const fa_tensor_arg *output, const fa_kv_prep_fused_params *params,
+                                     uint32_t kv_len_bound);
 
 /* Causal flash prefill for one sequence reading K/V through the block table. q is head-major
  * [n_heads, m, head_dim]; out token-major [m, n_heads*head_dim]. Mask as in fa_flash_attention. */

@@ -791,6 +791,110 @@ extern "C" fa_status fa_flash_decode_dyn(fa_ctx *ctx, const fa_tensor_arg *q, co
     return fa_launch_decode(ctx, L);
 }
 
+// Shared argument handling of the fused step: fills the RoPE / raw-projection part of a DecodeLaunch.
+static fa_status fused_common(const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                              const fa_tensor_arg *q_rot, const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                              const fa_kv_prep_fused_params *p, uint32_t n_tokens, DecodeLaunch &L) {
+    FA_TRY(check_kv_prep_params(p));
+    if (p->head_dim != 64 && p->head_dim != 128)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Flash Decode only supports head_dim=64 or 128, got %u", p->head_dim);
+    if (p->seq_len != n_tokens)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: the fused decode step takes %u token(s), seq_len is %u", n_tokens, p->seq_len);
+    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, (size_t)n_tokens * p->d_model, 16));
+    FA_TRY(check_tensor(k, "k", FA_DTYPE_F16, (size_t)n_tokens * p->kv_dim, 16));
+    FA_TRY(check_tensor(v, "v", FA_DTYPE_F16, (size_t)n_tokens * p->kv_dim, 16));
+    FA_TRY(check_tensor(cos, "cos", FA_DTYPE_F16, 0, 16));
+    FA_TRY(check_tensor(sin, "sin", FA_DTYPE_F16, 0, 16));
+    if (!q_rot) return fa_fail(FA_ERR_NULL_POINTER, "tensor argument 'q_rot' is null");
+    if (q_rot->buffer) FA_TRY(check_tensor(q_rot, "q_rot", FA_DTYPE_F16, (size_t)n_tokens * p->d_model, 16));
+    const uint32_t half = p->head_dim / 2;
+    size_t rows = numel(cos) / half;
+    if (numel(sin) / half < rows) rows = numel(sin) / half;
+    if (cos->rank == 0 || sin->rank == 0) rows = 0xffffffffu;
+    if (rows == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: empty RoPE tables");
+    L.fused = true;
+    L.q = tptr<const void>(q);
+    L.k_in = tptr<const __half>(k), L.v_in = tptr<const __half>(v);
+    L.cos_t = tptr<const __half>(cos), L.sin_t = tptr<const __half>(sin);
+    L.q_rot_out = q_rot->buffer ? tptr<__half>(q_rot) : nullptr;
+    L.qin_stride_b = p->d_model, L.kvin_stride_b = p->kv_dim, L.qrot_stride_b = p->d_model;
+    L.rope_normal = p->rope_mode == FA_ROPE_MODE_NORMAL;
+    L.apply_rope = p->no_rope_layer_step == 0 || ((p->layer_idx + 1u) % p->no_rope_layer_step) != 0u;
+    L.table_rows = (uint32_t)(rows > 0xffffffffu ? 0xffffffffu : rows);
+    L.n_heads = p->n_heads, L.n_kv_heads = p->n_kv_heads, L.head_dim = p->head_dim;
+    L.q_stride_b = p->d_model, L.q_stride_h = p->head_dim;
+    L.out_stride_b = p->d_model, L.out_stride_h = p->head_dim;
+    L.scale = 1.0f / sqrtf((float)p->head_dim);
+    return FA_OK;
+}
+
+extern "C" fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                          const fa_tensor_arg *v, const fa_tensor_arg *q_rot,
+                                          const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
+                                          const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                          const fa_tensor_arg *output, const fa_kv_prep_fused_params *p,
+                                          const uint32_t *d_position, uint32_t kv_len_bound) {
+    FA_NEED(ctx, "ctx");
+    DecodeLaunch L;
+    memset(&L, 0, sizeof(L));
+    FA_NEED(p, "params");
+    FA_TRY(fused_common(q, k, v, q_rot, cos, sin, p, 1, L));
+    FA_TRY(check_tensor(k_cache, "k_cache", FA_DTYPE_F16, 0, 16));
+    FA_TRY(check_tensor(v_cache, "v_cache", FA_DTYPE_F16, 0, 16));
+    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, p->d_model, 2));
+    KvLayout kl, vl;
+    FA_TRY(kv_layout(k_cache, "k_cache", p->head_dim, kl));
+    FA_TRY(kv_layout(v_cache, "v_cache", p->head_dim, vl));
+    if (kl.n_kv_heads != p->n_kv_heads || vl.n_kv_heads != p->n_kv_heads || kl.capacity != vl.capacity)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: caches [%u,%u] / [%u,%u] do not match n_kv_heads %u", kl.n_kv_heads,
+                       kl.capacity, vl.n_kv_heads, vl.capacity, p->n_kv_heads);
+    if (p->max_seq_len != kl.capacity)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: max_seq_len %u != cache capacity %u", p->max_seq_len, kl.capacity);
+    L.k = tptr<const void>(k_cache), L.v = tptr<const __half>(v_cache), L.out = tptr<__half>(output);
+    L.k_stride_h = kl.stride_h, L.v_stride_h = vl.stride_h;
+    L.batch = 1, L.capacity = kl.capacity, L.kv_len_add = 1;
+    if (d_position) {
+        if (kv_len_bound == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_len_bound is 0");
+        L.d_len = d_position, L.d_len_stride = 0;
+        L.kv_len_bound = kv_len_bound < L.capacity ? kv_len_bound : L.capacity;
+    } else {
+        if ((uint64_t)p->position_offset + 1 > kl.capacity)
+            return fa_fail(FA_ERR_INVALID_OPERATION, "Invalid operation: position_offset %u + seq_len 1 exceeds max_seq_len %u",
+                           p->position_offset, kl.capacity);
+        if ((uint64_t)p->position_offset + 1 > L.table_rows)
+            return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: RoPE tables hold %u rows, %u needed", L.table_rows, p->position_offset + 1);
+        L.kv_len = p->position_offset + 1, L.kv_len_bound = L.kv_len;
+    }
+    return fa_launch_decode(ctx, L);
+}
+
+extern "C" fa_status fa_decode_step_fused_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                                const fa_tensor_arg *v, const fa_tensor_arg *q_rot,
+                                                const fa_paged_kv *cache, const fa_tensor_arg *cos,
+                                                const fa_tensor_arg *sin, const fa_tensor_arg *output,
+                                                const fa_kv_prep_fused_params *p, uint32_t kv_len_bound) {
+    FA_NEED(ctx, "ctx");
+    FA_TRY(check_paged(cache));
+    FA_NEED(p, "params");
+    if (!cache->seq_lens) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: seq_lens");
+    DecodeLaunch L;
+    memset(&L, 0, sizeof(L));
+    FA_TRY(fused_common(q, k, v, q_rot, cos, sin, p, cache->n_seqs, L));
+    if (p->head_dim != cache->head_dim || p->n_kv_heads != cache->n_kv_heads)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: params (Hkv %u, D %u) do not match the paged cache (Hkv %u, D %u)",
+                       p->n_kv_heads, p->head_dim, cache->n_kv_heads, cache->head_dim);
+    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, (size_t)cache->n_seqs * p->d_model, 2));
+    if (kv_len_bound == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_len_bound is 0");
+    L.k = cache->k_pool, L.v = (const __half *)cache->v_pool, L.out = tptr<__half>(output);
+    L.batch = cache->n_seqs;
+    L.d_len = cache->seq_lens, L.d_len_stride = 1, L.kv_len_add = 1;
+    L.capacity = cache->max_blocks_per_seq * cache->block_size;
+    L.kv_len_bound = kv_len_bound < L.capacity ? kv_len_bound : L.capacity;
+    L.paged = true, L.block_table = cache->block_table, L.bt_stride = cache->max_blocks_per_seq;
+    L.block_size = cache->block_size;
+    return fa_launch_decode(ctx, L);
+}
+
 extern "C" fa_status fa_flash_decode_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_paged_kv *cache,
                                            const fa_tensor_arg *output, uint32_t n_heads, uint32_t kv_len_add,
                                            uint32_t kv_len_bound) {

@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstring>
 #include <string>
 #include <vector>
 
@@ -109,6 +110,12 @@ struct DecodeLaunch {
     const float *q_scale;
     const __half *k_scale;
     uint32_t ks_stride;
+    // fused RoPE + append of the new token (q is then the raw projection row [H*D])
+    bool fused;
+    const __half *k_in, *v_in, *cos_t, *sin_t;
+    __half *q_rot_out;
+    uint64_t qin_stride_b, kvin_stride_b, qrot_stride_b;
+    uint32_t rope_normal, apply_rope, table_rows;
 };
 fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &a);
 

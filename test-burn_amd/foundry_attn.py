@@ -93,6 +93,9 @@ PROTOTYPES = {
     "fa_kv_prep_fused_dyn": [_vp, _PT, _PT, _PT, _PT, _PT, _PT, _PT, _PT, C.POINTER(KvPrepFusedParams), _vp],
     "fa_flash_attention": [_vp, _PT, _PT, _PT, _PT, _i, _u32, _u32, _u32, _u32, _u32, _i],
     "fa_flash_decode_dyn": [_vp, _PT, _PT, _PT, _PT, _u32, _u32, _vp, _u32, _u32],
+    "fa_decode_step_fused": [_vp, _PT, _PT, _PT, _PT, _PT, _PT, _PT, _PT, _PT, C.POINTER(KvPrepFusedParams), _vp, _u32],
+    "fa_decode_step_fused_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _PT, _PT, _PT,
+                                   C.POINTER(KvPrepFusedParams), _u32],
     "fa_set_decode_variant": [_vp, C.POINTER(DecodeVariant)],
     "fa_kv_prep_fused_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _u32, _PT, _PT,
                                C.POINTER(KvPrepFusedParams)],
@@ -286,6 +289,21 @@ class Foundry:
     def flash_decode_dyn(self, q, k, v, out, n_heads, head_dim, d_position, kv_len_add, kv_len_bound):
         check(self.lib.fa_flash_decode_dyn(self.h, C.byref(q), C.byref(k), C.byref(v), C.byref(out), n_heads, head_dim,
                                            d_position.ptr, kv_len_add, kv_len_bound))
+
+    def decode_step_fused(self, q, k, v, q_rot, k_cache, v_cache, cos, sin, out, params, d_position=None,
+                          kv_len_bound=0):
+        if q_rot is None:
+            q_rot = TensorArg()
+        a = [C.byref(x) for x in (q, k, v, q_rot, k_cache, v_cache, cos, sin, out)]
+        check(self.lib.fa_decode_step_fused(self.h, *a, C.byref(params), None if d_position is None else d_position.ptr,
+                                            kv_len_bound))
+
+    def decode_step_fused_paged(self, q, k, v, q_rot, cache, cos, sin, out, params, kv_len_bound):
+        if q_rot is None:
+            q_rot = TensorArg()
+        check(self.lib.fa_decode_step_fused_paged(self.h, C.byref(q), C.byref(k), C.byref(v), C.byref(q_rot),
+                                                  C.byref(cache), C.byref(cos), C.byref(sin), C.byref(out),
+                                                  C.byref(params), kv_len_bound))
 
     def kv_prep_fused_paged(self, q, k, v, q_rot, cache, seq_index, cos, sin, params):
         check(self.lib.fa_kv_prep_fused_paged(self.h, C.byref(q), C.byref(k), C.byref(v), C.byref(q_rot),

@@ -194,3 +194,113 @@ def test_decode_errors():
         f.set_decode_variant(100, 0)
     assert e.value.variant == "OperationNotSupported"
     f.synchronize()
+
+
+@pytest.mark.parametrize("H,Hkv,D,mode,base,layer,step", [
+    (14, 2, 64, fa.ROPE_NEOX, 1e6, 0, 0),      # Qwen2.5-0.5B
+    (24, 8, 128, fa.ROPE_NORMAL, 5e5, 0, 0),   # Llama-3.2-3B
+    (16, 4, 128, fa.ROPE_NORMAL, 5e6, 3, 4),   # SmolLM3 NoPE layer
+    (16, 4, 128, fa.ROPE_NORMAL, 5e6, 4, 4),   # SmolLM3 RoPE layer
+    (16, 2, 128, fa.ROPE_NEOX, 1e6, 0, 0),     # Qwen2.5-3B
+    (24, 2, 64, fa.ROPE_NEOX, 1e4, 0, 0),      # group 12: three workgroups share a KV head
+])
+def test_fused_decode_step_equals_separate_ops(H, Hkv, D, mode, base, layer, step):
+    """fa_decode_step_fused == fa_kv_prep_fused + fa_flash_attention: caches and q_rot bit-exact against the
+    oracle, outputs bit-identical to the two-op path."""
+    announce("fused step", H, Hkv, D, mode, layer, step)
+    f = ctx()
+    rng = np.random.default_rng(H + D + layer)
+    cap = 704
+    cos, sin = fa.rope_tables(base, D, cap)
+    dcos, dsin = f.array(cos), f.array(sin)
+    f.set_decode_variant(64, 0)
+    try:
+        for pos in (0, 1, 62, 63, 64, 127, 128, 300, 703):
+            kc0 = h16(rng.normal(size=(Hkv, cap, D)))
+            vc0 = h16(rng.normal(size=(Hkv, cap, D)))
+            q, k, v = (h16(rng.normal(size=(1, n * D))) for n in (H, Hkv, Hkv))
+            ok, ov = kc0.copy(), vc0.copy()
+            want_qr = orc.kv_prep_fused(q, k, v, ok, ov, cos, sin,
+                                        orc.make_params(H, Hkv, D, 1, pos, cap, rope_mode=mode, layer_idx=layer,
+                                                        no_rope_layer_step=step))
+            want = orc.sdpa_decode(want_qr[:, 0].copy(), ok, ov, H, Hkv, D, cap, pos + 1).reshape(H, D)
+            dq, dk, dv = f.array(q), f.array(k), f.array(v)
+            # two-op path
+            kc_a, vc_a, qr_a, out_a = f.array(kc0), f.array(vc0), f.zeros((H, 1, D)), f.zeros((1, H * D))
+            p = fa.KvPrepFusedParams.make(H, Hkv, D, 1, pos, cap, mode, layer, step)
+            f.kv_prep_fused(dq.arg(), dk.arg(), dv.arg(), qr_a.arg(), kc_a.arg(), vc_a.arg(), dcos.arg(), dsin.arg(), p)
+            f.flash_attention(qr_a.arg((1, H * D)), kc_a.arg(), vc_a.arg(), out_a.arg(), True, pos, H, D, pos + 1, 1)
+            # fused, static position
+            kc_b, vc_b, qr_b, out_b = f.array(kc0), f.array(vc0), f.zeros((H, 1, D)), f.zeros((1, H * D))
+            f.decode_step_fused(dq.arg(), dk.arg(), dv.arg(), qr_b.arg(), kc_b.arg(), vc_b.arg(), dcos.arg(), dsin.arg(),
+                                out_b.arg(), p)
+            # fused, device position, no q_rot output
+            kc_c, vc_c, out_c = f.array(kc0), f.array(vc0), f.zeros((1, H * D))
+            dpos = f.array(np.array([pos], np.uint32))
+            p0 = fa.KvPrepFusedParams.make(H, Hkv, D, 1, 0, cap, mode, layer, step)
+            f.decode_step_fused(dq.arg(), dk.arg(), dv.arg(), None, kc_c.arg(), vc_c.arg(), dcos.arg(), dsin.arg(),
+                                out_c.arg(), p0, d_position=dpos, kv_len_bound=cap)
+            f.synchronize()
+            for kc_x, vc_x in ((kc_a, vc_a), (kc_b, vc_b), (kc_c, vc_c)):
+                assert np.array_equal(bits(kc_x.download()), bits(ok)), pos
+                assert np.array_equal(bits(vc_x.download()), bits(ov)), pos
+            assert np.array_equal(bits(qr_a.download()), bits(want_qr)), pos
+            assert np.array_equal(bits(qr_b.download()), bits(want_qr)), pos
+            oa, ob, oc = out_a.download(), out_b.download(), out_c.download()
+            assert max_abs(oa.reshape(H, D), want) <= TOL, pos
+            assert np.array_equal(bits(ob), bits(oa)), pos
+            assert max_abs(oc.reshape(H, D), want) <= TOL, pos
+            for b in (dq, dk, dv, kc_a, vc_a, qr_a, out_a, kc_b, vc_b, qr_b, out_b, kc_c, vc_c, out_c, dpos):
+                b.free()
+    finally:
+        f.set_decode_variant(0, 0)
+
+
+def test_fused_step_errors_and_overflow_guard():
+    announce("fused step errors")
+    f = ctx()
+    H, Hkv, D, cap = 8, 2, 64, 64
+    q, k, v = f.zeros((1, H * D)), f.zeros((1, Hkv * D)), f.zeros((1, Hkv * D))
+    kc, vc, out = f.zeros((Hkv, cap, D)), f.zeros((Hkv, cap, D)), f.zeros((1, H * D))
+    cos, sin = f.zeros((cap, D // 2)), f.zeros((cap, D // 2))
+    with pytest.raises(fa.FoundryError) as e:
+        f.decode_step_fused(q.arg(), k.arg(), v.arg(), None, kc.arg(), vc.arg(), cos.arg(), sin.arg(), out.arg(),
+                            fa.KvPrepFusedParams.make(H, Hkv, D, 1, cap, cap))
+    assert e.value.variant == "InvalidOperation"
+    with pytest.raises(fa.FoundryError) as e:
+        f.decode_step_fused(q.arg(), k.arg(), v.arg(), None, kc.arg(), vc.arg(), cos.arg(), sin.arg(), out.arg(),
+                            fa.KvPrepFusedParams.make(H, Hkv, D, 2, 0, cap))
+    assert e.value.variant == "InvalidShape"
+    # a device position beyond the capacity appends nothing
+    dpos = f.array(np.array([cap + 5], np.uint32))
+    f.decode_step_fused(q.arg(), k.arg(), v.arg(), None, kc.arg(), vc.arg(), cos.arg(), sin.arg(), out.arg(),
+                        fa.KvPrepFusedParams.make(H, Hkv, D, 1, 0, cap), d_position=dpos, kv_len_bound=cap)
+    f.synchronize()
+    assert not kc.download().any()
+
+
+def test_in_kernel_merge_is_bit_identical_to_merge_kernel_over_many_launches():
+    """The merge by the last-arriving workgroup reads partials written by other workgroups of the same launch;
+    it must give the same bits as the two-launch merge, launch after launch."""
+    announce("merge stress")
+    f = ctx()
+    rng = np.random.default_rng(123)
+    H, Hkv, D, cap = 24, 8, 128, 4096
+    q = h16(rng.normal(size=(H, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    dq, dk, dv = f.array(q), f.array(k), f.array(v)
+    oa, ob = f.zeros((1, H * D)), f.zeros((1, H * D))
+    lens = [int(x) for x in rng.integers(65, cap, size=40)] + [cap, 64 * 17 + 1]
+    try:
+        for kps in (64, 128, 0):
+            for n in lens:
+                f.set_decode_variant(kps, 1)
+                f.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), oa.arg(), True, n - 1, H, D, n, 1)
+                f.set_decode_variant(kps, 0)
+                for _ in range(3):
+                    f.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), ob.arg(), True, n - 1, H, D, n, 1)
+                    f.synchronize()
+                    assert np.array_equal(bits(oa.download()), bits(ob.download())), (kps, n)
+    finally:
+        f.set_decode_variant(0, 0)

@@ -177,3 +177,46 @@ def test_paged_decode_multi_step_advances_lengths():
             assert max_abs(got[b], want) <= TOL, (t, b)
     assert np.array_equal(pg.dlens.download(), np.asarray(lens, np.uint32) + steps)
     pg.free()
+
+
+def test_paged_fused_step_equals_separate_ops():
+    """fa_decode_step_fused_paged == fa_kv_prep_decode_paged + fa_flash_decode_paged (bit-identical)."""
+    announce("paged fused step")
+    f = ctx()
+    rng = np.random.default_rng(17)
+    H, Hkv, D, bs = 16, 2, 128, 16
+    lens = [512, 15, 16, 1, 1000, 63, 64, 0]
+    B = len(lens)
+    ks = [h16(rng.normal(size=(Hkv, n + 1, D))) for n in lens]
+    vs = [h16(rng.normal(size=(Hkv, n + 1, D))) for n in lens]
+    q, kn, vn = (h16(rng.normal(size=(B, n * D))) for n in (H, Hkv, Hkv))
+    cos, sin = fa.rope_tables(1e6, D, 1024)
+    dcos, dsin = f.array(cos), f.array(sin)
+    dq, dkn, dvn = f.array(q), f.array(kn), f.array(vn)
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, B, 0, 0, fa.ROPE_NEOX)
+    outs = []
+    for fused in (False, True):
+        pg = Paged(f, np.random.default_rng(3), lens, Hkv, D, bs)
+        pg.fill_from(ks, vs)
+        pg.upload()
+        dqr, dout = f.zeros((B, H, D)), f.zeros((B, H * D))
+        if fused:
+            f.decode_step_fused_paged(dq.arg(), dkn.arg(), dvn.arg(), dqr.arg(), pg.desc, dcos.arg(), dsin.arg(),
+                                      dout.arg(), p, 1024)
+        else:
+            f.kv_prep_decode_paged(dq.arg(), dkn.arg(), dvn.arg(), dqr.arg(), pg.desc, dcos.arg(), dsin.arg(), p)
+            f.flash_decode_paged(dqr.arg(), pg.desc, dout.arg(), H, 1, 1024)
+        f.synchronize()
+        outs.append((dqr.download(), dout.download(), pg.dk.download(), pg.dv.download()))
+        pg.free()
+    for a, b in zip(outs[0], outs[1]):
+        assert np.array_equal(bits(a), bits(b))
+    # and against the oracle for two of the sequences
+    for b in (0, 7):
+        n = lens[b]
+        kc, vc = np.zeros((Hkv, n + 1, D), np.float16), np.zeros((Hkv, n + 1, D), np.float16)
+        kc[:, :n], vc[:, :n] = ks[b][:, :n], vs[b][:, :n]
+        qr = orc.kv_prep_fused(q[b:b + 1], kn[b:b + 1], vn[b:b + 1], kc, vc, cos, sin,
+                               orc.make_params(H, Hkv, D, 1, n, n + 1, rope_mode=0))
+        want = orc.sdpa_decode(qr[:, 0].copy(), kc, vc, H, Hkv, D, n + 1, n + 1).reshape(H, D)
+        assert max_abs(outs[1][1].reshape(B, H, D)[b], want) <= TOL
