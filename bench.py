@@ -61,13 +61,20 @@ def make_llama3b_decode(f, rng, start_ctx, room):
     return st
 
 
-def enqueue_step(f, st, slot):
-    """One decode step: per layer, fused RoPE + KV append then flash decode; then advance the position."""
+def enqueue_step(f, st, slot, fused=True):
+    """One decode step: per layer, RoPE + KV append + flash decode (one fused launch, or the two separate ops);
+    then advance the position."""
     L, H, Hkv, D, cap = st["L"], st["H"], st["Hkv"], st["D"], st["cap"]
     dm, kvd = H * D, Hkv * D
     for i in range(L):
         qo = (slot * L + i) * dm * 2
         ko = (slot * L + i) * kvd * 2
+        if fused:
+            f.decode_step_fused(st["dq"].arg((1, dm), offset=qo), st["dk"].arg((1, kvd), offset=ko),
+                                st["dv"].arg((1, kvd), offset=ko), None, st["kc"][i].arg(), st["vc"][i].arg(),
+                                st["dcos"].arg(), st["dsin"].arg(), st["dout"].arg((1, dm), offset=i * dm * 2),
+                                st["params"], d_position=st["dpos"], kv_len_bound=cap)
+            continue
         f.kv_prep_fused(st["dq"].arg((1, dm), offset=qo), st["dk"].arg((1, kvd), offset=ko),
                         st["dv"].arg((1, kvd), offset=ko), st["dqr"].arg((1, dm), offset=i * dm * 2), st["kc"][i].arg(),
                         st["vc"][i].arg(), st["dcos"].arg(), st["dsin"].arg(), st["params"], d_position=st["dpos"])
@@ -76,17 +83,16 @@ def enqueue_step(f, st, slot):
     f.u32_add(st["dpos"], 1, 1)
 
 
-def decode_bytes_per_launch(st, n):
-    """Algorithmic HBM bytes of one flash-decode launch at kv_len n: K and V read once per KV head, q read, out written."""
-    return 2 * st["Hkv"] * n * st["D"] * 2 + 2 * st["H"] * st["D"] * 2
+def layer_bytes(st, n):
+    """Algorithmic HBM bytes of one layer of one decode step at kv_len n (after the append): K and V read once per
+    KV head (2*Hkv*n*D*2), the appended K/V rows written (2*Hkv*D*2), q read and out written (2*H*D*2), the new
+    token's raw k/v read (2*Hkv*D*2) and one cos + one sin row (2*(D/2)*2)."""
+    H, Hkv, D = st["H"], st["Hkv"], st["D"]
+    return 2 * Hkv * n * D * 2 + 2 * Hkv * D * 2 + 2 * H * D * 2 + 2 * Hkv * D * 2 + 2 * (D // 2) * 2
 
 
 def step_bytes(st, n):
-    """Algorithmic HBM bytes of one whole decode step (all layers) at kv_len n: decode traffic + append writes +
-    q_rot write/read + cos/sin row."""
-    per_layer = (decode_bytes_per_launch(st, n) + 2 * st["Hkv"] * st["D"] * 2 + (st["H"] + 2 * st["Hkv"]) * st["D"] * 2 +
-                 st["H"] * st["D"] * 2 + 2 * (st["D"] // 2) * 2)
-    return st["L"] * per_layer
+    return st["L"] * layer_bytes(st, n)
 
 
 def run_steps(f, st, graph16, graph1, steps, room, history=None):
@@ -160,6 +166,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--keys-per-split", type=int, default=0)
     ap.add_argument("--merge", type=int, default=0)
+    ap.add_argument("--unfused", action="store_true", help="two launches per layer (KvPrepFused, FlashAttention)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is built and measured on a single MI355X (--gpus 1); "
@@ -176,11 +183,12 @@ def main():
     st = make_llama3b_decode(f, rng, 8192, room)
 
     f.start_capture()
+    fused = not args.unfused
     for s in range(GRAPH_STEPS):
-        enqueue_step(f, st, s)
+        enqueue_step(f, st, s, fused)
     graph16 = f.end_capture()
     f.start_capture()
-    enqueue_step(f, st, 0)
+    enqueue_step(f, st, 0, fused)
     graph1 = f.end_capture()
 
     # warmup (untimed), then reset the position so the timed window starts at 8192 context
@@ -203,14 +211,14 @@ def main():
     f.profile_reset()
     f.profile_enable(True)
     for s in range(prof_steps):
-        enqueue_step(f, st, s % GRAPH_STEPS)
-    n_dec, ms_dec = f.profile_query("flash_decode_splitk_kernel")
-    n_prep, ms_prep = f.profile_query("kv_prep_fused")
+        enqueue_step(f, st, s % GRAPH_STEPS, fused)
+    kernel = "fused_rope_append_decode_kernel" if fused else "flash_decode_mfma_kernel"
+    n_dec, ms_dec = f.profile_query(kernel)
     f.profile_enable(False)
     f.profile_reset()
     avg_dec_s = ms_dec / 1e3 / max(1, n_dec)
     avg_n = st["start"] + (prof_steps + 1) / 2.0
-    achieved = decode_bytes_per_launch(st, avg_n) / avg_dec_s / 1e9
+    achieved = layer_bytes(st, avg_n) / avg_dec_s / 1e9
 
     ns = [st["start"] + 1 + (i % room) for i in range(args.steps)]
     bytes_total = sum(step_bytes(st, n) for n in ns)
@@ -227,7 +235,7 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": "llama3.2-3b decode attention: 28 layers x (fused RoPE+KV append, flash decode), batch 1, "
+        "config": {"workload": "llama3.2-3b decode attention: 28 layers x (RoPE + KV append + flash decode), batch 1, "
                                "H24/Hkv8/D128, f16 contiguous KV cache, kv_len 8193..%d, %d-step HIP graphs"
                                % (st["start"] + min(args.steps, room), GRAPH_STEPS),
                    "device": name, "compute_units": cus},
@@ -235,9 +243,8 @@ def main():
         "whole_step_hbm_frac_of_peak": bytes_total / dt / 1e9 / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
-                     "kernel": "flash_decode_splitk_kernel", "avg_launch_us": avg_dec_s * 1e6, "launches": n_dec,
-                     "bytes_per_launch": decode_bytes_per_launch(st, avg_n),
-                     "kv_prep_avg_launch_us": ms_prep / max(1, n_prep) * 1e3},
+                     "kernel": kernel, "avg_launch_us": avg_dec_s * 1e6, "launches": n_dec,
+                     "bytes_per_launch": layer_bytes(st, avg_n)},
         "parity": {"cache_bit_exact": cache_ok, "decode_max_abs_err": err},
     }
     if not args.no_cpu:

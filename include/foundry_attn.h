@@ -205,8 +205,8 @@ fa_status fa_flash_decode_dyn(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tens
  * reference fuses RoPE into decode in RopeFlashDecodeStep (src/metals/flashattention/step.rs:16-306).
  * q/k/v are the raw projections of the new token ([1, d_model] / [1, kv_dim]); the token is rotated, appended at
  * row P of the caches and attended together with rows [0, P), where P = *d_position if d_position != NULL,
- * else params->position_offset. Results are bit-identical to calling the two ops one after the other: the cache
- * rows and q_rot carry the same bits, and the attention reads the same f16 values. q_rot may have a NULL buffer
+ * else params->position_offset. The cache rows and q_rot carry the same bits as after calling the two ops one
+ * after the other and the attention reads the same f16 values (outputs agree up to f32 summation order). q_rot may have a NULL buffer
  * (then it is not written). kv_len_bound >= P + 1 as in fa_flash_decode_dyn. params->seq_len must be 1. */
 fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
                                const fa_tensor_arg *q_rot, const fa_tensor_arg *k_cache,
@@ -215,7 +215,8 @@ fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_ten
                                const uint32_t *d_position, uint32_t kv_len_bound);
 
 /* Tuning override, the counterpart of FlashDecodeVariant + METALLIC_FA_DECODE_* (src/metals/flashattention/
- * variants.rs:36-140). keys_per_split: context partition per workgroup (multiple of 64; 0 = auto).
+ * variants.rs:36-140). keys_per_split: context partition per workgroup (multiple of 64, rounded up to the
+ * kernel's 64-key tile; 0 = auto).
  * merge: 0 = merged by the last workgroup to finish (one launch), 1 = separate merge kernel.
  * Environment: FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT, FOUNDRY_ATTN_DECODE_MERGE (read at fa_ctx_create). */
 typedef struct fa_decode_variant {

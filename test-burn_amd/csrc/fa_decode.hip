@@ -3,10 +3,9 @@
 
 namespace {
 
-// Heads of a group served by one workgroup: the largest supported count that divides the group.
+// Heads of a group served by one workgroup: the largest divisor of the group that fits the MFMA N dimension.
 int heads_per_workgroup(uint32_t group) {
-    static const int opts[] = {8, 7, 4, 3, 2, 1};
-    for (int o : opts)
+    for (int o = fa_decode::MAX_GT; o > 1; --o)
         if (group % (uint32_t)o == 0) return o;
     return 1;
 }
@@ -22,20 +21,24 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     const uint32_t bound = L.kv_len_bound < L.capacity ? L.kv_len_bound : L.capacity;
     if (bound == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "flash decode: kv_len bound is 0");
 
-    // Context partition per workgroup: aim at ~3 workgroups per CU over the whole launch.
+    // Context partition per workgroup, in 64-key tiles. Every workgroup should be resident at once (2 per CU):
+    // a workgroup that has to wait for a slot starts after the others have drained the memory queues and
+    // lengthens the launch by its whole latency. Within that limit every wave gets as few tiles as possible
+    // (one if the context allows), so that all of the data is requested in the first instant.
     uint32_t chunk = ctx->decode_variant.keys_per_split;
     if (chunk == 0) {
-        const uint64_t total_keys = (uint64_t)L.batch * ny * bound;
-        const uint64_t target_wgs = (uint64_t)(ctx->n_cus > 0 ? ctx->n_cus : 256) * 3;
-        uint64_t c = (total_keys + target_wgs - 1) / target_wgs;
-        c = (c + 63) / 64 * 64;
-        if (c < 64) c = 64;
-        if (c > 2048) c = 2048;
-        chunk = (uint32_t)c;
+        const uint32_t tiles = ceil_div_u32(bound, (uint32_t)TK);
+        const uint64_t groups = (uint64_t)L.batch * ny;
+        const uint64_t slots = (uint64_t)(ctx->n_cus > 0 ? ctx->n_cus : 256) * 2;
+        uint32_t rounds = 1;  // tiles per wave
+        while (rounds < 4 && groups * ceil_div_u32(tiles, (uint32_t)NW * rounds) > slots) ++rounds;
+        chunk = (uint32_t)NW * rounds * (uint32_t)TK;
     }
-    if (chunk % 64 != 0)
-        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "decode keys_per_split must be a multiple of 64, got %u", chunk);
+    chunk = (chunk + TK - 1) / TK * TK;
     const uint32_t S = ceil_div_u32(bound, chunk);
+    // a contiguous cache slab is addressed with 32-bit byte offsets (tile base included)
+    if (!L.paged && ((uint64_t)L.capacity + chunk + TK) * L.head_dim * 2 >= (1ull << 32))
+        return fa_fail(FA_ERR_INVALID_SHAPE, "flash decode: one KV head of the contiguous cache must stay below 4 GiB");
 
     DecodeDev a;
     memset(&a, 0, sizeof(a));
@@ -46,6 +49,7 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     a.d_len = L.d_len, a.block_table = L.block_table;
     a.kv_len = L.kv_len, a.d_len_stride = L.d_len_stride, a.kv_len_add = L.kv_len_add, a.kv_len_bound = bound;
     a.capacity = L.capacity, a.chunk = chunk, a.n_kv_heads = L.n_kv_heads, a.sub_per_kv = sub_per_kv;
+    a.gt = (uint32_t)gt;
     a.bt_stride = L.bt_stride, a.block_size = L.block_size;
     a.merge_in_kernel = ctx->decode_variant.merge == 0 ? 1u : 0u;
     a.scale_log2e = L.scale * 1.4426950408889634f;
@@ -71,7 +75,7 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     else if (L.paged)
         mode = MODE_PAGED;
     dim3 grid(S, ny, L.batch);
-    if (L.head_dim == 128) return fa_decode_launch_d128(ctx, a, grid, mode, gt);
-    if (L.head_dim == 64) return fa_decode_launch_d64(ctx, a, grid, mode, gt);
+    if (L.head_dim == 128) return fa_decode_launch_d128(ctx, a, grid, mode);
+    if (L.head_dim == 64) return fa_decode_launch_d64(ctx, a, grid, mode);
     return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Flash Decode only supports head_dim=64 or 128, got %u", L.head_dim);
 }

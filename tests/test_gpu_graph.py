@@ -70,7 +70,7 @@ def test_per_kernel_profiling_counts_launches():
     try:
         for _ in range(5):
             f.flash_attention(dq.arg(), dk.arg(), dv.arg(), do.arg(), True, N - 1, H, D, N, 1)
-        n, ms = f.profile_query("flash_decode_splitk")
+        n, ms = f.profile_query("flash_decode_mfma")
         assert n == 5 and 0.0 < ms < 50.0
         with pytest.raises(fa.FoundryError):
             f.start_capture()

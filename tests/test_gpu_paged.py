@@ -180,7 +180,8 @@ def test_paged_decode_multi_step_advances_lengths():
 
 
 def test_paged_fused_step_equals_separate_ops():
-    """fa_decode_step_fused_paged == fa_kv_prep_decode_paged + fa_flash_decode_paged (bit-identical)."""
+    """fa_decode_step_fused_paged == fa_kv_prep_decode_paged + fa_flash_decode_paged: q_rot and pools bit-identical,
+    outputs equal up to f32 summation order."""
     announce("paged fused step")
     f = ctx()
     rng = np.random.default_rng(17)
@@ -209,8 +210,11 @@ def test_paged_fused_step_equals_separate_ops():
         f.synchronize()
         outs.append((dqr.download(), dout.download(), pg.dk.download(), pg.dv.download()))
         pg.free()
-    for a, b in zip(outs[0], outs[1]):
-        assert np.array_equal(bits(a), bits(b))
+    for i, (a, b) in enumerate(zip(outs[0], outs[1])):
+        if i == 1:
+            assert max_abs(a, b) <= 2e-3
+        else:
+            assert np.array_equal(bits(a), bits(b))
     # and against the oracle for two of the sequences
     for b in (0, 7):
         n = lens[b]
