@@ -156,6 +156,30 @@ def check_against_oracle(f, st, history):
     return cache_ok, err
 
 
+# HBM bytes per launch of the fused decode kernel from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+# profiles/decode_llama3b_8k_hbm_counters.txt (scaled by the copy kernel of known size); a counter run cannot be made
+# from inside this script, so the figure is carried here and re-measured whenever the kernel changes.
+MEASURED_TRAFFIC_BYTES = 35.15e6
+
+
+def calibration_copy(f, reps=3):
+    """A plain copy of known size through the library's gather kernel (pool rows -> contiguous rows): the HBM
+    counters of a profiler run read against it give the factor between counter units and bytes."""
+    Hkv, D, bs, tokens = 8, 128, 16, 65536
+    nblk = tokens // bs
+    k_pool, v_pool = f.zeros((nblk, Hkv, bs, D)), f.zeros((nblk, Hkv, bs, D))
+    bt, lens = f.array(np.arange(nblk, dtype=np.int32).reshape(1, nblk)), f.array(np.array([tokens], np.uint32))
+    desc = fa.paged_kv(k_pool, v_pool, bt, lens, nblk, Hkv, bs, D, 1, nblk)
+    k_out, v_out = f.empty((Hkv, tokens, D)), f.empty((Hkv, tokens, D))
+    for _ in range(reps):
+        f.paged_gather(desc, 0, tokens, k_out, v_out, tokens)
+    f.synchronize()
+    nbytes = 2 * Hkv * tokens * D * 2  # read once, written once
+    for b in (k_pool, v_pool, bt, lens, k_out, v_out):
+        b.free()
+    return {"kernel": "paged_gather_kernel", "launches": reps, "bytes_read": nbytes, "bytes_written": nbytes}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -165,8 +189,12 @@ def main():
     ap.add_argument("--cpu-sample-steps", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--keys-per-split", type=int, default=0)
-    ap.add_argument("--merge", type=int, default=0)
+    ap.add_argument("--merge", type=int, default=1)
     ap.add_argument("--unfused", action="store_true", help="two launches per layer (KvPrepFused, FlashAttention)")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run a copy kernel of known size (reference point for profiler HBM counters)")
+    ap.add_argument("--traffic-bytes", type=float, default=MEASURED_TRAFFIC_BYTES,
+                    help="measured HBM bytes per launch of the dominant kernel (from profiler counters) to report")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is built and measured on a single MI355X (--gpus 1); "
@@ -214,6 +242,7 @@ def main():
         enqueue_step(f, st, s % GRAPH_STEPS, fused)
     kernel = "fused_rope_append_decode_kernel" if fused else "flash_decode_mfma_kernel"
     n_dec, ms_dec = f.profile_query(kernel)
+    n_mrg, ms_mrg = f.profile_query("flash_decode_merge_kernel")
     f.profile_enable(False)
     f.profile_reset()
     avg_dec_s = ms_dec / 1e3 / max(1, n_dec)
@@ -242,11 +271,14 @@ def main():
         "whole_step_hbm_gbps": bytes_total / dt / 1e9,
         "whole_step_hbm_frac_of_peak": bytes_total / dt / 1e9 / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": args.traffic_bytes,
                      "kernel": kernel, "avg_launch_us": avg_dec_s * 1e6, "launches": n_dec,
-                     "bytes_per_launch": layer_bytes(st, avg_n)},
+                     "bytes_per_launch": layer_bytes(st, avg_n),
+                     "merge_kernel_avg_launch_us": (ms_mrg * 1e3 / n_mrg) if n_mrg else None},
         "parity": {"cache_bit_exact": cache_ok, "decode_max_abs_err": err},
     }
+    if args.calibration_copy:
+        result["calibration_copy"] = calibration_copy(f)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(st, args.cpu_sample_steps)
     print(json.dumps(result))

@@ -215,9 +215,10 @@ fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_ten
                                const uint32_t *d_position, uint32_t kv_len_bound);
 
 /* Tuning override, the counterpart of FlashDecodeVariant + METALLIC_FA_DECODE_* (src/metals/flashattention/
- * variants.rs:36-140). keys_per_split: context partition per workgroup (multiple of 64, rounded up to the
- * kernel's 64-key tile; 0 = auto).
- * merge: 0 = merged by the last workgroup to finish (one launch), 1 = separate merge kernel.
+ * variants.rs:36-140). keys_per_split: context partition per workgroup (rounded up to the kernel's 16-key
+ * block; 0 = auto: one partition per compute unit).
+ * merge: 0 = merged by the last workgroup to finish (one launch), 1 = separate merge kernel (the default of a
+ * new context: measured slightly faster).
  * Environment: FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT, FOUNDRY_ATTN_DECODE_MERGE (read at fa_ctx_create). */
 typedef struct fa_decode_variant {
     uint32_t keys_per_split;

@@ -42,7 +42,7 @@ extern "C" const char *fa_version(void) { return "foundry_attn 0.1 (gfx950)"; }
 
 // ------------------------------------------------------------------------------------------------ profiling scope
 
-FaLaunchScope::FaLaunchScope(fa_ctx *c, const char *n) : ctx(c), name(n) {
+FaLaunchScope::FaLaunchScope(fa_ctx *c, const char *n, bool dispatch_events) : ctx(c), name(n) {
     if (!ctx->profiling || ctx->capturing) return;
     auto get = [&]() -> hipEvent_t {
         if (!ctx->event_pool.empty()) {
@@ -56,13 +56,13 @@ FaLaunchScope::FaLaunchScope(fa_ctx *c, const char *n) : ctx(c), name(n) {
     };
     start = get();
     stop = get();
-    if (start) (void)hipEventRecord(start, ctx->stream);
+    if (start && !dispatch_events) (void)hipEventRecord(start, ctx->stream);
 }
 
 fa_status FaLaunchScope::finish() {
     hipError_t e = hipGetLastError();
     if (start && stop) {
-        (void)hipEventRecord(stop, ctx->stream);
+        if (!tight) (void)hipEventRecord(stop, ctx->stream);
         ctx->prof.push_back({name, start, stop});
     }
     if (e != hipSuccess) return fa_fail(FA_ERR_OPERATION_FAILED, "launch of %s failed: %s", name, hipGetErrorString(e));
@@ -101,7 +101,7 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
         return fa_fail(FA_ERR_OPERATION_FAILED, "hipStreamCreate failed: %s", hipGetErrorString(e));
     }
     ctx->decode_variant.keys_per_split = env_u32("FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT", 0);
-    ctx->decode_variant.merge = env_u32("FOUNDRY_ATTN_DECODE_MERGE", 0);
+    ctx->decode_variant.merge = env_u32("FOUNDRY_ATTN_DECODE_MERGE", 1);
     fa_status s = fa_ensure_workspace(ctx, (size_t)64 << 20);
     if (s == FA_OK) s = fa_ensure_counters(ctx, 4096);
     if (s != FA_OK) {

@@ -21,23 +21,22 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     const uint32_t bound = L.kv_len_bound < L.capacity ? L.kv_len_bound : L.capacity;
     if (bound == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "flash decode: kv_len bound is 0");
 
-    // Context partition per workgroup, in 64-key tiles. Every workgroup should be resident at once (2 per CU):
-    // a workgroup that has to wait for a slot starts after the others have drained the memory queues and
-    // lengthens the launch by its whole latency. Within that limit every wave gets as few tiles as possible
-    // (one if the context allows), so that all of the data is requested in the first instant.
+    // Context partition per workgroup, in 16-key blocks. At most one workgroup per CU: what bounds a small launch
+    // is the number of requests a CU can keep outstanding, so a CU that gets two partitions takes nearly twice as
+    // long and every other one waits for it in the merge. Within that limit the partitions are as small as the
+    // granularity allows, but not below one block per wave.
     uint32_t chunk = ctx->decode_variant.keys_per_split;
     if (chunk == 0) {
-        const uint32_t tiles = ceil_div_u32(bound, (uint32_t)TK);
         const uint64_t groups = (uint64_t)L.batch * ny;
-        const uint64_t slots = (uint64_t)(ctx->n_cus > 0 ? ctx->n_cus : 256) * 2;
-        uint32_t rounds = 1;  // tiles per wave
-        while (rounds < 4 && groups * ceil_div_u32(tiles, (uint32_t)NW * rounds) > slots) ++rounds;
-        chunk = (uint32_t)NW * rounds * (uint32_t)TK;
+        const uint64_t slots = (uint64_t)(ctx->n_cus > 0 ? ctx->n_cus : 256);
+        const uint32_t s_max = groups >= slots ? 1u : (uint32_t)(slots / groups);
+        chunk = ceil_div_u32(ceil_div_u32(bound, s_max), (uint32_t)BK) * BK;
+        if (chunk < (uint32_t)(NW * BK)) chunk = NW * BK;
     }
-    chunk = (chunk + TK - 1) / TK * TK;
+    chunk = (chunk + BK - 1) / BK * BK;
     const uint32_t S = ceil_div_u32(bound, chunk);
     // a contiguous cache slab is addressed with 32-bit byte offsets (tile base included)
-    if (!L.paged && ((uint64_t)L.capacity + chunk + TK) * L.head_dim * 2 >= (1ull << 32))
+    if (!L.paged && ((uint64_t)L.capacity + chunk + MBX * BK) * L.head_dim * 2 >= (1ull << 32))
         return fa_fail(FA_ERR_INVALID_SHAPE, "flash decode: one KV head of the contiguous cache must stay below 4 GiB");
 
     DecodeDev a;

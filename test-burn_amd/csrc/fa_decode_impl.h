@@ -22,12 +22,14 @@
 // four 16-lane rows. The VALU only does the exponentials. Work per 16-key tile is independent of the number of
 // heads served (<= 16).
 //
-// Data movement: a wave owns 64-key tiles (four 16-row MFMA blocks, 32 KiB of K + V at D = 128) and requests a
-// whole tile before it touches any of it; K is read as 16 rows x 64-byte runs per instruction, V as 1 KiB fully
-// contiguous per instruction. One wave per SIMD with 32 KiB each keeps ~128 KiB per CU in flight. The launch is
-// sized so that every workgroup is resident at once (2 per CU) and, where the context allows, every wave owns
-// exactly one tile: a workgroup that waits for a slot, or a wave that fetches a second tile after the first,
-// adds a whole memory latency under load (~4 us) to the launch.
+// Data movement: the unit is a block of 16 keys (one MFMA M dimension; 8 KiB of K + V at D = 128). A workgroup
+// owns one context partition, split evenly over its 8 waves in whole blocks; a wave requests up to 3 blocks
+// (24 KiB) at once, before it touches any of them. K is read as 16 rows x 64-byte runs per instruction, V as 1 KiB
+// fully contiguous per instruction. What bounds a batch-1 launch is not HBM bandwidth but how many requests one CU
+// can keep outstanding, so the bytes must be spread evenly over the CUs: the launch is sized to at most ONE
+// workgroup per CU (a CU that gets two needs nearly twice as long, and every partition waits for the slowest), with
+// partitions cut to 16-key granularity so that all CUs get the same share, and every wave has all of its share
+// in flight from the first instant where the context allows (a second round adds a whole memory latency).
 // Algorithmic HBM bytes per (KV head, key): 2 * D * 2 (K row + V row), independent of the group size.
 //
 // FUSED adds the reference's KvPrepFused arithmetic (src/metals/kv_prep/kv_prep_fused.metal:26-123) for
@@ -46,6 +48,7 @@ typedef float f2_t __attribute__((ext_vector_type(2)));
 typedef int i4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int u4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int u2_t __attribute__((ext_vector_type(2)));
+typedef unsigned int u16_t __attribute__((ext_vector_type(16)));
 typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
 
 union U4H {
@@ -55,11 +58,10 @@ union U4H {
     _Float16 e[8];
 };
 
-constexpr int NW = 4;        // waves per workgroup, one per SIMD: 2 workgroups per CU at <= 256 VGPRs
+constexpr int NW = 8;        // waves per workgroup, two per SIMD: one workgroup per CU at <= 256 VGPRs
 constexpr int NT = NW * 64;  // threads per workgroup
-constexpr int TK = 64;       // keys per tile: four 16-row MFMA blocks, attended as two 32-key halves
-constexpr int MB = TK / 16;  // 16-row MFMA blocks per tile
-constexpr int HB = TK / 32;  // 32-key halves per tile
+constexpr int BK = 16;       // keys per block (MFMA M dimension)
+constexpr int MBX = 3;       // blocks a wave keeps in flight (one round)
 constexpr int MAX_GT = 16;   // query heads served by one workgroup (the MFMA N dimension)
 
 struct DecodeDev {
@@ -228,11 +230,10 @@ __device__ __forceinline__ U4H rope8(const U4H &x, const U4H &mate, const U4H &c
 }
 
 template <int D, bool PAGED, bool SAGE, bool FUSED>
-__global__ void __launch_bounds__(NT, 2) flash_decode_mfma_kernel(DecodeDev a) {
+__global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
     constexpr int KSTEPS = SAGE ? D / 64 : D / 32;  // MFMA steps over head_dim for S^T; 16 B per lane each
     constexpr int SEGS = SAGE ? D / 16 : D / 8;     // 16-byte segments per K row
-    constexpr int VLH = D / 16;                     // 1 KiB V loads per 32-key half
-    constexpr int VLD = HB * VLH;                   // 1 KiB V loads per tile
+    constexpr int VLB = D / 32;                     // 1 KiB V loads per block
     constexpr int VLPR = D / 8;                     // lanes per V row
     constexpr int VRPL = 64 / VLPR;                 // V rows per load
     constexpr int DBLK = D / 16;                    // 16-row blocks of O^T
@@ -272,88 +273,98 @@ __global__ void __launch_bounds__(NT, 2) flash_decode_mfma_kernel(DecodeDev a) {
         return (size_t)key * D;
     };
 
-    // K operand: lane (n, c) reads rows tbase + 16mb + n, 16-byte segment 4j + c in step j.
-    // V tile   : lane reads row tbase + i*VRPL + lane / VLPR, segment lane % VLPR in load i (1 KiB per load).
-    // `lim` = last row that may be addressed (rows up to it are allocated; rows >= kv_len are masked later).
+    // K operand: lane (n, c) reads row n of a block, 16-byte segment 4j + c in step j.
+    // V block  : lane reads row i*VRPL + lane / VLPR, segment lane % VLPR in load i (1 KiB per load).
     // A contiguous cache is read through buffer descriptors that span the (sequence, KV head) slab: one VGPR of
-    // lane offset serves every load of the tile (per-load 64-bit addresses would cost 64 VGPRs next to the 128 of
-    // the tile itself), and rows past the slab read as zero instead of needing a clamp.
-    U4H kk[MB][KSTEPS], vv[VLD];
+    // lane offset serves every load (per-load 64-bit addresses would cost as many VGPRs as the data), and rows past
+    // the slab read as zero instead of needing a clamp. A paged cache looks every row up in the block table;
+    // `lim` = last row that may be addressed there.
+    U4H kk[MBX][KSTEPS], vv[MBX][VLB];
     __amdgpu_buffer_rsrc_t krs, vrs;
     if (!PAGED) {
-        krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char *>(kbase), 0, (int)(a.capacity * (uint32_t)(D * KES)), 0x00020000);
-        vrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<__half *>(vbase), 0, (int)(a.capacity * (uint32_t)(D * 2)), 0x00020000);
+        krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char *>(kbase), 0,
+                                                (int)(a.capacity * (uint32_t)(D * KES)), 0x00020000);
+        vrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<__half *>(vbase), 0, (int)(a.capacity * (uint32_t)(D * 2)),
+                                                0x00020000);
     }
     const int k_lane_off = n * (D * KES) + c * 16, v_lane_off = (lane / VLPR) * (D * 2) + (lane % VLPR) * 16;
-    auto issue_k = [&](int t, uint32_t lim) {
-        if (!PAGED) {
-            const int tb = (int)((k0 + (uint32_t)t * TK) * (uint32_t)(D * KES));
+    // blocks blk .. blk+m-1 of the partition (m <= MBX, wave-uniform)
+    auto issue_k = [&](uint32_t blk, uint32_t m, uint32_t lim) {
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
+        for (int mb = 0; mb < MBX; ++mb) {
+            if ((uint32_t)mb >= m) break;
+            const uint32_t row0 = k0 + (blk + mb) * BK;
+            if (!PAGED) {
 #pragma unroll
                 for (int j = 0; j < KSTEPS; ++j)
                     kk[mb][j].u = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                                krs, k_lane_off + j * 64, tb + mb * 16 * (D * KES), 0));
-            return;
-        }
+                                                                krs, k_lane_off + j * 64, (int)(row0 * (uint32_t)(D * KES)), 0));
+            } else {
+                const unsigned char *row = kbase + row_offset(min(row0 + n, lim)) * KES;
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-            const uint32_t key = min(k0 + (uint32_t)t * TK + 16 * mb + n, lim);
-            const unsigned char *row = kbase + row_offset(key) * KES;
-#pragma unroll
-            for (int j = 0; j < KSTEPS; ++j) kk[mb][j].u = *reinterpret_cast<const uint4 *>(row + (4 * j + c) * 16);
+                for (int j = 0; j < KSTEPS; ++j) kk[mb][j].u = *reinterpret_cast<const uint4 *>(row + (4 * j + c) * 16);
+            }
         }
     };
-    auto issue_v = [&](int t, uint32_t lim) {
-        if (!PAGED) {
-            const int tb = (int)((k0 + (uint32_t)t * TK) * (uint32_t)(D * 2));
+    auto issue_v = [&](uint32_t blk, uint32_t m, uint32_t lim) {
 #pragma unroll
-            for (int i = 0; i < VLD; ++i)
-                vv[i].u = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(vrs, v_lane_off, tb + i * VRPL * (D * 2), 0));
-            return;
-        }
+        for (int mb = 0; mb < MBX; ++mb) {
+            if ((uint32_t)mb >= m) break;
+            const uint32_t row0 = k0 + (blk + mb) * BK;
 #pragma unroll
-        for (int i = 0; i < VLD; ++i) {
-            const uint32_t key = min(k0 + (uint32_t)t * TK + i * VRPL + lane / VLPR, lim);
-            vv[i].u = *reinterpret_cast<const uint4 *>(vbase + row_offset(key) + (lane % VLPR) * 8);
+            for (int i = 0; i < VLB; ++i) {
+                if (!PAGED) {
+                    vv[mb][i].u = __builtin_bit_cast(
+                        uint4, __builtin_amdgcn_raw_buffer_load_b128(vrs, v_lane_off + i * VRPL * (D * 2),
+                                                                     (int)(row0 * (uint32_t)(D * 2)), 0));
+                } else {
+                    const uint32_t key = min(row0 + i * VRPL + lane / VLPR, lim);
+                    vv[mb][i].u = *reinterpret_cast<const uint4 *>(vbase + row_offset(key) + (lane % VLPR) * 8);
+                }
+            }
         }
     };
 
-    // Vector loads of one wave return in issue order. The first MFMA needs the query rows, and when FUSED their
-    // rotation needs the RoPE table row of the position, which is only known once the length has been read: issued
-    // after a K/V tile they would only return after it. So when FUSED, the last wave alone reads the length, fetches the raw
-    // query rows and the table row, rotates them and publishes the MFMA operand through LDS BEFORE it requests its
-    // own K/V tile, while the other waves request theirs at once (the memory system stays saturated by them,
-    // so the late one does not lengthen the transfer). A contiguous cache is allocated up to `capacity`, so a
-    // first tile can be requested before the length is known; a paged cache needs the length to stay inside its
-    // block table.
-    int t = wave;
+    // This wave's blocks of the partition: [wb0, wb1), the remainder going to the first streaming waves. When
+    // FUSED, wave 0 streams no blocks: it prepares the query operand and attends the new token.
+    constexpr int KW = FUSED ? NW - 1 : NW;  // streaming waves
+    const int sw = FUSED ? wave - 1 : wave;  // index among them (-1: none)
+    const uint32_t nb = a.chunk / BK;
+    const uint32_t wb0 = sw >= 0 ? nb - ((uint32_t)(KW - sw) * nb) / KW : 0u;
+    const uint32_t wb1 = sw >= 0 ? nb - ((uint32_t)(KW - 1 - sw) * nb) / KW : 0u;
+    uint32_t cur = wb0;
+
+    // A CU accepts vector memory requests in order and only as fast as its earlier ones complete, so anything
+    // requested after the other waves have queued their blocks arrives microseconds late. The first MFMA needs the
+    // query rows, and when FUSED their rotation needs the RoPE table row of the position, which is only known
+    // once the length has been read. So when FUSED, wave 0 requests no blocks at all: it reads the length and
+    // requests the raw query rows and the new token's raw K / V row before any other wave may request anything
+    // (a barrier holds them until then), rotates, and publishes the MFMA operand through LDS while the blocks
+    // are in flight. A contiguous cache is allocated up to `capacity`, so the blocks can be requested before the
+    // length is known; a paged cache needs the length to stay inside its block table.
     const bool rope_normal = a.rope_normal != 0, rope_on = a.apply_rope != 0;
     const bool head_ok = (uint32_t)n < gt;
-    // Q^T operand [KSTEPS][64] in LDS (shared by the workgroup when FUSED, else one copy per wave): reading it
-    // per MFMA step instead of holding it saves 12 VGPRs next to the 128 that a tile in flight occupies
-    uint4 *q_lds = reinterpret_cast<uint4 *>(smem + NW * (32 * VRS)) + (FUSED ? 0 : wave * (KSTEPS * 64));
+    // Q^T operand [KSTEPS][64], shared by the workgroup through LDS: reading it per MFMA step instead of holding
+    // it saves 12 VGPRs next to those that the blocks in flight occupy
+    uint4 *q_lds = reinterpret_cast<uint4 *>(smem + NW * (MBX * BK * VRS));
 
-    // Raw 16-byte segments 4j + c of one row rotated at position `pos`
+    // The RoPE table row of the position, staged in LDS by the last wave: D/2 cos values, then D/2 sin values.
+    unsigned char *rope_lds = reinterpret_cast<unsigned char *>(q_lds + KSTEPS * 64);
+    // Rotates the raw 16-byte segments 4j + c of one row held in x
     // (neox pairs segment s with s +- SEGS/2 = 4(j +- KSTEPS/2) + c: the mate lives in the same lane).
-    auto rope_row = [&](const __half *row, uint32_t pos, U4H(&o)[KSTEPS]) {
-        U4H x[KSTEPS];
-#pragma unroll
-        for (int j = 0; j < KSTEPS; ++j) x[j].u = *reinterpret_cast<const uint4 *>(row + (4 * j + c) * 8);
+    auto rope_apply = [&](const U4H(&x)[KSTEPS], U4H(&o)[KSTEPS]) {
         if (!rope_on) {
 #pragma unroll
             for (int j = 0; j < KSTEPS; ++j) o[j] = x[j];
             return;
         }
-        const uint32_t tp = min(pos, a.table_rows - 1);
-        const unsigned char *cp = (const unsigned char *)a.cos_t + (size_t)tp * D;
-        const unsigned char *sp = (const unsigned char *)a.sin_t + (size_t)tp * D;
+        const unsigned char *cp = rope_lds, *sp = rope_lds + D;
         if (rope_normal) {
 #pragma unroll
             for (int j = 0; j < KSTEPS; ++j) {
                 const int seg = 4 * j + c;
-                const uint2 c4 = *reinterpret_cast<const uint2 *>(__builtin_assume_aligned(cp + seg * 8, 8));
-                const uint2 s4 = *reinterpret_cast<const uint2 *>(__builtin_assume_aligned(sp + seg * 8, 8));
+                const uint2 c4 = *reinterpret_cast<const uint2 *>(cp + seg * 8);
+                const uint2 s4 = *reinterpret_cast<const uint2 *>(sp + seg * 8);
                 U4H cu, su;
                 cu.u = make_uint4(c4.x, c4.y, 0, 0), su.u = make_uint4(s4.x, s4.y, 0, 0);
                 o[j] = rope8(x[j], x[j], cu, su, true, true);
@@ -363,125 +374,194 @@ __global__ void __launch_bounds__(NT, 2) flash_decode_mfma_kernel(DecodeDev a) {
             for (int j = 0; j < KSTEPS / 2; ++j) {  // steps j and j + KSTEPS/2 share their cos / sin values
                 const int seg = 4 * j + c;
                 U4H cu, su;
-                cu.u = *reinterpret_cast<const uint4 *>(__builtin_assume_aligned(cp + seg * 16, 16));
-                su.u = *reinterpret_cast<const uint4 *>(__builtin_assume_aligned(sp + seg * 16, 16));
+                cu.u = *reinterpret_cast<const uint4 *>(cp + seg * 16);
+                su.u = *reinterpret_cast<const uint4 *>(sp + seg * 16);
                 o[j] = rope8(x[j], x[j + KSTEPS / 2], cu, su, false, true);
                 o[j + KSTEPS / 2] = rope8(x[j + KSTEPS / 2], x[j], cu, su, false, false);
             }
         }
     };
 
-    // Q^T operand: lane (n, c) keeps segment 4j + c of head head0 + n for every step j (zero for unused columns)
-    U4H qb[KSTEPS];
+    // The length is not written during the launch and its address is wave-uniform: read as constant memory it
+    // comes through the scalar cache.
+    auto read_len = [&]() -> uint32_t {
+        typedef const uint32_t __attribute__((address_space(4))) *const_u32p;
+        return a.d_len ? ((const_u32p)a.d_len)[(size_t)b * a.d_len_stride] + a.kv_len_add : a.kv_len;
+    };
+    // Q^T operand: lane (n, c) of step j holds segment 4j + c of head head0 + n (zero for unused columns)
     float qsc = a.scale_log2e;
-#pragma unroll
-    for (int j = 0; j < KSTEPS; ++j) qb[j].u = make_uint4(0, 0, 0, 0);
     uint32_t n_raw = 0;
+    U4H qraw;
+    qraw.u = make_uint4(0, 0, 0, 0);
     if (FUSED) {
-        if (wave == NW - 1) {
-            n_raw = a.d_len ? a.d_len[(size_t)b * a.d_len_stride] + a.kv_len_add : a.kv_len;
-            const uint32_t p0 = min(n_raw, min(a.capacity, a.kv_len_bound)) - 1;
-            if (head_ok) {
-                rope_row(a.q + (size_t)b * a.qin_stride_b + (size_t)(head0 + n) * D, p0, qb);
-                if (a.q_rot_out && split == 0) {
+        if (wave == 0) {
+            // First everything that does not depend on the length: the raw query rows and the new token's
+            // raw K / V row (parked in the block registers that this wave does not otherwise use). All lanes load
+            // from valid addresses and select afterwards, so that no divergent branch separates the requests.
+            __builtin_amdgcn_s_setprio(3);
+            U4H qx[KSTEPS], qb[KSTEPS];
+            const __half *qrow = a.q + (size_t)b * a.qin_stride_b + (size_t)(head0 + (head_ok ? n : 0)) * D;
+            const __half *krow = a.k_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D;
+            const __half *vrow_in = a.v_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D;
 #pragma unroll
-                    for (int j = 0; j < KSTEPS; ++j)
-                        *reinterpret_cast<uint4 *>(a.q_rot_out + (size_t)b * a.qrot_stride_b + (size_t)(head0 + n) * D +
-                                                   (4 * j + c) * 8) = qb[j].u;
+            for (int j = 0; j < KSTEPS; ++j) {
+                qx[j].u = *reinterpret_cast<const uint4 *>(qrow + (4 * j + c) * 8);
+                kk[1][j].u = *reinterpret_cast<const uint4 *>(krow + (4 * j + c) * 8);
+            }
+            vv[1][0].u = *reinterpret_cast<const uint4 *>(vrow_in + (lane % VLPR) * 8);
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();  // releases the streaming waves
+            __builtin_amdgcn_sched_barrier(0);
+            n_raw = read_len();
+            const uint32_t p0 = min(n_raw, min(a.capacity, a.kv_len_bound)) - 1;
+            if (rope_on) {
+                // The table row (D/2 cos values, then D/2 sin values) comes through the scalar cache, which does not
+                // share the vector queue: the address is wave-uniform and the tables are read-only. All of it is
+                // requested at once; lane 0 then stores it to LDS.
+                const uint32_t tp = min(p0, a.table_rows - 1);
+                const __half *ct = a.cos_t + (size_t)tp * (D / 2), *st = a.sin_t + (size_t)tp * (D / 2);
+                if constexpr (D == 128) {
+                    u16_t c0, c1, s0, s1;
+                    asm volatile(
+                        "s_load_dwordx16 %0, %4, 0x0\n\ts_load_dwordx16 %1, %4, 0x40\n\t"
+                        "s_load_dwordx16 %2, %5, 0x0\n\ts_load_dwordx16 %3, %5, 0x40\n\ts_waitcnt lgkmcnt(0)"
+                        : "=&s"(c0), "=&s"(c1), "=&s"(s0), "=&s"(s1)
+                        : "s"(ct), "s"(st)
+                        : "memory");
+                    if (lane == 0) {
+                        u16_t *dst = reinterpret_cast<u16_t *>(rope_lds);
+                        dst[0] = c0, dst[1] = c1, dst[2] = s0, dst[3] = s1;
+                    }
+                } else {
+                    u16_t c0, s0;
+                    asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                                 : "=&s"(c0), "=&s"(s0)
+                                 : "s"(ct), "s"(st)
+                                 : "memory");
+                    if (lane == 0) {
+                        u16_t *dst = reinterpret_cast<u16_t *>(rope_lds);
+                        dst[0] = c0, dst[1] = s0;
+                    }
                 }
+                __builtin_amdgcn_wave_barrier();  // LDS executes a wave's accesses in order
+            }
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j)
+                if (!head_ok) qx[j].u = make_uint4(0, 0, 0, 0);
+            if (lane >= VLPR) vv[1][0].u = make_uint4(0, 0, 0, 0);
+            rope_apply(qx, qb);
+            if (head_ok && a.q_rot_out && split == 0) {
+#pragma unroll
+                for (int j = 0; j < KSTEPS; ++j)
+                    *reinterpret_cast<uint4 *>(a.q_rot_out + (size_t)b * a.qrot_stride_b + (size_t)(head0 + n) * D +
+                                               (4 * j + c) * 8) = qb[j].u;
             }
 #pragma unroll
             for (int j = 0; j < KSTEPS; ++j) q_lds[j * 64 + lane] = qb[j].u;
+            __builtin_amdgcn_s_setprio(0);
+        } else {
+            __syncthreads();  // wave 0 has queued its requests
         }
-    } else if (head_ok) {
-        const unsigned char *qrow =
-            (const unsigned char *)a.q + ((size_t)b * a.q_stride_b + (size_t)(head0 + n) * a.q_stride_h) * KES;
-#pragma unroll
-        for (int j = 0; j < KSTEPS; ++j) qb[j].u = *reinterpret_cast<const uint4 *>(qrow + (4 * j + c) * 16);
-        if (SAGE) qsc = a.q_scale[head0 + n] * a.scale_log2e;
+    } else {
+        // wave j < KSTEPS fetches step j of the operand (requested before its K/V blocks, so it returns first)
+        if (wave < KSTEPS && head_ok) {
+            const unsigned char *qrow =
+                (const unsigned char *)a.q + ((size_t)b * a.q_stride_b + (size_t)(head0 + n) * a.q_stride_h) * KES;
+            qraw.u = *reinterpret_cast<const uint4 *>(qrow + (4 * wave + c) * 16);
+        }
+        if (SAGE && head_ok) qsc = a.q_scale[head0 + n] * a.scale_log2e;
     }
-    if (!PAGED) {
-        issue_k(t, a.capacity - 1);
-        issue_v(t, a.capacity - 1);
+    if (!PAGED && cur < wb1) {
+        const uint32_t m = min((uint32_t)MBX, wb1 - cur);
+        issue_k(cur, m, 0);
+        issue_v(cur, m, 0);
     }
-    if (!(FUSED && wave == NW - 1)) n_raw = a.d_len ? a.d_len[(size_t)b * a.d_len_stride] + a.kv_len_add : a.kv_len;
+    if (!FUSED && wave < KSTEPS) q_lds[wave * 64 + lane] = qraw.u;
+    if (!(FUSED && wave == 0)) n_raw = read_len();
     const uint32_t N = min(n_raw, min(a.capacity, a.kv_len_bound));
     const uint32_t nsplits = (N + a.chunk - 1) / a.chunk;
     if (split >= nsplits) return;  // uniform over the workgroup
     const uint32_t k1 = min(N, k0 + a.chunk);
-    if (PAGED && k0 + (uint32_t)t * TK < k1) {
-        issue_k(t, k1 - 1);
-        issue_v(t, k1 - 1);
-    }
 
-    // FUSED: row p is the new token. It is appended only if it lies inside the cache and the launch bound.
+    // FUSED: row p is the new token. It is appended only if it lies inside the cache and the launch bound; the
+    // cache rows of its partition end before it, and it is attended as a one-key block of its own.
     const uint32_t p = N - 1;
     const bool owns_new = FUSED && n_raw == N && p >= k0 && p < k1;
-    if (FUSED) {
-        __syncthreads();
-    } else {
-#pragma unroll
-        for (int j = 0; j < KSTEPS; ++j) q_lds[j * 64 + lane] = qb[j].u;
+    const uint32_t kend = owns_new ? k1 - 1 : k1;
+    const uint32_t wbe = min(wb1, (kend - k0 + BK - 1) / BK);  // this wave's blocks that hold a valid key end here
+    if (PAGED && cur < wbe) {
+        const uint32_t m = min((uint32_t)MBX, wbe - cur);
+        issue_k(cur, m, k1 - 1);
+        issue_v(cur, m, k1 - 1);
     }
+    __syncthreads();  // the Q^T operand is in LDS
 
     f4_t oacc[DBLK];
 #pragma unroll
     for (int blk = 0; blk < DBLK; ++blk) oacc[blk] = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-    float m_run = -1e30f, l_run = 0.0f;  // l_run: this lane's share (its 4 keys per tile) of the head's sum
+    float m_run = -1e30f, l_run = 0.0f;  // l_run: this lane's share (its 4 keys per block) of the head's sum
 
-    unsigned char *v_lds = smem + wave * (32 * VRS);  // one 32-key half of V at a time
-    // One tile held in kk / vv: rows tbase .. tbase+TK-1, of which rows >= kend carry no weight.
+    unsigned char *v_lds = smem + wave * (MBX * BK * VRS);
     auto q_op = [&](int j) {
         U4H x;
         x.u = q_lds[j * 64 + lane];
         return x;
     };
-    auto consume = [&](int t, uint32_t tbase, uint32_t kend, bool more) {
+    // m blocks held in kk / vv, starting at row tbase; rows >= kend carry no weight. If `mnext`, the next round's
+    // blocks (from block `nblk`) are requested as soon as the registers of this round are free.
+    auto consume = [&](uint32_t tbase, uint32_t m, uint32_t kend, uint32_t nblk, uint32_t mnext) {
         // S^T: accumulator i of block mb in lane (n, c) is key tbase + 16mb + 4c + i against head n
-        float s[4 * MB];
+        float s[4 * MBX];
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-            if (SAGE) {
-                i4_t si = {0, 0, 0, 0};
+        for (int mb = 0; mb < MBX; ++mb) {
+            if ((uint32_t)mb < m) {
+                if (SAGE) {
+                    i4_t si = {0, 0, 0, 0};
 #pragma unroll
-                for (int j = 0; j < KSTEPS; ++j)
-                    si = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk[mb][j].i, q_op(j).i, si, 0, 0, 0);
-                // each 32-key half is one scale block
-                const uint32_t key = min(tbase + 16 * mb, kend - 1);
-                const float ks = __half2float(a.k_scale[(size_t)kvh * a.ks_stride + key / FA_SAGE_BLOCK]);
+                    for (int j = 0; j < KSTEPS; ++j)
+                        si = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk[mb][j].i, q_op(j).i, si, 0, 0, 0);
+                    // a block lies inside one 32-key scale block
+                    const uint32_t key = min(tbase + BK * mb, kend - 1);
+                    const float ks = __half2float(a.k_scale[(size_t)kvh * a.ks_stride + key / FA_SAGE_BLOCK]);
 #pragma unroll
-                for (int i = 0; i < 4; ++i) s[mb * 4 + i] = (float)si[i] * (qsc * ks);
+                    for (int i = 0; i < 4; ++i) s[mb * 4 + i] = (float)si[i] * (qsc * ks);
+                } else {
+                    f4_t sf = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int j = 0; j < KSTEPS; ++j)
+                        sf = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk[mb][j].h, q_op(j).h, sf, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) s[mb * 4 + i] = sf[i] * qsc;
+                }
             } else {
-                f4_t sf = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int j = 0; j < KSTEPS; ++j)
-                    sf = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk[mb][j].h, q_op(j).h, sf, 0, 0, 0);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) s[mb * 4 + i] = sf[i] * qsc;
+                for (int i = 0; i < 4; ++i) s[mb * 4 + i] = -INFINITY;
             }
         }
-        if (more) issue_k(t + NW, kend - 1);  // K registers are free again
+        if (mnext) issue_k(nblk, mnext, k1 - 1);  // K registers are free again
         float mt = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 4 * MB; ++i) {
+        for (int i = 0; i < 4 * MBX; ++i) {
             // flash_decode.metal:393-395 maps non-finite scores to -1e30 (weight 0 unless all are)
-            s[i] = isfinite(s[i]) ? s[i] : -1e30f;
-            if (tbase + 16 * (i >> 2) + 4 * c + (i & 3) >= kend) s[i] = -INFINITY;
+            if ((uint32_t)(i >> 2) < m) {
+                s[i] = isfinite(s[i]) ? s[i] : -1e30f;
+                if (tbase + BK * (i >> 2) + 4 * c + (i & 3) >= kend) s[i] = -INFINITY;
+            }
             mt = fmaxf(mt, s[i]);
         }
         mt = fmaxf(mt, xor16(mt));
         mt = fmaxf(mt, xor32(mt));
         const float mn = fmaxf(m_run, mt);
         const float al = fast_exp2(m_run - mn);
-        // P^T operands, one per 32-key half: k-slot i of lane (n, c) is key 16*(i/4) + 4c + i%4 of the half, the
-        // order the accumulators already have
-        h8_t pb[HB];
+        // P^T operand of block mb: k-slot i of lane (n, c) is key 4c + i of the block, the order the accumulators
+        // already have
+        h4_t pb[MBX];
         float ps = 0.0f;
 #pragma unroll
-        for (int i = 0; i < 4 * MB; ++i) {
+        for (int i = 0; i < 4 * MBX; ++i) {
             const float pw = fast_exp2(s[i] - mn);
             ps += pw;
-            pb[i >> 3][i & 7] = (_Float16)pw;
+            pb[i >> 2][i & 3] = (_Float16)pw;
         }
         l_run = l_run * al + ps;
         m_run = mn;
@@ -491,59 +571,63 @@ __global__ void __launch_bounds__(NT, 2) flash_decode_mfma_kernel(DecodeDev a) {
         }
         const int L = lane & 15;
         const unsigned char *vrow = v_lds + (c * 4 + (L >> 2)) * VRS + (L & 3) * 8;
+        // V blocks -> this wave's LDS region (rows past the end are zeroed: weight 0 times NaN is NaN)
 #pragma unroll
-        for (int hb = 0; hb < HB; ++hb) {
-            // V half -> this wave's LDS region (rows past the end are zeroed: weight 0 times NaN is NaN)
+        for (int mb = 0; mb < MBX; ++mb) {
+            if ((uint32_t)mb >= m) break;
 #pragma unroll
-            for (int i = 0; i < VLH; ++i) {
+            for (int i = 0; i < VLB; ++i) {
                 const int row = i * VRPL + lane / VLPR;
-                U4H &x = vv[hb * VLH + i];
-                if (tbase + 32 * hb + row >= kend) x.u = make_uint4(0, 0, 0, 0);
-                *reinterpret_cast<uint4 *>(v_lds + row * VRS + (lane % VLPR) * 16) = x.u;
+                U4H &x = vv[mb][i];
+                if (tbase + BK * mb + row >= kend) x.u = make_uint4(0, 0, 0, 0);
+                *reinterpret_cast<uint4 *>(v_lds + (mb * BK + row) * VRS + (lane % VLPR) * 16) = x.u;
             }
-            // O^T += V^T . P^T : two transpose loads hand lane (n, c) keys 4c..4c+3 and 16+4c..16+4c+3 of dim 16*blk + n
+        }
+        // O^T += V^T . P^T : a transpose load hands lane (n, c) keys 4c..4c+3 of dim 16*blk + n
+#pragma unroll
+        for (int mb = 0; mb < MBX; ++mb) {
+            if ((uint32_t)mb >= m) break;
 #pragma unroll
             for (int blk = 0; blk < DBLK; ++blk) {
                 fp16x4_t v0 = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
-                    (fp16x4_t __attribute__((address_space(3))) *)(vrow + blk * 32));
-                fp16x4_t v1 = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
-                    (fp16x4_t __attribute__((address_space(3))) *)(vrow + 16 * VRS + blk * 32));
-                h8_t vh;
+                    (fp16x4_t __attribute__((address_space(3))) *)(vrow + mb * BK * VRS + blk * 32));
+                h4_t vh;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) vh[i] = (_Float16)v0[i], vh[4 + i] = (_Float16)v1[i];
-                oacc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vh, pb[hb], oacc[blk], 0, 0, 0);
+                for (int i = 0; i < 4; ++i) vh[i] = (_Float16)v0[i];
+                oacc[blk] = __builtin_amdgcn_mfma_f32_16x16x16f16(vh, pb[mb], oacc[blk], 0, 0, 0);
             }
         }
-        if (more) issue_v(t + NW, kend - 1);  // V registers are free again
+        if (mnext) issue_v(nblk, mnext, k1 - 1);  // V registers are free again
     };
 
-    // FUSED: the cache rows of this partition end before the new row; the new token is a one-key tile of its own.
-    const uint32_t kend = owns_new ? k1 - 1 : k1;
-    const int ntiles_cache = (int)((kend - k0 + TK - 1) / TK);
-    for (; t < ntiles_cache; t += NW) consume(t, k0 + (uint32_t)t * TK, kend, t + NW < ntiles_cache);
+    while (cur < wbe) {
+        const uint32_t m = min((uint32_t)MBX, wbe - cur);
+        const uint32_t nblk = cur + m;
+        const uint32_t mnext = nblk < wbe ? min((uint32_t)MBX, wbe - nblk) : 0u;
+        consume(k0 + cur * BK, m, kend, nblk, mnext);
+        cur = nblk;
+    }
 
-    if (FUSED && owns_new && wave == ntiles_cache % NW) {
+    if (FUSED && owns_new && wave == 0) {
         // The new row is not in the cache: rotate K / copy V from the raw projections (kv_prep_fused.metal:89-122),
-        // attend it as a tile whose only valid key is row 0, and let one workgroup of the KV head store it.
+        // attend it as a block whose only valid key is row 0, and let one workgroup of the KV head store it.
         const bool writer = y % a.sub_per_kv == 0;
-        U4H knew[KSTEPS];
-        rope_row(a.k_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D, p, knew);
+        U4H kraw[KSTEPS], knew[KSTEPS];
+#pragma unroll
+        for (int j = 0; j < KSTEPS; ++j) kraw[j] = kk[1][j];
+        rope_apply(kraw, knew);
         __half *kw = const_cast<__half *>(reinterpret_cast<const __half *>(kbase)) + row_offset(p);
         __half *vw = const_cast<__half *>(vbase) + row_offset(p);
 #pragma unroll
         for (int j = 0; j < KSTEPS; ++j) {
             kk[0][j].u = n == 0 ? knew[j].u : make_uint4(0, 0, 0, 0);
-#pragma unroll
-            for (int mb = 1; mb < MB; ++mb) kk[mb][j].u = make_uint4(0, 0, 0, 0);
             if (writer && n == 0) *reinterpret_cast<uint4 *>(kw + (4 * j + c) * 8) = knew[j].u;
         }
 #pragma unroll
-        for (int i = 0; i < VLD; ++i) vv[i].u = make_uint4(0, 0, 0, 0);
-        if (lane < VLPR) {
-            vv[0].u = *reinterpret_cast<const uint4 *>(a.v_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D + lane * 8);
-            if (writer) *reinterpret_cast<uint4 *>(vw + lane * 8) = vv[0].u;
-        }
-        consume(0, p, p + 1, false);
+        for (int i = 0; i < VLB; ++i) vv[0][i].u = make_uint4(0, 0, 0, 0);
+        vv[0][0] = vv[1][0];
+        if (writer && lane < VLPR) *reinterpret_cast<uint4 *>(vw + lane * 8) = vv[0][0].u;
+        consume(p, 1, p + 1, 0, 0);
     }
 
     // the head's sum over the four 16-lane rows (the running max is already common to them)
@@ -639,7 +723,8 @@ enum Mode { MODE_PLAIN = 0, MODE_PAGED = 1, MODE_SAGE = 2, MODE_FUSED = 3, MODE_
 // Dynamic LDS: the per-wave V tiles during the main loop, then the wave fold / the partition merge.
 template <int D>
 size_t decode_lds_bytes(uint32_t gt) {
-    const size_t v_tiles = (size_t)NW * 32 * (D * 2 + 32) + (size_t)NW * (D / 32) * 64 * 16;  // + the Q^T operands
+    // the per-wave V blocks + the Q^T operand + one RoPE table row
+    const size_t v_tiles = (size_t)NW * MBX * BK * (D * 2 + 32) + (size_t)(D / 32) * 64 * 16 + 2 * D;
     const size_t fold = ((size_t)NW * gt * D + (size_t)NW * gt * 2) * sizeof(float);
     const size_t merge = (size_t)NT * 6 * sizeof(float);
     size_t m = v_tiles > fold ? v_tiles : fold;
@@ -650,32 +735,45 @@ template <int D>
 fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
     const size_t lds = decode_lds_bytes<D>(a.gt);
     {
+        // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
+        static bool lds_allowed = false;
+        if (!lds_allowed) {
+            const int cap = (int)decode_lds_bytes<D>(MAX_GT);
+            FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
+            FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, true, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
+            FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
+            FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
+            FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, true, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
+            lds_allowed = true;
+        }
+    }
+    {
         const char *name = mode == MODE_SAGE ? "sage_decode_mfma_kernel"
                            : (mode == MODE_FUSED || mode == MODE_FUSED_PAGED) ? "fused_rope_append_decode_kernel"
                                                                               : "flash_decode_mfma_kernel";
-        FaLaunchScope scope(ctx, name);
+        FaLaunchScope scope(ctx, name, true);
         switch (mode) {
             case MODE_PLAIN:
-                hipLaunchKernelGGL((flash_decode_mfma_kernel<D, false, false, false>), grid, dim3(NT), lds, ctx->stream, a);
+                scope.launch((flash_decode_mfma_kernel<D, false, false, false>), grid, dim3(NT), lds, a);
                 break;
             case MODE_PAGED:
-                hipLaunchKernelGGL((flash_decode_mfma_kernel<D, true, false, false>), grid, dim3(NT), lds, ctx->stream, a);
+                scope.launch((flash_decode_mfma_kernel<D, true, false, false>), grid, dim3(NT), lds, a);
                 break;
             case MODE_SAGE:
-                hipLaunchKernelGGL((flash_decode_mfma_kernel<D, false, true, false>), grid, dim3(NT), lds, ctx->stream, a);
+                scope.launch((flash_decode_mfma_kernel<D, false, true, false>), grid, dim3(NT), lds, a);
                 break;
             case MODE_FUSED:
-                hipLaunchKernelGGL((flash_decode_mfma_kernel<D, false, false, true>), grid, dim3(NT), lds, ctx->stream, a);
+                scope.launch((flash_decode_mfma_kernel<D, false, false, true>), grid, dim3(NT), lds, a);
                 break;
             default:
-                hipLaunchKernelGGL((flash_decode_mfma_kernel<D, true, false, true>), grid, dim3(NT), lds, ctx->stream, a);
+                scope.launch((flash_decode_mfma_kernel<D, true, false, true>), grid, dim3(NT), lds, a);
                 break;
         }
         FA_TRY(scope.finish());
     }
     if (!a.merge_in_kernel && grid.x > 1) {
-        FaLaunchScope scope(ctx, "flash_decode_merge_kernel");
-        hipLaunchKernelGGL((flash_decode_merge_kernel<D>), dim3(1, grid.y, grid.z), dim3(NT), 0, ctx->stream, a, grid.x);
+        FaLaunchScope scope(ctx, "flash_decode_merge_kernel", true);
+        scope.launch((flash_decode_merge_kernel<D>), dim3(1, grid.y, grid.z), dim3(NT), 0, a, grid.x);
         FA_TRY(scope.finish());
     }
     return FA_OK;

@@ -2,6 +2,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hip_fp16.h>
 
 #include <cstdarg>
@@ -33,7 +34,7 @@ struct fa_ctx {
     // per-(sequence, kv head) arrival counters for the in-kernel split merge; always zero between launches
     uint32_t *counters = nullptr;
     uint32_t n_counters = 0;
-    fa_decode_variant decode_variant{0, 0};
+    fa_decode_variant decode_variant{0, 1};
     // per-kernel profiling
     bool profiling = false;
     std::vector<FaProfileRec> prof;
@@ -63,8 +64,21 @@ struct FaLaunchScope {
     fa_ctx *ctx;
     const char *name;
     hipEvent_t start = nullptr, stop = nullptr;
-    FaLaunchScope(fa_ctx *c, const char *n);
+    bool tight = false;
+    // `dispatch_events`: the caller will use launch(), which attaches the events to the dispatch
+    FaLaunchScope(fa_ctx *c, const char *n, bool dispatch_events = false);
     fa_status finish();
+    // Launches `kernel`; when profiling, the events are attached to the dispatch itself, so their difference is
+    // the kernel's execution time without the queue's processing of separate event markers.
+    template <typename K, typename... Args>
+    void launch(K kernel, dim3 grid, dim3 block, size_t lds, Args... args) {
+        if (start && stop) {
+            tight = true;
+            hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds, ctx->stream, start, stop, 0, args...);
+        } else {
+            hipLaunchKernelGGL(kernel, grid, block, lds, ctx->stream, args...);
+        }
+    }
 };
 
 static inline uint32_t ceil_div_u32(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
