@@ -180,6 +180,84 @@ def calibration_copy(f, reps=3):
     return {"kernel": "paged_gather_kernel", "launches": reps, "bytes_read": nbytes, "bytes_written": nbytes}
 
 
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense f16 / bf16 matrix peak
+
+
+def bench_prefill(f, args):
+    """Llama-3.2-3B-shaped prefill of one layer: 2048 tokens, RoPE + append into an empty paged cache, then causal
+    flash prefill from the paged cache. One step = both launches."""
+    H, Hkv, D, M, bs = 24, 8, 128, 2048, 16
+    rng = np.random.default_rng(0xF0DD + 4)
+    nblk = M // bs
+    perm = rng.permutation(nblk).astype(np.int32).reshape(1, nblk)
+    k_pool, v_pool = f.zeros((nblk, Hkv, bs, D)), f.zeros((nblk, Hkv, bs, D))
+    bt, lens = f.array(perm), f.array(np.array([0], np.uint32))
+    desc = fa.paged_kv(k_pool, v_pool, bt, lens, nblk, Hkv, bs, D, 1, nblk)
+    q, k, v = (rng.standard_normal((M, n * D), dtype=np.float32).astype(np.float16) for n in (H, Hkv, Hkv))
+    cos, sin = fa.rope_tables(5e5, D, M)
+    dq, dk, dv, dcos, dsin = (f.array(x) for x in (q, k, v, cos, sin))
+    dqr, dout = f.zeros((H, M, D)), f.zeros((M, H * D))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, M, 0, 0, fa.ROPE_NORMAL)
+
+    def step():
+        f.kv_prep_fused_paged(dq.arg(), dk.arg(), dv.arg(), dqr.arg(), desc, 0, dcos.arg(), dsin.arg(), p)
+        f.flash_prefill_paged(dqr.arg(), desc, 0, dout.arg(), True, 0, H, M, M)
+
+    for _ in range(args.warmup):
+        step()
+    f.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    f.synchronize()
+    dt = time.perf_counter() - t0
+
+    # parity: cache bit-exact against the oracle's append; the last 64 query rows against the oracle's prefill
+    import orc  # the CPU oracle is only the checker here
+    kc, vc = np.zeros((Hkv, M, D), np.float16), np.zeros((Hkv, M, D), np.float16)
+    qr = orc.kv_prep_fused(q, k, v, kc, vc, cos, sin, orc.make_params(H, Hkv, D, M, 0, M, rope_mode=1))
+    cache_ok = (np.array_equal(orc.paged_gather(k_pool.download(), perm[0], Hkv, bs, D, M).view(np.uint16), kc.view(np.uint16))
+                and np.array_equal(orc.paged_gather(v_pool.download(), perm[0], Hkv, bs, D, M).view(np.uint16), vc.view(np.uint16))
+                and np.array_equal(dqr.download().view(np.uint16), qr.view(np.uint16)))
+    tail = 64
+    want = orc.sdpa_prefill(np.ascontiguousarray(qr[:, M - tail:]), kc, vc, H, Hkv, D, tail, M, M - tail, M, causal=True,
+                            out_layout="head_major", n_threads=max(1, min(16, os.cpu_count() or 1, orc.lib().orc_max_threads())))
+    got = dout.download().reshape(M, H, D).transpose(1, 0, 2)[:, M - tail:]
+    err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64))))
+
+    prof_steps = 20
+    f.profile_reset()
+    f.profile_enable(True)
+    for _ in range(prof_steps):
+        step()
+    n_pf, ms_pf = f.profile_query("flash_prefill_mfma_kernel")
+    n_kp, ms_kp = f.profile_query("kv_prep_fused")
+    f.profile_enable(False)
+    f.profile_reset()
+    flops = 4.0 * D * H * M * (M + 1) / 2  # QK^T and PV over the causal pairs
+    avg_pf_s = ms_pf / 1e3 / max(1, n_pf)
+    achieved = flops / avg_pf_s / 1e12
+    append_bytes = 2.0 * M * (H + 2 * Hkv) * D * 2  # read q, k, v; write q_rot and the cache rows
+    result = {
+        "metric": "prefill-attn steps/s + achieved f16 MFMA TFLOP/s (% peak), Llama-3.2-3B shape, 2048 tokens",
+        "value": args.steps / dt, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "llama3.2-3b prefill attention, one layer: RoPE + append of 2048 tokens into an empty paged "
+                               "f16 cache (16-token blocks, permuted block table), then causal flash prefill, H24/Hkv8/D128"},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / MFMA_F16_PEAK_TFLOPS, "traffic": None, "kernel": "flash_prefill_mfma_kernel",
+                     "avg_launch_us": avg_pf_s * 1e6, "launches": n_pf, "flops_per_launch": flops},
+        "append": {"kernel": "kv_prep_fused_vec_kernel", "avg_launch_us": ms_kp * 1e3 / max(1, n_kp),
+                   "achieved_gbps": append_bytes / (ms_kp / 1e3 / max(1, n_kp)) / 1e9, "bytes_per_launch": append_bytes,
+                   "frac_of_hbm_peak": append_bytes / (ms_kp / 1e3 / max(1, n_kp)) / 1e9 / HBM_PEAK_GBPS},
+        "parity": {"cache_bit_exact": bool(cache_ok), "prefill_max_abs_err_last64": err},
+    }
+    print(json.dumps(result))
+    if not cache_ok or err > 2e-3:
+        sys.exit("parity check failed: cache_bit_exact=%s prefill_max_abs_err=%g" % (cache_ok, err))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -199,9 +277,15 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is built and measured on a single MI355X (--gpus 1); "
                  "how it would shard across GPUs is described in DESIGN.md")
+    if args.workload == "llama3b_prefill_2k":  # secondary line: the MFMA-bound half of the path
+        f = fa.Foundry(0)
+        args.steps, args.warmup = min(args.steps, 200), min(args.warmup, 20)
+        bench_prefill(f, args)
+        f.close()
+        return
     if args.workload != "llama3b_decode_8k":
-        sys.exit("unknown workload %r (only llama3b_decode_8k is a bench line; the other configurations are "
-                 "parity-test cases)" % args.workload)
+        sys.exit("unknown workload %r (llama3b_decode_8k is the bench line, llama3b_prefill_2k a secondary one; the "
+                 "other configurations are parity-test cases)" % args.workload)
 
     room = 256  # the metric's timed window: 256 consecutive decode steps from 8192 context
     rng = np.random.default_rng(0xF0DD + 2)

@@ -224,20 +224,20 @@ fa_status fa_launch_kv_prep(fa_ctx *ctx, const KvPrepLaunch &L) {
     if (a.seq_len == 0) return FA_OK;
     if (a.head_dim % 16 == 0) {
         uint64_t total = (uint64_t)a.seq_len * (a.n_heads + 2 * a.n_kv_heads) * (a.head_dim / 16);
-        FaLaunchScope scope(ctx, "kv_prep_fused_vec_kernel");
-        hipLaunchKernelGGL(kv_prep_fused_vec_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, a);
+        FaLaunchScope scope(ctx, "kv_prep_fused_vec_kernel", true);
+        scope.launch(kv_prep_fused_vec_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, a);
         return scope.finish();
     }
     uint64_t total = (uint64_t)a.n_heads * a.seq_len * a.head_dim;
-    FaLaunchScope scope(ctx, "kv_prep_fused_elem_kernel");
-    hipLaunchKernelGGL(kv_prep_fused_elem_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, a);
+    FaLaunchScope scope(ctx, "kv_prep_fused_elem_kernel", true);
+    scope.launch(kv_prep_fused_elem_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, a);
     return scope.finish();
 }
 
 fa_status fa_launch_u32_add(fa_ctx *ctx, uint32_t *vals, uint32_t n, uint32_t delta) {
     if (n == 0) return FA_OK;
-    FaLaunchScope scope(ctx, "u32_add_kernel");
-    hipLaunchKernelGGL(u32_add_kernel, dim3(ceil_div_u32(n, 64)), dim3(64), 0, ctx->stream, vals, n, delta);
+    FaLaunchScope scope(ctx, "u32_add_kernel", true);
+    scope.launch(u32_add_kernel, dim3(ceil_div_u32(n, 64)), dim3(64), 0, vals, n, delta);
     return scope.finish();
 }
 
@@ -245,8 +245,8 @@ fa_status fa_launch_paged_gather(fa_ctx *ctx, const fa_paged_kv *c, uint32_t seq
                                  void *v_out, uint32_t out_capacity) {
     if (seq_len == 0) return FA_OK;
     uint64_t total = (uint64_t)c->n_kv_heads * seq_len * (c->head_dim / 8);
-    FaLaunchScope scope(ctx, "paged_gather_kernel");
-    hipLaunchKernelGGL(paged_gather_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream,
+    FaLaunchScope scope(ctx, "paged_gather_kernel", true);
+    scope.launch(paged_gather_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
                        (const __half *)c->k_pool, (const __half *)c->v_pool,
                        c->block_table + (size_t)seq_index * c->max_blocks_per_seq, (__half *)k_out, (__half *)v_out,
                        c->n_kv_heads, c->block_size, c->head_dim, seq_len, out_capacity);

@@ -51,7 +51,7 @@ struct Lds {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 template <int D>
-__global__ void __launch_bounds__(256) flash_prefill_mfma_kernel(PrefillDev a) {
+__global__ void __launch_bounds__(256, 2) flash_prefill_mfma_kernel(PrefillDev a) {
     constexpr int DSTEPS = D / 16;  // MFMA k-steps over head_dim for S^T
     constexpr int DBLKS = D / 32;   // 32-row blocks of O^T
     constexpr int KRS = Lds<D>::KRS, VRS = Lds<D>::VRS;
@@ -90,7 +90,19 @@ __global__ void __launch_bounds__(256) flash_prefill_mfma_kernel(PrefillDev a) {
         for (int s = 0; s < DSTEPS; ++s) qreg[s].u = *reinterpret_cast<const uint4 *>(qp + s * 16 + hi * 8);
     }
 
+    // A paged cache needs the page of every row before the row itself can be requested. The page ids of a tile are
+    // fetched one tile ahead of its rows (which are fetched one tile ahead of their use), so that no iteration
+    // waits for two dependent memory round trips.
     uint4 kreg[LOADS], vreg[LOADS];
+    int32_t page[LOADS];
+    auto fetch_pages = [&](int tile) {
+        if (!a.paged) return;
+#pragma unroll
+        for (int j = 0; j < LOADS; ++j) {
+            const uint32_t key = (uint32_t)tile * BN + (tid + 256 * j) / CPR;
+            page[j] = key < kv_end ? a.block_table[key / a.block_size] : 0;
+        }
+    };
     auto fetch = [&](int tile) {
 #pragma unroll
         for (int j = 0; j < LOADS; ++j) {
@@ -100,8 +112,7 @@ __global__ void __launch_bounds__(256) flash_prefill_mfma_kernel(PrefillDev a) {
             if (key < kv_end) {
                 size_t off;
                 if (a.paged) {
-                    const size_t blk = (size_t)a.block_table[key / a.block_size];
-                    off = ((blk * a.n_kv_heads + kvh) * a.block_size + key % a.block_size) * (size_t)D;
+                    off = (((size_t)page[j] * a.n_kv_heads + kvh) * a.block_size + key % a.block_size) * (size_t)D;
                 } else {
                     off = (size_t)key * D;
                 }
@@ -134,12 +145,17 @@ __global__ void __launch_bounds__(256) flash_prefill_mfma_kernel(PrefillDev a) {
     // first key index that some row of this wave cannot see
     const uint32_t wave_min_limit = a.causal ? (min(q0 + wave * 32, a.q_len - 1) + a.query_offset) : 0xffffffffu;
 
-    if (n_tiles > 0) fetch(0);
+    if (n_tiles > 0) {
+        fetch_pages(0);
+        fetch(0);
+        if (n_tiles > 1) fetch_pages(1);
+    }
     for (int tile = 0; tile < n_tiles; ++tile) {
         __syncthreads();  // previous tile fully consumed
         stash();
         __syncthreads();
         if (tile + 1 < n_tiles) fetch(tile + 1);
+        if (tile + 2 < n_tiles) fetch_pages(tile + 2);
 
         const uint32_t key0 = (uint32_t)tile * BN;
         // S^T for the two 32-key blocks of the tile
@@ -256,11 +272,11 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
     a.scale_log2e = L.scale * 1.4426950408889634f;
     if (L.q_len == 0) return FA_OK;
     dim3 grid(ceil_div_u32(L.q_len, BM), L.n_heads, 1);
-    FaLaunchScope scope(ctx, "flash_prefill_mfma_kernel");
+    FaLaunchScope scope(ctx, "flash_prefill_mfma_kernel", true);
     if (L.head_dim == 128)
-        hipLaunchKernelGGL(flash_prefill_mfma_kernel<128>, grid, dim3(256), 0, ctx->stream, a);
+        scope.launch(flash_prefill_mfma_kernel<128>, grid, dim3(256), 0, a);
     else if (L.head_dim == 64)
-        hipLaunchKernelGGL(flash_prefill_mfma_kernel<64>, grid, dim3(256), 0, ctx->stream, a);
+        scope.launch(flash_prefill_mfma_kernel<64>, grid, dim3(256), 0, a);
     else
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill only supports head_dim=64 or 128, got %u", L.head_dim);
     return scope.finish();

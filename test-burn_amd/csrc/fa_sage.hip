@@ -100,13 +100,13 @@ fa_status fa_launch_sage_k_mean(fa_ctx *ctx, const void *k, uint32_t n_kv_heads,
     FA_TRY(fa_ensure_workspace(ctx, (size_t)n_kv_heads * MEAN_PARTS * head_dim * sizeof(float)));
     float *partial = (float *)ctx->workspace;
     {
-        FaLaunchScope scope(ctx, "sage_k_colsum_kernel");
-        hipLaunchKernelGGL(sage_k_colsum_kernel, dim3(MEAN_PARTS, n_kv_heads), dim3(256), 0, ctx->stream,
+        FaLaunchScope scope(ctx, "sage_k_colsum_kernel", true);
+        scope.launch(sage_k_colsum_kernel, dim3(MEAN_PARTS, n_kv_heads), dim3(256), 0,
                            (const __half *)k, capacity, head_dim, kv_len, partial);
         FA_TRY(scope.finish());
     }
-    FaLaunchScope scope(ctx, "sage_k_mean_finish_kernel");
-    hipLaunchKernelGGL(sage_k_mean_finish_kernel, dim3(n_kv_heads), dim3(head_dim), 0, ctx->stream, partial, head_dim,
+    FaLaunchScope scope(ctx, "sage_k_mean_finish_kernel", true);
+    scope.launch(sage_k_mean_finish_kernel, dim3(n_kv_heads), dim3(head_dim), 0, partial, head_dim,
                        kv_len, mean_out);
     return scope.finish();
 }
@@ -116,8 +116,8 @@ fa_status fa_launch_sage_quantize_k(fa_ctx *ctx, const void *k, const float *mea
                                     void *k_q, void *k_scale) {
     if (row_end <= row_begin) return FA_OK;
     const uint32_t nblk = ceil_div_u32(row_end - row_begin, FA_SAGE_BLOCK);
-    FaLaunchScope scope(ctx, "sage_quantize_k_kernel");
-    hipLaunchKernelGGL(sage_quantize_k_kernel, dim3(nblk, n_kv_heads), dim3(256), 0, ctx->stream, (const __half *)k, mean,
+    FaLaunchScope scope(ctx, "sage_quantize_k_kernel", true);
+    scope.launch(sage_quantize_k_kernel, dim3(nblk, n_kv_heads), dim3(256), 0, (const __half *)k, mean,
                        capacity, head_dim, row_begin, row_end, (int8_t *)k_q, (__half *)k_scale,
                        ceil_div_u32(capacity, FA_SAGE_BLOCK));
     return scope.finish();
@@ -125,8 +125,8 @@ fa_status fa_launch_sage_quantize_k(fa_ctx *ctx, const void *k, const float *mea
 
 fa_status fa_launch_sage_quantize_q(fa_ctx *ctx, const void *q, uint32_t n_heads, uint32_t head_dim, void *q_q,
                                     float *q_scale) {
-    FaLaunchScope scope(ctx, "sage_quantize_q_kernel");
-    hipLaunchKernelGGL(sage_quantize_q_kernel, dim3(n_heads), dim3((head_dim + 63) / 64 * 64), 0, ctx->stream,
+    FaLaunchScope scope(ctx, "sage_quantize_q_kernel", true);
+    scope.launch(sage_quantize_q_kernel, dim3(n_heads), dim3((head_dim + 63) / 64 * 64), 0,
                        (const __half *)q, head_dim, (int8_t *)q_q, q_scale);
     return scope.finish();
 }
