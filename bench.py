@@ -258,6 +258,206 @@ def bench_prefill(f, args):
         sys.exit("parity check failed: cache_bit_exact=%s prefill_max_abs_err=%g" % (cache_ok, err))
 
 
+def _finish_secondary(f, args, name, workload, kernel, bytes_per_launch, dt, parity, extra=None):
+    n, ms = f.profile_query(kernel)
+    avg_s = ms / 1e3 / max(1, n)
+    achieved = bytes_per_launch / avg_s / 1e9
+    result = {
+        "metric": name, "value": args.steps / dt, "unit": "layer-steps/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic", "config": {"workload": workload},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": kernel, "avg_launch_us": avg_s * 1e6,
+                     "launches": n, "bytes_per_launch": bytes_per_launch},
+        "parity": parity,
+    }
+    if extra:
+        result.update(extra)
+    print(json.dumps(result))
+
+
+def bench_small_decode(f, args):
+    """Qwen2.5-0.5B-shaped single-layer decode step at 1024 context (contiguous cache): launch-latency bound."""
+    import orc
+    H, Hkv, D, pos, cap, NL = 14, 2, 64, 1024, 1152, 16
+    rng = np.random.default_rng(0xF0DD + 1)
+    cos, sin = fa.rope_tables(1e6, D, cap)
+    dcos, dsin = f.array(cos), f.array(sin)
+    host, caches = [], []
+    for i in range(NL):  # distinct caches so that no launch finds the previous one's data in cache
+        kc, vc = np.zeros((Hkv, cap, D), np.float16), np.zeros((Hkv, cap, D), np.float16)
+        kc[:, :pos] = rng.standard_normal((Hkv, pos, D), dtype=np.float32).astype(np.float16)
+        vc[:, :pos] = rng.standard_normal((Hkv, pos, D), dtype=np.float32).astype(np.float16)
+        caches.append((f.array(kc), f.array(vc)))
+        if i == 0:
+            host = [kc, vc]
+    q, k, v = (rng.standard_normal((1, n * D), dtype=np.float32).astype(np.float16) for n in (H, Hkv, Hkv))
+    dq, dk, dv, dqr, dout = f.array(q), f.array(k), f.array(v), f.zeros((H, 1, D)), f.zeros((1, H * D))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, 1, pos, cap, fa.ROPE_NEOX)
+
+    def step(i):
+        kc, vc = caches[i % NL]
+        f.decode_step_fused(dq.arg(), dk.arg(), dv.arg(), dqr.arg(), kc.arg(), vc.arg(), dcos.arg(), dsin.arg(),
+                            dout.arg(), p)
+
+    step(0)
+    f.synchronize()
+    want_qr = orc.kv_prep_fused(q, k, v, host[0], host[1], cos, sin, orc.make_params(H, Hkv, D, 1, pos, cap, rope_mode=0))
+    want = orc.sdpa_decode(want_qr[:, 0].copy(), host[0], host[1], H, Hkv, D, cap, pos + 1)
+    err = float(np.max(np.abs(dout.download().reshape(-1).astype(np.float64) - want.reshape(-1).astype(np.float64))))
+    ok = bool(np.array_equal(caches[0][0].download().view(np.uint16), host[0].view(np.uint16)))
+    for i in range(args.warmup):
+        step(i)
+    f.synchronize()
+    f.profile_reset()
+    f.profile_enable(True)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    nbytes = 2.0 * Hkv * (pos + 1) * D * 2 + 2 * Hkv * D * 2 + 2 * H * D * 2 + 2 * D
+    _finish_secondary(f, args, "decode-attn layer-steps/s + achieved HBM GB/s, Qwen2.5-0.5B shape @1K ctx",
+                      "qwen2.5-0.5b single-layer decode step: RoPE + KV append + flash decode, batch 1, H14/Hkv2/D64, "
+                      "kv_len 1025, eager launches (profiling events on)", "fused_rope_append_decode_kernel", nbytes, dt,
+                      {"cache_bit_exact": ok, "decode_max_abs_err": err})
+    f.profile_enable(False)
+
+
+def bench_paged_decode(f, args):
+    """Qwen2.5-3B-shaped batched paged decode, one layer per step: 32 ragged sequences, 16-token blocks."""
+    import orc
+    H, Hkv, D, bs, B, NL = 16, 2, 128, 16, 32, 4
+    rng = np.random.default_rng(0xF0DD + 3)
+    lens = rng.integers(512, 16385, size=B).astype(np.uint32)
+    need = [(int(n) + 1 + bs - 1) // bs for n in lens]
+    mb, nblk = max(need), sum(need) + 3
+    cos, sin = fa.rope_tables(1e6, D, 16400)
+    dcos, dsin = f.array(cos), f.array(sin)
+    layers, host0 = [], None
+    for i in range(NL):  # distinct pools, each larger than the last-level cache
+        perm = rng.permutation(nblk).astype(np.int32)
+        bt = np.zeros((B, mb), np.int32)
+        o = 0
+        for s_, n in enumerate(need):
+            bt[s_, :n] = perm[o:o + n]
+            o += n
+        kp = rng.standard_normal((nblk, Hkv, bs, D), dtype=np.float32).astype(np.float16)
+        vp = rng.standard_normal((nblk, Hkv, bs, D), dtype=np.float32).astype(np.float16)
+        dkp, dvp, dbt, dl = f.array(kp), f.array(vp), f.array(bt), f.array(lens)
+        layers.append((dkp, dvp, dbt, dl, fa.paged_kv(dkp, dvp, dbt, dl, nblk, Hkv, bs, D, B, mb)))
+        if i == 0:
+            host0 = (kp, vp, bt)
+    q, k, v = (rng.standard_normal((B, n * D), dtype=np.float32).astype(np.float16) for n in (H, Hkv, Hkv))
+    dq, dk, dv, dqr, dout = f.array(q), f.array(k), f.array(v), f.zeros((B, H, D)), f.zeros((B, H * D))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, B, 0, 0, fa.ROPE_NEOX)
+
+    def step(i):
+        f.decode_step_fused_paged(dq.arg(), dk.arg(), dv.arg(), dqr.arg(), layers[i % NL][4], dcos.arg(), dsin.arg(),
+                                  dout.arg(), p, 16400)
+
+    step(0)
+    f.synchronize()
+    got = dout.download().reshape(B, H, D)
+    err = 0.0
+    for b_ in (0, int(np.argmin(lens)), int(np.argmax(lens))):  # three sequences against the oracle
+        n = int(lens[b_])
+        kc = orc.paged_gather(host0[0], host0[2][b_], Hkv, bs, D, n, n + 1)
+        vc = orc.paged_gather(host0[1], host0[2][b_], Hkv, bs, D, n, n + 1)
+        qr = orc.kv_prep_fused(q[b_:b_ + 1], k[b_:b_ + 1], v[b_:b_ + 1], kc, vc, cos, sin,
+                               orc.make_params(H, Hkv, D, 1, n, n + 1, rope_mode=0))
+        want = orc.sdpa_decode(qr[:, 0].copy(), kc, vc, H, Hkv, D, n + 1, n + 1, n_threads=8).reshape(H, D)
+        err = max(err, float(np.max(np.abs(got[b_].astype(np.float64) - want.astype(np.float64)))))
+    for i in range(args.warmup):
+        step(i)
+    f.synchronize()
+    f.profile_reset()
+    f.profile_enable(True)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    total = float(np.sum(lens.astype(np.float64) + 1))
+    nbytes = 2.0 * Hkv * total * D * 2 + B * (2 * Hkv * D * 2 + 2 * H * D * 2 + 2 * D + 4) + 4.0 * sum(need)
+    _finish_secondary(f, args, "paged decode-attn layer-steps/s + achieved HBM GB/s, Qwen2.5-3B shape, 32 ragged sequences",
+                      "qwen2.5-3b batched paged decode, one layer per step: 32 sequences of %d..%d tokens (sum %d), "
+                      "H16/Hkv2/D128, 16-token blocks with a permuted block table, RoPE + append + flash decode in one "
+                      "launch + merge" % (int(lens.min()), int(lens.max()), int(lens.sum())),
+                      "fused_rope_append_decode_kernel", nbytes, dt, {"decode_max_abs_err_3_sequences": err})
+    f.profile_enable(False)
+
+
+def bench_sage_decode(f, args):
+    """SmolLM3-shaped decode with int8 Q/K (per-32-token scales, mean-smoothed K) at 32K context, one layer per step."""
+    import orc
+    H, Hkv, D, N, NL = 16, 4, 128, 32768, 6
+    rng = np.random.default_rng(0xF0DD + 5)
+
+    def outliers(shape):
+        x = rng.standard_normal(shape, dtype=np.float32)
+        mask = rng.random(shape) < 0.01
+        x[mask] = np.sign(x[mask]) * 8.0
+        return x.astype(np.float16)
+
+    layers, host0 = [], None
+    for i in range(NL):
+        k, v = outliers((Hkv, N, D)), outliers((Hkv, N, D))
+        dk, dv = f.array(k), f.array(v)
+        dmean = f.zeros((Hkv, D), np.float32)
+        dkq, dks = f.zeros((Hkv, N, D), np.int8), f.zeros((Hkv, N // 32), np.float16)
+        f.sage_k_mean(dk, Hkv, N, D, N, dmean)
+        f.sage_quantize_k(dk, dmean, Hkv, N, D, 0, N, dkq, dks)
+        f.synchronize()
+        dk.free()
+        layers.append((dkq, dks, dv))
+        if i == 0:
+            host0 = (k, v)
+    q = outliers((H, D))
+    dq, dqq, dqs, dout = f.array(q), f.zeros((H, D), np.int8), f.zeros((H,), np.float32), f.zeros((H * D,))
+
+    def step(i):
+        dkq, dks, dv = layers[i % NL]
+        f.sage_quantize_q(dq, H, D, dqq, dqs)
+        f.sage_decode(dqq, dqs, dkq, dks, dv, dout, H, Hkv, D, N, N)
+
+    step(0)
+    f.synchronize()
+    got = dout.download().reshape(H, D).astype(np.float64)
+    kq, ks = layers[0][0].download(), layers[0][1].download()
+    qq, qs = orc.sage_quantize_q(q, H, D)
+    model = orc.sage_decode(qq, qs, kq, ks, host0[1], H, Hkv, D, N, N, n_threads=8).reshape(H, D).astype(np.float64)
+    err_model = float(np.max(np.abs(got - model)))
+    kf, vf, qf = host0[0].astype(np.float64), host0[1].astype(np.float64), q.astype(np.float64)
+    full = np.zeros((H, D))
+    for h in range(H):  # f16 SDPA on the unquantised tensors, in float64
+        s_ = kf[h // (H // Hkv)] @ qf[h] / np.sqrt(D)
+        w = np.exp(s_ - s_.max())
+        full[h] = (w / w.sum()) @ vf[h // (H // Hkv)]
+    err_full = float(np.max(np.abs(got - full)))
+    for i in range(args.warmup):
+        step(i)
+    f.synchronize()
+    f.profile_reset()
+    f.profile_enable(True)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    nbytes = float(Hkv * N * D + Hkv * (N // 32) * 2 + Hkv * N * D * 2 + 2 * H * D * 2)
+    _finish_secondary(f, args, "int8-QK decode-attn layer-steps/s + achieved HBM GB/s, SmolLM3 shape @32K ctx",
+                      "smollm3 decode attention with int8 Q/K (K mean-smoothed, per-32-token f16 scales; f16 V), one layer per "
+                      "step, batch 1, H16/Hkv4/D128, kv_len 32768, 1% of entries at 8 sigma", "sage_decode_mfma_kernel",
+                      nbytes, dt, {"max_abs_err_vs_int8_cpu_model": err_model, "max_abs_err_vs_f16_sdpa_unquantised": err_full},
+                      {"dtype": "i8 (QK^T) / f16 (PV)"})
+    f.profile_enable(False)
+
+
+SECONDARY = {"llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
+             "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -277,15 +477,15 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is built and measured on a single MI355X (--gpus 1); "
                  "how it would shard across GPUs is described in DESIGN.md")
-    if args.workload == "llama3b_prefill_2k":  # secondary line: the MFMA-bound half of the path
+    if args.workload in SECONDARY:  # secondary lines: the other configurations of the path, one layer per step
         f = fa.Foundry(0)
         args.steps, args.warmup = min(args.steps, 200), min(args.warmup, 20)
-        bench_prefill(f, args)
+        SECONDARY[args.workload](f, args)
         f.close()
         return
     if args.workload != "llama3b_decode_8k":
-        sys.exit("unknown workload %r (llama3b_decode_8k is the bench line, llama3b_prefill_2k a secondary one; the "
-                 "other configurations are parity-test cases)" % args.workload)
+        sys.exit("unknown workload %r (llama3b_decode_8k is the bench line; secondary: %s)"
+                 % (args.workload, ", ".join(sorted(SECONDARY))))
 
     room = 256  # the metric's timed window: 256 consecutive decode steps from 8192 context
     rng = np.random.default_rng(0xF0DD + 2)

@@ -30,7 +30,11 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
         const uint64_t groups = (uint64_t)L.batch * ny;
         const uint64_t slots = (uint64_t)(ctx->n_cus > 0 ? ctx->n_cus : 256);
         const uint32_t s_max = groups >= slots ? 1u : (uint32_t)(slots / groups);
-        chunk = ceil_div_u32(ceil_div_u32(bound, s_max), (uint32_t)BK) * BK;
+        // Long partitions are cut further, into a whole number of workgroups per CU, so that a batch of ragged
+        // sequences (whose short members leave most of their partitions empty) still balances over the CUs.
+        const uint32_t long_chunk = 2u * NW * MBX * BK;  // two rounds of a workgroup
+        const uint32_t per_cu = ceil_div_u32(ceil_div_u32(bound, s_max), long_chunk);
+        chunk = ceil_div_u32(ceil_div_u32(bound, s_max * per_cu), (uint32_t)BK) * BK;
         if (chunk < (uint32_t)(NW * BK)) chunk = NW * BK;
     }
     chunk = (chunk + BK - 1) / BK * BK;
