@@ -35,7 +35,7 @@ struct PrefillDev {
     __half *out;
     uint64_t q_stride_h, q_stride_m, k_stride_h, v_stride_h, out_stride_h, out_stride_m;
     const int32_t *block_table;
-    uint32_t n_heads, group_size, q_len, kv_len, query_offset, causal, block_size, n_kv_heads, paged;
+    uint32_t n_heads, group_size, q_len, kv_len, query_offset, causal, block_size, block_shift, n_kv_heads, paged;
     float scale_log2e;
 };
 
@@ -51,21 +51,51 @@ struct Lds {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 template <int D>
-__global__ void __launch_bounds__(256, 2) flash_prefill_mfma_kernel(PrefillDev a) {
+struct Chunk;  // what one of the 16 threads of a row moves: D*2/16 bytes
+template <>
+struct Chunk<128> {
+    typedef uint4 type;
+    static __device__ __forceinline__ uint4 zero() { return make_uint4(0, 0, 0, 0); }
+    static __device__ __forceinline__ uint4 buffer_load(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+        return __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+    }
+};
+template <>
+struct Chunk<64> {
+    typedef uint2 type;
+    static __device__ __forceinline__ uint2 zero() { return make_uint2(0, 0); }
+    static __device__ __forceinline__ uint2 buffer_load(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+        return __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
+    }
+};
+
+template <int D>
+__global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a) {
     constexpr int DSTEPS = D / 16;  // MFMA k-steps over head_dim for S^T
     constexpr int DBLKS = D / 32;   // 32-row blocks of O^T
     constexpr int KRS = Lds<D>::KRS, VRS = Lds<D>::VRS;
-    constexpr int CPR = D / 8;             // 16-byte chunks per row
-    constexpr int LOADS = BN * CPR / 256;  // chunks per thread per tile
+    constexpr int CB = D * 2 / 16;   // bytes per thread per row: 16 threads move one row
+    constexpr int LOADS = BN / 16;   // 16-row groups per tile; a group never straddles a page (block_size % 16 == 0)
+    typedef typename Chunk<D>::type chunk_t;
 
-    __shared__ __attribute__((aligned(16))) unsigned char k_lds[BN * KRS];
-    __shared__ __attribute__((aligned(16))) unsigned char v_lds[BN * VRS];
+    // The 8 waves form two groups of 4. Both groups serve the same 128 query rows; group g attends the key tiles
+    // t = g, g + 2, ... from LDS buffers of its own, and the two running states are merged through LDS at the end.
+    // Under the causal mask the last query tile sees the most keys and bounds the launch: splitting its keys
+    // inside the workgroup halves that critical path without any traffic to memory.
+    constexpr int TILE_LDS = BN * KRS + BN * VRS;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * TILE_LDS];
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int lane = threadIdx.x & 63;
+    const int wave8 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int grp = wave8 >> 2, wave = wave8 & 3;
+    const int tid = threadIdx.x & 255;  // thread within the group
+    unsigned char *k_lds = lds + grp * TILE_LDS, *v_lds = k_lds + BN * KRS;
     const int n = lane & 31, hi = lane >> 5;
-    // heaviest (latest) query tiles first: they see the most keys under the causal mask
-    const uint32_t q_tile = gridDim.x - 1 - blockIdx.x;
-    const uint32_t head = blockIdx.y;
+    // heaviest (latest) query tiles first, over all heads: they see the most keys under the causal mask.
+    // Workgroup ids that are equal modulo 8 share an L2 (one XCD): they get the same few heads.
+    const uint32_t n_qt = gridDim.x / a.n_heads;
+    const uint32_t q_tile = n_qt - 1 - blockIdx.x / a.n_heads;
+    const uint32_t head = blockIdx.x % a.n_heads;
     const uint32_t kvh = head / a.group_size;
     const uint32_t q0 = q_tile * BM;
     const uint32_t q_row = q0 + wave * 32 + n;  // the query row this lane's column belongs to
@@ -79,9 +109,6 @@ __global__ void __launch_bounds__(256, 2) flash_prefill_mfma_kernel(PrefillDev a
     }
     const int n_tiles = (int)((kv_end + BN - 1) / BN);
 
-    const __half *kbase = a.paged ? a.k : a.k + (size_t)kvh * a.k_stride_h;
-    const __half *vbase = a.paged ? a.v : a.v + (size_t)kvh * a.v_stride_h;
-
     // Q^T operand: lane (n, hi) keeps Q[q_row][16*s + 8*hi .. +8] for every k-step s
     U4H8 qreg[DSTEPS];
     {
@@ -90,47 +117,66 @@ __global__ void __launch_bounds__(256, 2) flash_prefill_mfma_kernel(PrefillDev a
         for (int s = 0; s < DSTEPS; ++s) qreg[s].u = *reinterpret_cast<const uint4 *>(qp + s * 16 + hi * 8);
     }
 
-    // A paged cache needs the page of every row before the row itself can be requested. The page ids of a tile are
-    // fetched one tile ahead of its rows (which are fetched one tile ahead of their use), so that no iteration
-    // waits for two dependent memory round trips.
-    uint4 kreg[LOADS], vreg[LOADS];
+    // Tile fetch: thread (r = tid / 16, c = tid % 16) moves chunk c of rows 16j + r of the tile, j < LOADS.
+    // Contiguous cache: buffer loads over the visible rows of the KV head (rows past them read as zero, tile base
+    // in an SGPR). Paged cache: the page id of a 16-row group is wave-uniform and read through the scalar cache one
+    // tile before its rows are requested (which is one tile before they are used), so no iteration waits for two
+    // dependent memory round trips.
+    const int fr = tid >> 4, fc = tid & 15;
+    const int lane_off = fr * (D * 2) + fc * CB;
+    chunk_t kreg[LOADS], vreg[LOADS];
+    __amdgpu_buffer_rsrc_t krs, vrs;
+    if (!a.paged) {
+        krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<__half *>(a.k + (size_t)kvh * a.k_stride_h), 0,
+                                                (int)(kv_end * (uint32_t)(D * 2)), 0x00020000);
+        vrs = __builtin_amdgcn_make_buffer_rsrc(const_cast<__half *>(a.v + (size_t)kvh * a.v_stride_h), 0,
+                                                (int)(kv_end * (uint32_t)(D * 2)), 0x00020000);
+    }
+    typedef const int32_t __attribute__((address_space(4))) *const_i32p;
+    const const_i32p bt = (const_i32p)a.block_table;
+    const uint32_t bs_shift = a.block_shift;  // log2(block_size), or 32 when it is not a power of two
     int32_t page[LOADS];
     auto fetch_pages = [&](int tile) {
         if (!a.paged) return;
 #pragma unroll
         for (int j = 0; j < LOADS; ++j) {
-            const uint32_t key = (uint32_t)tile * BN + (tid + 256 * j) / CPR;
-            page[j] = key < kv_end ? a.block_table[key / a.block_size] : 0;
+            const uint32_t key = (uint32_t)tile * BN + 16 * j;  // wave-uniform
+            page[j] = key < kv_end ? bt[bs_shift < 32 ? key >> bs_shift : key / a.block_size] : 0;
         }
     };
     auto fetch = [&](int tile) {
+        if (!a.paged) {
+            const int tb = tile * (BN * D * 2);
+#pragma unroll
+            for (int j = 0; j < LOADS; ++j) {
+                kreg[j] = Chunk<D>::buffer_load(krs, lane_off, tb + j * (16 * D * 2));
+                vreg[j] = Chunk<D>::buffer_load(vrs, lane_off, tb + j * (16 * D * 2));
+            }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < LOADS; ++j) {
-            const int id = tid + 256 * j;
-            const int row = id / CPR, seg = id % CPR;
-            const uint32_t key = (uint32_t)tile * BN + row;
+            const uint32_t key = (uint32_t)tile * BN + 16 * j;  // first row of the group, wave-uniform
             if (key < kv_end) {
-                size_t off;
-                if (a.paged) {
-                    off = (((size_t)page[j] * a.n_kv_heads + kvh) * a.block_size + key % a.block_size) * (size_t)D;
-                } else {
-                    off = (size_t)key * D;
+                const uint32_t rip = bs_shift < 32 ? key & (a.block_size - 1) : key % a.block_size;  // row in page
+                const size_t base = (((size_t)page[j] * a.n_kv_heads + kvh) * a.block_size + rip) * (size_t)(D * 2);
+                kreg[j] = *reinterpret_cast<const chunk_t *>(reinterpret_cast<const unsigned char *>(a.k) + base + lane_off);
+                vreg[j] = *reinterpret_cast<const chunk_t *>(reinterpret_cast<const unsigned char *>(a.v) + base + lane_off);
+                if (key + 16 > kv_end && key + fr >= kv_end) {  // rows past the end must be finite: their weight is 0
+                    kreg[j] = Chunk<D>::zero();
+                    vreg[j] = Chunk<D>::zero();
                 }
-                kreg[j] = *reinterpret_cast<const uint4 *>(kbase + off + seg * 8);
-                vreg[j] = *reinterpret_cast<const uint4 *>(vbase + off + seg * 8);
-            } else {  // rows past the end must be finite: their probabilities are 0
-                kreg[j] = make_uint4(0, 0, 0, 0);
-                vreg[j] = make_uint4(0, 0, 0, 0);
+            } else {
+                kreg[j] = Chunk<D>::zero();
+                vreg[j] = Chunk<D>::zero();
             }
         }
     };
     auto stash = [&]() {
 #pragma unroll
         for (int j = 0; j < LOADS; ++j) {
-            const int id = tid + 256 * j;
-            const int row = id / CPR, seg = id % CPR;
-            *reinterpret_cast<uint4 *>(k_lds + row * KRS + seg * 16) = kreg[j];
-            *reinterpret_cast<uint4 *>(v_lds + row * VRS + seg * 16) = vreg[j];
+            *reinterpret_cast<chunk_t *>(k_lds + (16 * j + fr) * KRS + fc * CB) = kreg[j];
+            *reinterpret_cast<chunk_t *>(v_lds + (16 * j + fr) * VRS + fc * CB) = vreg[j];
         }
     };
 
@@ -139,23 +185,28 @@ __global__ void __launch_bounds__(256, 2) flash_prefill_mfma_kernel(PrefillDev a
     for (int b = 0; b < DBLKS; ++b)
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[b][i] = 0.0f;
+    // running max in the exp2 domain (score * scale * log2 e); l_run: this lane's share of the row sum
     float m_run = -1e30f, l_run = 0.0f;
     const float c = a.scale_log2e;
     const uint32_t q_abs = q_row_c + a.query_offset;  // last visible key of this lane's row when causal
     // first key index that some row of this wave cannot see
     const uint32_t wave_min_limit = a.causal ? (min(q0 + wave * 32, a.q_len - 1) + a.query_offset) : 0xffffffffu;
 
-    if (n_tiles > 0) {
-        fetch_pages(0);
-        fetch(0);
-        if (n_tiles > 1) fetch_pages(1);
+    if (grp < n_tiles) {
+        fetch_pages(grp);
+        fetch(grp);
+        if (grp + 2 < n_tiles) fetch_pages(grp + 2);
     }
-    for (int tile = 0; tile < n_tiles; ++tile) {
+    const int iters = (n_tiles + 1) / 2;  // the same for both groups: the barriers are workgroup-wide
+    for (int it = 0; it < iters; ++it) {
+        const int tile = 2 * it + grp;
+        const bool active = tile < n_tiles;
         __syncthreads();  // previous tile fully consumed
-        stash();
+        if (active) stash();
         __syncthreads();
-        if (tile + 1 < n_tiles) fetch(tile + 1);
-        if (tile + 2 < n_tiles) fetch_pages(tile + 2);
+        if (!active) continue;
+        if (tile + 2 < n_tiles) fetch(tile + 2);
+        if (tile + 4 < n_tiles) fetch_pages(tile + 4);
 
         const uint32_t key0 = (uint32_t)tile * BN;
         // S^T for the two 32-key blocks of the tile
@@ -188,27 +239,30 @@ __global__ void __launch_bounds__(256, 2) flash_prefill_mfma_kernel(PrefillDev a
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, sacc[kb][i]);
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-        const float m_new = fmaxf(m_run, mloc);
-        const float alpha = fast_exp2((m_run - m_new) * c);
-        const float mc = m_new * c;
-        float lsum = 0.0f;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float p = fast_exp2(fmaf(sacc[kb][i], c, -mc));
-                sacc[kb][i] = p;
-                lsum += p;
-            }
-        l_run = l_run * alpha + lsum;
-        m_run = m_new;
-        if (__any(alpha != 1.0f)) {
+        mloc = fmaxf(mloc, __shfl_xor(mloc, 32)) * c;
+        // The accumulators are rescaled only when the row maximum has grown by more than 2^8: until then the stale
+        // maximum is kept (weights up to 256 instead of 1; the final division by l removes the common factor), which
+        // saves the 16 * DBLKS multiplications on almost every tile after the first.
+        if (__any(mloc > m_run + 8.0f)) {
+            const float m_new = fmaxf(m_run, mloc);
+            const float alpha = fast_exp2(m_run - m_new);
+            l_run *= alpha;
+            m_run = m_new;
 #pragma unroll
             for (int b = 0; b < DBLKS; ++b)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
         }
+        float lsum = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float p = fast_exp2(fmaf(sacc[kb][i], c, -m_run));
+                sacc[kb][i] = p;
+                lsum += p;
+            }
+        l_run += lsum;
         // O^T += V^T . P^T : k-slot j of k-step ks <-> key 32*kb + 16*ks' ... = accumulator 8*ks + j of block kb
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
@@ -225,21 +279,41 @@ __global__ void __launch_bounds__(256, 2) flash_prefill_mfma_kernel(PrefillDev a
                 for (int b = 0; b < DBLKS; ++b) {
                     const unsigned char *p0 = v_lds + (kbase16 + jr) * VRS + (b * 32 + dsub + cc * 4) * 2;
                     const unsigned char *p1 = p0 + 8 * VRS;
-                    fp16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
-                        (fp16x4_t __attribute__((address_space(3))) *)(p0));
-                    fp16x4_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
-                        (fp16x4_t __attribute__((address_space(3))) *)(p1));
-                    h8_t va;
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        va[j] = (_Float16)lo[j];
-                        va[4 + j] = (_Float16)hi4[j];
-                    }
-                    oacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va, pb, oacc[b], 0, 0, 0);
+                    union {
+                        fp16x4_t f[2];
+                        h8_t h;
+                    } va;
+                    va.f[0] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p0));
+                    va.f[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p1));
+                    oacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va.h, pb, oacc[b], 0, 0, 0);
                 }
             }
     }
 
+    // merge the two groups' states: group 1 parks (m, l, acc) in LDS as [value][wave][lane], group 0 folds them in
+    {
+        float *mx = reinterpret_cast<float *>(lds);
+        const int slot = wave * 64 + lane;
+        __syncthreads();  // both groups are done with their tiles
+        if (grp == 1) {
+            mx[slot] = m_run;
+            mx[256 + slot] = l_run;
+#pragma unroll
+            for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) mx[(2 + b * 16 + i) * 256 + slot] = oacc[b][i];
+        }
+        __syncthreads();
+        if (grp == 1) return;
+        const float m1 = mx[slot], l1 = mx[256 + slot];
+        const float m = fmaxf(m_run, m1);
+        const float e0 = fast_exp2(m_run - m), e1 = fast_exp2(m1 - m);
+        l_run = l_run * e0 + l1 * e1;
+#pragma unroll
+        for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[b][i] = oacc[b][i] * e0 + mx[(2 + b * 16 + i) * 256 + slot] * e1;
+    }
     // finalise: l over both lane halves, flash_prefill.metal:255-261
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     const float inv_l = (isfinite(l_tot) && fabsf(l_tot) > 1e-6f) ? (1.0f / l_tot) : 0.0f;
@@ -269,14 +343,18 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
     a.n_heads = L.n_heads, a.group_size = L.group_size, a.q_len = L.q_len, a.kv_len = L.kv_len;
     a.query_offset = L.query_offset, a.causal = L.causal ? 1u : 0u, a.block_size = L.block_size;
     a.n_kv_heads = L.n_kv_heads, a.paged = L.paged ? 1u : 0u;
+    a.block_shift = 32;
+    if (L.paged && L.block_size && (L.block_size & (L.block_size - 1)) == 0) a.block_shift = (uint32_t)__builtin_ctz(L.block_size);
+    if (!L.paged && (uint64_t)L.kv_len * L.head_dim * 2 >= (1ull << 32))
+        return fa_fail(FA_ERR_INVALID_SHAPE, "prefill: one KV head of the contiguous cache must stay below 4 GiB");
     a.scale_log2e = L.scale * 1.4426950408889634f;
     if (L.q_len == 0) return FA_OK;
-    dim3 grid(ceil_div_u32(L.q_len, BM), L.n_heads, 1);
+    dim3 grid(ceil_div_u32(L.q_len, BM) * L.n_heads, 1, 1);
     FaLaunchScope scope(ctx, "flash_prefill_mfma_kernel", true);
     if (L.head_dim == 128)
-        scope.launch(flash_prefill_mfma_kernel<128>, grid, dim3(256), 0, a);
+        scope.launch(flash_prefill_mfma_kernel<128>, grid, dim3(512), 0, a);
     else if (L.head_dim == 64)
-        scope.launch(flash_prefill_mfma_kernel<64>, grid, dim3(256), 0, a);
+        scope.launch(flash_prefill_mfma_kernel<64>, grid, dim3(512), 0, a);
     else
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill only supports head_dim=64 or 128, got %u", L.head_dim);
     return scope.finish();
