@@ -24,6 +24,7 @@ typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
 typedef float f16_t __attribute__((ext_vector_type(16)));
 typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
+typedef unsigned int u4_t __attribute__((ext_vector_type(4)));
 
 union U4H8 {
     uint4 u;
@@ -83,13 +84,13 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
     // Under the causal mask the last query tile sees the most keys and bounds the launch: splitting its keys
     // inside the workgroup halves that critical path without any traffic to memory.
     constexpr int TILE_LDS = BN * KRS + BN * VRS;
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * TILE_LDS];
+    __shared__ __attribute__((aligned(16))) unsigned char lds[4 * TILE_LDS];  // [group][buffer]
 
     const int lane = threadIdx.x & 63;
     const int wave8 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int grp = wave8 >> 2, wave = wave8 & 3;
     const int tid = threadIdx.x & 255;  // thread within the group
-    unsigned char *k_lds = lds + grp * TILE_LDS, *v_lds = k_lds + BN * KRS;
+    unsigned char *grp_lds = lds + grp * (2 * TILE_LDS);
     const int n = lane & 31, hi = lane >> 5;
     // heaviest (latest) query tiles first, over all heads: they see the most keys under the causal mask.
     // Workgroup ids that are equal modulo 8 share an L2 (one XCD): they get the same few heads.
@@ -172,11 +173,12 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
             }
         }
     };
-    auto stash = [&]() {
+    auto stash = [&](int buf) {
+        unsigned char *kd = grp_lds + buf * TILE_LDS, *vd = kd + BN * KRS;
 #pragma unroll
         for (int j = 0; j < LOADS; ++j) {
-            *reinterpret_cast<chunk_t *>(k_lds + (16 * j + fr) * KRS + fc * CB) = kreg[j];
-            *reinterpret_cast<chunk_t *>(v_lds + (16 * j + fr) * VRS + fc * CB) = vreg[j];
+            *reinterpret_cast<chunk_t *>(kd + (16 * j + fr) * KRS + fc * CB) = kreg[j];
+            *reinterpret_cast<chunk_t *>(vd + (16 * j + fr) * VRS + fc * CB) = vreg[j];
         }
     };
 
@@ -192,21 +194,36 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
     // first key index that some row of this wave cannot see
     const uint32_t wave_min_limit = a.causal ? (min(q0 + wave * 32, a.q_len - 1) + a.query_offset) : 0xffffffffu;
 
+    // Two LDS buffers per group and one barrier per tile: while a tile is attended from one buffer, the next
+    // one (requested a whole tile earlier) is stored into the other, and the one after that is requested.
     if (grp < n_tiles) {
         fetch_pages(grp);
         fetch(grp);
         if (grp + 2 < n_tiles) fetch_pages(grp + 2);
+        stash(0);
+        if (grp + 2 < n_tiles) {
+            fetch(grp + 2);
+            if (grp + 4 < n_tiles) fetch_pages(grp + 4);
+        }
     }
+    // Pin the query operand as "arrived" before the loop. Left to itself the compiler sinks the (loop-invariant)
+    // query loads below the prefetch of the second tile, and then has to wait, at the top of EVERY iteration, for
+    // everything requested before them - which in steady state is the prefetch it should be overlapping.
+#pragma unroll
+    for (int s = 0; s < DSTEPS; ++s) {
+        u4_t t = __builtin_bit_cast(u4_t, qreg[s].u);
+        asm volatile("" : "+v"(t));
+        qreg[s].u = __builtin_bit_cast(uint4, t);
+    }
+    __syncthreads();
     const int iters = (n_tiles + 1) / 2;  // the same for both groups: the barriers are workgroup-wide
     for (int it = 0; it < iters; ++it) {
         const int tile = 2 * it + grp;
-        const bool active = tile < n_tiles;
-        __syncthreads();  // previous tile fully consumed
-        if (active) stash();
-        __syncthreads();
-        if (!active) continue;
-        if (tile + 2 < n_tiles) fetch(tile + 2);
-        if (tile + 4 < n_tiles) fetch_pages(tile + 4);
+        if (tile >= n_tiles) {  // this group has one tile less
+            __syncthreads();
+            continue;
+        }
+        const unsigned char *k_lds = grp_lds + (it & 1) * TILE_LDS, *v_lds = k_lds + BN * KRS;
 
         const uint32_t key0 = (uint32_t)tile * BN;
         // S^T for the two 32-key blocks of the tile
@@ -288,14 +305,21 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
                     oacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va.h, pb, oacc[b], 0, 0, 0);
                 }
             }
+        if (tile + 2 < n_tiles) {
+            stash((it + 1) & 1);
+            if (tile + 4 < n_tiles) {
+                fetch(tile + 4);
+                if (tile + 6 < n_tiles) fetch_pages(tile + 6);
+            }
+        }
+        __syncthreads();
     }
 
     // merge the two groups' states: group 1 parks (m, l, acc) in LDS as [value][wave][lane], group 0 folds them in
     {
         float *mx = reinterpret_cast<float *>(lds);
         const int slot = wave * 64 + lane;
-        __syncthreads();  // both groups are done with their tiles
-        if (grp == 1) {
+        if (grp == 1) {  // (the loop ended with a barrier: both groups are done with their tiles)
             mx[slot] = m_run;
             mx[256 + slot] = l_run;
 #pragma unroll
