@@ -54,6 +54,7 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     a.capacity = L.capacity, a.chunk = chunk, a.n_kv_heads = L.n_kv_heads, a.sub_per_kv = sub_per_kv;
     a.gt = (uint32_t)gt;
     a.bt_stride = L.bt_stride, a.block_size = L.block_size;
+    a.block_shift = (L.block_size && (L.block_size & (L.block_size - 1)) == 0) ? (uint32_t)__builtin_ctz(L.block_size) : 32u;
     a.merge_in_kernel = ctx->decode_variant.merge == 0 ? 1u : 0u;
     a.scale_log2e = L.scale * 1.4426950408889634f;
     a.q_scale = L.q_scale, a.k_scale = L.k_scale, a.ks_stride = L.ks_stride;

@@ -74,7 +74,7 @@ struct DecodeDev {
     float *part_ml;      // [batch][y][S][gt][2]
     uint32_t *counters;  // [batch][y]
     uint32_t kv_len, d_len_stride, kv_len_add, kv_len_bound, capacity, chunk, n_kv_heads, sub_per_kv, gt;
-    uint32_t bt_stride, block_size, merge_in_kernel;
+    uint32_t bt_stride, block_size, block_shift /* log2(block_size), 32 if not a power of two */, merge_in_kernel;
     float scale_log2e;
     // Sage-style int8 Q/K: q and k point at int8 data, scores are rescaled by q_scale[h] * k_scale[kvh][key/32]
     const float *q_scale;
@@ -277,9 +277,26 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
     // V block  : lane reads row i*VRPL + lane / VLPR, segment lane % VLPR in load i (1 KiB per load).
     // A contiguous cache is read through buffer descriptors that span the (sequence, KV head) slab: one VGPR of
     // lane offset serves every load (per-load 64-bit addresses would cost as many VGPRs as the data), and rows past
-    // the slab read as zero instead of needing a clamp. A paged cache looks every row up in the block table;
-    // `lim` = last row that may be addressed there.
+    // the slab read as zero instead of needing a clamp. In a paged cache a 16-key block lies inside one page (the
+    // page size is a multiple of 16), so its page id is wave-uniform: it is read through the scalar cache one round
+    // ahead (`pgn`), and the rows are addressed as page base (SGPRs) + the same lane offset. Rows of the page past
+    // the sequence end exist, so nothing needs a clamp there either.
     U4H kk[MBX][KSTEPS], vv[MBX][VLB];
+    typedef const int32_t __attribute__((address_space(4))) *const_i32p;
+    const const_i32p btc = (const_i32p)bt;
+    int32_t pgi[MBX] = {}, pgn[MBX] = {};  // page ids of the round being requested / of the one after
+    auto load_pages = [&](uint32_t blk, uint32_t m, int32_t(&dst)[MBX]) {
+#pragma unroll
+        for (int mb = 0; mb < MBX; ++mb) {
+            if ((uint32_t)mb >= m) break;
+            const uint32_t row0 = k0 + (blk + mb) * BK;
+            dst[mb] = btc[a.block_shift < 32 ? row0 >> a.block_shift : row0 / a.block_size];
+        }
+    };
+    auto page_row = [&](int32_t page, uint32_t row0) -> size_t {  // element offset of row `row0` inside `page`
+        const uint32_t rip = a.block_shift < 32 ? row0 & (a.block_size - 1) : row0 % a.block_size;
+        return (((size_t)page * a.n_kv_heads + kvh) * a.block_size + rip) * (size_t)D;
+    };
     __amdgpu_buffer_rsrc_t krs, vrs;
     if (!PAGED) {
         krs = __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char *>(kbase), 0,
@@ -300,9 +317,9 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
                     kk[mb][j].u = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
                                                                 krs, k_lane_off + j * 64, (int)(row0 * (uint32_t)(D * KES)), 0));
             } else {
-                const unsigned char *row = kbase + row_offset(min(row0 + n, lim)) * KES;
+                const unsigned char *blk0 = kbase + page_row(pgi[mb], row0) * KES;  // wave-uniform
 #pragma unroll
-                for (int j = 0; j < KSTEPS; ++j) kk[mb][j].u = *reinterpret_cast<const uint4 *>(row + (4 * j + c) * 16);
+                for (int j = 0; j < KSTEPS; ++j) kk[mb][j].u = *reinterpret_cast<const uint4 *>(blk0 + k_lane_off + j * 64);
             }
         }
     };
@@ -318,8 +335,8 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
                         uint4, __builtin_amdgcn_raw_buffer_load_b128(vrs, v_lane_off + i * VRPL * (D * 2),
                                                                      (int)(row0 * (uint32_t)(D * 2)), 0));
                 } else {
-                    const uint32_t key = min(row0 + i * VRPL + lane / VLPR, lim);
-                    vv[mb][i].u = *reinterpret_cast<const uint4 *>(vbase + row_offset(key) + (lane % VLPR) * 8);
+                    const unsigned char *blk0 = reinterpret_cast<const unsigned char *>(vbase + page_row(pgi[mb], row0));
+                    vv[mb][i].u = *reinterpret_cast<const uint4 *>(blk0 + v_lane_off + i * VRPL * (D * 2));
                 }
             }
         }
@@ -491,8 +508,10 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
     const uint32_t wbe = min(wb1, (kend - k0 + BK - 1) / BK);  // this wave's blocks that hold a valid key end here
     if (PAGED && cur < wbe) {
         const uint32_t m = min((uint32_t)MBX, wbe - cur);
+        load_pages(cur, m, pgi);
         issue_k(cur, m, k1 - 1);
         issue_v(cur, m, k1 - 1);
+        if (cur + m < wbe) load_pages(cur + m, min((uint32_t)MBX, wbe - (cur + m)), pgn);
     }
     __syncthreads();  // the Q^T operand is in LDS
 
@@ -537,6 +556,10 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) s[mb * 4 + i] = -INFINITY;
             }
+        }
+        if (PAGED && mnext) {
+#pragma unroll
+            for (int mb = 0; mb < MBX; ++mb) pgi[mb] = pgn[mb];
         }
         if (mnext) issue_k(nblk, mnext, k1 - 1);  // K registers are free again
         float mt = -INFINITY;
@@ -598,6 +621,7 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
             }
         }
         if (mnext) issue_v(nblk, mnext, k1 - 1);  // V registers are free again
+        if (PAGED && mnext && nblk + mnext < wbe) load_pages(nblk + mnext, min((uint32_t)MBX, wbe - (nblk + mnext)), pgn);
     };
 
     while (cur < wbe) {
