@@ -226,6 +226,13 @@ typedef struct fa_decode_variant {
 } fa_decode_variant;
 fa_status fa_set_decode_variant(fa_ctx *ctx, const fa_decode_variant *variant);
 
+/* Prefill split-K override, the counterpart of the reference's prefill split-K selector and its environment
+ * override (src/metals/flashattention/step.rs:849-864): the key tiles of every query tile are divided over
+ * `split_k` workgroups whose states are merged by a second kernel (flash_prefill.metal:452-457,843-888).
+ * 0 = auto (split only when the query tiles alone would leave most compute units idle), 1 = never, max 64.
+ * Environment: FOUNDRY_ATTN_PREFILL_SPLIT_K (read at fa_ctx_create). */
+fa_status fa_set_prefill_split_k(fa_ctx *ctx, uint32_t split_k);
+
 /* ---------------------------------------------------------------------------------------------
  * Paged KV cache (no counterpart in the reference, whose cache is contiguous per layer and batch 1:
  * models/llama.json:301-330). Contract: gathering a sequence's blocks in block-table order yields,

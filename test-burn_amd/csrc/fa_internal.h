@@ -35,6 +35,7 @@ struct fa_ctx {
     uint32_t *counters = nullptr;
     uint32_t n_counters = 0;
     fa_decode_variant decode_variant{0, 1};
+    uint32_t prefill_split_k = 0;  // 0 = auto
     // per-kernel profiling
     bool profiling = false;
     std::vector<FaProfileRec> prof;

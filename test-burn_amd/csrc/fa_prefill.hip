@@ -37,6 +37,8 @@ struct PrefillDev {
     uint64_t q_stride_h, q_stride_m, k_stride_h, v_stride_h, out_stride_h, out_stride_m;
     const int32_t *block_table;
     uint32_t n_heads, group_size, q_len, kv_len, query_offset, causal, block_size, block_shift, n_kv_heads, paged;
+    uint32_t splits;             // > 1: the key tiles of a query tile are divided over `splits` workgroups
+    float *part_acc, *part_ml;   // [head][query tile][split][BM][D] unnormalised sums, [..][BM][2] (max, sum)
     float scale_log2e;
 };
 
@@ -94,9 +96,11 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
     const int n = lane & 31, hi = lane >> 5;
     // heaviest (latest) query tiles first, over all heads: they see the most keys under the causal mask.
     // Workgroup ids that are equal modulo 8 share an L2 (one XCD): they get the same few heads.
-    const uint32_t n_qt = gridDim.x / a.n_heads;
-    const uint32_t q_tile = n_qt - 1 - blockIdx.x / a.n_heads;
-    const uint32_t head = blockIdx.x % a.n_heads;
+    const uint32_t S = a.splits;
+    const uint32_t n_qt = gridDim.x / (a.n_heads * S);
+    const uint32_t q_tile = n_qt - 1 - blockIdx.x / (a.n_heads * S);
+    const uint32_t head = (blockIdx.x / S) % a.n_heads;
+    const uint32_t split = blockIdx.x % S;
     const uint32_t kvh = head / a.group_size;
     const uint32_t q0 = q_tile * BM;
     const uint32_t q_row = q0 + wave * 32 + n;  // the query row this lane's column belongs to
@@ -108,7 +112,12 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
         const uint64_t last = (uint64_t)min(q0 + BM - 1, a.q_len - 1) + a.query_offset + 1;
         kv_end = (uint32_t)min((uint64_t)a.kv_len, last);
     }
-    const int n_tiles = (int)((kv_end + BN - 1) / BN);
+    // this workgroup's key tiles [t_lo, n_tiles): all of them, or one of `splits` equal ranges
+    // (flash_prefill.metal:452-457)
+    const int all_tiles = (int)((kv_end + BN - 1) / BN);
+    const int per_split = (all_tiles + (int)S - 1) / (int)S;
+    const int t_lo = min(all_tiles, (int)split * per_split);
+    const int n_tiles = min(all_tiles, t_lo + per_split);
 
     // Q^T operand: lane (n, hi) keeps Q[q_row][16*s + 8*hi .. +8] for every k-step s
     U4H8 qreg[DSTEPS];
@@ -196,14 +205,15 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
 
     // Two LDS buffers per group and one barrier per tile: while a tile is attended from one buffer, the next
     // one (requested a whole tile earlier) is stored into the other, and the one after that is requested.
-    if (grp < n_tiles) {
-        fetch_pages(grp);
-        fetch(grp);
-        if (grp + 2 < n_tiles) fetch_pages(grp + 2);
+    const int t0 = t_lo + grp;  // this group's first tile
+    if (t0 < n_tiles) {
+        fetch_pages(t0);
+        fetch(t0);
+        if (t0 + 2 < n_tiles) fetch_pages(t0 + 2);
         stash(0);
-        if (grp + 2 < n_tiles) {
-            fetch(grp + 2);
-            if (grp + 4 < n_tiles) fetch_pages(grp + 4);
+        if (t0 + 2 < n_tiles) {
+            fetch(t0 + 2);
+            if (t0 + 4 < n_tiles) fetch_pages(t0 + 4);
         }
     }
     // Pin the query operand as "arrived" before the loop. Left to itself the compiler sinks the (loop-invariant)
@@ -216,9 +226,9 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
         qreg[s].u = __builtin_bit_cast(uint4, t);
     }
     __syncthreads();
-    const int iters = (n_tiles + 1) / 2;  // the same for both groups: the barriers are workgroup-wide
+    const int iters = (n_tiles - t_lo + 1) / 2;  // the same for both groups: the barriers are workgroup-wide
     for (int it = 0; it < iters; ++it) {
-        const int tile = 2 * it + grp;
+        const int tile = t0 + 2 * it;
         if (tile >= n_tiles) {  // this group has one tile less
             __syncthreads();
             continue;
@@ -337,9 +347,24 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
         for (int b = 0; b < DBLKS; ++b)
 #pragma unroll
             for (int i = 0; i < 16; ++i) oacc[b][i] = oacc[b][i] * e0 + mx[(2 + b * 16 + i) * 256 + slot] * e1;
+        m_run = m;
     }
-    // finalise: l over both lane halves, flash_prefill.metal:255-261
     const float l_tot = l_run + __shfl_xor(l_run, 32);
+    if (S > 1) {  // unnormalised partial state for the merge kernel (flash_prefill.metal:592-617)
+        if (q_row >= a.q_len) return;  // the merge kernel skips these rows too
+        const size_t prow = (((size_t)head * n_qt + q_tile) * S + split) * BM + wave * 32 + n;
+        float *pa = a.part_acc + prow * D;
+#pragma unroll
+        for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+            for (int gi = 0; gi < 4; ++gi) {
+                float4 v = make_float4(oacc[b][gi * 4], oacc[b][gi * 4 + 1], oacc[b][gi * 4 + 2], oacc[b][gi * 4 + 3]);
+                *reinterpret_cast<float4 *>(pa + b * 32 + gi * 8 + hi * 4) = v;
+            }
+        if (hi == 0) a.part_ml[prow * 2] = m_run, a.part_ml[prow * 2 + 1] = l_tot;
+        return;
+    }
+    // finalise, flash_prefill.metal:255-261
     const float inv_l = (isfinite(l_tot) && fabsf(l_tot) > 1e-6f) ? (1.0f / l_tot) : 0.0f;
     if (q_row < a.q_len) {
         __half *op = a.out + (size_t)head * a.out_stride_h + (size_t)q_row * a.out_stride_m;
@@ -354,6 +379,52 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
                 *reinterpret_cast<h4_t *>(op + b * 32 + gi * 8 + hi * 4) = o;
             }
     }
+}
+
+// Merge of the per-split states (flash_prefill.metal:843-888): m* = max m_s, L = sum l_s 2^(m_s - m*) over the
+// splits with l_s > 0, out = sum acc_s 2^(m_s - m*) / L (0 when L is unusable). m is kept in the exp2 domain.
+template <int D>
+__global__ void __launch_bounds__(256) flash_prefill_merge_kernel(PrefillDev a) {
+    constexpr int CG = D / 4;           // float4 columns per row
+    constexpr int ROWS = 256 / CG;      // rows per workgroup (8 at D = 128, 16 at D = 64)
+    constexpr int SLABS = BM / ROWS;    // workgroups per query tile
+    constexpr int PB = 8;               // splits loaded per batch
+    const uint32_t S = a.splits;
+    const uint32_t n_qt = gridDim.x / (a.n_heads * SLABS);
+    const uint32_t slab = blockIdx.x % SLABS, qh = blockIdx.x / SLABS;
+    const uint32_t q_tile = qh / a.n_heads, head = qh % a.n_heads;
+    const int r = slab * ROWS + threadIdx.x / CG, c4 = threadIdx.x % CG;
+    const uint32_t q_row = q_tile * BM + r;
+    if (q_row >= a.q_len) return;
+    const size_t base = (((size_t)head * n_qt + q_tile) * S) * BM + r;
+    float mstar = -1e30f;
+    for (uint32_t s = 0; s < S; ++s) {
+        const float *ml = a.part_ml + (base + (size_t)s * BM) * 2;
+        if (ml[1] > 0.0f) mstar = fmaxf(mstar, ml[0]);
+    }
+    float L = 0.0f;
+    float4 o = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (uint32_t s0 = 0; s0 < S; s0 += PB) {
+        float4 v[PB];
+        float2 ml[PB];
+#pragma unroll
+        for (int k = 0; k < PB; ++k) {
+            const uint32_t s = min(s0 + k, S - 1);  // clamped; masked below
+            v[k] = *reinterpret_cast<const float4 *>(a.part_acc + (base + (size_t)s * BM) * D + c4 * 4);
+            ml[k] = *reinterpret_cast<const float2 *>(a.part_ml + (base + (size_t)s * BM) * 2);
+        }
+#pragma unroll
+        for (int k = 0; k < PB; ++k) {
+            if (s0 + k >= S || !(ml[k].y > 0.0f)) continue;
+            const float w = fast_exp2(ml[k].x - mstar);
+            L += ml[k].y * w;
+            o.x += v[k].x * w, o.y += v[k].y * w, o.z += v[k].z * w, o.w += v[k].w * w;
+        }
+    }
+    const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 0.0f;
+    h4_t h;
+    h[0] = (_Float16)(o.x * inv), h[1] = (_Float16)(o.y * inv), h[2] = (_Float16)(o.z * inv), h[3] = (_Float16)(o.w * inv);
+    *reinterpret_cast<h4_t *>(a.out + (size_t)head * a.out_stride_h + (size_t)q_row * a.out_stride_m + c4 * 4) = h;
 }
 
 }  // namespace
@@ -373,13 +444,46 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
         return fa_fail(FA_ERR_INVALID_SHAPE, "prefill: one KV head of the contiguous cache must stay below 4 GiB");
     a.scale_log2e = L.scale * 1.4426950408889634f;
     if (L.q_len == 0) return FA_OK;
-    dim3 grid(ceil_div_u32(L.q_len, BM) * L.n_heads, 1, 1);
-    FaLaunchScope scope(ctx, "flash_prefill_mfma_kernel", true);
-    if (L.head_dim == 128)
-        scope.launch(flash_prefill_mfma_kernel<128>, grid, dim3(512), 0, a);
-    else if (L.head_dim == 64)
-        scope.launch(flash_prefill_mfma_kernel<64>, grid, dim3(512), 0, a);
-    else
+    if (L.head_dim != 128 && L.head_dim != 64)
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill only supports head_dim=64 or 128, got %u", L.head_dim);
-    return scope.finish();
+    // Split-K (src/metals/flashattention/step.rs:849-864): few query tiles against a long context (a prefill chunk
+    // after a long prefix) would leave most CUs idle, so the key tiles of each query tile are divided over several
+    // workgroups, at least 4 tiles each, up to one workgroup per CU.
+    const uint32_t base_wgs = ceil_div_u32(L.q_len, BM) * L.n_heads;
+    const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
+    const uint32_t key_tiles = ceil_div_u32(L.kv_len, BN);
+    uint32_t splits = ctx->prefill_split_k;
+    if (splits == 0) {
+        splits = 1;
+        if (base_wgs * 2 <= n_cus) splits = n_cus / base_wgs;  // all workgroups resident at once, one per CU
+        if (splits > key_tiles / 4) splits = key_tiles / 4;
+    }
+    if (splits > key_tiles) splits = key_tiles;
+    if (splits < 1) splits = 1;
+    a.splits = splits, a.part_acc = nullptr, a.part_ml = nullptr;
+    if (splits > 1) {
+        const size_t rows = (size_t)base_wgs * splits * BM;
+        const size_t acc_bytes = rows * L.head_dim * sizeof(float);
+        FA_TRY(fa_ensure_workspace(ctx, acc_bytes + rows * 2 * sizeof(float)));
+        a.part_acc = (float *)ctx->workspace;
+        a.part_ml = (float *)((char *)ctx->workspace + acc_bytes);
+    }
+    dim3 grid(base_wgs * splits, 1, 1);
+    {
+        FaLaunchScope scope(ctx, "flash_prefill_mfma_kernel", true);
+        if (L.head_dim == 128)
+            scope.launch(flash_prefill_mfma_kernel<128>, grid, dim3(512), 0, a);
+        else
+            scope.launch(flash_prefill_mfma_kernel<64>, grid, dim3(512), 0, a);
+        FA_TRY(scope.finish());
+    }
+    if (splits > 1) {
+        FaLaunchScope scope(ctx, "flash_prefill_merge_kernel", true);
+        if (L.head_dim == 128)
+            scope.launch(flash_prefill_merge_kernel<128>, dim3(base_wgs * (BM / 8)), dim3(256), 0, a);
+        else
+            scope.launch(flash_prefill_merge_kernel<64>, dim3(base_wgs * (BM / 16)), dim3(256), 0, a);
+        FA_TRY(scope.finish());
+    }
+    return FA_OK;
 }

@@ -97,6 +97,7 @@ PROTOTYPES = {
     "fa_decode_step_fused_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _PT, _PT, _PT,
                                    C.POINTER(KvPrepFusedParams), _u32],
     "fa_set_decode_variant": [_vp, C.POINTER(DecodeVariant)],
+    "fa_set_prefill_split_k": [_vp, C.c_uint32],
     "fa_kv_prep_fused_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _u32, _PT, _PT,
                                C.POINTER(KvPrepFusedParams)],
     "fa_kv_prep_decode_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _PT, _PT, C.POINTER(KvPrepFusedParams)],
@@ -241,6 +242,9 @@ class Foundry:
     def set_decode_variant(self, keys_per_split=0, merge=0):
         v = DecodeVariant(keys_per_split, merge)
         check(self.lib.fa_set_decode_variant(self.h, C.byref(v)))
+
+    def set_prefill_split_k(self, split_k=0):
+        check(self.lib.fa_set_prefill_split_k(self.h, split_k))
 
     def profile_enable(self, on=True):
         check(self.lib.fa_profile_enable(self.h, int(on)))

@@ -170,3 +170,62 @@ def test_prefill_errors():
         f.flash_attention(dq.arg(), dk.arg(), dv.arg(), do.arg(), True, 0, H, D, cap + 1, M)
     assert e.value.variant == "InvalidShape"
     f.synchronize()
+
+
+@pytest.mark.parametrize("split_k", [0, 1, 2, 3, 4, 8])
+def test_prefill_split_k_independent_of_split_count(split_k):
+    """A prefill chunk after a long prefix, key tiles divided over split_k workgroups + merge kernel
+    (flash_prefill.metal:452-457, 843-888): same result for every split count, including splits that get no tile."""
+    announce("prefill split-k", split_k)
+    f = ctx()
+    rng = np.random.default_rng(11)
+    H, Hkv, D, M, prefix = 6, 2, 128, 37, 700
+    N, cap = M + prefix, 800
+    q = h16(rng.normal(size=(H, M, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    k[:, N:], v[:, N:] = np.float16(np.nan), np.float16(np.nan)
+    want = orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, prefix, cap, causal=True, out_layout="head_major", n_threads=8)
+    f.set_prefill_split_k(split_k)
+    try:
+        got = gpu_prefill(q, k, v, H, D, M, N, prefix)
+    finally:
+        f.set_prefill_split_k(0)
+    assert np.all(np.isfinite(got))
+    assert max_abs(got, want) <= TOL
+
+
+def test_prefill_split_k_more_splits_than_tiles_and_d64():
+    announce("prefill split-k edge")
+    f = ctx()
+    rng = np.random.default_rng(12)
+    H, Hkv, D, M, prefix = 14, 2, 64, 130, 61   # 2 query tiles; the first sees only 3 key tiles
+    N, cap = M + prefix, 256
+    q = h16(rng.normal(size=(H, M, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    want = orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, prefix, cap, causal=True, out_layout="head_major", n_threads=8)
+    for split_k in (3, 64):
+        f.set_prefill_split_k(split_k)
+        try:
+            got = gpu_prefill(q, k, v, H, D, M, N, prefix)
+        finally:
+            f.set_prefill_split_k(0)
+        assert max_abs(got, want) <= TOL, split_k
+    with pytest.raises(fa.FoundryError) as e:
+        f.set_prefill_split_k(65)
+    assert e.value.variant == "OperationNotSupported"
+
+
+def test_prefill_chunk_after_long_prefix_auto_split():
+    """The reference's default prefill chunk (32 rows) against an 8K prefix: the automatic split-K path."""
+    announce("prefill chunk 32 @ 8k")
+    rng = np.random.default_rng(13)
+    H, Hkv, D, M, prefix = 24, 8, 128, 32, 8160
+    N, cap = M + prefix, 8192
+    q = h16(rng.normal(size=(H, M, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    want = orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, prefix, cap, causal=True, out_layout="head_major", n_threads=8)
+    got = gpu_prefill(q, k, v, H, D, M, N, prefix)
+    assert max_abs(got, want) <= TOL
