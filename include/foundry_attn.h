@@ -21,6 +21,12 @@
  *    (src/metals/flashattention/step.rs:927-929).
  *  - Tensors are f16 (IEEE binary16) unless stated; strides are in elements, offsets in bytes, exactly
  *    as in TensorArg (src/types/mod.rs:339-347).
+ *  - bfloat16 (an extension; the reference path is f16 only): the data tensors of fa_kv_prep_fused*,
+ *    fa_flash_attention, fa_flash_decode*, fa_decode_step_fused*, fa_flash_prefill* (q, k, v, q_rot, caches,
+ *    output) may all be FA_DTYPE_BF16 instead. The type of `q` selects the kernels, every other data tensor
+ *    must have the same type (UNSUPPORTED_DTYPE otherwise) and the pools of a paged cache are taken to hold
+ *    that type. RoPE tables stay f16; arithmetic stays f32 with one round-to-nearest-even at each store.
+ *    The int8 Q/K variant is f16 only.
  */
 #ifndef FOUNDRY_ATTN_H
 #define FOUNDRY_ATTN_H

@@ -78,6 +78,37 @@ orc_f16 orc_f32_to_f16(float f) {
     return (orc_f16)(sign | r);
 }
 
+/* ------------------------------------------------------------------ bf16 <-> f32 and the element-type switch */
+
+float orc_bf16_to_f32(uint16_t h) {
+    uint32_t bits = (uint32_t)h << 16;
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+/* round-to-nearest-even on the upper 16 bits; NaNs stay NaNs (quiet bit set) */
+uint16_t orc_f32_to_bf16(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x0040u);
+    uint32_t lsb = (x >> 16) & 1u;
+    x += 0x7fffu + lsb;
+    return (uint16_t)(x >> 16);
+}
+
+/* Element type of the DATA tensors (q, k, v, caches, outputs): 0 = f16 (the reference's only type), 1 = bf16
+ * (an extension of this build). RoPE tables and the int8 variant's scales are f16 in both modes. */
+static int g_elem_bf16 = 0;
+static int g_lut_ready = 0;
+void orc_set_elem_type(int bf16) {
+    g_elem_bf16 = bf16 ? 1 : 0;
+    g_lut_ready = 0;
+}
+int orc_get_elem_type(void) { return g_elem_bf16; }
+static inline float elem_to_f32(orc_f16 h) { return g_elem_bf16 ? orc_bf16_to_f32(h) : orc_f16_to_f32(h); }
+static inline orc_f16 f32_to_elem(float f) { return g_elem_bf16 ? orc_f32_to_bf16(f) : orc_f32_to_f16(f); }
+
 void orc_f16_to_f32_n(const orc_f16 *src, float *dst, size_t n) {
     for (size_t i = 0; i < n; ++i) dst[i] = orc_f16_to_f32(src[i]);
 }
@@ -241,7 +272,7 @@ void orc_kv_prep_fused(const orc_f16 *q_in, const orc_f16 *k_in, const orc_f16 *
         size_t q_src = (size_t)s * p->d_model + ((size_t)h * head_dim + hd);
         size_t pos = (size_t)p->position_offset + s;
 
-        float q_out = orc_f16_to_f32(q_in[q_src]);
+        float q_out = elem_to_f32(q_in[q_src]);
         int first = 1;
         uint32_t mate = hd;
         float cosv = 1.0f, sinv = 0.0f;
@@ -251,25 +282,25 @@ void orc_kv_prep_fused(const orc_f16 *q_in, const orc_f16 *k_in, const orc_f16 *
             sinv = orc_f16_to_f32(sin_t[pos * half_dim + pair]);
             first = rope_norm ? ((hd & 1u) == 0u) : (hd < half_dim);
             mate = rope_norm ? (first ? hd + 1 : hd - 1) : (first ? hd + half_dim : hd - half_dim);
-            float x_self = orc_f16_to_f32(q_in[q_src]);
-            float x_mate = orc_f16_to_f32(q_in[(size_t)s * p->d_model + ((size_t)h * head_dim + mate)]);
+            float x_self = elem_to_f32(q_in[q_src]);
+            float x_mate = elem_to_f32(q_in[(size_t)s * p->d_model + ((size_t)h * head_dim + mate)]);
             float a = x_self * cosv, b = x_mate * sinv;
             q_out = first ? (a - b) : (a + b);
         }
-        q_rot[gid] = orc_f32_to_f16(q_out);
+        q_rot[gid] = f32_to_elem(q_out);
 
         if ((h % p->group_size) != 0) continue;
         uint32_t kv_h = h / p->group_size;
         size_t kv_src = (size_t)s * p->kv_dim + ((size_t)kv_h * head_dim + hd);
         size_t cache_idx = (size_t)kv_h * p->max_seq_len * head_dim + pos * head_dim + hd;
-        float k_out = orc_f16_to_f32(k_in[kv_src]);
+        float k_out = elem_to_f32(k_in[kv_src]);
         if (apply_rope) {
-            float x_self = orc_f16_to_f32(k_in[kv_src]);
-            float x_mate = orc_f16_to_f32(k_in[(size_t)s * p->kv_dim + ((size_t)kv_h * head_dim + mate)]);
+            float x_self = elem_to_f32(k_in[kv_src]);
+            float x_mate = elem_to_f32(k_in[(size_t)s * p->kv_dim + ((size_t)kv_h * head_dim + mate)]);
             float a = x_self * cosv, b = x_mate * sinv;
             k_out = first ? (a - b) : (a + b);
         }
-        k_cache[cache_idx] = orc_f32_to_f16(k_out);
+        k_cache[cache_idx] = f32_to_elem(k_out);
         v_cache[cache_idx] = v_in[kv_src];
     }
 }
@@ -280,13 +311,12 @@ static inline float finite_or(float x, float alt) { return isfinite(x) ? x : alt
 
 /* f16 -> f32 table for the inner loops (same values as orc_f16_to_f32). */
 static float g_lut[65536];
-static int g_lut_ready = 0;
 static void lut_init(void) {
     if (g_lut_ready) return;
 #pragma omp critical(orc_lut)
     {
         if (!g_lut_ready) {
-            for (uint32_t i = 0; i < 65536u; ++i) g_lut[i] = orc_f16_to_f32((orc_f16)i);
+            for (uint32_t i = 0; i < 65536u; ++i) g_lut[i] = elem_to_f32((orc_f16)i);
             g_lut_ready = 1;
         }
     }
@@ -350,7 +380,7 @@ static void decode_one_head(const orc_f16 *qh, const orc_f16 *kh, const orc_f16 
         for (uint32_t d = 0; d < D; ++d) acc[d] = acc[d] * alpha + block_out[d] * beta;
     }
     float inv = (isfinite(l) && fabsf(l) > 1e-6f) ? (1.0f / l) : 1.0f;
-    for (uint32_t d = 0; d < D; ++d) outh[d] = orc_f32_to_f16(finite_or(acc[d] * inv, 0.0f));
+    for (uint32_t d = 0; d < D; ++d) outh[d] = f32_to_elem(finite_or(acc[d] * inv, 0.0f));
 }
 
 void orc_sdpa_decode(const orc_f16 *q, const orc_f16 *k, const orc_f16 *v, orc_f16 *out, uint32_t n_heads,
@@ -446,7 +476,7 @@ void orc_sdpa_prefill(const orc_f16 *q, const orc_f16 *k, const orc_f16 *v, orc_
             /* flash_prefill.metal:255-261: inv_l = 0 when l is unusable */
             float inv_l = (isfinite(l) && fabsf(l) > 1e-6f) ? (1.0f / l) : 0.0f;
             orc_f16 *o = out + (size_t)h * out_stride_h + (size_t)r * out_stride_m;
-            for (uint32_t d = 0; d < head_dim; ++d) o[d] = orc_f32_to_f16(acc[d] * inv_l);
+            for (uint32_t d = 0; d < head_dim; ++d) o[d] = f32_to_elem(acc[d] * inv_l);
         }
         free(tmp);
     }
@@ -495,7 +525,7 @@ void orc_splitk_merge(const float *acc, const float *m, const float *l, uint32_t
     for (uint32_t d = 0; d < head_dim; ++d) {
         float sum = 0.0f;
         for (uint32_t s = 0; s < split_k; ++s) sum += acc[(size_t)s * head_dim + d] * expf(m[s] - m_max);
-        out_row[d] = orc_f32_to_f16(sum * inv_l);
+        out_row[d] = f32_to_elem(sum * inv_l);
     }
 }
 

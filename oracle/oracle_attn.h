@@ -51,6 +51,15 @@ typedef struct {
         max_seq_len, total_elements, rope_mode /*0 neox, 1 normal*/, layer_idx, no_rope_layer_step;
 } orc_kv_prep_params;
 
+/* Element type of the data tensors: 0 = f16 (default, the reference's only type), 1 = bf16 (extension; no
+ * reference counterpart, PARITY UNPINNED - conversions pinned against an independent bf16 implementation).
+ * Affects orc_kv_prep_fused, orc_sdpa_decode, orc_sdpa_prefill, orc_sdpa_row_partials and orc_splitk_merge;
+ * RoPE tables stay f16. Not thread-safe: set it before calling, restore 0 afterwards. */
+void orc_set_elem_type(int bf16);
+int orc_get_elem_type(void);
+float orc_bf16_to_f32(uint16_t h);
+uint16_t orc_f32_to_bf16(float f);
+
 float orc_f16_to_f32(orc_f16 h);
 orc_f16 orc_f32_to_f16(float f);
 void orc_f16_to_f32_n(const orc_f16 *src, float *dst, size_t n);

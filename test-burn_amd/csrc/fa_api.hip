@@ -438,6 +438,11 @@ static fa_status check_tensor(const fa_tensor_arg *t, const char *name, fa_dtype
     return FA_OK;
 }
 
+// Element type of the data tensors of a call: bf16 when q is bf16, else f16 (so that any other type fails q's own
+// check). All data tensors of a call share it; RoPE tables are always f16; paged pools hold the same type as q.
+#define FA_DT(q) (((q) && (q)->dtype == (uint32_t)FA_DTYPE_BF16) ? FA_DTYPE_BF16 : FA_DTYPE_F16)
+#define FA_IS_BF16(q) ((q)->dtype == (uint32_t)FA_DTYPE_BF16)
+
 template <typename T>
 static T *tptr(const fa_tensor_arg *t) {
     return reinterpret_cast<T *>((char *)t->buffer + t->offset);
@@ -471,10 +476,10 @@ static fa_status kv_prep_common(fa_ctx *ctx, const fa_tensor_arg *q, const fa_te
     FA_TRY(check_kv_prep_params(p));
     const int al = p->head_dim % 16 == 0 ? 16 : 2;
     const size_t nq = (size_t)p->seq_len * p->d_model, nkv = (size_t)p->seq_len * p->kv_dim;
-    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, nq, al));
-    FA_TRY(check_tensor(k, "k", FA_DTYPE_F16, nkv, al));
-    FA_TRY(check_tensor(v, "v", FA_DTYPE_F16, nkv, al));
-    FA_TRY(check_tensor(q_rot, "q_rot", FA_DTYPE_F16, nq, al));
+    FA_TRY(check_tensor(q, "q", FA_DT(q), nq, al));
+    FA_TRY(check_tensor(k, "k", FA_DT(q), nkv, al));
+    FA_TRY(check_tensor(v, "v", FA_DT(q), nkv, al));
+    FA_TRY(check_tensor(q_rot, "q_rot", FA_DT(q), nq, al));
     FA_TRY(check_tensor(cos, "cos", FA_DTYPE_F16, 0, al));
     FA_TRY(check_tensor(sin, "sin", FA_DTYPE_F16, 0, al));
     const uint32_t half = p->head_dim / 2;
@@ -490,6 +495,7 @@ static fa_status kv_prep_common(fa_ctx *ctx, const fa_tensor_arg *q, const fa_te
     L.d_position = nullptr, L.block_table = nullptr, L.seq_lens = nullptr;
     L.bt_stride = 0, L.block_size = 1;
     L.table_rows = (uint32_t)(rows > 0xffffffffu ? 0xffffffffu : rows);
+    L.bf16 = FA_IS_BF16(q);
     return FA_OK;
 }
 
@@ -501,8 +507,8 @@ static fa_status kv_prep_contig(fa_ctx *ctx, const fa_tensor_arg *q, const fa_te
     FA_TRY(kv_prep_common(ctx, q, k, v, q_rot, cos, sin, p, L));
     const int al = p->head_dim % 16 == 0 ? 16 : 2;
     const size_t ncache = (size_t)p->n_kv_heads * p->max_seq_len * p->head_dim;
-    FA_TRY(check_tensor(k_cache, "k_cache", FA_DTYPE_F16, ncache, al));
-    FA_TRY(check_tensor(v_cache, "v_cache", FA_DTYPE_F16, ncache, al));
+    FA_TRY(check_tensor(k_cache, "k_cache", FA_DT(q), ncache, al));
+    FA_TRY(check_tensor(v_cache, "v_cache", FA_DT(q), ncache, al));
     if (!d_pos) {
         if ((uint64_t)p->position_offset + p->seq_len > p->max_seq_len)
             return fa_fail(FA_ERR_INVALID_OPERATION, "Invalid operation: position_offset %u + seq_len %u exceeds max_seq_len %u",
@@ -710,10 +716,10 @@ static fa_status decode_common(fa_ctx *ctx, const fa_tensor_arg *q, const fa_ten
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Flash Decode only supports head_dim=64 or 128, got %u", head_dim);
     if (n_heads == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_heads is 0");
     const size_t dm = (size_t)n_heads * head_dim;
-    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, dm, 16));
-    FA_TRY(check_tensor(k, "k", FA_DTYPE_F16, 0, 16));
-    FA_TRY(check_tensor(v, "v", FA_DTYPE_F16, 0, 16));
-    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, dm, 2));
+    FA_TRY(check_tensor(q, "q", FA_DT(q), dm, 16));
+    FA_TRY(check_tensor(k, "k", FA_DT(q), 0, 16));
+    FA_TRY(check_tensor(v, "v", FA_DT(q), 0, 16));
+    FA_TRY(check_tensor(output, "output", FA_DT(q), dm, 2));
     KvLayout kl, vl;
     FA_TRY(kv_layout(k, "k", head_dim, kl));
     FA_TRY(kv_layout(v, "v", head_dim, vl));
@@ -732,6 +738,7 @@ static fa_status decode_common(fa_ctx *ctx, const fa_tensor_arg *q, const fa_ten
     L.capacity = kl.capacity;
     L.scale = 1.0f / sqrtf((float)head_dim);  // step.rs:1042
     L.paged = false;
+    L.bf16 = FA_IS_BF16(q);
     return FA_OK;
 }
 
@@ -758,10 +765,10 @@ extern "C" fa_status fa_flash_attention(fa_ctx *ctx, const fa_tensor_arg *q, con
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill only supports head_dim=64 or 128, got %u", head_dim);
     if (n_heads == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_heads is 0");
     const size_t need = (size_t)m * n_heads * head_dim;
-    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, need, 16));
-    FA_TRY(check_tensor(k, "k", FA_DTYPE_F16, 0, 16));
-    FA_TRY(check_tensor(v, "v", FA_DTYPE_F16, 0, 16));
-    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, need, 8));
+    FA_TRY(check_tensor(q, "q", FA_DT(q), need, 16));
+    FA_TRY(check_tensor(k, "k", FA_DT(q), 0, 16));
+    FA_TRY(check_tensor(v, "v", FA_DT(q), 0, 16));
+    FA_TRY(check_tensor(output, "output", FA_DT(q), need, 8));
     KvLayout kl, vl;
     FA_TRY(kv_layout(k, "k", head_dim, kl));
     FA_TRY(kv_layout(v, "v", head_dim, vl));
@@ -783,6 +790,7 @@ extern "C" fa_status fa_flash_attention(fa_ctx *ctx, const fa_tensor_arg *q, con
     P.q_len = m, P.kv_len = kv_seq_len, P.query_offset = query_offset, P.causal = causal;
     P.scale = 1.0f / sqrtf((float)head_dim);
     P.paged = false, P.n_kv_heads = kl.n_kv_heads;
+    P.bf16 = FA_IS_BF16(q);
     return fa_launch_prefill(ctx, P);
 }
 
@@ -808,13 +816,13 @@ static fa_status fused_common(const fa_tensor_arg *q, const fa_tensor_arg *k, co
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Flash Decode only supports head_dim=64 or 128, got %u", p->head_dim);
     if (p->seq_len != n_tokens)
         return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: the fused decode step takes %u token(s), seq_len is %u", n_tokens, p->seq_len);
-    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, (size_t)n_tokens * p->d_model, 16));
-    FA_TRY(check_tensor(k, "k", FA_DTYPE_F16, (size_t)n_tokens * p->kv_dim, 16));
-    FA_TRY(check_tensor(v, "v", FA_DTYPE_F16, (size_t)n_tokens * p->kv_dim, 16));
+    FA_TRY(check_tensor(q, "q", FA_DT(q), (size_t)n_tokens * p->d_model, 16));
+    FA_TRY(check_tensor(k, "k", FA_DT(q), (size_t)n_tokens * p->kv_dim, 16));
+    FA_TRY(check_tensor(v, "v", FA_DT(q), (size_t)n_tokens * p->kv_dim, 16));
     FA_TRY(check_tensor(cos, "cos", FA_DTYPE_F16, 0, 16));
     FA_TRY(check_tensor(sin, "sin", FA_DTYPE_F16, 0, 16));
     if (!q_rot) return fa_fail(FA_ERR_NULL_POINTER, "tensor argument 'q_rot' is null");
-    if (q_rot->buffer) FA_TRY(check_tensor(q_rot, "q_rot", FA_DTYPE_F16, (size_t)n_tokens * p->d_model, 16));
+    if (q_rot->buffer) FA_TRY(check_tensor(q_rot, "q_rot", FA_DT(q), (size_t)n_tokens * p->d_model, 16));
     const uint32_t half = p->head_dim / 2;
     size_t rows = numel(cos) / half;
     if (numel(sin) / half < rows) rows = numel(sin) / half;
@@ -833,6 +841,7 @@ static fa_status fused_common(const fa_tensor_arg *q, const fa_tensor_arg *k, co
     L.q_stride_b = p->d_model, L.q_stride_h = p->head_dim;
     L.out_stride_b = p->d_model, L.out_stride_h = p->head_dim;
     L.scale = 1.0f / sqrtf((float)p->head_dim);
+    L.bf16 = FA_IS_BF16(q);
     return FA_OK;
 }
 
@@ -847,9 +856,9 @@ extern "C" fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, c
     memset(&L, 0, sizeof(L));
     FA_NEED(p, "params");
     FA_TRY(fused_common(q, k, v, q_rot, cos, sin, p, 1, L));
-    FA_TRY(check_tensor(k_cache, "k_cache", FA_DTYPE_F16, 0, 16));
-    FA_TRY(check_tensor(v_cache, "v_cache", FA_DTYPE_F16, 0, 16));
-    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, p->d_model, 2));
+    FA_TRY(check_tensor(k_cache, "k_cache", FA_DT(q), 0, 16));
+    FA_TRY(check_tensor(v_cache, "v_cache", FA_DT(q), 0, 16));
+    FA_TRY(check_tensor(output, "output", FA_DT(q), p->d_model, 2));
     KvLayout kl, vl;
     FA_TRY(kv_layout(k_cache, "k_cache", p->head_dim, kl));
     FA_TRY(kv_layout(v_cache, "v_cache", p->head_dim, vl));
@@ -891,7 +900,7 @@ extern "C" fa_status fa_decode_step_fused_paged(fa_ctx *ctx, const fa_tensor_arg
     if (p->head_dim != cache->head_dim || p->n_kv_heads != cache->n_kv_heads)
         return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: params (Hkv %u, D %u) do not match the paged cache (Hkv %u, D %u)",
                        p->n_kv_heads, p->head_dim, cache->n_kv_heads, cache->head_dim);
-    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, (size_t)cache->n_seqs * p->d_model, 2));
+    FA_TRY(check_tensor(output, "output", FA_DT(q), (size_t)cache->n_seqs * p->d_model, 2));
     if (kv_len_bound == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_len_bound is 0");
     L.k = cache->k_pool, L.v = (const __half *)cache->v_pool, L.out = tptr<__half>(output);
     L.batch = cache->n_seqs;
@@ -912,8 +921,8 @@ extern "C" fa_status fa_flash_decode_paged(fa_ctx *ctx, const fa_tensor_arg *q, 
     if (n_heads == 0 || n_heads % cache->n_kv_heads != 0)
         return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_heads %u not a multiple of n_kv_heads %u", n_heads, cache->n_kv_heads);
     const size_t need = (size_t)cache->n_seqs * n_heads * cache->head_dim;
-    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, need, 16));
-    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, need, 2));
+    FA_TRY(check_tensor(q, "q", FA_DT(q), need, 16));
+    FA_TRY(check_tensor(output, "output", FA_DT(q), need, 2));
     if (kv_len_bound == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_len_bound is 0");
     DecodeLaunch L;
     memset(&L, 0, sizeof(L));
@@ -925,6 +934,7 @@ extern "C" fa_status fa_flash_decode_paged(fa_ctx *ctx, const fa_tensor_arg *q, 
     L.capacity = cache->max_blocks_per_seq * cache->block_size;
     L.kv_len_bound = kv_len_bound < L.capacity ? kv_len_bound : L.capacity;
     L.scale = 1.0f / sqrtf((float)cache->head_dim);
+    L.bf16 = FA_IS_BF16(q);
     L.paged = true, L.block_table = cache->block_table, L.bt_stride = cache->max_blocks_per_seq;
     L.block_size = cache->block_size;
     return fa_launch_decode(ctx, L);
@@ -944,8 +954,8 @@ extern "C" fa_status fa_flash_prefill_paged(fa_ctx *ctx, const fa_tensor_arg *q,
         return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_seq_len %u outside (0, capacity %llu]", kv_seq_len, (unsigned long long)cap);
     const uint32_t D = cache->head_dim;
     const size_t need = (size_t)m * n_heads * D;
-    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, need, 16));
-    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, need, 8));
+    FA_TRY(check_tensor(q, "q", FA_DT(q), need, 16));
+    FA_TRY(check_tensor(output, "output", FA_DT(q), need, 8));
     PrefillLaunch P;
     memset(&P, 0, sizeof(P));
     P.q = tptr<const __half>(q), P.k = (const __half *)cache->k_pool, P.v = (const __half *)cache->v_pool;
@@ -955,6 +965,7 @@ extern "C" fa_status fa_flash_prefill_paged(fa_ctx *ctx, const fa_tensor_arg *q,
     P.n_heads = n_heads, P.group_size = n_heads / cache->n_kv_heads, P.head_dim = D;
     P.q_len = m, P.kv_len = kv_seq_len, P.query_offset = query_offset, P.causal = causal;
     P.scale = 1.0f / sqrtf((float)D);
+    P.bf16 = FA_IS_BF16(q);
     P.paged = true, P.block_table = cache->block_table + (size_t)seq_index * cache->max_blocks_per_seq;
     P.block_size = cache->block_size, P.n_kv_heads = cache->n_kv_heads;
     return fa_launch_prefill(ctx, P);

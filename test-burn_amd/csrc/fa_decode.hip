@@ -53,6 +53,7 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     a.kv_len = L.kv_len, a.d_len_stride = L.d_len_stride, a.kv_len_add = L.kv_len_add, a.kv_len_bound = bound;
     a.capacity = L.capacity, a.chunk = chunk, a.n_kv_heads = L.n_kv_heads, a.sub_per_kv = sub_per_kv;
     a.gt = (uint32_t)gt;
+    a.bf16 = L.bf16 ? 1u : 0u;
     a.bt_stride = L.bt_stride, a.block_size = L.block_size;
     a.block_shift = (L.block_size && (L.block_size & (L.block_size - 1)) == 0) ? (uint32_t)__builtin_ctz(L.block_size) : 32u;
     a.merge_in_kernel = ctx->decode_variant.merge == 0 ? 1u : 0u;

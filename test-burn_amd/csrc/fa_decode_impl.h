@@ -51,9 +51,13 @@ typedef unsigned int u2_t __attribute__((ext_vector_type(2)));
 typedef unsigned int u16_t __attribute__((ext_vector_type(16)));
 typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
 
+typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+typedef short s4_t __attribute__((ext_vector_type(4)));
+
 union U4H {
     uint4 u;
     h8_t h;
+    bf8_t b;
     i4_t i;
     _Float16 e[8];
 };
@@ -85,9 +89,28 @@ struct DecodeDev {
     __half *q_rot_out;  // nullable
     uint64_t qin_stride_b, kvin_stride_b, qrot_stride_b;
     uint32_t rope_normal, apply_rope, table_rows;
+    uint32_t bf16;  // data tensors are bf16 (RoPE tables stay f16)
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Element i of a 16-byte data chunk as f32 / an f32 rounded (to nearest even) to the storage type.
+__device__ __forceinline__ float elem_f32(const U4H &x, int i, bool bf16) {
+    if (!bf16) return (float)x.e[i];
+    return __uint_as_float((uint32_t)__builtin_bit_cast(unsigned short, x.e[i]) << 16);
+}
+__device__ __forceinline__ _Float16 f32_elem(float v, bool bf16) {
+    if (!bf16) return (_Float16)v;
+    return __builtin_bit_cast(_Float16, (__bf16)v);
+}
+__device__ __forceinline__ void store_out4(__half *op, const float (&o)[4], bool bf16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float v = isfinite(o[i]) ? o[i] : 0.0f;
+        op[i] = __builtin_bit_cast(__half, f32_elem(v, bf16));
+    }
+}
+
 
 // Value of lane (l ^ 16) / (l ^ 32): one VALU lane-swap each on gfx950.
 __device__ __forceinline__ float xor16(float x) {
@@ -191,12 +214,8 @@ __device__ __forceinline__ void merge_and_store(const DecodeDev &a, uint32_t b, 
             const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 1.0f;
             const uint32_t head = y * gt + h;
             __half *op = a.out + (size_t)b * a.out_stride_b + (size_t)head * a.out_stride_h + c * 4;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float v = o[i] * inv;
-                v = isfinite(v) ? v : 0.0f;
-                op[i] = __float2half_rn(v);
-            }
+            const float ov[4] = {o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
+            store_out4(op, ov, a.bf16 != 0);
         }
         __syncthreads();
     }
@@ -207,29 +226,29 @@ __device__ __forceinline__ void merge_and_store(const DecodeDev &a, uint32_t b, 
 //   normal: x = 8 consecutive dims (4 adjacent pairs), c/s = 4 values
 //   neox  : x = 8 dims, mate = the 8 dims D/2 away, c/s = 8 values, `first` = x is the low half of its pairs
 __device__ __forceinline__ U4H rope8(const U4H &x, const U4H &mate, const U4H &c, const U4H &s, bool normal,
-                                     bool first) {
+                                     bool first, bool bf16) {
 #pragma clang fp contract(off)
     U4H o;
     if (normal) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const float xe = (float)x.e[2 * i], xo = (float)x.e[2 * i + 1], cc = (float)c.e[i], ss = (float)s.e[i];
+            const float xe = elem_f32(x, 2 * i, bf16), xo = elem_f32(x, 2 * i + 1, bf16), cc = (float)c.e[i], ss = (float)s.e[i];
             const float a0 = xe * cc, b0 = xo * ss, a1 = xo * cc, b1 = xe * ss;
-            o.e[2 * i] = (_Float16)(a0 - b0);
-            o.e[2 * i + 1] = (_Float16)(a1 + b1);
+            o.e[2 * i] = f32_elem(a0 - b0, bf16);
+            o.e[2 * i + 1] = f32_elem(a1 + b1, bf16);
         }
     } else {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const float xs = (float)x.e[i], xm = (float)mate.e[i];
+            const float xs = elem_f32(x, i, bf16), xm = elem_f32(mate, i, bf16);
             const float p0 = xs * (float)c.e[i], p1 = xm * (float)s.e[i];
-            o.e[i] = (_Float16)(first ? p0 - p1 : p0 + p1);
+            o.e[i] = f32_elem(first ? p0 - p1 : p0 + p1, bf16);
         }
     }
     return o;
 }
 
-template <int D, bool PAGED, bool SAGE, bool FUSED>
+template <int D, bool PAGED, bool SAGE, bool FUSED, bool BF16 = false>
 __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
     constexpr int KSTEPS = SAGE ? D / 64 : D / 32;  // MFMA steps over head_dim for S^T; 16 B per lane each
     constexpr int SEGS = SAGE ? D / 16 : D / 8;     // 16-byte segments per K row
@@ -240,6 +259,7 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
     constexpr int VRS = D * 2 + 32;                 // LDS row stride of the V tile (bank spread for the transpose loads)
     constexpr int KES = SAGE ? 1 : 2;               // K element size in bytes
     static_assert(!(SAGE && FUSED), "the fused append is f16 only");
+    static_assert(!(SAGE && BF16), "the int8 variant keeps V in f16");
     static_assert(KSTEPS * 4 == SEGS, "a K row is KSTEPS x 4 segments");
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -384,7 +404,7 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
                 const uint2 s4 = *reinterpret_cast<const uint2 *>(sp + seg * 8);
                 U4H cu, su;
                 cu.u = make_uint4(c4.x, c4.y, 0, 0), su.u = make_uint4(s4.x, s4.y, 0, 0);
-                o[j] = rope8(x[j], x[j], cu, su, true, true);
+                o[j] = rope8(x[j], x[j], cu, su, true, true, BF16);
             }
         } else {
 #pragma unroll
@@ -393,8 +413,8 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
                 U4H cu, su;
                 cu.u = *reinterpret_cast<const uint4 *>(cp + seg * 16);
                 su.u = *reinterpret_cast<const uint4 *>(sp + seg * 16);
-                o[j] = rope8(x[j], x[j + KSTEPS / 2], cu, su, false, true);
-                o[j + KSTEPS / 2] = rope8(x[j + KSTEPS / 2], x[j], cu, su, false, false);
+                o[j] = rope8(x[j], x[j + KSTEPS / 2], cu, su, false, true, BF16);
+                o[j + KSTEPS / 2] = rope8(x[j + KSTEPS / 2], x[j], cu, su, false, false, BF16);
             }
         }
     };
@@ -548,7 +568,8 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
                     f4_t sf = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                     for (int j = 0; j < KSTEPS; ++j)
-                        sf = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk[mb][j].h, q_op(j).h, sf, 0, 0, 0);
+                        sf = BF16 ? __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk[mb][j].b, q_op(j).b, sf, 0, 0, 0)
+                                  : __builtin_amdgcn_mfma_f32_16x16x32_f16(kk[mb][j].h, q_op(j).h, sf, 0, 0, 0);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) s[mb * 4 + i] = sf[i] * qsc;
                 }
@@ -584,7 +605,7 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
         for (int i = 0; i < 4 * MBX; ++i) {
             const float pw = fast_exp2(s[i] - mn);
             ps += pw;
-            pb[i >> 2][i & 3] = (_Float16)pw;
+            pb[i >> 2][i & 3] = f32_elem(pw, BF16);
         }
         l_run = l_run * al + ps;
         m_run = mn;
@@ -617,7 +638,9 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
                 h4_t vh;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) vh[i] = (_Float16)v0[i];
-                oacc[blk] = __builtin_amdgcn_mfma_f32_16x16x16f16(vh, pb[mb], oacc[blk], 0, 0, 0);
+                oacc[blk] = BF16 ? __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s4_t, vh),
+                                                                              __builtin_bit_cast(s4_t, pb[mb]), oacc[blk], 0, 0, 0)
+                                 : __builtin_amdgcn_mfma_f32_16x16x16f16(vh, pb[mb], oacc[blk], 0, 0, 0);
             }
         }
         if (mnext) issue_v(nblk, mnext, k1 - 1);  // V registers are free again
@@ -690,12 +713,8 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
         if (nsplits == 1) {
             const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 1.0f;
             __half *op = a.out + (size_t)b * a.out_stride_b + (size_t)(head0 + h) * a.out_stride_h + c4 * 4;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                float o = A[i] * inv;
-                o = isfinite(o) ? o : 0.0f;
-                op[i] = __float2half_rn(o);
-            }
+            const float ov[4] = {A[0] * inv, A[1] * inv, A[2] * inv, A[3] * inv};
+            store_out4(op, ov, BF16);
         } else if (in_kernel) {
             float *pa = a.part_acc + gbase * D, *pm = a.part_ml + gbase * 2;
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, A), make_rsrc(pa),
@@ -768,6 +787,10 @@ fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, true, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
+            FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, false, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
+            FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, true, false, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
+            FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, false, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
+            FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, true, false, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
             lds_allowed = true;
         }
     }
@@ -778,19 +801,31 @@ fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
         FaLaunchScope scope(ctx, name, true);
         switch (mode) {
             case MODE_PLAIN:
-                scope.launch((flash_decode_mfma_kernel<D, false, false, false>), grid, dim3(NT), lds, a);
+                if (a.bf16)
+                    scope.launch((flash_decode_mfma_kernel<D, false, false, false, true>), grid, dim3(NT), lds, a);
+                else
+                    scope.launch((flash_decode_mfma_kernel<D, false, false, false>), grid, dim3(NT), lds, a);
                 break;
             case MODE_PAGED:
-                scope.launch((flash_decode_mfma_kernel<D, true, false, false>), grid, dim3(NT), lds, a);
+                if (a.bf16)
+                    scope.launch((flash_decode_mfma_kernel<D, true, false, false, true>), grid, dim3(NT), lds, a);
+                else
+                    scope.launch((flash_decode_mfma_kernel<D, true, false, false>), grid, dim3(NT), lds, a);
                 break;
             case MODE_SAGE:
                 scope.launch((flash_decode_mfma_kernel<D, false, true, false>), grid, dim3(NT), lds, a);
                 break;
             case MODE_FUSED:
-                scope.launch((flash_decode_mfma_kernel<D, false, false, true>), grid, dim3(NT), lds, a);
+                if (a.bf16)
+                    scope.launch((flash_decode_mfma_kernel<D, false, false, true, true>), grid, dim3(NT), lds, a);
+                else
+                    scope.launch((flash_decode_mfma_kernel<D, false, false, true>), grid, dim3(NT), lds, a);
                 break;
             default:
-                scope.launch((flash_decode_mfma_kernel<D, true, false, true>), grid, dim3(NT), lds, a);
+                if (a.bf16)
+                    scope.launch((flash_decode_mfma_kernel<D, true, false, true, true>), grid, dim3(NT), lds, a);
+                else
+                    scope.launch((flash_decode_mfma_kernel<D, true, false, true>), grid, dim3(NT), lds, a);
                 break;
         }
         FA_TRY(scope.finish());

@@ -100,6 +100,7 @@ struct KvPrepLaunch {
     uint32_t block_size;
     uint32_t capacity;           // rows addressable through the cache (contiguous: max_seq_len)
     uint32_t table_rows;         // rows available in cos/sin
+    bool bf16 = false;           // data tensors are bf16 instead of f16 (tables stay f16)
 };
 fa_status fa_launch_kv_prep(fa_ctx *ctx, const KvPrepLaunch &a);
 
@@ -131,6 +132,7 @@ struct DecodeLaunch {
     __half *q_rot_out;
     uint64_t qin_stride_b, kvin_stride_b, qrot_stride_b;
     uint32_t rope_normal, apply_rope, table_rows;
+    bool bf16;  // q, k, v, caches and out are bf16 instead of f16 (not with the int8 variant)
 };
 fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &a);
 
@@ -144,6 +146,7 @@ struct PrefillLaunch {
     bool paged;
     const int32_t *block_table;
     uint32_t block_size, n_kv_heads;
+    bool bf16;  // q, k, v and out are bf16 instead of f16
 };
 fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &a);
 

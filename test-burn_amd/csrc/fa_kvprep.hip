@@ -21,6 +21,28 @@ struct alignas(16) H8 {
 __device__ __forceinline__ H8 ld16(const __half *p) { return *reinterpret_cast<const H8 *>(p); }
 __device__ __forceinline__ void st16(__half *p, const H8 &x) { *reinterpret_cast<H8 *>(p) = x; }
 
+// Data tensors are f16 or bf16 (`bf16` is uniform over a launch); the RoPE tables are always f16. Conversions to
+// the storage type round to nearest even.
+__device__ __forceinline__ float2 elem2_to_f32(__half2 x, bool bf16) {
+    if (!bf16) return __half22float2(x);
+    const uint32_t u = __builtin_bit_cast(uint32_t, x);
+    return make_float2(__uint_as_float(u << 16), __uint_as_float(u & 0xffff0000u));
+}
+__device__ __forceinline__ __half2 f32_to_elem2(float lo, float hi, bool bf16) {
+    if (!bf16) return __halves2half2(__float2half_rn(lo), __float2half_rn(hi));
+    typedef __bf16 bf2_t __attribute__((ext_vector_type(2)));
+    bf2_t r = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(__half2, r);
+}
+__device__ __forceinline__ float elem_to_f32(__half x, bool bf16) {
+    if (!bf16) return __half2float(x);
+    return __uint_as_float((uint32_t)__builtin_bit_cast(unsigned short, x) << 16);
+}
+__device__ __forceinline__ __half f32_to_elem(float x, bool bf16) {
+    if (!bf16) return __float2half_rn(x);
+    return __builtin_bit_cast(__half, (__bf16)x);
+}
+
 // One rotation pair, products and sum rounded separately (matches the reference's op order).
 __device__ __forceinline__ void rot_pair(float xi, float xj, float c, float s, float &oi, float &oj) {
 #pragma clang fp contract(off)
@@ -36,16 +58,16 @@ __device__ __forceinline__ float rot_one(float x, float m, float c, float s, boo
     return first ? p0 - p1 : p0 + p1;
 }
 
-__device__ __forceinline__ void rope16(const H8 &a, const H8 &b, const H8 &c8, const H8 &s8, bool normal, H8 &oa,
-                                       H8 &ob) {
+__device__ __forceinline__ void rope16(const H8 &a, const H8 &b, const H8 &c8, const H8 &s8, bool normal, bool bf16,
+                                       H8 &oa, H8 &ob) {
     // a, b: the thread's two 16-byte input chunks; c8/s8: eight cos/sin values (pair order).
     float af[8], bf[8], cf[8], sf[8], ra[8], rb[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         float2 t;
-        t = __half22float2(a.v[i]);
+        t = elem2_to_f32(a.v[i], bf16);
         af[2 * i] = t.x, af[2 * i + 1] = t.y;
-        t = __half22float2(b.v[i]);
+        t = elem2_to_f32(b.v[i], bf16);
         bf[2 * i] = t.x, bf[2 * i + 1] = t.y;
         t = __half22float2(c8.v[i]);
         cf[2 * i] = t.x, cf[2 * i + 1] = t.y;
@@ -65,8 +87,8 @@ __device__ __forceinline__ void rope16(const H8 &a, const H8 &b, const H8 &c8, c
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        oa.v[i] = __halves2half2(__float2half_rn(ra[2 * i]), __float2half_rn(ra[2 * i + 1]));
-        ob.v[i] = __halves2half2(__float2half_rn(rb[2 * i]), __float2half_rn(rb[2 * i + 1]));
+        oa.v[i] = f32_to_elem2(ra[2 * i], ra[2 * i + 1], bf16);
+        ob.v[i] = f32_to_elem2(rb[2 * i], rb[2 * i + 1], bf16);
     }
 }
 
@@ -78,7 +100,7 @@ struct KvPrepDev {
     const int32_t *block_table;
     const uint32_t *seq_lens;
     uint32_t d_model, kv_dim, head_dim, n_heads, n_kv_heads, seq_len, position_offset, max_seq_len;
-    uint32_t rope_normal, apply_rope, mode, bt_stride, block_size, capacity, table_rows;
+    uint32_t rope_normal, apply_rope, mode, bt_stride, block_size, capacity, table_rows, bf16;
 };
 
 // Destination row base (element index) of cache row `pos` of kv head `kvh` for token `s`.
@@ -137,7 +159,7 @@ __global__ void __launch_bounds__(256) kv_prep_fused_vec_kernel(KvPrepDev a) {
     const uint32_t tp = pos < a.table_rows ? pos : a.table_rows - 1;  // stay inside the tables
     const H8 c8 = ld16(a.cos_t + (size_t)tp * half + c * 8), s8 = ld16(a.sin_t + (size_t)tp * half + c * 8);
     H8 oa, ob;
-    rope16(xa, xb, c8, s8, normal, oa, ob);
+    rope16(xa, xb, c8, s8, normal, a.bf16 != 0, oa, ob);
     st16(dst + offA, oa);
     st16(dst + offB, ob);
 }
@@ -163,23 +185,24 @@ __global__ void __launch_bounds__(256) kv_prep_fused_elem_kernel(KvPrepDev a) {
         sn = __half2float(a.sin_t[(size_t)tp * half + pair]);
     }
     const __half *qrow = a.q + (size_t)s * a.d_model + (size_t)h * D;
-    float xo = __half2float(qrow[hd]);
+    const bool bf16 = a.bf16 != 0;
+    float xo = elem_to_f32(qrow[hd], bf16);
     if (rope) {
-        xo = rot_one(xo, __half2float(qrow[mate]), c, sn, first);
+        xo = rot_one(xo, elem_to_f32(qrow[mate], bf16), c, sn, first);
     }
     __half *qdst = a.mode == 2 ? a.q_rot + ((size_t)s * a.n_heads + h) * D : a.q_rot + ((size_t)h * a.seq_len + s) * D;
-    qdst[hd] = __float2half_rn(xo);
+    qdst[hd] = f32_to_elem(xo, bf16);
 
     const uint32_t group = a.n_heads / a.n_kv_heads;
     if (h % group != 0 || pos >= a.capacity) return;
     const uint32_t kvh = h / group;
     const __half *krow = a.k + (size_t)s * a.kv_dim + (size_t)kvh * D;
-    float ko = __half2float(krow[hd]);
+    float ko = elem_to_f32(krow[hd], bf16);
     if (rope) {
-        ko = rot_one(ko, __half2float(krow[mate]), c, sn, first);
+        ko = rot_one(ko, elem_to_f32(krow[mate], bf16), c, sn, first);
     }
     const size_t row = cache_row(a, s, kvh, pos);
-    a.k_cache[row + hd] = __float2half_rn(ko);
+    a.k_cache[row + hd] = f32_to_elem(ko, bf16);
     a.v_cache[row + hd] = a.v[(size_t)s * a.kv_dim + (size_t)kvh * D + hd];
 }
 
@@ -220,7 +243,7 @@ fa_status fa_launch_kv_prep(fa_ctx *ctx, const KvPrepLaunch &L) {
     a.rope_normal = L.p.rope_mode == FA_ROPE_MODE_NORMAL;
     a.apply_rope = L.p.no_rope_layer_step == 0 || ((L.p.layer_idx + 1u) % L.p.no_rope_layer_step) != 0u;
     a.mode = (uint32_t)L.mode, a.bt_stride = L.bt_stride, a.block_size = L.block_size, a.capacity = L.capacity;
-    a.table_rows = L.table_rows;
+    a.table_rows = L.table_rows, a.bf16 = L.bf16 ? 1u : 0u;
     if (a.seq_len == 0) return FA_OK;
     if (a.head_dim % 16 == 0) {
         uint64_t total = (uint64_t)a.seq_len * (a.n_heads + 2 * a.n_kv_heads) * (a.head_dim / 16);

@@ -26,10 +26,20 @@ typedef float f16_t __attribute__((ext_vector_type(16)));
 typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
 typedef unsigned int u4_t __attribute__((ext_vector_type(4)));
 
+typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+
 union U4H8 {
     uint4 u;
     h8_t h;
+    bf8_t b;
 };
+
+// f32 rounded (to nearest even) to the storage type of the data tensors
+template <bool BF16>
+__device__ __forceinline__ _Float16 to_elem(float v) {
+    if (BF16) return __builtin_bit_cast(_Float16, (__bf16)v);
+    return (_Float16)v;
+}
 
 struct PrefillDev {
     const __half *q, *k, *v;
@@ -72,7 +82,7 @@ struct Chunk<64> {
     }
 };
 
-template <int D>
+template <int D, bool BF16>
 __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a) {
     constexpr int DSTEPS = D / 16;  // MFMA k-steps over head_dim for S^T
     constexpr int DBLKS = D / 32;   // 32-row blocks of O^T
@@ -246,7 +256,8 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
             for (int s = 0; s < DSTEPS; ++s) {
                 U4H8 kk;
                 kk.u = *reinterpret_cast<const uint4 *>(k_lds + (kb * 32 + n) * KRS + (s * 16 + hi * 8) * 2);
-                sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kk.h, qreg[s].h, sacc[kb], 0, 0, 0);
+                sacc[kb] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(kk.b, qreg[s].b, sacc[kb], 0, 0, 0)
+                                : __builtin_amdgcn_mfma_f32_32x32x16_f16(kk.h, qreg[s].h, sacc[kb], 0, 0, 0);
             }
         }
         // mask: accumulator i of block kb is key key0 + 32*kb + 8*(i/4) + 4*hi + i%4
@@ -297,7 +308,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
             for (int ks = 0; ks < 2; ++ks) {
                 h8_t pb;
 #pragma unroll
-                for (int j = 0; j < 8; ++j) pb[j] = (_Float16)sacc[kb][8 * ks + j];
+                for (int j = 0; j < 8; ++j) pb[j] = to_elem<BF16>(sacc[kb][8 * ks + j]);
                 // keys of this k-step for lane half hi: base + {0..3} and base + 8 + {0..3}, base = 32kb+16ks+4hi
                 const int kbase16 = kb * 32 + ks * 16 + hi * 4;
                 const int L = lane & 15, jr = L >> 2, cc = L & 3;  // source-lane role inside a 16-lane block
@@ -312,7 +323,9 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
                     } va;
                     va.f[0] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p0));
                     va.f[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p1));
-                    oacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va.h, pb, oacc[b], 0, 0, 0);
+                    oacc[b] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, va.h),
+                                                                           __builtin_bit_cast(bf8_t, pb), oacc[b], 0, 0, 0)
+                                   : __builtin_amdgcn_mfma_f32_32x32x16_f16(va.h, pb, oacc[b], 0, 0, 0);
                 }
             }
         if (tile + 2 < n_tiles) {
@@ -375,7 +388,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
                 // accumulators 4gi..4gi+3 are d = 32b + 8gi + 4hi + 0..3
                 h4_t o;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) o[j] = (_Float16)(oacc[b][gi * 4 + j] * inv_l);
+                for (int j = 0; j < 4; ++j) o[j] = to_elem<BF16>(oacc[b][gi * 4 + j] * inv_l);
                 *reinterpret_cast<h4_t *>(op + b * 32 + gi * 8 + hi * 4) = o;
             }
     }
@@ -383,7 +396,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
 
 // Merge of the per-split states (flash_prefill.metal:843-888): m* = max m_s, L = sum l_s 2^(m_s - m*) over the
 // splits with l_s > 0, out = sum acc_s 2^(m_s - m*) / L (0 when L is unusable). m is kept in the exp2 domain.
-template <int D>
+template <int D, bool BF16>
 __global__ void __launch_bounds__(256) flash_prefill_merge_kernel(PrefillDev a) {
     constexpr int CG = D / 4;           // float4 columns per row
     constexpr int ROWS = 256 / CG;      // rows per workgroup (8 at D = 128, 16 at D = 64)
@@ -423,7 +436,7 @@ __global__ void __launch_bounds__(256) flash_prefill_merge_kernel(PrefillDev a) 
     }
     const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 0.0f;
     h4_t h;
-    h[0] = (_Float16)(o.x * inv), h[1] = (_Float16)(o.y * inv), h[2] = (_Float16)(o.z * inv), h[3] = (_Float16)(o.w * inv);
+    h[0] = to_elem<BF16>(o.x * inv), h[1] = to_elem<BF16>(o.y * inv), h[2] = to_elem<BF16>(o.z * inv), h[3] = to_elem<BF16>(o.w * inv);
     *reinterpret_cast<h4_t *>(a.out + (size_t)head * a.out_stride_h + (size_t)q_row * a.out_stride_m + c4 * 4) = h;
 }
 
@@ -471,18 +484,26 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
     dim3 grid(base_wgs * splits, 1, 1);
     {
         FaLaunchScope scope(ctx, "flash_prefill_mfma_kernel", true);
-        if (L.head_dim == 128)
-            scope.launch(flash_prefill_mfma_kernel<128>, grid, dim3(512), 0, a);
+        if (L.head_dim == 128 && L.bf16)
+            scope.launch(flash_prefill_mfma_kernel<128, true>, grid, dim3(512), 0, a);
+        else if (L.head_dim == 128)
+            scope.launch(flash_prefill_mfma_kernel<128, false>, grid, dim3(512), 0, a);
+        else if (L.bf16)
+            scope.launch(flash_prefill_mfma_kernel<64, true>, grid, dim3(512), 0, a);
         else
-            scope.launch(flash_prefill_mfma_kernel<64>, grid, dim3(512), 0, a);
+            scope.launch(flash_prefill_mfma_kernel<64, false>, grid, dim3(512), 0, a);
         FA_TRY(scope.finish());
     }
     if (splits > 1) {
         FaLaunchScope scope(ctx, "flash_prefill_merge_kernel", true);
-        if (L.head_dim == 128)
-            scope.launch(flash_prefill_merge_kernel<128>, dim3(base_wgs * (BM / 8)), dim3(256), 0, a);
+        if (L.head_dim == 128 && L.bf16)
+            scope.launch(flash_prefill_merge_kernel<128, true>, dim3(base_wgs * (BM / 8)), dim3(256), 0, a);
+        else if (L.head_dim == 128)
+            scope.launch(flash_prefill_merge_kernel<128, false>, dim3(base_wgs * (BM / 8)), dim3(256), 0, a);
+        else if (L.bf16)
+            scope.launch(flash_prefill_merge_kernel<64, true>, dim3(base_wgs * (BM / 16)), dim3(256), 0, a);
         else
-            scope.launch(flash_prefill_merge_kernel<64>, dim3(base_wgs * (BM / 16)), dim3(256), 0, a);
+            scope.launch(flash_prefill_merge_kernel<64, false>, dim3(base_wgs * (BM / 16)), dim3(256), 0, a);
         FA_TRY(scope.finish());
     }
     return FA_OK;

@@ -43,6 +43,11 @@ def lib():
         L.orc_f32_to_f16.restype = C.c_uint16
         L.orc_f32_to_f16.argtypes = [C.c_float]
         L.orc_max_threads.restype = C.c_int
+        L.orc_bf16_to_f32.restype = C.c_float
+        L.orc_bf16_to_f32.argtypes = [C.c_uint16]
+        L.orc_f32_to_bf16.restype = C.c_uint16
+        L.orc_f32_to_bf16.argtypes = [C.c_float]
+        L.orc_set_elem_type.argtypes = [C.c_int]
         _lib = L
     return _lib
 
@@ -261,3 +266,28 @@ def lcg_fill_f16(state, n, scale):
     out = np.empty((n,), np.float16)
     lib().orc_lcg_fill_f16(C.byref(st), _p(out, u16p), C.c_size_t(n), C.c_float(scale))
     return out, st.value
+
+
+class bf16_mode:
+    """Context manager: the oracle's data tensors are bf16 inside (arrays are still passed as 16-bit patterns in
+    numpy float16 containers: use bf16_pack / bf16_unpack)."""
+
+    def __enter__(self):
+        lib().orc_set_elem_type(1)
+
+    def __exit__(self, *a):
+        lib().orc_set_elem_type(0)
+
+
+def bf16_pack(x):
+    """float32 array -> bf16 bit patterns (round to nearest even) in a float16-typed container."""
+    import torch  # an implementation independent of the oracle's
+
+    t = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(torch.bfloat16)
+    return t.view(torch.int16).numpy().view(np.float16).copy()
+
+
+def bf16_unpack(h):
+    """bf16 bit patterns (float16-typed or uint16 container) -> float32."""
+    u = np.ascontiguousarray(h).view(np.uint16).astype(np.uint32) << 16
+    return u.view(np.float32)

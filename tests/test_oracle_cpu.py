@@ -456,3 +456,70 @@ def test_sage_quantizer_and_decode():
     # and the quantisation error against f16 SDPA on the unquantised tensors stays small
     full = rm.gqa_decode_f64(q, k, v, H, Hkv, D, N)
     assert np.max(np.abs(got - full)) < 5e-2
+
+
+# ---------------------------------------------------------------------------------------- bf16 element mode (extension)
+
+def test_bf16_conversions_match_an_independent_implementation():
+    """orc_f32_to_bf16 / orc_bf16_to_f32 against torch's bfloat16 (round to nearest even), incl. ties, subnormals,
+    infinities and NaN."""
+    import torch
+
+    rng = np.random.default_rng(5)
+    x = np.concatenate([
+        rng.normal(size=4000).astype(np.float32) * np.float32(10.0) ** rng.integers(-30, 30, size=4000).astype(np.float32),
+        np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3895314e38, np.inf, -np.inf, 1e-40, -1e-45], np.float32),
+        (np.arange(0x3F800000, 0x3F800000 + 0x30000, 0x800, dtype=np.uint32)).view(np.float32),  # ties around 1.0
+    ])
+    want = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = np.array([orc.lib().orc_f32_to_bf16(float(v)) for v in x], np.uint16)
+    assert np.array_equal(got, want)
+    assert np.isnan(orc.lib().orc_bf16_to_f32(orc.lib().orc_f32_to_bf16(float("nan"))))
+    bits = np.arange(0, 65536, 7, dtype=np.uint16)
+    back = np.array([orc.lib().orc_bf16_to_f32(int(b)) for b in bits], np.float32)
+    ref = (bits.astype(np.uint32) << 16).view(np.float32)
+    finite = ~np.isnan(ref)  # NaN payloads do not survive the trip through a Python float
+    assert np.array_equal(back.view(np.uint32)[finite], ref.view(np.uint32)[finite])
+    assert np.all(np.isnan(back[~finite]))
+
+
+def test_bf16_mode_attention_matches_float64_on_the_bf16_inputs():
+    """In bf16 mode the same recurrences run on bf16 inputs: decode and prefill against float64 softmax of the
+    (exactly representable) bf16 values, to bf16 output rounding."""
+    rng = np.random.default_rng(6)
+    H, Hkv, D, N, cap = 4, 2, 64, 77, 80
+    q = orc.bf16_pack(rng.normal(size=(H, D)))
+    k = orc.bf16_pack(rng.normal(size=(Hkv, cap, D)))
+    v = orc.bf16_pack(rng.normal(size=(Hkv, cap, D)))
+    with orc.bf16_mode():
+        out = orc.sdpa_decode(q, k, v, H, Hkv, D, cap, N)
+    want = rm.gqa_decode_f64(orc.bf16_unpack(q), orc.bf16_unpack(k), orc.bf16_unpack(v), H, Hkv, D, N)
+    got = orc.bf16_unpack(out).reshape(H, D)
+    assert np.max(np.abs(got - want)) <= 2.0 ** -8 * max(1.0, float(np.max(np.abs(want))))
+    # and f16 mode is restored afterwards
+    qh = rng.normal(size=(H, D)).astype(np.float16)
+    kh, vh = rng.normal(size=(Hkv, cap, D)).astype(np.float16), rng.normal(size=(Hkv, cap, D)).astype(np.float16)
+    assert np.max(np.abs(orc.sdpa_decode(qh, kh, vh, H, Hkv, D, cap, N).reshape(H, D).astype(np.float64)
+                         - rm.gqa_decode_f64(qh, kh, vh, H, Hkv, D, N))) <= 2e-3
+
+
+def test_bf16_mode_kv_prep_rotation_is_rounded_once_to_bf16():
+    rng = np.random.default_rng(7)
+    H, Hkv, D, T, cap, pos = 4, 2, 32, 3, 16, 5
+    qf, kf, vf = (rng.normal(size=(T, n * D)).astype(np.float32) for n in (H, Hkv, Hkv))
+    q, k, v = orc.bf16_pack(qf), orc.bf16_pack(kf), orc.bf16_pack(vf)
+    cos, sin = orc.rope_tables(1e4, D, cap)
+    kc, vc = np.zeros((Hkv, cap, D), np.float16), np.zeros((Hkv, cap, D), np.float16)
+    with orc.bf16_mode():
+        qr = orc.kv_prep_fused(q, k, v, kc, vc, cos, sin, orc.make_params(H, Hkv, D, T, pos, cap, rope_mode=0))
+    # V is copied bit for bit; rotated values equal the float64 rotation of the bf16 inputs up to one bf16 rounding
+    assert np.array_equal(vc[:, pos:pos + T].view(np.uint16),
+                          v.reshape(T, Hkv, D).transpose(1, 0, 2).view(np.uint16))
+    x = orc.bf16_unpack(q).reshape(T, H, D).astype(np.float64)
+    c, s_ = cos[pos:pos + T].astype(np.float64), sin[pos:pos + T].astype(np.float64)
+    half = D // 2
+    lo = x[..., :half] * c[:, None, :] - x[..., half:] * s_[:, None, :]
+    hi = x[..., half:] * c[:, None, :] + x[..., :half] * s_[:, None, :]
+    want = np.concatenate([lo, hi], axis=-1).transpose(1, 0, 2)
+    got = orc.bf16_unpack(qr).astype(np.float64)
+    assert np.max(np.abs(got - want)) <= 2.0 ** -8 * max(1.0, float(np.max(np.abs(want))))
