@@ -239,6 +239,15 @@ fa_status fa_set_decode_variant(fa_ctx *ctx, const fa_decode_variant *variant);
  * Environment: FOUNDRY_ATTN_PREFILL_SPLIT_K (read at fa_ctx_create). */
 fa_status fa_set_prefill_split_k(fa_ctx *ctx, uint32_t split_k);
 
+/* Prefill kernel variant, in the spirit of the reference's per-kernel variant overrides
+ * (src/metals/flashattention/variants.rs): 1 = K/V tiles staged through registers, one barrier per key tile;
+ * 2 = K/V tiles loaded straight into LDS, softmax and MFMA work of the two wave groups alternating in two
+ * barrier-separated phases, row sums on the matrix pipe (measured 3 % faster at 2048 tokens, 14 % at 8192 and on
+ * a paged cache); 0 (default) = 2. Same contract; variant 2 normalises by the sum of the f16-rounded weights that
+ * enter the PV product, variant 1 by the sum of the unrounded ones (outputs agree to one f16 ulp).
+ * Environment: FOUNDRY_ATTN_PREFILL_VARIANT (read at fa_ctx_create). */
+fa_status fa_set_prefill_variant(fa_ctx *ctx, uint32_t variant);
+
 /* ---------------------------------------------------------------------------------------------
  * Paged KV cache (no counterpart in the reference, whose cache is contiguous per layer and batch 1:
  * models/llama.json:301-330). Contract: gathering a sequence's blocks in block-table order yields,

@@ -103,6 +103,8 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     ctx->decode_variant.keys_per_split = env_u32("FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT", 0);
     ctx->decode_variant.merge = env_u32("FOUNDRY_ATTN_DECODE_MERGE", 1);
     ctx->prefill_split_k = env_u32("FOUNDRY_ATTN_PREFILL_SPLIT_K", 0);
+    ctx->prefill_variant = env_u32("FOUNDRY_ATTN_PREFILL_VARIANT", 0);
+    if (ctx->prefill_variant > 2) ctx->prefill_variant = 0;
     fa_status s = fa_ensure_workspace(ctx, (size_t)64 << 20);
     if (s == FA_OK) s = fa_ensure_counters(ctx, 4096);
     if (s != FA_OK) {
@@ -180,6 +182,13 @@ extern "C" fa_status fa_set_prefill_split_k(fa_ctx *ctx, uint32_t split_k) {
     FA_NEED(ctx, "ctx");
     if (split_k > 64) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "prefill split_k must be <= 64, got %u", split_k);
     ctx->prefill_split_k = split_k;
+    return FA_OK;
+}
+
+extern "C" fa_status fa_set_prefill_variant(fa_ctx *ctx, uint32_t variant) {
+    FA_NEED(ctx, "ctx");
+    if (variant > 2) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "prefill variant must be 0, 1 or 2, got %u", variant);
+    ctx->prefill_variant = variant;
     return FA_OK;
 }
 

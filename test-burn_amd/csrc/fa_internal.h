@@ -36,6 +36,7 @@ struct fa_ctx {
     uint32_t n_counters = 0;
     fa_decode_variant decode_variant{0, 1};
     uint32_t prefill_split_k = 0;  // 0 = auto
+    uint32_t prefill_variant = 0;  // 0 = auto, 1 = tiles staged through registers, 2 = tiles straight into LDS, two-phase loop
     // per-kernel profiling
     bool profiling = false;
     std::vector<FaProfileRec> prof;

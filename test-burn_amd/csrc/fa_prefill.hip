@@ -394,6 +394,424 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_mfma_kernel(PrefillDev a
     }
 }
 
+// value of lane l ^ 32 folded in with max: one VALU lane-half swap (both results hold {x[l], x[l ^ 32]})
+__device__ __forceinline__ float max_with_other_half(float x) {
+    typedef unsigned int u2v __attribute__((ext_vector_type(2)));
+    const unsigned v = __float_as_uint(x);
+    const u2v r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return fmaxf(__uint_as_float(r.x), __uint_as_float(r.y));
+}
+
+// A barrier the instruction scheduler moves nothing across (it would otherwise be free to sink MFMAs below it or
+// hoist VALU work above it, which is exactly what the two-phase loop must not allow).
+__device__ __forceinline__ void phase_barrier() {
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// 16 bytes per lane from a buffer straight into LDS: lane l's bytes land at lds_addr + imm + 16 l, read from
+// base + voff + soff + imm; out-of-range lanes deliver zeros. Written as assembly so that the compiler does not
+// serialise every later LDS read behind it (it cannot tell which LDS bytes such a load writes); completion is
+// tracked by vmcnt, and the waits are placed by hand.
+typedef unsigned int rsrc_words __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ rsrc_words make_rsrc_words(const void *base, uint32_t bytes) {
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    rsrc_words r;
+    r.x = (uint32_t)b, r.y = (uint32_t)(b >> 32) & 0xffffu, r.z = bytes, r.w = 0x00020000u;
+    return r;
+}
+// N such loads whose sources are SRC_STEP bytes apart and whose destinations are DST_STEP bytes apart. When the two
+// steps are equal the instruction's immediate offset (which moves source and destination alike) does the stepping.
+template <int N, int SRC_STEP, int DST_STEP>
+__device__ __forceinline__ void buffer_to_lds_b128(rsrc_words rs, uint32_t lds_addr, int voff, int soff) {
+    static_assert(N == 1 || N == 2 || N == 4, "1, 2 or 4 loads");
+    if constexpr (SRC_STEP == DST_STEP) {
+        static_assert((N - 1) * SRC_STEP < 4096, "12-bit immediate");
+        if constexpr (N == 4)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                         "buffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
+                         "buffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds\n\t"
+                         "buffer_load_dwordx4 %1, %2, %3 offen offset:%5 lds\n\t"
+                         "buffer_load_dwordx4 %1, %2, %3 offen offset:%6 lds"
+                         :
+                         : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff), "n"(SRC_STEP), "n"(2 * SRC_STEP), "n"(3 * SRC_STEP)
+                         : "memory");
+        else if constexpr (N == 2)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                         "buffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
+                         "buffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds"
+                         :
+                         : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff), "n"(SRC_STEP)
+                         : "memory");
+        else
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :
+                         : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
+                         : "memory");
+    } else {  // (the source-offset update sits between the m0 write and the load that needs it)
+        int so = soff;
+        if constexpr (N == 4)
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\t"
+                         "buffer_load_dwordx4 %2, %3, %0 offen lds\n\t"
+                         "s_add_i32 m0, %1, %5\n\ts_add_i32 %0, %0, %4\n\t"
+                         "buffer_load_dwordx4 %2, %3, %0 offen lds\n\t"
+                         "s_add_i32 m0, %1, %6\n\ts_add_i32 %0, %0, %4\n\t"
+                         "buffer_load_dwordx4 %2, %3, %0 offen lds\n\t"
+                         "s_add_i32 m0, %1, %7\n\ts_add_i32 %0, %0, %4\n\t"
+                         "buffer_load_dwordx4 %2, %3, %0 offen lds"
+                         : "+s"(so)
+                         : "s"(lds_addr), "v"(voff), "s"(rs), "n"(SRC_STEP), "n"(DST_STEP), "n"(2 * DST_STEP), "n"(3 * DST_STEP)
+                         : "memory", "scc");
+        else if constexpr (N == 2)
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\t"
+                         "buffer_load_dwordx4 %2, %3, %0 offen lds\n\t"
+                         "s_add_i32 m0, %1, %5\n\ts_add_i32 %0, %0, %4\n\t"
+                         "buffer_load_dwordx4 %2, %3, %0 offen lds"
+                         : "+s"(so)
+                         : "s"(lds_addr), "v"(voff), "s"(rs), "n"(SRC_STEP), "n"(DST_STEP)
+                         : "memory", "scc");
+        else
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                         :
+                         : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
+                         : "memory");
+    }
+}
+
+// Two-phase variant of the kernel above (same tiling and arithmetic; results differ only by the order in which a
+// row's weights are summed).
+//
+// What bounds the loop is the rate at which ONE wave issues instructions (about one per 5 cycles on this part, of
+// any kind; a dependent VALU pair 8.6, an exp 9), not the throughput of a unit: a key tile costs a wave some 400
+// instructions of which 32 are MFMAs, and two waves share a SIMD. So the work of a tile is cut into
+//   a VALU phase  softmax of S_j -> P_j (about 150 instructions), the requests for the next tiles, and the first
+//                 operand reads of the coming MFMA phase, and
+//   an MFMA phase S_{j+1} = K_{j+1} Q^T and O^T += V_j^T P_j as ONE scheduling region: 32 MFMAs fed by LDS reads
+//                 issued six operands ahead (left alone the scheduler keeps two in flight and the pipe idles),
+// each ended by a workgroup barrier, and the two groups of four waves run one phase apart: the two waves that share
+// a SIMD are then never in the same phase.
+// K/V tiles go from memory straight into LDS (buffer_load ... lds: the 64 lanes of one instruction fill 1 KB of
+// consecutive LDS bytes), so no registers and no issue slots are spent on staging them. Row padding is impossible inside such a 1 KB run, so the tiles are laid out for conflict-free
+// reads with plain base + constant addressing instead:
+//   K tile  [16-row block rb][16-byte chunk c][row r of 16]        one instruction = 4 chunks x 16 rows;
+//           the S^T operand read of 16 lanes (16 rows, same chunk) is 256 consecutive bytes.
+//   V tile  [4-row group rg][64-byte column block cb][row r4][64 B] one instruction = 4 (D=128) or 8 rows;
+//           the 32 lanes of a transpose-read pass (4 rows x 64 B) are 256 consecutive bytes.
+// Wave w of a group moves rows 16w..16w+15 of every tile of its group (16 rows never straddle a page). Rows past
+// the visible keys come out of the buffer descriptor's bound check as zeros.
+template <int D, bool BF16, bool PAGED>
+__global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a) {
+    constexpr int DSTEPS = D / 16, DBLKS = D / 32, ROWB = D * 2, CHK = D / 8;
+    constexpr int K_TILE = BN * ROWB, V_TILE = BN * ROWB, GRP_LDS = 2 * K_TILE + 2 * V_TILE;
+    constexpr int RB_BYTES = CHK * 256;  // one 16-row block of a K tile
+    constexpr int RG_BYTES = 4 * ROWB;   // one 4-row group of a V tile
+    constexpr int K_DMA = CHK / 4, V_DMA = 16 * ROWB / 1024;  // instructions per wave per tile
+    constexpr int K_AHEAD = 6, V_AHEAD = 6;
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * GRP_LDS];  // [group]{K[2], V[2]}
+
+    const int lane = threadIdx.x & 63;
+    const int wave8 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int grp = wave8 >> 2, wave = wave8 & 3;
+    unsigned char *k_base = lds + grp * GRP_LDS, *v_base = k_base + 2 * K_TILE;
+    const uint32_t k_lds_addr = (uint32_t)(uintptr_t)(lds_ptr)lds + grp * GRP_LDS, v_lds_addr = k_lds_addr + 2 * K_TILE;
+    const int n = lane & 31, hi = lane >> 5;
+    const uint32_t S = a.splits;
+    const uint32_t n_qt = gridDim.x / (a.n_heads * S);
+    const uint32_t q_tile = n_qt - 1 - blockIdx.x / (a.n_heads * S);  // heaviest query tiles first
+    const uint32_t head = (blockIdx.x / S) % a.n_heads;
+    const uint32_t split = blockIdx.x % S;
+    const uint32_t kvh = head / a.group_size;
+    const uint32_t q0 = q_tile * BM;
+    const uint32_t q_row = q0 + wave * 32 + n;
+    const uint32_t q_row_c = min(q_row, a.q_len - 1);
+    uint32_t kv_end = a.kv_len;
+    if (a.causal) {
+        const uint64_t last = (uint64_t)min(q0 + BM - 1, a.q_len - 1) + a.query_offset + 1;
+        kv_end = (uint32_t)min((uint64_t)a.kv_len, last);
+    }
+    const int all_tiles = (int)((kv_end + BN - 1) / BN);
+    const int per_split = (all_tiles + (int)S - 1) / (int)S;
+    const int t_lo = min(all_tiles, (int)split * per_split);
+    const int n_tiles = min(all_tiles, t_lo + per_split);
+    const int t0 = t_lo + grp;                                  // group g attends tiles t0, t0 + 2, ...
+    const int ntg = t0 < n_tiles ? (n_tiles - t0 + 1) / 2 : 0;  // how many
+    const int iters = (n_tiles - t_lo + 1) / 2;                 // of group 0: the barriers are workgroup-wide
+
+    U4H8 qreg[DSTEPS];
+    {
+        const __half *qp = a.q + (size_t)head * a.q_stride_h + (size_t)q_row_c * a.q_stride_m;
+#pragma unroll
+        for (int s = 0; s < DSTEPS; ++s) qreg[s].u = *reinterpret_cast<const uint4 *>(qp + s * 16 + hi * 8);
+    }
+
+    // ---- memory -> LDS. Lane l of a K instruction takes chunk l / 16 of row l % 16; of a V instruction, piece
+    // l % 4 of column block (l / 16) % (ROWB / 64) of row (l / (16 ROWB / 64)) * 4 + (l % 16) / 4.
+    constexpr int CBR = ROWB / 64;
+    const int k_lane_src = (lane & 15) * ROWB + (lane >> 4) * 16;
+    const int v_lane_src = ((lane / (16 * CBR)) * 4 + ((lane & 15) >> 2)) * ROWB + ((lane >> 4) % CBR) * 64 + (lane & 3) * 16;
+    rsrc_words krs = make_rsrc_words(nullptr, 0), vrs = krs;
+    if (!PAGED) {
+        krs = make_rsrc_words(a.k + (size_t)kvh * a.k_stride_h, kv_end * (uint32_t)ROWB);
+        vrs = make_rsrc_words(a.v + (size_t)kvh * a.v_stride_h, kv_end * (uint32_t)ROWB);
+    }
+    typedef const int32_t __attribute__((address_space(4))) *const_i32p;
+    const const_i32p bt = (const_i32p)a.block_table;
+    const uint32_t bs_shift = a.block_shift;
+    // page id of this wave's 16 rows of group-local tile i (wave-uniform: a scalar load)
+    auto page_of = [&](int i) -> int32_t {
+        const uint32_t key = (uint32_t)(t0 + 2 * i) * BN + 16 * wave;
+        return (PAGED && key < kv_end) ? bt[bs_shift < 32 ? key >> bs_shift : key / a.block_size] : 0;
+    };
+    // this wave's 16 rows of group-local tile i of one tensor into LDS buffer `buf`
+    auto dma = [&](bool is_k, int i, int buf, int32_t page) {
+        const uint32_t key = (uint32_t)(t0 + 2 * i) * BN + 16 * wave;
+        rsrc_words rs = is_k ? krs : vrs;
+        int so = (int)(key * (uint32_t)ROWB);
+        if (PAGED) {
+            const uint32_t valid = key < kv_end ? min(16u, kv_end - key) : 0u;
+            const uint32_t rip = bs_shift < 32 ? key & (a.block_size - 1) : key % a.block_size;
+            const size_t base = (((size_t)page * a.n_kv_heads + kvh) * a.block_size + rip) * (size_t)ROWB;
+            const unsigned char *pool = reinterpret_cast<const unsigned char *>(is_k ? a.k : a.v);
+            rs = make_rsrc_words(pool + base, valid * ROWB);
+            so = 0;
+        }
+        if (is_k) {
+            // chunk quads: 64 bytes apart in a row, 1 KB apart in LDS
+            buffer_to_lds_b128<K_DMA, 64, 1024>(rs, k_lds_addr + buf * K_TILE + wave * RB_BYTES, k_lane_src, so);
+        } else {
+            // 1 KB of rows after 1 KB of rows, in memory as in LDS
+            buffer_to_lds_b128<V_DMA, 1024, 1024>(rs, v_lds_addr + buf * V_TILE + wave * (4 * RG_BYTES), v_lane_src, so);
+        }
+    };
+
+    f16_t oacc[DBLKS];
+#pragma unroll
+    for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[b][i] = 0.0f;
+    // Row sums ride on the matrix pipe: an all-ones A operand against P^T leaves, in every accumulator of a lane,
+    // the sum of that lane's query row over the keys of the step (both lane halves included) - 4 more MFMAs a tile
+    // instead of 32 more additions in the VALU phase, which is the longer one. Only element 0 is ever read.
+    f16_t lacc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) lacc[i] = 0.0f;
+    h8_t ones;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ones[i] = to_elem<BF16>(1.0f);
+    float m_run = -1e30f;
+    const float c = a.scale_log2e;
+    const uint32_t q_abs = q_row_c + a.query_offset;
+    const uint32_t wave_min_limit = a.causal ? (min(q0 + wave * 32, a.q_len - 1) + a.query_offset) : 0xffffffffu;
+
+    // On entry to MFMA phase j the LDS holds K_{j+1} in K[(j+1)&1] and V_j in V[j&1]. VALU phase j starts by
+    // requesting K_{j+2} into K[j&1] and V_{j+1} into V[(j+1)&1] (both buffers were last read in MFMA phase j-1);
+    // the requests are complete (vmcnt) before the barrier that ends MFMA phase j, two phases later, so VALU phase
+    // j+1 may already fetch the first operands of MFMA phase j+1 ahead of its barrier.
+    int32_t pg_k = 0, pg_v = 0, pg_next = 0;  // pages of the K tile / V tile requested next, and of the K tile after
+    if (ntg > 0) {
+        const int32_t p0 = page_of(0), p1 = page_of(1);
+        pg_k = page_of(2), pg_next = page_of(3), pg_v = p1;
+        dma(true, 0, 0, p0);
+        dma(false, 0, 0, p0);
+        if (ntg > 1) dma(true, 1, 1, p1);
+    }
+#pragma unroll
+    for (int s = 0; s < DSTEPS; ++s) {  // the query operand has arrived: keep its wait out of the loop
+        u4_t t = __builtin_bit_cast(u4_t, qreg[s].u);
+        asm volatile("" : "+v"(t));
+        qreg[s].u = __builtin_bit_cast(uint4, t);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's rows are in LDS
+    __syncthreads();
+
+    const int k_lane = (n >> 4) * RB_BYTES + hi * 256 + (n & 15) * 16;
+    const int v_lane = hi * RG_BYTES + ((lane & 15) >> 2) * 64 + ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
+    f16_t sacc[2];
+    h8_t pb[2][2];
+    U4H8 kpre[K_AHEAD];  // the first K operands of the next MFMA phase, read before the barrier that starts it
+    auto k_prefetch = [&](int buf) {
+        const unsigned char *k_lds = k_base + buf * K_TILE + k_lane;
+#pragma unroll
+        for (int i = 0; i < K_AHEAD; ++i)
+            kpre[i].u = *reinterpret_cast<const uint4 *>(k_lds + (i / DSTEPS) * (2 * RB_BYTES) + (i % DSTEPS) * 512);
+    };
+    auto s_tile = [&](int buf, bool own_pipeline) {
+        const unsigned char *k_lds = k_base + buf * K_TILE + k_lane;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < DSTEPS; ++s) {
+                U4H8 kk;
+                if (kb * DSTEPS + s < K_AHEAD) kk = kpre[kb * DSTEPS + s];
+                else kk.u = *reinterpret_cast<const uint4 *>(k_lds + kb * (2 * RB_BYTES) + s * 512);
+                sacc[kb] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(kk.b, qreg[s].b, sacc[kb], 0, 0, 0)
+                                : __builtin_amdgcn_mfma_f32_32x32x16_f16(kk.h, qreg[s].h, sacc[kb], 0, 0, 0);
+            }
+        }
+        if (!own_pipeline) return;
+#pragma unroll
+        for (int i = 0; i < 2 * DSTEPS; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+    };
+    // One scheduling region, nothing conditional. (After the group's last tile S_{j+1} is computed from whatever the
+    // buffer holds and never used: cheaper than a second copy of this code, which also made the register allocator
+    // shuffle the 64 accumulator registers between two homes on every iteration.)
+    auto mfma_phase = [&](int j) {
+        s_tile((j + 1) & 1, false);
+        const unsigned char *v_lds = v_base + (j & 1) * V_TILE + v_lane;
+        // k-slot jj of k-step ks <-> key 32 kb + 16 ks + ... = accumulator 8 ks + jj of block kb, for both operands
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                lacc = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, ones), __builtin_bit_cast(bf8_t, pb[kb][ks]), lacc, 0, 0, 0)
+                            : __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pb[kb][ks], lacc, 0, 0, 0);
+#pragma unroll
+                for (int b = 0; b < DBLKS; ++b) {
+                    const unsigned char *p0 = v_lds + (kb * 8 + ks * 4) * RG_BYTES + b * 256;
+                    const unsigned char *p1 = p0 + 2 * RG_BYTES;
+                    union {
+                        fp16x4_t f[2];
+                        h8_t h;
+                    } va;
+                    va.f[0] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p0));
+                    va.f[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p1));
+                    oacc[b] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, va.h),
+                                                                           __builtin_bit_cast(bf8_t, pb[kb][ks]), oacc[b], 0, 0, 0)
+                                   : __builtin_amdgcn_mfma_f32_32x32x16_f16(va.h, pb[kb][ks], oacc[b], 0, 0, 0);
+                }
+            }
+        // operand reads run K_AHEAD / V_AHEAD MFMAs ahead across both contractions
+        constexpr int NS = 2 * DSTEPS, NPV = 4 * DBLKS + 4, VR = 8 * DBLKS, V_EARLY = 2 * V_AHEAD;
+#pragma unroll
+        for (int i = 0; i < NS; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 2);
+            if (i < NS - K_AHEAD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 2);
+            else __builtin_amdgcn_sched_group_barrier(0x100, 2, 2);
+        }
+#pragma unroll
+        for (int i = 0; i < NPV; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 2);
+            if (V_EARLY + 2 * i < VR) __builtin_amdgcn_sched_group_barrier(0x100, 2, 2);
+        }
+    };
+    if (ntg > 0) {
+        k_prefetch(0);
+        s_tile(0, true);
+    }
+    if (grp == 1) phase_barrier();  // one phase behind group 0
+    for (int j = 0; j < iters; ++j) {
+        if (j < ntg) {  // ---- VALU phase: P_j = 2^(c S_j - m), running max and sum
+            if (j + 2 < ntg) dma(true, j + 2, j & 1, pg_k);
+            if (j + 1 < ntg) dma(false, j + 1, (j + 1) & 1, pg_v);
+            pg_v = pg_k, pg_k = pg_next;
+            if (PAGED && j + 4 < ntg) pg_next = page_of(j + 4);
+            const uint32_t key0 = (uint32_t)(t0 + 2 * j) * BN;
+            const bool need_mask = (key0 + BN - 1 > wave_min_limit) || (key0 + BN > kv_end);
+            if (need_mask) {  // accumulator i of block kb is key key0 + 32 kb + 8 (i / 4) + 4 hi + i % 4
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const uint32_t key = key0 + kb * 32 + (i / 4) * 8 + hi * 4 + (i % 4);
+                        const bool vis = key < kv_end && (!a.causal || key <= q_abs);
+                        sacc[kb][i] = vis ? sacc[kb][i] : -INFINITY;
+                    }
+            }
+            float part[4] = {sacc[0][0], sacc[0][1], sacc[0][2], sacc[0][3]};  // four short chains, not one long
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) part[i & 3] = fmaxf(part[i & 3], sacc[kb][i]);
+            const float mloc = max_with_other_half(fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]))) * c;
+            // lazy rescale: only when a row maximum has grown by more than 2^8 (weights up to 256 until then; the
+            // final division by l removes the common factor)
+            if (__any(mloc > m_run + 8.0f)) {
+                const float m_new = fmaxf(m_run, mloc);
+                const float alpha = fast_exp2(m_run - m_new);
+                lacc[0] *= alpha;
+                m_run = m_new;
+#pragma unroll
+                for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
+            }
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                    for (int jj = 0; jj < 8; ++jj)
+                        pb[kb][ks][jj] = to_elem<BF16>(fast_exp2(fmaf(sacc[kb][8 * ks + jj], c, -m_run)));
+            k_prefetch((j + 1) & 1);
+        }
+        phase_barrier();
+        if (j < ntg) mfma_phase(j);  // ---- MFMA phase
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the rows requested in the last VALU phase have landed
+        phase_barrier();
+    }
+    if (grp == 0) phase_barrier();  // same number of barriers for both groups
+
+    // merge the two groups' states: group 1 parks (m, l, acc) in LDS as [value][wave][lane], group 0 folds them in
+    {
+        float *mx = reinterpret_cast<float *>(lds);
+        const int slot = wave * 64 + lane;
+        if (grp == 1) {
+            mx[slot] = m_run;
+            mx[256 + slot] = lacc[0];
+#pragma unroll
+            for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) mx[(2 + b * 16 + i) * 256 + slot] = oacc[b][i];
+        }
+        __syncthreads();
+        if (grp == 1) return;
+        const float m1 = mx[slot], l1 = mx[256 + slot];
+        const float m = fmaxf(m_run, m1);
+        const float e0 = fast_exp2(m_run - m), e1 = fast_exp2(m1 - m);
+        lacc[0] = lacc[0] * e0 + l1 * e1;
+#pragma unroll
+        for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[b][i] = oacc[b][i] * e0 + mx[(2 + b * 16 + i) * 256 + slot] * e1;
+        m_run = m;
+    }
+    const float l_tot = lacc[0];
+    if (S > 1) {  // unnormalised partial state for the merge kernel (flash_prefill.metal:592-617)
+        if (q_row >= a.q_len) return;
+        const size_t prow = (((size_t)head * n_qt + q_tile) * S + split) * BM + wave * 32 + n;
+        float *pa = a.part_acc + prow * D;
+#pragma unroll
+        for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+            for (int gi = 0; gi < 4; ++gi) {
+                float4 v = make_float4(oacc[b][gi * 4], oacc[b][gi * 4 + 1], oacc[b][gi * 4 + 2], oacc[b][gi * 4 + 3]);
+                *reinterpret_cast<float4 *>(pa + b * 32 + gi * 8 + hi * 4) = v;
+            }
+        if (hi == 0) a.part_ml[prow * 2] = m_run, a.part_ml[prow * 2 + 1] = l_tot;
+        return;
+    }
+    const float inv_l = (isfinite(l_tot) && fabsf(l_tot) > 1e-6f) ? (1.0f / l_tot) : 0.0f;  // flash_prefill.metal:255-261
+    if (q_row < a.q_len) {
+        __half *op = a.out + (size_t)head * a.out_stride_h + (size_t)q_row * a.out_stride_m;
+#pragma unroll
+        for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+            for (int gi = 0; gi < 4; ++gi) {  // accumulators 4gi..4gi+3 are d = 32b + 8gi + 4hi + 0..3
+                h4_t o;
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) o[jj] = to_elem<BF16>(oacc[b][gi * 4 + jj] * inv_l);
+                *reinterpret_cast<h4_t *>(op + b * 32 + gi * 8 + hi * 4) = o;
+            }
+    }
+}
+
 // Merge of the per-split states (flash_prefill.metal:843-888): m* = max m_s, L = sum l_s 2^(m_s - m*) over the
 // splits with l_s > 0, out = sum acc_s 2^(m_s - m*) / L (0 when L is unusable). m is kept in the exp2 domain.
 template <int D, bool BF16>
@@ -483,8 +901,19 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
     }
     dim3 grid(base_wgs * splits, 1, 1);
     {
-        FaLaunchScope scope(ctx, "flash_prefill_mfma_kernel", true);
-        if (L.head_dim == 128 && L.bf16)
+        const bool lds_direct = ctx->prefill_variant != 1;  // measured faster at every size (8 to 15 %)
+        FaLaunchScope scope(ctx, lds_direct ? "flash_prefill_dma_kernel" : "flash_prefill_mfma_kernel", true);
+        if (lds_direct) {
+            auto kern = flash_prefill_dma_kernel<128, false, false>;
+            if (L.head_dim == 128) {
+                kern = L.bf16 ? (L.paged ? flash_prefill_dma_kernel<128, true, true> : flash_prefill_dma_kernel<128, true, false>)
+                              : (L.paged ? flash_prefill_dma_kernel<128, false, true> : flash_prefill_dma_kernel<128, false, false>);
+            } else {
+                kern = L.bf16 ? (L.paged ? flash_prefill_dma_kernel<64, true, true> : flash_prefill_dma_kernel<64, true, false>)
+                              : (L.paged ? flash_prefill_dma_kernel<64, false, true> : flash_prefill_dma_kernel<64, false, false>);
+            }
+            scope.launch(kern, grid, dim3(512), 0, a);
+        } else if (L.head_dim == 128 && L.bf16)
             scope.launch(flash_prefill_mfma_kernel<128, true>, grid, dim3(512), 0, a);
         else if (L.head_dim == 128)
             scope.launch(flash_prefill_mfma_kernel<128, false>, grid, dim3(512), 0, a);

@@ -98,6 +98,7 @@ PROTOTYPES = {
                                    C.POINTER(KvPrepFusedParams), _u32],
     "fa_set_decode_variant": [_vp, C.POINTER(DecodeVariant)],
     "fa_set_prefill_split_k": [_vp, C.c_uint32],
+    "fa_set_prefill_variant": [_vp, C.c_uint32],
     "fa_kv_prep_fused_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _u32, _PT, _PT,
                                C.POINTER(KvPrepFusedParams)],
     "fa_kv_prep_decode_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _PT, _PT, C.POINTER(KvPrepFusedParams)],
@@ -245,6 +246,9 @@ class Foundry:
 
     def set_prefill_split_k(self, split_k=0):
         check(self.lib.fa_set_prefill_split_k(self.h, split_k))
+
+    def set_prefill_variant(self, variant):
+        check(self.lib.fa_set_prefill_variant(self.h, variant))
 
     def profile_enable(self, on=True):
         check(self.lib.fa_profile_enable(self.h, int(on)))

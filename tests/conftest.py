@@ -10,3 +10,12 @@ sys.path.insert(0, os.path.join(ROOT, "test-burn_amd"))
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(params=[1, 2], ids=["staged", "lds_direct"])
+def prefill_variant(request):
+    """Runs a GPU test once per prefill kernel variant (fa_set_prefill_variant) and restores the default."""
+    from gpu_util import ctx
+    ctx().set_prefill_variant(request.param)
+    yield request.param
+    ctx().set_prefill_variant(0)

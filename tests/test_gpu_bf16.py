@@ -102,6 +102,7 @@ def test_fused_decode_step_bf16_contiguous_and_paged():
         b.free()
 
 
+@pytest.mark.usefixtures("prefill_variant")
 @pytest.mark.parametrize("D,H,Hkv,M,prefix", [(128, 6, 2, 200, 333), (64, 14, 2, 70, 0), (128, 24, 8, 33, 2000)])
 def test_prefill_bf16_vs_oracle(D, H, Hkv, M, prefix):
     announce("prefill bf16", D, M, prefix)

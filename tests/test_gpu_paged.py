@@ -108,6 +108,7 @@ def test_paged_batched_decode_step(H, Hkv, D, bs, lens):
         b.free()
 
 
+@pytest.mark.usefixtures("prefill_variant")
 def test_paged_prefill_append_then_decode_equals_contiguous():
     """Multi-token append into an empty paged cache (one sequence of a batch), compared with the contiguous op."""
     announce("paged prefill append")

@@ -10,7 +10,7 @@ import orc
 import refmath as rm
 from gpu_util import announce, bits, ctx, h16, max_abs
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.usefixtures("prefill_variant")]  # every case under both kernels
 TOL = 2e-3
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
