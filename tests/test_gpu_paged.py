@@ -225,3 +225,33 @@ def test_paged_fused_step_equals_separate_ops():
                                orc.make_params(H, Hkv, D, 1, n, n + 1, rope_mode=0))
         want = orc.sdpa_decode(qr[:, 0].copy(), kc, vc, H, Hkv, D, n + 1, n + 1).reshape(H, D)
         assert max_abs(outs[1][1].reshape(B, H, D)[b], want) <= TOL
+
+
+def test_paged_decode_full_batch_of_32_ragged_sequences():
+    """The Qwen2.5-3B-shaped batched paged decode at full size: 32 sequences with lengths drawn from 512..16384,
+    16-token blocks behind a random block permutation. Every sequence against the oracle over its gathered cache."""
+    announce("paged decode, 32 ragged sequences")
+    f = ctx()
+    rng = np.random.default_rng(2024)
+    H, Hkv, D, bs, B = 16, 2, 128, 16, 32
+    lens = [int(x) for x in rng.integers(512, 16385, size=B)]
+    ks = [h16(rng.normal(size=(Hkv, n, D))) for n in lens]
+    vs = [h16(rng.normal(size=(Hkv, n, D))) for n in lens]
+    pg = Paged(f, rng, lens, Hkv, D, bs, extra_tokens=0)
+    pg.fill_from(ks, vs)
+    pg.upload()
+    q = h16(rng.normal(size=(B, H, D)))
+    dq, dout = f.array(q), f.zeros((B, H * D))
+    f.flash_decode_paged(dq.arg(), pg.desc, dout.arg(), H, 0, max(lens))
+    f.synchronize()
+    got = dout.download().reshape(B, H, D)
+    assert np.all(np.isfinite(got))
+    worst = 0.0
+    for b, n in enumerate(lens):
+        want = orc.sdpa_decode(q[b], ks[b], vs[b], H, Hkv, D, n, n, n_threads=8).reshape(H, D)
+        worst = max(worst, max_abs(got[b], want))
+    print("32 ragged sequences, %d keys in total: max abs err %.2e" % (sum(lens), worst), flush=True)
+    assert worst <= TOL
+    pg.free()
+    for b in (dq, dout):
+        b.free()

@@ -19,7 +19,8 @@ def outlier_normal(rng, shape, frac=0.01, sigma=8.0):
 
 
 @pytest.mark.parametrize("H,Hkv,D,N,cap", [(16, 4, 128, 4096, 4096), (16, 4, 128, 1000, 1024), (14, 2, 64, 333, 352),
-                                           (8, 8, 128, 31, 64)])
+                                           (8, 8, 128, 31, 64),
+                                           (16, 4, 128, 32768, 32768)])  # SmolLM3 shape at the full 32K context
 def test_sage_quantize_and_decode(H, Hkv, D, N, cap):
     announce("sage", H, Hkv, D, N)
     f = ctx()
