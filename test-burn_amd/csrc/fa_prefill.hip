@@ -540,11 +540,6 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     const int iters = (n_tiles - t_lo + 1) / 2;                 // of group 0: the barriers are workgroup-wide
 
     U4H8 qreg[DSTEPS];
-    {
-        const __half *qp = a.q + (size_t)head * a.q_stride_h + (size_t)q_row_c * a.q_stride_m;
-#pragma unroll
-        for (int s = 0; s < DSTEPS; ++s) qreg[s].u = *reinterpret_cast<const uint4 *>(qp + s * 16 + hi * 8);
-    }
 
     // ---- memory -> LDS. Lane l of a K instruction takes chunk l / 16 of row l % 16; of a V instruction, piece
     // l % 4 of column block (l / 16) % (ROWB / 64) of row (l / (16 ROWB / 64)) * 4 + (l % 16) / 4.
@@ -609,22 +604,46 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     // requesting K_{j+2} into K[j&1] and V_{j+1} into V[(j+1)&1] (both buffers were last read in MFMA phase j-1);
     // the requests are complete (vmcnt) before the barrier that ends MFMA phase j, two phases later, so VALU phase
     // j+1 may already fetch the first operands of MFMA phase j+1 ahead of its barrier.
+    // The query rows take the same road once: into LDS in the K tile's layout (wave w moves rows 16w..16w+15 as one
+    // 16-row block; rows past the last query come out of the descriptor's bound check as zeros), then each lane
+    // picks its operand pieces out of them. (Loading the pieces straight from memory, 16 bytes from each of 64
+    // places per instruction, cost every workgroup 2.6 us.) The 8 blocks are parked in the two groups' second V
+    // buffers, which no tile needs yet.
+    {
+        const size_t q_bytes = ((size_t)(a.q_len - 1) * a.q_stride_m + D) * 2;
+        const rsrc_words qrs = make_rsrc_words(a.q + (size_t)head * a.q_stride_h, (uint32_t)q_bytes);
+        const int q_lane_src = (lane & 15) * (int)(a.q_stride_m * 2) + (lane >> 4) * 16;
+        const uint32_t dst = (uint32_t)(uintptr_t)(lds_ptr)lds + (wave8 >> 2) * GRP_LDS + 2 * K_TILE + V_TILE + (wave8 & 3) * RB_BYTES;
+        buffer_to_lds_b128<K_DMA, 64, 1024>(qrs, dst, q_lane_src, (int)((q0 + 16 * wave8) * (uint32_t)(a.q_stride_m * 2)));
+    }
     int32_t pg_k = 0, pg_v = 0, pg_next = 0;  // pages of the K tile / V tile requested next, and of the K tile after
     if (ntg > 0) {
         const int32_t p0 = page_of(0), p1 = page_of(1);
         pg_k = page_of(2), pg_next = page_of(3), pg_v = p1;
         dma(true, 0, 0, p0);
-        dma(false, 0, 0, p0);
         if (ntg > 1) dma(true, 1, 1, p1);
+        dma(false, 0, 0, p0);
     }
-#pragma unroll
-    for (int s = 0; s < DSTEPS; ++s) {  // the query operand has arrived: keep its wait out of the loop
-        u4_t t = __builtin_bit_cast(u4_t, qreg[s].u);
-        asm volatile("" : "+v"(t));
-        qreg[s].u = __builtin_bit_cast(uint4, t);
-    }
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's rows are in LDS
+    // Q, K_0 (for S_0) and K_1 (whose first operands the first VALU phase reads ahead) must be there now; V_0,
+    // requested last (loads complete in order), has until the first MFMA phase. A CU pulls about 25 GB/s on its
+    // own, so every 16 KB not waited for here is worth half a microsecond.
+    constexpr int VMCNT_V = 0x0F70 | V_DMA, VMCNT_KV = 0x0F70 | (V_DMA + K_DMA);
+    if (ntg > 0) __builtin_amdgcn_s_waitcnt(VMCNT_V);
+    else __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
+    {
+        const int rb = wave * 2 + (n >> 4);  // 16-row block of this lane's row; both groups hold the same 128 rows
+        const unsigned char *qp = lds + (rb >> 2) * GRP_LDS + 2 * K_TILE + V_TILE + (rb & 3) * RB_BYTES + hi * 256 + (n & 15) * 16;
+#pragma unroll
+        for (int s = 0; s < DSTEPS; ++s) qreg[s].u = *reinterpret_cast<const uint4 *>(qp + s * 512);
+#pragma unroll
+        for (int s = 0; s < DSTEPS; ++s) {  // arrived: keep the wait out of the loop
+            u4_t t = __builtin_bit_cast(u4_t, qreg[s].u);
+            asm volatile("" : "+v"(t));
+            qreg[s].u = __builtin_bit_cast(uint4, t);
+        }
+    }
+    __syncthreads();  // before the buffers the rows were parked in receive their first V tiles
 
     const int k_lane = (n >> 4) * RB_BYTES + hi * 256 + (n & 15) * 16;
     const int v_lane = hi * RG_BYTES + ((lane & 15) >> 2) * 64 + ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
@@ -750,6 +769,11 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
                     for (int jj = 0; jj < 8; ++jj)
                         pb[kb][ks][jj] = to_elem<BF16>(fast_exp2(fmaf(sacc[kb][8 * ks + jj], c, -m_run)));
             k_prefetch((j + 1) & 1);
+            if (j == 0) {  // V_0 has landed: everything but what this phase requested (K_2, V_1)
+                if (ntg > 2) __builtin_amdgcn_s_waitcnt(VMCNT_KV);
+                else if (ntg > 1) __builtin_amdgcn_s_waitcnt(VMCNT_V);
+                else __builtin_amdgcn_s_waitcnt(0x0F70);
+            }
         }
         phase_barrier();
         if (j < ntg) mfma_phase(j);  // ---- MFMA phase
@@ -901,7 +925,8 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
     }
     dim3 grid(base_wgs * splits, 1, 1);
     {
-        const bool lds_direct = ctx->prefill_variant != 1;  // measured faster at every size (8 to 15 %)
+        // the LDS-direct kernel (measured faster at every size) addresses the query rows of a head with 32-bit offsets
+        const bool lds_direct = ctx->prefill_variant != 1 && ((uint64_t)(L.q_len - 1) * L.q_stride_m + L.head_dim) * 2 < (1ull << 32);
         FaLaunchScope scope(ctx, lds_direct ? "flash_prefill_dma_kernel" : "flash_prefill_mfma_kernel", true);
         if (lds_direct) {
             auto kern = flash_prefill_dma_kernel<128, false, false>;
