@@ -255,3 +255,36 @@ def test_paged_decode_full_batch_of_32_ragged_sequences():
     pg.free()
     for b in (dq, dout):
         b.free()
+
+
+@pytest.mark.usefixtures("prefill_variant")
+@pytest.mark.parametrize("H,Hkv,D,bs,prefix,M", [
+    (6, 2, 128, 16, 333, 100),    # context ends inside a block and inside a key tile
+    (14, 2, 64, 48, 70, 37),      # block size not a power of two, head_dim 64
+    (8, 8, 128, 32, 0, 129),      # no prefix, one row into a second query tile
+    (4, 2, 128, 16, 2000, 32),    # a 32-row chunk after a long prefix: few query tiles, split over the keys
+])
+def test_paged_prefill_chunk_after_prefix(H, Hkv, D, bs, prefix, M):
+    """A prefill chunk attending a paged cache that already holds a prefix (sequence 1 of 3, random block
+    permutation), against the oracle over the gathered contiguous cache."""
+    announce("paged prefill chunk", H, Hkv, D, bs, prefix, M)
+    f = ctx()
+    rng = np.random.default_rng(prefix * 7 + M)
+    N = prefix + M
+    lens = [5, N, 40]
+    ks = [h16(rng.normal(size=(Hkv, n, D))) for n in lens]
+    vs = [h16(rng.normal(size=(Hkv, n, D))) for n in lens]
+    pg = Paged(f, rng, lens, Hkv, D, bs, extra_tokens=0)
+    pg.fill_from(ks, vs)
+    pg.upload()
+    q = h16(rng.normal(size=(H, M, D)))
+    dq, dout = f.array(q), f.zeros((M, H * D))
+    f.flash_prefill_paged(dq.arg(), pg.desc, 1, dout.arg(), True, prefix, H, N, M)
+    f.synchronize()
+    got = dout.download()
+    want = orc.sdpa_prefill(q, ks[1], vs[1], H, Hkv, D, M, N, prefix, N, causal=True, n_threads=8)  # token-major
+    assert np.all(np.isfinite(got))
+    assert max_abs(got, want) <= TOL
+    pg.free()
+    for b in (dq, dout):
+        b.free()
