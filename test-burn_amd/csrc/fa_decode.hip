@@ -31,8 +31,10 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
         const uint64_t slots = (uint64_t)(ctx->n_cus > 0 ? ctx->n_cus : 256);
         const uint32_t s_max = groups >= slots ? 1u : (uint32_t)(slots / groups);
         // Long partitions are cut further, into a whole number of workgroups per CU, so that a batch of ragged
-        // sequences (whose short members leave most of their partitions empty) still balances over the CUs.
-        const uint32_t long_chunk = 2u * NW * MBX * BK;  // two rounds of a workgroup
+        // sequences (whose short members leave most of their partitions empty) still balances over the CUs - but
+        // not too far: a workgroup costs about 5 us before and after its keys stream in at 31 KB per microsecond,
+        // which 768 keys (393 KB) do not amortise (C3: 62.9 us with <= 768 keys, 52.0 us with <= 1536).
+        const uint32_t long_chunk = 4u * NW * MBX * BK;  // 1536 keys: four rounds of a workgroup
         const uint32_t per_cu = ceil_div_u32(ceil_div_u32(bound, s_max), long_chunk);
         chunk = ceil_div_u32(ceil_div_u32(bound, s_max * per_cu), (uint32_t)BK) * BK;
         if (chunk < (uint32_t)(NW * BK)) chunk = NW * BK;

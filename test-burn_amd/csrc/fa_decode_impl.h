@@ -268,12 +268,18 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: tile addresses stay in SGPRs
     const int n = lane & 15, c = lane >> 4;  // MFMA column (head slot / key row) and 16-lane row
-    const uint32_t split = blockIdx.x, y = blockIdx.y, b = blockIdx.z;
+    // Consecutive workgroup ids go to consecutive XCDs (8). With the partition index taken straight from blockIdx.x
+    // and a partition count that is a multiple of 8 (or 4), partition p of EVERY sequence lands on the same XCD -
+    // and in a ragged batch the low partitions always exist while the high ones are mostly empty: some XCDs queue
+    // work while others idle (measured: 62 us with 12 partitions per sequence, 55 us with 11). Rotating the index
+    // by the head-group index spreads every sequence's partitions over all XCDs.
+    const uint32_t y = blockIdx.y, b = blockIdx.z;
+    const uint32_t split = (blockIdx.x + y + gridDim.y * b) % gridDim.x;
     const uint32_t gt = a.gt;
     const uint32_t kvh = y / a.sub_per_kv;
     const uint32_t head0 = y * gt;
     const uint32_t S = gridDim.x;
-    const uint32_t k0 = split * a.chunk;
+    uint32_t chunk = a.chunk, k0 = split * chunk;  // (a paged launch evens its partitions out once the length is known)
 
     const unsigned char *kbase;
     const __half *vbase;
@@ -366,9 +372,9 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
     // FUSED, wave 0 streams no blocks: it prepares the query operand and attends the new token.
     constexpr int KW = FUSED ? NW - 1 : NW;  // streaming waves
     const int sw = FUSED ? wave - 1 : wave;  // index among them (-1: none)
-    const uint32_t nb = a.chunk / BK;
-    const uint32_t wb0 = sw >= 0 ? nb - ((uint32_t)(KW - sw) * nb) / KW : 0u;
-    const uint32_t wb1 = sw >= 0 ? nb - ((uint32_t)(KW - 1 - sw) * nb) / KW : 0u;
+    uint32_t nb = chunk / BK;
+    uint32_t wb0 = sw >= 0 ? nb - ((uint32_t)(KW - sw) * nb) / KW : 0u;
+    uint32_t wb1 = sw >= 0 ? nb - ((uint32_t)(KW - 1 - sw) * nb) / KW : 0u;
     uint32_t cur = wb0;
 
     // A CU accepts vector memory requests in order and only as fast as its earlier ones complete, so anything
@@ -518,7 +524,18 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
     const uint32_t N = min(n_raw, min(a.capacity, a.kv_len_bound));
     const uint32_t nsplits = (N + a.chunk - 1) / a.chunk;
     if (split >= nsplits) return;  // uniform over the workgroup
-    const uint32_t k1 = min(N, k0 + a.chunk);
+    if (PAGED) {
+        // Nothing has been requested yet (a paged cache needs the length first), so the partitions of this
+        // sequence can still be made equal: the same number of them, none a few keys long. A short tail partition
+        // costs a workgroup's fixed time (launch, first requests, one memory latency, fold, store: about 5 us) for
+        // next to no keys, and in a ragged batch every sequence has one.
+        chunk = ((N + nsplits - 1) / nsplits + BK - 1) / BK * BK;
+        k0 = split * chunk, nb = chunk / BK;
+        wb0 = sw >= 0 ? nb - ((uint32_t)(KW - sw) * nb) / KW : 0u;
+        wb1 = sw >= 0 ? nb - ((uint32_t)(KW - 1 - sw) * nb) / KW : 0u;
+        cur = wb0;
+    }
+    const uint32_t k1 = min(N, k0 + chunk);
 
     // FUSED: row p is the new token. It is appended only if it lies inside the cache and the launch bound; the
     // cache rows of its partition end before it, and it is attended as a one-key block of its own.
