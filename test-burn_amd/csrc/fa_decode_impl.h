@@ -38,6 +38,7 @@
 // token as a one-key tile built from the rotated K / copied V, which one workgroup also stores into the cache.
 #pragma once
 #include "fa_internal.h"
+#include <type_traits>
 
 namespace fa_decode {
 
@@ -159,7 +160,7 @@ __device__ __forceinline__ void merge_and_store(const DecodeDev &a, uint32_t b, 
                                                 uint32_t S, int tid, float *sm /* NT * 6 floats */) {
     constexpr int CG = D / 4;    // float4 columns per head
     constexpr int RL = NT / CG;  // row lanes (12 at D = 128, 24 at D = 64)
-    constexpr int PPT = 17;      // partitions per thread per batch (102 VGPRs in flight)
+    constexpr int PPT_MAX = 17;  // partitions per thread in the largest batch (102 VGPRs in flight)
     const int gt = (int)a.gt;
     const int hpp = gt < RL ? gt : RL;  // heads per pass
     const int lph = RL / hpp;           // lanes per head
@@ -175,7 +176,12 @@ __device__ __forceinline__ void merge_and_store(const DecodeDev &a, uint32_t b, 
         float m_run = -1e30f, l_run = 0.0f;
         f4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
         if (active) {
-            for (uint32_t s0 = q; s0 < nsplits; s0 += lph * PPT) {
+            // One batch: all loads of up to PPT partitions are issued before the first is used (one memory round
+            // trip), then folded in partition order. The batch size is the smallest that covers what is left for
+            // lane 0 of a head: the clamped loads and the masked folds of a larger batch are not free (a coherent load
+            // never hits in the CU's cache, and 17 folds of 8 waves are over a microsecond).
+            auto batch = [&](auto ppt, uint32_t s0) {
+                constexpr int PPT = decltype(ppt)::value;
                 f4_t x[PPT];
                 f2_t ml[PPT];
 #pragma unroll
@@ -194,6 +200,19 @@ __device__ __forceinline__ void merge_and_store(const DecodeDev &a, uint32_t b, 
                     l_run = l_run * e1 + ls * e2;
                     acc = acc * e1 + x[k] * e2;
                     m_run = mn;
+                }
+            };
+            for (uint32_t s0 = q, done = 0; done < nsplits;) {  // `done` is uniform over the workgroup
+                const uint32_t left = (nsplits - done + lph - 1) / lph;
+                if (left > 8) {
+                    batch(std::integral_constant<int, PPT_MAX>{}, s0);
+                    s0 += lph * PPT_MAX, done += lph * PPT_MAX;
+                } else if (left > 4) {
+                    batch(std::integral_constant<int, 8>{}, s0);
+                    s0 += lph * 8, done += lph * 8;
+                } else {
+                    batch(std::integral_constant<int, 4>{}, s0);
+                    s0 += lph * 4, done += lph * 4;
                 }
             }
             float *slot = sm + (size_t)(r * CG + c) * 6;
