@@ -151,18 +151,20 @@ __device__ __forceinline__ f2_t ld_f2(const float *base, __amdgpu_buffer_rsrc_t 
     return *reinterpret_cast<const f2_t *>(base + elem);
 }
 
-// Merges the `nsplits` partial states of one (sequence, head group) and stores the normalised output.
+// Merges the partial states of one (sequence, head group) and stores the normalised output.
 // Thread (c, r): float4 column c of head r / lph, partitions (r % lph), +lph, ...; all of a thread's loads of a
 // batch are issued before the first is used, so a typical launch pays one memory round trip. An LDS pass folds
 // the lph lanes of a head.
-template <int D, bool COHERENT>
+// The workgroup has NTM threads and merges the heads [h_first, h_first + h_count) of the group.
+template <int D, bool COHERENT, int NTM>
 __device__ __forceinline__ void merge_and_store(const DecodeDev &a, uint32_t b, uint32_t y, uint32_t nsplits,
-                                                uint32_t S, int tid, float *sm /* NT * 6 floats */) {
-    constexpr int CG = D / 4;    // float4 columns per head
-    constexpr int RL = NT / CG;  // row lanes (12 at D = 128, 24 at D = 64)
+                                                uint32_t S, int tid, float *sm /* NTM * 6 floats, 16-byte aligned */,
+                                                int h_first, int h_count) {
+    constexpr int CG = D / 4;     // float4 columns per head
+    constexpr int RL = NTM / CG;  // row lanes
     constexpr int PPT_MAX = 17;  // partitions per thread in the largest batch (102 VGPRs in flight)
     const int gt = (int)a.gt;
-    const int hpp = gt < RL ? gt : RL;  // heads per pass
+    const int hpp = h_count < RL ? h_count : RL;  // heads per pass
     const int lph = RL / hpp;           // lanes per head
     const int c = tid % CG, r = tid / CG;
     const int hl = r / lph, q = r % lph;
@@ -170,20 +172,20 @@ __device__ __forceinline__ void merge_and_store(const DecodeDev &a, uint32_t b, 
     const float *acc_base = a.part_acc + base * D;
     const float *ml_base = a.part_ml + base * 2;
     const __amdgpu_buffer_rsrc_t rs_acc = make_rsrc(acc_base), rs_ml = make_rsrc(ml_base);
-    for (int h0 = 0; h0 < gt; h0 += hpp) {
+    for (int h0 = h_first; h0 < h_first + h_count; h0 += hpp) {
         const int h = h0 + hl;
-        const bool active = hl < hpp && h < gt;
+        const bool active = hl < hpp && h < h_first + h_count;
         float m_run = -1e30f, l_run = 0.0f;
         f4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (active) {
-            // One batch: all loads of up to PPT partitions are issued before the first is used (one memory round
-            // trip), then folded in partition order. The batch size is the smallest that covers what is left for
-            // lane 0 of a head: the clamped loads and the masked folds of a larger batch are not free (a coherent load
-            // never hits in the CU's cache, and 17 folds of 8 waves are over a microsecond).
-            auto batch = [&](auto ppt, uint32_t s0) {
-                constexpr int PPT = decltype(ppt)::value;
-                f4_t x[PPT];
-                f2_t ml[PPT];
+        // One batch: all loads of up to PPT partitions are issued before the first is used (one memory round
+        // trip), then folded in partition order. The batch size is the smallest that covers what is left for
+        // lane 0 of a head: the clamped loads and the masked folds of a larger batch are not free (a coherent load
+        // never hits in the CU's cache, and 17 folds of 8 waves are over a microsecond).
+        auto batch = [&](auto ppt, uint32_t s0) {
+            constexpr int PPT = decltype(ppt)::value;
+            f4_t x[PPT];
+            f2_t ml[PPT];
+            if (active) {
 #pragma unroll
                 for (int k = 0; k < PPT; ++k) {
                     const uint32_t s = min(s0 + k * lph, nsplits - 1);  // clamped; masked below
@@ -191,44 +193,54 @@ __device__ __forceinline__ void merge_and_store(const DecodeDev &a, uint32_t b, 
                     x[k] = ld_f4<COHERENT>(acc_base, rs_acc, row * D + c * 4);
                     ml[k] = ld_f2<COHERENT>(ml_base, rs_ml, row * 2);
                 }
+                // the batch's maximum first, then one weight per partition
+                float mb = m_run;
+#pragma unroll
+                for (int k = 0; k < PPT; ++k) mb = fmaxf(mb, s0 + k * lph < nsplits ? ml[k].x : -1e30f);
+                const float e0 = fast_exp2(m_run - mb);
+                l_run *= e0;
+                acc *= e0;
 #pragma unroll
                 for (int k = 0; k < PPT; ++k) {
-                    const bool ok = s0 + k * lph < nsplits;
-                    const float ms = ok ? ml[k].x : -1e30f, ls = ok ? ml[k].y : 0.0f;
-                    const float mn = fmaxf(m_run, ms);
-                    const float e1 = fast_exp2(m_run - mn), e2 = ok ? fast_exp2(ms - mn) : 0.0f;
-                    l_run = l_run * e1 + ls * e2;
-                    acc = acc * e1 + x[k] * e2;
-                    m_run = mn;
+                    const float w = s0 + k * lph < nsplits ? fast_exp2(ml[k].x - mb) : 0.0f;
+                    l_run += ml[k].y * w;
+                    acc += x[k] * w;
                 }
-            };
-            for (uint32_t s0 = q, done = 0; done < nsplits;) {  // `done` is uniform over the workgroup
-                const uint32_t left = (nsplits - done + lph - 1) / lph;
-                if (left > 8) {
-                    batch(std::integral_constant<int, PPT_MAX>{}, s0);
-                    s0 += lph * PPT_MAX, done += lph * PPT_MAX;
-                } else if (left > 4) {
-                    batch(std::integral_constant<int, 8>{}, s0);
-                    s0 += lph * 8, done += lph * 8;
-                } else {
-                    batch(std::integral_constant<int, 4>{}, s0);
-                    s0 += lph * 4, done += lph * 4;
-                }
+                m_run = mb;
             }
-            float *slot = sm + (size_t)(r * CG + c) * 6;
-            slot[0] = m_run, slot[1] = l_run, slot[2] = acc.x, slot[3] = acc.y, slot[4] = acc.z, slot[5] = acc.w;
+        };
+        for (uint32_t s0 = q, done = 0; done < nsplits;) {  // `done` is uniform over the workgroup
+            const uint32_t left = (nsplits - done + lph - 1) / lph;
+            if (left > 8) {
+                batch(std::integral_constant<int, PPT_MAX>{}, s0);
+                s0 += lph * PPT_MAX, done += lph * PPT_MAX;
+            } else if (left > 4) {
+                batch(std::integral_constant<int, 8>{}, s0);
+                s0 += lph * 8, done += lph * 8;
+            } else {
+                batch(std::integral_constant<int, 4>{}, s0);
+                s0 += lph * 4, done += lph * 4;
+            }
+        }
+        if (active) {
+            // per thread {m, l} in sm[0, 2 NTM) and the four sums in sm[2 NTM, 6 NTM): consecutive lanes, consecutive words
+            *reinterpret_cast<f2_t *>(sm + (size_t)(r * CG + c) * 2) = f2_t{m_run, l_run};
+            *reinterpret_cast<f4_t *>(sm + 2 * NTM + (size_t)(r * CG + c) * 4) = acc;
         }
         __syncthreads();
         if (active && q == 0) {
             float mstar = -1e30f;
-            for (int j = 0; j < lph; ++j) mstar = fmaxf(mstar, sm[(size_t)((r + j) * CG + c) * 6]);
-            float L = 0.0f, o[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 4
+            for (int j = 0; j < lph; ++j) mstar = fmaxf(mstar, sm[(size_t)((r + j) * CG + c) * 2]);
+            float L = 0.0f;
+            f4_t o = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 4
             for (int j = 0; j < lph; ++j) {
-                const float *sl = sm + (size_t)((r + j) * CG + c) * 6;
-                const float w = fast_exp2(sl[0] - mstar);
-                L += sl[1] * w;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) o[i] += sl[2 + i] * w;
+                const size_t t = (size_t)((r + j) * CG + c);
+                const f2_t mlj = *reinterpret_cast<const f2_t *>(sm + t * 2);
+                const float w = fast_exp2(mlj.x - mstar);
+                L += mlj.y * w;
+                o += *reinterpret_cast<const f4_t *>(sm + 2 * NTM + t * 4) * w;
             }
             const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 1.0f;
             const uint32_t head = y * gt + h;
@@ -781,20 +793,25 @@ __global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
     }
     __syncthreads();
     if (!sm_last) return;
-    merge_and_store<D, true>(a, b, y, nsplits, S, tid, reinterpret_cast<float *>(smem));
+    merge_and_store<D, true, NT>(a, b, y, nsplits, S, tid, reinterpret_cast<float *>(smem), 0, (int)gt);
     if (tid == 0)  // ready for the next launch
         __hip_atomic_store(&a.counters[(size_t)b * gridDim.y + y], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// One small workgroup per head (blockIdx.x): the merge is a launch gap plus the time a CU needs to request the
+// partials, so the requests are spread over as many CUs as there are heads (measured on 24 heads x 32 partitions:
+// one 512-thread workgroup per head group 4.3 us and 2444 decode steps/s; per head with 512 / 256 / 128 / 64
+// threads 2497 / 2590 / 2622 / 2578 steps/s).
+constexpr int NT_MERGE = 128;
 template <int D>
-__global__ void __launch_bounds__(NT) flash_decode_merge_kernel(DecodeDev a, uint32_t S) {
-    __shared__ float sm[NT * 6];
+__global__ void __launch_bounds__(NT_MERGE) flash_decode_merge_kernel(DecodeDev a, uint32_t S) {
+    __shared__ __attribute__((aligned(16))) float sm[NT_MERGE * 6];
     const uint32_t y = blockIdx.y, b = blockIdx.z;
     uint32_t N = a.d_len ? a.d_len[(size_t)b * a.d_len_stride] + a.kv_len_add : a.kv_len;
     N = min(N, min(a.capacity, a.kv_len_bound));
     const uint32_t nsplits = (N + a.chunk - 1) / a.chunk;
     if (nsplits <= 1) return;  // written directly by the partition kernel
-    merge_and_store<D, false>(a, b, y, nsplits, S, threadIdx.x, sm);
+    merge_and_store<D, false, NT_MERGE>(a, b, y, nsplits, S, threadIdx.x, sm, (int)blockIdx.x, 1);
 }
 
 enum Mode { MODE_PLAIN = 0, MODE_PAGED = 1, MODE_SAGE = 2, MODE_FUSED = 3, MODE_FUSED_PAGED = 4 };
@@ -868,7 +885,7 @@ fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
     }
     if (!a.merge_in_kernel && grid.x > 1) {
         FaLaunchScope scope(ctx, "flash_decode_merge_kernel", true);
-        scope.launch((flash_decode_merge_kernel<D>), dim3(1, grid.y, grid.z), dim3(NT), 0, a, grid.x);
+        scope.launch((flash_decode_merge_kernel<D>), dim3(a.gt, grid.y, grid.z), dim3(NT_MERGE), 0, a, grid.x);
         FA_TRY(scope.finish());
     }
     return FA_OK;

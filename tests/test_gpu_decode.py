@@ -68,7 +68,7 @@ def test_decode_ragged_lengths_and_splits(N, D, H, Hkv):
             assert np.all(np.isfinite(got)), (kps, merge)
             assert max_abs(got, want) <= TOL, (kps, merge)
     finally:
-        f.set_decode_variant(0, 0)
+        f.set_decode_variant()
 
 
 def test_decode_known_answer_fixture():
@@ -253,7 +253,7 @@ def test_fused_decode_step_equals_separate_ops(H, Hkv, D, mode, base, layer, ste
             for b in (dq, dk, dv, kc_a, vc_a, qr_a, out_a, kc_b, vc_b, qr_b, out_b, kc_c, vc_c, out_c, dpos):
                 b.free()
     finally:
-        f.set_decode_variant(0, 0)
+        f.set_decode_variant()
 
 
 def test_fused_step_errors_and_overflow_guard():
@@ -279,9 +279,11 @@ def test_fused_step_errors_and_overflow_guard():
     assert not kc.download().any()
 
 
-def test_in_kernel_merge_is_bit_identical_to_merge_kernel_over_many_launches():
-    """The merge by the last-arriving workgroup reads partials written by other workgroups of the same launch;
-    it must give the same bits as the two-launch merge, launch after launch."""
+def test_in_kernel_merge_equals_merge_kernel_over_many_launches():
+    """The merge by the last-arriving workgroup reads partials written by other workgroups of the same launch. It
+    folds the same partials as the two-launch merge in another f32 order (one workgroup per head group there, one
+    per head here), so the outputs agree to one f16 unit in the last place; and it is deterministic: repeated
+    launches give the same bits (a stale partial would show in either check)."""
     announce("merge stress")
     f = ctx()
     rng = np.random.default_rng(123)
@@ -298,9 +300,16 @@ def test_in_kernel_merge_is_bit_identical_to_merge_kernel_over_many_launches():
                 f.set_decode_variant(kps, 1)
                 f.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), oa.arg(), True, n - 1, H, D, n, 1)
                 f.set_decode_variant(kps, 0)
+                a = oa.download().astype(np.float32)
+                first = None
                 for _ in range(3):
                     f.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), ob.arg(), True, n - 1, H, D, n, 1)
                     f.synchronize()
-                    assert np.array_equal(bits(oa.download()), bits(ob.download())), (kps, n)
+                    got = ob.download()
+                    if first is None:
+                        first = bits(got)
+                    assert np.array_equal(bits(got), first), (kps, n)
+                    g = got.astype(np.float32)
+                    assert np.all(np.abs(g - a) <= np.maximum(np.abs(a), 2.0 ** -14) * 2.0 ** -10), (kps, n)
     finally:
-        f.set_decode_variant(0, 0)
+        f.set_decode_variant()
