@@ -267,12 +267,12 @@ def bench_prefill(f, args):
         sys.exit("parity check failed: cache_bit_exact=%s prefill_max_abs_err=%g" % (cache_ok, err))
 
 
-def _finish_secondary(f, args, name, workload, kernel, bytes_per_launch, dt, parity, extra=None):
+def _finish_secondary(f, args, name, workload, kernel, bytes_per_launch, dt, parity, extra=None, unit="layer-steps/s"):
     n, ms = f.profile_query(kernel)
     avg_s = ms / 1e3 / max(1, n)
     achieved = bytes_per_launch / avg_s / 1e9
     result = {
-        "metric": name, "value": args.steps / dt, "unit": "layer-steps/s", "n_gpus": 1, "steps": args.steps,
+        "metric": name, "value": args.steps / dt, "unit": unit, "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic", "config": {"workload": workload},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -330,6 +330,47 @@ def bench_small_decode(f, args):
                       "qwen2.5-0.5b single-layer decode step: RoPE + KV append + flash decode, batch 1, H14/Hkv2/D64, "
                       "kv_len 1025, eager launches (profiling events on)", "fused_rope_append_decode_kernel", nbytes, dt,
                       {"cache_bit_exact": ok, "decode_max_abs_err": err})
+    f.profile_enable(False)
+
+
+def bench_kv_growth(f, args):
+    """KV-cache growth of a Llama-3.2-3B session at 8448 tokens: the first 8448 rows of every head of all 56 cache
+    tensors [8, 8448, 128] move into tensors of twice the capacity (one batched prefix copy)."""
+    import orc
+    L, Hkv, D, pos = 28, 8, 128, 8448
+    new_cap = fa.grown_capacity(pos, pos + 1, 131072)
+    rng = np.random.default_rng(0xF0DD + 6)
+    base = rng.standard_normal((Hkv, pos, D), dtype=np.float32).astype(np.float16)
+    old, new = [], []
+    for i in range(2 * L):
+        host = base if i == 0 else np.roll(base, i, axis=1)
+        old.append(f.array(host))
+        new.append(f.zeros((Hkv, new_cap, D)))
+    srcs, dsts = [b.arg() for b in old], [b.arg() for b in new]
+
+    def step(i):
+        f.kv_prefix_copy_batch(srcs, dsts, pos)
+
+    step(0)
+    f.synchronize()
+    want = np.zeros((Hkv, new_cap, D), np.float16)
+    orc.kv_prefix_copy(np.roll(base, 5, axis=1), want, pos)
+    ok = bool(np.array_equal(new[5].download().view(np.uint16), want.view(np.uint16)))
+    for i in range(args.warmup):
+        step(i)
+    f.synchronize()
+    f.profile_reset()
+    f.profile_enable(True)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    nbytes = 2.0 * 2 * L * Hkv * pos * D * 2  # read + written
+    _finish_secondary(f, args, "KV-cache growth copies/s + achieved HBM GB/s, Llama-3.2-3B caches @8448 tokens",
+                      "llama3.2-3b KV-cache growth %d -> %d rows: per-head prefix copy of 56 tensors [8, 8448, 128] f16, "
+                      "one launch (profiling events on)" % (pos, new_cap), "kv_prefix_copy_vec_kernel", nbytes, dt,
+                      {"copy_bit_exact": ok}, unit="growths/s")
     f.profile_enable(False)
 
 
@@ -464,7 +505,8 @@ def bench_sage_decode(f, args):
 
 
 SECONDARY = {"llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
-             "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode}
+             "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
+             "llama3b_kv_growth": bench_kv_growth}
 
 
 def main():

@@ -314,6 +314,44 @@ fa_status fa_paged_gather(fa_ctx *ctx, const fa_paged_kv *cache, uint32_t seq_in
                           void *k_out, void *v_out, uint32_t out_capacity);
 
 /* ---------------------------------------------------------------------------------------------
+ * KV-cache prefix copies: the executor's second use of the cache layout. The reference moves the first
+ * `prefix_len` rows of every head with one blit per head in three places, all the same strided copy:
+ *   capture_kv_prefix_snapshot  live [heads, cap, D]  -> snapshot [heads, prefix_len, D]  (src/model/executor.rs:1136-1261)
+ *   restore_kv_prefix_snapshot  snapshot              -> live                             (src/model/executor.rs:1263-1350)
+ *   preserve_kv_cache (growth)  old [heads, old_cap, D] -> new [heads, new_cap, D], prefix_len = current_pos
+ *                                                                                        (src/model/executor.rs:2437-2513)
+ * Here it is one launch for all heads (and, in the batch form, all tensors of a model).
+ * ------------------------------------------------------------------------------------------- */
+
+/* Copies rows [0, prefix_len) of every head of src into dst. Both are rank-3 [heads, capacity, head_dim] with
+ * contiguous strides [capacity*head_dim, head_dim, 1] (kv_tensor_copy_shape, src/model/executor.rs:1105-1134);
+ * capacities may differ, heads, head_dim and dtype must match and prefix_len must fit both capacities, else
+ * FA_ERR_INVALID_SHAPE. Rows at and past prefix_len of dst are not touched. prefix_len 0 is a no-op. */
+fa_status fa_kv_prefix_copy(fa_ctx *ctx, const fa_tensor_arg *src, const fa_tensor_arg *dst, size_t prefix_len);
+
+/* The same copy for n tensor pairs in as few launches as possible (a model's k_cache_i / v_cache_i of all
+ * layers). src[i] is copied to dst[i]; every pair is validated as above before anything is enqueued. */
+fa_status fa_kv_prefix_copy_batch(fa_ctx *ctx, const fa_tensor_arg *src, const fa_tensor_arg *dst, uint32_t n,
+                                  size_t prefix_len);
+
+/* Capacity policy of the cache (host arithmetic, no GPU work).
+ * fa_align_capacity: next multiple of 128, 0 -> 128 (ContextConfig::align_capacity, src/model/context.rs:213-219).
+ * fa_grown_capacity: the capacity ensure_kv_capacity allocates when `required_len` exceeds `allocated`
+ * (src/model/executor.rs:2354-2382): growth_factor <= 0 selects FullReserve (max_context_len), otherwise
+ * max((usize)(allocated * growth_factor), required_len) capped at max_context_len; the result is then aligned (and
+ * may therefore exceed max_context_len, as in the reference). Returns `allocated` when it already suffices and 0
+ * when required_len > max_context_len (the reference's InvalidOperation). */
+size_t fa_align_capacity(size_t capacity);
+size_t fa_grown_capacity(size_t allocated, size_t required_len, size_t max_context_len, float growth_factor);
+
+/* Paged form: copies whole physical blocks inside the pools, K and V: block d_src_ids[i] -> d_dst_ids[i] for
+ * i < n_pairs (device arrays). Sharing a prefix between sequences is a block-table edit (no copy); this call
+ * is for the one partly filled tail block a fork has to own (copy-on-write) and for compaction. Pairs with an id
+ * outside [0, n_blocks) or with src == dst are skipped. No counterpart in the reference. */
+fa_status fa_paged_copy_blocks(fa_ctx *ctx, const fa_paged_kv *cache, const int32_t *d_src_ids,
+                               const int32_t *d_dst_ids, uint32_t n_pairs);
+
+/* ---------------------------------------------------------------------------------------------
  * SageAttention-style int8 Q/K decode (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170 - prose only in
  * the reference). K is mean-smoothed over the sequence per (kv head, channel), then quantised per block
  * of 32 tokens: scale = max|k - mean| / 127 stored as f16, k_q = rint((k - mean)/scale) in [-127,127].

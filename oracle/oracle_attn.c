@@ -554,6 +554,55 @@ void orc_paged_scatter(orc_f16 *pool, const int32_t *block_table, uint32_t n_kv_
         }
 }
 
+void orc_paged_copy_blocks(orc_f16 *pool, uint32_t n_blocks, uint32_t n_kv_heads, uint32_t block_size,
+                           uint32_t head_dim, const int32_t *src_ids, const int32_t *dst_ids, uint32_t n_pairs) {
+    const size_t block_elems = (size_t)n_kv_heads * block_size * head_dim;
+    for (uint32_t i = 0; i < n_pairs; ++i) {
+        const int32_t s = src_ids[i], d = dst_ids[i];
+        if (s < 0 || d < 0 || (uint32_t)s >= n_blocks || (uint32_t)d >= n_blocks || s == d) continue;
+        memcpy(pool + (size_t)d * block_elems, pool + (size_t)s * block_elems, block_elems * sizeof(orc_f16));
+    }
+}
+
+/* ------------------------------------------------------------------ KV prefix copies, capacity policy */
+
+/* src/model/executor.rs:1195-1212 / :1296-1318 / :2494-2505: for h in 0..heads: blit bytes_per_head bytes from
+ * src + h*src_capacity*head_dim*elem to dst + h*dst_capacity*head_dim*elem. */
+int orc_kv_prefix_copy(const void *src, void *dst, size_t heads, size_t src_capacity, size_t dst_capacity,
+                       size_t head_dim, size_t elem_bytes, size_t prefix_len) {
+    if (prefix_len > src_capacity || prefix_len > dst_capacity) return -1;
+    const size_t bytes_per_head = prefix_len * head_dim * elem_bytes;
+    for (size_t h = 0; h < heads; ++h) {
+        const size_t src_head_offset = h * src_capacity * head_dim * elem_bytes;
+        const size_t dst_head_offset = h * dst_capacity * head_dim * elem_bytes;
+        memcpy((unsigned char *)dst + dst_head_offset, (const unsigned char *)src + src_head_offset, bytes_per_head);
+    }
+    return 0;
+}
+
+/* src/model/context.rs:213-219 */
+size_t orc_align_capacity(size_t capacity) {
+    const size_t ALIGN = 128;
+    if (capacity == 0) return ALIGN;
+    return (capacity + ALIGN - 1) / ALIGN * ALIGN;
+}
+
+/* src/model/executor.rs:2354-2382 */
+size_t orc_grown_capacity(size_t allocated, size_t required_len, size_t max_context_len, float growth_factor) {
+    if (required_len <= allocated) return allocated;       /* :2354 capacity already sufficient */
+    if (required_len > max_context_len) return 0;          /* :2363 InvalidOperation */
+    size_t new_capacity;
+    if (growth_factor <= 0.0f) {
+        new_capacity = max_context_len;                     /* FullReserve, :2372 */
+    } else {
+        float g = (float)allocated * growth_factor;         /* :2374 `as usize` saturates */
+        size_t grown = g <= 0.0f ? 0 : (g >= 18446744073709551615.0f ? SIZE_MAX : (size_t)g);
+        if (grown < required_len) grown = required_len;     /* .max(required_len) */
+        new_capacity = grown < max_context_len ? grown : max_context_len;
+    }
+    return orc_align_capacity(new_capacity);                /* :2381 */
+}
+
 /* ------------------------------------------------------------------ Sage-style int8 Q/K */
 
 void orc_sage_k_mean(const orc_f16 *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim, uint32_t kv_len,

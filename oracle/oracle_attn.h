@@ -32,6 +32,13 @@
  *   orc_paged_*               no reference counterpart; pinned by gather(paged) == contiguous
  *   orc_sage_*                PARITY UNPINNED: the reference holds only a prose sketch (docs/SAGE.md);
  *                             pinned by softmax shift identity and error vs f16 SDPA
+ *   orc_align_capacity        pinned: the reference's own vectors (src/model/context.rs:318-323)
+ *   orc_grown_capacity        no reference test; pinned by hand-worked cases of the formula at
+ *                             src/model/executor.rs:2371-2382 and by its invariants (aligned, >= required,
+ *                             monotone in required)
+ *   orc_kv_prefix_copy        no reference test; a byte copy, pinned by brute-force index checks and by the
+ *                             snapshot -> clobber -> restore round trip
+ *   orc_paged_copy_blocks     no reference counterpart; pinned by gather(fork) == gather(parent) on the prefix
  */
 #ifndef ORACLE_ATTN_H
 #define ORACLE_ATTN_H
@@ -133,6 +140,24 @@ void orc_paged_gather(const orc_f16 *pool, const int32_t *block_table, uint32_t 
 void orc_paged_scatter(orc_f16 *pool, const int32_t *block_table, uint32_t n_kv_heads, uint32_t block_size,
                        uint32_t head_dim, uint32_t pos_begin, uint32_t pos_end, uint32_t in_capacity,
                        const orc_f16 *in /*[n_kv_heads,in_capacity,head_dim]*/);
+
+/* Physical block copies inside one pool: block src_ids[i] -> dst_ids[i]; pairs with an id outside [0, n_blocks)
+ * or with src == dst are skipped (no reference counterpart). */
+void orc_paged_copy_blocks(orc_f16 *pool, uint32_t n_blocks, uint32_t n_kv_heads, uint32_t block_size,
+                           uint32_t head_dim, const int32_t *src_ids, const int32_t *dst_ids, uint32_t n_pairs);
+
+/* KV prefix copy: rows [0, prefix_len) of every head, src [heads, src_capacity, head_dim] -> dst [heads,
+ * dst_capacity, head_dim], elements of elem_bytes bytes: the per-head blits of capture_kv_prefix_snapshot
+ * (src/model/executor.rs:1195-1212, dst_capacity = prefix_len), restore_kv_prefix_snapshot (:1296-1318,
+ * src_capacity = prefix_len) and growth (:2494-2505, prefix_len = current_pos). Returns 0, or -1 when prefix_len
+ * exceeds a capacity (kv_tensor_copy_shape, :1115-1120) and nothing is copied. */
+int orc_kv_prefix_copy(const void *src, void *dst, size_t heads, size_t src_capacity, size_t dst_capacity,
+                       size_t head_dim, size_t elem_bytes, size_t prefix_len);
+/* ContextConfig::align_capacity (src/model/context.rs:213-219). */
+size_t orc_align_capacity(size_t capacity);
+/* New capacity chosen by ensure_kv_capacity (src/model/executor.rs:2354-2382); growth_factor <= 0 = FullReserve.
+ * `allocated` if it suffices, 0 if required_len > max_context_len. */
+size_t orc_grown_capacity(size_t allocated, size_t required_len, size_t max_context_len, float growth_factor);
 
 /* Sage-style int8 Q/K (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170).
  * K smoothing: subtract per-(head, channel) mean over the sequence (f32), quantise per block of

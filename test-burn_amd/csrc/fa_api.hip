@@ -624,6 +624,107 @@ extern "C" fa_status fa_paged_gather(fa_ctx *ctx, const fa_paged_kv *cache, uint
     return fa_launch_paged_gather(ctx, cache, seq_index, seq_len, k_out, v_out, out_capacity);
 }
 
+// ------------------------------------------------------------------------------------------------ KV prefix copies
+
+static size_t dtype_bytes(uint32_t dtype) {
+    switch (dtype) {
+        case FA_DTYPE_F64: return 8;
+        case FA_DTYPE_F32: case FA_DTYPE_I32: case FA_DTYPE_U32: return 4;
+        case FA_DTYPE_F16: case FA_DTYPE_BF16: case FA_DTYPE_I16: case FA_DTYPE_U16: return 2;
+        case FA_DTYPE_I8: case FA_DTYPE_U8: return 1;
+        default: return 0;
+    }
+}
+
+// kv_tensor_copy_shape (src/model/executor.rs:1105-1134): rank 3, prefix within capacity, contiguous strides.
+static fa_status kv_copy_shape(const fa_tensor_arg *t, const char *name, size_t prefix_len) {
+    if (!t->buffer) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: KV tensor '%s' has no backing buffer", name);
+    if (t->rank != 3)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: KV tensor '%s' must be rank-3 for prefix caching, got rank %u", name, t->rank);
+    if (prefix_len > t->dims[1])
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: KV tensor '%s' prefix_len %zu exceeds capacity %zu", name, prefix_len, t->dims[1]);
+    if (t->strides[0] != t->dims[1] * t->dims[2] || t->strides[1] != t->dims[2] || t->strides[2] != 1)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: KV tensor '%s' has unsupported strides [%zu, %zu, %zu], expected [%zu, %zu, 1]",
+                       name, t->strides[0], t->strides[1], t->strides[2], t->dims[1] * t->dims[2], t->dims[2]);
+    if (dtype_bytes(t->dtype) == 0) return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "Unsupported dtype %u for KV tensor '%s'", t->dtype, name);
+    return FA_OK;
+}
+
+extern "C" fa_status fa_kv_prefix_copy_batch(fa_ctx *ctx, const fa_tensor_arg *src, const fa_tensor_arg *dst, uint32_t n,
+                                             size_t prefix_len) {
+    FA_NEED(ctx, "ctx");
+    if (n == 0) return FA_OK;
+    FA_NEED(src, "src");
+    FA_NEED(dst, "dst");
+    for (uint32_t i = 0; i < n; ++i) {  // everything is checked before anything is enqueued
+        FA_TRY(kv_copy_shape(&src[i], "src", prefix_len));
+        FA_TRY(kv_copy_shape(&dst[i], "dst", prefix_len));
+        if (src[i].dtype != dst[i].dtype)
+            return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: KV tensor dtype mismatch during prefix copy: src=%u dst=%u", src[i].dtype, dst[i].dtype);
+        if (src[i].dims[0] != dst[i].dims[0] || src[i].dims[2] != dst[i].dims[2])
+            return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: KV tensor shape mismatch during prefix copy: src=[%zu, %zu, %zu], dst=[%zu, %zu, %zu]",
+                           src[i].dims[0], src[i].dims[1], src[i].dims[2], dst[i].dims[0], dst[i].dims[1], dst[i].dims[2]);
+    }
+    if (prefix_len == 0) return FA_OK;
+    // consecutive pairs of one geometry share a launch
+    uint32_t i = 0;
+    while (i < n) {
+        KvPrefixCopyLaunch L;
+        const size_t eb = dtype_bytes(src[i].dtype);
+        L.heads = (uint32_t)src[i].dims[0];
+        L.src_pitch = (uint64_t)src[i].strides[0] * eb, L.dst_pitch = (uint64_t)dst[i].strides[0] * eb;
+        L.bytes_per_head = (uint64_t)prefix_len * src[i].dims[2] * eb;
+        if (src[i].dims[0] > 65535) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %zu heads", src[i].dims[0]);
+        L.n = 0;
+        while (i < n && L.n < PREFIX_COPY_MAX_TENSORS && src[i].dims[0] == L.heads && dtype_bytes(src[i].dtype) == eb &&
+               (uint64_t)src[i].strides[0] * eb == L.src_pitch && (uint64_t)dst[i].strides[0] * eb == L.dst_pitch &&
+               (uint64_t)prefix_len * src[i].dims[2] * eb == L.bytes_per_head) {
+            L.src[L.n] = static_cast<const char *>(src[i].buffer) + src[i].offset;
+            L.dst[L.n] = static_cast<char *>(dst[i].buffer) + dst[i].offset;
+            ++L.n, ++i;
+        }
+        FA_TRY(fa_launch_kv_prefix_copy(ctx, L));
+    }
+    return FA_OK;
+}
+
+extern "C" fa_status fa_kv_prefix_copy(fa_ctx *ctx, const fa_tensor_arg *src, const fa_tensor_arg *dst, size_t prefix_len) {
+    FA_NEED(src, "src");
+    FA_NEED(dst, "dst");
+    return fa_kv_prefix_copy_batch(ctx, src, dst, 1, prefix_len);
+}
+
+extern "C" size_t fa_align_capacity(size_t capacity) {
+    const size_t align = 128;
+    if (capacity == 0) return align;
+    return (capacity + align - 1) / align * align;
+}
+
+extern "C" size_t fa_grown_capacity(size_t allocated, size_t required_len, size_t max_context_len, float growth_factor) {
+    if (required_len <= allocated) return allocated;
+    if (required_len > max_context_len) return 0;
+    size_t cap;
+    if (growth_factor <= 0.0f) {
+        cap = max_context_len;
+    } else {
+        const float grown_f = (float)allocated * growth_factor;  // `as usize` saturates
+        size_t grown = grown_f <= 0.0f ? 0 : grown_f >= 18446744073709551615.0f ? SIZE_MAX : (size_t)grown_f;
+        if (grown < required_len) grown = required_len;
+        cap = grown < max_context_len ? grown : max_context_len;
+    }
+    return fa_align_capacity(cap);
+}
+
+extern "C" fa_status fa_paged_copy_blocks(fa_ctx *ctx, const fa_paged_kv *cache, const int32_t *d_src_ids,
+                                          const int32_t *d_dst_ids, uint32_t n_pairs) {
+    FA_NEED(ctx, "ctx");
+    FA_TRY(check_paged(cache));
+    if (n_pairs == 0) return FA_OK;
+    FA_NEED(d_src_ids, "d_src_ids");
+    FA_NEED(d_dst_ids, "d_dst_ids");
+    return fa_launch_paged_copy_blocks(ctx, cache, d_src_ids, d_dst_ids, n_pairs);
+}
+
 // ------------------------------------------------------------------------------------------------ FlashAttention
 
 struct KvLayout {

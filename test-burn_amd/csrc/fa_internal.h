@@ -155,6 +155,18 @@ fa_status fa_launch_u32_add(fa_ctx *ctx, uint32_t *vals, uint32_t n, uint32_t de
 fa_status fa_launch_paged_gather(fa_ctx *ctx, const fa_paged_kv *c, uint32_t seq_index, uint32_t seq_len, void *k_out,
                                  void *v_out, uint32_t out_capacity);
 
+// Strided per-head prefix copy of up to PREFIX_COPY_MAX_TENSORS tensors of one geometry (pointers already offset).
+constexpr uint32_t PREFIX_COPY_MAX_TENSORS = 64;
+struct KvPrefixCopyLaunch {
+    const void *src[PREFIX_COPY_MAX_TENSORS];
+    void *dst[PREFIX_COPY_MAX_TENSORS];
+    uint32_t n, heads;
+    uint64_t src_pitch, dst_pitch, bytes_per_head;
+};
+fa_status fa_launch_kv_prefix_copy(fa_ctx *ctx, const KvPrefixCopyLaunch &l);
+fa_status fa_launch_paged_copy_blocks(fa_ctx *ctx, const fa_paged_kv *c, const int32_t *src_ids, const int32_t *dst_ids,
+                                      uint32_t n_pairs);
+
 fa_status fa_launch_sage_k_mean(fa_ctx *ctx, const void *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim,
                                 uint32_t kv_len, float *mean_out);
 fa_status fa_launch_sage_quantize_k(fa_ctx *ctx, const void *k, const float *mean, uint32_t n_kv_heads,

@@ -105,6 +105,11 @@ PROTOTYPES = {
     "fa_flash_decode_paged": [_vp, _PT, C.POINTER(PagedKv), _PT, _u32, _u32, _u32],
     "fa_flash_prefill_paged": [_vp, _PT, C.POINTER(PagedKv), _u32, _PT, _i, _u32, _u32, _u32, _u32],
     "fa_paged_gather": [_vp, C.POINTER(PagedKv), _u32, _u32, _vp, _vp, _u32],
+    "fa_paged_copy_blocks": [_vp, C.POINTER(PagedKv), _vp, _vp, _u32],
+    "fa_kv_prefix_copy": [_vp, _PT, _PT, _sz],
+    "fa_kv_prefix_copy_batch": [_vp, _PT, _PT, _u32, _sz],
+    "fa_align_capacity": [_sz],
+    "fa_grown_capacity": [_sz, _sz, _sz, C.c_float],
     "fa_sage_k_mean": [_vp, _vp, _u32, _u32, _u32, _u32, _vp],
     "fa_sage_quantize_k": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _vp, _vp],
     "fa_sage_quantize_q": [_vp, _vp, _u32, _u32, _vp, _vp],
@@ -112,9 +117,18 @@ PROTOTYPES = {
     "fa_device_info": [_vp, C.c_char_p, _sz, C.POINTER(_u32), C.POINTER(C.c_uint64)],
 }
 _RESTYPES = {"fa_status_name": C.c_char_p, "fa_last_error_string": C.c_char_p, "fa_version": C.c_char_p,
-             "fa_ctx_stream": _vp, "fa_is_capturing": _i}
+             "fa_ctx_stream": _vp, "fa_is_capturing": _i, "fa_align_capacity": _sz, "fa_grown_capacity": _sz}
 
 _lib = None
+
+
+def align_capacity(capacity):
+    return load().fa_align_capacity(capacity)
+
+
+def grown_capacity(allocated, required_len, max_context_len, growth_factor=2.0):
+    """0 = required_len exceeds max_context_len (the reference raises InvalidOperation there)."""
+    return load().fa_grown_capacity(allocated, required_len, max_context_len, growth_factor)
 
 
 def load():
@@ -332,6 +346,20 @@ class Foundry:
 
     def paged_gather(self, cache, seq_index, seq_len, k_out, v_out, out_capacity):
         check(self.lib.fa_paged_gather(self.h, C.byref(cache), seq_index, seq_len, k_out.ptr, v_out.ptr, out_capacity))
+
+    def paged_copy_blocks(self, cache, src_ids, dst_ids, n_pairs):
+        """src_ids / dst_ids: device i32 buffers."""
+        check(self.lib.fa_paged_copy_blocks(self.h, C.byref(cache), src_ids.ptr, dst_ids.ptr, n_pairs))
+
+    def kv_prefix_copy(self, src, dst, prefix_len):
+        """src, dst: TensorArg [heads, capacity, head_dim] (snapshot, restore and growth are this one copy)."""
+        check(self.lib.fa_kv_prefix_copy(self.h, C.byref(src), C.byref(dst), prefix_len))
+
+    def kv_prefix_copy_batch(self, srcs, dsts, prefix_len):
+        n = len(srcs)
+        assert n == len(dsts)
+        sa, da = (TensorArg * max(n, 1))(*srcs), (TensorArg * max(n, 1))(*dsts)
+        check(self.lib.fa_kv_prefix_copy_batch(self.h, sa, da, n, prefix_len))
 
     def sage_k_mean(self, k, n_kv_heads, capacity, head_dim, kv_len, mean_out):
         check(self.lib.fa_sage_k_mean(self.h, k.ptr, n_kv_heads, capacity, head_dim, kv_len, mean_out.ptr))

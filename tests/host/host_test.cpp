@@ -1,4 +1,4 @@
-// Exercises the C++ host mirror (test-burn_amd/host/foundry.hpp) and, through it, the C ABI, in the shape of the
+// Exercises the C++ host mirror (test-burn_amd/host/foundry.hpp, kv_session.hpp) and, through it, the C ABI, in the shape of the
 // reference's own tests for this path:
 //   tests/kv_prep_fused.rs:249-267            run_fused_parity(seq, offset, max_seq, heads, kv_heads, head_dim)
 //   tests/flashattention_decode_parity.rs     LCG inputs (seeds 1, 7, 42), decode vs a CPU reference
@@ -12,6 +12,7 @@
 #include <functional>
 
 #include "foundry.hpp"
+#include "kv_session.hpp"
 extern "C" {
 #include "oracle_attn.h"
 }
@@ -88,6 +89,68 @@ static void test_steps_compile_against_interpolated_names() {
     FlashAttentionStep fa_step{"q_rot", "k_cache_{i}", "v_cache_{i}", "attn_out"};
     auto c2 = fa_step.compile(b, s);
     EXPECT(s.len() == 9 && std::string(c2[0]->name()) == "FlashAttention");  // cache names are shared symbols
+}
+
+// src/model/context.rs:286-323 (test_context_config_priority, test_alignment) and the defaults at :42-49.
+static void test_capacity_policy() {
+    const size_t in[] = {0, 1, 127, 128, 129, 200}, want[] = {128, 128, 128, 128, 256, 256};
+    for (int i = 0; i < 6; ++i) EXPECT(ContextConfig::align_capacity(in[i]) == want[i]);
+    EXPECT(ContextConfig::from_limits(4096, 0).max_context_len == 4096);     // default to the model maximum
+    EXPECT(ContextConfig::from_limits(4096, 2048).max_context_len == 2048);  // an override acts as a cap
+    EXPECT(ContextConfig::from_limits(4096, 1024).max_context_len == 1024);
+    EXPECT(ContextConfig::from_limits(4096, 8192).max_context_len == 4096);  // never above the model
+    EXPECT(ContextConfig::from_limits(0, 0).max_context_len == 2048);
+    EXPECT(ContextConfig::from_limits(131072, 0).allocated_capacity == 2048);  // GrowOnDemand { initial: 2048 }
+    EXPECT(ContextConfig::from_limits(1000, 0).allocated_capacity == 1024);    // min(initial, max), aligned
+    EXPECT(ContextConfig::from_limits(5000, 0, GrowthStrategy::FullReserve()).allocated_capacity == 5120);
+    for (size_t a : {128u, 2048u, 8448u})
+        for (size_t r : {1u, 2049u, 5000u, 9000u, 70000u})
+            for (float g : {0.0f, 1.5f, 2.0f}) EXPECT(fa_grown_capacity(a, r, 65536, g) == orc_grown_capacity(a, r, 65536, g));
+    KvCopyShape s{};
+    Tensor t;
+    t.dims = {8, 256, 128}, t.strides = Tensor::contiguous_strides(t.dims);
+    s = kv_tensor_copy_shape(t, "k_cache_0", 256);
+    EXPECT(s.heads == 8 && s.capacity == 256 && s.head_dim == 128 && s.elem_bytes == 2);
+    EXPECT(thrown_by([&] { kv_tensor_copy_shape(t, "k_cache_0", 257); }) == MetalError::InvalidShape);
+    t.strides[1] = 256;
+    EXPECT(thrown_by([&] { kv_tensor_copy_shape(t, "k_cache_0", 1); }) == MetalError::InvalidShape);
+    t.dims = {8, 256}, t.strides = {256, 1};
+    EXPECT(thrown_by([&] { kv_tensor_copy_shape(t, "k_cache_0", 1); }) == MetalError::InvalidShape);
+}
+
+// src/model/executor.rs:232-250 and src/workflow/ops/prefill.rs:278-314.
+static void test_prefill_schedule() {
+    PrefillConfig c = prefill_config(nullptr, nullptr);
+    EXPECT(c.max_prefill_chunk == 32 && c.prefill_chunk_size == 32);
+    c = prefill_config("600", "700");
+    EXPECT(c.max_prefill_chunk == 512 && c.prefill_chunk_size == 512);
+    c = prefill_config("8", "64");  // the allocation must cover the largest runtime M
+    EXPECT(c.max_prefill_chunk == 64 && c.prefill_chunk_size == 64);
+    c = prefill_config(" 16 ", "abc");  // values are trimmed; what does not parse falls back to the default
+    EXPECT(c.max_prefill_chunk == 32 && c.prefill_chunk_size == 32);  // 16 raised to the chunk size 32
+    c = prefill_config(" 16 ", "8");
+    EXPECT(c.max_prefill_chunk == 16 && c.prefill_chunk_size == 8);
+    EXPECT(prefill_config("0", "0").prefill_chunk_size == 1);
+    EXPECT(rebalance_chunk_size(100, 32, 32) == 25);   // 4 chunks of 25 instead of 32+32+32+4
+    EXPECT(rebalance_chunk_size(33, 32, 32) == 17);
+    EXPECT(rebalance_chunk_size(32, 32, 32) == 32);
+    EXPECT(rebalance_chunk_size(1, 32, 32) == 1 && rebalance_chunk_size(0, 32, 32) == 1);
+    EXPECT(rebalance_chunk_size(2048, 512, 512) == 512);
+    EXPECT(rebalance_chunk_size(70, 0, 32) == 1);      // requested is raised to 1
+    EXPECT(rebalance_chunk_size(70, 64, 32) == 24);    // requested is capped at max_allowed: 3 chunks
+    for (size_t len = 0; len < 300; ++len)
+        for (size_t req : {1u, 7u, 32u, 64u}) {
+            const size_t cs = rebalance_chunk_size(len, req, 64);
+            EXPECT(cs >= 1 && cs <= std::max<size_t>(std::min<size_t>(req, 64), 1));
+            auto sched = prefill_schedule(11, len, cs);
+            size_t pos = 11;
+            for (const PrefillChunk &ch : sched) {
+                EXPECT(ch.base_pos == pos && ch.m >= 1 && ch.m <= cs);
+                pos += ch.m;
+            }
+            EXPECT(pos == 11 + len);
+            if (len > 1) EXPECT(sched.size() == (len + std::min<size_t>(req, 64) - 1) / std::min<size_t>(req, 64));  // same chunk count as requested
+        }
 }
 
 // ------------------------------------------------------------------------------------------------ GPU tests
@@ -229,10 +292,137 @@ static void test_error_variants(Foundry &foundry) {
     foundry.synchronize();
 }
 
+// A two-layer "model" of the path's two steps driven the way the executor drives them: chunked prefill of a prompt
+// (run_prefill_chunks), a prefix snapshot, a batched decode loop that outgrows the cache twice (run_decode_loop ->
+// ensure_kv_capacity), then restore of the snapshot. Every token's attention output is checked against the oracle's
+// decode at that position over the oracle's caches; caches are compared bit for bit.
+static void test_session_prefill_chunks_decode_loop_growth_snapshot(Foundry &foundry) {
+    const size_t L = 2, H = 8, Hkv = 2, D = 64, prompt = 70, gen = 100, total = prompt + gen, table_rows = 1024;
+    const size_t dm = H * D, kvd = Hkv * D;
+    Rng rng{99};
+    std::vector<std::vector<orc_f16>> q(L), k(L), v(L);
+    for (size_t i = 0; i < L; ++i) q[i] = rng.fill(total * dm, 1.0f), k[i] = rng.fill(total * kvd, 1.0f), v[i] = rng.fill(total * kvd, 1.0f);
+    std::vector<orc_f16> cos(table_rows * D / 2), sin(cos.size());
+    orc_rope_tables(10000.0f, (uint32_t)D, 0, (uint32_t)table_rows, nullptr, cos.data(), sin.data());
+
+    ContextConfig config = ContextConfig::from_limits(1024, 0, GrowthStrategy::GrowOnDemand(100, 2.0f));
+    EXPECT(config.allocated_capacity == 128);
+    TensorBindings b;
+    std::vector<std::string> kv_names;
+    std::vector<Tensor> q_full(L), k_full(L), v_full(L);
+    for (size_t i = 0; i < L; ++i) {
+        q_full[i] = foundry.from_host(Dtype::F16, {total, dm}, q[i].data());
+        k_full[i] = foundry.from_host(Dtype::F16, {total, kvd}, k[i].data());
+        v_full[i] = foundry.from_host(Dtype::F16, {total, kvd}, v[i].data());
+        for (const char *pre : {"k_cache_", "v_cache_"}) {
+            kv_names.push_back(pre + std::to_string(i));
+            b.insert(kv_names.back(), foundry.zeros(Dtype::F16, {Hkv, config.allocated_capacity, D}));
+        }
+    }
+    b.insert("rope_cos", foundry.from_host(Dtype::F16, {table_rows, D / 2}, cos.data()));
+    b.insert("rope_sin", foundry.from_host(Dtype::F16, {table_rows, D / 2}, sin.data()));
+    Tensor q_rot_buf = foundry.zeros(Dtype::F16, {H * 32 * D});           // one chunk's rotated q, head-major [H, m, D]
+    Tensor out_full = foundry.zeros(Dtype::F16, {L, total, dm});          // every token's attention output, per layer
+    b.set_int_global("max_seq_len", config.allocated_capacity);
+
+    KvPrepFusedStep kp{"q", "k", "v", "q_rot", "k_cache_{i}", "v_cache_{i}", "rope_cos", "rope_sin", {}};
+    kp.params.d_model = (uint32_t)dm, kp.params.kv_dim = (uint32_t)kvd, kp.params.head_dim = (uint32_t)D;
+    kp.params.n_heads = (uint32_t)H, kp.params.n_kv_heads = (uint32_t)Hkv, kp.params.group_size = (uint32_t)(H / Hkv);
+    kp.params.seq_len = DynamicU32::var("seq_len"), kp.params.position_offset = DynamicU32::var("position_offset");
+    kp.params.max_seq_len = DynamicU32::var("max_seq_len"), kp.params.total_elements = DynamicU32::var("total_elements");
+    FlashAttentionStep at{"q_rot", "k_cache_{i}", "v_cache_{i}", "attn_out"};
+    at.causal = true, at.kv_head_major = true, at.n_heads = (uint32_t)H, at.head_dim = (uint32_t)D;
+    at.query_offset = DynamicU32::var("position_offset"), at.kv_seq_len = DynamicU32::var("kv_seq_len"), at.m = DynamicU32::var("m");
+
+    // the model's forward pass over the current globals: per layer, inputs are rows [row0, row0 + m) of the layer's q/k/v
+    auto forward_rows = [&](size_t row0) {
+        const size_t m = *b.get_int_global("m");
+        b.set_int_global("total_elements", H * m * D);
+        for (size_t i = 0; i < L; ++i) {
+            b.set_int_global("i", i);
+            b.insert("q", q_full[i].view({m, dm}, row0 * dm * 2));
+            b.insert("k", k_full[i].view({m, kvd}, row0 * kvd * 2));
+            b.insert("v", v_full[i].view({m, kvd}, row0 * kvd * 2));
+            b.insert("q_rot", q_rot_buf.view({H, m, D}));
+            b.insert("attn_out", out_full.view({m, dm}, (i * total + row0) * dm * 2));
+            kp.execute(foundry, b);
+            at.execute(foundry, b);
+        }
+    };
+
+    // prefill: 70 tokens, requested chunk 32 -> 3 chunks of 24, 24, 22
+    std::vector<PrefillChunk> seen;
+    const size_t last_m = run_prefill_chunks(foundry, b, 0, prompt, prefill_config(nullptr, nullptr),
+                                             [&](const PrefillChunk &c) { seen.push_back(c); }, [&] { forward_rows(seen.back().base_pos); });
+    EXPECT(seen.size() == 3 && seen[0].m == 24 && seen[1].base_pos == 24 && seen[2].m == 22 && last_m == 22);
+    EXPECT(*b.get_int_global("kv_seq_len") == prompt);
+
+    std::vector<uint32_t> tokens(prompt, 7);
+    auto snap = capture_kv_prefix_snapshot(foundry, b, kv_names, tokens, 50);
+    EXPECT(snap && snap->kv_tensors.size() == 2 * L && snap->bytes == 2 * L * Hkv * 50 * D * 2 && snap->prefix_len == 50);
+    EXPECT(!capture_kv_prefix_snapshot(foundry, b, kv_names, tokens, 0));
+
+    // decode: 100 tokens in batches of 16 from position 70; capacity 128 -> 256 at position 128 (lookahead) -> no more
+    const size_t end = run_decode_loop(foundry, b, config, kv_names, prompt, gen, 16, [&](size_t pos) { forward_rows(pos); });
+    EXPECT(end == total && config.allocated_capacity == 256 && *b.get_int_global("max_seq_len") == 256);
+    EXPECT(b.get("k_cache_0")->dims[1] == 256);
+    EXPECT(thrown_by([&] { ensure_kv_capacity(foundry, b, config, kv_names, total, 2000); }) == MetalError::InvalidOperation);
+
+    // oracle: all 170 tokens appended at once into caches of the final capacity
+    const size_t cap = config.allocated_capacity;
+    auto out_got = foundry.to_host<orc_f16>(out_full);
+    float worst = 0.0f;
+    for (size_t i = 0; i < L; ++i) {
+        std::vector<orc_f16> q_ref(H * total * D), k_ref(Hkv * cap * D, 0), v_ref(k_ref.size(), 0);
+        orc_kv_prep_params p = {(uint32_t)dm, (uint32_t)kvd, (uint32_t)D, (uint32_t)H, (uint32_t)Hkv, (uint32_t)(H / Hkv), (uint32_t)total,
+                                0, (uint32_t)cap, (uint32_t)(H * total * D), 0, 0, 0};
+        orc_kv_prep_fused(q[i].data(), k[i].data(), v[i].data(), q_ref.data(), k_ref.data(), v_ref.data(), cos.data(), sin.data(), &p);
+        auto k_got = foundry.to_host<orc_f16>(*b.get("k_cache_" + std::to_string(i)));
+        auto v_got = foundry.to_host<orc_f16>(*b.get("v_cache_" + std::to_string(i)));
+        EXPECT(k_got.size() == k_ref.size() && std::memcmp(k_got.data(), k_ref.data(), k_ref.size() * 2) == 0);
+        EXPECT(v_got.size() == v_ref.size() && std::memcmp(v_got.data(), v_ref.data(), v_ref.size() * 2) == 0);
+        std::vector<orc_f16> q_row(H * D), want(H * D), got(H * D);
+        for (size_t t = 0; t < total; ++t) {
+            for (size_t h = 0; h < H; ++h) std::memcpy(&q_row[h * D], &q_ref[(h * total + t) * D], D * 2);
+            orc_sdpa_decode(q_row.data(), k_ref.data(), v_ref.data(), want.data(), (uint32_t)H, (uint32_t)Hkv, (uint32_t)D, (uint32_t)cap,
+                            (uint32_t)(t + 1), 1.0f / std::sqrt((float)D), 256, 8, 0, 1);
+            std::memcpy(got.data(), &out_got[(i * total + t) * dm], dm * 2);
+            worst = std::fmax(worst, max_abs_diff(want, got, dm));
+        }
+    }
+    if (worst > 2e-3f) std::printf("  session: max abs diff %g\n", worst);
+    EXPECT(worst <= 2e-3f);
+
+    // restore: the first 50 rows of every head come back, rows past them stay as they are
+    auto before = foundry.to_host<orc_f16>(*b.get("v_cache_1"));
+    for (const std::string &name : kv_names) check(fa_device_memset(foundry.ctx(), b.get(name)->buffer->ptr(), 0x11, Hkv * 60 * D * 2));  // head 0 rows 0..119
+    EXPECT(restore_kv_prefix_snapshot(foundry, b, *snap) == 50);
+    auto after = foundry.to_host<orc_f16>(*b.get("v_cache_1"));
+    bool prefix_ok = true, rest_ok = true;
+    for (size_t h = 0; h < Hkv; ++h)
+        for (size_t r = 0; r < cap; ++r) {
+            const bool same = std::memcmp(&after[(h * cap + r) * D], &before[(h * cap + r) * D], D * 2) == 0;
+            const bool clobbered = h == 0 && r < 120;
+            if (r < 50) prefix_ok = prefix_ok && same;
+            else if (!clobbered) rest_ok = rest_ok && same;
+            else rest_ok = rest_ok && after[(h * cap + r) * D] == 0x1111;
+        }
+    EXPECT(prefix_ok && rest_ok);
+    // a snapshot does not fit a cache of other geometry
+    TensorBindings other;
+    for (const std::string &name : kv_names) other.insert(name, foundry.zeros(Dtype::F16, {Hkv + 1, cap, D}));
+    EXPECT(thrown_by([&] { restore_kv_prefix_snapshot(foundry, other, *snap); }) == MetalError::InvalidShape);
+    TensorBindings small;
+    for (const std::string &name : kv_names) small.insert(name, foundry.zeros(Dtype::F16, {Hkv, 32, D}));
+    EXPECT(thrown_by([&] { restore_kv_prefix_snapshot(foundry, small, *snap); }) == MetalError::InvalidShape);
+}
+
 int main(int argc, char **argv) {
     const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu";
     run_test("bindings and dynamic values", test_bindings_and_dynamic_values);
     run_test("steps compile against interpolated names", test_steps_compile_against_interpolated_names);
+    run_test("capacity policy", test_capacity_policy);
+    run_test("prefill chunk schedule", test_prefill_schedule);
     if (!cpu_only) {
         Foundry foundry(0);
         run_test("kv_prep_fused decode (1, 5, 16, 14, 2, 64)", [&] { run_fused_parity(foundry, 1, 5, 16, 14, 2, 64); });
@@ -249,6 +439,8 @@ int main(int argc, char **argv) {
             }
         run_test("closed-form prefill H2 N15 D64", [&] { test_closed_form_prefill(foundry); });
         run_test("error variants", [&] { test_error_variants(foundry); });
+        run_test("session: chunked prefill, snapshot, decode loop with growth, restore",
+                 [&] { test_session_prefill_chunks_decode_loop_growth_snapshot(foundry); });
     }
     std::printf("%d cases, %d failed checks\n", g_run, g_failed);
     return g_failed == 0 ? 0 : 1;

@@ -216,6 +216,39 @@ def paged_gather(pool, block_table, n_kv_heads, block_size, head_dim, seq_len, o
     return out
 
 
+def paged_copy_blocks(pool, n_kv_heads, block_size, head_dim, src_ids, dst_ids):
+    """In place on `pool` [n_blocks, n_kv_heads, block_size, head_dim] f16."""
+    assert pool.dtype == np.float16 and pool.flags.c_contiguous
+    s = np.ascontiguousarray(src_ids, dtype=np.int32)
+    d = np.ascontiguousarray(dst_ids, dtype=np.int32)
+    lib().orc_paged_copy_blocks(_p(pool, u16p), C.c_uint32(pool.shape[0]), C.c_uint32(n_kv_heads), C.c_uint32(block_size),
+                                C.c_uint32(head_dim), _p(s, i32p), _p(d, i32p), C.c_uint32(len(s)))
+
+
+def kv_prefix_copy(src, dst, prefix_len):
+    """Rows [0, prefix_len) of every head of src [heads, cap_s, D] into dst [heads, cap_d, D] (in place); any dtype."""
+    assert src.flags.c_contiguous and dst.flags.c_contiguous and src.dtype == dst.dtype
+    assert src.shape[0] == dst.shape[0] and src.shape[2] == dst.shape[2]
+    L = lib()
+    L.orc_kv_prefix_copy.restype = C.c_int
+    return L.orc_kv_prefix_copy(C.c_void_p(src.ctypes.data), C.c_void_p(dst.ctypes.data), C.c_size_t(src.shape[0]),
+                                C.c_size_t(src.shape[1]), C.c_size_t(dst.shape[1]), C.c_size_t(src.shape[2]),
+                                C.c_size_t(src.dtype.itemsize), C.c_size_t(prefix_len))
+
+
+def align_capacity(capacity):
+    L = lib()
+    L.orc_align_capacity.restype = C.c_size_t
+    return L.orc_align_capacity(C.c_size_t(capacity))
+
+
+def grown_capacity(allocated, required_len, max_context_len, growth_factor=2.0):
+    L = lib()
+    L.orc_grown_capacity.restype = C.c_size_t
+    return L.orc_grown_capacity(C.c_size_t(allocated), C.c_size_t(required_len), C.c_size_t(max_context_len),
+                                C.c_float(growth_factor))
+
+
 def paged_scatter(pool, block_table, n_kv_heads, block_size, head_dim, pos_begin, pos_end, src):
     assert pool.dtype == np.float16 and pool.flags.c_contiguous
     bt = np.ascontiguousarray(block_table, dtype=np.int32)

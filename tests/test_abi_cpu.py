@@ -67,3 +67,17 @@ def test_host_errors_without_a_device():
     assert st == 1 and "Device not found" in lib.fa_last_error_string().decode()
     assert lib.fa_synchronize(None) == 2
     assert lib.fa_graph_destroy(None) == 0 and lib.fa_ctx_destroy(None) == 0
+
+
+def test_capacity_policy_equals_oracle():
+    """fa_align_capacity / fa_grown_capacity are host arithmetic: same values as the oracle's restatement of
+    src/model/context.rs:213-219 and src/model/executor.rs:2354-2382 over a sweep."""
+    for c in list(range(0, 400)) + [2047, 2048, 2049, 65535, 65536, 1 << 20]:
+        assert fa.align_capacity(c) == orc.align_capacity(c)
+    rng = np.random.default_rng(7)
+    for _ in range(3000):
+        alloc = int(rng.integers(0, 40000))
+        mx = int(rng.integers(1, 140000))
+        req = int(rng.integers(0, 150000))
+        gf = float(rng.choice([0.0, 1.1, 1.5, 2.0, 3.0]))
+        assert fa.grown_capacity(alloc, req, mx, gf) == orc.grown_capacity(alloc, req, mx, gf), (alloc, req, mx, gf)

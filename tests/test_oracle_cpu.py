@@ -523,3 +523,73 @@ def test_bf16_mode_kv_prep_rotation_is_rounded_once_to_bf16():
     want = np.concatenate([lo, hi], axis=-1).transpose(1, 0, 2)
     got = orc.bf16_unpack(qr).astype(np.float64)
     assert np.max(np.abs(got - want)) <= 2.0 ** -8 * max(1.0, float(np.max(np.abs(want))))
+
+
+# ---------------------------------------------------------------- KV prefix copies and the capacity policy
+
+def test_align_capacity_reference_vectors():
+    """The reference's own vectors (src/model/context.rs:318-323)."""
+    for c, want in [(0, 128), (1, 128), (127, 128), (128, 128), (129, 256), (200, 256)]:
+        assert orc.align_capacity(c) == want
+
+
+def test_grown_capacity_hand_worked_cases_and_invariants():
+    """ensure_kv_capacity (src/model/executor.rs:2354-2382) with the default strategy (initial 2048, factor 2.0,
+    src/model/context.rs:42-49), worked by hand; then invariants over a sweep."""
+    assert orc.grown_capacity(2048, 2048, 8192) == 2048          # already sufficient
+    assert orc.grown_capacity(2048, 2049, 8192) == 4096          # 2048 * 2
+    assert orc.grown_capacity(2048, 5000, 8192) == 5120          # max(4096, 5000) = 5000 -> aligned
+    assert orc.grown_capacity(4096, 4097, 6000) == 6016          # min(8192, 6000) = 6000 -> aligned past the maximum
+    assert orc.grown_capacity(2048, 8193, 8192) == 0             # exceeds max_context_len: InvalidOperation
+    assert orc.grown_capacity(2048, 3000, 8192, 0.0) == 8192     # FullReserve
+    assert orc.grown_capacity(2048, 2100, 8192, 1.5) == 3072     # (2048 * 1.5) as usize
+    assert orc.grown_capacity(1000, 1001, 8192, 1.1) == 1152     # (1000 * 1.1f32) as usize = 1100 -> 1152
+    rng = np.random.default_rng(0)
+    for _ in range(2000):
+        alloc = int(orc.align_capacity(int(rng.integers(1, 20000))))
+        mx = int(rng.integers(alloc, 70000))
+        req = int(rng.integers(1, mx + 1))
+        g = orc.grown_capacity(alloc, req, mx)
+        if req <= alloc:
+            assert g == alloc
+        else:
+            assert g % 128 == 0 and g >= req and g <= orc.align_capacity(mx)
+            assert g >= min(2 * alloc, mx) and orc.grown_capacity(alloc, min(req + 1, mx), mx) >= g
+
+
+def test_kv_prefix_copy_is_the_per_head_blit():
+    """Brute force over indices: dst[h, p, :] = src[h, p, :] for p < prefix_len, everything else unchanged; and the
+    snapshot -> clobber -> restore round trip (src/model/executor.rs:1195-1212, 1296-1318)."""
+    rng = np.random.default_rng(1)
+    for heads, cs, cd, D, n, dt in [(3, 10, 16, 6, 7, np.float16), (2, 8, 8, 4, 8, np.int8), (1, 5, 9, 3, 0, np.float32)]:
+        src = rng.integers(0, 250, size=(heads, cs, D)).astype(dt)
+        dst = rng.integers(0, 250, size=(heads, cd, D)).astype(dt)
+        want = dst.copy()
+        for h in range(heads):
+            for p in range(n):
+                for d in range(D):
+                    want[h, p, d] = src[h, p, d]
+        got = dst.copy()
+        assert orc.kv_prefix_copy(src, got, n) == 0
+        assert np.array_equal(got, want)
+    live = rng.normal(size=(4, 32, 8)).astype(np.float16)
+    snap = np.zeros((4, 20, 8), np.float16)
+    assert orc.kv_prefix_copy(live, snap, 20) == 0
+    assert np.array_equal(snap, live[:, :20])
+    clob = rng.normal(size=(4, 32, 8)).astype(np.float16)
+    cur = clob.copy()
+    assert orc.kv_prefix_copy(snap, cur, 20) == 0
+    assert np.array_equal(cur[:, :20], live[:, :20]) and np.array_equal(cur[:, 20:], clob[:, 20:])
+    assert orc.kv_prefix_copy(live, snap, 21) == -1  # prefix_len exceeds the snapshot's capacity: nothing copied
+    assert np.array_equal(snap, live[:, :20])
+
+
+def test_paged_copy_blocks_index_map():
+    rng = np.random.default_rng(2)
+    pool = rng.normal(size=(6, 2, 16, 8)).astype(np.float16)
+    want = pool.copy()
+    want[5] = pool[1]
+    want[0] = pool[3]
+    got = pool.copy()
+    orc.paged_copy_blocks(got, 2, 16, 8, [1, 3, 2, -1, 6, 4], [5, 0, 2, 1, 0, 9])
+    assert np.array_equal(got, want)
