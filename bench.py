@@ -374,6 +374,49 @@ def bench_kv_growth(f, args):
     f.profile_enable(False)
 
 
+def bench_fused_qkv(f, args):
+    """The step before the path at Llama-3.2-3B decode shape: RMSNorm + Q/K/V projections of one token, F16 weights in
+    the reference's canonical blocked layout, one layer per step over 8 distinct layers' weights."""
+    import orc
+    K, N, NK, NL = 3072, 3072, 1024, 8
+    rng = np.random.default_rng(0xF0DD + 7)
+    x = rng.uniform(-1, 1, (1, K)).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, K).astype(np.float16)
+    layers, host0 = [], None
+    for i in range(NL):  # distinct weights so that no launch finds the previous one's in cache
+        ws = [rng.uniform(-0.1, 0.1, (n, K)).astype(np.float16) for n in (N, NK, NK)]
+        layers.append([f.array(orc.to_canonical(w)) for w in ws])
+        if i == 0:
+            host0 = ws
+    dx, dg = f.array(x), f.array(g)
+    oq, ok, ov = f.zeros((1, N)), f.zeros((1, NK)), f.zeros((1, NK))
+
+    def step(i):
+        w = layers[i % NL]
+        f.fused_qkv(dx.arg(), w[0].arg(), w[1].arg(), w[2].arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1, gamma=dg.arg())
+
+    step(0)
+    f.synchronize()
+    want = orc.fused_qkv(x, *host0, gamma=g)
+    err = max(float(np.max(np.abs(o.download().astype(np.float64) - w.astype(np.float64)))) for o, w in zip((oq, ok, ov), want))
+    for i in range(args.warmup):
+        step(i)
+    f.synchronize()
+    f.profile_reset()
+    f.profile_enable(True)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    nbytes = 2.0 * (N + 2 * NK) * K + 2 * K * 2 + 2 * (N + 2 * NK)  # weights, input + gamma, outputs
+    _finish_secondary(f, args, "FusedQkv layer-steps/s + achieved HBM GB/s, Llama-3.2-3B decode shape",
+                      "llama3.2-3b FusedQkv at decode: RMSNorm + Q/K/V projections of one token, k_dim 3072, n_dim 3072, "
+                      "n_kv 1024, F16 canonical weights, eager launches (profiling events on)", "fused_qkv_kernel", nbytes, dt,
+                      {"qkv_max_abs_err": err})
+    f.profile_enable(False)
+
+
 def bench_paged_decode(f, args):
     """Qwen2.5-3B-shaped batched paged decode, one layer per step: 32 ragged sequences, 16-token blocks."""
     import orc
@@ -506,7 +549,7 @@ def bench_sage_decode(f, args):
 
 SECONDARY = {"llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
-             "llama3b_kv_growth": bench_kv_growth}
+             "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv}
 
 
 def main():

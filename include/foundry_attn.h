@@ -352,6 +352,43 @@ fa_status fa_paged_copy_blocks(fa_ctx *ctx, const fa_paged_kv *cache, const int3
                                const int32_t *d_dst_ids, uint32_t n_pairs);
 
 /* ---------------------------------------------------------------------------------------------
+ * FusedQkv: the step before the path. RMSNorm(input) -> Q, K and V projections in one launch -> the three
+ * token-major tensors KvPrepFused consumes (src/metals/gemv/qkv_step.rs:14-120,220-460, op `FusedQkv` of
+ * models/llama.json:509-528; kernel src/metals/gemv/qkv_project.metal). F16 weights only (PolicyF16,
+ * src/metals/policies/policy_f16.metal:18-70): the reference's block-quantised policies are not built here and
+ * are refused with FA_ERR_UNSUPPORTED_DTYPE.
+ *   out_q[b, r] = f16( sum_k xn[b, k] * W_q[r, k] + bias_q[r] ),  r < n_dim;  out_k, out_v likewise, r < n_kv
+ *   xn[b, k]    = f16( x[b, k] * rsqrt(mean_k x[b, k]^2 + epsilon) * gamma[k] )  with gamma, else x[b, k]
+ * (the normalised input is rounded to f16 before the products, qkv_project.metal:48-67; f32 accumulation; the
+ * bias is added in f32 and the result rounded once, :260-268).
+ * ------------------------------------------------------------------------------------------- */
+typedef enum fa_weight_layout {
+    FA_WEIGHT_LAYOUT_ROW_MAJOR = 0, /* weights[row * k_dim + k]                    (src/compound/stages/layout.rs:79-82) */
+    FA_WEIGHT_LAYOUT_CANONICAL = 1  /* weights[(k % 32) + 32 * (row + (k / 32) * n_rows)], weights_per_block = 32
+                                       (src/compound/stages/layout.rs:95-100, qkv_project.metal:83-96) */
+} fa_weight_layout;
+
+/* Field meaning as FusedQkvArgs (src/metals/gemv/qkv_step.rs:57-99). */
+typedef struct fa_fused_qkv_params {
+    uint32_t k_dim;             /* input features; a multiple of 32 */
+    uint32_t n_dim;             /* rows of W_q */
+    uint32_t n_kv;              /* rows of W_k and of W_v */
+    uint32_t m;                 /* input rows (tokens); 0 is treated as 1 (qkv_step.rs:236) */
+    uint32_t weights_per_block; /* 32 for the canonical layout; ignored for row-major */
+    uint32_t layout;            /* fa_weight_layout */
+    float epsilon;              /* RMSNorm epsilon (the reference's `rms_eps` variable, default 1e-6) */
+} fa_fused_qkv_params;
+
+/* input [m, k_dim] (any rank with k_dim innermost and contiguous); w_q [n_dim * k_dim], w_k, w_v [n_kv * k_dim] f16
+ * in `layout`; gamma [k_dim] or NULL / NULL buffer (no RMSNorm); bias_q [n_dim], bias_k, bias_v [n_kv]: all three or
+ * none (the reference takes has_bias from bias_q alone and would read the input buffer for a missing bias_k);
+ * out_q [m, n_dim], out_k, out_v [m, n_kv]. */
+fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *input, const fa_tensor_arg *w_q, const fa_tensor_arg *w_k,
+                       const fa_tensor_arg *w_v, const fa_tensor_arg *gamma, const fa_tensor_arg *bias_q,
+                       const fa_tensor_arg *bias_k, const fa_tensor_arg *bias_v, const fa_tensor_arg *out_q,
+                       const fa_tensor_arg *out_k, const fa_tensor_arg *out_v, const fa_fused_qkv_params *params);
+
+/* ---------------------------------------------------------------------------------------------
  * SageAttention-style int8 Q/K decode (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170 - prose only in
  * the reference). K is mean-smoothed over the sequence per (kv head, channel), then quantised per block
  * of 32 tokens: scale = max|k - mean| / 127 stored as f16, k_q = rint((k - mean)/scale) in [-127,127].

@@ -603,6 +603,54 @@ size_t orc_grown_capacity(size_t allocated, size_t required_len, size_t max_cont
     return orc_align_capacity(new_capacity);                /* :2381 */
 }
 
+/* ------------------------------------------------------------------ FusedQkv */
+
+/* src/compound/stages/layout.rs:79-82 (RowMajor) and :95-100 (Canonical) */
+size_t orc_weight_index(int layout, size_t row, size_t k, size_t k_dim, size_t n_rows, size_t wpb) {
+    if (layout == 0) return row * k_dim + k;
+    return (k % wpb) + wpb * (row + (k / wpb) * n_rows);
+}
+
+/* One projection: tests/qkv_parity_f16.rs:47-69 */
+static void qkv_project(const orc_f16 *xn, const orc_f16 *w, const orc_f16 *bias, orc_f16 *out, uint32_t k_dim,
+                        uint32_t n_rows, int layout, uint32_t wpb, int n_threads) {
+    (void)n_threads;
+#ifdef _OPENMP
+#pragma omp parallel for num_threads(n_threads > 0 ? n_threads : 1) schedule(static)
+#endif
+    for (int64_t i = 0; i < (int64_t)n_rows; ++i) {
+        float sum = 0.0f;
+        for (uint32_t j = 0; j < k_dim; ++j)
+            sum += orc_f16_to_f32(xn[j]) * orc_f16_to_f32(w[orc_weight_index(layout, (size_t)i, j, k_dim, n_rows, wpb)]);
+        out[i] = orc_f32_to_f16(sum + (bias ? orc_f16_to_f32(bias[i]) : 0.0f));
+    }
+}
+
+void orc_fused_qkv(const orc_f16 *x, const orc_f16 *w_q, const orc_f16 *w_k, const orc_f16 *w_v, const orc_f16 *gamma,
+                   const orc_f16 *bias_q, const orc_f16 *bias_k, const orc_f16 *bias_v, orc_f16 *out_q, orc_f16 *out_k,
+                   orc_f16 *out_v, uint32_t k_dim, uint32_t n_dim, uint32_t n_kv, uint32_t m, int layout, uint32_t wpb,
+                   float eps, int n_threads) {
+    orc_f16 *xn = (orc_f16 *)malloc(sizeof(orc_f16) * (k_dim ? k_dim : 1));
+    for (uint32_t b = 0; b < m; ++b) {
+        const orc_f16 *xr = x + (size_t)b * k_dim;
+        if (gamma) { /* tests/qkv_parity_f16.rs:17-30 */
+            float sum_sq = 0.0f;
+            for (uint32_t j = 0; j < k_dim; ++j) {
+                const float xf = orc_f16_to_f32(xr[j]);
+                sum_sq += xf * xf;
+            }
+            const float inv_rms = 1.0f / sqrtf(sum_sq / (float)k_dim + eps);
+            for (uint32_t j = 0; j < k_dim; ++j) xn[j] = orc_f32_to_f16(orc_f16_to_f32(xr[j]) * inv_rms * orc_f16_to_f32(gamma[j]));
+        } else {
+            memcpy(xn, xr, sizeof(orc_f16) * k_dim);
+        }
+        qkv_project(xn, w_q, bias_q, out_q + (size_t)b * n_dim, k_dim, n_dim, layout, wpb, n_threads);
+        qkv_project(xn, w_k, bias_k, out_k + (size_t)b * n_kv, k_dim, n_kv, layout, wpb, n_threads);
+        qkv_project(xn, w_v, bias_v, out_v + (size_t)b * n_kv, k_dim, n_kv, layout, wpb, n_threads);
+    }
+    free(xn);
+}
+
 /* ------------------------------------------------------------------ Sage-style int8 Q/K */
 
 void orc_sage_k_mean(const orc_f16 *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim, uint32_t kv_len,

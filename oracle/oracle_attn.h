@@ -39,6 +39,9 @@
  *   orc_kv_prefix_copy        no reference test; a byte copy, pinned by brute-force index checks and by the
  *                             snapshot -> clobber -> restore round trip
  *   orc_paged_copy_blocks     no reference counterpart; pinned by gather(fork) == gather(parent) on the prefix
+ *   orc_fused_qkv             pinned: transcription of the reference test's CPU helpers (tests/qkv_parity_f16.rs:17-72)
+ *                             checked against float64 matrix products; orc_weight_index pinned as a bijection that
+ *                             reduces to the row-major index per 32-feature block (src/compound/stages/layout.rs:79-100)
  */
 #ifndef ORACLE_ATTN_H
 #define ORACLE_ATTN_H
@@ -158,6 +161,18 @@ size_t orc_align_capacity(size_t capacity);
 /* New capacity chosen by ensure_kv_capacity (src/model/executor.rs:2354-2382); growth_factor <= 0 = FullReserve.
  * `allocated` if it suffices, 0 if required_len > max_context_len. */
 size_t orc_grown_capacity(size_t allocated, size_t required_len, size_t max_context_len, float growth_factor);
+
+/* FusedQkv (src/metals/gemv/qkv_step.rs, src/metals/gemv/qkv_project.metal), F16 weights.
+ * orc_weight_index: element index of weight (row, k) of a [n_rows, k_dim] matrix (src/compound/stages/layout.rs:79-100):
+ * layout 0 row-major row*k_dim + k; layout 1 canonical (k % wpb) + wpb*(row + (k / wpb)*n_rows).
+ * orc_fused_qkv follows the reference test's CPU helpers (tests/qkv_parity_f16.rs:17-72) per input row b:
+ *   inv_rms = 1/sqrt(sum_k x^2 / k_dim + eps); xn[k] = f16(x[k]*inv_rms*gamma[k]) (gamma NULL: xn = x);
+ *   out_q[b, i] = f16(sum_k xn[k]*W_q[i,k] + bias_q[i]) in f32, k ascending; out_k, out_v likewise. bias_* NULL = none. */
+size_t orc_weight_index(int layout, size_t row, size_t k, size_t k_dim, size_t n_rows, size_t wpb);
+void orc_fused_qkv(const orc_f16 *x, const orc_f16 *w_q, const orc_f16 *w_k, const orc_f16 *w_v, const orc_f16 *gamma,
+                   const orc_f16 *bias_q, const orc_f16 *bias_k, const orc_f16 *bias_v, orc_f16 *out_q, orc_f16 *out_k,
+                   orc_f16 *out_v, uint32_t k_dim, uint32_t n_dim, uint32_t n_kv, uint32_t m, int layout, uint32_t wpb,
+                   float eps, int n_threads);
 
 /* Sage-style int8 Q/K (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170).
  * K smoothing: subtract per-(head, channel) mean over the sequence (f32), quantise per block of

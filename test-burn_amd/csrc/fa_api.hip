@@ -725,6 +725,74 @@ extern "C" fa_status fa_paged_copy_blocks(fa_ctx *ctx, const fa_paged_kv *cache,
     return fa_launch_paged_copy_blocks(ctx, cache, d_src_ids, d_dst_ids, n_pairs);
 }
 
+// ------------------------------------------------------------------------------------------------ FusedQkv
+
+static bool present(const fa_tensor_arg *t) { return t && t->buffer; }
+static const __half *half_ptr(const fa_tensor_arg *t) {
+    return reinterpret_cast<const __half *>(static_cast<const char *>(t->buffer) + t->offset);
+}
+
+extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *input, const fa_tensor_arg *w_q, const fa_tensor_arg *w_k,
+                                  const fa_tensor_arg *w_v, const fa_tensor_arg *gamma, const fa_tensor_arg *bias_q,
+                                  const fa_tensor_arg *bias_k, const fa_tensor_arg *bias_v, const fa_tensor_arg *out_q,
+                                  const fa_tensor_arg *out_k, const fa_tensor_arg *out_v, const fa_fused_qkv_params *p) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(p, "params");
+    const struct { const fa_tensor_arg *t; const char *name; } req[] = {{input, "input"}, {w_q, "w_q"}, {w_k, "w_k"}, {w_v, "w_v"},
+                                                                         {out_q, "out_q"}, {out_k, "out_k"}, {out_v, "out_v"}};
+    for (const auto &r : req) {
+        FA_NEED(r.t, r.name);
+        if (!r.t->buffer) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: %s", r.name);
+    }
+    for (const fa_tensor_arg *w : {w_q, w_k, w_v})
+        if (w->dtype != FA_DTYPE_F16)
+            return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: weight dtype %u: only F16 weights are built (no block-quantised policies)", w->dtype);
+    if (w_q->dtype != w_k->dtype || w_q->dtype != w_v->dtype)
+        return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: mixed weight dtypes are not supported");
+    for (const fa_tensor_arg *t : {input, out_q, out_k, out_v})
+        if (t->dtype != FA_DTYPE_F16) return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: activations must be F16, got dtype %u", t->dtype);
+    const uint32_t m = p->m ? p->m : 1;
+    if (p->k_dim == 0 || p->n_dim == 0 || p->n_kv == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv k_dim %u n_dim %u n_kv %u", p->k_dim, p->n_dim, p->n_kv);
+    if (p->k_dim % 32 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: k_dim %u must be a multiple of 32", p->k_dim);
+    if (p->layout > FA_WEIGHT_LAYOUT_CANONICAL) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: unknown weight layout %u", p->layout);
+    if (p->layout == FA_WEIGHT_LAYOUT_CANONICAL && p->weights_per_block != 32)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: the canonical layout is built for weights_per_block = 32, got %u", p->weights_per_block);
+    if (input->rank == 0 || input->dims[input->rank - 1] != p->k_dim || input->strides[input->rank - 1] != 1)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv input must have k_dim %u as its contiguous last dim", p->k_dim);
+    if (numel(input) < (size_t)m * p->k_dim) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv input holds %zu elements, m * k_dim = %zu", numel(input), (size_t)m * p->k_dim);
+    for (uint32_t i = 0; i + 1 < input->rank; ++i) {  // rows must be packed: stride of dim i = product of the inner dims
+        size_t inner = 1;
+        for (uint32_t j = i + 1; j < input->rank; ++j) inner *= input->dims[j];
+        if (input->dims[i] > 1 && input->strides[i] != inner)
+            return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: input rows must be contiguous");
+    }
+    if (numel(w_q) < (size_t)p->n_dim * p->k_dim || numel(w_k) < (size_t)p->n_kv * p->k_dim || numel(w_v) < (size_t)p->n_kv * p->k_dim)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv weights smaller than rows * k_dim");
+    if (numel(out_q) < (size_t)m * p->n_dim || numel(out_k) < (size_t)m * p->n_kv || numel(out_v) < (size_t)m * p->n_kv)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv outputs smaller than m * rows");
+    const bool has_norm = present(gamma), has_bias = present(bias_q);
+    if (has_norm && (gamma->dtype != FA_DTYPE_F16 || numel(gamma) < p->k_dim))
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv gamma must be F16 [k_dim]");
+    if (has_bias) {
+        if (!present(bias_k) || !present(bias_v)) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: bias_k / bias_v (bias_q is bound)");
+        if (bias_q->dtype != FA_DTYPE_F16 || bias_k->dtype != FA_DTYPE_F16 || bias_v->dtype != FA_DTYPE_F16 || numel(bias_q) < p->n_dim ||
+            numel(bias_k) < p->n_kv || numel(bias_v) < p->n_kv)
+            return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv biases must be F16 [n_dim], [n_kv], [n_kv]");
+    }
+    FusedQkvLaunch L;
+    L.w[0] = half_ptr(w_q), L.w[1] = half_ptr(w_k), L.w[2] = half_ptr(w_v);
+    L.bias[0] = has_bias ? half_ptr(bias_q) : nullptr, L.bias[1] = has_bias ? half_ptr(bias_k) : nullptr;
+    L.bias[2] = has_bias ? half_ptr(bias_v) : nullptr;
+    L.out[0] = const_cast<__half *>(half_ptr(out_q)), L.out[1] = const_cast<__half *>(half_ptr(out_k));
+    L.out[2] = const_cast<__half *>(half_ptr(out_v));
+    L.x = half_ptr(input), L.gamma = has_norm ? half_ptr(gamma) : nullptr;
+    L.k_dim = p->k_dim, L.n_dim = p->n_dim, L.n_kv = p->n_kv, L.m = m, L.eps = p->epsilon;
+    L.canonical = p->layout == FA_WEIGHT_LAYOUT_CANONICAL;
+    for (const void *ptr : {(const void *)L.w[0], (const void *)L.w[1], (const void *)L.w[2], (const void *)L.x, (const void *)L.gamma})
+        if (ptr && (uintptr_t)ptr % 16 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: input, gamma and weights must be 16-byte aligned");
+    return fa_launch_fused_qkv(ctx, L);
+}
+
 // ------------------------------------------------------------------------------------------------ FlashAttention
 
 struct KvLayout {

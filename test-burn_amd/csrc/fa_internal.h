@@ -167,6 +167,17 @@ fa_status fa_launch_kv_prefix_copy(fa_ctx *ctx, const KvPrefixCopyLaunch &l);
 fa_status fa_launch_paged_copy_blocks(fa_ctx *ctx, const fa_paged_kv *c, const int32_t *src_ids, const int32_t *dst_ids,
                                       uint32_t n_pairs);
 
+// FusedQkv: out_i[m, rows_i] = f16(norm(x)[m, k_dim] . W_i^T + bias_i) for W_q [n_dim, k_dim], W_k, W_v [n_kv, k_dim].
+struct FusedQkvLaunch {
+    const __half *w[3], *bias[3] /* all three or none */;
+    __half *out[3];
+    const __half *x, *gamma /* nullable: no RMSNorm */;
+    uint32_t k_dim, n_dim, n_kv, m;
+    float eps;
+    bool canonical;  // weights blocked by 32 features, else row-major [rows, k_dim]
+};
+fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l);
+
 fa_status fa_launch_sage_k_mean(fa_ctx *ctx, const void *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim,
                                 uint32_t kv_len, float *mean_out);
 fa_status fa_launch_sage_quantize_k(fa_ctx *ctx, const void *k, const float *mean, uint32_t n_kv_heads,

@@ -1,0 +1,239 @@
+// FusedQkv: RMSNorm(input) -> Q, K and V projections in one launch -> three token-major outputs, F16 weights.
+// Reference: src/metals/gemv/qkv_step.rs:14-120,220-460 (step, arguments, dispatch), src/metals/gemv/qkv_project.metal
+// (projection, reduce, bias + write), src/metals/rmsnorm/rmsnorm.metal:17-96 (inv_rms), weight layouts
+// src/compound/stages/layout.rs:79-100.
+//
+// The reference gives every output row a 32-lane warp and re-reads the input per row. Here the step is what it is
+// at decode, a weight stream (HBM-bound: every weight is read once per launch, the input is a few KB):
+//   * the rows of W_q, W_k, W_v are treated as one list and dealt evenly to a multiple of the CU count of
+//     workgroups (not in 16-row quanta: 5120 rows over 256 CUs are 512 workgroups of 10), so that every CU
+//     requests the same number of bytes;
+//   * a workgroup walks its rows in tiles of 16; a tile times 32 input features is one 1 KiB load per wave in the
+//     blocked ("canonical") layout, and one v_mfma_f32_16x16x32_f16 with the (<= 16) input rows as the other
+//     operand - the matrix unit is used for its shape, not its rate: columns past m are zero;
+//   * the 8 waves split the feature blocks of a tile; their 16 x 16 partial results are summed through LDS in a
+//     fixed order, the bias is added and the row is rounded to f16 once, as the reference does.
+// The normalised input is rounded to f16 before the products (qkv_project.metal:66-67), f32 accumulation.
+#include "fa_internal.h"
+
+namespace {
+
+constexpr int QKV_NT = 512, QKV_NW = QKV_NT / 64;
+constexpr int QKV_UNITS = 8;  // feature blocks per batch of requests; a wave keeps two batches in flight
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef float f4v_t __attribute__((ext_vector_type(4)));
+
+struct QkvDev {
+    const __half *w[3];     // W_q, W_k, W_v
+    const __half *bias[3];  // nullable as a set
+    __half *out[3];         // [m, rows[i]]
+    uint32_t rows[3];       // n_dim, n_kv, n_kv
+    const __half *x;        // [m, k_dim]
+    const __half *gamma;    // nullable: no RMSNorm
+    uint32_t k_dim, m, cols_per_pass, rows_per_wg, x_stride /* bytes of an input row in LDS */, canonical;
+    float eps;
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+__global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, c = lane >> 4;
+    const uint32_t K = a.k_dim, nkb = K / 32;
+    const uint32_t total_rows = a.rows[0] + a.rows[1] + a.rows[2];
+    const uint32_t row_begin = blockIdx.x * a.rows_per_wg;
+    const uint32_t row_end = min(total_rows, row_begin + a.rows_per_wg);
+    if (row_begin >= row_end) return;
+    const uint32_t n_tiles = (row_end - row_begin + 15) / 16;
+    const uint32_t m0 = blockIdx.y * a.cols_per_pass, cols = min(a.cols_per_pass, a.m - m0);
+    unsigned char *x_lds = smem;
+    float *red = reinterpret_cast<float *>(smem + (size_t)a.cols_per_pass * a.x_stride);  // [QKV_NW][16][17], and scratch
+
+    // Where a row of the concatenated list lives: matrix, row inside it, the matrix's row count.
+    auto locate = [&](uint32_t gr, int &mat, uint32_t &lrow) {
+        mat = 0, lrow = gr;
+        if (lrow >= a.rows[0]) {
+            lrow -= a.rows[0], mat = 1;
+            if (lrow >= a.rows[1]) lrow -= a.rows[1], mat = 2;
+        }
+    };
+    // Weight operand of (tile, feature block kb): lane (n, c) holds features 8c..8c+7 of the block for row n of the
+    // tile (consecutive lanes 64 bytes apart; requesting in address order, four lanes per row, and moving the words
+    // into place with LDS permutes was slower: 10.6 us against 9.5 on 31.5 MB of weights).
+    // Per tile a lane keeps the address of its block 0 and its stride from block to block.
+    auto tile_base = [&](uint32_t tile, const __half *&p0, size_t &kb_stride, bool &ok) {
+        const uint32_t gr = row_begin + tile * 16 + n;
+        ok = gr < row_end;
+        int mat;
+        uint32_t lrow;
+        locate(ok ? gr : row_begin, mat, lrow);
+        const __half *base = mat == 0 ? a.w[0] : mat == 1 ? a.w[1] : a.w[2];
+        const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
+        // canonical (blocked by 32 features): (k % 32) + 32 * (row + (k / 32) * N); row-major: row * K + k
+        p0 = a.canonical ? base + (size_t)lrow * 32 + c * 8 : base + (size_t)lrow * K + c * 8;
+        kb_stride = a.canonical ? (size_t)N * 32 : 32;
+    };
+
+    // A wave takes the feature blocks kb = wave, wave + 8, ... of every tile, in batches of QKV_UNITS; two batches
+    // are in flight. The first two are requested before anything else: they do not depend on the input.
+    const uint32_t per_tile = (nkb + QKV_NW - 1) / QKV_NW;                // blocks of a tile per wave (upper bound)
+    const uint32_t bpt = (per_tile + QKV_UNITS - 1) / QKV_UNITS;          // batches per tile
+    const uint32_t n_batches = n_tiles * bpt;
+    h8_t wbuf[2][QKV_UNITS];
+    auto request = [&](h8_t(&buf)[QKV_UNITS], uint32_t batch) {
+        const uint32_t tile = batch / bpt, j0 = (batch % bpt) * QKV_UNITS;
+        const __half *p0;
+        size_t kb_stride;
+        bool ok;
+        tile_base(tile, p0, kb_stride, ok);
+#pragma unroll
+        for (int i = 0; i < QKV_UNITS; ++i) {
+            const uint32_t kb = (uint32_t)wave + (j0 + i) * QKV_NW;
+            const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+            buf[i] = (ok && kb < nkb) ? *reinterpret_cast<const h8_t *>(p0 + (size_t)kb * kb_stride) : z;
+        }
+    };
+    // The first input row is requested before the weights (a CU's vector loads return in request order), then the
+    // first two batches, which do not depend on the input.
+    constexpr int XPRE = 2;  // 16-byte pieces per thread: rows of up to 8192 features
+    h8_t x0[XPRE];
+#pragma unroll
+    for (int j = 0; j < XPRE; ++j) {
+        const uint32_t k8 = tid + j * QKV_NT;
+        const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+        x0[j] = k8 < K / 8 ? *reinterpret_cast<const h8_t *>(a.x + (size_t)m0 * K + k8 * 8) : z;
+    }
+    request(wbuf[0], 0);
+    if (n_batches > 1) request(wbuf[1], 1);
+
+    // Input rows of this pass into LDS, normalised: x * rsqrt(mean(x^2) + eps) * gamma in f32, rounded to f16.
+    for (uint32_t r = 0; r < cols; ++r) {
+        const __half *xr = a.x + (size_t)(m0 + r) * K;
+        unsigned char *dst = x_lds + (size_t)r * a.x_stride;
+        float ss = 0.0f;
+        for (uint32_t k8 = tid, j = 0; k8 < K / 8; k8 += QKV_NT, ++j) {
+            h8_t v;
+            if (r == 0 && j < (uint32_t)XPRE) v = j == 0 ? x0[0] : x0[1];
+            else v = *reinterpret_cast<const h8_t *>(xr + k8 * 8);
+            *reinterpret_cast<h8_t *>(dst + k8 * 16) = v;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ss += (float)v[i] * (float)v[i];
+        }
+        if (a.gamma) {
+            ss = wave_sum(ss);
+            if (lane == 0) red[wave] = ss;
+            __syncthreads();
+            float tot = 0.0f;
+#pragma unroll
+            for (int w = 0; w < QKV_NW; ++w) tot += red[w];
+            const float inv_rms = rsqrtf(tot / (float)K + a.eps);
+            for (uint32_t k8 = tid; k8 < K / 8; k8 += QKV_NT) {  // each thread rewrites what it wrote
+                h8_t v = *reinterpret_cast<const h8_t *>(dst + k8 * 16);
+                const h8_t g = *reinterpret_cast<const h8_t *>(a.gamma + k8 * 8);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v[i] = (_Float16)(((float)v[i] * inv_rms) * (float)g[i]);
+                *reinterpret_cast<h8_t *>(dst + k8 * 16) = v;
+            }
+            __syncthreads();  // `red` is reused by the next row
+        }
+    }
+    __syncthreads();
+
+    // Sums the 8 waves' partial results of tile t in wave order, adds the bias, rounds once, stores token-major.
+    auto finish_tile = [&](uint32_t t, const f4v_t &mine) {
+        __syncthreads();  // `red` may still be read for the previous tile
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[((size_t)wave * 16 + c * 4 + i) * 17 + n] = mine[i];
+        __syncthreads();
+        if (tid < 256) {
+            const int row = tid >> 4, col = tid & 15;
+            const uint32_t gr = row_begin + t * 16 + row;
+            if (gr < row_end && (uint32_t)col < cols) {
+                float s = 0.0f;
+#pragma unroll
+                for (int w = 0; w < QKV_NW; ++w) s += red[((size_t)w * 16 + row) * 17 + col];
+                int mat;
+                uint32_t lrow;
+                locate(gr, mat, lrow);
+                const __half *bias = mat == 0 ? a.bias[0] : mat == 1 ? a.bias[1] : a.bias[2];
+                __half *out = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
+                const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
+                if (bias) s += __half2float(bias[lrow]);
+                out[(size_t)(m0 + col) * N + lrow] = __float2half(s);
+            }
+        }
+    };
+
+    // Stream: d = 16 rows of the current tile x 16 input rows, this wave's share of the feature blocks. Batches run
+    // tile after tile and every wave sees the same sequence, so a tile is finished when its last batch is consumed.
+    f4v_t d = {0.0f, 0.0f, 0.0f, 0.0f};
+    const bool col_ok = (uint32_t)n < cols;
+    const unsigned char *x_lane = x_lds + (size_t)(col_ok ? n : 0) * a.x_stride + c * 16;
+    auto consume = [&](const h8_t(&buf)[QKV_UNITS], uint32_t batch) {
+        const uint32_t tile = batch / bpt, j0 = (batch % bpt) * QKV_UNITS;
+#pragma unroll
+        for (int i = 0; i < QKV_UNITS; ++i) {
+            const uint32_t kb = (uint32_t)wave + (j0 + i) * QKV_NW;
+            if (kb >= nkb) break;  // wave-uniform
+            h8_t xb = *reinterpret_cast<const h8_t *>(x_lane + kb * 64);
+            if (!col_ok) xb = h8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            d = __builtin_amdgcn_mfma_f32_16x16x32_f16(buf[i], xb, d, 0, 0, 0);
+        }
+        if ((batch + 1) % bpt == 0) {
+            finish_tile(tile, d);
+            d = f4v_t{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    };
+    for (uint32_t b = 0; b < n_batches; b += 2) {
+        consume(wbuf[0], b);
+        if (b + 2 < n_batches) request(wbuf[0], b + 2);
+        if (b + 1 < n_batches) {
+            consume(wbuf[1], b + 1);
+            if (b + 3 < n_batches) request(wbuf[1], b + 3);
+        }
+    }
+}
+
+}  // namespace
+
+fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
+    QkvDev a;
+    for (int i = 0; i < 3; ++i) a.w[i] = l.w[i], a.bias[i] = l.bias[i], a.out[i] = l.out[i];
+    a.rows[0] = l.n_dim, a.rows[1] = l.n_kv, a.rows[2] = l.n_kv;
+    a.x = l.x, a.gamma = l.gamma, a.k_dim = l.k_dim, a.m = l.m, a.eps = l.eps, a.canonical = l.canonical ? 1u : 0u;
+    const uint32_t total_rows = l.n_dim + 2 * l.n_kv;
+    const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
+    // Workgroups: a multiple of the CU count, enough of them that a workgroup's rows fit one 16-row tile where the
+    // matrix allows (5120 rows, 256 CUs: 512 workgroups of 10 rows, two resident per CU - every CU requests the same
+    // bytes, and all of a wave's blocks are in flight at once); at most 64 rows (4 tiles) per workgroup. Measured on
+    // 5120 x 3072: 10 rows 9.35 us, 16 rows (320 workgroups) 9.18, 20 rows (one workgroup per CU, two tiles) 10.8,
+    // 8 rows (640 workgroups, a third of them waiting for a slot) 13.3.
+    uint32_t n_wg = n_cus * ceil_div_u32(ceil_div_u32(total_rows, 16), n_cus);
+    uint32_t rows_per_wg = ceil_div_u32(total_rows, n_wg);
+    if (rows_per_wg > 64) rows_per_wg = 64;
+    a.rows_per_wg = rows_per_wg;
+    a.x_stride = l.k_dim * 2 + 64;  // 64 bytes of padding: the 64 lanes of an operand read fall into different banks
+    const uint32_t lds_budget = 128u * 1024u;
+    uint32_t cols = lds_budget / a.x_stride;
+    if (cols == 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: k_dim %u is too large for one input row in LDS", l.k_dim);
+    if (cols > 16) cols = 16;
+    if (cols > l.m) cols = l.m;
+    a.cols_per_pass = cols;
+    const size_t lds = (size_t)cols * a.x_stride + (size_t)QKV_NW * 16 * 17 * sizeof(float);
+    static bool lds_allowed = false;
+    if (!lds_allowed) {
+        FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)(lds_budget + 16 * 1024)));
+        lds_allowed = true;
+    }
+    const dim3 grid(ceil_div_u32(total_rows, rows_per_wg), ceil_div_u32(l.m, cols));
+    if (grid.y > 65535u) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv m %u needs %u passes", l.m, grid.y);
+    FaLaunchScope scope(ctx, "fused_qkv_kernel", true);
+    scope.launch(fused_qkv_kernel, grid, dim3(QKV_NT), lds, a);
+    return scope.finish();
+}

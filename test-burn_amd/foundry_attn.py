@@ -49,6 +49,15 @@ class KvPrepFusedParams(C.Structure):
                    no_rope_layer_step)
 
 
+class FusedQkvParams(C.Structure):
+    """fa_fused_qkv_params (FusedQkvArgs scalars, src/metals/gemv/qkv_step.rs:57-99)."""
+    _fields_ = [("k_dim", C.c_uint32), ("n_dim", C.c_uint32), ("n_kv", C.c_uint32), ("m", C.c_uint32),
+                ("weights_per_block", C.c_uint32), ("layout", C.c_uint32), ("epsilon", C.c_float)]
+
+
+WEIGHT_LAYOUT_ROW_MAJOR, WEIGHT_LAYOUT_CANONICAL = 0, 1
+
+
 class DecodeVariant(C.Structure):
     _fields_ = [("keys_per_split", C.c_uint32), ("merge", C.c_uint32)]
 
@@ -106,6 +115,7 @@ PROTOTYPES = {
     "fa_flash_prefill_paged": [_vp, _PT, C.POINTER(PagedKv), _u32, _PT, _i, _u32, _u32, _u32, _u32],
     "fa_paged_gather": [_vp, C.POINTER(PagedKv), _u32, _u32, _vp, _vp, _u32],
     "fa_paged_copy_blocks": [_vp, C.POINTER(PagedKv), _vp, _vp, _u32],
+    "fa_fused_qkv": [_vp] + [_PT] * 11 + [C.POINTER(FusedQkvParams)],
     "fa_kv_prefix_copy": [_vp, _PT, _PT, _sz],
     "fa_kv_prefix_copy_batch": [_vp, _PT, _PT, _u32, _sz],
     "fa_align_capacity": [_sz],
@@ -346,6 +356,16 @@ class Foundry:
 
     def paged_gather(self, cache, seq_index, seq_len, k_out, v_out, out_capacity):
         check(self.lib.fa_paged_gather(self.h, C.byref(cache), seq_index, seq_len, k_out.ptr, v_out.ptr, out_capacity))
+
+    def fused_qkv(self, x, w_q, w_k, w_v, out_q, out_k, out_v, k_dim, n_dim, n_kv, m=1, gamma=None, biases=None,
+                  layout=WEIGHT_LAYOUT_CANONICAL, weights_per_block=32, epsilon=1e-6):
+        """All tensors as TensorArg; gamma None = no RMSNorm; biases None or (bias_q, bias_k, bias_v)."""
+        p = FusedQkvParams(k_dim, n_dim, n_kv, m, weights_per_block, layout, epsilon)
+        none = TensorArg()
+        g = gamma if gamma is not None else none
+        bq, bk, bv = biases if biases is not None else (none, none, none)
+        check(self.lib.fa_fused_qkv(self.h, C.byref(x), C.byref(w_q), C.byref(w_k), C.byref(w_v), C.byref(g), C.byref(bq),
+                                    C.byref(bk), C.byref(bv), C.byref(out_q), C.byref(out_k), C.byref(out_v), C.byref(p)))
 
     def paged_copy_blocks(self, cache, src_ids, dst_ids, n_pairs):
         """src_ids / dst_ids: device i32 buffers."""

@@ -23,6 +23,8 @@
 #include <utility>
 #include <vector>
 
+#include <algorithm>
+
 #include "foundry_attn.h"
 
 namespace metallic_foundry {
@@ -395,6 +397,68 @@ inline void CompiledFlashAttentionStep::execute(Foundry &foundry, const FastBind
     check(fa_flash_attention(foundry.ctx(), q.c(), k.c(), v.c(), out.c(), s.causal ? 1 : 0, s.query_offset.resolve(bindings),
                              s.n_heads.resolve(bindings), s.head_dim.resolve(bindings), s.kv_seq_len.resolve(bindings), m,
                              s.kv_head_major ? 1 : 0));
+}
+
+// ---------------------------------------------------------------------------------------------- FusedQkv
+enum class WeightLayout : uint32_t { RowMajor = FA_WEIGHT_LAYOUT_ROW_MAJOR, Canonical = FA_WEIGHT_LAYOUT_CANONICAL };
+
+struct FusedQkvStep;
+struct CompiledFusedQkvStep : CompiledStep {
+    const FusedQkvStep *step;
+    size_t input_idx, w_q_idx, w_k_idx, w_v_idx, out_q_idx, out_k_idx, out_v_idx;
+    std::optional<size_t> gamma_idx, bias_q_idx, bias_k_idx, bias_v_idx;
+    void execute(Foundry &foundry, const FastBindings &fast, const TensorBindings &bindings, const SymbolTable &) const override;
+    const char *name() const override { return "FusedQkv"; }
+};
+
+// src/metals/gemv/qkv_step.rs:14-37: RMSNorm(input) -> parallel Q/K/V projection -> three outputs. The scale
+// tensors (s_q, s_k, s_v) and `strategy` of the reference belong to its block-quantised policies and dispatch
+// tuning and have no counterpart; `rms_eps` is the reference's string variable of that name (default 1e-6).
+struct FusedQkvStep {
+    Ref input, w_q, w_k, w_v, out_q, out_k, out_v;
+    std::optional<Ref> gamma, bias_q, bias_k, bias_v;
+    DynamicU32 k_dim, n_dim, n_kv, m, weights_per_block = 32;
+    WeightLayout layout = WeightLayout::Canonical;
+    float rms_eps = 1e-6f;
+    std::vector<std::unique_ptr<CompiledStep>> compile(TensorBindings &b, SymbolTable &s) const {
+        auto c = std::make_unique<CompiledFusedQkvStep>();
+        c->step = this;
+        c->input_idx = s.get_or_create(b.interpolate(input));
+        c->w_q_idx = s.get_or_create(b.interpolate(w_q)), c->w_k_idx = s.get_or_create(b.interpolate(w_k));
+        c->w_v_idx = s.get_or_create(b.interpolate(w_v));
+        c->out_q_idx = s.get_or_create(b.interpolate(out_q)), c->out_k_idx = s.get_or_create(b.interpolate(out_k));
+        c->out_v_idx = s.get_or_create(b.interpolate(out_v));
+        auto opt = [&](const std::optional<Ref> &r) -> std::optional<size_t> {
+            if (!r) return std::nullopt;
+            return s.get_or_create(b.interpolate(*r));
+        };
+        c->gamma_idx = opt(gamma), c->bias_q_idx = opt(bias_q), c->bias_k_idx = opt(bias_k), c->bias_v_idx = opt(bias_v);
+        std::vector<std::unique_ptr<CompiledStep>> out;
+        out.push_back(std::move(c));
+        return out;
+    }
+    void execute(Foundry &foundry, TensorBindings &bindings) const { execute_step(*this, foundry, bindings); }
+    const char *name() const { return "FusedQkv"; }
+};
+
+inline void CompiledFusedQkvStep::execute(Foundry &foundry, const FastBindings &fast, const TensorBindings &bindings,
+                                          const SymbolTable &) const {
+    const FusedQkvStep &s = *step;
+    const TensorArg input = TensorArg::from_tensor(need(fast, input_idx, "input"));
+    const TensorArg w_q = TensorArg::from_tensor(need(fast, w_q_idx, "w_q")), w_k = TensorArg::from_tensor(need(fast, w_k_idx, "w_k"));
+    const TensorArg w_v = TensorArg::from_tensor(need(fast, w_v_idx, "w_v"));
+    const TensorArg out_q = TensorArg::from_tensor(need(fast, out_q_idx, "out_q")), out_k = TensorArg::from_tensor(need(fast, out_k_idx, "out_k"));
+    const TensorArg out_v = TensorArg::from_tensor(need(fast, out_v_idx, "out_v"));
+    auto opt = [&](const std::optional<size_t> &idx, const char *what) {
+        return idx ? TensorArg::from_tensor(need(fast, *idx, what)) : TensorArg();
+    };
+    const TensorArg gamma = opt(gamma_idx, "gamma"), b_q = opt(bias_q_idx, "bias_q"), b_k = opt(bias_k_idx, "bias_k"), b_v = opt(bias_v_idx, "bias_v");
+    fa_fused_qkv_params p;
+    p.k_dim = s.k_dim.resolve(bindings), p.n_dim = s.n_dim.resolve(bindings), p.n_kv = s.n_kv.resolve(bindings);
+    p.m = std::max<uint32_t>(s.m.resolve(bindings), 1);  // qkv_step.rs:236
+    p.weights_per_block = s.weights_per_block.resolve(bindings), p.layout = (uint32_t)s.layout, p.epsilon = s.rms_eps;
+    check(fa_fused_qkv(foundry.ctx(), input.c(), w_q.c(), w_k.c(), w_v.c(), gamma.c(), b_q.c(), b_k.c(), b_v.c(), out_q.c(), out_k.c(),
+                       out_v.c(), &p));
 }
 
 }  // namespace metallic_foundry

@@ -417,6 +417,51 @@ static void test_session_prefill_chunks_decode_loop_growth_snapshot(Foundry &fou
     EXPECT(thrown_by([&] { restore_kv_prefix_snapshot(foundry, small, *snap); }) == MetalError::InvalidShape);
 }
 
+// tests/qkv_parity_f16.rs:88-339: the fused QKV step at K 1024, N 1024, N_kv 128 with RMSNorm and biases against the
+// test's CPU helpers (here: the oracle's transcription of them), and the canonical weight layout the models use.
+static void test_fused_qkv_step(Foundry &foundry, WeightLayout layout) {
+    const size_t K = 1024, N = 1024, NKV = 128;
+    Rng rng{2024};
+    auto x = rng.fill(K, 1.0f), gamma = rng.fill(K, 0.5f);
+    for (auto &g : gamma) g = orc_f32_to_f16(orc_f16_to_f32(g) + 1.0f);  // 0.5 .. 1.5
+    auto wq = rng.fill(N * K, 0.1f), wk = rng.fill(NKV * K, 0.1f), wv = rng.fill(NKV * K, 0.1f);
+    auto bq = rng.fill(N, 0.1f), bk = rng.fill(NKV, 0.1f), bv = rng.fill(NKV, 0.1f);
+    std::vector<orc_f16> want_q(N), want_k(NKV), want_v(NKV);
+    orc_fused_qkv(x.data(), wq.data(), wk.data(), wv.data(), gamma.data(), bq.data(), bk.data(), bv.data(), want_q.data(), want_k.data(),
+                  want_v.data(), (uint32_t)K, (uint32_t)N, (uint32_t)NKV, 1, 0, 32, 1e-6f, 4);
+    auto arrange = [&](const std::vector<orc_f16> &w, size_t rows) {
+        if (layout == WeightLayout::RowMajor) return w;
+        std::vector<orc_f16> c(w.size());
+        for (size_t r = 0; r < rows; ++r)
+            for (size_t k = 0; k < K; ++k) c[orc_weight_index(1, r, k, K, rows, 32)] = w[r * K + k];
+        return c;
+    };
+    TensorBindings b;
+    b.set_int_global("i", 3);
+    b.insert("hidden", foundry.from_host(Dtype::F16, {1, K}, x.data()));
+    b.insert("layer.attn_norm_3", foundry.from_host(Dtype::F16, {K}, gamma.data()));
+    b.insert("layer.wq_3", foundry.from_host(Dtype::F16, {N * K}, arrange(wq, N).data()));
+    b.insert("layer.wk_3", foundry.from_host(Dtype::F16, {NKV * K}, arrange(wk, NKV).data()));
+    b.insert("layer.wv_3", foundry.from_host(Dtype::F16, {NKV * K}, arrange(wv, NKV).data()));
+    b.insert("layer.bq_3", foundry.from_host(Dtype::F16, {N}, bq.data()));
+    b.insert("layer.bk_3", foundry.from_host(Dtype::F16, {NKV}, bk.data()));
+    b.insert("layer.bv_3", foundry.from_host(Dtype::F16, {NKV}, bv.data()));
+    b.insert("q", foundry.zeros(Dtype::F16, {1, N}));
+    b.insert("k", foundry.zeros(Dtype::F16, {1, NKV}));
+    b.insert("v", foundry.zeros(Dtype::F16, {1, NKV}));
+    FusedQkvStep step{"hidden", "layer.wq_{i}", "layer.wk_{i}", "layer.wv_{i}", "q", "k", "v"};
+    step.gamma = "layer.attn_norm_{i}", step.bias_q = "layer.bq_{i}", step.bias_k = "layer.bk_{i}", step.bias_v = "layer.bv_{i}";
+    step.k_dim = (uint32_t)K, step.n_dim = (uint32_t)N, step.n_kv = (uint32_t)NKV, step.m = 0 /* treated as 1 */, step.layout = layout;
+    step.execute(foundry, b);
+    foundry.synchronize();
+    auto q = foundry.to_host<orc_f16>(*b.get("q")), k = foundry.to_host<orc_f16>(*b.get("k")), v = foundry.to_host<orc_f16>(*b.get("v"));
+    EXPECT(max_abs_diff(want_q, q, N) <= 8e-3f && max_abs_diff(want_k, k, NKV) <= 8e-3f && max_abs_diff(want_v, v, NKV) <= 8e-3f);
+    FusedQkvStep missing = step;
+    missing.bias_k = "not_bound";
+    EXPECT(thrown_by([&] { missing.execute(foundry, b); }) == MetalError::InputNotFound);
+    foundry.synchronize();
+}
+
 int main(int argc, char **argv) {
     const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu";
     run_test("bindings and dynamic values", test_bindings_and_dynamic_values);
@@ -439,6 +484,8 @@ int main(int argc, char **argv) {
             }
         run_test("closed-form prefill H2 N15 D64", [&] { test_closed_form_prefill(foundry); });
         run_test("error variants", [&] { test_error_variants(foundry); });
+        run_test("fused qkv step, row-major weights", [&] { test_fused_qkv_step(foundry, WeightLayout::RowMajor); });
+        run_test("fused qkv step, canonical weights", [&] { test_fused_qkv_step(foundry, WeightLayout::Canonical); });
         run_test("session: chunked prefill, snapshot, decode loop with growth, restore",
                  [&] { test_session_prefill_chunks_decode_loop_growth_snapshot(foundry); });
     }

@@ -216,6 +216,40 @@ def paged_gather(pool, block_table, n_kv_heads, block_size, head_dim, seq_len, o
     return out
 
 
+def weight_index(layout, row, k, k_dim, n_rows, wpb=32):
+    L = lib()
+    L.orc_weight_index.restype = C.c_size_t
+    return L.orc_weight_index(C.c_int(layout), C.c_size_t(row), C.c_size_t(k), C.c_size_t(k_dim), C.c_size_t(n_rows),
+                              C.c_size_t(wpb))
+
+
+def to_canonical(w, wpb=32):
+    """[n_rows, k_dim] row-major -> the canonical blocked order (flat), by the layout's own index formula."""
+    n, k = w.shape
+    kk = np.arange(k)
+    idx = (kk % wpb)[None, :] + wpb * (np.arange(n)[:, None] + (kk // wpb)[None, :] * n)
+    out = np.empty(n * k, w.dtype)
+    out[idx.reshape(-1)] = w.reshape(-1)
+    return out
+
+
+def fused_qkv(x, w_q, w_k, w_v, gamma=None, biases=None, layout=0, wpb=32, eps=1e-6, n_threads=8):
+    """x [m, K]; w_* flat or 2-D in `layout`; returns (q [m, n_dim], k [m, n_kv], v [m, n_kv])."""
+    x = _h(x)
+    m, K = x.shape
+    wq, wk, wv = (_h(np.asarray(w).reshape(-1)) for w in (w_q, w_k, w_v))
+    n_dim, n_kv = wq.size // K, wk.size // K
+    oq, ok, ov = np.zeros((m, n_dim), np.float16), np.zeros((m, n_kv), np.float16), np.zeros((m, n_kv), np.float16)
+    g = _h(gamma) if gamma is not None else None
+    bs = [_h(b) for b in biases] if biases is not None else [None] * 3
+    nul = C.cast(None, u16p)
+    lib().orc_fused_qkv(_p(x, u16p), _p(wq, u16p), _p(wk, u16p), _p(wv, u16p), _p(g, u16p) if g is not None else nul,
+                        *[(_p(b, u16p) if b is not None else nul) for b in bs], _p(oq, u16p), _p(ok, u16p), _p(ov, u16p),
+                        C.c_uint32(K), C.c_uint32(n_dim), C.c_uint32(n_kv), C.c_uint32(m), C.c_int(layout), C.c_uint32(wpb),
+                        C.c_float(eps), C.c_int(n_threads))
+    return oq, ok, ov
+
+
 def paged_copy_blocks(pool, n_kv_heads, block_size, head_dim, src_ids, dst_ids):
     """In place on `pool` [n_blocks, n_kv_heads, block_size, head_dim] f16."""
     assert pool.dtype == np.float16 and pool.flags.c_contiguous

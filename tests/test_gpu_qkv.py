@@ -1,0 +1,127 @@
+"""GPU parity: FusedQkv (RMSNorm -> Q/K/V projections, F16 weights) against the oracle's restatement of the
+reference test's CPU helpers (tests/qkv_parity_f16.rs:17-72). The reference accepts |diff| < 0.1 there; the bar
+here is two f16 units in the last place of the expected value (f32 sums of k_dim products in another order, rounded
+once), plus the f16 rounding of a normalised input that sits on a rounding boundary (rsqrt against 1/sqrt)."""
+import numpy as np
+import pytest
+
+import foundry_attn as fa
+import orc
+from gpu_util import announce, ctx
+
+pytestmark = pytest.mark.gpu
+
+
+def _data(rng, K, N, NK, m):
+    # distributions of tests/qkv_parity_f16.rs:100-118
+    x = rng.uniform(-1, 1, (m, K)).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, K).astype(np.float16)
+    ws = [rng.uniform(-0.1, 0.1, (n, K)).astype(np.float16) for n in (N, NK, NK)]
+    bs = [rng.uniform(-0.1, 0.1, n).astype(np.float16) for n in (N, NK, NK)]
+    return x, g, ws, bs
+
+
+def _close(got, want, K):
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    ulp = np.maximum(np.abs(w), 2.0 ** -10) * 2.0 ** -10
+    # the f16 rounding of the normalised input may differ in isolated elements (rsqrt vs 1/sqrt): each moves a sum by
+    # one input ulp (2^-10 relative of |x| <= 2) times |w| <= 0.1
+    slack = 4 * 2.0 ** -10 * 0.1
+    return bool(np.all(np.abs(g - w) <= 2 * ulp + slack))
+
+
+@pytest.mark.parametrize("K,N,NK,m,norm,bias,layout", [
+    (1024, 1024, 128, 1, True, True, 0),      # the reference test's shape (tests/qkv_parity_f16.rs:92-95), row-major
+    (1024, 1024, 128, 1, True, True, 1),      # same, canonical blocked weights
+    (3072, 3072, 1024, 1, True, False, 1),    # Llama-3.2-3B decode
+    (896, 896, 128, 1, True, True, 1),        # Qwen2.5-0.5B (biases)
+    (2048, 2048, 256, 1, False, False, 1),    # no RMSNorm
+    (3072, 3072, 1024, 5, True, False, 1),    # a few tokens
+    (896, 896, 128, 32, True, True, 1),       # a default prefill chunk: two passes of 16 input rows
+    (896, 896, 128, 17, True, True, 0),
+    (64, 40, 24, 3, True, True, 1),           # rows that do not fill tiles, tiles that straddle the three matrices
+    (8192, 256, 64, 2, True, False, 1),       # long rows: more units than one request batch
+])
+def test_fused_qkv_equals_oracle(K, N, NK, m, norm, bias, layout):
+    announce("fused qkv", K, N, NK, m, norm, bias, layout)
+    f = ctx()
+    rng = np.random.default_rng(K + N + m)
+    x, g, ws, bs = _data(rng, K, N, NK, m)
+    want = orc.fused_qkv(x, *ws, gamma=g if norm else None, biases=bs if bias else None, layout=0)
+    dev_w = [f.array(orc.to_canonical(w) if layout == 1 else w.reshape(-1)) for w in ws]
+    dx, dg = f.array(x), f.array(g)
+    db = [f.array(b) for b in bs]
+    outs = [f.zeros((m, n)) for n in (N, NK, NK)]
+    f.fused_qkv(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), outs[0].arg(), outs[1].arg(), outs[2].arg(),
+                K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout)
+    for o, w, name in zip(outs, want, "qkv"):
+        got = o.download()
+        assert np.all(np.isfinite(got)), name
+        assert _close(got, w, K), (name, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
+    for b in dev_w + [dx, dg] + db + outs:
+        b.free()
+
+
+def test_fused_qkv_feeds_kv_prep_and_decode():
+    """The step before the path and the path: FusedQkv -> fused RoPE + append + decode equals the oracle's chain."""
+    announce("fused qkv -> decode step")
+    f = ctx()
+    rng = np.random.default_rng(77)
+    H, Hkv, D, K, cap, pos = 8, 2, 64, 512, 256, 100
+    x, g, ws, _ = _data(rng, K, H * D, Hkv * D, 1)
+    kc = rng.normal(size=(Hkv, cap, D)).astype(np.float16)
+    vc = rng.normal(size=(Hkv, cap, D)).astype(np.float16)
+    cos, sin = fa.rope_tables(1e4, D, cap)
+    q, k, v = orc.fused_qkv(x, *ws, gamma=g)
+    kc_w, vc_w = kc.copy(), vc.copy()
+    qr = orc.kv_prep_fused(q, k, v, kc_w, vc_w, cos, sin, orc.make_params(H, Hkv, D, 1, pos, cap, rope_mode=0))
+    want = orc.sdpa_decode(qr[:, 0].copy(), kc_w, vc_w, H, Hkv, D, cap, pos + 1)
+    dev_w = [f.array(orc.to_canonical(w)) for w in ws]
+    dx, dg, dkc, dvc, dcos, dsin = f.array(x), f.array(g), f.array(kc), f.array(vc), f.array(cos), f.array(sin)
+    dq, dk, dv, dout = f.zeros((1, H * D)), f.zeros((1, Hkv * D)), f.zeros((1, Hkv * D)), f.zeros((1, H * D))
+    f.fused_qkv(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), dq.arg(), dk.arg(), dv.arg(), K, H * D, Hkv * D, 1,
+                gamma=dg.arg())
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, 1, pos, cap, fa.ROPE_NEOX)
+    f.decode_step_fused(dq.arg(), dk.arg(), dv.arg(), None, dkc.arg(), dvc.arg(), dcos.arg(), dsin.arg(), dout.arg(), p)
+    got = dout.download().reshape(H, D).astype(np.float64)
+    assert float(np.max(np.abs(got - want.reshape(H, D).astype(np.float64)))) <= 4e-3  # projection ulps carried through
+    for b in dev_w + [dx, dg, dkc, dvc, dcos, dsin, dq, dk, dv, dout]:
+        b.free()
+
+
+def test_fused_qkv_errors():
+    announce("fused qkv errors")
+    f = ctx()
+    K, N, NK = 64, 32, 16
+    x, wq, wk, wv = f.zeros((1, K)), f.zeros((N * K,)), f.zeros((NK * K,)), f.zeros((NK * K,))
+    oq, ok, ov = f.zeros((1, N)), f.zeros((1, NK)), f.zeros((1, NK))
+    args = lambda: (x.arg(), wq.arg(), wk.arg(), wv.arg(), oq.arg(), ok.arg(), ov.arg())  # noqa: E731
+    f.fused_qkv(*args(), K, N, NK, 1)  # fine
+    w8 = f.zeros((N * K,), np.int8)
+    with pytest.raises(fa.FoundryError) as e:  # block-quantised policies are not built
+        f.fused_qkv(x.arg(), w8.arg(), wk.arg(), wv.arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1)
+    assert e.value.variant == "UnsupportedDtype"
+    with pytest.raises(fa.FoundryError) as e:
+        f.fused_qkv(*args(), 48, N, NK, 1)
+    assert e.value.variant in ("OperationNotSupported", "InvalidShape")
+    with pytest.raises(fa.FoundryError) as e:
+        f.fused_qkv(*args(), K, N, NK, 1, weights_per_block=64)
+    assert e.value.variant == "OperationNotSupported"
+    with pytest.raises(fa.FoundryError) as e:
+        f.fused_qkv(*args(), K, N + 1, NK, 1)
+    assert e.value.variant == "InvalidShape"
+    with pytest.raises(fa.FoundryError) as e:
+        f.fused_qkv(*args(), K, N, NK, 2)
+    assert e.value.variant == "InvalidShape"
+    b = f.zeros((N,))
+    with pytest.raises(fa.FoundryError) as e:  # bias_q without bias_k / bias_v
+        f.fused_qkv(*args(), K, N, NK, 1, biases=(b.arg(), fa.TensorArg(), fa.TensorArg()))
+    assert e.value.variant == "InputNotFound"
+    t = x.arg()
+    t.buffer = None
+    with pytest.raises(fa.FoundryError) as e:
+        f.fused_qkv(t, wq.arg(), wk.arg(), wv.arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1)
+    assert e.value.variant == "InputNotFound"
+    f.synchronize()
+    for z in (x, wq, wk, wv, oq, ok, ov, w8, b):
+        z.free()

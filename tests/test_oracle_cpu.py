@@ -593,3 +593,52 @@ def test_paged_copy_blocks_index_map():
     got = pool.copy()
     orc.paged_copy_blocks(got, 2, 16, 8, [1, 3, 2, -1, 6, 4], [5, 0, 2, 1, 0, 9])
     assert np.array_equal(got, want)
+
+
+# ---------------------------------------------------------------- FusedQkv
+
+def test_weight_index_layouts():
+    """Row-major is row*K + k; the canonical layout is a bijection onto [0, N*K) that keeps each 32-feature block of a
+    row contiguous and places block kb of row n at 32*(n + kb*N) (src/compound/stages/layout.rs:95-100,
+    src/metals/gemv/qkv_project.metal:83-96)."""
+    K, N = 96, 7
+    seen = set()
+    for n in range(N):
+        for k in range(K):
+            assert orc.weight_index(0, n, k, K, N) == n * K + k
+            i = orc.weight_index(1, n, k, K, N)
+            assert i == (k & 31) + (n << 5) + (k & ~31) * N  # the kernel's own fast form for weights_per_block = 32
+            seen.add(i)
+    assert seen == set(range(N * K))
+    w = np.arange(N * K, dtype=np.float32).reshape(N, K).astype(np.float16)
+    c = orc.to_canonical(w)
+    assert np.array_equal(c.reshape(K // 32, N, 32)[1, 3], w[3, 32:64])
+
+
+@pytest.mark.parametrize("K,N,NK,m,norm,bias", [(1024, 1024, 128, 1, True, True), (64, 40, 24, 3, True, False),
+                                                 (96, 16, 8, 2, False, True)])
+def test_fused_qkv_vs_float64(K, N, NK, m, norm, bias):
+    """Against float64 matrix products on the same f16-rounded normalised input, with the reference test's data
+    distributions (tests/qkv_parity_f16.rs:100-118); both layouts give the same bits."""
+    rng = np.random.default_rng(K + m)
+    x = rng.uniform(-1, 1, (m, K)).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, K).astype(np.float16)
+    ws = [rng.uniform(-0.1, 0.1, (n, K)).astype(np.float16) for n in (N, NK, NK)]
+    bs = [rng.uniform(-0.1, 0.1, n).astype(np.float16) for n in (N, NK, NK)]
+    got = orc.fused_qkv(x, *ws, gamma=g if norm else None, biases=bs if bias else None)
+    got_c = orc.fused_qkv(x, *[orc.to_canonical(w) for w in ws], gamma=g if norm else None, biases=bs if bias else None, layout=1)
+    xf = x.astype(np.float32)
+    if norm:
+        inv = (1.0 / np.sqrt((xf.astype(np.float64) ** 2).sum(1, keepdims=True) / K + 1e-6)).astype(np.float32)
+        xn = (xf * inv * g.astype(np.float32)).astype(np.float16).astype(np.float64)
+    else:
+        xn = xf.astype(np.float64)
+    for o, oc, w, b in zip(got, got_c, ws, bs):
+        assert np.array_equal(o, oc)
+        ref = xn @ w.astype(np.float64).T + (b.astype(np.float64) if bias else 0.0)
+        ulp = np.maximum(np.abs(ref), 2.0 ** -10) * 2.0 ** -10
+        assert np.all(np.abs(o.astype(np.float64) - ref) <= 1.5 * ulp + 1e-4)
+    # identity weights: the projection returns the normalised input
+    eye = np.eye(K, dtype=np.float16)
+    q, _, _ = orc.fused_qkv(x, eye, eye[:8], eye[:8], gamma=g if norm else None)
+    assert np.array_equal(q.astype(np.float64), xn)
