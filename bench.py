@@ -417,6 +417,46 @@ def bench_fused_qkv(f, args):
     f.profile_enable(False)
 
 
+def bench_o_proj(f, args):
+    """The step after the path at Llama-3.2-3B decode shape: attn_out [1, 3072] x W_o^T + hidden (MatMul with residual,
+    alpha = beta = 1), F16 weights in the canonical blocked layout, one layer per step over 12 layers' weights."""
+    import orc
+    K, N, NL = 3072, 3072, 12
+    rng = np.random.default_rng(0xF0DD + 8)
+    x = rng.uniform(-1, 1, (1, K)).astype(np.float16)
+    c = rng.uniform(-1, 1, (1, N)).astype(np.float16)
+    layers, host0 = [], None
+    for i in range(NL):  # distinct weights so that no launch finds the previous one's in cache
+        w = rng.uniform(-0.1, 0.1, (N, K)).astype(np.float16)
+        layers.append(f.array(orc.to_canonical(w)))
+        if i == 0:
+            host0 = w
+    dx, dc, out = f.array(x), f.array(c), f.zeros((1, N))
+
+    def step(i):
+        f.matmul(dx.arg(), layers[i % NL].arg(), out.arg(), 1, N, K, c=dc.arg(), transpose_b=False, alpha=1.0, beta=1.0)
+
+    step(0)
+    f.synchronize()
+    want = orc.matmul_gemv(x, host0, None, c, 0, 32, 1.0, 1.0)
+    err = float(np.max(np.abs(out.download().astype(np.float64) - want.astype(np.float64))))
+    for i in range(args.warmup):
+        step(i)
+    f.synchronize()
+    f.profile_reset()
+    f.profile_enable(True)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    nbytes = 2.0 * N * K + 2 * K + 2 * 2 * N  # weights, input, residual + output
+    _finish_secondary(f, args, "o_proj MatMul layer-steps/s + achieved HBM GB/s, Llama-3.2-3B decode shape",
+                      "llama3.2-3b o_proj at decode: attn_out [1, 3072] x W_o^T + hidden, n 3072, k 3072, F16 canonical "
+                      "weights, eager launches (profiling events on)", "matmul_gemv_kernel", nbytes, dt, {"max_abs_err": err})
+    f.profile_enable(False)
+
+
 def bench_paged_decode(f, args):
     """Qwen2.5-3B-shaped batched paged decode, one layer per step: 32 ragged sequences, 16-token blocks."""
     import orc
@@ -549,7 +589,8 @@ def bench_sage_decode(f, args):
 
 SECONDARY = {"llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
-             "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv}
+             "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
+             "llama3b_o_proj": bench_o_proj}
 
 
 def main():

@@ -389,6 +389,28 @@ fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *input, const fa_tensor_
                        const fa_tensor_arg *out_k, const fa_tensor_arg *out_v, const fa_fused_qkv_params *params);
 
 /* ---------------------------------------------------------------------------------------------
+ * MatMul, weight-stream form: the step after the path (o_proj: `attn_out [m, H*D]` x W_o, residual `hidden`,
+ * models/llama.json:566-585; op src/metals/matmul.rs:11-239, which runs GemvV2 for m == 1 and for canonical
+ * weights; write stage src/metals/gemv/stages.rs:200-224). F16 weights only.
+ *   output[b, r] = f16( alpha * sum_k a[b, k] * B[r, k] + bias[r] + beta * c[b, r] ),  r < n, b < m
+ * transpose_b != 0: B is row-major [n, k] (Layout::RowMajor); transpose_b == 0: B is in the canonical blocked
+ * layout (matmul.rs:199-207). transpose_a and activations other than none are not built
+ * (FA_ERR_OPERATION_NOT_SUPPORTED). bias, c: NULL or NULL buffer = absent (the reference's "zero" placeholder).
+ * Any m is accepted (16 input rows per pass over the weights); the reference's GEMM for large m is not built.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct fa_matmul_params {
+    uint32_t m, n, k;            /* k a multiple of 32 */
+    uint32_t transpose_a;        /* must be 0 */
+    uint32_t transpose_b;        /* 1: row-major [n, k]; 0: canonical blocked, weights_per_block = 32 */
+    float alpha, beta;           /* defaults of the op: 1.0, 0.0 */
+    uint32_t weights_per_block;  /* 32 */
+    uint32_t activation;         /* 0 = none */
+} fa_matmul_params;
+
+fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b, const fa_tensor_arg *output,
+                    const fa_tensor_arg *bias, const fa_tensor_arg *c, const fa_matmul_params *params);
+
+/* ---------------------------------------------------------------------------------------------
  * SageAttention-style int8 Q/K decode (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170 - prose only in
  * the reference). K is mean-smoothed over the sequence per (kv head, channel), then quantised per block
  * of 32 tokens: scale = max|k - mean| / 127 stored as f16, k_q = rint((k - mean)/scale) in [-127,127].

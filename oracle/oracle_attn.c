@@ -651,6 +651,26 @@ void orc_fused_qkv(const orc_f16 *x, const orc_f16 *w_q, const orc_f16 *w_k, con
     free(xn);
 }
 
+/* tests/gemv_v2_parity.rs:58-80 + src/metals/gemv/stages.rs:206-222 */
+void orc_matmul_gemv(const orc_f16 *x, const orc_f16 *w, const orc_f16 *bias, const orc_f16 *residual, orc_f16 *out,
+                     uint32_t m, uint32_t n, uint32_t k_dim, int layout, uint32_t wpb, float alpha, float beta, int n_threads) {
+    (void)n_threads;
+    for (uint32_t b = 0; b < m; ++b) {
+#ifdef _OPENMP
+#pragma omp parallel for num_threads(n_threads > 0 ? n_threads : 1) schedule(static)
+#endif
+        for (int64_t row = 0; row < (int64_t)n; ++row) {
+            float acc = 0.0f;
+            for (uint32_t ki = 0; ki < k_dim; ++ki)
+                acc += orc_f16_to_f32(w[orc_weight_index(layout, (size_t)row, ki, k_dim, n, wpb)]) * orc_f16_to_f32(x[(size_t)b * k_dim + ki]);
+            float res = acc * alpha;
+            if (bias) res += orc_f16_to_f32(bias[row]);
+            if (residual) res += orc_f16_to_f32(residual[(size_t)b * n + row]) * beta;
+            out[(size_t)b * n + row] = orc_f32_to_f16(res);
+        }
+    }
+}
+
 /* ------------------------------------------------------------------ Sage-style int8 Q/K */
 
 void orc_sage_k_mean(const orc_f16 *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim, uint32_t kv_len,

@@ -39,6 +39,10 @@
  *   orc_kv_prefix_copy        no reference test; a byte copy, pinned by brute-force index checks and by the
  *                             snapshot -> clobber -> restore round trip
  *   orc_paged_copy_blocks     no reference counterpart; pinned by gather(fork) == gather(parent) on the prefix
+ *   orc_matmul_gemv           pinned: transcription of the reference test's CPU helper (tests/gemv_v2_parity.rs:58-80)
+ *                             plus the write stage's residual term (src/metals/gemv/stages.rs:206-222, source only:
+ *                             no reference test exercises beta / residual -> that term is PARITY UNPINNED by tests,
+ *                             pinned here against float64 and by linearity in beta)
  *   orc_fused_qkv             pinned: transcription of the reference test's CPU helpers (tests/qkv_parity_f16.rs:17-72)
  *                             checked against float64 matrix products; orc_weight_index pinned as a bijection that
  *                             reduces to the row-major index per 32-feature block (src/compound/stages/layout.rs:79-100)
@@ -173,6 +177,13 @@ void orc_fused_qkv(const orc_f16 *x, const orc_f16 *w_q, const orc_f16 *w_k, con
                    const orc_f16 *bias_q, const orc_f16 *bias_k, const orc_f16 *bias_v, orc_f16 *out_q, orc_f16 *out_k,
                    orc_f16 *out_v, uint32_t k_dim, uint32_t n_dim, uint32_t n_kv, uint32_t m, int layout, uint32_t wpb,
                    float eps, int n_threads);
+
+/* MatMul at m rows through the GEMV path (src/metals/matmul.rs:190-239), F16 weights:
+ *   out[b, r] = f16(alpha * sum_k w[r,k]*x[b,k] + bias[r] + beta * residual[b, r])
+ * sum in f32 with k ascending (tests/gemv_v2_parity.rs:58-80); bias / residual NULL = absent
+ * (src/metals/gemv/stages.rs:206-222). layout / wpb as in orc_weight_index. */
+void orc_matmul_gemv(const orc_f16 *x, const orc_f16 *w, const orc_f16 *bias, const orc_f16 *residual, orc_f16 *out,
+                     uint32_t m, uint32_t n, uint32_t k_dim, int layout, uint32_t wpb, float alpha, float beta, int n_threads);
 
 /* Sage-style int8 Q/K (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170).
  * K smoothing: subtract per-(head, channel) mean over the sequence (f32), quantise per block of

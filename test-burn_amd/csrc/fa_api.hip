@@ -793,6 +793,49 @@ extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *input, const
     return fa_launch_fused_qkv(ctx, L);
 }
 
+extern "C" fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b, const fa_tensor_arg *output,
+                               const fa_tensor_arg *bias, const fa_tensor_arg *c, const fa_matmul_params *p) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(p, "params");
+    const struct { const fa_tensor_arg *t; const char *name; } req[] = {{a, "a"}, {b, "b"}, {output, "output"}};
+    for (const auto &r : req) {
+        FA_NEED(r.t, r.name);
+        if (!r.t->buffer) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: %s", r.name);
+    }
+    if (b->dtype != FA_DTYPE_F16)
+        return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "MatMul: weight dtype %u: only F16 weights are built (no block-quantised policies)", b->dtype);
+    if (a->dtype != FA_DTYPE_F16 || output->dtype != FA_DTYPE_F16) return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "MatMul: a and output must be F16");
+    if (p->transpose_a) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: transpose_a is not supported");
+    if (p->activation != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: activation %u is not built", p->activation);
+    const uint32_t m = p->m ? p->m : 1;
+    if (p->n == 0 || p->k == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: MatMul n %u k %u", p->n, p->k);
+    if (p->k % 32 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: k %u must be a multiple of 32", p->k);
+    if (!p->transpose_b && p->weights_per_block != 32)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: the canonical layout is built for weights_per_block = 32, got %u", p->weights_per_block);
+    if (a->rank == 0 || a->dims[a->rank - 1] != p->k || a->strides[a->rank - 1] != 1)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: MatMul a must have k %u as its contiguous last dim", p->k);
+    for (uint32_t i = 0; i + 1 < a->rank; ++i) {
+        size_t inner = 1;
+        for (uint32_t j = i + 1; j < a->rank; ++j) inner *= a->dims[j];
+        if (a->dims[i] > 1 && a->strides[i] != inner) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: rows of a must be contiguous");
+    }
+    if (numel(a) < (size_t)m * p->k || numel(b) < (size_t)p->n * p->k || numel(output) < (size_t)m * p->n)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: MatMul tensors smaller than m %u n %u k %u need", m, p->n, p->k);
+    const bool has_bias = present(bias), has_c = present(c);
+    if (has_bias && (bias->dtype != FA_DTYPE_F16 || numel(bias) < p->n)) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: MatMul bias must be F16 [n]");
+    if (has_c && (c->dtype != FA_DTYPE_F16 || numel(c) < (size_t)m * p->n)) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: MatMul c must be F16 [m, n]");
+    FusedQkvLaunch L;
+    L.w[0] = half_ptr(b), L.w[1] = L.w[2] = nullptr;
+    L.bias[0] = has_bias ? half_ptr(bias) : nullptr, L.bias[1] = L.bias[2] = nullptr;
+    L.out[0] = const_cast<__half *>(half_ptr(output)), L.out[1] = L.out[2] = nullptr;
+    L.x = half_ptr(a), L.gamma = nullptr;
+    L.k_dim = p->k, L.n_dim = p->n, L.n_kv = 0, L.m = m, L.eps = 0.0f;
+    L.canonical = p->transpose_b == 0;
+    L.residual = has_c ? half_ptr(c) : nullptr, L.alpha = p->alpha, L.beta = p->beta;
+    if ((uintptr_t)L.w[0] % 16 != 0 || (uintptr_t)L.x % 16 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: a and b must be 16-byte aligned");
+    return fa_launch_fused_qkv(ctx, L);
+}
+
 // ------------------------------------------------------------------------------------------------ FlashAttention
 
 struct KvLayout {

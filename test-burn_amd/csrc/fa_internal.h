@@ -175,6 +175,9 @@ struct FusedQkvLaunch {
     uint32_t k_dim, n_dim, n_kv, m;
     float eps;
     bool canonical;  // weights blocked by 32 features, else row-major [rows, k_dim]
+    // MatMul form (n_kv = 0, w[1] = w[2] = nullptr): out = f16(alpha * sum + bias + beta * residual)
+    const __half *residual = nullptr;
+    float alpha = 1.0f, beta = 0.0f;
 };
 fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l);
 

@@ -14,6 +14,10 @@
 //   * the 8 waves split the feature blocks of a tile; their 16 x 16 partial results are summed through LDS in a
 //     fixed order, the bias is added and the row is rounded to f16 once, as the reference does.
 // The normalised input is rounded to f16 before the products (qkv_project.metal:66-67), f32 accumulation.
+//
+// The same kernel with one matrix, no norm and the write stage's alpha / bias / beta * residual is the m = 1 path of
+// the MatMul op (src/metals/matmul.rs:190-239 -> GemvV2, write stage src/metals/gemv/stages.rs:200-224): the o_proj
+// consumer of the attention output.
 #include "fa_internal.h"
 
 namespace {
@@ -32,6 +36,9 @@ struct QkvDev {
     const __half *gamma;    // nullable: no RMSNorm
     uint32_t k_dim, m, cols_per_pass, rows_per_wg, x_stride /* bytes of an input row in LDS */, canonical;
     float eps;
+    // MatMul form (one matrix): out = f16(alpha * sum + bias + beta * residual)
+    const __half *residual;  // nullable; [m, rows[0]]
+    float alpha, beta;
 };
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -163,7 +170,9 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
                 const __half *bias = mat == 0 ? a.bias[0] : mat == 1 ? a.bias[1] : a.bias[2];
                 __half *out = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
                 const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
+                s *= a.alpha;
                 if (bias) s += __half2float(bias[lrow]);
+                if (a.residual) s += __half2float(a.residual[(size_t)(m0 + col) * N + lrow]) * a.beta;
                 out[(size_t)(m0 + col) * N + lrow] = __float2half(s);
             }
         }
@@ -206,6 +215,7 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     for (int i = 0; i < 3; ++i) a.w[i] = l.w[i], a.bias[i] = l.bias[i], a.out[i] = l.out[i];
     a.rows[0] = l.n_dim, a.rows[1] = l.n_kv, a.rows[2] = l.n_kv;
     a.x = l.x, a.gamma = l.gamma, a.k_dim = l.k_dim, a.m = l.m, a.eps = l.eps, a.canonical = l.canonical ? 1u : 0u;
+    a.residual = l.residual, a.alpha = l.alpha, a.beta = l.beta;
     const uint32_t total_rows = l.n_dim + 2 * l.n_kv;
     const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
     // Workgroups: a multiple of the CU count, enough of them that a workgroup's rows fit one 16-row tile where the
@@ -233,7 +243,7 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     }
     const dim3 grid(ceil_div_u32(total_rows, rows_per_wg), ceil_div_u32(l.m, cols));
     if (grid.y > 65535u) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv m %u needs %u passes", l.m, grid.y);
-    FaLaunchScope scope(ctx, "fused_qkv_kernel", true);
+    FaLaunchScope scope(ctx, l.n_kv ? "fused_qkv_kernel" : "matmul_gemv_kernel", true);
     scope.launch(fused_qkv_kernel, grid, dim3(QKV_NT), lds, a);
     return scope.finish();
 }

@@ -58,6 +58,13 @@ class FusedQkvParams(C.Structure):
 WEIGHT_LAYOUT_ROW_MAJOR, WEIGHT_LAYOUT_CANONICAL = 0, 1
 
 
+class MatMulParams(C.Structure):
+    """fa_matmul_params (MatMulStep scalars, src/metals/matmul.rs:11-31)."""
+    _fields_ = [("m", C.c_uint32), ("n", C.c_uint32), ("k", C.c_uint32), ("transpose_a", C.c_uint32),
+                ("transpose_b", C.c_uint32), ("alpha", C.c_float), ("beta", C.c_float), ("weights_per_block", C.c_uint32),
+                ("activation", C.c_uint32)]
+
+
 class DecodeVariant(C.Structure):
     _fields_ = [("keys_per_split", C.c_uint32), ("merge", C.c_uint32)]
 
@@ -116,6 +123,7 @@ PROTOTYPES = {
     "fa_paged_gather": [_vp, C.POINTER(PagedKv), _u32, _u32, _vp, _vp, _u32],
     "fa_paged_copy_blocks": [_vp, C.POINTER(PagedKv), _vp, _vp, _u32],
     "fa_fused_qkv": [_vp] + [_PT] * 11 + [C.POINTER(FusedQkvParams)],
+    "fa_matmul": [_vp] + [_PT] * 5 + [C.POINTER(MatMulParams)],
     "fa_kv_prefix_copy": [_vp, _PT, _PT, _sz],
     "fa_kv_prefix_copy_batch": [_vp, _PT, _PT, _u32, _sz],
     "fa_align_capacity": [_sz],
@@ -366,6 +374,14 @@ class Foundry:
         bq, bk, bv = biases if biases is not None else (none, none, none)
         check(self.lib.fa_fused_qkv(self.h, C.byref(x), C.byref(w_q), C.byref(w_k), C.byref(w_v), C.byref(g), C.byref(bq),
                                     C.byref(bk), C.byref(bv), C.byref(out_q), C.byref(out_k), C.byref(out_v), C.byref(p)))
+
+    def matmul(self, a, b, output, m, n, k, bias=None, c=None, transpose_b=True, alpha=1.0, beta=0.0, transpose_a=False,
+               weights_per_block=32, activation=0):
+        """output[m, n] = alpha * a[m, k] . b^T + bias + beta * c; b row-major [n, k] (transpose_b) or canonical."""
+        p = MatMulParams(m, n, k, int(transpose_a), int(transpose_b), alpha, beta, weights_per_block, activation)
+        none = TensorArg()
+        check(self.lib.fa_matmul(self.h, C.byref(a), C.byref(b), C.byref(output), C.byref(bias if bias is not None else none),
+                                 C.byref(c if c is not None else none), C.byref(p)))
 
     def paged_copy_blocks(self, cache, src_ids, dst_ids, n_pairs):
         """src_ids / dst_ids: device i32 buffers."""

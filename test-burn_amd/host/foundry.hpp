@@ -461,4 +461,55 @@ inline void CompiledFusedQkvStep::execute(Foundry &foundry, const FastBindings &
                        out_v.c(), &p));
 }
 
+// ---------------------------------------------------------------------------------------------- MatMul
+struct MatMulStep;
+struct CompiledMatMulStep : CompiledStep {
+    const MatMulStep *step;
+    size_t a_idx, b_idx, output_idx;
+    std::optional<size_t> bias_idx, c_idx;
+    void execute(Foundry &foundry, const FastBindings &fast, const TensorBindings &bindings, const SymbolTable &) const override;
+    const char *name() const override { return "MatMul (Unified)"; }
+};
+
+// src/metals/matmul.rs:11-31 with its defaults (:33-70): alpha 1, beta 0, weights_per_block 32. `bias` / `c` named
+// "zero" are placeholders for "absent" (:195-196). `b_scales` belongs to the block-quantised policies.
+struct MatMulStep {
+    Ref a = "a", b = "b", output = "output";
+    std::optional<Ref> bias, c;
+    DynamicU32 m = 1, n = 1, k = 1;
+    bool transpose_a = false, transpose_b = false;
+    float alpha = 1.0f, beta = 0.0f;
+    uint32_t weights_per_block = 32;
+    std::vector<std::unique_ptr<CompiledStep>> compile(TensorBindings &bd, SymbolTable &s) const {
+        auto cs = std::make_unique<CompiledMatMulStep>();
+        cs->step = this;
+        cs->a_idx = s.get_or_create(bd.interpolate(a)), cs->b_idx = s.get_or_create(bd.interpolate(b));
+        cs->output_idx = s.get_or_create(bd.interpolate(output));
+        auto opt = [&](const std::optional<Ref> &r) -> std::optional<size_t> {
+            if (!r || *r == "zero") return std::nullopt;
+            return s.get_or_create(bd.interpolate(*r));
+        };
+        cs->bias_idx = opt(bias), cs->c_idx = opt(c);
+        std::vector<std::unique_ptr<CompiledStep>> out;
+        out.push_back(std::move(cs));
+        return out;
+    }
+    void execute(Foundry &foundry, TensorBindings &bindings) const { execute_step(*this, foundry, bindings); }
+    const char *name() const { return "MatMul"; }
+};
+
+inline void CompiledMatMulStep::execute(Foundry &foundry, const FastBindings &fast, const TensorBindings &bindings,
+                                        const SymbolTable &) const {
+    const MatMulStep &s = *step;
+    const TensorArg a = TensorArg::from_tensor(need(fast, a_idx, "a")), b = TensorArg::from_tensor(need(fast, b_idx, "b"));
+    const TensorArg output = TensorArg::from_tensor(need(fast, output_idx, "output"));
+    const TensorArg bias = bias_idx ? TensorArg::from_tensor(need(fast, *bias_idx, "bias")) : TensorArg();
+    const TensorArg c = c_idx ? TensorArg::from_tensor(need(fast, *c_idx, "c")) : TensorArg();
+    fa_matmul_params p;
+    p.m = s.m.resolve(bindings), p.n = s.n.resolve(bindings), p.k = s.k.resolve(bindings);
+    p.transpose_a = s.transpose_a ? 1 : 0, p.transpose_b = s.transpose_b ? 1 : 0, p.alpha = s.alpha, p.beta = s.beta;
+    p.weights_per_block = s.weights_per_block, p.activation = 0;
+    check(fa_matmul(foundry.ctx(), a.c(), b.c(), output.c(), bias.c(), c.c(), &p));
+}
+
 }  // namespace metallic_foundry

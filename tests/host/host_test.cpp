@@ -462,6 +462,34 @@ static void test_fused_qkv_step(Foundry &foundry, WeightLayout layout) {
     foundry.synchronize();
 }
 
+// The o_proj step of models/llama.json:566-585: MatMul with transpose_b, c = hidden, alpha = beta = 1, bias "zero".
+static void test_matmul_step_o_proj(Foundry &foundry) {
+    const size_t K = 512, N = 384;
+    Rng rng{5};
+    auto attn = rng.fill(K, 1.0f), hidden = rng.fill(N, 1.0f), w = rng.fill(N * K, 0.1f);
+    std::vector<orc_f16> want(N);
+    orc_matmul_gemv(attn.data(), w.data(), nullptr, hidden.data(), want.data(), 1, (uint32_t)N, (uint32_t)K, 0, 32, 1.0f, 1.0f, 4);
+    TensorBindings b;
+    b.set_int_global("i", 0);
+    b.set_int_global("m", 1);
+    b.set_int_global("d_model", N);
+    b.insert("attn_out", foundry.from_host(Dtype::F16, {1, K}, attn.data()));
+    b.insert("hidden", foundry.from_host(Dtype::F16, {1, N}, hidden.data()));
+    b.insert("layer.attn_output_0", foundry.from_host(Dtype::F16, {N, K}, w.data()));
+    b.insert("residual_1", foundry.zeros(Dtype::F16, {1, N}));
+    MatMulStep step;
+    step.a = "attn_out", step.b = "layer.attn_output_{i}", step.output = "residual_1", step.bias = "zero", step.c = "hidden";
+    step.m = DynamicU32::var("m"), step.n = DynamicU32::var("d_model"), step.k = (uint32_t)K;
+    step.transpose_b = true, step.alpha = 1.0f, step.beta = 1.0f;
+    step.execute(foundry, b);
+    foundry.synchronize();
+    auto got = foundry.to_host<orc_f16>(*b.get("residual_1"));
+    EXPECT(max_abs_diff(want, got, N) <= 4e-3f);
+    step.transpose_a = true;
+    EXPECT(thrown_by([&] { step.execute(foundry, b); }) == MetalError::OperationNotSupported);
+    foundry.synchronize();
+}
+
 int main(int argc, char **argv) {
     const bool cpu_only = argc > 1 && std::string(argv[1]) == "--cpu";
     run_test("bindings and dynamic values", test_bindings_and_dynamic_values);
@@ -486,6 +514,7 @@ int main(int argc, char **argv) {
         run_test("error variants", [&] { test_error_variants(foundry); });
         run_test("fused qkv step, row-major weights", [&] { test_fused_qkv_step(foundry, WeightLayout::RowMajor); });
         run_test("fused qkv step, canonical weights", [&] { test_fused_qkv_step(foundry, WeightLayout::Canonical); });
+        run_test("matmul step as o_proj with residual", [&] { test_matmul_step_o_proj(foundry); });
         run_test("session: chunked prefill, snapshot, decode loop with growth, restore",
                  [&] { test_session_prefill_chunks_decode_loop_growth_snapshot(foundry); });
     }

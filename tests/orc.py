@@ -250,6 +250,22 @@ def fused_qkv(x, w_q, w_k, w_v, gamma=None, biases=None, layout=0, wpb=32, eps=1
     return oq, ok, ov
 
 
+def matmul_gemv(x, w, bias=None, residual=None, layout=0, wpb=32, alpha=1.0, beta=0.0, n_threads=8):
+    """x [m, K]; w flat or 2-D in `layout`; returns out [m, n]."""
+    x = _h(x)
+    m, K = x.shape
+    wf = _h(np.asarray(w).reshape(-1))
+    n = wf.size // K
+    out = np.zeros((m, n), np.float16)
+    nul = C.cast(None, u16p)
+    b = _h(bias) if bias is not None else None
+    r = _h(residual) if residual is not None else None
+    lib().orc_matmul_gemv(_p(x, u16p), _p(wf, u16p), _p(b, u16p) if b is not None else nul, _p(r, u16p) if r is not None else nul,
+                          _p(out, u16p), C.c_uint32(m), C.c_uint32(n), C.c_uint32(K), C.c_int(layout), C.c_uint32(wpb),
+                          C.c_float(alpha), C.c_float(beta), C.c_int(n_threads))
+    return out
+
+
 def paged_copy_blocks(pool, n_kv_heads, block_size, head_dim, src_ids, dst_ids):
     """In place on `pool` [n_blocks, n_kv_heads, block_size, head_dim] f16."""
     assert pool.dtype == np.float16 and pool.flags.c_contiguous

@@ -125,3 +125,61 @@ def test_fused_qkv_errors():
     f.synchronize()
     for z in (x, wq, wk, wv, oq, ok, ov, w8, b):
         z.free()
+
+
+# ---------------------------------------------------------------- MatMul (the o_proj consumer of attn_out)
+
+@pytest.mark.parametrize("m,n,k,canonical,bias,resid,alpha,beta", [
+    (1, 128, 128, False, False, False, 1.0, 0.0),    # tests/gemv_v2_parity.rs:244-254
+    (1, 256, 256, False, False, False, 0.5, 0.0),    # :280-289 (alpha)
+    (1, 128, 512, False, True, False, 1.0, 0.0),     # :303-330 (k > n, bias)
+    (1, 4096, 4096, False, False, False, 1.0, 0.0),  # :406-416
+    (1, 3072, 3072, True, False, True, 1.0, 1.0),    # Llama-3.2-3B o_proj: canonical weights, residual, beta 1
+    (1, 896, 896, True, True, True, 1.0, 1.0),
+    (5, 3072, 3072, True, False, True, 1.0, 1.0),
+    (32, 896, 896, False, False, True, 0.25, 0.75),  # a prefill chunk through the same path
+    (3, 40, 64, True, True, True, 1.0, 0.5),
+])
+def test_matmul_gemv_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta):
+    announce("matmul", m, n, k, canonical, bias, resid, alpha, beta)
+    f = ctx()
+    rng = np.random.default_rng(m + n + k)
+    x = rng.uniform(-1, 1, (m, k)).astype(np.float16)
+    w = rng.uniform(-0.1, 0.1, (n, k)).astype(np.float16)
+    b = rng.uniform(-0.1, 0.1, n).astype(np.float16)
+    c = rng.uniform(-1, 1, (m, n)).astype(np.float16)
+    want = orc.matmul_gemv(x, w, b if bias else None, c if resid else None, 0, 32, alpha, beta)
+    dx, dw = f.array(x), f.array(orc.to_canonical(w) if canonical else w.reshape(-1))
+    db, dc, out = f.array(b), f.array(c), f.zeros((m, n))
+    f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, bias=db.arg() if bias else None, c=dc.arg() if resid else None,
+             transpose_b=not canonical, alpha=alpha, beta=beta)
+    got = out.download()
+    # the reference's own bar is 1e-3 * sqrt(k) (tests/gemv_v2_parity.rs:214); here: 2 f16 ulps of the expected value
+    g, wv = got.astype(np.float64), want.astype(np.float64)
+    assert np.all(np.abs(g - wv) <= 2 * np.maximum(np.abs(wv), 2.0 ** -10) * 2.0 ** -10 + 1e-4), float(np.max(np.abs(g - wv)))
+    assert float(np.max(np.abs(g - wv))) <= 1e-3 * np.sqrt(k)
+    for z in (dx, dw, db, dc, out):
+        z.free()
+
+
+def test_matmul_errors():
+    announce("matmul errors")
+    f = ctx()
+    a, b, o = f.zeros((1, 64)), f.zeros((32 * 64,)), f.zeros((1, 32))
+    f.matmul(a.arg(), b.arg(), o.arg(), 1, 32, 64)
+    with pytest.raises(fa.FoundryError) as e:
+        f.matmul(a.arg(), b.arg(), o.arg(), 1, 32, 64, transpose_a=True)
+    assert e.value.variant == "OperationNotSupported"
+    with pytest.raises(fa.FoundryError) as e:
+        f.matmul(a.arg(), b.arg(), o.arg(), 1, 32, 64, activation=1)
+    assert e.value.variant == "OperationNotSupported"
+    with pytest.raises(fa.FoundryError) as e:
+        f.matmul(a.arg(), b.arg(), o.arg(), 1, 33, 64)
+    assert e.value.variant == "InvalidShape"
+    b8 = f.zeros((32 * 64,), np.int8)
+    with pytest.raises(fa.FoundryError) as e:
+        f.matmul(a.arg(), b8.arg(), o.arg(), 1, 32, 64)
+    assert e.value.variant == "UnsupportedDtype"
+    f.synchronize()
+    for z in (a, b, o, b8):
+        z.free()

@@ -642,3 +642,20 @@ def test_fused_qkv_vs_float64(K, N, NK, m, norm, bias):
     eye = np.eye(K, dtype=np.float16)
     q, _, _ = orc.fused_qkv(x, eye, eye[:8], eye[:8], gamma=g if norm else None)
     assert np.array_equal(q.astype(np.float64), xn)
+
+
+@pytest.mark.parametrize("m,n,k,alpha,beta", [(1, 128, 128, 1.0, 0.0), (1, 256, 256, 0.5, 0.0), (2, 40, 96, 1.0, 1.0), (3, 16, 64, 0.25, 0.75)])
+def test_matmul_gemv_vs_float64_and_linearity(m, n, k, alpha, beta):
+    """alpha * x.W^T + bias + beta * residual against float64 (shapes and alpha of tests/gemv_v2_parity.rs:244-301);
+    both layouts give the same bits; the residual term is linear in beta (beta = 0 drops it exactly)."""
+    rng = np.random.default_rng(n + k)
+    x = rng.uniform(-1, 1, (m, k)).astype(np.float16)
+    w = rng.uniform(-0.1, 0.1, (n, k)).astype(np.float16)
+    b = rng.uniform(-0.1, 0.1, n).astype(np.float16)
+    c = rng.uniform(-1, 1, (m, n)).astype(np.float16)
+    got = orc.matmul_gemv(x, w, b, c, 0, 32, alpha, beta)
+    assert np.array_equal(got, orc.matmul_gemv(x, orc.to_canonical(w), b, c, 1, 32, alpha, beta))
+    ref = alpha * (x.astype(np.float64) @ w.astype(np.float64).T) + b.astype(np.float64) + beta * c.astype(np.float64)
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= 1.5 * np.maximum(np.abs(ref), 2.0 ** -10) * 2.0 ** -10 + 1e-4)
+    assert np.array_equal(orc.matmul_gemv(x, w, b, c, 0, 32, alpha, 0.0), orc.matmul_gemv(x, w, b, None, 0, 32, alpha, 0.0))
+    assert np.array_equal(orc.matmul_gemv(x, np.zeros_like(w), None, c, 0, 32, 1.0, 1.0), c)  # zero weights: out = residual
