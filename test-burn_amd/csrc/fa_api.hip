@@ -102,6 +102,8 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     }
     ctx->decode_variant.keys_per_split = env_u32("FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT", 0);
     ctx->decode_variant.merge = env_u32("FOUNDRY_ATTN_DECODE_MERGE", 1);
+    ctx->decode_waves = env_u32("FOUNDRY_ATTN_DECODE_WAVES", 0);
+    if (ctx->decode_waves != 4 && ctx->decode_waves != 8) ctx->decode_waves = 0;
     ctx->prefill_split_k = env_u32("FOUNDRY_ATTN_PREFILL_SPLIT_K", 0);
     ctx->prefill_variant = env_u32("FOUNDRY_ATTN_PREFILL_VARIANT", 0);
     if (ctx->prefill_variant > 2) ctx->prefill_variant = 0;

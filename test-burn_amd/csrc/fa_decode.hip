@@ -25,20 +25,31 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     // is the number of requests a CU can keep outstanding, so a CU that gets two partitions takes nearly twice as
     // long and every other one waits for it in the merge. Within that limit the partitions are as small as the
     // granularity allows, but not below one block per wave.
+    // Workgroup size: 8 waves (one workgroup per CU) while the launch has at most one workgroup per CU; otherwise
+    // 4 waves (two resident per CU), so that one workgroup's ~5 us of start and end overlap the other's stream and
+    // the rounds of workgroups balance at a finer grain.
     uint32_t chunk = ctx->decode_variant.keys_per_split;
-    if (chunk == 0) {
-        const uint64_t groups = (uint64_t)L.batch * ny;
-        const uint64_t slots = (uint64_t)(ctx->n_cus > 0 ? ctx->n_cus : 256);
+    const uint64_t groups = (uint64_t)L.batch * ny;
+    const uint64_t n_cus = (uint64_t)(ctx->n_cus > 0 ? ctx->n_cus : 256);
+    auto auto_chunk = [&](uint32_t nw, uint64_t slots) {
         const uint32_t s_max = groups >= slots ? 1u : (uint32_t)(slots / groups);
-        // Long partitions are cut further, into a whole number of workgroups per CU, so that a batch of ragged
+        // Long partitions are cut further, into a whole number of workgroups per slot, so that a batch of ragged
         // sequences (whose short members leave most of their partitions empty) still balances over the CUs - but
         // not too far: a workgroup costs about 5 us before and after its keys stream in at 31 KB per microsecond,
-        // which 768 keys (393 KB) do not amortise (C3: 62.9 us with <= 768 keys, 52.0 us with <= 1536).
-        const uint32_t long_chunk = 4u * NW * MBX * BK;  // 1536 keys: four rounds of a workgroup
-        const uint32_t per_cu = ceil_div_u32(ceil_div_u32(bound, s_max), long_chunk);
-        chunk = ceil_div_u32(ceil_div_u32(bound, s_max * per_cu), (uint32_t)BK) * BK;
-        if (chunk < (uint32_t)(NW * BK)) chunk = NW * BK;
+        // which 768 keys (393 KB) do not amortise when workgroups run one after the other on a CU
+        // (C3, 8 waves: 62.9 us with <= 768 keys, 52.0 us with <= 1536).
+        const uint32_t long_chunk = 4u * nw * MBX * BK;  // four rounds of a workgroup: 1536 keys at 8 waves
+        const uint32_t per_slot = ceil_div_u32(ceil_div_u32(bound, s_max), long_chunk);
+        uint32_t c = ceil_div_u32(ceil_div_u32(bound, s_max * per_slot), (uint32_t)BK) * BK;
+        if (c < nw * BK) c = nw * BK;
+        return c;
+    };
+    uint32_t waves = ctx->decode_waves;  // 0 = by the rule above
+    if (waves == 0) {
+        const uint32_t c8 = chunk ? chunk : auto_chunk(8, n_cus);
+        waves = groups * ceil_div_u32(bound, (c8 + BK - 1) / BK * BK) > n_cus ? 4u : 8u;
     }
+    if (chunk == 0) chunk = waves == 4 ? auto_chunk(4, 2 * n_cus) : auto_chunk(8, n_cus);
     chunk = (chunk + BK - 1) / BK * BK;
     const uint32_t S = ceil_div_u32(bound, chunk);
     // a contiguous cache slab is addressed with 32-bit byte offsets (tile base included)
@@ -82,7 +93,7 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     else if (L.paged)
         mode = MODE_PAGED;
     dim3 grid(S, ny, L.batch);
-    if (L.head_dim == 128) return fa_decode_launch_d128(ctx, a, grid, mode);
-    if (L.head_dim == 64) return fa_decode_launch_d64(ctx, a, grid, mode);
+    if (L.head_dim == 128) return waves == 4 ? fa_decode_launch_d128_w4(ctx, a, grid, mode) : fa_decode_launch_d128(ctx, a, grid, mode);
+    if (L.head_dim == 64) return waves == 4 ? fa_decode_launch_d64_w4(ctx, a, grid, mode) : fa_decode_launch_d64(ctx, a, grid, mode);
     return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Flash Decode only supports head_dim=64 or 128, got %u", L.head_dim);
 }

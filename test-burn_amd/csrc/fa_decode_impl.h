@@ -36,11 +36,23 @@
 // the one new token: every workgroup rotates the group's query rows in registers (rounded to f16 exactly
 // as q_rot would be); the partition that ends at the new row attends its cache rows first and then the new
 // token as a one-key tile built from the rotated K / copied V, which one workgroup also stores into the cache.
+//
+// The file is compiled once per workgroup size: FA_DECODE_NW (waves per workgroup, default 8) and FA_DECODE_NS (the
+// namespace of that build, default fa_decode) are set by the including translation unit. 8 waves = one workgroup
+// per CU, for launches of at most one workgroup per CU; 4 waves = two resident workgroups per CU, for launches
+// with several rounds of workgroups, where one workgroup's start and end overlap the other's stream.
 #pragma once
 #include "fa_internal.h"
 #include <type_traits>
 
-namespace fa_decode {
+#ifndef FA_DECODE_NW
+#define FA_DECODE_NW 8
+#endif
+#ifndef FA_DECODE_NS
+#define FA_DECODE_NS fa_decode
+#endif
+
+namespace FA_DECODE_NS {
 
 typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
@@ -63,35 +75,13 @@ union U4H {
     _Float16 e[8];
 };
 
-constexpr int NW = 8;        // waves per workgroup, two per SIMD: one workgroup per CU at <= 256 VGPRs
+constexpr int NW = FA_DECODE_NW;  // waves per workgroup; two per SIMD in all: 8 = one workgroup per CU, 4 = two, at <= 256 VGPRs
 constexpr int NT = NW * 64;  // threads per workgroup
 constexpr int BK = 16;       // keys per block (MFMA M dimension)
 constexpr int MBX = 3;       // blocks a wave keeps in flight (one round)
 constexpr int MAX_GT = 16;   // query heads served by one workgroup (the MFMA N dimension)
 
-struct DecodeDev {
-    const __half *q, *k, *v;
-    __half *out;
-    uint64_t q_stride_b, q_stride_h, k_stride_b, k_stride_h, v_stride_b, v_stride_h, out_stride_b, out_stride_h;
-    const uint32_t *d_len;
-    const int32_t *block_table;
-    float *part_acc;     // [batch][y][S][gt][D]
-    float *part_ml;      // [batch][y][S][gt][2]
-    uint32_t *counters;  // [batch][y]
-    uint32_t kv_len, d_len_stride, kv_len_add, kv_len_bound, capacity, chunk, n_kv_heads, sub_per_kv, gt;
-    uint32_t bt_stride, block_size, block_shift /* log2(block_size), 32 if not a power of two */, merge_in_kernel;
-    float scale_log2e;
-    // Sage-style int8 Q/K: q and k point at int8 data, scores are rescaled by q_scale[h] * k_scale[kvh][key/32]
-    const float *q_scale;
-    const __half *k_scale;
-    uint32_t ks_stride;
-    // FUSED: raw projections of the new token (row b of token-major [batch, H*D] / [batch, Hkv*D]) and RoPE tables
-    const __half *k_in, *v_in, *cos_t, *sin_t;
-    __half *q_rot_out;  // nullable
-    uint64_t qin_stride_b, kvin_stride_b, qrot_stride_b;
-    uint32_t rope_normal, apply_rope, table_rows;
-    uint32_t bf16;  // data tensors are bf16 (RoPE tables stay f16)
-};
+using DecodeDev = ::FaDecodeDev;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -280,7 +270,7 @@ __device__ __forceinline__ U4H rope8(const U4H &x, const U4H &mate, const U4H &c
 }
 
 template <int D, bool PAGED, bool SAGE, bool FUSED, bool BF16 = false>
-__global__ void __launch_bounds__(NT, 1) flash_decode_mfma_kernel(DecodeDev a) {
+__global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(DecodeDev a) {
     constexpr int KSTEPS = SAGE ? D / 64 : D / 32;  // MFMA steps over head_dim for S^T; 16 B per lane each
     constexpr int SEGS = SAGE ? D / 16 : D / 8;     // 16-byte segments per K row
     constexpr int VLB = D / 32;                     // 1 KiB V loads per block
@@ -891,8 +881,11 @@ fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
     return FA_OK;
 }
 
-}  // namespace fa_decode
+}  // namespace FA_DECODE_NS
 
-// Defined in fa_decode_d64.hip / fa_decode_d128.hip.
-fa_status fa_decode_launch_d64(fa_ctx *ctx, const fa_decode::DecodeDev &a, dim3 grid, int mode);
-fa_status fa_decode_launch_d128(fa_ctx *ctx, const fa_decode::DecodeDev &a, dim3 grid, int mode);
+// Defined in fa_decode_d64.hip / fa_decode_d128.hip (8 waves per workgroup) and fa_decode_d64_w4.hip /
+// fa_decode_d128_w4.hip (4 waves).
+fa_status fa_decode_launch_d64(fa_ctx *ctx, const FaDecodeDev &a, dim3 grid, int mode);
+fa_status fa_decode_launch_d128(fa_ctx *ctx, const FaDecodeDev &a, dim3 grid, int mode);
+fa_status fa_decode_launch_d64_w4(fa_ctx *ctx, const FaDecodeDev &a, dim3 grid, int mode);
+fa_status fa_decode_launch_d128_w4(fa_ctx *ctx, const FaDecodeDev &a, dim3 grid, int mode);

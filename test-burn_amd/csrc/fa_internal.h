@@ -35,6 +35,7 @@ struct fa_ctx {
     uint32_t *counters = nullptr;
     uint32_t n_counters = 0;
     fa_decode_variant decode_variant{0, 1};
+    uint32_t decode_waves = 0;     // waves per decode workgroup: 0 = by launch size, 4 or 8
     uint32_t prefill_split_k = 0;  // 0 = auto
     uint32_t prefill_variant = 0;  // 0 = auto, 1 = tiles staged through registers, 2 = tiles straight into LDS, two-phase loop
     // per-kernel profiling
@@ -136,6 +137,32 @@ struct DecodeLaunch {
     bool bf16;  // q, k, v, caches and out are bf16 instead of f16 (not with the int8 variant)
 };
 fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &a);
+
+// Kernel argument block of the flash-decode kernels (all workgroup sizes).
+struct FaDecodeDev {
+    const __half *q, *k, *v;
+    __half *out;
+    uint64_t q_stride_b, q_stride_h, k_stride_b, k_stride_h, v_stride_b, v_stride_h, out_stride_b, out_stride_h;
+    const uint32_t *d_len;
+    const int32_t *block_table;
+    float *part_acc;     // [batch][y][S][gt][D]
+    float *part_ml;      // [batch][y][S][gt][2]
+    uint32_t *counters;  // [batch][y]
+    uint32_t kv_len, d_len_stride, kv_len_add, kv_len_bound, capacity, chunk, n_kv_heads, sub_per_kv, gt;
+    uint32_t bt_stride, block_size, block_shift /* log2(block_size), 32 if not a power of two */, merge_in_kernel;
+    float scale_log2e;
+    // Sage-style int8 Q/K: q and k point at int8 data, scores are rescaled by q_scale[h] * k_scale[kvh][key/32]
+    const float *q_scale;
+    const __half *k_scale;
+    uint32_t ks_stride;
+    // FUSED: raw projections of the new token (row b of token-major [batch, H*D] / [batch, Hkv*D]) and RoPE tables
+    const __half *k_in, *v_in, *cos_t, *sin_t;
+    __half *q_rot_out;  // nullable
+    uint64_t qin_stride_b, kvin_stride_b, qrot_stride_b;
+    uint32_t rope_normal, apply_rope, table_rows;
+    uint32_t bf16;  // data tensors are bf16 (RoPE tables stay f16)
+};
+
 
 struct PrefillLaunch {
     const __half *q, *k, *v;
