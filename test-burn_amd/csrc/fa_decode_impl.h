@@ -665,6 +665,9 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                 *reinterpret_cast<uint4 *>(v_lds + (mb * BK + row) * VRS + (lane % VLPR) * 16) = x.u;
             }
         }
+        // The V registers are free as soon as the blocks are in LDS: the next round's V is requested before this
+        // round's second contraction, not after it (the wait for V was the exposed latency of every round).
+        if (mnext) issue_v(nblk, mnext, k1 - 1);
         // O^T += V^T . P^T : a transpose load hands lane (n, c) keys 4c..4c+3 of dim 16*blk + n
 #pragma unroll
         for (int mb = 0; mb < MBX; ++mb) {
@@ -681,7 +684,6 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                                  : __builtin_amdgcn_mfma_f32_16x16x16f16(vh, pb[mb], oacc[blk], 0, 0, 0);
             }
         }
-        if (mnext) issue_v(nblk, mnext, k1 - 1);  // V registers are free again
         if (PAGED && mnext && nblk + mnext < wbe) load_pages(nblk + mnext, min((uint32_t)MBX, wbe - (nblk + mnext)), pgn);
     };
 
