@@ -374,9 +374,9 @@ def bench_kv_growth(f, args):
     f.profile_enable(False)
 
 
-def bench_fused_qkv(f, args):
-    """The step before the path at Llama-3.2-3B decode shape: RMSNorm + Q/K/V projections of one token, F16 weights in
-    the reference's canonical blocked layout, one layer per step over 8 distinct layers' weights."""
+def bench_fused_qkv(f, args, q8=False):
+    """The step before the path at Llama-3.2-3B decode shape: RMSNorm + Q/K/V projections of one token, F16 (or Q8_0)
+    weights in the reference's canonical blocked layout, one layer per step over 8 distinct layers' weights."""
     import orc
     K, N, NK, NL = 3072, 3072, 1024, 8
     rng = np.random.default_rng(0xF0DD + 7)
@@ -385,19 +385,27 @@ def bench_fused_qkv(f, args):
     layers, host0 = [], None
     for i in range(NL):  # distinct weights so that no launch finds the previous one's in cache
         ws = [rng.uniform(-0.1, 0.1, (n, K)).astype(np.float16) for n in (N, NK, NK)]
-        layers.append([f.array(orc.to_canonical(w)) for w in ws])
+        if q8:
+            ws = [orc.quantize_q8_0(w) for w in ws]
+            layers.append(([f.array(orc.to_canonical(w)) for w, _ in ws], [f.array(sc) for _, sc in ws]))
+        else:
+            layers.append(([f.array(orc.to_canonical(w)) for w in ws], None))
         if i == 0:
             host0 = ws
     dx, dg = f.array(x), f.array(g)
     oq, ok, ov = f.zeros((1, N)), f.zeros((1, NK)), f.zeros((1, NK))
 
     def step(i):
-        w = layers[i % NL]
-        f.fused_qkv(dx.arg(), w[0].arg(), w[1].arg(), w[2].arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1, gamma=dg.arg())
+        w, sc = layers[i % NL]
+        f.fused_qkv(dx.arg(), w[0].arg(), w[1].arg(), w[2].arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1, gamma=dg.arg(),
+                    scales=[t.arg() for t in sc] if sc else None)
 
     step(0)
     f.synchronize()
-    want = orc.fused_qkv(x, *host0, gamma=g)
+    if q8:
+        want = orc.fused_qkv_q8(x, [w for w, _ in host0], [sc for _, sc in host0], gamma=g)
+    else:
+        want = orc.fused_qkv(x, *host0, gamma=g)
     err = max(float(np.max(np.abs(o.download().astype(np.float64) - w.astype(np.float64)))) for o, w in zip((oq, ok, ov), want))
     for i in range(args.warmup):
         step(i)
@@ -409,15 +417,16 @@ def bench_fused_qkv(f, args):
         step(i)
     f.synchronize()
     dt = time.perf_counter() - t0
-    nbytes = 2.0 * (N + 2 * NK) * K + 2 * K * 2 + 2 * (N + 2 * NK)  # weights, input + gamma, outputs
+    wbytes = (1.0 + 2.0 / 32) if q8 else 2.0  # per weight: int8 + an f16 scale per 32, or f16
+    nbytes = wbytes * (N + 2 * NK) * K + 2 * K * 2 + 2 * (N + 2 * NK)  # weights, input + gamma, outputs
     _finish_secondary(f, args, "FusedQkv layer-steps/s + achieved HBM GB/s, Llama-3.2-3B decode shape",
                       "llama3.2-3b FusedQkv at decode: RMSNorm + Q/K/V projections of one token, k_dim 3072, n_dim 3072, "
-                      "n_kv 1024, F16 canonical weights, eager launches (profiling events on)", "fused_qkv_kernel", nbytes, dt,
-                      {"qkv_max_abs_err": err})
+                      "n_kv 1024, %s canonical weights, eager launches (profiling events on)" % ("Q8_0" if q8 else "F16"),
+                      "fused_qkv_kernel", nbytes, dt, {"qkv_max_abs_err": err})
     f.profile_enable(False)
 
 
-def bench_o_proj(f, args):
+def bench_o_proj(f, args, q8=False):
     """The step after the path at Llama-3.2-3B decode shape: attn_out [1, 3072] x W_o^T + hidden (MatMul with residual,
     alpha = beta = 1), F16 weights in the canonical blocked layout, one layer per step over 12 layers' weights."""
     import orc
@@ -428,17 +437,24 @@ def bench_o_proj(f, args):
     layers, host0 = [], None
     for i in range(NL):  # distinct weights so that no launch finds the previous one's in cache
         w = rng.uniform(-0.1, 0.1, (N, K)).astype(np.float16)
-        layers.append(f.array(orc.to_canonical(w)))
+        if q8:
+            w8, sc = orc.quantize_q8_0(w)
+            layers.append((f.array(orc.to_canonical(w8)), f.array(sc)))
+            w = (w8, sc)
+        else:
+            layers.append((f.array(orc.to_canonical(w)), None))
         if i == 0:
             host0 = w
     dx, dc, out = f.array(x), f.array(c), f.zeros((1, N))
 
     def step(i):
-        f.matmul(dx.arg(), layers[i % NL].arg(), out.arg(), 1, N, K, c=dc.arg(), transpose_b=False, alpha=1.0, beta=1.0)
+        w, sc = layers[i % NL]
+        f.matmul(dx.arg(), w.arg(), out.arg(), 1, N, K, c=dc.arg(), transpose_b=False, alpha=1.0, beta=1.0,
+                 b_scales=sc.arg() if sc else None)
 
     step(0)
     f.synchronize()
-    want = orc.matmul_gemv(x, host0, None, c, 0, 32, 1.0, 1.0)
+    want = orc.matmul_gemv_q8(x, host0[0], host0[1], None, c, 0, 32, 1.0, 1.0) if q8 else orc.matmul_gemv(x, host0, None, c, 0, 32, 1.0, 1.0)
     err = float(np.max(np.abs(out.download().astype(np.float64) - want.astype(np.float64))))
     for i in range(args.warmup):
         step(i)
@@ -450,10 +466,11 @@ def bench_o_proj(f, args):
         step(i)
     f.synchronize()
     dt = time.perf_counter() - t0
-    nbytes = 2.0 * N * K + 2 * K + 2 * 2 * N  # weights, input, residual + output
+    nbytes = ((1.0 + 2.0 / 32) if q8 else 2.0) * N * K + 2 * K + 2 * 2 * N  # weights, input, residual + output
     _finish_secondary(f, args, "o_proj MatMul layer-steps/s + achieved HBM GB/s, Llama-3.2-3B decode shape",
-                      "llama3.2-3b o_proj at decode: attn_out [1, 3072] x W_o^T + hidden, n 3072, k 3072, F16 canonical "
-                      "weights, eager launches (profiling events on)", "matmul_gemv_kernel", nbytes, dt, {"max_abs_err": err})
+                      "llama3.2-3b o_proj at decode: attn_out [1, 3072] x W_o^T + hidden, n 3072, k 3072, %s canonical "
+                      "weights, eager launches (profiling events on)" % ("Q8_0" if q8 else "F16"), "matmul_gemv_kernel", nbytes,
+                      dt, {"max_abs_err": err})
     f.profile_enable(False)
 
 
@@ -590,7 +607,9 @@ def bench_sage_decode(f, args):
 SECONDARY = {"llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
-             "llama3b_o_proj": bench_o_proj}
+             "llama3b_o_proj": bench_o_proj,
+             "llama3b_fused_qkv_q8": lambda f, args: bench_fused_qkv(f, args, q8=True),
+             "llama3b_o_proj_q8": lambda f, args: bench_o_proj(f, args, q8=True)}
 
 
 def main():

@@ -60,7 +60,7 @@ const char *fa_last_error_string(void);
 
 /* Dtype, same order as metallic-sdk's enum (crates/metallic-sdk/src/tensor.rs:7-30). */
 typedef enum fa_dtype {
-    FA_DTYPE_F32 = 0, FA_DTYPE_F16 = 1, FA_DTYPE_BF16 = 2,
+    FA_DTYPE_F32 = 0, FA_DTYPE_F16 = 1, FA_DTYPE_BF16 = 2, FA_DTYPE_Q8_0 = 7,
     FA_DTYPE_I8 = 15, FA_DTYPE_I16 = 16, FA_DTYPE_I32 = 17, FA_DTYPE_U8 = 18, FA_DTYPE_U16 = 19,
     FA_DTYPE_U32 = 20, FA_DTYPE_F64 = 21
 } fa_dtype;
@@ -354,9 +354,11 @@ fa_status fa_paged_copy_blocks(fa_ctx *ctx, const fa_paged_kv *cache, const int3
 /* ---------------------------------------------------------------------------------------------
  * FusedQkv: the step before the path. RMSNorm(input) -> Q, K and V projections in one launch -> the three
  * token-major tensors KvPrepFused consumes (src/metals/gemv/qkv_step.rs:14-120,220-460, op `FusedQkv` of
- * models/llama.json:509-528; kernel src/metals/gemv/qkv_project.metal). F16 weights only (PolicyF16,
- * src/metals/policies/policy_f16.metal:18-70): the reference's block-quantised policies are not built here and
- * are refused with FA_ERR_UNSUPPORTED_DTYPE.
+ * models/llama.json:509-528; kernel src/metals/gemv/qkv_project.metal). Weights are F16 (PolicyF16,
+ * src/metals/policies/policy_f16.metal:18-70) or Q8_0 (PolicyQ8, src/metals/policies/policy_q8.metal: int8 values in
+ * the same element order, dtype FA_DTYPE_Q8_0 or FA_DTYPE_I8, plus a scale tensor s_* of f16 [rows, k_dim / 32],
+ * row-major, weight = int8 * scale of its 32-block); the other block-quantised policies are refused with
+ * FA_ERR_UNSUPPORTED_DTYPE.
  *   out_q[b, r] = f16( sum_k xn[b, k] * W_q[r, k] + bias_q[r] ),  r < n_dim;  out_k, out_v likewise, r < n_kv
  *   xn[b, k]    = f16( x[b, k] * rsqrt(mean_k x[b, k]^2 + epsilon) * gamma[k] )  with gamma, else x[b, k]
  * (the normalised input is rounded to f16 before the products, qkv_project.metal:48-67; f32 accumulation; the
@@ -379,19 +381,21 @@ typedef struct fa_fused_qkv_params {
     float epsilon;              /* RMSNorm epsilon (the reference's `rms_eps` variable, default 1e-6) */
 } fa_fused_qkv_params;
 
-/* input [m, k_dim] (any rank with k_dim innermost and contiguous); w_q [n_dim * k_dim], w_k, w_v [n_kv * k_dim] f16
- * in `layout`; gamma [k_dim] or NULL / NULL buffer (no RMSNorm); bias_q [n_dim], bias_k, bias_v [n_kv]: all three or
- * none (the reference takes has_bias from bias_q alone and would read the input buffer for a missing bias_k);
- * out_q [m, n_dim], out_k, out_v [m, n_kv]. */
-fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *input, const fa_tensor_arg *w_q, const fa_tensor_arg *w_k,
-                       const fa_tensor_arg *w_v, const fa_tensor_arg *gamma, const fa_tensor_arg *bias_q,
-                       const fa_tensor_arg *bias_k, const fa_tensor_arg *bias_v, const fa_tensor_arg *out_q,
-                       const fa_tensor_arg *out_k, const fa_tensor_arg *out_v, const fa_fused_qkv_params *params);
+/* Argument order of FusedQkvArgs. input [m, k_dim] (any rank with k_dim innermost and contiguous); w_q [n_dim *
+ * k_dim], w_k, w_v [n_kv * k_dim] in `layout`; s_q, s_k, s_v: the Q8_0 scales, NULL / NULL buffer for F16 weights (the
+ * reference passes dummies there); gamma [k_dim] or NULL / NULL buffer (no RMSNorm); bias_q [n_dim], bias_k, bias_v
+ * [n_kv]: all three or none (the reference takes has_bias from bias_q alone and would read the input buffer for a
+ * missing bias_k); out_q [m, n_dim], out_k, out_v [m, n_kv]. */
+fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
+                       const fa_tensor_arg *s_k, const fa_tensor_arg *w_v, const fa_tensor_arg *s_v,
+                       const fa_tensor_arg *input, const fa_tensor_arg *out_q, const fa_tensor_arg *out_k,
+                       const fa_tensor_arg *out_v, const fa_tensor_arg *bias_q, const fa_tensor_arg *bias_k,
+                       const fa_tensor_arg *bias_v, const fa_tensor_arg *gamma, const fa_fused_qkv_params *params);
 
 /* ---------------------------------------------------------------------------------------------
  * MatMul, weight-stream form: the step after the path (o_proj: `attn_out [m, H*D]` x W_o, residual `hidden`,
  * models/llama.json:566-585; op src/metals/matmul.rs:11-239, which runs GemvV2 for m == 1 and for canonical
- * weights; write stage src/metals/gemv/stages.rs:200-224). F16 weights only.
+ * weights; write stage src/metals/gemv/stages.rs:200-224). F16 or Q8_0 weights (b_scales as in fa_fused_qkv).
  *   output[b, r] = f16( alpha * sum_k a[b, k] * B[r, k] + bias[r] + beta * c[b, r] ),  r < n, b < m
  * transpose_b != 0: B is row-major [n, k] (Layout::RowMajor); transpose_b == 0: B is in the canonical blocked
  * layout (matmul.rs:199-207). transpose_a and activations other than none are not built
@@ -407,8 +411,9 @@ typedef struct fa_matmul_params {
     uint32_t activation;         /* 0 = none */
 } fa_matmul_params;
 
-fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b, const fa_tensor_arg *output,
-                    const fa_tensor_arg *bias, const fa_tensor_arg *c, const fa_matmul_params *params);
+fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b, const fa_tensor_arg *b_scales,
+                    const fa_tensor_arg *output, const fa_tensor_arg *bias, const fa_tensor_arg *c,
+                    const fa_matmul_params *params);
 
 /* ---------------------------------------------------------------------------------------------
  * SageAttention-style int8 Q/K decode (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170 - prose only in

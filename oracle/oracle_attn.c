@@ -671,6 +671,69 @@ void orc_matmul_gemv(const orc_f16 *x, const orc_f16 *w, const orc_f16 *bias, co
     }
 }
 
+/* One row by the Q8 recurrence of tests/gemv_v2_parity.rs:95-116 */
+static float q8_row_dot(const orc_f16 *x, const int8_t *w8, const orc_f16 *scales, size_t row, uint32_t k_dim, uint32_t n,
+                        int layout, uint32_t wpb) {
+    const size_t blocks_per_k = (k_dim + wpb - 1) / wpb;
+    float acc = 0.0f;
+    uint32_t ki = 0;
+    while (ki < k_dim) {
+        const uint32_t chunk_size = ki + 8 <= k_dim ? 8 : k_dim - ki;
+        float chunk_acc = 0.0f;
+        const float scale = orc_f16_to_f32(scales[row * blocks_per_k + ki / wpb]);
+        for (uint32_t i = 0; i < chunk_size; ++i) {
+            const uint32_t curr_k = ki + i;
+            chunk_acc += (float)w8[orc_weight_index(layout, row, curr_k, k_dim, n, wpb)] * orc_f16_to_f32(x[curr_k]);
+        }
+        acc += chunk_acc * scale;
+        ki += chunk_size;
+    }
+    return acc;
+}
+
+void orc_matmul_gemv_q8(const orc_f16 *x, const int8_t *w8, const orc_f16 *scales, const orc_f16 *bias,
+                        const orc_f16 *residual, orc_f16 *out, uint32_t m, uint32_t n, uint32_t k_dim, int layout,
+                        uint32_t wpb, float alpha, float beta, int n_threads) {
+    (void)n_threads;
+    for (uint32_t b = 0; b < m; ++b) {
+#ifdef _OPENMP
+#pragma omp parallel for num_threads(n_threads > 0 ? n_threads : 1) schedule(static)
+#endif
+        for (int64_t row = 0; row < (int64_t)n; ++row) {
+            float res = q8_row_dot(x + (size_t)b * k_dim, w8, scales, (size_t)row, k_dim, n, layout, wpb) * alpha;
+            if (bias) res += orc_f16_to_f32(bias[row]);
+            if (residual) res += orc_f16_to_f32(residual[(size_t)b * n + row]) * beta;
+            out[(size_t)b * n + row] = orc_f32_to_f16(res);
+        }
+    }
+}
+
+void orc_fused_qkv_q8(const orc_f16 *x, const int8_t *w_q, const orc_f16 *s_q, const int8_t *w_k, const orc_f16 *s_k,
+                      const int8_t *w_v, const orc_f16 *s_v, const orc_f16 *gamma, const orc_f16 *bias_q,
+                      const orc_f16 *bias_k, const orc_f16 *bias_v, orc_f16 *out_q, orc_f16 *out_k, orc_f16 *out_v,
+                      uint32_t k_dim, uint32_t n_dim, uint32_t n_kv, uint32_t m, int layout, uint32_t wpb, float eps,
+                      int n_threads) {
+    orc_f16 *xn = (orc_f16 *)malloc(sizeof(orc_f16) * (k_dim ? k_dim : 1));
+    for (uint32_t b = 0; b < m; ++b) {
+        const orc_f16 *xr = x + (size_t)b * k_dim;
+        if (gamma) {
+            float sum_sq = 0.0f;
+            for (uint32_t j = 0; j < k_dim; ++j) {
+                const float xf = orc_f16_to_f32(xr[j]);
+                sum_sq += xf * xf;
+            }
+            const float inv_rms = 1.0f / sqrtf(sum_sq / (float)k_dim + eps);
+            for (uint32_t j = 0; j < k_dim; ++j) xn[j] = orc_f32_to_f16(orc_f16_to_f32(xr[j]) * inv_rms * orc_f16_to_f32(gamma[j]));
+        } else {
+            memcpy(xn, xr, sizeof(orc_f16) * k_dim);
+        }
+        orc_matmul_gemv_q8(xn, w_q, s_q, bias_q, NULL, out_q + (size_t)b * n_dim, 1, n_dim, k_dim, layout, wpb, 1.0f, 0.0f, n_threads);
+        orc_matmul_gemv_q8(xn, w_k, s_k, bias_k, NULL, out_k + (size_t)b * n_kv, 1, n_kv, k_dim, layout, wpb, 1.0f, 0.0f, n_threads);
+        orc_matmul_gemv_q8(xn, w_v, s_v, bias_v, NULL, out_v + (size_t)b * n_kv, 1, n_kv, k_dim, layout, wpb, 1.0f, 0.0f, n_threads);
+    }
+    free(xn);
+}
+
 /* ------------------------------------------------------------------ Sage-style int8 Q/K */
 
 void orc_sage_k_mean(const orc_f16 *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim, uint32_t kv_len,

@@ -43,6 +43,9 @@
  *                             plus the write stage's residual term (src/metals/gemv/stages.rs:206-222, source only:
  *                             no reference test exercises beta / residual -> that term is PARITY UNPINNED by tests,
  *                             pinned here against float64 and by linearity in beta)
+ *   orc_*_q8                  pinned: transcription of the reference test's Q8 CPU helper (tests/gemv_v2_parity.rs:82-125)
+ *                             checked against float64 on the dequantised weights; the fused QKV form applies the same
+ *                             per-8-chunk recurrence to the normalised input (no reference CPU helper combines them)
  *   orc_fused_qkv             pinned: transcription of the reference test's CPU helpers (tests/qkv_parity_f16.rs:17-72)
  *                             checked against float64 matrix products; orc_weight_index pinned as a bijection that
  *                             reduces to the row-major index per 32-feature block (src/compound/stages/layout.rs:79-100)
@@ -184,6 +187,19 @@ void orc_fused_qkv(const orc_f16 *x, const orc_f16 *w_q, const orc_f16 *w_k, con
  * (src/metals/gemv/stages.rs:206-222). layout / wpb as in orc_weight_index. */
 void orc_matmul_gemv(const orc_f16 *x, const orc_f16 *w, const orc_f16 *bias, const orc_f16 *residual, orc_f16 *out,
                      uint32_t m, uint32_t n, uint32_t k_dim, int layout, uint32_t wpb, float alpha, float beta, int n_threads);
+
+/* Q8_0 weights (src/metals/policies/policy_q8.metal): int8 values w8 in `layout`, f16 scales [n, ceil(k_dim / wpb)]
+ * row-major. Per row: acc += (sum over a chunk of 8 consecutive k of w8*x) * scale(block of the chunk), k ascending
+ * (tests/gemv_v2_parity.rs:82-125); then alpha, bias, beta*residual, one rounding, as orc_matmul_gemv. */
+void orc_matmul_gemv_q8(const orc_f16 *x, const int8_t *w8, const orc_f16 *scales, const orc_f16 *bias,
+                        const orc_f16 *residual, orc_f16 *out, uint32_t m, uint32_t n, uint32_t k_dim, int layout,
+                        uint32_t wpb, float alpha, float beta, int n_threads);
+/* orc_fused_qkv with Q8_0 weights: same normalisation, each projection by the Q8 recurrence above. */
+void orc_fused_qkv_q8(const orc_f16 *x, const int8_t *w_q, const orc_f16 *s_q, const int8_t *w_k, const orc_f16 *s_k,
+                      const int8_t *w_v, const orc_f16 *s_v, const orc_f16 *gamma, const orc_f16 *bias_q,
+                      const orc_f16 *bias_k, const orc_f16 *bias_v, orc_f16 *out_q, orc_f16 *out_k, orc_f16 *out_v,
+                      uint32_t k_dim, uint32_t n_dim, uint32_t n_kv, uint32_t m, int layout, uint32_t wpb, float eps,
+                      int n_threads);
 
 /* Sage-style int8 Q/K (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170).
  * K smoothing: subtract per-(head, channel) mean over the sequence (f32), quantise per block of

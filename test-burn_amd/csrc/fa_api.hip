@@ -734,10 +734,31 @@ static const __half *half_ptr(const fa_tensor_arg *t) {
     return reinterpret_cast<const __half *>(static_cast<const char *>(t->buffer) + t->offset);
 }
 
-extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *input, const fa_tensor_arg *w_q, const fa_tensor_arg *w_k,
-                                  const fa_tensor_arg *w_v, const fa_tensor_arg *gamma, const fa_tensor_arg *bias_q,
-                                  const fa_tensor_arg *bias_k, const fa_tensor_arg *bias_v, const fa_tensor_arg *out_q,
-                                  const fa_tensor_arg *out_k, const fa_tensor_arg *out_v, const fa_fused_qkv_params *p) {
+// Weight dtype of a projection: F16, or Q8_0 (int8 values + f16 block scales [rows, k / 32]).
+static fa_status weight_kind(const fa_tensor_arg *w, const fa_tensor_arg *scales, const char *what, size_t rows, size_t k, bool &q8) {
+    if (w->dtype == FA_DTYPE_F16) {
+        q8 = false;
+        return FA_OK;
+    }
+    if (w->dtype == FA_DTYPE_Q8_0 || w->dtype == FA_DTYPE_I8) {
+        q8 = true;
+        if (!present(scales)) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: scales of the Q8_0 weights %s", what);
+        const size_t need = rows * (k / 32);
+        const size_t have = scales->dtype == FA_DTYPE_F16 ? numel(scales) : numel(scales) / 2;  // f16, or the scale bytes
+        if (scales->dtype != FA_DTYPE_F16 && scales->dtype != FA_DTYPE_U8 && scales->dtype != FA_DTYPE_I8)
+            return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "%s: Q8_0 scales must be f16 values (F16, or their bytes as U8)", what);
+        if (scales->rank > 0 && have < need) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %s holds %zu scales, %zu needed", what, have, need);
+        if ((uintptr_t)half_ptr(scales) % 2 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "%s: scales must be 2-byte aligned", what);
+        return FA_OK;
+    }
+    return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "%s: weight dtype %u: F16 and Q8_0 weights are built, no other block-quantised policy", what, w->dtype);
+}
+
+extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
+                                  const fa_tensor_arg *s_k, const fa_tensor_arg *w_v, const fa_tensor_arg *s_v,
+                                  const fa_tensor_arg *input, const fa_tensor_arg *out_q, const fa_tensor_arg *out_k,
+                                  const fa_tensor_arg *out_v, const fa_tensor_arg *bias_q, const fa_tensor_arg *bias_k,
+                                  const fa_tensor_arg *bias_v, const fa_tensor_arg *gamma, const fa_fused_qkv_params *p) {
     FA_NEED(ctx, "ctx");
     FA_NEED(p, "params");
     const struct { const fa_tensor_arg *t; const char *name; } req[] = {{input, "input"}, {w_q, "w_q"}, {w_k, "w_k"}, {w_v, "w_v"},
@@ -746,10 +767,11 @@ extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *input, const
         FA_NEED(r.t, r.name);
         if (!r.t->buffer) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: %s", r.name);
     }
-    for (const fa_tensor_arg *w : {w_q, w_k, w_v})
-        if (w->dtype != FA_DTYPE_F16)
-            return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: weight dtype %u: only F16 weights are built (no block-quantised policies)", w->dtype);
-    if (w_q->dtype != w_k->dtype || w_q->dtype != w_v->dtype)
+    bool q8 = false, q8_k = false, q8_v = false;
+    FA_TRY(weight_kind(w_q, s_q, "w_q", p->n_dim, p->k_dim, q8));
+    FA_TRY(weight_kind(w_k, s_k, "w_k", p->n_kv, p->k_dim, q8_k));
+    FA_TRY(weight_kind(w_v, s_v, "w_v", p->n_kv, p->k_dim, q8_v));
+    if (q8 != q8_k || q8 != q8_v)  // the reference falls back to three separate projections there (qkv_step.rs:243-259)
         return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: mixed weight dtypes are not supported");
     for (const fa_tensor_arg *t : {input, out_q, out_k, out_v})
         if (t->dtype != FA_DTYPE_F16) return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: activations must be F16, got dtype %u", t->dtype);
@@ -790,13 +812,15 @@ extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *input, const
     L.x = half_ptr(input), L.gamma = has_norm ? half_ptr(gamma) : nullptr;
     L.k_dim = p->k_dim, L.n_dim = p->n_dim, L.n_kv = p->n_kv, L.m = m, L.eps = p->epsilon;
     L.canonical = p->layout == FA_WEIGHT_LAYOUT_CANONICAL;
+    if (q8) L.scales[0] = half_ptr(s_q), L.scales[1] = half_ptr(s_k), L.scales[2] = half_ptr(s_v);
     for (const void *ptr : {(const void *)L.w[0], (const void *)L.w[1], (const void *)L.w[2], (const void *)L.x, (const void *)L.gamma})
         if (ptr && (uintptr_t)ptr % 16 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: input, gamma and weights must be 16-byte aligned");
     return fa_launch_fused_qkv(ctx, L);
 }
 
-extern "C" fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b, const fa_tensor_arg *output,
-                               const fa_tensor_arg *bias, const fa_tensor_arg *c, const fa_matmul_params *p) {
+extern "C" fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b, const fa_tensor_arg *b_scales,
+                               const fa_tensor_arg *output, const fa_tensor_arg *bias, const fa_tensor_arg *c,
+                               const fa_matmul_params *p) {
     FA_NEED(ctx, "ctx");
     FA_NEED(p, "params");
     const struct { const fa_tensor_arg *t; const char *name; } req[] = {{a, "a"}, {b, "b"}, {output, "output"}};
@@ -804,8 +828,8 @@ extern "C" fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_ten
         FA_NEED(r.t, r.name);
         if (!r.t->buffer) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: %s", r.name);
     }
-    if (b->dtype != FA_DTYPE_F16)
-        return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "MatMul: weight dtype %u: only F16 weights are built (no block-quantised policies)", b->dtype);
+    bool q8 = false;
+    FA_TRY(weight_kind(b, b_scales, "b", p->n, p->k, q8));
     if (a->dtype != FA_DTYPE_F16 || output->dtype != FA_DTYPE_F16) return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "MatMul: a and output must be F16");
     if (p->transpose_a) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: transpose_a is not supported");
     if (p->activation != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: activation %u is not built", p->activation);
@@ -834,6 +858,7 @@ extern "C" fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_ten
     L.k_dim = p->k, L.n_dim = p->n, L.n_kv = 0, L.m = m, L.eps = 0.0f;
     L.canonical = p->transpose_b == 0;
     L.residual = has_c ? half_ptr(c) : nullptr, L.alpha = p->alpha, L.beta = p->beta;
+    if (q8) L.scales[0] = half_ptr(b_scales);
     if ((uintptr_t)L.w[0] % 16 != 0 || (uintptr_t)L.x % 16 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: a and b must be 16-byte aligned");
     return fa_launch_fused_qkv(ctx, L);
 }

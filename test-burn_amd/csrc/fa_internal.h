@@ -205,6 +205,8 @@ struct FusedQkvLaunch {
     // MatMul form (n_kv = 0, w[1] = w[2] = nullptr): out = f16(alpha * sum + bias + beta * residual)
     const __half *residual = nullptr;
     float alpha = 1.0f, beta = 0.0f;
+    // Q8_0: w[i] are int8 values in the same layouts, scales[i] f16 [rows, k_dim / 32]; nullptr = F16 weights
+    const __half *scales[3] = {nullptr, nullptr, nullptr};
 };
 fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l);
 

@@ -14,11 +14,15 @@
 //   * the 8 waves split the feature blocks of a tile; their 16 x 16 partial results are summed through LDS in a
 //     fixed order, the bias is added and the row is rounded to f16 once, as the reference does.
 // The normalised input is rounded to f16 before the products (qkv_project.metal:66-67), f32 accumulation.
+// Q8_0 weights (src/metals/policies/policy_q8.metal: int8 values, one f16 scale per 32 weights of a row, separate
+// buffers) take the same route at half the bytes: 8 bytes per lane and block, converted to f16 exactly, one matrix
+// instruction per 32-weight block whose row sums are multiplied by the block's scales (staged in LDS) and added up.
 //
 // The same kernel with one matrix, no norm and the write stage's alpha / bias / beta * residual is the m = 1 path of
 // the MatMul op (src/metals/matmul.rs:190-239 -> GemvV2, write stage src/metals/gemv/stages.rs:200-224): the o_proj
 // consumer of the attention output.
 #include "fa_internal.h"
+#include <type_traits>
 
 namespace {
 
@@ -26,6 +30,7 @@ constexpr int QKV_NT = 512, QKV_NW = QKV_NT / 64;
 constexpr int QKV_UNITS = 8;  // feature blocks per batch of requests; a wave keeps two batches in flight
 typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef float f4v_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u2v_t __attribute__((ext_vector_type(2)));
 
 struct QkvDev {
     const __half *w[3];     // W_q, W_k, W_v
@@ -39,6 +44,8 @@ struct QkvDev {
     // MatMul form (one matrix): out = f16(alpha * sum + bias + beta * residual)
     const __half *residual;  // nullable; [m, rows[0]]
     float alpha, beta;
+    // Q8_0 weights: w[i] point at int8 values (same two layouts, in elements), scales[i] at f16 [rows, k_dim / 32]
+    const __half *scales[3];
 };
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -47,6 +54,7 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+template <bool Q8>
 __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -60,6 +68,8 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     const uint32_t m0 = blockIdx.y * a.cols_per_pass, cols = min(a.cols_per_pass, a.m - m0);
     unsigned char *x_lds = smem;
     float *red = reinterpret_cast<float *>(smem + (size_t)a.cols_per_pass * a.x_stride);  // [QKV_NW][16][17], and scratch
+    // Q8: the block scales of this workgroup's rows, [tile][feature block][16 rows] f16
+    _Float16 *sc_lds = reinterpret_cast<_Float16 *>(red + QKV_NW * 16 * 17);
 
     // Where a row of the concatenated list lives: matrix, row inside it, the matrix's row count.
     auto locate = [&](uint32_t gr, int &mat, uint32_t &lrow) {
@@ -73,17 +83,20 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     // tile (consecutive lanes 64 bytes apart; requesting in address order, four lanes per row, and moving the words
     // into place with LDS permutes was slower: 10.6 us against 9.5 on 31.5 MB of weights).
     // Per tile a lane keeps the address of its block 0 and its stride from block to block.
-    auto tile_base = [&](uint32_t tile, const __half *&p0, size_t &kb_stride, bool &ok) {
+    // (Q8: the same element indices, one byte per element.)
+    typedef typename std::conditional<Q8, u2v_t, h8_t>::type wreg_t;
+    constexpr size_t WES = Q8 ? 1 : 2;  // weight element size in bytes
+    auto tile_base = [&](uint32_t tile, const unsigned char *&p0, size_t &kb_stride, bool &ok) {
         const uint32_t gr = row_begin + tile * 16 + n;
         ok = gr < row_end;
         int mat;
         uint32_t lrow;
         locate(ok ? gr : row_begin, mat, lrow);
-        const __half *base = mat == 0 ? a.w[0] : mat == 1 ? a.w[1] : a.w[2];
+        const unsigned char *base = reinterpret_cast<const unsigned char *>(mat == 0 ? a.w[0] : mat == 1 ? a.w[1] : a.w[2]);
         const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
         // canonical (blocked by 32 features): (k % 32) + 32 * (row + (k / 32) * N); row-major: row * K + k
-        p0 = a.canonical ? base + (size_t)lrow * 32 + c * 8 : base + (size_t)lrow * K + c * 8;
-        kb_stride = a.canonical ? (size_t)N * 32 : 32;
+        p0 = base + (a.canonical ? (size_t)lrow * 32 + c * 8 : (size_t)lrow * K + c * 8) * WES;
+        kb_stride = (a.canonical ? (size_t)N * 32 : 32) * WES;
     };
 
     // A wave takes the feature blocks kb = wave, wave + 8, ... of every tile, in batches of QKV_UNITS; two batches
@@ -91,18 +104,20 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     const uint32_t per_tile = (nkb + QKV_NW - 1) / QKV_NW;                // blocks of a tile per wave (upper bound)
     const uint32_t bpt = (per_tile + QKV_UNITS - 1) / QKV_UNITS;          // batches per tile
     const uint32_t n_batches = n_tiles * bpt;
-    h8_t wbuf[2][QKV_UNITS];
-    auto request = [&](h8_t(&buf)[QKV_UNITS], uint32_t batch) {
+    wreg_t wbuf[2][QKV_UNITS];
+    auto request = [&](wreg_t(&buf)[QKV_UNITS], uint32_t batch) {
         const uint32_t tile = batch / bpt, j0 = (batch % bpt) * QKV_UNITS;
-        const __half *p0;
+        const unsigned char *p0;
         size_t kb_stride;
         bool ok;
         tile_base(tile, p0, kb_stride, ok);
 #pragma unroll
         for (int i = 0; i < QKV_UNITS; ++i) {
             const uint32_t kb = (uint32_t)wave + (j0 + i) * QKV_NW;
-            const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-            buf[i] = (ok && kb < nkb) ? *reinterpret_cast<const h8_t *>(p0 + (size_t)kb * kb_stride) : z;
+            wreg_t z;
+            if constexpr (Q8) z = u2v_t{0u, 0u};
+            else z = h8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            buf[i] = (ok && kb < nkb) ? *reinterpret_cast<const wreg_t *>(p0 + (size_t)kb * kb_stride) : z;
         }
     };
     // The first input row is requested before the weights (a CU's vector loads return in request order), then the
@@ -114,6 +129,28 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
         const uint32_t k8 = tid + j * QKV_NT;
         const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
         x0[j] = k8 < K / 8 ? *reinterpret_cast<const h8_t *>(a.x + (size_t)m0 * K + k8 * 8) : z;
+    }
+    // Q8: the block scales of this workgroup's rows (scales[row][kb] f16, row-major,
+    // tests/gemv_v2_parity.rs:100-102), requested before the weights as well; they go to LDS as [tile][kb][row].
+    constexpr int SPRE = 4;
+    _Float16 sc0[SPRE];
+    const uint32_t n_scales = Q8 ? n_tiles * 16 * nkb : 0u;
+    auto scale_of = [&](uint32_t idx) -> _Float16 {
+        const uint32_t tr = idx / nkb, kb = idx - tr * nkb;  // tr = tile * 16 + row
+        const uint32_t gr = row_begin + tr;
+        if (gr >= row_end) return (_Float16)0.0f;
+        int mat;
+        uint32_t lrow;
+        locate(gr, mat, lrow);
+        const __half *sp = mat == 0 ? a.scales[0] : mat == 1 ? a.scales[1] : a.scales[2];
+        return *reinterpret_cast<const _Float16 *>(sp + (size_t)lrow * nkb + kb);
+    };
+    if (Q8) {
+#pragma unroll
+        for (int j = 0; j < SPRE; ++j) {
+            const uint32_t idx = tid + j * QKV_NT;
+            sc0[j] = idx < n_scales ? scale_of(idx) : (_Float16)0.0f;
+        }
     }
     request(wbuf[0], 0);
     if (n_batches > 1) request(wbuf[1], 1);
@@ -147,6 +184,13 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
                 *reinterpret_cast<h8_t *>(dst + k8 * 16) = v;
             }
             __syncthreads();  // `red` is reused by the next row
+        }
+    }
+    if (Q8) {
+        for (uint32_t idx = tid, j = 0; idx < n_scales; idx += QKV_NT, ++j) {
+            const _Float16 v = j < (uint32_t)SPRE ? (j == 0 ? sc0[0] : j == 1 ? sc0[1] : j == 2 ? sc0[2] : sc0[3]) : scale_of(idx);
+            const uint32_t tr = idx / nkb, kb = idx - tr * nkb;
+            sc_lds[((size_t)(tr >> 4) * nkb + kb) * 16 + (tr & 15)] = v;
         }
     }
     __syncthreads();
@@ -183,7 +227,7 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     f4v_t d = {0.0f, 0.0f, 0.0f, 0.0f};
     const bool col_ok = (uint32_t)n < cols;
     const unsigned char *x_lane = x_lds + (size_t)(col_ok ? n : 0) * a.x_stride + c * 16;
-    auto consume = [&](const h8_t(&buf)[QKV_UNITS], uint32_t batch) {
+    auto consume = [&](const wreg_t(&buf)[QKV_UNITS], uint32_t batch) {
         const uint32_t tile = batch / bpt, j0 = (batch % bpt) * QKV_UNITS;
 #pragma unroll
         for (int i = 0; i < QKV_UNITS; ++i) {
@@ -191,7 +235,31 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
             if (kb >= nkb) break;  // wave-uniform
             h8_t xb = *reinterpret_cast<const h8_t *>(x_lane + kb * 64);
             if (!col_ok) xb = h8_t{0, 0, 0, 0, 0, 0, 0, 0};
-            d = __builtin_amdgcn_mfma_f32_16x16x32_f16(buf[i], xb, d, 0, 0, 0);
+            if constexpr (Q8) {
+                // 8 int8 weights -> f16 (exact); one MFMA covers exactly one 32-weight block, whose sums are scaled
+                // per row (lane (n, c) of the result holds rows 4c..4c+3) and then accumulated
+                // int8 -> f16 without a conversion per element: s + 128 is a byte u, the f16 with bits 0x6400 | u is
+                // 1024 + u, and 1024 + u - 1152 = s exactly (two byte permutes and one packed subtraction per four)
+                const u2v_t raw = buf[i];
+                typedef _Float16 h2v_t __attribute__((ext_vector_type(2)));
+                h8_t wv;
+#pragma unroll
+                for (int hw = 0; hw < 2; ++hw) {
+                    const uint32_t u = raw[hw] ^ 0x80808080u;
+                    const h2v_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+                    const h2v_t lo = __builtin_bit_cast(h2v_t, __builtin_amdgcn_perm(0x64646464u, u, 0x05010400u)) - bias;
+                    const h2v_t hi = __builtin_bit_cast(h2v_t, __builtin_amdgcn_perm(0x64646464u, u, 0x07030602u)) - bias;
+                    wv[4 * hw + 0] = lo[0], wv[4 * hw + 1] = lo[1], wv[4 * hw + 2] = hi[0], wv[4 * hw + 3] = hi[1];
+                }
+                const f4v_t z = {0.0f, 0.0f, 0.0f, 0.0f};
+                const f4v_t blk = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv, xb, z, 0, 0, 0);
+                typedef _Float16 h4v_t __attribute__((ext_vector_type(4)));
+                const h4v_t sc = *reinterpret_cast<const h4v_t *>(sc_lds + ((size_t)tile * nkb + kb) * 16 + c * 4);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) d[q] += blk[q] * (float)sc[q];
+            } else {
+                d = __builtin_amdgcn_mfma_f32_16x16x32_f16(buf[i], xb, d, 0, 0, 0);
+            }
         }
         if ((batch + 1) % bpt == 0) {
             finish_tile(tile, d);
@@ -216,6 +284,8 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     a.rows[0] = l.n_dim, a.rows[1] = l.n_kv, a.rows[2] = l.n_kv;
     a.x = l.x, a.gamma = l.gamma, a.k_dim = l.k_dim, a.m = l.m, a.eps = l.eps, a.canonical = l.canonical ? 1u : 0u;
     a.residual = l.residual, a.alpha = l.alpha, a.beta = l.beta;
+    for (int i = 0; i < 3; ++i) a.scales[i] = l.scales[i];
+    const bool q8 = l.scales[0] != nullptr;
     const uint32_t total_rows = l.n_dim + 2 * l.n_kv;
     const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
     // Workgroups: a multiple of the CU count, enough of them that a workgroup's rows fit one 16-row tile where the
@@ -234,16 +304,22 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     if (cols > 16) cols = 16;
     if (cols > l.m) cols = l.m;
     a.cols_per_pass = cols;
-    const size_t lds = (size_t)cols * a.x_stride + (size_t)QKV_NW * 16 * 17 * sizeof(float);
+    const uint32_t tiles_per_wg = ceil_div_u32(rows_per_wg, 16);
+    const size_t lds = (size_t)cols * a.x_stride + (size_t)QKV_NW * 16 * 17 * sizeof(float) +
+                       (q8 ? (size_t)tiles_per_wg * 16 * (l.k_dim / 32) * 2 : 0);
     static bool lds_allowed = false;
     if (!lds_allowed) {
-        FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+        FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)(lds_budget + 16 * 1024)));
+        FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)(lds_budget + 16 * 1024)));
         lds_allowed = true;
     }
     const dim3 grid(ceil_div_u32(total_rows, rows_per_wg), ceil_div_u32(l.m, cols));
     if (grid.y > 65535u) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv m %u needs %u passes", l.m, grid.y);
     FaLaunchScope scope(ctx, l.n_kv ? "fused_qkv_kernel" : "matmul_gemv_kernel", true);
-    scope.launch(fused_qkv_kernel, grid, dim3(QKV_NT), lds, a);
+    if (lds > lds_budget + 16 * 1024) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: k_dim %u needs %zu bytes of LDS", l.k_dim, lds);
+    if (q8) scope.launch(fused_qkv_kernel<true>, grid, dim3(QKV_NT), lds, a);
+    else scope.launch(fused_qkv_kernel<false>, grid, dim3(QKV_NT), lds, a);
     return scope.finish();
 }

@@ -122,8 +122,8 @@ PROTOTYPES = {
     "fa_flash_prefill_paged": [_vp, _PT, C.POINTER(PagedKv), _u32, _PT, _i, _u32, _u32, _u32, _u32],
     "fa_paged_gather": [_vp, C.POINTER(PagedKv), _u32, _u32, _vp, _vp, _u32],
     "fa_paged_copy_blocks": [_vp, C.POINTER(PagedKv), _vp, _vp, _u32],
-    "fa_fused_qkv": [_vp] + [_PT] * 11 + [C.POINTER(FusedQkvParams)],
-    "fa_matmul": [_vp] + [_PT] * 5 + [C.POINTER(MatMulParams)],
+    "fa_fused_qkv": [_vp] + [_PT] * 14 + [C.POINTER(FusedQkvParams)],
+    "fa_matmul": [_vp] + [_PT] * 6 + [C.POINTER(MatMulParams)],
     "fa_kv_prefix_copy": [_vp, _PT, _PT, _sz],
     "fa_kv_prefix_copy_batch": [_vp, _PT, _PT, _u32, _sz],
     "fa_align_capacity": [_sz],
@@ -366,21 +366,26 @@ class Foundry:
         check(self.lib.fa_paged_gather(self.h, C.byref(cache), seq_index, seq_len, k_out.ptr, v_out.ptr, out_capacity))
 
     def fused_qkv(self, x, w_q, w_k, w_v, out_q, out_k, out_v, k_dim, n_dim, n_kv, m=1, gamma=None, biases=None,
-                  layout=WEIGHT_LAYOUT_CANONICAL, weights_per_block=32, epsilon=1e-6):
-        """All tensors as TensorArg; gamma None = no RMSNorm; biases None or (bias_q, bias_k, bias_v)."""
+                  layout=WEIGHT_LAYOUT_CANONICAL, weights_per_block=32, epsilon=1e-6, scales=None):
+        """All tensors as TensorArg; gamma None = no RMSNorm; biases None or (bias_q, bias_k, bias_v); scales None (F16
+        weights) or (s_q, s_k, s_v) for Q8_0 weights."""
         p = FusedQkvParams(k_dim, n_dim, n_kv, m, weights_per_block, layout, epsilon)
         none = TensorArg()
         g = gamma if gamma is not None else none
         bq, bk, bv = biases if biases is not None else (none, none, none)
-        check(self.lib.fa_fused_qkv(self.h, C.byref(x), C.byref(w_q), C.byref(w_k), C.byref(w_v), C.byref(g), C.byref(bq),
-                                    C.byref(bk), C.byref(bv), C.byref(out_q), C.byref(out_k), C.byref(out_v), C.byref(p)))
+        sq, sk, sv = scales if scales is not None else (none, none, none)
+        check(self.lib.fa_fused_qkv(self.h, C.byref(w_q), C.byref(sq), C.byref(w_k), C.byref(sk), C.byref(w_v), C.byref(sv),
+                                    C.byref(x), C.byref(out_q), C.byref(out_k), C.byref(out_v), C.byref(bq), C.byref(bk),
+                                    C.byref(bv), C.byref(g), C.byref(p)))
 
     def matmul(self, a, b, output, m, n, k, bias=None, c=None, transpose_b=True, alpha=1.0, beta=0.0, transpose_a=False,
-               weights_per_block=32, activation=0):
-        """output[m, n] = alpha * a[m, k] . b^T + bias + beta * c; b row-major [n, k] (transpose_b) or canonical."""
+               weights_per_block=32, activation=0, b_scales=None):
+        """output[m, n] = alpha * a[m, k] . b^T + bias + beta * c; b row-major [n, k] (transpose_b) or canonical; b_scales
+        for Q8_0 weights."""
         p = MatMulParams(m, n, k, int(transpose_a), int(transpose_b), alpha, beta, weights_per_block, activation)
         none = TensorArg()
-        check(self.lib.fa_matmul(self.h, C.byref(a), C.byref(b), C.byref(output), C.byref(bias if bias is not None else none),
+        check(self.lib.fa_matmul(self.h, C.byref(a), C.byref(b), C.byref(b_scales if b_scales is not None else none),
+                                 C.byref(output), C.byref(bias if bias is not None else none),
                                  C.byref(c if c is not None else none), C.byref(p)))
 
     def paged_copy_blocks(self, cache, src_ids, dst_ids, n_pairs):

@@ -406,17 +406,17 @@ struct FusedQkvStep;
 struct CompiledFusedQkvStep : CompiledStep {
     const FusedQkvStep *step;
     size_t input_idx, w_q_idx, w_k_idx, w_v_idx, out_q_idx, out_k_idx, out_v_idx;
-    std::optional<size_t> gamma_idx, bias_q_idx, bias_k_idx, bias_v_idx;
+    std::optional<size_t> gamma_idx, bias_q_idx, bias_k_idx, bias_v_idx, s_q_idx, s_k_idx, s_v_idx;
     void execute(Foundry &foundry, const FastBindings &fast, const TensorBindings &bindings, const SymbolTable &) const override;
     const char *name() const override { return "FusedQkv"; }
 };
 
-// src/metals/gemv/qkv_step.rs:14-37: RMSNorm(input) -> parallel Q/K/V projection -> three outputs. The scale
-// tensors (s_q, s_k, s_v) and `strategy` of the reference belong to its block-quantised policies and dispatch
-// tuning and have no counterpart; `rms_eps` is the reference's string variable of that name (default 1e-6).
+// src/metals/gemv/qkv_step.rs:14-37: RMSNorm(input) -> parallel Q/K/V projection -> three outputs. s_q, s_k, s_v are
+// the block scales of Q8_0 weights (absent for F16); `strategy` of the reference is dispatch tuning and has no
+// counterpart; `rms_eps` is the reference's string variable of that name (default 1e-6).
 struct FusedQkvStep {
     Ref input, w_q, w_k, w_v, out_q, out_k, out_v;
-    std::optional<Ref> gamma, bias_q, bias_k, bias_v;
+    std::optional<Ref> gamma, bias_q, bias_k, bias_v, s_q, s_k, s_v;
     DynamicU32 k_dim, n_dim, n_kv, m, weights_per_block = 32;
     WeightLayout layout = WeightLayout::Canonical;
     float rms_eps = 1e-6f;
@@ -433,6 +433,7 @@ struct FusedQkvStep {
             return s.get_or_create(b.interpolate(*r));
         };
         c->gamma_idx = opt(gamma), c->bias_q_idx = opt(bias_q), c->bias_k_idx = opt(bias_k), c->bias_v_idx = opt(bias_v);
+        c->s_q_idx = opt(s_q), c->s_k_idx = opt(s_k), c->s_v_idx = opt(s_v);
         std::vector<std::unique_ptr<CompiledStep>> out;
         out.push_back(std::move(c));
         return out;
@@ -457,8 +458,9 @@ inline void CompiledFusedQkvStep::execute(Foundry &foundry, const FastBindings &
     p.k_dim = s.k_dim.resolve(bindings), p.n_dim = s.n_dim.resolve(bindings), p.n_kv = s.n_kv.resolve(bindings);
     p.m = std::max<uint32_t>(s.m.resolve(bindings), 1);  // qkv_step.rs:236
     p.weights_per_block = s.weights_per_block.resolve(bindings), p.layout = (uint32_t)s.layout, p.epsilon = s.rms_eps;
-    check(fa_fused_qkv(foundry.ctx(), input.c(), w_q.c(), w_k.c(), w_v.c(), gamma.c(), b_q.c(), b_k.c(), b_v.c(), out_q.c(), out_k.c(),
-                       out_v.c(), &p));
+    const TensorArg s_q = opt(s_q_idx, "s_q"), s_k = opt(s_k_idx, "s_k"), s_v = opt(s_v_idx, "s_v");
+    check(fa_fused_qkv(foundry.ctx(), w_q.c(), s_q.c(), w_k.c(), s_k.c(), w_v.c(), s_v.c(), input.c(), out_q.c(), out_k.c(), out_v.c(),
+                       b_q.c(), b_k.c(), b_v.c(), gamma.c(), &p));
 }
 
 // ---------------------------------------------------------------------------------------------- MatMul
@@ -466,16 +468,16 @@ struct MatMulStep;
 struct CompiledMatMulStep : CompiledStep {
     const MatMulStep *step;
     size_t a_idx, b_idx, output_idx;
-    std::optional<size_t> bias_idx, c_idx;
+    std::optional<size_t> bias_idx, c_idx, b_scales_idx;
     void execute(Foundry &foundry, const FastBindings &fast, const TensorBindings &bindings, const SymbolTable &) const override;
     const char *name() const override { return "MatMul (Unified)"; }
 };
 
 // src/metals/matmul.rs:11-31 with its defaults (:33-70): alpha 1, beta 0, weights_per_block 32. `bias` / `c` named
-// "zero" are placeholders for "absent" (:195-196). `b_scales` belongs to the block-quantised policies.
+// "zero" are placeholders for "absent" (:195-196); `b_scales` naming the weights themselves means "no scales" (:192).
 struct MatMulStep {
     Ref a = "a", b = "b", output = "output";
-    std::optional<Ref> bias, c;
+    std::optional<Ref> bias, c, b_scales;
     DynamicU32 m = 1, n = 1, k = 1;
     bool transpose_a = false, transpose_b = false;
     float alpha = 1.0f, beta = 0.0f;
@@ -490,6 +492,7 @@ struct MatMulStep {
             return s.get_or_create(bd.interpolate(*r));
         };
         cs->bias_idx = opt(bias), cs->c_idx = opt(c);
+        if (b_scales && *b_scales != b) cs->b_scales_idx = s.get_or_create(bd.interpolate(*b_scales));
         std::vector<std::unique_ptr<CompiledStep>> out;
         out.push_back(std::move(cs));
         return out;
@@ -509,7 +512,8 @@ inline void CompiledMatMulStep::execute(Foundry &foundry, const FastBindings &fa
     p.m = s.m.resolve(bindings), p.n = s.n.resolve(bindings), p.k = s.k.resolve(bindings);
     p.transpose_a = s.transpose_a ? 1 : 0, p.transpose_b = s.transpose_b ? 1 : 0, p.alpha = s.alpha, p.beta = s.beta;
     p.weights_per_block = s.weights_per_block, p.activation = 0;
-    check(fa_matmul(foundry.ctx(), a.c(), b.c(), output.c(), bias.c(), c.c(), &p));
+    const TensorArg b_scales = b_scales_idx ? TensorArg::from_tensor(need(fast, *b_scales_idx, "b_scales")) : TensorArg();
+    check(fa_matmul(foundry.ctx(), a.c(), b.c(), b_scales.c(), output.c(), bias.c(), c.c(), &p));
 }
 
 }  // namespace metallic_foundry

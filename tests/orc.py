@@ -266,6 +266,58 @@ def matmul_gemv(x, w, bias=None, residual=None, layout=0, wpb=32, alpha=1.0, bet
     return out
 
 
+def quantize_q8_0(w, wpb=32):
+    """GGUF Q8_0 of a row-major [n, k] matrix: per 32 weights of a row, scale = max|w| / 127 stored as f16 and
+    q = round(w / scale) in [-127, 127] (the generator of tests/gemv_v2_parity.rs' Q8 cases). Returns (int8 [n, k],
+    f16 scales [n, k / wpb])."""
+    w = np.asarray(w, np.float32)
+    n, k = w.shape
+    blocks = w.reshape(n, k // wpb, wpb)
+    scale = (np.abs(blocks).max(axis=2) / 127.0).astype(np.float16)
+    sf = np.where(scale == 0, np.float16(1.0), scale).astype(np.float32)
+    q = np.clip(np.rint(blocks / sf[:, :, None]), -127, 127).astype(np.int8)
+    return q.reshape(n, k), scale
+
+
+def _i8(a):
+    return np.ascontiguousarray(a, dtype=np.int8)
+
+
+def matmul_gemv_q8(x, w8, scales, bias=None, residual=None, layout=0, wpb=32, alpha=1.0, beta=0.0, n_threads=8):
+    x = _h(x)
+    m, K = x.shape
+    wf = _i8(np.asarray(w8).reshape(-1))
+    n = wf.size // K
+    sc = _h(scales)
+    out = np.zeros((m, n), np.float16)
+    nul = C.cast(None, u16p)
+    b = _h(bias) if bias is not None else None
+    r = _h(residual) if residual is not None else None
+    lib().orc_matmul_gemv_q8(_p(x, u16p), _p(wf, i8p), _p(sc, u16p), _p(b, u16p) if b is not None else nul,
+                             _p(r, u16p) if r is not None else nul, _p(out, u16p), C.c_uint32(m), C.c_uint32(n), C.c_uint32(K),
+                             C.c_int(layout), C.c_uint32(wpb), C.c_float(alpha), C.c_float(beta), C.c_int(n_threads))
+    return out
+
+
+def fused_qkv_q8(x, ws8, scales, gamma=None, biases=None, layout=0, wpb=32, eps=1e-6, n_threads=8):
+    """ws8: three int8 matrices (flat or 2-D in `layout`), scales: three f16 [rows, K / wpb]."""
+    x = _h(x)
+    m, K = x.shape
+    w = [_i8(np.asarray(a).reshape(-1)) for a in ws8]
+    sc = [_h(a) for a in scales]
+    n_dim, n_kv = w[0].size // K, w[1].size // K
+    oq, ok, ov = np.zeros((m, n_dim), np.float16), np.zeros((m, n_kv), np.float16), np.zeros((m, n_kv), np.float16)
+    g = _h(gamma) if gamma is not None else None
+    bs = [_h(b) for b in biases] if biases is not None else [None] * 3
+    nul = C.cast(None, u16p)
+    lib().orc_fused_qkv_q8(_p(x, u16p), _p(w[0], i8p), _p(sc[0], u16p), _p(w[1], i8p), _p(sc[1], u16p), _p(w[2], i8p),
+                           _p(sc[2], u16p), _p(g, u16p) if g is not None else nul,
+                           *[(_p(b, u16p) if b is not None else nul) for b in bs], _p(oq, u16p), _p(ok, u16p), _p(ov, u16p),
+                           C.c_uint32(K), C.c_uint32(n_dim), C.c_uint32(n_kv), C.c_uint32(m), C.c_int(layout), C.c_uint32(wpb),
+                           C.c_float(eps), C.c_int(n_threads))
+    return oq, ok, ov
+
+
 def paged_copy_blocks(pool, n_kv_heads, block_size, head_dim, src_ids, dst_ids):
     """In place on `pool` [n_blocks, n_kv_heads, block_size, head_dim] f16."""
     assert pool.dtype == np.float16 and pool.flags.c_contiguous

@@ -98,9 +98,19 @@ def test_fused_qkv_errors():
     args = lambda: (x.arg(), wq.arg(), wk.arg(), wv.arg(), oq.arg(), ok.arg(), ov.arg())  # noqa: E731
     f.fused_qkv(*args(), K, N, NK, 1)  # fine
     w8 = f.zeros((N * K,), np.int8)
-    with pytest.raises(fa.FoundryError) as e:  # block-quantised policies are not built
+    with pytest.raises(fa.FoundryError) as e:  # int8 (Q8_0) weights need their scales
         f.fused_qkv(x.arg(), w8.arg(), wk.arg(), wv.arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1)
+    assert e.value.variant == "InputNotFound"
+    sc = f.zeros((N, K // 32))
+    with pytest.raises(fa.FoundryError) as e:  # mixed policies: the reference falls back to three projections
+        f.fused_qkv(x.arg(), w8.arg(), wk.arg(), wv.arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1,
+                    scales=(sc.arg(), fa.TensorArg(), fa.TensorArg()))
     assert e.value.variant == "UnsupportedDtype"
+    wq4 = wq.arg(dtype=3)  # Q4_0: not built
+    with pytest.raises(fa.FoundryError) as e:
+        f.fused_qkv(x.arg(), wq4, wk.arg(), wv.arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1)
+    assert e.value.variant == "UnsupportedDtype"
+    sc.free()
     with pytest.raises(fa.FoundryError) as e:
         f.fused_qkv(*args(), 48, N, NK, 1)
     assert e.value.variant in ("OperationNotSupported", "InvalidShape")
@@ -177,9 +187,73 @@ def test_matmul_errors():
         f.matmul(a.arg(), b.arg(), o.arg(), 1, 33, 64)
     assert e.value.variant == "InvalidShape"
     b8 = f.zeros((32 * 64,), np.int8)
-    with pytest.raises(fa.FoundryError) as e:
+    with pytest.raises(fa.FoundryError) as e:  # Q8_0 weights without scales
         f.matmul(a.arg(), b8.arg(), o.arg(), 1, 32, 64)
+    assert e.value.variant == "InputNotFound"
+    with pytest.raises(fa.FoundryError) as e:  # Q4_0: not built
+        f.matmul(a.arg(), b.arg(dtype=3), o.arg(), 1, 32, 64)
     assert e.value.variant == "UnsupportedDtype"
     f.synchronize()
     for z in (a, b, o, b8):
+        z.free()
+
+
+# ---------------------------------------------------------------- Q8_0 weights
+
+@pytest.mark.parametrize("K,N,NK,m,norm,bias,layout", [
+    (1024, 1024, 128, 1, True, True, 1),
+    (3072, 3072, 1024, 1, True, False, 1),   # Llama-3.2-3B decode
+    (896, 896, 128, 5, True, True, 1),
+    (896, 896, 128, 20, False, True, 0),     # row-major, two passes of input rows
+    (64, 40, 24, 3, True, True, 1),
+])
+def test_fused_qkv_q8_equals_oracle(K, N, NK, m, norm, bias, layout):
+    announce("fused qkv q8", K, N, NK, m, norm, bias, layout)
+    f = ctx()
+    rng = np.random.default_rng(K + N + m + 1)
+    x, g, ws, bs = _data(rng, K, N, NK, m)
+    q8 = [orc.quantize_q8_0(w) for w in ws]
+    want = orc.fused_qkv_q8(x, [q for q, _ in q8], [s for _, s in q8], gamma=g if norm else None, biases=bs if bias else None)
+    dev_w = [f.array(orc.to_canonical(q) if layout == 1 else q.reshape(-1)) for q, _ in q8]
+    dev_s = [f.array(s) for _, s in q8]
+    dx, dg = f.array(x), f.array(g)
+    db = [f.array(b) for b in bs]
+    outs = [f.zeros((m, n)) for n in (N, NK, NK)]
+    f.fused_qkv(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), outs[0].arg(), outs[1].arg(), outs[2].arg(),
+                K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout,
+                scales=[s.arg() for s in dev_s])
+    for o, w, name in zip(outs, want, "qkv"):
+        got = o.download()
+        assert np.all(np.isfinite(got)), name
+        assert _close(got, w, K), (name, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
+    for b in dev_w + dev_s + [dx, dg] + db + outs:
+        b.free()
+
+
+@pytest.mark.parametrize("m,n,k,canonical,bias,resid,alpha,beta", [
+    (1, 128, 128, False, False, False, 1.0, 0.0),
+    (1, 3072, 3072, True, False, True, 1.0, 1.0),   # o_proj
+    (1, 256, 256, True, True, False, 0.5, 0.0),
+    (7, 896, 896, True, True, True, 1.0, 0.5),
+])
+def test_matmul_q8_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta):
+    announce("matmul q8", m, n, k, canonical, bias, resid, alpha, beta)
+    f = ctx()
+    rng = np.random.default_rng(m + n + k + 2)
+    x = rng.uniform(-1, 1, (m, k)).astype(np.float16)
+    w8, sc = orc.quantize_q8_0(rng.uniform(-0.1, 0.1, (n, k)).astype(np.float16))
+    b = rng.uniform(-0.1, 0.1, n).astype(np.float16)
+    c = rng.uniform(-1, 1, (m, n)).astype(np.float16)
+    want = orc.matmul_gemv_q8(x, w8, sc, b if bias else None, c if resid else None, 0, 32, alpha, beta)
+    dx, dw, ds = f.array(x), f.array(orc.to_canonical(w8) if canonical else w8.reshape(-1)), f.array(sc)
+    db, dc, out = f.array(b), f.array(c), f.zeros((m, n))
+    f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, bias=db.arg() if bias else None, c=dc.arg() if resid else None,
+             transpose_b=not canonical, alpha=alpha, beta=beta, b_scales=ds.arg())
+    g, wv = out.download().astype(np.float64), want.astype(np.float64)
+    assert np.all(np.abs(g - wv) <= 2 * np.maximum(np.abs(wv), 2.0 ** -10) * 2.0 ** -10 + 1e-4), float(np.max(np.abs(g - wv)))
+    with pytest.raises(fa.FoundryError) as e:  # Q8_0 weights without their scales
+        f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, transpose_b=not canonical)
+    assert e.value.variant == "InputNotFound"
+    f.synchronize()
+    for z in (dx, dw, ds, db, dc, out):
         z.free()

@@ -659,3 +659,35 @@ def test_matmul_gemv_vs_float64_and_linearity(m, n, k, alpha, beta):
     assert np.all(np.abs(got.astype(np.float64) - ref) <= 1.5 * np.maximum(np.abs(ref), 2.0 ** -10) * 2.0 ** -10 + 1e-4)
     assert np.array_equal(orc.matmul_gemv(x, w, b, c, 0, 32, alpha, 0.0), orc.matmul_gemv(x, w, b, None, 0, 32, alpha, 0.0))
     assert np.array_equal(orc.matmul_gemv(x, np.zeros_like(w), None, c, 0, 32, 1.0, 1.0), c)  # zero weights: out = residual
+
+
+def test_q8_0_projections_vs_float64_on_dequantised_weights():
+    """The Q8 recurrence (tests/gemv_v2_parity.rs:82-125: per 8 weights an integer-valued partial sum times the block
+    scale) against float64 products with the dequantised weights w8 * scale; the quantiser's round trip error is
+    within half a step of each block's scale; both layouts give the same bits."""
+    rng = np.random.default_rng(9)
+    m, n, k = 3, 40, 96
+    x = rng.uniform(-1, 1, (m, k)).astype(np.float16)
+    w = rng.uniform(-0.1, 0.1, (n, k)).astype(np.float16)
+    b = rng.uniform(-0.1, 0.1, n).astype(np.float16)
+    c = rng.uniform(-1, 1, (m, n)).astype(np.float16)
+    w8, sc = orc.quantize_q8_0(w)
+    deq = w8.astype(np.float64).reshape(n, k // 32, 32) * sc.astype(np.float64)[:, :, None]
+    assert np.all(np.abs(deq.reshape(n, k) - w.astype(np.float64)) <= 0.5 * np.repeat(sc.astype(np.float64), 32, axis=1) + 1e-6)
+    got = orc.matmul_gemv_q8(x, w8, sc, b, c, 0, 32, 0.5, 0.75)
+    assert np.array_equal(got, orc.matmul_gemv_q8(x, orc.to_canonical(w8), sc, b, c, 1, 32, 0.5, 0.75))
+    ref = 0.5 * (x.astype(np.float64) @ deq.reshape(n, k).T) + b.astype(np.float64) + 0.75 * c.astype(np.float64)
+    assert np.all(np.abs(got.astype(np.float64) - ref) <= 1.5 * np.maximum(np.abs(ref), 2.0 ** -10) * 2.0 ** -10 + 1e-4)
+    # unit scales and small integers: the result is the exact integer dot product
+    xi = rng.integers(-3, 4, (1, 64)).astype(np.float16)
+    wi = rng.integers(-5, 6, (8, 64)).astype(np.int8)
+    one = np.ones((8, 2), np.float16)
+    assert np.array_equal(orc.matmul_gemv_q8(xi, wi, one).astype(np.int64), xi.astype(np.int64) @ wi.astype(np.int64).T)
+    # fused QKV = the same projections on the normalised input
+    g = rng.uniform(0.5, 1.5, k).astype(np.float16)
+    q, kk, v = orc.fused_qkv_q8(x, [w8, w8[:8], w8[8:16]], [sc, sc[:8], sc[8:16]], gamma=g)
+    xf = x.astype(np.float32)
+    inv = (1.0 / np.sqrt((xf.astype(np.float64) ** 2).sum(1, keepdims=True) / k + 1e-6)).astype(np.float32)
+    xn = (xf * inv * g.astype(np.float32)).astype(np.float16)
+    assert np.array_equal(q, orc.matmul_gemv_q8(xn, w8, sc))
+    assert np.array_equal(kk, orc.matmul_gemv_q8(xn, w8[:8], sc[:8])) and np.array_equal(v, orc.matmul_gemv_q8(xn, w8[8:16], sc[8:16]))
