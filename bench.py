@@ -474,6 +474,55 @@ def bench_o_proj(f, args, q8=False):
     f.profile_enable(False)
 
 
+def bench_long_decode(f, args):
+    """Llama-3.2-3B-shaped single-layer decode step at 131072 tokens of context (contiguous cache, 537 MB of K and V
+    per layer): the decode kernel where one launch is large. Two layers' caches in rotation (more than the last-level
+    cache holds)."""
+    import orc
+    H, Hkv, D, pos, NL = 24, 8, 128, 131071, 2
+    cap = pos + 1 + 128
+    rng = np.random.default_rng(0xF0DD + 9)
+    cos, sin = fa.rope_tables(5e5, D, cap)
+    dcos, dsin = f.array(cos), f.array(sin)
+    block = rng.standard_normal((Hkv, 8192, D), dtype=np.float32).astype(np.float16)
+    caches, host0 = [], None
+    for i in range(NL):
+        kc = np.tile(np.roll(block, i, axis=1), (1, (cap + 8191) // 8192, 1))[:, :cap].copy()
+        vc = np.tile(np.roll(block, i + 7, axis=1), (1, (cap + 8191) // 8192, 1))[:, :cap].copy()
+        caches.append((f.array(kc), f.array(vc)))
+        if i == 0:
+            host0 = [kc, vc]
+    q, k, v = (rng.standard_normal((1, n * D), dtype=np.float32).astype(np.float16) for n in (H, Hkv, Hkv))
+    dq, dk, dv, dout = f.array(q), f.array(k), f.array(v), f.zeros((1, H * D))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, 1, pos, cap, fa.ROPE_NORMAL)
+
+    def step(i):
+        kc, vc = caches[i % NL]
+        f.decode_step_fused(dq.arg(), dk.arg(), dv.arg(), None, kc.arg(), vc.arg(), dcos.arg(), dsin.arg(), dout.arg(), p)
+
+    step(0)
+    f.synchronize()
+    want_qr = orc.kv_prep_fused(q, k, v, host0[0], host0[1], cos, sin, orc.make_params(H, Hkv, D, 1, pos, cap, rope_mode=1))
+    want = orc.sdpa_decode(want_qr[:, 0].copy(), host0[0], host0[1], H, Hkv, D, cap, pos + 1, n_threads=16)
+    err = float(np.max(np.abs(dout.download().reshape(-1).astype(np.float64) - want.reshape(-1).astype(np.float64))))
+    for i in range(args.warmup):
+        step(i)
+    f.synchronize()
+    f.profile_reset()
+    f.profile_enable(True)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    nbytes = 2.0 * Hkv * (pos + 1) * D * 2 + 2 * Hkv * D * 2 + 2 * H * D * 2 + 2 * Hkv * D * 2 + 2 * D
+    _finish_secondary(f, args, "decode-attn layer-steps/s + achieved HBM GB/s, Llama-3.2-3B shape @128K ctx",
+                      "llama3.2-3b single-layer decode step at long context: RoPE + KV append + flash decode, batch 1, "
+                      "H24/Hkv8/D128, kv_len 131072, eager launches (profiling events on)", "fused_rope_append_decode_kernel",
+                      nbytes, dt, {"decode_max_abs_err": err})
+    f.profile_enable(False)
+
+
 def bench_paged_decode(f, args):
     """Qwen2.5-3B-shaped batched paged decode, one layer per step: 32 ragged sequences, 16-token blocks."""
     import orc
@@ -604,7 +653,7 @@ def bench_sage_decode(f, args):
     f.profile_enable(False)
 
 
-SECONDARY = {"llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
+SECONDARY = {"llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
              "llama3b_o_proj": bench_o_proj,
