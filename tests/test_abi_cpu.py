@@ -81,3 +81,25 @@ def test_capacity_policy_equals_oracle():
         req = int(rng.integers(0, 150000))
         gf = float(rng.choice([0.0, 1.1, 1.5, 2.0, 3.0]))
         assert fa.grown_capacity(alloc, req, mx, gf) == orc.grown_capacity(alloc, req, mx, gf), (alloc, req, mx, gf)
+
+
+def test_header_is_plain_c99_and_links_from_c(tmp_path):
+    """The boundary is a C ABI: the header must compile as C99 (pedantic) and a C program must link against the library
+    and call its host-only entry points."""
+    import subprocess
+    src = tmp_path / "abi.c"
+    src.write_text('#include <stdio.h>\n#include "foundry_attn.h"\n'
+                   'int main(void) {\n'
+                   '    fa_fused_qkv_params q; fa_matmul_params m; fa_kv_prep_fused_params k; fa_tensor_arg t; fa_paged_kv pg;\n'
+                   '    (void)q; (void)m; (void)k; (void)t; (void)pg;\n'
+                   '    if (fa_align_capacity(129) != 256) return 1;\n'
+                   '    if (fa_grown_capacity(2048, 2049, 8192, 2.0f) != 4096) return 2;\n'
+                   '    printf("%s %s\\n", fa_version(), fa_status_name(FA_ERR_INVALID_SHAPE));\n'
+                   '    return 0;\n}\n')
+    exe = tmp_path / "abi"
+    libdir = os.path.join(ROOT, "test-burn_amd")
+    subprocess.check_call(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                           str(src), "-o", str(exe), "-L", libdir, "-lfoundry_attn", "-Wl,-rpath," + libdir])
+    out = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, out.stdout + out.stderr
+    assert "InvalidShape" in out.stdout

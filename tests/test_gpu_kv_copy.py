@@ -182,3 +182,46 @@ def test_paged_copy_blocks_equals_oracle_and_forks_a_sequence(Hkv, D, bs):
     assert np.array_equal(bits(ko[1].download()), bits(orc.paged_gather(k_pool, parent, Hkv, bs, D, n_tok)))
     for b in [dk, dv, dbt, dl, dsrc, ddst] + ko + vo:
         b.free()
+
+
+def test_forked_sequence_shares_prefix_blocks_and_decodes_independently():
+    """Prefix sharing on the paged cache: a fork points at its parent's full blocks, owns a copy of the partly filled
+    tail block (fa_paged_copy_blocks), and then both sequences append and attend different tokens in one batched step.
+    Each must equal the oracle over its own contiguous history; the parent's tail block must not see the fork's token."""
+    announce("paged fork + decode")
+    f = ctx()
+    rng = np.random.default_rng(404)
+    H, Hkv, D, bs, n = 8, 2, 128, 16, 16 * 5 + 9   # 5 full blocks + 9 rows in the tail block
+    nblk, mb = 16, 7
+    k_hist = h16(rng.normal(size=(Hkv, n, D)))
+    v_hist = h16(rng.normal(size=(Hkv, n, D)))
+    parent = np.array([3, 11, 0, 7, 14, 5, 9], np.int32)          # block 5 is the tail, 9 is room to grow
+    fork = np.array([3, 11, 0, 7, 14, 2, 13], np.int32)           # shares five blocks, owns 2 (copy of 5) and 13
+    k_pool = h16(rng.normal(size=(nblk, Hkv, bs, D)))
+    v_pool = h16(rng.normal(size=(nblk, Hkv, bs, D)))
+    orc.paged_scatter(k_pool, parent, Hkv, bs, D, 0, n, k_hist)
+    orc.paged_scatter(v_pool, parent, Hkv, bs, D, 0, n, v_hist)
+    bt = np.stack([parent, fork])
+    dk, dv, dbt, dl = f.array(k_pool), f.array(v_pool), f.array(bt), f.array(np.array([n, n], np.uint32))
+    desc = fa.paged_kv(dk, dv, dbt, dl, nblk, Hkv, bs, D, 2, mb)
+    dsrc, ddst = f.array(np.array([5], np.int32)), f.array(np.array([2], np.int32))
+    f.paged_copy_blocks(desc, dsrc, ddst, 1)
+    cos, sin = fa.rope_tables(1e6, D, 256)
+    q, kn, vn = (h16(rng.normal(size=(2, m * D))) for m in (H, Hkv, Hkv))   # different new tokens for the two sequences
+    dq, dkn, dvn, dcos, dsin, dout = f.array(q), f.array(kn), f.array(vn), f.array(cos), f.array(sin), f.zeros((2, H * D))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, 2, 0, 0, fa.ROPE_NEOX)
+    f.decode_step_fused_paged(dq.arg(), dkn.arg(), dvn.arg(), None, desc, dcos.arg(), dsin.arg(), dout.arg(), p, mb * bs)
+    f.synchronize()
+    got = dout.download().reshape(2, H, D)
+    gk, gv = dk.download(), dv.download()
+    for s, table in enumerate((parent, fork)):
+        kc, vc = np.zeros((Hkv, n + 1, D), np.float16), np.zeros((Hkv, n + 1, D), np.float16)
+        kc[:, :n], vc[:, :n] = k_hist, v_hist
+        qr = orc.kv_prep_fused(q[s:s + 1], kn[s:s + 1], vn[s:s + 1], kc, vc, cos, sin, orc.make_params(H, Hkv, D, 1, n, n + 1, rope_mode=0))
+        want = orc.sdpa_decode(qr[:, 0].copy(), kc, vc, H, Hkv, D, n + 1, n + 1).reshape(H, D)
+        assert float(np.max(np.abs(got[s].astype(np.float64) - want.astype(np.float64)))) <= 2e-3, s
+        assert np.array_equal(bits(orc.paged_gather(gk, table, Hkv, bs, D, n + 1)), bits(kc)), s
+        assert np.array_equal(bits(orc.paged_gather(gv, table, Hkv, bs, D, n + 1)), bits(vc)), s
+    assert not np.array_equal(bits(gk[5][:, 9]), bits(gk[2][:, 9]))   # the two tails diverged at the new row
+    for b in (dk, dv, dbt, dl, dsrc, ddst, dq, dkn, dvn, dcos, dsin, dout):
+        b.free()
