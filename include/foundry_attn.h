@@ -1,7 +1,8 @@
 /*
  * foundry_attn.h - C ABI of libfoundry_attn.so: the KV-cache attention path of metallic-foundry
  * (fused RoPE + KV-cache append, flash decode, flash prefill, Sage-style int8 decode) for AMD MI355X
- * (gfx950), written in HIP.
+ * (gfx950), written in HIP; plus the steps either side of it in their decode form (FusedQkv, the o_proj
+ * MatMul) and the executor's KV-cache prefix copies and capacity policy.
  *
  * This header is the single source of truth for the boundary. Every entry point names the reference
  * interface it stands in for; paths are relative to crates/metallic-foundry/ of cchance27/test-burn.
