@@ -387,9 +387,9 @@ def bench_fused_qkv(f, args, q8=False):
         ws = [rng.uniform(-0.1, 0.1, (n, K)).astype(np.float16) for n in (N, NK, NK)]
         if q8:
             ws = [orc.quantize_q8_0(w) for w in ws]
-            layers.append(([f.array(orc.to_canonical(w)) for w, _ in ws], [f.array(sc) for _, sc in ws]))
+            layers.append(([f.array(fa.canonical_layout(w)) for w, _ in ws], [f.array(sc) for _, sc in ws]))
         else:
-            layers.append(([f.array(orc.to_canonical(w)) for w in ws], None))
+            layers.append(([f.array(fa.canonical_layout(w)) for w in ws], None))
         if i == 0:
             host0 = ws
     dx, dg = f.array(x), f.array(g)
@@ -439,10 +439,10 @@ def bench_o_proj(f, args, q8=False):
         w = rng.uniform(-0.1, 0.1, (N, K)).astype(np.float16)
         if q8:
             w8, sc = orc.quantize_q8_0(w)
-            layers.append((f.array(orc.to_canonical(w8)), f.array(sc)))
+            layers.append((f.array(fa.canonical_layout(w8)), f.array(sc)))
             w = (w8, sc)
         else:
-            layers.append((f.array(orc.to_canonical(w)), None))
+            layers.append((f.array(fa.canonical_layout(w)), None))
         if i == 0:
             host0 = w
     dx, dc, out = f.array(x), f.array(c), f.zeros((1, N))
@@ -521,6 +521,64 @@ def bench_long_decode(f, args):
                       "H24/Hkv8/D128, kv_len 131072, eager launches (profiling events on)", "fused_rope_append_decode_kernel",
                       nbytes, dt, {"decode_max_abs_err": err})
     f.profile_enable(False)
+
+
+def bench_attn_block(f, args):
+    """The attention block of a Llama-3.2-3B decode step, all 28 layers, as the reference's graph runs it
+    (models/llama.json:509-585): FusedQkv (RMSNorm + projections) -> RoPE + KV append + flash decode -> o_proj MatMul
+    with residual; F16 weights in the canonical layout, 8192 keys of context, one HIP graph of the 28 layers per step.
+    The MLP between the blocks is not part of this path; each layer's block reads the previous one's residual."""
+    L, H, Hkv, D, pos = 28, 24, 8, 128, 8192
+    dm, kvd, cap = H * D, Hkv * D, 8448
+    rng = np.random.default_rng(0xF0DD + 10)
+    cos, sin = fa.rope_tables(5e5, D, cap)
+    dcos, dsin = f.array(cos), f.array(sin)
+    base_kv = rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16)
+    wq = fa.canonical_layout(rng.uniform(-0.05, 0.05, (dm, dm)).astype(np.float16))
+    wk = fa.canonical_layout(rng.uniform(-0.05, 0.05, (kvd, dm)).astype(np.float16))
+    layers = []
+    for i in range(L):  # distinct device buffers per layer (contents rolled copies: only the addresses matter for timing)
+        layers.append(dict(kc=f.array(np.roll(base_kv, i, axis=1)), vc=f.array(np.roll(base_kv, i + 3, axis=1)),
+                           wq=f.array(np.roll(wq, i)), wk=f.array(np.roll(wk, i)), wv=f.array(np.roll(wk, i + 5)),
+                           wo=f.array(np.roll(wq, i + 9)), g=f.array(rng.uniform(0.5, 1.5, dm).astype(np.float16))))
+    hid = [f.array(rng.uniform(-1, 1, (1, dm)).astype(np.float16)), f.zeros((1, dm))]
+    dq, dk, dv, dattn = f.zeros((1, dm)), f.zeros((1, kvd)), f.zeros((1, kvd)), f.zeros((1, dm))
+    dpos = f.array(np.array([pos], np.uint32))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, 1, 0, cap, fa.ROPE_NORMAL)
+
+    def enqueue():
+        for i, ly in enumerate(layers):
+            src, dst = hid[i % 2], hid[(i + 1) % 2]
+            f.fused_qkv(src.arg(), ly["wq"].arg(), ly["wk"].arg(), ly["wv"].arg(), dq.arg(), dk.arg(), dv.arg(), dm, dm, kvd, 1,
+                        gamma=ly["g"].arg())
+            f.decode_step_fused(dq.arg(), dk.arg(), dv.arg(), None, ly["kc"].arg(), ly["vc"].arg(), dcos.arg(), dsin.arg(),
+                                dattn.arg(), p, d_position=dpos, kv_len_bound=cap)
+            f.matmul(dattn.arg(), ly["wo"].arg(), dst.arg(), 1, dm, dm, c=src.arg(), transpose_b=False, alpha=1.0, beta=1.0)
+
+    f.start_capture()
+    enqueue()
+    graph = f.end_capture()
+    for _ in range(args.warmup):
+        graph.launch()
+    f.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graph.launch()
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    finite = bool(np.all(np.isfinite(hid[0].download())))
+    nbytes = L * (2.0 * (dm + 2 * kvd) * dm + 2.0 * dm * dm + 2.0 * 2 * Hkv * (pos + 1) * D)
+    per_step = dt / args.steps
+    print(json.dumps({
+        "metric": "attention-block steps/s + achieved HBM GB/s, Llama-3.2-3B decode @8K ctx", "value": 1.0 / per_step,
+        "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": per_step * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "llama3.2-3b attention block x 28 layers per step: FusedQkv, fused RoPE + append + decode "
+                               "(+ merge), o_proj with residual; one HIP graph per step"},
+        "roofline": {"bound": "hbm", "achieved": nbytes / per_step / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": nbytes / per_step / 1e9 / HBM_PEAK_GBPS, "traffic": None, "kernel": "whole step (4 kernels per layer)",
+                     "bytes_per_step": nbytes, "us_per_layer": per_step * 1e6 / L},
+        "parity": {"outputs_finite": finite, "note": "stage-by-stage parity of this chain: tests/test_gpu_block.py"}}))
 
 
 def bench_paged_decode(f, args):
@@ -653,7 +711,7 @@ def bench_sage_decode(f, args):
     f.profile_enable(False)
 
 
-SECONDARY = {"llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
+SECONDARY = {"llama3b_attn_block": bench_attn_block, "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
              "llama3b_o_proj": bench_o_proj,

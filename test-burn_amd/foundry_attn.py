@@ -140,6 +140,17 @@ _RESTYPES = {"fa_status_name": C.c_char_p, "fa_last_error_string": C.c_char_p, "
 _lib = None
 
 
+def canonical_layout(w, weights_per_block=32):
+    """[n_rows, k_dim] row-major weights -> the flat canonical blocked order FusedQkv and MatMul read
+    (element (row, k) at (k % wpb) + wpb * (row + (k // wpb) * n_rows); metallic-loader lays tensors out this way)."""
+    n, k = w.shape
+    kk = np.arange(k)
+    idx = (kk % weights_per_block)[None, :] + weights_per_block * (np.arange(n)[:, None] + (kk // weights_per_block)[None, :] * n)
+    out = np.empty(n * k, w.dtype)
+    out[idx.reshape(-1)] = w.reshape(-1)
+    return out
+
+
 def align_capacity(capacity):
     return load().fa_align_capacity(capacity)
 
