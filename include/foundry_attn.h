@@ -401,7 +401,9 @@ fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_ar
  * transpose_b != 0: B is row-major [n, k] (Layout::RowMajor); transpose_b == 0: B is in the canonical blocked
  * layout (matmul.rs:199-207). transpose_a and activations other than none are not built
  * (FA_ERR_OPERATION_NOT_SUPPORTED). bias, c: NULL or NULL buffer = absent (the reference's "zero" placeholder).
- * Any m is accepted (16 input rows per pass over the weights); the reference's GEMM for large m is not built.
+ * Any m is accepted: up to fa_set_gemm_min_m() - 1 input rows run as passes of 16 over the weight stream; from there
+ * on (F16 weights) the op is a tiled GEMM on the matrix cores, the counterpart of the reference's GEMM for large m
+ * (src/metals/mma). Q8_0 weights take the passes at any m.
  * ------------------------------------------------------------------------------------------- */
 typedef struct fa_matmul_params {
     uint32_t m, n, k;            /* k a multiple of 32 */
@@ -415,6 +417,13 @@ typedef struct fa_matmul_params {
 fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b, const fa_tensor_arg *b_scales,
                     const fa_tensor_arg *output, const fa_tensor_arg *bias, const fa_tensor_arg *c,
                     const fa_matmul_params *params);
+
+/* Tuning override for fa_fused_qkv and fa_matmul with F16 weights: the number of input rows m from which the tiled
+ * GEMM runs instead of passes of 16 rows over the weight stream (the reference makes the same choice between GemvV2
+ * and its GEMM by m, src/metals/matmul.rs:190-239). 0 = the library's default. With a gamma the GEMM writes the
+ * normalised input (m * k_dim f16) into the context's workspace (fa_ctx_reserve_workspace before a capture).
+ * Environment: FOUNDRY_ATTN_GEMM_MIN_M (read at fa_ctx_create). */
+fa_status fa_set_gemm_min_m(fa_ctx *ctx, uint32_t min_m);
 
 /* ---------------------------------------------------------------------------------------------
  * SageAttention-style int8 Q/K decode (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170 - prose only in

@@ -1,0 +1,393 @@
+// FusedQkv and MatMul for many input rows (a prefill chunk): a tiled f16 GEMM on the matrix cores.
+// Reference: the same ops as fa_qkv.hip - src/metals/gemv/qkv_step.rs:14-120 (FusedQkv), src/metals/matmul.rs:190-239
+// (MatMul; its large-m form is a GEMM, src/metals/mma) - with the write stage of src/metals/gemv/stages.rs:200-224.
+//
+// With more than a few input rows the step is no longer a weight stream: out[m, n] = x[m, :] . W[n, :] is
+// 2 * m * n * k flops on m * k + n * k operands, so it runs as a GEMM:
+//   * a workgroup (4 waves) owns a 128 (weight rows) x 128 (input rows) output tile; a wave owns 64 x 64 of it as
+//     2 x 2 v_mfma_f32_32x32x16_f16 tiles (64 accumulator registers);
+//   * both operands move through LDS in steps of 64 features, two stages: the next step's 16-byte pieces are
+//     requested into registers before this step's matrix work and written after it, one barrier per step;
+//   * LDS layout per stage and operand: [16-byte piece of the 64 features][row], piece stride padded so that the
+//     writes (the global load's lane order) and the operand reads (32 consecutive rows per half wave) are both free of
+//     bank conflicts; the blocked ("canonical") weight layout is one contiguous 8 KiB per (tile, 32 features);
+//   * the rows of W_q, W_k, W_v are tiled per matrix (a tile never straddles two); the workgroups of one XCD take
+//     consecutive tiles of the weight rows over all input rows, so a weight tile is fetched into one L2 only;
+//   * epilogue: accumulators to LDS as f32 [input row][weight row], then alpha * sum + bias + beta * residual, one
+//     rounding to f16 (as the GEMV path), 16-byte token-major stores.
+// RMSNorm: a small kernel in front writes the normalised input, rounded to f16 as qkv_project.metal:66-67 does, into
+// the context's workspace; the GEMM reads that.
+#include "fa_internal.h"
+
+namespace {
+
+constexpr int GM_NT = 256;
+constexpr int GM_TN = 128, GM_TM = 128, GM_BK = 64;
+constexpr int GM_PIECES = GM_BK / 8;                   // 16-byte pieces of a row per step
+constexpr int GM_STRIDE_ROWMAJOR = GM_TN * 16 + 32;    // piece stride in bytes when a wave's 64 loads are 8 rows x 8 pieces
+constexpr int GM_STRIDE_CANONICAL = GM_TN * 16 + 64;   // ... and when they are 16 rows x 4 pieces
+constexpr int GM_OPERAND_BYTES = GM_PIECES * GM_STRIDE_CANONICAL;  // the larger of the two
+constexpr int GM_STAGE_BYTES = 2 * GM_OPERAND_BYTES;
+constexpr int GM_T_STRIDE = GM_TN * 4 + 16;             // epilogue tile: bytes per input row
+constexpr int GM_LDS_BYTES = 2 * GM_STAGE_BYTES > GM_TM * GM_T_STRIDE ? 2 * GM_STAGE_BYTES : GM_TM * GM_T_STRIDE;
+constexpr int GM_LOADS = GM_TN * GM_PIECES / GM_NT;     // 16-byte pieces per thread, operand and step (4)
+
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef float f4v_t __attribute__((ext_vector_type(4)));
+typedef float f16v_t __attribute__((ext_vector_type(16)));
+
+struct GemmDev {
+    const __half *w[3];
+    const __half *bias[3];
+    __half *out[3];
+    uint32_t rows[3];       // weight rows per matrix
+    uint32_t tiles[3];      // 128-row tiles per matrix
+    const __half *x;        // [m, k_dim] (already normalised when the op has a gamma)
+    const __half *residual; // nullable, [m, rows[0]]
+    uint32_t k_dim, m, m_tiles, n_tiles, canonical, vec_store;
+    float alpha, beta;
+    // split-K: the feature steps are divided over k_splits workgroups per output tile, which store f32 partial tiles
+    // [split][m][n_total]; gemm_finish_kernel adds them up in split order and applies the write stage
+    uint32_t k_splits, steps_per_split, n_total;
+    float *partial;
+};
+
+// inv_rms of each input row, then (x * inv_rms) * gamma in f32, rounded to f16 (rmsnorm.metal:17-96).
+__global__ void __launch_bounds__(256) rmsnorm_rows_kernel(const __half *x, const __half *gamma, __half *y, uint32_t K,
+                                                           float eps) {
+    __shared__ float red[4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const __half *xr = x + (size_t)blockIdx.x * K;
+    __half *yr = y + (size_t)blockIdx.x * K;
+    float ss = 0.0f;
+    for (uint32_t k8 = tid; k8 < K / 8; k8 += 256) {
+        const h8_t v = *reinterpret_cast<const h8_t *>(xr + k8 * 8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += (float)v[i] * (float)v[i];
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    if (lane == 0) red[wave] = ss;
+    __syncthreads();
+    const float tot = ((red[0] + red[1]) + red[2]) + red[3];
+    const float inv_rms = rsqrtf(tot / (float)K + eps);
+    for (uint32_t k8 = tid; k8 < K / 8; k8 += 256) {
+        h8_t v = *reinterpret_cast<const h8_t *>(xr + k8 * 8);
+        const h8_t g = *reinterpret_cast<const h8_t *>(gamma + k8 * 8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (_Float16)(((float)v[i] * inv_rms) * (float)g[i]);
+        *reinterpret_cast<h8_t *>(yr + k8 * 8) = v;
+    }
+}
+
+template <bool CANON>
+__global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    constexpr int W_STRIDE = CANON ? GM_STRIDE_CANONICAL : GM_STRIDE_ROWMAJOR;
+    constexpr int X_STRIDE = GM_STRIDE_ROWMAJOR;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t K = a.k_dim;
+
+    // Tile of this workgroup. Workgroup ids go round the 8 XCDs; the ids of one XCD are given consecutive tiles.
+    const uint32_t total = a.n_tiles * a.m_tiles * a.k_splits;
+    uint32_t v = blockIdx.x;
+    if (total % 8 == 0) v = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+    const uint32_t split = v % a.k_splits;
+    v /= a.k_splits;
+    uint32_t nt = v / a.m_tiles;
+    const uint32_t mt = v - nt * a.m_tiles;
+    int mat = 0;
+    if (nt >= a.tiles[0]) {
+        nt -= a.tiles[0], mat = 1;
+        if (nt >= a.tiles[1]) nt -= a.tiles[1], mat = 2;
+    }
+    const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
+    const __half *W = mat == 0 ? a.w[0] : mat == 1 ? a.w[1] : a.w[2];
+    const uint32_t n0 = nt * GM_TN, m0 = mt * GM_TM;
+
+    // Global pieces of this thread: GM_LOADS per operand and step.
+    //   weights, canonical: piece p = tid + 256 i of a step = (32-feature block p / 512, row (p % 512) / 4, piece p % 4)
+    //   weights, row-major and input: piece p = (row p / 8, piece p % 8)
+    const unsigned char *wp[GM_LOADS];
+    const unsigned char *xp[GM_LOADS];
+    uint32_t w_lds[GM_LOADS], x_lds[GM_LOADS];
+    bool w_ok[GM_LOADS], x_ok[GM_LOADS];
+    uint32_t w_kpiece[GM_LOADS];  // first feature of the piece within the step, for the tail guard
+    uint32_t x_kpiece[GM_LOADS];
+#pragma unroll
+    for (int i = 0; i < GM_LOADS; ++i) {
+        const uint32_t p = tid + GM_NT * i;
+        uint32_t row, piece;
+        if (CANON) {
+            const uint32_t blk = p / 512, within = p % 512;
+            row = within / 4, piece = blk * 4 + within % 4;
+            wp[i] = reinterpret_cast<const unsigned char *>(W) +
+                    ((size_t)(n0 + row) * 32 + (size_t)blk * N * 32 + (within % 4) * 8) * 2;
+        } else {
+            row = p / 8, piece = p % 8;
+            wp[i] = reinterpret_cast<const unsigned char *>(W) + ((size_t)(n0 + row) * K + piece * 8) * 2;
+        }
+        w_ok[i] = n0 + row < N;
+        w_lds[i] = piece * W_STRIDE + row * 16;
+        w_kpiece[i] = piece * 8;
+        const uint32_t xrow = p / 8, xpiece = p % 8;
+        xp[i] = reinterpret_cast<const unsigned char *>(a.x) + ((size_t)(m0 + xrow) * K + xpiece * 8) * 2;
+        x_ok[i] = m0 + xrow < a.m;
+        x_lds[i] = xpiece * X_STRIDE + xrow * 16;
+        x_kpiece[i] = xpiece * 8;
+    }
+    const size_t w_step = CANON ? (size_t)2 * N * 32 * 2 : (size_t)GM_BK * 2;  // bytes between steps
+    const size_t x_step = (size_t)GM_BK * 2;
+
+    h8_t wr[GM_LOADS], xr[GM_LOADS];
+    auto fetch = [&](uint32_t ks) {
+        const uint32_t k0 = ks * GM_BK;
+#pragma unroll
+        for (int i = 0; i < GM_LOADS; ++i) {
+            const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+            wr[i] = (w_ok[i] && k0 + w_kpiece[i] < K) ? *reinterpret_cast<const h8_t *>(wp[i] + ks * w_step) : z;
+            xr[i] = (x_ok[i] && k0 + x_kpiece[i] < K) ? *reinterpret_cast<const h8_t *>(xp[i] + ks * x_step) : z;
+        }
+    };
+    auto stash = [&](int stage) {
+        unsigned char *base = smem + stage * GM_STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < GM_LOADS; ++i) {
+            *reinterpret_cast<h8_t *>(base + w_lds[i]) = wr[i];
+            *reinterpret_cast<h8_t *>(base + GM_OPERAND_BYTES + x_lds[i]) = xr[i];
+        }
+    };
+
+    // Wave (wn, wm) owns weight rows 64 wn .. +63 and input rows 64 wm .. +63 of the tile.
+    const int wn = wave & 1, wm = wave >> 1;
+    const uint32_t a_off = (lane >> 5) * W_STRIDE + (wn * 64 + (lane & 31)) * 16;
+    const uint32_t b_off = (lane >> 5) * X_STRIDE + (wm * 64 + (lane & 31)) * 16;
+    f16v_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    const uint32_t all_steps = (K + GM_BK - 1) / GM_BK;
+    const uint32_t ks_begin = split * a.steps_per_split;
+    const uint32_t n_steps = min(all_steps, ks_begin + a.steps_per_split);  // end of this workgroup's range
+    fetch(ks_begin);
+    stash(ks_begin & 1);
+    __syncthreads();
+    for (uint32_t ks = ks_begin; ks < n_steps; ++ks) {
+        const bool more = ks + 1 < n_steps;
+        if (more) fetch(ks + 1);
+        const unsigned char *wa = smem + (ks & 1) * GM_STAGE_BYTES;
+        const unsigned char *xa = wa + GM_OPERAND_BYTES;
+#pragma unroll
+        for (int kk = 0; kk < GM_BK / 16; ++kk) {
+            h8_t fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fa[i] = *reinterpret_cast<const h8_t *>(wa + a_off + kk * 2 * W_STRIDE + i * 32 * 16);
+                fb[i] = *reinterpret_cast<const h8_t *>(xa + b_off + kk * 2 * X_STRIDE + i * 32 * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) stash((ks + 1) & 1);
+        __syncthreads();
+    }
+
+    // Accumulators -> LDS as f32 [input row][weight row]. Register r of lane l of a 32 x 32 tile is weight row
+    // 8 (r / 4) + 4 (l / 32) + r % 4, input row l % 32: four consecutive weight rows per 16-byte write.
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const uint32_t nrow = wn * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
+                const uint32_t mrow = wm * 64 + j * 32 + (lane & 31);
+                const f4v_t q = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+                *reinterpret_cast<f4v_t *>(smem + mrow * GM_T_STRIDE + nrow * 4) = q;
+            }
+    __syncthreads();
+
+    if (a.k_splits > 1) {  // partial sums only; the write stage runs in gemm_finish_kernel
+        const uint32_t col0 = (mat >= 1 ? a.rows[0] : 0u) + (mat == 2 ? a.rows[1] : 0u) + n0;
+        for (uint32_t q = tid; q < GM_TM * GM_TN / 4; q += GM_NT) {
+            const uint32_t mrow = q / (GM_TN / 4), n4 = q % (GM_TN / 4);
+            const uint32_t gm = m0 + mrow, gn = n0 + n4 * 4;
+            if (gm >= a.m || gn >= N) continue;
+            const f4v_t s = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n4 * 16);
+            float *dst = a.partial + ((size_t)split * a.m + gm) * a.n_total + col0 + n4 * 4;
+            if (a.vec_store) {
+                *reinterpret_cast<f4v_t *>(dst) = s;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (gn + e < N) dst[e] = s[e];
+            }
+        }
+        return;
+    }
+    const __half *bias = mat == 0 ? a.bias[0] : mat == 1 ? a.bias[1] : a.bias[2];
+    __half *out = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
+    for (uint32_t q = tid; q < GM_TM * GM_TN / 8; q += GM_NT) {
+        const uint32_t mrow = q / (GM_TN / 8), n8 = q % (GM_TN / 8);
+        const uint32_t gm = m0 + mrow, gn = n0 + n8 * 8;
+        if (gm >= a.m || gn >= N) continue;
+        const f4v_t s0 = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n8 * 32);
+        const f4v_t s1 = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n8 * 32 + 16);
+        const size_t o = (size_t)gm * N + gn;
+        if (a.vec_store) {  // N % 8 == 0 and 16-byte aligned tensors: whole pieces
+            const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+            const h8_t bv = bias ? *reinterpret_cast<const h8_t *>(bias + gn) : z;
+            const h8_t rv = a.residual ? *reinterpret_cast<const h8_t *>(a.residual + o) : z;
+            h8_t y;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float t = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
+                if (bias) t += (float)bv[e];
+                if (a.residual) t += a.beta * (float)rv[e];
+                y[e] = (_Float16)t;
+            }
+            *reinterpret_cast<h8_t *>(out + o) = y;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (gn + e >= N) break;
+                float t = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
+                if (bias) t += __half2float(bias[gn + e]);
+                if (a.residual) t += a.beta * __half2float(a.residual[o + e]);
+                out[o + e] = __float2half(t);
+            }
+        }
+    }
+}
+
+// Adds the split-K partial tiles in split order and applies the write stage: one thread per 8 output columns.
+__global__ void __launch_bounds__(256) gemm_finish_kernel(GemmDev a) {
+    const uint32_t groups = (a.n_total + 7) / 8;
+    const uint32_t id = blockIdx.x * 256 + threadIdx.x;
+    if (id >= a.m * groups) return;
+    const uint32_t gm = id / groups, col = (id - gm * groups) * 8;
+    int mat = 0;
+    uint32_t gn = col;
+    if (gn >= a.rows[0]) {
+        gn -= a.rows[0], mat = 1;
+        if (gn >= a.rows[1]) gn -= a.rows[1], mat = 2;
+    }
+    const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
+    const __half *bias = mat == 0 ? a.bias[0] : mat == 1 ? a.bias[1] : a.bias[2];
+    __half *out = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
+    const size_t o = (size_t)gm * N + gn;
+    if (a.vec_store) {
+        f4v_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
+        for (uint32_t sp = 0; sp < a.k_splits; ++sp) {
+            const float *src = a.partial + ((size_t)sp * a.m + gm) * a.n_total + col;
+            s0 += *reinterpret_cast<const f4v_t *>(src);
+            s1 += *reinterpret_cast<const f4v_t *>(src + 4);
+        }
+        const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+        const h8_t bv = bias ? *reinterpret_cast<const h8_t *>(bias + gn) : z;
+        const h8_t rv = a.residual ? *reinterpret_cast<const h8_t *>(a.residual + o) : z;
+        h8_t y;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float t = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
+            if (bias) t += (float)bv[e];
+            if (a.residual) t += a.beta * (float)rv[e];
+            y[e] = (_Float16)t;
+        }
+        *reinterpret_cast<h8_t *>(out + o) = y;
+    } else {
+        // a group of 8 columns of the concatenated list may straddle two matrices: element by element
+        for (uint32_t e = 0; e < 8 && col + e < a.n_total; ++e) {
+            int me = 0;
+            uint32_t ge = col + e;
+            if (ge >= a.rows[0]) {
+                ge -= a.rows[0], me = 1;
+                if (ge >= a.rows[1]) ge -= a.rows[1], me = 2;
+            }
+            const uint32_t Ne = me == 0 ? a.rows[0] : a.rows[1];
+            const __half *be = me == 0 ? a.bias[0] : me == 1 ? a.bias[1] : a.bias[2];
+            __half *oe = me == 0 ? a.out[0] : me == 1 ? a.out[1] : a.out[2];
+            float s = 0.0f;
+            for (uint32_t sp = 0; sp < a.k_splits; ++sp) s += a.partial[((size_t)sp * a.m + gm) * a.n_total + col + e];
+            float t = s * a.alpha;
+            if (be) t += __half2float(be[ge]);
+            if (a.residual) t += a.beta * __half2float(a.residual[(size_t)gm * Ne + ge]);
+            oe[(size_t)gm * Ne + ge] = __float2half(t);
+        }
+    }
+}
+
+}  // namespace
+
+fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
+    if (l.scales[0]) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "the GEMM path takes F16 weights only");
+    if (l.k_dim % 8 != 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: k_dim %u must be a multiple of 8", l.k_dim);
+    GemmDev a;
+    memset(&a, 0, sizeof(a));
+    for (int i = 0; i < 3; ++i) a.w[i] = l.w[i], a.bias[i] = l.bias[i], a.out[i] = l.out[i];
+    a.rows[0] = l.n_dim, a.rows[1] = l.n_kv, a.rows[2] = l.n_kv;
+    a.n_tiles = 0;
+    for (int i = 0; i < 3; ++i) a.tiles[i] = ceil_div_u32(a.rows[i], GM_TN), a.n_tiles += a.tiles[i];
+    a.k_dim = l.k_dim, a.m = l.m, a.m_tiles = ceil_div_u32(l.m, GM_TM), a.canonical = l.canonical ? 1u : 0u;
+    a.residual = l.residual, a.alpha = l.alpha, a.beta = l.beta;
+    a.x = l.x;
+    auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    bool vec = true;
+    for (int i = 0; i < 3; ++i) {
+        if (a.rows[i] == 0) continue;
+        vec = vec && a.rows[i] % 8 == 0 && aligned16(a.out[i]) && (!a.bias[i] || aligned16(a.bias[i]));
+    }
+    vec = vec && (!a.residual || aligned16(a.residual));
+    a.vec_store = vec ? 1u : 0u;
+    if (!aligned16(l.x) || !aligned16(l.w[0]) || (l.w[1] && !aligned16(l.w[1])) || (l.w[2] && !aligned16(l.w[2])) ||
+        (l.gamma && !aligned16(l.gamma)))
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: the GEMM path needs 16-byte aligned input and weights");
+    const uint64_t n_wg = (uint64_t)a.n_tiles * a.m_tiles;
+    if (n_wg > 0x7fffffffull) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %llu output tiles", (unsigned long long)n_wg);
+    // Few output tiles (a short prefill chunk): the feature steps of a tile are divided over enough workgroups to
+    // give every CU a share of the weight stream, at least 4 steps each (a 32-row chunk of Llama-3.2-3B: 47.5 us
+    // unsplit, 19.2 us with the 48 steps over 6 to 12 workgroups per tile; 512 rows: 52.9 -> 38.8 us with 3).
+    const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
+    const uint32_t all_steps = ceil_div_u32(l.k_dim, GM_BK);
+    const uint32_t target = 2 * n_cus;  // two workgroups are resident per CU
+    uint32_t splits = (uint32_t)(target / n_wg);
+    if (splits > all_steps / 4) splits = all_steps / 4;
+    if (splits < 1) splits = 1;
+    a.steps_per_split = ceil_div_u32(all_steps, splits);
+    a.k_splits = ceil_div_u32(all_steps, a.steps_per_split);
+    a.n_total = a.rows[0] + a.rows[1] + a.rows[2];
+    const size_t norm_bytes = l.gamma ? (((size_t)l.m * l.k_dim * sizeof(__half) + 255) & ~(size_t)255) : 0;
+    const size_t partial_bytes = a.k_splits > 1 ? (size_t)a.k_splits * l.m * a.n_total * sizeof(float) : 0;
+    if (norm_bytes + partial_bytes) FA_TRY(fa_ensure_workspace(ctx, norm_bytes + partial_bytes));
+    a.partial = (float *)((char *)ctx->workspace + norm_bytes);
+    if (a.k_splits > 1 && a.n_total % 8 != 0) a.vec_store = 0;
+    if (l.gamma) {
+        FaLaunchScope norm(ctx, "rmsnorm_rows_kernel", true);
+        norm.launch(rmsnorm_rows_kernel, dim3(l.m), dim3(256), 0, l.x, l.gamma, (__half *)ctx->workspace, l.k_dim, l.eps);
+        FA_TRY(norm.finish());
+        a.x = (const __half *)ctx->workspace;
+    }
+    static bool lds_allowed = false;
+    if (!lds_allowed) {
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        lds_allowed = true;
+    }
+    FaLaunchScope scope(ctx, l.n_kv ? "fused_qkv_gemm_kernel" : "matmul_gemm_kernel", true);
+    const uint32_t grid = (uint32_t)n_wg * a.k_splits;
+    if (l.canonical) scope.launch(qkv_gemm_kernel<true>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+    else scope.launch(qkv_gemm_kernel<false>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+    FA_TRY(scope.finish());
+    if (a.k_splits > 1) {
+        FaLaunchScope fin(ctx, "gemm_finish_kernel", true);
+        fin.launch(gemm_finish_kernel, dim3(ceil_div_u32(l.m * ceil_div_u32(a.n_total, 8), 256)), dim3(256), 0, a);
+        FA_TRY(fin.finish());
+    }
+    return FA_OK;
+}

@@ -286,6 +286,15 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     a.residual = l.residual, a.alpha = l.alpha, a.beta = l.beta;
     for (int i = 0; i < 3; ++i) a.scales[i] = l.scales[i];
     const bool q8 = l.scales[0] != nullptr;
+    // More than a few input rows: no longer a weight stream but a GEMM (fa_gemm.hip). Measured on 5120 x 3072 with a
+    // gamma, passes of this kernel against the GEMM (norm kernel, split-K GEMM, finish kernel): m = 8: 15.0 / 18.5 us,
+    // m = 12 (from where only one workgroup's input rows fit a CU's LDS): 30.3 / 18.2, m = 16: 37.3 / 18.7,
+    // m = 32: 76.8 / 19.8.
+    constexpr uint32_t GEMM_MIN_M_DEFAULT = 12;
+    auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    const bool gemm_ok = !q8 && l.k_dim % 8 == 0 && aligned16(l.x) && aligned16(l.w[0]) && aligned16(l.w[1]) &&
+                         aligned16(l.w[2]) && aligned16(l.gamma);
+    if (gemm_ok && l.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : GEMM_MIN_M_DEFAULT)) return fa_launch_fused_qkv_gemm(ctx, l);
     const uint32_t total_rows = l.n_dim + 2 * l.n_kv;
     const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
     // Workgroups: a multiple of the CU count, enough of them that a workgroup's rows fit one 16-row tile where the

@@ -115,6 +115,7 @@ PROTOTYPES = {
     "fa_set_decode_variant": [_vp, C.POINTER(DecodeVariant)],
     "fa_set_prefill_split_k": [_vp, C.c_uint32],
     "fa_set_prefill_variant": [_vp, C.c_uint32],
+    "fa_set_gemm_min_m": [_vp, C.c_uint32],
     "fa_kv_prep_fused_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _u32, _PT, _PT,
                                C.POINTER(KvPrepFusedParams)],
     "fa_kv_prep_decode_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _PT, _PT, C.POINTER(KvPrepFusedParams)],
@@ -287,6 +288,10 @@ class Foundry:
         """No arguments: the library's defaults (partition size by the launch rule, separate merge kernel)."""
         v = DecodeVariant(keys_per_split, merge)
         check(self.lib.fa_set_decode_variant(self.h, C.byref(v)))
+
+    def set_gemm_min_m(self, min_m=0):
+        """Input rows from which FusedQkv / MatMul with F16 weights run as a GEMM; 0 = the library's default."""
+        check(self.lib.fa_set_gemm_min_m(self.h, min_m))
 
     def set_prefill_split_k(self, split_k=0):
         check(self.lib.fa_set_prefill_split_k(self.h, split_k))
