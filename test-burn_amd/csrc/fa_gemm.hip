@@ -24,8 +24,13 @@ namespace {
 constexpr int GM_NT = 256;
 constexpr int GM_TN = 128, GM_TM = 128, GM_BK = 64;
 constexpr int GM_PIECES = GM_BK / 8;                   // 16-byte pieces of a row per step
-constexpr int GM_STRIDE_ROWMAJOR = GM_TN * 16 + 32;    // piece stride in bytes when a wave's 64 loads are 8 rows x 8 pieces
-constexpr int GM_STRIDE_CANONICAL = GM_TN * 16 + 64;   // ... and when they are 16 rows x 4 pieces
+// Piece stride in LDS, in bytes. An LDS write of 16 bytes per lane is served 8 lanes (128 bytes) at a time, and the 8
+// must fall into different 16-byte bank groups: with the stride an odd number of pieces when 8 consecutive lanes hold
+// the 8 pieces of one row, and 2 (mod 8) pieces when they hold 4 pieces of 2 rows. (Measured: with 130 and 132
+// pieces a third of the LDS cycles were bank conflicts. Giving consecutive lanes consecutive rows instead also
+// removes them, but such a request touches 64 cache lines instead of 8 and the loads get slower by more.)
+constexpr int GM_STRIDE_ROWMAJOR = GM_TN * 16 + 16;    // a wave's 64 loads are 8 rows x 8 pieces
+constexpr int GM_STRIDE_CANONICAL = GM_TN * 16 + 32;   // ... 16 rows x 4 pieces
 constexpr int GM_OPERAND_BYTES = GM_PIECES * GM_STRIDE_CANONICAL;  // the larger of the two
 constexpr int GM_STAGE_BYTES = 2 * GM_OPERAND_BYTES;
 constexpr int GM_T_STRIDE = GM_TN * 4 + 16;             // epilogue tile: bytes per input row
