@@ -426,6 +426,66 @@ def bench_fused_qkv(f, args, q8=False):
     f.profile_enable(False)
 
 
+def bench_fused_qkv_chunk(f, args, m):
+    """FusedQkv on a prefill chunk of m tokens at Llama-3.2-3B shape (F16 canonical weights, with RMSNorm): the tiled GEMM
+    (norm kernel in front; split-K and a finish kernel when the chunk is short). m = 32 is the reference's default chunk
+    - still a weight stream, priced against HBM; m = 2048 is the C4 prompt in one piece, priced against the matrix cores."""
+    import orc
+    K, N, NK, NL = 3072, 3072, 1024, 8
+    rng = np.random.default_rng(0xF0DD + 11)
+    x = rng.uniform(-1, 1, (m, K)).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, K).astype(np.float16)
+    layers, host0 = [], None
+    for i in range(NL):
+        ws = [rng.uniform(-0.1, 0.1, (n, K)).astype(np.float16) for n in (N, NK, NK)]
+        layers.append([f.array(fa.canonical_layout(w)) for w in ws])
+        if i == 0:
+            host0 = ws
+    dx, dg = f.array(x), f.array(g)
+    oq, ok, ov = f.zeros((m, N)), f.zeros((m, NK)), f.zeros((m, NK))
+
+    def step(i):
+        w = layers[i % NL]
+        f.fused_qkv(dx.arg(), w[0].arg(), w[1].arg(), w[2].arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, m, gamma=dg.arg())
+
+    step(0)
+    f.synchronize()
+    rows = min(m, 64)  # the oracle on the first rows (seconds of CPU time at most)
+    want = orc.fused_qkv(x[:rows], *host0, gamma=g)
+    err = max(float(np.max(np.abs(o.download()[:rows].astype(np.float64) - w.astype(np.float64)))) for o, w in zip((oq, ok, ov), want))
+    for i in range(args.warmup):
+        step(i)
+    f.synchronize()
+    f.profile_reset()
+    f.profile_enable(True)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    kernels = {k: f.profile_query(k) for k in ("rmsnorm_rows_kernel", "fused_qkv_gemm_kernel", "gemm_finish_kernel")}
+    f.profile_enable(False)
+    us = {k: (ms * 1e3 / n if n else 0.0) for k, (n, ms) in kernels.items()}
+    total_s = sum(us.values()) * 1e-6
+    flops = 2.0 * m * (N + 2 * NK) * K
+    nbytes = 2.0 * (N + 2 * NK) * K + 2.0 * m * K + 2.0 * K + 2.0 * m * (N + 2 * NK)
+    if m <= 128:
+        roof = {"bound": "hbm", "achieved": nbytes / total_s / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": nbytes / total_s / 1e9 / HBM_PEAK_GBPS, "bytes_per_step": nbytes}
+    else:
+        roof = {"bound": "mfma", "achieved": flops / total_s / 1e12, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": flops / total_s / 1e12 / MFMA_F16_PEAK_TFLOPS, "flops_per_step": flops}
+    roof.update({"traffic": None, "kernel": "rmsnorm_rows_kernel + fused_qkv_gemm_kernel (+ gemm_finish_kernel)",
+                 "avg_launch_us": us, "launches": kernels["fused_qkv_gemm_kernel"][0]})
+    print(json.dumps({
+        "metric": "FusedQkv chunk-steps/s, Llama-3.2-3B prefill chunk of %d tokens" % m, "value": args.steps / dt,
+        "unit": "chunk-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "llama3.2-3b FusedQkv on a chunk of %d tokens: RMSNorm + Q/K/V projections, k_dim 3072, n_dim "
+                               "3072, n_kv 1024, F16 canonical weights, eager launches (profiling events on)" % m},
+        "roofline": roof, "parity": {"qkv_max_abs_err_first_rows": err, "rows_checked": rows}}))
+
+
 def bench_o_proj(f, args, q8=False):
     """The step after the path at Llama-3.2-3B decode shape: attn_out [1, 3072] x W_o^T + hidden (MatMul with residual,
     alpha = beta = 1), F16 weights in the canonical blocked layout, one layer per step over 12 layers' weights."""
@@ -715,6 +775,8 @@ SECONDARY = {"llama3b_attn_block": bench_attn_block, "llama3b_decode_128k": benc
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
              "llama3b_o_proj": bench_o_proj,
+             "llama3b_fused_qkv_chunk32": lambda f, args: bench_fused_qkv_chunk(f, args, 32),
+             "llama3b_fused_qkv_prefill_2k": lambda f, args: bench_fused_qkv_chunk(f, args, 2048),
              "llama3b_fused_qkv_q8": lambda f, args: bench_fused_qkv(f, args, q8=True),
              "llama3b_o_proj_q8": lambda f, args: bench_o_proj(f, args, q8=True)}
 
