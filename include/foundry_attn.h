@@ -402,8 +402,8 @@ fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_ar
  * layout (matmul.rs:199-207). transpose_a and activations other than none are not built
  * (FA_ERR_OPERATION_NOT_SUPPORTED). bias, c: NULL or NULL buffer = absent (the reference's "zero" placeholder).
  * Any m is accepted: up to fa_set_gemm_min_m() - 1 input rows run as passes of 16 over the weight stream; from there
- * on (F16 weights) the op is a tiled GEMM on the matrix cores, the counterpart of the reference's GEMM for large m
- * (src/metals/mma). Q8_0 weights take the passes at any m.
+ * on the op is a tiled GEMM on the matrix cores (F16 and Q8_0 weights), the counterpart of the reference's GEMM for
+ * large m (src/metals/mma).
  * ------------------------------------------------------------------------------------------- */
 typedef struct fa_matmul_params {
     uint32_t m, n, k;            /* k a multiple of 32 */
@@ -418,7 +418,7 @@ fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b,
                     const fa_tensor_arg *output, const fa_tensor_arg *bias, const fa_tensor_arg *c,
                     const fa_matmul_params *params);
 
-/* Tuning override for fa_fused_qkv and fa_matmul with F16 weights: the number of input rows m from which the tiled
+/* Tuning override for fa_fused_qkv and fa_matmul: the number of input rows m from which the tiled
  * GEMM runs instead of passes of 16 rows over the weight stream (the reference makes the same choice between GemvV2
  * and its GEMM by m, src/metals/matmul.rs:190-239). 0 = the library's default. With a gamma the GEMM writes the
  * normalised input (m * k_dim f16) into the context's workspace (fa_ctx_reserve_workspace before a capture).

@@ -1,4 +1,4 @@
-// FusedQkv and MatMul for many input rows (a prefill chunk): a tiled f16 GEMM on the matrix cores.
+// FusedQkv and MatMul for many input rows (a prefill chunk): a tiled f16 GEMM on the matrix cores, F16 or Q8_0 weights.
 // Reference: the same ops as fa_qkv.hip - src/metals/gemv/qkv_step.rs:14-120 (FusedQkv), src/metals/matmul.rs:190-239
 // (MatMul; its large-m form is a GEMM, src/metals/mma) - with the write stage of src/metals/gemv/stages.rs:200-224.
 //
@@ -18,6 +18,7 @@
 // RMSNorm: a small kernel in front writes the normalised input, rounded to f16 as qkv_project.metal:66-67 does, into
 // the context's workspace; the GEMM reads that.
 #include "fa_internal.h"
+#include <type_traits>
 
 namespace {
 
@@ -34,7 +35,8 @@ constexpr int GM_STRIDE_CANONICAL = GM_TN * 16 + 32;   // ... 16 rows x 4 pieces
 constexpr int GM_OPERAND_BYTES = GM_PIECES * GM_STRIDE_CANONICAL;  // the larger of the two
 constexpr int GM_STAGE_BYTES = 2 * GM_OPERAND_BYTES;
 constexpr int GM_T_STRIDE = GM_TN * 4 + 16;             // epilogue tile: bytes per input row
-constexpr int GM_LDS_BYTES = 2 * GM_STAGE_BYTES > GM_TM * GM_T_STRIDE ? 2 * GM_STAGE_BYTES : GM_TM * GM_T_STRIDE;
+constexpr int GM_LDS_BYTES = (2 * GM_STAGE_BYTES > GM_TM * GM_T_STRIDE ? 2 * GM_STAGE_BYTES : GM_TM * GM_T_STRIDE) +
+                             2 * 2 * GM_TN * 2;  // + Q8 block scales [stage][2 blocks][128 rows] f16
 constexpr int GM_LOADS = GM_TN * GM_PIECES / GM_NT;     // 16-byte pieces per thread, operand and step (4)
 
 typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
@@ -42,7 +44,8 @@ typedef float f4v_t __attribute__((ext_vector_type(4)));
 typedef float f16v_t __attribute__((ext_vector_type(16)));
 
 struct GemmDev {
-    const __half *w[3];
+    const void *w[3];       // f16, or int8 (Q8_0) in the same element order
+    const __half *scales[3];  // Q8_0: f16 [rows, k_dim / 32] per matrix
     const __half *bias[3];
     __half *out[3];
     uint32_t rows[3];       // weight rows per matrix
@@ -85,7 +88,29 @@ __global__ void __launch_bounds__(256) rmsnorm_rows_kernel(const __half *x, cons
     }
 }
 
-template <bool CANON>
+typedef unsigned int u4v_t __attribute__((ext_vector_type(4)));
+typedef _Float16 h2v_t __attribute__((ext_vector_type(2)));
+
+// 16 int8 weights -> two pieces of 8 f16, exactly: s + 128 is a byte u, the f16 with bits 0x6400 | u is 1024 + u, and
+// 1024 + u - 1152 = s (two byte permutes and one packed subtraction per four weights).
+__device__ __forceinline__ void q8_to_f16(const u4v_t raw, h8_t &p0, h8_t &p1) {
+    const h2v_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+#pragma unroll
+    for (int hw = 0; hw < 4; ++hw) {
+        const uint32_t u = raw[hw] ^ 0x80808080u;
+        const h2v_t lo = __builtin_bit_cast(h2v_t, __builtin_amdgcn_perm(0x64646464u, u, 0x05010400u)) - bias;
+        const h2v_t hi = __builtin_bit_cast(h2v_t, __builtin_amdgcn_perm(0x64646464u, u, 0x07030602u)) - bias;
+        h8_t &dst = hw < 2 ? p0 : p1;
+        const int o = (hw & 1) * 4;
+        dst[o + 0] = lo[0], dst[o + 1] = lo[1], dst[o + 2] = hi[0], dst[o + 3] = hi[1];
+    }
+}
+
+// Q8: the weights become exact f16 integers on their way into LDS; the matrix instructions of one 32-feature block
+// start from zero and their sums are multiplied by the block's scale of the weight row before they are added up (the
+// recurrence of tests/gemv_v2_parity.rs:95-116). For that the operands are swapped (input rows x weight rows), so that
+// a lane holds one weight row and needs one scale per block and tile.
+template <bool CANON, bool Q8>
 __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr int W_STRIDE = CANON ? GM_STRIDE_CANONICAL : GM_STRIDE_ROWMAJOR;
@@ -107,60 +132,108 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
         if (nt >= a.tiles[1]) nt -= a.tiles[1], mat = 2;
     }
     const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
-    const __half *W = mat == 0 ? a.w[0] : mat == 1 ? a.w[1] : a.w[2];
+    const unsigned char *W = reinterpret_cast<const unsigned char *>(mat == 0 ? a.w[0] : mat == 1 ? a.w[1] : a.w[2]);
     const uint32_t n0 = nt * GM_TN, m0 = mt * GM_TM;
 
-    // Global pieces of this thread: GM_LOADS per operand and step.
+    // Global pieces of this thread: GM_LOADS 16-byte pieces per operand and step (Q8 weights: half as many).
     //   weights, canonical: piece p = tid + 256 i of a step = (32-feature block p / 512, row (p % 512) / 4, piece p % 4)
     //   weights, row-major and input: piece p = (row p / 8, piece p % 8)
-    const unsigned char *wp[GM_LOADS];
+    //   Q8 weights: 16 bytes are 16 features = two f16 pieces; canonical (block i, row tid / 2, half tid % 2),
+    //   row-major (row p / 4, quarter p % 4)
+    constexpr int W_LOADS = Q8 ? GM_LOADS / 2 : GM_LOADS;
+    const unsigned char *wp[W_LOADS];
     const unsigned char *xp[GM_LOADS];
-    uint32_t w_lds[GM_LOADS], x_lds[GM_LOADS];
-    bool w_ok[GM_LOADS], x_ok[GM_LOADS];
-    uint32_t w_kpiece[GM_LOADS];  // first feature of the piece within the step, for the tail guard
+    uint32_t w_lds[W_LOADS], x_lds[GM_LOADS];
+    bool w_ok[W_LOADS], x_ok[GM_LOADS];
+    uint32_t w_kpiece[W_LOADS];  // first feature of the piece within the step, for the tail guard
     uint32_t x_kpiece[GM_LOADS];
 #pragma unroll
-    for (int i = 0; i < GM_LOADS; ++i) {
+    for (int i = 0; i < W_LOADS; ++i) {
         const uint32_t p = tid + GM_NT * i;
         uint32_t row, piece;
-        if (CANON) {
+        if constexpr (Q8) {
+            if (CANON) {
+                row = tid / 2, piece = i * 4 + (tid % 2) * 2;
+                wp[i] = W + (size_t)(n0 + row) * 32 + (size_t)i * N * 32 + (tid % 2) * 16;
+            } else {
+                row = p / 4, piece = (p % 4) * 2;
+                wp[i] = W + (size_t)(n0 + row) * K + (p % 4) * 16;
+            }
+        } else if (CANON) {
             const uint32_t blk = p / 512, within = p % 512;
             row = within / 4, piece = blk * 4 + within % 4;
-            wp[i] = reinterpret_cast<const unsigned char *>(W) +
-                    ((size_t)(n0 + row) * 32 + (size_t)blk * N * 32 + (within % 4) * 8) * 2;
+            wp[i] = W + ((size_t)(n0 + row) * 32 + (size_t)blk * N * 32 + (within % 4) * 8) * 2;
         } else {
             row = p / 8, piece = p % 8;
-            wp[i] = reinterpret_cast<const unsigned char *>(W) + ((size_t)(n0 + row) * K + piece * 8) * 2;
+            wp[i] = W + ((size_t)(n0 + row) * K + piece * 8) * 2;
         }
         w_ok[i] = n0 + row < N;
         w_lds[i] = piece * W_STRIDE + row * 16;
         w_kpiece[i] = piece * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < GM_LOADS; ++i) {
+        const uint32_t p = tid + GM_NT * i;
         const uint32_t xrow = p / 8, xpiece = p % 8;
         xp[i] = reinterpret_cast<const unsigned char *>(a.x) + ((size_t)(m0 + xrow) * K + xpiece * 8) * 2;
         x_ok[i] = m0 + xrow < a.m;
         x_lds[i] = xpiece * X_STRIDE + xrow * 16;
         x_kpiece[i] = xpiece * 8;
     }
-    const size_t w_step = CANON ? (size_t)2 * N * 32 * 2 : (size_t)GM_BK * 2;  // bytes between steps
+    constexpr size_t WES = Q8 ? 1 : 2;  // bytes per weight
+    const size_t w_step = CANON ? (size_t)2 * N * 32 * WES : (size_t)GM_BK * WES;  // bytes between steps
     const size_t x_step = (size_t)GM_BK * 2;
+    // Q8: thread t fetches the scale of (weight row t % 128, block t / 128 of the step); scales are [row][k_dim / 32]
+    const uint32_t nkb = K / 32;
+    const __half *sc_src = nullptr;
+    bool sc_ok = false;
+    if constexpr (Q8) {
+        const __half *sp = mat == 0 ? a.scales[0] : mat == 1 ? a.scales[1] : a.scales[2];
+        const uint32_t row = tid % GM_TN;
+        sc_ok = n0 + row < N;
+        sc_src = sp + (size_t)(n0 + row) * nkb + tid / GM_TN;
+    }
+    _Float16 *sc_lds = reinterpret_cast<_Float16 *>(smem + 2 * GM_STAGE_BYTES);  // [stage][2 blocks][128 rows]
 
-    h8_t wr[GM_LOADS], xr[GM_LOADS];
+    typedef typename std::conditional<Q8, u4v_t, h8_t>::type wreg_t;
+    wreg_t wr[W_LOADS];
+    h8_t xr[GM_LOADS];
+    _Float16 sr = (_Float16)0.0f;
     auto fetch = [&](uint32_t ks) {
         const uint32_t k0 = ks * GM_BK;
 #pragma unroll
+        for (int i = 0; i < W_LOADS; ++i) {
+            wreg_t z;
+            if constexpr (Q8) z = u4v_t{0u, 0u, 0u, 0u};
+            else z = h8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            wr[i] = (w_ok[i] && k0 + w_kpiece[i] < K) ? *reinterpret_cast<const wreg_t *>(wp[i] + ks * w_step) : z;
+        }
+#pragma unroll
         for (int i = 0; i < GM_LOADS; ++i) {
             const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-            wr[i] = (w_ok[i] && k0 + w_kpiece[i] < K) ? *reinterpret_cast<const h8_t *>(wp[i] + ks * w_step) : z;
             xr[i] = (x_ok[i] && k0 + x_kpiece[i] < K) ? *reinterpret_cast<const h8_t *>(xp[i] + ks * x_step) : z;
+        }
+        if constexpr (Q8) {
+            const uint32_t kb = ks * 2 + tid / GM_TN;
+            sr = (sc_ok && kb < nkb) ? *reinterpret_cast<const _Float16 *>(sc_src + ks * 2) : (_Float16)0.0f;
         }
     };
     auto stash = [&](int stage) {
         unsigned char *base = smem + stage * GM_STAGE_BYTES;
 #pragma unroll
-        for (int i = 0; i < GM_LOADS; ++i) {
-            *reinterpret_cast<h8_t *>(base + w_lds[i]) = wr[i];
-            *reinterpret_cast<h8_t *>(base + GM_OPERAND_BYTES + x_lds[i]) = xr[i];
+        for (int i = 0; i < W_LOADS; ++i) {
+            if constexpr (Q8) {
+                h8_t p0, p1;
+                q8_to_f16(wr[i], p0, p1);
+                *reinterpret_cast<h8_t *>(base + w_lds[i]) = p0;
+                *reinterpret_cast<h8_t *>(base + w_lds[i] + W_STRIDE) = p1;
+            } else {
+                *reinterpret_cast<h8_t *>(base + w_lds[i]) = wr[i];
+            }
         }
+#pragma unroll
+        for (int i = 0; i < GM_LOADS; ++i) *reinterpret_cast<h8_t *>(base + GM_OPERAND_BYTES + x_lds[i]) = xr[i];
+        if constexpr (Q8) sc_lds[stage * 2 * GM_TN + tid] = sr;
     };
 
     // Wave (wn, wm) owns weight rows 64 wn .. +63 and input rows 64 wm .. +63 of the tile.
@@ -186,35 +259,82 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
         if (more) fetch(ks + 1);
         const unsigned char *wa = smem + (ks & 1) * GM_STAGE_BYTES;
         const unsigned char *xa = wa + GM_OPERAND_BYTES;
+        if constexpr (Q8) {
+            // not unrolled: unrolled, the scheduler starts all eight block tiles before the first scaled add and their
+            // 128 result registers spill
+#pragma unroll 1
+            for (int blk = 0; blk < 2; ++blk) {
+                h8_t fb[2][2];  // [tile][16-feature half of the block]
 #pragma unroll
-        for (int kk = 0; kk < GM_BK / 16; ++kk) {
-            h8_t fa[2], fb[2];
+                for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                fa[i] = *reinterpret_cast<const h8_t *>(wa + a_off + kk * 2 * W_STRIDE + i * 32 * 16);
-                fb[i] = *reinterpret_cast<const h8_t *>(xa + b_off + kk * 2 * X_STRIDE + i * 32 * 16);
+                    for (int h = 0; h < 2; ++h)
+                        fb[j][h] = *reinterpret_cast<const h8_t *>(xa + b_off + (blk * 2 + h) * 2 * X_STRIDE + j * 32 * 16);
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    // two tiles' block sums at a time (the scheduling fences keep the rest out of the registers)
+                    h8_t fa[2];
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        fa[h] = *reinterpret_cast<const h8_t *>(wa + a_off + (blk * 2 + h) * 2 * W_STRIDE + i * 32 * 16);
+                    const float sc = (float)sc_lds[((ks & 1) * 2 + blk) * GM_TN + wn * 64 + i * 32 + (lane & 31)];
+                    f16v_t t[2];
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) t[j][r] = 0.0f;
+                        t[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j][0], fa[0], t[j], 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) t[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j][1], fa[1], t[j], 0, 0, 0);
+#pragma unroll
+                    for (int j = 0; j < 2; ++j)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) acc[i][j][r] += t[j][r] * sc;
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
+        } else {
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int kk = 0; kk < GM_BK / 16; ++kk) {
+                h8_t fa[2], fb[2];
 #pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                for (int i = 0; i < 2; ++i) {
+                    fa[i] = *reinterpret_cast<const h8_t *>(wa + a_off + kk * 2 * W_STRIDE + i * 32 * 16);
+                    fb[i] = *reinterpret_cast<const h8_t *>(xa + b_off + kk * 2 * X_STRIDE + i * 32 * 16);
+                }
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+            }
         }
         if (more) stash((ks + 1) & 1);
         __syncthreads();
     }
 
-    // Accumulators -> LDS as f32 [input row][weight row]. Register r of lane l of a 32 x 32 tile is weight row
-    // 8 (r / 4) + 4 (l / 32) + r % 4, input row l % 32: four consecutive weight rows per 16-byte write.
+    // Accumulators -> LDS as f32 [input row][weight row]. Register r of lane l of a 32 x 32 tile is row
+    // 8 (r / 4) + 4 (l / 32) + r % 4 of the first operand and row l % 32 of the second: with the weights first, four
+    // consecutive weight rows per 16-byte write; with the input first (Q8), one float per register.
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const uint32_t nrow = wn * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
-                const uint32_t mrow = wm * 64 + j * 32 + (lane & 31);
-                const f4v_t q = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-                *reinterpret_cast<f4v_t *>(smem + mrow * GM_T_STRIDE + nrow * 4) = q;
+                if constexpr (Q8) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t mrow = wm * 64 + j * 32 + g * 8 + (lane >> 5) * 4 + e;
+                        const uint32_t nrow = wn * 64 + i * 32 + (lane & 31);
+                        *reinterpret_cast<float *>(smem + mrow * GM_T_STRIDE + nrow * 4) = acc[i][j][g * 4 + e];
+                    }
+                } else {
+                    const uint32_t nrow = wn * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
+                    const uint32_t mrow = wm * 64 + j * 32 + (lane & 31);
+                    const f4v_t q = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+                    *reinterpret_cast<f4v_t *>(smem + mrow * GM_T_STRIDE + nrow * 4) = q;
+                }
             }
     __syncthreads();
 
@@ -331,11 +451,11 @@ __global__ void __launch_bounds__(256) gemm_finish_kernel(GemmDev a) {
 }  // namespace
 
 fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
-    if (l.scales[0]) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "the GEMM path takes F16 weights only");
     if (l.k_dim % 8 != 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: k_dim %u must be a multiple of 8", l.k_dim);
     GemmDev a;
     memset(&a, 0, sizeof(a));
-    for (int i = 0; i < 3; ++i) a.w[i] = l.w[i], a.bias[i] = l.bias[i], a.out[i] = l.out[i];
+    for (int i = 0; i < 3; ++i) a.w[i] = l.w[i], a.bias[i] = l.bias[i], a.out[i] = l.out[i], a.scales[i] = l.scales[i];
+    const bool q8 = l.scales[0] != nullptr;
     a.rows[0] = l.n_dim, a.rows[1] = l.n_kv, a.rows[2] = l.n_kv;
     a.n_tiles = 0;
     for (int i = 0; i < 3; ++i) a.tiles[i] = ceil_div_u32(a.rows[i], GM_TN), a.n_tiles += a.tiles[i];
@@ -380,14 +500,21 @@ fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
     }
     static bool lds_allowed = false;
     if (!lds_allowed) {
-        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
-        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
         lds_allowed = true;
     }
     FaLaunchScope scope(ctx, l.n_kv ? "fused_qkv_gemm_kernel" : "matmul_gemm_kernel", true);
     const uint32_t grid = (uint32_t)n_wg * a.k_splits;
-    if (l.canonical) scope.launch(qkv_gemm_kernel<true>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
-    else scope.launch(qkv_gemm_kernel<false>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+    if (q8) {
+        if (l.canonical) scope.launch(qkv_gemm_kernel<true, true>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+        else scope.launch(qkv_gemm_kernel<false, true>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+    } else {
+        if (l.canonical) scope.launch(qkv_gemm_kernel<true, false>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+        else scope.launch(qkv_gemm_kernel<false, false>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+    }
     FA_TRY(scope.finish());
     if (a.k_splits > 1) {
         FaLaunchScope fin(ctx, "gemm_finish_kernel", true);

@@ -36,7 +36,7 @@ struct fa_ctx {
     uint32_t n_counters = 0;
     fa_decode_variant decode_variant{0, 1};
     uint32_t decode_waves = 0;     // waves per decode workgroup: 0 = by launch size, 4 or 8
-    uint32_t gemm_min_m = 0;       // FusedQkv / MatMul with F16 weights: input rows from which the GEMM runs (0 = default)
+    uint32_t gemm_min_m = 0;       // FusedQkv / MatMul: input rows from which the GEMM runs (0 = default)
     uint32_t prefill_split_k = 0;  // 0 = auto
     uint32_t prefill_variant = 0;  // 0 = auto, 1 = tiles staged through registers, 2 = tiles straight into LDS, two-phase loop
     // per-kernel profiling
@@ -210,7 +210,7 @@ struct FusedQkvLaunch {
     const __half *scales[3] = {nullptr, nullptr, nullptr};
 };
 fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l);
-fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l);  // fa_gemm.hip: many input rows, F16 weights
+fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l);  // fa_gemm.hip: many input rows
 
 fa_status fa_launch_sage_k_mean(fa_ctx *ctx, const void *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim,
                                 uint32_t kv_len, float *mean_out);

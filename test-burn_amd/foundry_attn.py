@@ -290,7 +290,7 @@ class Foundry:
         check(self.lib.fa_set_decode_variant(self.h, C.byref(v)))
 
     def set_gemm_min_m(self, min_m=0):
-        """Input rows from which FusedQkv / MatMul with F16 weights run as a GEMM; 0 = the library's default."""
+        """Input rows from which FusedQkv / MatMul run as a GEMM; 0 = the library's default."""
         check(self.lib.fa_set_gemm_min_m(self.h, min_m))
 
     def set_prefill_split_k(self, split_k=0):

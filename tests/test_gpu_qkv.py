@@ -21,6 +21,12 @@ def _data(rng, K, N, NK, m):
     return x, g, ws, bs
 
 
+def _paths(m):
+    """Values of the GEMM threshold to run a shape with: the library's default, plus - for a few input rows - the
+    GEMM forced, and - for short chunks - the passes of 16 rows over the weight stream forced."""
+    return [0] if m == 1 else [0, 1] if m < 12 else [0, 1 << 30] if m <= 64 else [0]
+
+
 def _close(got, want, K):
     g, w = got.astype(np.float64), want.astype(np.float64)
     ulp = np.maximum(np.abs(w), 2.0 ** -10) * 2.0 ** -10
@@ -62,11 +68,10 @@ def test_fused_qkv_equals_oracle(K, N, NK, m, norm, bias, layout):
     dx, dg = f.array(x), f.array(g)
     db = [f.array(b) for b in bs]
     outs = [f.zeros((m, n)) for n in (N, NK, NK)]
-    # from 12 input rows on the library runs the GEMM; such shapes are also forced through the passes of 16 rows over
-    # the weight stream, and the small GEMM shapes' neighbours (m < 12) through the GEMM
-    paths = [0] if m == 1 else [0, 1 << 30] if m >= 12 and m <= 64 else [0, 1] if m < 12 else [0]
+    # from 12 input rows on the library runs the GEMM; short chunks are also forced through the passes of 16 rows over
+    # the weight stream, and shapes of a few rows through the GEMM
     try:
-        for min_m in paths:
+        for min_m in _paths(m):
             f.set_gemm_min_m(min_m)
             for o in outs:
                 o.upload(np.zeros(o.shape, np.float16))
@@ -185,9 +190,8 @@ def test_matmul_gemv_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta)
     want = orc.matmul_gemv(x, w, b if bias else None, c if resid else None, 0, 32, alpha, beta)
     dx, dw = f.array(x), f.array(orc.to_canonical(w) if canonical else w.reshape(-1))
     db, dc, out = f.array(b), f.array(c), f.zeros((m, n))
-    paths = [0] if m == 1 else [0, 1 << 30] if m >= 12 and m <= 64 else [0, 1] if m < 12 else [0]
     try:
-        for min_m in paths:  # the GEMM and the passes over the weight stream, as in the FusedQkv test
+        for min_m in _paths(m):  # the GEMM and the passes over the weight stream, as in the FusedQkv test
             f.set_gemm_min_m(min_m)
             out.upload(np.zeros((m, n), np.float16))
             f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, bias=db.arg() if bias else None, c=dc.arg() if resid else None,
@@ -235,8 +239,13 @@ def test_matmul_errors():
     (1024, 1024, 128, 1, True, True, 1),
     (3072, 3072, 1024, 1, True, False, 1),   # Llama-3.2-3B decode
     (896, 896, 128, 5, True, True, 1),
-    (896, 896, 128, 20, False, True, 0),     # row-major, two passes of input rows
+    (896, 896, 128, 20, False, True, 0),     # row-major; the split-K GEMM, and two passes of input rows
     (64, 40, 24, 3, True, True, 1),
+    (896, 896, 128, 32, True, True, 1),      # a default prefill chunk
+    (3072, 3072, 1024, 200, True, False, 1), # Llama-3.2-3B, ragged input tiles
+    (1056, 200, 72, 130, True, True, 0),     # k_dim = 16.5 steps, weight rows that do not fill tiles, row-major
+    (1056, 200, 72, 130, False, True, 1),
+    (64, 40, 20, 70, True, True, 1),         # element-wise stores
 ])
 def test_fused_qkv_q8_equals_oracle(K, N, NK, m, norm, bias, layout):
     announce("fused qkv q8", K, N, NK, m, norm, bias, layout)
@@ -250,13 +259,20 @@ def test_fused_qkv_q8_equals_oracle(K, N, NK, m, norm, bias, layout):
     dx, dg = f.array(x), f.array(g)
     db = [f.array(b) for b in bs]
     outs = [f.zeros((m, n)) for n in (N, NK, NK)]
-    f.fused_qkv(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), outs[0].arg(), outs[1].arg(), outs[2].arg(),
-                K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout,
-                scales=[s.arg() for s in dev_s])
-    for o, w, name in zip(outs, want, "qkv"):
-        got = o.download()
-        assert np.all(np.isfinite(got)), name
-        assert _close(got, w, K), (name, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
+    try:
+        for min_m in _paths(m):
+            f.set_gemm_min_m(min_m)
+            for o in outs:
+                o.upload(np.zeros(o.shape, np.float16))
+            f.fused_qkv(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), outs[0].arg(), outs[1].arg(), outs[2].arg(),
+                        K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout,
+                        scales=[s.arg() for s in dev_s])
+            for o, w, name in zip(outs, want, "qkv"):
+                got = o.download()
+                assert np.all(np.isfinite(got)), (name, min_m)
+                assert _close(got, w, K), (name, min_m, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
+    finally:
+        f.set_gemm_min_m()
     for b in dev_w + dev_s + [dx, dg] + db + outs:
         b.free()
 
@@ -266,6 +282,8 @@ def test_fused_qkv_q8_equals_oracle(K, N, NK, m, norm, bias, layout):
     (1, 3072, 3072, True, False, True, 1.0, 1.0),   # o_proj
     (1, 256, 256, True, True, False, 0.5, 0.0),
     (7, 896, 896, True, True, True, 1.0, 0.5),
+    (40, 896, 896, False, True, True, 0.25, 0.75),   # the split-K GEMM, and passes of 16 rows
+    (256, 3072, 3072, True, False, True, 1.0, 1.0),  # o_proj of a 256-token prefill chunk
 ])
 def test_matmul_q8_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta):
     announce("matmul q8", m, n, k, canonical, bias, resid, alpha, beta)
@@ -278,10 +296,16 @@ def test_matmul_q8_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta):
     want = orc.matmul_gemv_q8(x, w8, sc, b if bias else None, c if resid else None, 0, 32, alpha, beta)
     dx, dw, ds = f.array(x), f.array(orc.to_canonical(w8) if canonical else w8.reshape(-1)), f.array(sc)
     db, dc, out = f.array(b), f.array(c), f.zeros((m, n))
-    f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, bias=db.arg() if bias else None, c=dc.arg() if resid else None,
-             transpose_b=not canonical, alpha=alpha, beta=beta, b_scales=ds.arg())
-    g, wv = out.download().astype(np.float64), want.astype(np.float64)
-    assert np.all(np.abs(g - wv) <= 2 * np.maximum(np.abs(wv), 2.0 ** -10) * 2.0 ** -10 + 1e-4), float(np.max(np.abs(g - wv)))
+    try:
+        for min_m in _paths(m):
+            f.set_gemm_min_m(min_m)
+            out.upload(np.zeros((m, n), np.float16))
+            f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, bias=db.arg() if bias else None, c=dc.arg() if resid else None,
+                     transpose_b=not canonical, alpha=alpha, beta=beta, b_scales=ds.arg())
+            g, wv = out.download().astype(np.float64), want.astype(np.float64)
+            assert np.all(np.abs(g - wv) <= 2 * np.maximum(np.abs(wv), 2.0 ** -10) * 2.0 ** -10 + 1e-4), (min_m, float(np.max(np.abs(g - wv))))
+    finally:
+        f.set_gemm_min_m()
     with pytest.raises(fa.FoundryError) as e:  # Q8_0 weights without their scales
         f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, transpose_b=not canonical)
     assert e.value.variant == "InputNotFound"
