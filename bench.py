@@ -426,8 +426,8 @@ def bench_fused_qkv(f, args, q8=False):
     f.profile_enable(False)
 
 
-def bench_fused_qkv_chunk(f, args, m):
-    """FusedQkv on a prefill chunk of m tokens at Llama-3.2-3B shape (F16 canonical weights, with RMSNorm): the tiled GEMM
+def bench_fused_qkv_chunk(f, args, m, q8=False):
+    """FusedQkv on a prefill chunk of m tokens at Llama-3.2-3B shape (F16 or Q8_0 canonical weights, with RMSNorm): the tiled GEMM
     (norm kernel in front; split-K and a finish kernel when the chunk is short). m = 32 is the reference's default chunk
     - still a weight stream, priced against HBM; m = 2048 is the C4 prompt in one piece, priced against the matrix cores."""
     import orc
@@ -438,20 +438,28 @@ def bench_fused_qkv_chunk(f, args, m):
     layers, host0 = [], None
     for i in range(NL):
         ws = [rng.uniform(-0.1, 0.1, (n, K)).astype(np.float16) for n in (N, NK, NK)]
-        layers.append([f.array(fa.canonical_layout(w)) for w in ws])
+        if q8:
+            ws = [orc.quantize_q8_0(w) for w in ws]
+            layers.append(([f.array(fa.canonical_layout(w)) for w, _ in ws], [f.array(sc) for _, sc in ws]))
+        else:
+            layers.append(([f.array(fa.canonical_layout(w)) for w in ws], None))
         if i == 0:
             host0 = ws
     dx, dg = f.array(x), f.array(g)
     oq, ok, ov = f.zeros((m, N)), f.zeros((m, NK)), f.zeros((m, NK))
 
     def step(i):
-        w = layers[i % NL]
-        f.fused_qkv(dx.arg(), w[0].arg(), w[1].arg(), w[2].arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, m, gamma=dg.arg())
+        w, sc = layers[i % NL]
+        f.fused_qkv(dx.arg(), w[0].arg(), w[1].arg(), w[2].arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, m, gamma=dg.arg(),
+                    scales=[t.arg() for t in sc] if sc else None)
 
     step(0)
     f.synchronize()
     rows = min(m, 64)  # the oracle on the first rows (seconds of CPU time at most)
-    want = orc.fused_qkv(x[:rows], *host0, gamma=g)
+    if q8:
+        want = orc.fused_qkv_q8(x[:rows], [w for w, _ in host0], [sc for _, sc in host0], gamma=g)
+    else:
+        want = orc.fused_qkv(x[:rows], *host0, gamma=g)
     err = max(float(np.max(np.abs(o.download()[:rows].astype(np.float64) - w.astype(np.float64)))) for o, w in zip((oq, ok, ov), want))
     for i in range(args.warmup):
         step(i)
@@ -468,7 +476,8 @@ def bench_fused_qkv_chunk(f, args, m):
     us = {k: (ms * 1e3 / n if n else 0.0) for k, (n, ms) in kernels.items()}
     total_s = sum(us.values()) * 1e-6
     flops = 2.0 * m * (N + 2 * NK) * K
-    nbytes = 2.0 * (N + 2 * NK) * K + 2.0 * m * K + 2.0 * K + 2.0 * m * (N + 2 * NK)
+    wbytes = (1.0 + 2.0 / 32) if q8 else 2.0  # per weight: int8 + an f16 scale per 32, or f16
+    nbytes = wbytes * (N + 2 * NK) * K + 2.0 * m * K + 2.0 * K + 2.0 * m * (N + 2 * NK)
     if m <= 128:
         roof = {"bound": "hbm", "achieved": nbytes / total_s / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": nbytes / total_s / 1e9 / HBM_PEAK_GBPS, "bytes_per_step": nbytes}
@@ -482,7 +491,8 @@ def bench_fused_qkv_chunk(f, args, m):
         "unit": "chunk-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "llama3.2-3b FusedQkv on a chunk of %d tokens: RMSNorm + Q/K/V projections, k_dim 3072, n_dim "
-                               "3072, n_kv 1024, F16 canonical weights, eager launches (profiling events on)" % m},
+                               "3072, n_kv 1024, %s canonical weights, eager launches (profiling events on)"
+                               % (m, "Q8_0" if q8 else "F16")},
         "roofline": roof, "parity": {"qkv_max_abs_err_first_rows": err, "rows_checked": rows}}))
 
 
@@ -777,6 +787,8 @@ SECONDARY = {"llama3b_attn_block": bench_attn_block, "llama3b_decode_128k": benc
              "llama3b_o_proj": bench_o_proj,
              "llama3b_fused_qkv_chunk32": lambda f, args: bench_fused_qkv_chunk(f, args, 32),
              "llama3b_fused_qkv_prefill_2k": lambda f, args: bench_fused_qkv_chunk(f, args, 2048),
+             "llama3b_fused_qkv_q8_chunk32": lambda f, args: bench_fused_qkv_chunk(f, args, 32, q8=True),
+             "llama3b_fused_qkv_q8_prefill_2k": lambda f, args: bench_fused_qkv_chunk(f, args, 2048, q8=True),
              "llama3b_fused_qkv_q8": lambda f, args: bench_fused_qkv(f, args, q8=True),
              "llama3b_o_proj_q8": lambda f, args: bench_o_proj(f, args, q8=True)}
 
