@@ -651,6 +651,68 @@ def bench_attn_block(f, args):
         "parity": {"outputs_finite": finite, "note": "stage-by-stage parity of this chain: tests/test_gpu_block.py"}}))
 
 
+def bench_prefill_block(f, args):
+    """The attention block of one Llama-3.2-3B layer on a 2048-token prompt in one chunk (models/llama.json:509-585):
+    FusedQkv (norm kernel + GEMM) -> KvPrepFused (RoPE + append of 2048 rows) -> FlashAttention (causal prefill) -> o_proj
+    MatMul with residual (GEMM); F16 canonical weights, contiguous cache, eager launches, 4 layers' buffers in rotation."""
+    L, H, Hkv, D, M = 4, 24, 8, 128, 2048
+    dm, kvd, cap = H * D, Hkv * D, 2048
+    rng = np.random.default_rng(0xF0DD + 12)
+    cos, sin = fa.rope_tables(5e5, D, cap)
+    dcos, dsin = f.array(cos), f.array(sin)
+    wq = fa.canonical_layout(rng.uniform(-0.05, 0.05, (dm, dm)).astype(np.float16))
+    wk = fa.canonical_layout(rng.uniform(-0.05, 0.05, (kvd, dm)).astype(np.float16))
+    layers = []
+    for i in range(L):
+        layers.append(dict(kc=f.zeros((Hkv, cap, D)), vc=f.zeros((Hkv, cap, D)), wq=f.array(np.roll(wq, i)),
+                           wk=f.array(np.roll(wk, i)), wv=f.array(np.roll(wk, i + 5)), wo=f.array(np.roll(wq, i + 9)),
+                           g=f.array(rng.uniform(0.5, 1.5, dm).astype(np.float16))))
+    hid = f.array(rng.uniform(-1, 1, (M, dm)).astype(np.float16))
+    dq, dk, dv = f.zeros((M, dm)), f.zeros((M, kvd)), f.zeros((M, kvd))
+    dqr, dattn, dout = f.zeros((H, M, D)), f.zeros((M, dm)), f.zeros((M, dm))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, M, 0, cap, fa.ROPE_NORMAL)
+
+    def step(i):
+        ly = layers[i % L]
+        f.fused_qkv(hid.arg(), ly["wq"].arg(), ly["wk"].arg(), ly["wv"].arg(), dq.arg(), dk.arg(), dv.arg(), dm, dm, kvd, M,
+                    gamma=ly["g"].arg())
+        f.kv_prep_fused(dq.arg(), dk.arg(), dv.arg(), dqr.arg(), ly["kc"].arg(), ly["vc"].arg(), dcos.arg(), dsin.arg(), p)
+        f.flash_attention(dqr.arg(), ly["kc"].arg(), ly["vc"].arg(), dattn.arg(), True, 0, H, D, M, M)
+        f.matmul(dattn.arg(), ly["wo"].arg(), dout.arg(), M, dm, dm, c=hid.arg(), transpose_b=False, alpha=1.0, beta=1.0)
+
+    for i in range(max(args.warmup, 1)):
+        step(i)
+    f.synchronize()
+    f.profile_reset()
+    f.profile_enable(True)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    names = ("rmsnorm_rows_kernel", "fused_qkv_gemm_kernel", "kv_prep_fused", "flash_prefill_dma_kernel",
+             "flash_prefill_mfma_kernel", "matmul_gemm_kernel")
+    us = {}
+    for k in names:
+        n, ms = f.profile_query(k)
+        if n:
+            us[k] = ms * 1e3 / n
+    f.profile_enable(False)
+    finite = bool(np.all(np.isfinite(dout.download())))
+    flops = 2.0 * M * (dm + 2 * kvd) * dm + 4.0 * D * H * M * (M + 1) / 2 + 2.0 * M * dm * dm
+    total_s = sum(us.values()) * 1e-6
+    print(json.dumps({
+        "metric": "attention-block layer-steps/s, Llama-3.2-3B prefill of 2048 tokens", "value": args.steps / dt,
+        "unit": "layer-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "llama3.2-3b attention block on a 2048-token prompt, one layer per step: FusedQkv, KvPrepFused, "
+                               "causal FlashAttention, o_proj with residual; eager launches (profiling events on)"},
+        "roofline": {"bound": "mfma", "achieved": flops / total_s / 1e12, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flops / total_s / 1e12 / MFMA_F16_PEAK_TFLOPS, "traffic": None, "kernel": "sum of the block's kernels",
+                     "avg_launch_us": us, "flops_per_step": flops},
+        "parity": {"outputs_finite": finite, "note": "stage-by-stage parity of this chain: tests/test_gpu_block.py"}}))
+
+
 def bench_paged_decode(f, args):
     """Qwen2.5-3B-shaped batched paged decode, one layer per step: 32 ragged sequences, 16-token blocks."""
     import orc
@@ -781,7 +843,7 @@ def bench_sage_decode(f, args):
     f.profile_enable(False)
 
 
-SECONDARY = {"llama3b_attn_block": bench_attn_block, "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
+SECONDARY = {"llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
              "llama3b_o_proj": bench_o_proj,

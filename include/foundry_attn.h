@@ -425,6 +425,12 @@ fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b,
  * Environment: FOUNDRY_ATTN_GEMM_MIN_M (read at fa_ctx_create). */
 fa_status fa_set_gemm_min_m(fa_ctx *ctx, uint32_t min_m);
 
+/* Which of the two GEMM kernels fa_fused_qkv / fa_matmul use (same tiling and arithmetic, bit-equal results): 1 = operand
+ * tiles staged through registers (any shape, F16 and Q8_0 weights); 2 or 0 (default) = tiles loaded from memory straight
+ * into LDS where the shape allows it (F16 weights, k_dim a multiple of 64, operands below 2 GiB), else as 1. No
+ * counterpart in the reference (a tuning switch like fa_set_prefill_variant). Environment: FOUNDRY_ATTN_GEMM_VARIANT. */
+fa_status fa_set_gemm_variant(fa_ctx *ctx, uint32_t variant);
+
 /* ---------------------------------------------------------------------------------------------
  * SageAttention-style int8 Q/K decode (docs/SAGE.md:51-65,117-126; docs/FLASH.md:153-170 - prose only in
  * the reference). K is mean-smoothed over the sequence per (kv head, channel), then quantised per block

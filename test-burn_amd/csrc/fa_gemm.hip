@@ -88,6 +88,90 @@ __global__ void __launch_bounds__(256) rmsnorm_rows_kernel(const __half *x, cons
     }
 }
 
+// The end of an output tile, shared by the GEMM kernels: accumulators -> LDS (f32, [input row][weight row]) -> either
+// the write stage and token-major f16 stores, or (split-K) the f32 partial tile.
+template <bool Q8>
+__device__ __forceinline__ void gemm_epilogue(const GemmDev &a, unsigned char *smem, const f16v_t (&acc)[2][2], int tid,
+                                              int lane, int wn, int wm, int mat, uint32_t N, uint32_t n0, uint32_t m0,
+                                              uint32_t split) {
+    // Accumulators -> LDS as f32 [input row][weight row]. Register r of lane l of a 32 x 32 tile is row
+    // 8 (r / 4) + 4 (l / 32) + r % 4 of the first operand and row l % 32 of the second: with the weights first, four
+    // consecutive weight rows per 16-byte write; with the input first (Q8), one float per register.
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                if constexpr (Q8) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t mrow = wm * 64 + j * 32 + g * 8 + (lane >> 5) * 4 + e;
+                        const uint32_t nrow = wn * 64 + i * 32 + (lane & 31);
+                        *reinterpret_cast<float *>(smem + mrow * GM_T_STRIDE + nrow * 4) = acc[i][j][g * 4 + e];
+                    }
+                } else {
+                    const uint32_t nrow = wn * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
+                    const uint32_t mrow = wm * 64 + j * 32 + (lane & 31);
+                    const f4v_t q = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+                    *reinterpret_cast<f4v_t *>(smem + mrow * GM_T_STRIDE + nrow * 4) = q;
+                }
+            }
+    __syncthreads();
+
+    if (a.k_splits > 1) {  // partial sums only; the write stage runs in gemm_finish_kernel
+        const uint32_t col0 = (mat >= 1 ? a.rows[0] : 0u) + (mat == 2 ? a.rows[1] : 0u) + n0;
+        for (uint32_t q = tid; q < GM_TM * GM_TN / 4; q += GM_NT) {
+            const uint32_t mrow = q / (GM_TN / 4), n4 = q % (GM_TN / 4);
+            const uint32_t gm = m0 + mrow, gn = n0 + n4 * 4;
+            if (gm >= a.m || gn >= N) continue;
+            const f4v_t s = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n4 * 16);
+            float *dst = a.partial + ((size_t)split * a.m + gm) * a.n_total + col0 + n4 * 4;
+            if (a.vec_store) {
+                *reinterpret_cast<f4v_t *>(dst) = s;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (gn + e < N) dst[e] = s[e];
+            }
+        }
+        return;
+    }
+    const __half *bias = mat == 0 ? a.bias[0] : mat == 1 ? a.bias[1] : a.bias[2];
+    __half *out = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
+    for (uint32_t q = tid; q < GM_TM * GM_TN / 8; q += GM_NT) {
+        const uint32_t mrow = q / (GM_TN / 8), n8 = q % (GM_TN / 8);
+        const uint32_t gm = m0 + mrow, gn = n0 + n8 * 8;
+        if (gm >= a.m || gn >= N) continue;
+        const f4v_t s0 = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n8 * 32);
+        const f4v_t s1 = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n8 * 32 + 16);
+        const size_t o = (size_t)gm * N + gn;
+        if (a.vec_store) {  // N % 8 == 0 and 16-byte aligned tensors: whole pieces
+            const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+            const h8_t bv = bias ? *reinterpret_cast<const h8_t *>(bias + gn) : z;
+            const h8_t rv = a.residual ? *reinterpret_cast<const h8_t *>(a.residual + o) : z;
+            h8_t y;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float t = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
+                if (bias) t += (float)bv[e];
+                if (a.residual) t += a.beta * (float)rv[e];
+                y[e] = (_Float16)t;
+            }
+            *reinterpret_cast<h8_t *>(out + o) = y;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if (gn + e >= N) break;
+                float t = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
+                if (bias) t += __half2float(bias[gn + e]);
+                if (a.residual) t += a.beta * __half2float(a.residual[o + e]);
+                out[o + e] = __float2half(t);
+            }
+        }
+    }
+}
+
 typedef unsigned int u4v_t __attribute__((ext_vector_type(4)));
 typedef _Float16 h2v_t __attribute__((ext_vector_type(2)));
 
@@ -313,82 +397,170 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
         __syncthreads();
     }
 
-    // Accumulators -> LDS as f32 [input row][weight row]. Register r of lane l of a 32 x 32 tile is row
-    // 8 (r / 4) + 4 (l / 32) + r % 4 of the first operand and row l % 32 of the second: with the weights first, four
-    // consecutive weight rows per 16-byte write; with the input first (Q8), one float per register.
+    gemm_epilogue<Q8>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// The same GEMM with the operand tiles going from memory straight into LDS (buffer_load ... lds), F16 weights, k_dim a
+// multiple of 64: no staging registers, no LDS write instructions, no wait for the loads before a write - the next
+// step's tiles are requested before this step's matrix work and waited for after it. The 64 lanes of such a load fill
+// 1 KiB of consecutive LDS bytes in lane order, so padding is impossible; instead each 1 KiB holds a whole number of
+// rows and a lane fetches, within its row, the 16-byte piece that belongs into its slot:
+//   input and row-major weights: 1 KiB = 8 rows x 8 pieces, slot = piece ^ (row % 8)
+//   canonical weights:           1 KiB = 16 rows x 4 pieces of a 32-feature block, slot = piece ^ ((row / 2) % 4)
+// so that the 8 lanes that read one piece column of 8 consecutive rows fall into 8 different 16-byte bank groups,
+// while the lanes of a request still cover whole 64- or 128-byte runs of memory. Rows past the end of a matrix (or of
+// the input) are out of the buffer descriptor's range and arrive as zeros.
+typedef unsigned int rsrc_words __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ rsrc_words gemm_rsrc(const void *base, uint32_t bytes) {
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    rsrc_words r;
+    r.x = (uint32_t)b, r.y = (uint32_t)(b >> 32) & 0xffffu, r.z = bytes, r.w = 0x00020000u;
+    return r;
+}
+// Four 1 KiB requests into consecutive KiB of LDS. Written as assembly: the compiler cannot tell which LDS bytes such
+// a load writes and would serialise every later LDS read behind it; completion is tracked by vmcnt, waited for by hand.
+__device__ __forceinline__ void lds_dma_4x(rsrc_words rs, uint32_t lds_addr, int v0, int v1, int v2, int v3, int soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                 "buffer_load_dwordx4 %2, %1, %6 offen lds\n\t"
+                 "s_add_i32 m0, %0, 0x400\n\ts_nop 0\n\t"
+                 "buffer_load_dwordx4 %3, %1, %6 offen lds\n\t"
+                 "s_add_i32 m0, %0, 0x800\n\ts_nop 0\n\t"
+                 "buffer_load_dwordx4 %4, %1, %6 offen lds\n\t"
+                 "s_add_i32 m0, %0, 0xc00\n\ts_nop 0\n\t"
+                 "buffer_load_dwordx4 %5, %1, %6 offen lds"
+                 :
+                 : "s"(lds_addr), "s"(rs), "v"(v0), "v"(v1), "v"(v2), "v"(v3), "s"(soff)
+                 : "memory", "scc");
+}
+// ... with one lane offset and sources 1 KiB apart as well (canonical weights): the immediate offset moves both sides
+__device__ __forceinline__ void lds_dma_4x_contiguous(rsrc_words rs, uint32_t lds_addr, int voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                 "buffer_load_dwordx4 %2, %1, 0 offen lds\n\t"
+                 "buffer_load_dwordx4 %2, %1, 0 offen offset:1024 lds\n\t"
+                 "buffer_load_dwordx4 %2, %1, 0 offen offset:2048 lds\n\t"
+                 "buffer_load_dwordx4 %2, %1, 0 offen offset:3072 lds"
+                 :
+                 : "s"(lds_addr), "s"(rs), "v"(voff)
+                 : "memory");
+}
+
+constexpr int GD_OPERAND_BYTES = GM_TN * GM_BK * 2;  // 16 KiB, no padding
+constexpr int GD_STAGE_BYTES = 2 * GD_OPERAND_BYTES;
+
+template <bool CANON>
+__global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_dma_kernel(GemmDev a) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr)smem;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t K = a.k_dim;
+
+    const uint32_t total = a.n_tiles * a.m_tiles * a.k_splits;
+    uint32_t v = blockIdx.x;
+    if (total % 8 == 0) v = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+    const uint32_t split = v % a.k_splits;
+    v /= a.k_splits;
+    uint32_t nt = v / a.m_tiles;
+    const uint32_t mt = v - nt * a.m_tiles;
+    int mat = 0;
+    if (nt >= a.tiles[0]) {
+        nt -= a.tiles[0], mat = 1;
+        if (nt >= a.tiles[1]) nt -= a.tiles[1], mat = 2;
+    }
+    const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
+    const unsigned char *W = reinterpret_cast<const unsigned char *>(mat == 0 ? a.w[0] : mat == 1 ? a.w[1] : a.w[2]);
+    const uint32_t n0 = nt * GM_TN, m0 = mt * GM_TM;
+
+    // Requests of this wave: KiB 4 wave .. 4 wave + 3 of each operand tile.
+    // Input (and row-major weights): KiB c = rows 8c .. 8c + 7; lane l = (row l / 8, slot l % 8), piece = slot ^ row % 8.
+    const uint32_t xr_lane = lane >> 3, x_piece = (lane & 7) ^ (xr_lane & 7);
+    int xv[4], wv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t row = (wave * 4 + i) * 8 + xr_lane;
+        xv[i] = (int)(row * K * 2 + x_piece * 16);  // rows past the input's end are past the descriptor's range
+        wv[i] = xv[i];
+    }
+    const rsrc_words x_rs = gemm_rsrc(reinterpret_cast<const unsigned char *>(a.x) + (size_t)m0 * K * 2,
+                                      (uint32_t)min((uint64_t)(a.m - m0) * K * 2, (uint64_t)0x7fffffffu));
+    // Canonical weights: KiB c of a step = 32-feature block c / 8, rows 16 (c % 8) .. + 15; lane l = (row l / 4, slot
+    // l % 4), piece = slot ^ (row / 2) % 4; the descriptor covers one block's N rows of 64 bytes and is moved per step.
+    const uint32_t cw_row = lane >> 2, cw_piece = (lane & 3) ^ ((cw_row >> 1) & 3);
+    const int cw_voff = (int)((n0 + (wave & 1) * 64 + cw_row) * 64 + cw_piece * 16);
+    const rsrc_words w_rs = CANON ? gemm_rsrc(W, 0)
+                                  : gemm_rsrc(W + (size_t)n0 * K * 2, (uint32_t)min((uint64_t)(N - n0) * K * 2, (uint64_t)0x7fffffffu));
+    auto request = [&](uint32_t ks) {
+        const uint32_t stage = lds_base + (ks & 1) * GD_STAGE_BYTES;
+        if constexpr (CANON) {
+            const rsrc_words rs = gemm_rsrc(W + (size_t)(2 * ks + (wave >> 1)) * N * 64, N * 64);
+            lds_dma_4x_contiguous(rs, stage + wave * 4096, cw_voff);
+        } else {
+            lds_dma_4x(w_rs, stage + wave * 4096, wv[0], wv[1], wv[2], wv[3], (int)(ks * GM_BK * 2));
+        }
+        lds_dma_4x(x_rs, stage + GD_OPERAND_BYTES + wave * 4096, xv[0], xv[1], xv[2], xv[3], (int)(ks * GM_BK * 2));
+    };
+    (void)w_rs;
+
+    // Operand reads. Wave (wn, wm) owns weight rows 64 wn .. +63 and input rows 64 wm .. +63; lane l reads row l % 32
+    // (+ 32 per tile) and the 16-feature half l / 32 of each 32 features.
+    const int wn = wave & 1, wm = wave >> 1;
+    const uint32_t h = lane >> 5, r32 = lane & 31;
+    // input layout (also row-major weights): row r at KiB r / 8, 128 bytes per row, slot = piece ^ r % 8
+    auto rowmajor_base = [&](uint32_t row) { return (row >> 3) * 1024 + (row & 7) * 128; };
+    uint32_t x_slot[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) x_slot[kk] = ((2 * kk + h) ^ (r32 & 7)) * 16;
+    const uint32_t b_base = rowmajor_base(wm * 64 + r32);  // + 4096 per tile of 32 rows
+    // canonical layout: row r of block b at KiB 8 b + r / 16, 64 bytes per row, slot = piece ^ (r / 2) % 4
+    uint32_t a_base, a_slot[4];
+    if constexpr (CANON) {
+        const uint32_t row = wn * 64 + r32;
+        a_base = (row >> 4) * 1024 + (row & 15) * 64;  // + 2048 per tile of 32 rows
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) a_slot[kk] = (kk >> 1) * 8192 + (((2 * (kk & 1) + h) ^ ((row >> 1) & 3)) * 16);
+    } else {
+        a_base = rowmajor_base(wn * 64 + r32);
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) a_slot[kk] = x_slot[kk];
+    }
+    constexpr uint32_t A_TILE = CANON ? 2048 : 4096;
+
+    f16v_t acc[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                if constexpr (Q8) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t mrow = wm * 64 + j * 32 + g * 8 + (lane >> 5) * 4 + e;
-                        const uint32_t nrow = wn * 64 + i * 32 + (lane & 31);
-                        *reinterpret_cast<float *>(smem + mrow * GM_T_STRIDE + nrow * 4) = acc[i][j][g * 4 + e];
-                    }
-                } else {
-                    const uint32_t nrow = wn * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
-                    const uint32_t mrow = wm * 64 + j * 32 + (lane & 31);
-                    const f4v_t q = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-                    *reinterpret_cast<f4v_t *>(smem + mrow * GM_T_STRIDE + nrow * 4) = q;
-                }
-            }
-    __syncthreads();
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-    if (a.k_splits > 1) {  // partial sums only; the write stage runs in gemm_finish_kernel
-        const uint32_t col0 = (mat >= 1 ? a.rows[0] : 0u) + (mat == 2 ? a.rows[1] : 0u) + n0;
-        for (uint32_t q = tid; q < GM_TM * GM_TN / 4; q += GM_NT) {
-            const uint32_t mrow = q / (GM_TN / 4), n4 = q % (GM_TN / 4);
-            const uint32_t gm = m0 + mrow, gn = n0 + n4 * 4;
-            if (gm >= a.m || gn >= N) continue;
-            const f4v_t s = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n4 * 16);
-            float *dst = a.partial + ((size_t)split * a.m + gm) * a.n_total + col0 + n4 * 4;
-            if (a.vec_store) {
-                *reinterpret_cast<f4v_t *>(dst) = s;
-            } else {
+    const uint32_t all_steps = K / GM_BK;
+    const uint32_t ks_begin = split * a.steps_per_split;
+    const uint32_t n_steps = min(all_steps, ks_begin + a.steps_per_split);
+    request(ks_begin);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (uint32_t ks = ks_begin; ks < n_steps; ++ks) {
+        if (ks + 1 < n_steps) request(ks + 1);  // into the stage every wave finished reading before the last barrier
+        const unsigned char *wa = smem + (ks & 1) * GD_STAGE_BYTES;
+        const unsigned char *xa = wa + GD_OPERAND_BYTES;
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (gn + e < N) dst[e] = s[e];
+        for (int kk = 0; kk < GM_BK / 16; ++kk) {
+            h8_t fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fa[i] = *reinterpret_cast<const h8_t *>(wa + a_base + i * A_TILE + a_slot[kk]);
+                fb[i] = *reinterpret_cast<const h8_t *>(xa + b_base + i * 4096 + x_slot[kk]);
             }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
         }
-        return;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
     }
-    const __half *bias = mat == 0 ? a.bias[0] : mat == 1 ? a.bias[1] : a.bias[2];
-    __half *out = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
-    for (uint32_t q = tid; q < GM_TM * GM_TN / 8; q += GM_NT) {
-        const uint32_t mrow = q / (GM_TN / 8), n8 = q % (GM_TN / 8);
-        const uint32_t gm = m0 + mrow, gn = n0 + n8 * 8;
-        if (gm >= a.m || gn >= N) continue;
-        const f4v_t s0 = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n8 * 32);
-        const f4v_t s1 = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n8 * 32 + 16);
-        const size_t o = (size_t)gm * N + gn;
-        if (a.vec_store) {  // N % 8 == 0 and 16-byte aligned tensors: whole pieces
-            const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-            const h8_t bv = bias ? *reinterpret_cast<const h8_t *>(bias + gn) : z;
-            const h8_t rv = a.residual ? *reinterpret_cast<const h8_t *>(a.residual + o) : z;
-            h8_t y;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float t = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
-                if (bias) t += (float)bv[e];
-                if (a.residual) t += a.beta * (float)rv[e];
-                y[e] = (_Float16)t;
-            }
-            *reinterpret_cast<h8_t *>(out + o) = y;
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                if (gn + e >= N) break;
-                float t = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
-                if (bias) t += __half2float(bias[gn + e]);
-                if (a.residual) t += a.beta * __half2float(a.residual[o + e]);
-                out[o + e] = __float2half(t);
-            }
-        }
-    }
+    gemm_epilogue<false>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
 }
 
 // Adds the split-K partial tiles in split order and applies the write stage: one thread per 8 output columns.
@@ -508,7 +680,20 @@ fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
     }
     FaLaunchScope scope(ctx, l.n_kv ? "fused_qkv_gemm_kernel" : "matmul_gemm_kernel", true);
     const uint32_t grid = (uint32_t)n_wg * a.k_splits;
-    if (q8) {
+    // F16 weights, whole steps of 64 features, operands below 2 GiB (32-bit buffer offsets): tiles straight into LDS
+    const uint64_t max_rows = a.rows[0] > a.rows[1] ? a.rows[0] : a.rows[1];
+    const bool dma_ok = !q8 && l.k_dim % GM_BK == 0 && (uint64_t)l.m * l.k_dim * 2 < 0x7fffffffull &&
+                        max_rows * l.k_dim * 2 < 0x7fffffffull;
+    if (dma_ok && ctx->gemm_variant != 1) {
+        static bool dma_lds_allowed = false;
+        if (!dma_lds_allowed) {
+            FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_dma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+            FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_dma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+            dma_lds_allowed = true;
+        }
+        if (l.canonical) scope.launch(qkv_gemm_dma_kernel<true>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+        else scope.launch(qkv_gemm_dma_kernel<false>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+    } else if (q8) {
         if (l.canonical) scope.launch(qkv_gemm_kernel<true, true>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
         else scope.launch(qkv_gemm_kernel<false, true>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
     } else {

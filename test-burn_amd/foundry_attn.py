@@ -116,6 +116,7 @@ PROTOTYPES = {
     "fa_set_prefill_split_k": [_vp, C.c_uint32],
     "fa_set_prefill_variant": [_vp, C.c_uint32],
     "fa_set_gemm_min_m": [_vp, C.c_uint32],
+    "fa_set_gemm_variant": [_vp, C.c_uint32],
     "fa_kv_prep_fused_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _u32, _PT, _PT,
                                C.POINTER(KvPrepFusedParams)],
     "fa_kv_prep_decode_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _PT, _PT, C.POINTER(KvPrepFusedParams)],
@@ -288,6 +289,10 @@ class Foundry:
         """No arguments: the library's defaults (partition size by the launch rule, separate merge kernel)."""
         v = DecodeVariant(keys_per_split, merge)
         check(self.lib.fa_set_decode_variant(self.h, C.byref(v)))
+
+    def set_gemm_variant(self, variant=0):
+        """1 = GEMM operand tiles through registers, 0 / 2 = straight into LDS where the shape allows."""
+        check(self.lib.fa_set_gemm_variant(self.h, variant))
 
     def set_gemm_min_m(self, min_m=0):
         """Input rows from which FusedQkv / MatMul run as a GEMM; 0 = the library's default."""

@@ -22,9 +22,16 @@ def _data(rng, K, N, NK, m):
 
 
 def _paths(m):
-    """Values of the GEMM threshold to run a shape with: the library's default, plus - for a few input rows - the
-    GEMM forced, and - for short chunks - the passes of 16 rows over the weight stream forced."""
-    return [0] if m == 1 else [0, 1] if m < 12 else [0, 1 << 30] if m <= 64 else [0]
+    """(GEMM threshold, GEMM variant) pairs to run a shape with: the library's defaults, plus - for a few input rows -
+    the GEMM forced, - for short chunks - the passes of 16 rows over the weight stream forced, and - wherever the GEMM
+    runs - its second kernel (operand tiles through registers instead of straight into LDS)."""
+    if m == 1:
+        return [(0, 0)]
+    if m < 12:
+        return [(0, 0), (1, 0), (1, 1)]
+    if m <= 64:
+        return [(0, 0), (0, 1), (1 << 30, 0)]
+    return [(0, 0), (0, 1)]
 
 
 def _close(got, want, K):
@@ -71,18 +78,20 @@ def test_fused_qkv_equals_oracle(K, N, NK, m, norm, bias, layout):
     # from 12 input rows on the library runs the GEMM; short chunks are also forced through the passes of 16 rows over
     # the weight stream, and shapes of a few rows through the GEMM
     try:
-        for min_m in _paths(m):
+        for min_m, variant in _paths(m):
             f.set_gemm_min_m(min_m)
+            f.set_gemm_variant(variant)
             for o in outs:
                 o.upload(np.zeros(o.shape, np.float16))
             f.fused_qkv(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), outs[0].arg(), outs[1].arg(), outs[2].arg(),
                         K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout)
             for o, w, name in zip(outs, want, "qkv"):
                 got = o.download()
-                assert np.all(np.isfinite(got)), (name, min_m)
-                assert _close(got, w, K), (name, min_m, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
+                assert np.all(np.isfinite(got)), (name, min_m, variant)
+                assert _close(got, w, K), (name, min_m, variant, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
     finally:
         f.set_gemm_min_m()
+        f.set_gemm_variant()
     for b in dev_w + [dx, dg] + db + outs:
         b.free()
 
@@ -191,18 +200,20 @@ def test_matmul_gemv_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta)
     dx, dw = f.array(x), f.array(orc.to_canonical(w) if canonical else w.reshape(-1))
     db, dc, out = f.array(b), f.array(c), f.zeros((m, n))
     try:
-        for min_m in _paths(m):  # the GEMM and the passes over the weight stream, as in the FusedQkv test
+        for min_m, variant in _paths(m):  # the GEMM kernels and the passes over the weight stream, as in the FusedQkv test
             f.set_gemm_min_m(min_m)
+            f.set_gemm_variant(variant)
             out.upload(np.zeros((m, n), np.float16))
             f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, bias=db.arg() if bias else None, c=dc.arg() if resid else None,
                      transpose_b=not canonical, alpha=alpha, beta=beta)
             got = out.download()
             # the reference's own bar is 1e-3 * sqrt(k) (tests/gemv_v2_parity.rs:214); here: 2 f16 ulps of the expected value
             g, wv = got.astype(np.float64), want.astype(np.float64)
-            assert np.all(np.abs(g - wv) <= 2 * np.maximum(np.abs(wv), 2.0 ** -10) * 2.0 ** -10 + 1e-4), (min_m, float(np.max(np.abs(g - wv))))
+            assert np.all(np.abs(g - wv) <= 2 * np.maximum(np.abs(wv), 2.0 ** -10) * 2.0 ** -10 + 1e-4), (min_m, variant, float(np.max(np.abs(g - wv))))
             assert float(np.max(np.abs(g - wv))) <= 1e-3 * np.sqrt(k)
     finally:
         f.set_gemm_min_m()
+        f.set_gemm_variant()
     for z in (dx, dw, db, dc, out):
         z.free()
 
@@ -260,8 +271,9 @@ def test_fused_qkv_q8_equals_oracle(K, N, NK, m, norm, bias, layout):
     db = [f.array(b) for b in bs]
     outs = [f.zeros((m, n)) for n in (N, NK, NK)]
     try:
-        for min_m in _paths(m):
+        for min_m, variant in _paths(m):
             f.set_gemm_min_m(min_m)
+            f.set_gemm_variant(variant)
             for o in outs:
                 o.upload(np.zeros(o.shape, np.float16))
             f.fused_qkv(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), outs[0].arg(), outs[1].arg(), outs[2].arg(),
@@ -269,10 +281,11 @@ def test_fused_qkv_q8_equals_oracle(K, N, NK, m, norm, bias, layout):
                         scales=[s.arg() for s in dev_s])
             for o, w, name in zip(outs, want, "qkv"):
                 got = o.download()
-                assert np.all(np.isfinite(got)), (name, min_m)
-                assert _close(got, w, K), (name, min_m, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
+                assert np.all(np.isfinite(got)), (name, min_m, variant)
+                assert _close(got, w, K), (name, min_m, variant, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
     finally:
         f.set_gemm_min_m()
+        f.set_gemm_variant()
     for b in dev_w + dev_s + [dx, dg] + db + outs:
         b.free()
 
@@ -297,15 +310,17 @@ def test_matmul_q8_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta):
     dx, dw, ds = f.array(x), f.array(orc.to_canonical(w8) if canonical else w8.reshape(-1)), f.array(sc)
     db, dc, out = f.array(b), f.array(c), f.zeros((m, n))
     try:
-        for min_m in _paths(m):
+        for min_m, variant in _paths(m):
             f.set_gemm_min_m(min_m)
+            f.set_gemm_variant(variant)
             out.upload(np.zeros((m, n), np.float16))
             f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, bias=db.arg() if bias else None, c=dc.arg() if resid else None,
                      transpose_b=not canonical, alpha=alpha, beta=beta, b_scales=ds.arg())
             g, wv = out.download().astype(np.float64), want.astype(np.float64)
-            assert np.all(np.abs(g - wv) <= 2 * np.maximum(np.abs(wv), 2.0 ** -10) * 2.0 ** -10 + 1e-4), (min_m, float(np.max(np.abs(g - wv))))
+            assert np.all(np.abs(g - wv) <= 2 * np.maximum(np.abs(wv), 2.0 ** -10) * 2.0 ** -10 + 1e-4), (min_m, variant, float(np.max(np.abs(g - wv))))
     finally:
         f.set_gemm_min_m()
+        f.set_gemm_variant()
     with pytest.raises(fa.FoundryError) as e:  # Q8_0 weights without their scales
         f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, transpose_b=not canonical)
     assert e.value.variant == "InputNotFound"
