@@ -406,10 +406,11 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
 // step's tiles are requested before this step's matrix work and waited for after it. The 64 lanes of such a load fill
 // 1 KiB of consecutive LDS bytes in lane order, so padding is impossible; instead each 1 KiB holds a whole number of
 // rows and a lane fetches, within its row, the 16-byte piece that belongs into its slot:
-//   input and row-major weights: 1 KiB = 8 rows x 8 pieces, slot = piece ^ (row % 8)
-//   canonical weights:           1 KiB = 16 rows x 4 pieces of a 32-feature block, slot = piece ^ ((row / 2) % 4)
-// so that the 8 lanes that read one piece column of 8 consecutive rows fall into 8 different 16-byte bank groups,
-// while the lanes of a request still cover whole 64- or 128-byte runs of memory. Rows past the end of a matrix (or of
+//   input and row-major weights: 1 KiB = 8 rows x 8 pieces, slot = piece ^ ((row / 2) % 8)
+//   canonical weights:           1 KiB = 16 rows x 4 pieces of a 32-feature block, slot = piece ^ ((row / 4) % 4)
+// so that the 16 lanes that read one piece column of 16 consecutive rows fall into 16 different 16-byte bank groups
+// of the 256 bytes an LDS read serves per cycle (with row % 8 and (row / 2) % 4, distinct within 8 lanes only, a third
+// of the LDS cycles were bank conflicts), while the lanes of a request still cover whole 64- or 128-byte runs of memory. Rows past the end of a matrix (or of
 // the input) are out of the buffer descriptor's range and arrive as zeros.
 typedef unsigned int rsrc_words __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ rsrc_words gemm_rsrc(const void *base, uint32_t bytes) {
@@ -473,20 +474,21 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_dma_kernel(GemmDev a) {
     const uint32_t n0 = nt * GM_TN, m0 = mt * GM_TM;
 
     // Requests of this wave: KiB 4 wave .. 4 wave + 3 of each operand tile.
-    // Input (and row-major weights): KiB c = rows 8c .. 8c + 7; lane l = (row l / 8, slot l % 8), piece = slot ^ row % 8.
-    const uint32_t xr_lane = lane >> 3, x_piece = (lane & 7) ^ (xr_lane & 7);
+    // Input (and row-major weights): KiB c = rows 8c .. 8c + 7; lane l = (row l / 8, slot l % 8), piece = slot ^ (row / 2) % 8.
+    const uint32_t xr_lane = lane >> 3;
     int xv[4], wv[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const uint32_t row = (wave * 4 + i) * 8 + xr_lane;
+        const uint32_t x_piece = (lane & 7) ^ ((row >> 1) & 7);
         xv[i] = (int)(row * K * 2 + x_piece * 16);  // rows past the input's end are past the descriptor's range
         wv[i] = xv[i];
     }
     const rsrc_words x_rs = gemm_rsrc(reinterpret_cast<const unsigned char *>(a.x) + (size_t)m0 * K * 2,
                                       (uint32_t)min((uint64_t)(a.m - m0) * K * 2, (uint64_t)0x7fffffffu));
     // Canonical weights: KiB c of a step = 32-feature block c / 8, rows 16 (c % 8) .. + 15; lane l = (row l / 4, slot
-    // l % 4), piece = slot ^ (row / 2) % 4; the descriptor covers one block's N rows of 64 bytes and is moved per step.
-    const uint32_t cw_row = lane >> 2, cw_piece = (lane & 3) ^ ((cw_row >> 1) & 3);
+    // l % 4), piece = slot ^ (row / 4) % 4; the descriptor covers one block's N rows of 64 bytes and is moved per step.
+    const uint32_t cw_row = lane >> 2, cw_piece = (lane & 3) ^ ((cw_row >> 2) & 3);
     const int cw_voff = (int)((n0 + (wave & 1) * 64 + cw_row) * 64 + cw_piece * 16);
     const rsrc_words w_rs = CANON ? gemm_rsrc(W, 0)
                                   : gemm_rsrc(W + (size_t)n0 * K * 2, (uint32_t)min((uint64_t)(N - n0) * K * 2, (uint64_t)0x7fffffffu));
@@ -506,19 +508,19 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_dma_kernel(GemmDev a) {
     // (+ 32 per tile) and the 16-feature half l / 32 of each 32 features.
     const int wn = wave & 1, wm = wave >> 1;
     const uint32_t h = lane >> 5, r32 = lane & 31;
-    // input layout (also row-major weights): row r at KiB r / 8, 128 bytes per row, slot = piece ^ r % 8
+    // input layout (also row-major weights): row r at KiB r / 8, 128 bytes per row, slot = piece ^ (r / 2) % 8
     auto rowmajor_base = [&](uint32_t row) { return (row >> 3) * 1024 + (row & 7) * 128; };
     uint32_t x_slot[4];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) x_slot[kk] = ((2 * kk + h) ^ (r32 & 7)) * 16;
+    for (int kk = 0; kk < 4; ++kk) x_slot[kk] = ((2 * kk + h) ^ ((r32 >> 1) & 7)) * 16;
     const uint32_t b_base = rowmajor_base(wm * 64 + r32);  // + 4096 per tile of 32 rows
-    // canonical layout: row r of block b at KiB 8 b + r / 16, 64 bytes per row, slot = piece ^ (r / 2) % 4
+    // canonical layout: row r of block b at KiB 8 b + r / 16, 64 bytes per row, slot = piece ^ (r / 4) % 4
     uint32_t a_base, a_slot[4];
     if constexpr (CANON) {
         const uint32_t row = wn * 64 + r32;
         a_base = (row >> 4) * 1024 + (row & 15) * 64;  // + 2048 per tile of 32 rows
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) a_slot[kk] = (kk >> 1) * 8192 + (((2 * (kk & 1) + h) ^ ((row >> 1) & 3)) * 16);
+        for (int kk = 0; kk < 4; ++kk) a_slot[kk] = (kk >> 1) * 8192 + (((2 * (kk & 1) + h) ^ ((row >> 2) & 3)) * 16);
     } else {
         a_base = rowmajor_base(wn * 64 + r32);
 #pragma unroll
