@@ -425,10 +425,13 @@ fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b,
  * Environment: FOUNDRY_ATTN_GEMM_MIN_M (read at fa_ctx_create). */
 fa_status fa_set_gemm_min_m(fa_ctx *ctx, uint32_t min_m);
 
-/* Which of the two GEMM kernels fa_fused_qkv / fa_matmul use (same tiling and arithmetic, bit-equal results): 1 = operand
- * tiles staged through registers (any shape, F16 and Q8_0 weights); 2 or 0 (default) = tiles loaded from memory straight
- * into LDS where the shape allows it (F16 weights, k_dim a multiple of 64, operands below 2 GiB), else as 1. No
- * counterpart in the reference (a tuning switch like fa_set_prefill_variant). Environment: FOUNDRY_ATTN_GEMM_VARIANT. */
+/* Which GEMM kernel fa_fused_qkv / fa_matmul use (same tiling and arithmetic; results equal up to the f32 summation
+ * order of the split-K partials, which does not depend on the kernel): 1 = operand tiles staged through registers (any
+ * shape, F16 and Q8_0 weights); 2 = tiles loaded from memory straight into LDS in steps of 64 features, two workgroups
+ * per compute unit; 3 = the same in steps of 32 features, four workgroups per compute unit; 0 (default) = 2 or 3 by
+ * the number of output tiles. 2 and 3 need F16 weights, k_dim a multiple of 64 and operands below 2 GiB, and fall back
+ * to 1 otherwise. No counterpart in the reference (a tuning switch like fa_set_prefill_variant).
+ * Environment: FOUNDRY_ATTN_GEMM_VARIANT. */
 fa_status fa_set_gemm_variant(fa_ctx *ctx, uint32_t variant);
 
 /* ---------------------------------------------------------------------------------------------

@@ -106,7 +106,7 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     if (ctx->decode_waves != 4 && ctx->decode_waves != 8) ctx->decode_waves = 0;
     ctx->gemm_min_m = env_u32("FOUNDRY_ATTN_GEMM_MIN_M", 0);
     ctx->gemm_variant = env_u32("FOUNDRY_ATTN_GEMM_VARIANT", 0);
-    if (ctx->gemm_variant > 2) ctx->gemm_variant = 0;
+    if (ctx->gemm_variant > 3) ctx->gemm_variant = 0;
     ctx->prefill_split_k = env_u32("FOUNDRY_ATTN_PREFILL_SPLIT_K", 0);
     ctx->prefill_variant = env_u32("FOUNDRY_ATTN_PREFILL_VARIANT", 0);
     if (ctx->prefill_variant > 2) ctx->prefill_variant = 0;
@@ -192,7 +192,7 @@ extern "C" fa_status fa_set_prefill_split_k(fa_ctx *ctx, uint32_t split_k) {
 
 extern "C" fa_status fa_set_gemm_variant(fa_ctx *ctx, uint32_t variant) {
     FA_NEED(ctx, "ctx");
-    if (variant > 2) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "GEMM variant must be 0, 1 or 2, got %u", variant);
+    if (variant > 3) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "GEMM variant must be 0 ... 3, got %u", variant);
     ctx->gemm_variant = variant;
     return FA_OK;
 }

@@ -89,84 +89,95 @@ __global__ void __launch_bounds__(256) rmsnorm_rows_kernel(const __half *x, cons
 }
 
 // The end of an output tile, shared by the GEMM kernels: accumulators -> LDS (f32, [input row][weight row]) -> either
-// the write stage and token-major f16 stores, or (split-K) the f32 partial tile.
-template <bool Q8>
+// the write stage and token-major f16 stores, or (split-K) the f32 partial tile. HALVES: the tile goes through LDS in
+// two halves of 64 input rows (tile j of every wave), for kernels that keep their LDS footprint at half a tile.
+template <bool Q8, bool HALVES>
 __device__ __forceinline__ void gemm_epilogue(const GemmDev &a, unsigned char *smem, const f16v_t (&acc)[2][2], int tid,
                                               int lane, int wn, int wm, int mat, uint32_t N, uint32_t n0, uint32_t m0,
                                               uint32_t split) {
-    // Accumulators -> LDS as f32 [input row][weight row]. Register r of lane l of a 32 x 32 tile is row
-    // 8 (r / 4) + 4 (l / 32) + r % 4 of the first operand and row l % 32 of the second: with the weights first, four
-    // consecutive weight rows per 16-byte write; with the input first (Q8), one float per register.
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                if constexpr (Q8) {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t mrow = wm * 64 + j * 32 + g * 8 + (lane >> 5) * 4 + e;
-                        const uint32_t nrow = wn * 64 + i * 32 + (lane & 31);
-                        *reinterpret_cast<float *>(smem + mrow * GM_T_STRIDE + nrow * 4) = acc[i][j][g * 4 + e];
-                    }
-                } else {
-                    const uint32_t nrow = wn * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
-                    const uint32_t mrow = wm * 64 + j * 32 + (lane & 31);
-                    const f4v_t q = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-                    *reinterpret_cast<f4v_t *>(smem + mrow * GM_T_STRIDE + nrow * 4) = q;
-                }
-            }
-    __syncthreads();
-
-    if (a.k_splits > 1) {  // partial sums only; the write stage runs in gemm_finish_kernel
-        const uint32_t col0 = (mat >= 1 ? a.rows[0] : 0u) + (mat == 2 ? a.rows[1] : 0u) + n0;
-        for (uint32_t q = tid; q < GM_TM * GM_TN / 4; q += GM_NT) {
-            const uint32_t mrow = q / (GM_TN / 4), n4 = q % (GM_TN / 4);
-            const uint32_t gm = m0 + mrow, gn = n0 + n4 * 4;
-            if (gm >= a.m || gn >= N) continue;
-            const f4v_t s = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n4 * 16);
-            float *dst = a.partial + ((size_t)split * a.m + gm) * a.n_total + col0 + n4 * 4;
-            if (a.vec_store) {
-                *reinterpret_cast<f4v_t *>(dst) = s;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (gn + e < N) dst[e] = s[e];
-            }
-        }
-        return;
-    }
+    constexpr int NH = HALVES ? 2 : 1;
+    constexpr uint32_t T_ROWS = HALVES ? GM_TM / 2 : GM_TM;
     const __half *bias = mat == 0 ? a.bias[0] : mat == 1 ? a.bias[1] : a.bias[2];
     __half *out = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
-    for (uint32_t q = tid; q < GM_TM * GM_TN / 8; q += GM_NT) {
-        const uint32_t mrow = q / (GM_TN / 8), n8 = q % (GM_TN / 8);
-        const uint32_t gm = m0 + mrow, gn = n0 + n8 * 8;
-        if (gm >= a.m || gn >= N) continue;
-        const f4v_t s0 = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n8 * 32);
-        const f4v_t s1 = *reinterpret_cast<const f4v_t *>(smem + mrow * GM_T_STRIDE + n8 * 32 + 16);
-        const size_t o = (size_t)gm * N + gn;
-        if (a.vec_store) {  // N % 8 == 0 and 16-byte aligned tensors: whole pieces
-            const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-            const h8_t bv = bias ? *reinterpret_cast<const h8_t *>(bias + gn) : z;
-            const h8_t rv = a.residual ? *reinterpret_cast<const h8_t *>(a.residual + o) : z;
-            h8_t y;
+    const uint32_t col0 = (mat >= 1 ? a.rows[0] : 0u) + (mat == 2 ? a.rows[1] : 0u) + n0;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                float t = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
-                if (bias) t += (float)bv[e];
-                if (a.residual) t += a.beta * (float)rv[e];
-                y[e] = (_Float16)t;
+    for (int half = 0; half < NH; ++half) {
+        if (half) __syncthreads();  // the first half has been read out
+        // Accumulators -> LDS as f32 [input row][weight row]. Register r of lane l of a 32 x 32 tile is row
+        // 8 (r / 4) + 4 (l / 32) + r % 4 of the first operand and row l % 32 of the second: with the weights first, four
+        // consecutive weight rows per 16-byte write; with the input first (Q8), one float per register.
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (HALVES && j != half) continue;
+                const uint32_t t0 = HALVES ? wm * 32 : wm * 64 + j * 32;  // LDS row of the tile's first input row
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    if constexpr (Q8) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t trow = t0 + g * 8 + (lane >> 5) * 4 + e;
+                            const uint32_t nrow = wn * 64 + i * 32 + (lane & 31);
+                            *reinterpret_cast<float *>(smem + trow * GM_T_STRIDE + nrow * 4) = acc[i][j][g * 4 + e];
+                        }
+                    } else {
+                        const uint32_t nrow = wn * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
+                        const uint32_t trow = t0 + (lane & 31);
+                        const f4v_t q = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+                        *reinterpret_cast<f4v_t *>(smem + trow * GM_T_STRIDE + nrow * 4) = q;
+                    }
+                }
             }
-            *reinterpret_cast<h8_t *>(out + o) = y;
-        } else {
+        __syncthreads();
+        auto tile_row = [&](uint32_t t) { return HALVES ? (t >> 5) * 64 + half * 32 + (t & 31) : t; };
+
+        if (a.k_splits > 1) {  // partial sums only; the write stage runs in gemm_finish_kernel
+            for (uint32_t q = tid; q < T_ROWS * GM_TN / 4; q += GM_NT) {
+                const uint32_t t = q / (GM_TN / 4), n4 = q % (GM_TN / 4);
+                const uint32_t gm = m0 + tile_row(t), gn = n0 + n4 * 4;
+                if (gm >= a.m || gn >= N) continue;
+                const f4v_t s = *reinterpret_cast<const f4v_t *>(smem + t * GM_T_STRIDE + n4 * 16);
+                float *dst = a.partial + ((size_t)split * a.m + gm) * a.n_total + col0 + n4 * 4;
+                if (a.vec_store) {
+                    *reinterpret_cast<f4v_t *>(dst) = s;
+                } else {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                if (gn + e >= N) break;
-                float t = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
-                if (bias) t += __half2float(bias[gn + e]);
-                if (a.residual) t += a.beta * __half2float(a.residual[o + e]);
-                out[o + e] = __float2half(t);
+                    for (int e = 0; e < 4; ++e)
+                        if (gn + e < N) dst[e] = s[e];
+                }
+            }
+            continue;
+        }
+        for (uint32_t q = tid; q < T_ROWS * GM_TN / 8; q += GM_NT) {
+            const uint32_t t = q / (GM_TN / 8), n8 = q % (GM_TN / 8);
+            const uint32_t gm = m0 + tile_row(t), gn = n0 + n8 * 8;
+            if (gm >= a.m || gn >= N) continue;
+            const f4v_t s0 = *reinterpret_cast<const f4v_t *>(smem + t * GM_T_STRIDE + n8 * 32);
+            const f4v_t s1 = *reinterpret_cast<const f4v_t *>(smem + t * GM_T_STRIDE + n8 * 32 + 16);
+            const size_t o = (size_t)gm * N + gn;
+            if (a.vec_store) {  // N % 8 == 0 and 16-byte aligned tensors: whole pieces
+                const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+                const h8_t bv = bias ? *reinterpret_cast<const h8_t *>(bias + gn) : z;
+                const h8_t rv = a.residual ? *reinterpret_cast<const h8_t *>(a.residual + o) : z;
+                h8_t y;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float v = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
+                    if (bias) v += (float)bv[e];
+                    if (a.residual) v += a.beta * (float)rv[e];
+                    y[e] = (_Float16)v;
+                }
+                *reinterpret_cast<h8_t *>(out + o) = y;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (gn + e >= N) break;
+                    float v = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
+                    if (bias) v += __half2float(bias[gn + e]);
+                    if (a.residual) v += a.beta * __half2float(a.residual[o + e]);
+                    out[o + e] = __float2half(v);
+                }
             }
         }
     }
@@ -397,7 +408,7 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
         __syncthreads();
     }
 
-    gemm_epilogue<Q8>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
+    gemm_epilogue<Q8, false>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -562,7 +573,130 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_dma_kernel(GemmDev a) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
-    gemm_epilogue<false>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
+    gemm_epilogue<false, false>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
+}
+
+// The LDS-direct GEMM in steps of 32 features, two stages, with the output tile leaving through LDS in two halves: a
+// workgroup then needs 33 KiB of LDS instead of 66 and four of them share a CU instead of two. Per tile this is the
+// slower kernel (twice the barriers per feature), but when the launch has more workgroups than two per CU and at most
+// four, all of them are resident at once instead of a second, partly filled round (Llama-3.2-3B Q/K/V on 2048 rows,
+// 640 tiles: 80.4 us against 95.2; 1024 rows, 320 tiles: 56.8 against 50.8; 4096 rows, 1280 tiles: 169.7 against
+// 157.8). A ring of three or four such stages (requests two or three steps ahead, three or two workgroups per CU) was
+// measured as well and is never the fastest: the latency of the requests is not what limits these kernels.
+// Both operands use the layout 1 KiB = 16 rows x 4 pieces (64 bytes of a row), slot = piece ^ ((row / 4) % 4).
+__device__ __forceinline__ void lds_dma_2x(rsrc_words rs, uint32_t lds_addr, int v0, int v1, int soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                 "buffer_load_dwordx4 %2, %1, %4 offen lds\n\t"
+                 "s_add_i32 m0, %0, 0x400\n\ts_nop 0\n\t"
+                 "buffer_load_dwordx4 %3, %1, %4 offen lds"
+                 :
+                 : "s"(lds_addr), "s"(rs), "v"(v0), "v"(v1), "s"(soff)
+                 : "memory", "scc");
+}
+__device__ __forceinline__ void lds_dma_2x_contiguous(rsrc_words rs, uint32_t lds_addr, int voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                 "buffer_load_dwordx4 %2, %1, 0 offen lds\n\t"
+                 "buffer_load_dwordx4 %2, %1, 0 offen offset:1024 lds"
+                 :
+                 : "s"(lds_addr), "s"(rs), "v"(voff)
+                 : "memory");
+}
+constexpr int GR_BK = 32;
+constexpr int GR_OPERAND_BYTES = GM_TN * GR_BK * 2;  // 8 KiB
+constexpr int GR_STAGE_BYTES = 2 * GR_OPERAND_BYTES;
+constexpr int GR_T_BYTES = (GM_TM / 2) * GM_T_STRIDE;
+constexpr int GR_LDS_BYTES = 2 * GR_STAGE_BYTES > GR_T_BYTES ? 2 * GR_STAGE_BYTES : GR_T_BYTES;
+
+template <bool CANON>
+__global__ void __launch_bounds__(GM_NT, 4) qkv_gemm_dma32_kernel(GemmDev a) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr)smem;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t K = a.k_dim;
+
+    const uint32_t total = a.n_tiles * a.m_tiles * a.k_splits;
+    uint32_t v = blockIdx.x;
+    if (total % 8 == 0) v = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+    const uint32_t split = v % a.k_splits;
+    v /= a.k_splits;
+    uint32_t nt = v / a.m_tiles;
+    const uint32_t mt = v - nt * a.m_tiles;
+    int mat = 0;
+    if (nt >= a.tiles[0]) {
+        nt -= a.tiles[0], mat = 1;
+        if (nt >= a.tiles[1]) nt -= a.tiles[1], mat = 2;
+    }
+    const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
+    const unsigned char *W = reinterpret_cast<const unsigned char *>(mat == 0 ? a.w[0] : mat == 1 ? a.w[1] : a.w[2]);
+    const uint32_t n0 = nt * GM_TN, m0 = mt * GM_TM;
+
+    // Requests of this wave: KiB 2 wave and 2 wave + 1 of each operand tile = rows 32 wave .. + 31; lane l = (row l / 4,
+    // slot l % 4) of its KiB, piece = slot ^ (row / 4) % 4.
+    const uint32_t r16 = lane >> 2, piece = (lane & 3) ^ ((r16 >> 2) & 3);
+    const uint32_t row0 = wave * 32 + r16;
+    const int xv0 = (int)(row0 * K * 2 + piece * 16), xv1 = (int)((row0 + 16) * K * 2 + piece * 16);
+    const int cw_voff = (int)((n0 + row0) * 64 + piece * 16);
+    const rsrc_words x_rs = gemm_rsrc(reinterpret_cast<const unsigned char *>(a.x) + (size_t)m0 * K * 2,
+                                      (uint32_t)min((uint64_t)(a.m - m0) * K * 2, (uint64_t)0x7fffffffu));
+    const rsrc_words w_rs = CANON ? gemm_rsrc(W, 0)
+                                  : gemm_rsrc(W + (size_t)n0 * K * 2, (uint32_t)min((uint64_t)(N - n0) * K * 2, (uint64_t)0x7fffffffu));
+    auto request = [&](uint32_t ks) {
+        const uint32_t stage = lds_base + (ks & 1) * GR_STAGE_BYTES;
+        if constexpr (CANON) {  // one 32-feature block per step: N rows of 64 bytes
+            const rsrc_words rs = gemm_rsrc(W + (size_t)ks * N * 64, N * 64);
+            lds_dma_2x_contiguous(rs, stage + wave * 2048, cw_voff);
+        } else {
+            lds_dma_2x(w_rs, stage + wave * 2048, xv0, xv1, (int)(ks * GR_BK * 2));
+        }
+        lds_dma_2x(x_rs, stage + GR_OPERAND_BYTES + wave * 2048, xv0, xv1, (int)(ks * GR_BK * 2));
+    };
+    (void)w_rs;
+    (void)cw_voff;
+
+    // Operand reads: lane l reads row l % 32 (+ 32 per tile) of the wave's 64 rows, 16-feature half l / 32 of each 16.
+    const int wn = wave & 1, wm = wave >> 1;
+    const uint32_t h = lane >> 5, r32 = lane & 31;
+    auto row_base = [&](uint32_t row) { return (row >> 4) * 1024 + (row & 15) * 64; };
+    uint32_t slot[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) slot[kk] = ((2 * kk + h) ^ ((r32 >> 2) & 3)) * 16;
+    const uint32_t a_base = row_base(wn * 64 + r32), b_base = row_base(wm * 64 + r32);  // + 2048 per tile of 32 rows
+
+    f16v_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    const uint32_t all_steps = K / GR_BK;
+    const uint32_t ks_begin = split * a.steps_per_split * 2;  // steps_per_split counts steps of 64 features
+    const uint32_t n_steps = min(all_steps, ks_begin + a.steps_per_split * 2);
+    request(ks_begin);
+    for (uint32_t ks = ks_begin; ks < n_steps; ++ks) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's requests for step ks have landed ...
+        __syncthreads();  // ... and everybody's; every wave is also done reading the stage of step ks - 1,
+        if (ks + 1 < n_steps) request(ks + 1);  // which step ks + 1 reuses
+        const unsigned char *wa = smem + (ks & 1) * GR_STAGE_BYTES;
+        const unsigned char *xa = wa + GR_OPERAND_BYTES;
+#pragma unroll
+        for (int kk = 0; kk < GR_BK / 16; ++kk) {
+            h8_t fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fa[i] = *reinterpret_cast<const h8_t *>(wa + a_base + i * 2048 + slot[kk]);
+                fb[i] = *reinterpret_cast<const h8_t *>(xa + b_base + i * 2048 + slot[kk]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+    }
+    __syncthreads();  // the stages are reused by the output tile
+    gemm_epilogue<false, true>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
 }
 
 // Adds the split-K partial tiles in split order and applies the write stage: one thread per 8 output columns.
@@ -686,7 +820,14 @@ fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
     const uint64_t max_rows = a.rows[0] > a.rows[1] ? a.rows[0] : a.rows[1];
     const bool dma_ok = !q8 && l.k_dim % GM_BK == 0 && (uint64_t)l.m * l.k_dim * 2 < 0x7fffffffull &&
                         max_rows * l.k_dim * 2 < 0x7fffffffull;
-    if (dma_ok && ctx->gemm_variant != 1) {
+    // two LDS-direct kernels: steps of 64 features, two workgroups per CU - or steps of 32, four per CU, when that
+    // makes the whole launch resident at once
+    const uint32_t n_cus_l = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
+    const bool small_steps = ctx->gemm_variant == 3 || (ctx->gemm_variant == 0 && grid > 2 * n_cus_l && grid <= 4 * n_cus_l);
+    if (dma_ok && small_steps) {
+        if (l.canonical) scope.launch(qkv_gemm_dma32_kernel<true>, dim3(grid), dim3(GM_NT), GR_LDS_BYTES, a);
+        else scope.launch(qkv_gemm_dma32_kernel<false>, dim3(grid), dim3(GM_NT), GR_LDS_BYTES, a);
+    } else if (dma_ok && ctx->gemm_variant != 1) {
         static bool dma_lds_allowed = false;
         if (!dma_lds_allowed) {
             FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_dma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));

@@ -36,7 +36,7 @@ struct fa_ctx {
     uint32_t n_counters = 0;
     fa_decode_variant decode_variant{0, 1};
     uint32_t decode_waves = 0;     // waves per decode workgroup: 0 = by launch size, 4 or 8
-    uint32_t gemm_variant = 0;     // GEMM operand path: 0 = auto (straight into LDS where eligible), 1 = through registers, 2 = as 0
+    uint32_t gemm_variant = 0;     // GEMM kernel: 0 = auto, 1 = tiles through registers, 2 / 3 = straight into LDS in steps of 64 / 32 features
     uint32_t gemm_min_m = 0;       // FusedQkv / MatMul: input rows from which the GEMM runs (0 = default)
     uint32_t prefill_split_k = 0;  // 0 = auto
     uint32_t prefill_variant = 0;  // 0 = auto, 1 = tiles staged through registers, 2 = tiles straight into LDS, two-phase loop

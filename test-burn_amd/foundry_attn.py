@@ -291,7 +291,7 @@ class Foundry:
         check(self.lib.fa_set_decode_variant(self.h, C.byref(v)))
 
     def set_gemm_variant(self, variant=0):
-        """1 = GEMM operand tiles through registers, 0 / 2 = straight into LDS where the shape allows."""
+        """0 = auto; 1 = GEMM operand tiles through registers; 2 / 3 = straight into LDS in steps of 64 / 32 features."""
         check(self.lib.fa_set_gemm_variant(self.h, variant))
 
     def set_gemm_min_m(self, min_m=0):

@@ -24,14 +24,14 @@ def _data(rng, K, N, NK, m):
 def _paths(m):
     """(GEMM threshold, GEMM variant) pairs to run a shape with: the library's defaults, plus - for a few input rows -
     the GEMM forced, - for short chunks - the passes of 16 rows over the weight stream forced, and - wherever the GEMM
-    runs - its second kernel (operand tiles through registers instead of straight into LDS)."""
+    runs - each of its kernels (operand tiles through registers, straight into LDS in steps of 64 or of 32 features)."""
     if m == 1:
         return [(0, 0)]
     if m < 12:
         return [(0, 0), (1, 0), (1, 1)]
     if m <= 64:
-        return [(0, 0), (0, 1), (1 << 30, 0)]
-    return [(0, 0), (0, 1)]
+        return [(0, 0), (0, 1), (0, 2), (0, 3), (1 << 30, 0)]
+    return [(0, 0), (0, 1), (0, 2), (0, 3)]
 
 
 def _close(got, want, K):
