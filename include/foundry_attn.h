@@ -421,7 +421,9 @@ fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b,
 /* Tuning override for fa_fused_qkv and fa_matmul: the number of input rows m from which the tiled
  * GEMM runs instead of passes of 16 rows over the weight stream (the reference makes the same choice between GemvV2
  * and its GEMM by m, src/metals/matmul.rs:190-239). 0 = the library's default. With a gamma the GEMM writes the
- * normalised input (m * k_dim f16) into the context's workspace (fa_ctx_reserve_workspace before a capture).
+ * normalised input (m * k_dim f16) into the context's workspace, which also holds the f32 partial tiles of short chunks
+ * (k_splits * m * (n_dim + 2 n_kv) floats): inside a capture the workspace cannot grow - call the op once eagerly with
+ * the same shape, or fa_ctx_reserve_workspace, before fa_start_capture.
  * Environment: FOUNDRY_ATTN_GEMM_MIN_M (read at fa_ctx_create). */
 fa_status fa_set_gemm_min_m(fa_ctx *ctx, uint32_t min_m);
 

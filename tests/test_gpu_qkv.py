@@ -379,3 +379,46 @@ def test_gemm_path_replays_in_a_graph_with_new_inputs():
     graph.destroy()
     for b in dev_w + [dwo, dg, dx, dproj] + outs:
         b.free()
+
+
+def test_gemm_workspace_must_be_reserved_before_a_capture():
+    """The GEMM form keeps the normalised input (and split-K partial tiles) in the context's workspace; inside a capture
+    the workspace cannot grow, so a call that needs more than is reserved fails with a message naming
+    fa_ctx_reserve_workspace; after one eager call of the same shape (or that reservation) the capture works."""
+    announce("gemm workspace under capture")
+    f = fa.Foundry()  # a context of its own: the shared one may already hold a large workspace
+    try:
+        K, N, NK, m = 8192, 128, 64, 4608  # normalised input: 75.5 MB, more than a new context's 64 MB
+        rng = np.random.default_rng(5)
+        x = rng.uniform(-1, 1, (m, K)).astype(np.float16)
+        g = rng.uniform(0.5, 1.5, K).astype(np.float16)
+        ws = [rng.uniform(-0.1, 0.1, (n, K)).astype(np.float16) for n in (N, NK, NK)]
+        dev_w = [f.array(orc.to_canonical(w)) for w in ws]
+        dx, dg = f.array(x), f.array(g)
+        outs = [f.zeros((m, n)) for n in (N, NK, NK)]
+
+        def call():
+            f.fused_qkv(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), outs[0].arg(), outs[1].arg(), outs[2].arg(),
+                        K, N, NK, m, gamma=dg.arg(), layout=1)
+
+        f.start_capture()
+        with pytest.raises(fa.FoundryError) as e:
+            call()
+        assert "fa_ctx_reserve_workspace" in str(e.value)
+        f.end_capture().destroy()
+        call()  # eagerly, the call sizes the workspace itself (fa_ctx_reserve_workspace with the byte count does the same)
+        f.synchronize()
+        for o in outs:
+            o.upload(np.zeros(o.shape, np.float16))
+        f.start_capture()
+        call()
+        graph = f.end_capture()
+        graph.launch()
+        f.synchronize()
+        rows = slice(m - 24, m)  # the oracle on the last rows
+        want = orc.fused_qkv(x[rows], *ws, gamma=g, layout=0)
+        for o, w in zip(outs, want):
+            assert _close(o.download()[rows], w, K)
+        graph.destroy()
+    finally:
+        f.close()
