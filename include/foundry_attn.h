@@ -61,7 +61,7 @@ const char *fa_last_error_string(void);
 
 /* Dtype, same order as metallic-sdk's enum (crates/metallic-sdk/src/tensor.rs:7-30). */
 typedef enum fa_dtype {
-    FA_DTYPE_F32 = 0, FA_DTYPE_F16 = 1, FA_DTYPE_BF16 = 2, FA_DTYPE_Q8_0 = 7,
+    FA_DTYPE_F32 = 0, FA_DTYPE_F16 = 1, FA_DTYPE_BF16 = 2, FA_DTYPE_Q4_0 = 3, FA_DTYPE_Q8_0 = 7,
     FA_DTYPE_I8 = 15, FA_DTYPE_I16 = 16, FA_DTYPE_I32 = 17, FA_DTYPE_U8 = 18, FA_DTYPE_U16 = 19,
     FA_DTYPE_U32 = 20, FA_DTYPE_F64 = 21
 } fa_dtype;
@@ -358,7 +358,10 @@ fa_status fa_paged_copy_blocks(fa_ctx *ctx, const fa_paged_kv *cache, const int3
  * models/llama.json:509-528; kernel src/metals/gemv/qkv_project.metal). Weights are F16 (PolicyF16,
  * src/metals/policies/policy_f16.metal:18-70) or Q8_0 (PolicyQ8, src/metals/policies/policy_q8.metal: int8 values in
  * the same element order, dtype FA_DTYPE_Q8_0 or FA_DTYPE_I8, plus a scale tensor s_* of f16 [rows, k_dim / 32],
- * row-major, weight = int8 * scale of its 32-block); the other block-quantised policies are refused with
+ * row-major, weight = int8 * scale of its 32-block) or Q4_0 (PolicyQ4_0, src/metals/policies/policy_q4_0.metal: two
+ * weights per byte in the same element order - element 2i in the low nibble of byte i, the loader's adjacent-pair
+ * packing - dtype FA_DTYPE_Q4_0, weight = (nibble - 8) * scale, the same scale tensor; at decode sizes only: more than a
+ * few input rows run as passes of 16 over the weight stream); the other block-quantised policies are refused with
  * FA_ERR_UNSUPPORTED_DTYPE.
  *   out_q[b, r] = f16( sum_k xn[b, k] * W_q[r, k] + bias_q[r] ),  r < n_dim;  out_k, out_v likewise, r < n_kv
  *   xn[b, k]    = f16( x[b, k] * rsqrt(mean_k x[b, k]^2 + epsilon) * gamma[k] )  with gamma, else x[b, k]
@@ -396,14 +399,14 @@ fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_ar
 /* ---------------------------------------------------------------------------------------------
  * MatMul, weight-stream form: the step after the path (o_proj: `attn_out [m, H*D]` x W_o, residual `hidden`,
  * models/llama.json:566-585; op src/metals/matmul.rs:11-239, which runs GemvV2 for m == 1 and for canonical
- * weights; write stage src/metals/gemv/stages.rs:200-224). F16 or Q8_0 weights (b_scales as in fa_fused_qkv).
+ * weights; write stage src/metals/gemv/stages.rs:200-224). F16, Q8_0 or Q4_0 weights (b_scales as in fa_fused_qkv).
  *   output[b, r] = f16( alpha * sum_k a[b, k] * B[r, k] + bias[r] + beta * c[b, r] ),  r < n, b < m
  * transpose_b != 0: B is row-major [n, k] (Layout::RowMajor); transpose_b == 0: B is in the canonical blocked
  * layout (matmul.rs:199-207). transpose_a and activations other than none are not built
  * (FA_ERR_OPERATION_NOT_SUPPORTED). bias, c: NULL or NULL buffer = absent (the reference's "zero" placeholder).
  * Any m is accepted: up to fa_set_gemm_min_m() - 1 input rows run as passes of 16 over the weight stream; from there
- * on the op is a tiled GEMM on the matrix cores (F16 and Q8_0 weights), the counterpart of the reference's GEMM for
- * large m (src/metals/mma).
+ * on the op is a tiled GEMM on the matrix cores (F16 and Q8_0 weights; Q4_0 stays on the passes), the counterpart of
+ * the reference's GEMM for large m (src/metals/mma).
  * ------------------------------------------------------------------------------------------- */
 typedef struct fa_matmul_params {
     uint32_t m, n, k;            /* k a multiple of 32 */

@@ -691,6 +691,17 @@ static float q8_row_dot(const orc_f16 *x, const int8_t *w8, const orc_f16 *scale
     return acc;
 }
 
+/* Q4_0 weights as the policy reads them (src/metals/policies/policy_q4_0.metal:70-98): element e of the buffer's element
+ * order sits in byte e / 2, low nibble for even e, high nibble for odd e, and its value is nibble - 8. (The loader turns
+ * GGML's "weight j low, weight j + 16 high" bytes into these adjacent pairs, tests/gemm_v2_parity.rs:141-196.) The dot
+ * product is then the block recurrence of Q8 with these integers (policy_q4_0.metal:45-66: scale * sum of 8 products). */
+void orc_unpack_q4_0(const uint8_t *packed, size_t n_elems, int8_t *out) {
+    for (size_t e = 0; e < n_elems; ++e) {
+        const uint8_t b = packed[e / 2];
+        out[e] = (int8_t)((int)((e & 1) ? (b >> 4) : (b & 0x0F)) - 8);
+    }
+}
+
 void orc_matmul_gemv_q8(const orc_f16 *x, const int8_t *w8, const orc_f16 *scales, const orc_f16 *bias,
                         const orc_f16 *residual, orc_f16 *out, uint32_t m, uint32_t n, uint32_t k_dim, int layout,
                         uint32_t wpb, float alpha, float beta, int n_threads) {

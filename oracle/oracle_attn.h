@@ -191,6 +191,8 @@ void orc_matmul_gemv(const orc_f16 *x, const orc_f16 *w, const orc_f16 *bias, co
 /* Q8_0 weights (src/metals/policies/policy_q8.metal): int8 values w8 in `layout`, f16 scales [n, ceil(k_dim / wpb)]
  * row-major. Per row: acc += (sum over a chunk of 8 consecutive k of w8*x) * scale(block of the chunk), k ascending
  * (tests/gemv_v2_parity.rs:82-125); then alpha, bias, beta*residual, one rounding, as orc_matmul_gemv. */
+/* Q4_0 nibbles -> integers -8..7 in the buffer's element order (policy_q4_0.metal:70-98); feed them to the Q8 functions. */
+void orc_unpack_q4_0(const uint8_t *packed, size_t n_elems, int8_t *out);
 void orc_matmul_gemv_q8(const orc_f16 *x, const int8_t *w8, const orc_f16 *scales, const orc_f16 *bias,
                         const orc_f16 *residual, orc_f16 *out, uint32_t m, uint32_t n, uint32_t k_dim, int layout,
                         uint32_t wpb, float alpha, float beta, int n_threads);

@@ -751,23 +751,26 @@ static const __half *half_ptr(const fa_tensor_arg *t) {
 }
 
 // Weight dtype of a projection: F16, or Q8_0 (int8 values + f16 block scales [rows, k / 32]).
-static fa_status weight_kind(const fa_tensor_arg *w, const fa_tensor_arg *scales, const char *what, size_t rows, size_t k, bool &q8) {
+// Weight policy of a FusedQkv / MatMul operand: bits per weight (16 = F16, 8 = Q8_0, 4 = Q4_0), and the checks on the scale
+// tensor the block-quantised ones need.
+static fa_status weight_kind(const fa_tensor_arg *w, const fa_tensor_arg *scales, const char *what, size_t rows, size_t k, int &bits) {
     if (w->dtype == FA_DTYPE_F16) {
-        q8 = false;
+        bits = 16;
         return FA_OK;
     }
-    if (w->dtype == FA_DTYPE_Q8_0 || w->dtype == FA_DTYPE_I8) {
-        q8 = true;
-        if (!present(scales)) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: scales of the Q8_0 weights %s", what);
+    if (w->dtype == FA_DTYPE_Q8_0 || w->dtype == FA_DTYPE_I8 || w->dtype == FA_DTYPE_Q4_0) {
+        bits = w->dtype == FA_DTYPE_Q4_0 ? 4 : 8;
+        const char *policy = bits == 4 ? "Q4_0" : "Q8_0";
+        if (!present(scales)) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: scales of the %s weights %s", policy, what);
         const size_t need = rows * (k / 32);
         const size_t have = scales->dtype == FA_DTYPE_F16 ? numel(scales) : numel(scales) / 2;  // f16, or the scale bytes
         if (scales->dtype != FA_DTYPE_F16 && scales->dtype != FA_DTYPE_U8 && scales->dtype != FA_DTYPE_I8)
-            return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "%s: Q8_0 scales must be f16 values (F16, or their bytes as U8)", what);
+            return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "%s: %s scales must be f16 values (F16, or their bytes as U8)", what, policy);
         if (scales->rank > 0 && have < need) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %s holds %zu scales, %zu needed", what, have, need);
         if ((uintptr_t)half_ptr(scales) % 2 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "%s: scales must be 2-byte aligned", what);
         return FA_OK;
     }
-    return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "%s: weight dtype %u: F16 and Q8_0 weights are built, no other block-quantised policy", what, w->dtype);
+    return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "%s: weight dtype %u: F16, Q8_0 and Q4_0 weights are built, no other block-quantised policy", what, w->dtype);
 }
 
 extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
@@ -783,11 +786,12 @@ extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const f
         FA_NEED(r.t, r.name);
         if (!r.t->buffer) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: %s", r.name);
     }
-    bool q8 = false, q8_k = false, q8_v = false;
-    FA_TRY(weight_kind(w_q, s_q, "w_q", p->n_dim, p->k_dim, q8));
-    FA_TRY(weight_kind(w_k, s_k, "w_k", p->n_kv, p->k_dim, q8_k));
-    FA_TRY(weight_kind(w_v, s_v, "w_v", p->n_kv, p->k_dim, q8_v));
-    if (q8 != q8_k || q8 != q8_v)  // the reference falls back to three separate projections there (qkv_step.rs:243-259)
+    int wbits = 16, wbits_k = 16, wbits_v = 16;
+    FA_TRY(weight_kind(w_q, s_q, "w_q", p->n_dim, p->k_dim, wbits));
+    FA_TRY(weight_kind(w_k, s_k, "w_k", p->n_kv, p->k_dim, wbits_k));
+    FA_TRY(weight_kind(w_v, s_v, "w_v", p->n_kv, p->k_dim, wbits_v));
+    const bool q8 = wbits != 16;  // block-quantised (scales present)
+    if (wbits != wbits_k || wbits != wbits_v)  // the reference falls back to three separate projections there (qkv_step.rs:243-259)
         return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: mixed weight dtypes are not supported");
     for (const fa_tensor_arg *t : {input, out_q, out_k, out_v})
         if (t->dtype != FA_DTYPE_F16) return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: activations must be F16, got dtype %u", t->dtype);
@@ -829,6 +833,7 @@ extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const f
     L.k_dim = p->k_dim, L.n_dim = p->n_dim, L.n_kv = p->n_kv, L.m = m, L.eps = p->epsilon;
     L.canonical = p->layout == FA_WEIGHT_LAYOUT_CANONICAL;
     if (q8) L.scales[0] = half_ptr(s_q), L.scales[1] = half_ptr(s_k), L.scales[2] = half_ptr(s_v);
+    L.weight_bits = wbits;
     for (const void *ptr : {(const void *)L.w[0], (const void *)L.w[1], (const void *)L.w[2], (const void *)L.x, (const void *)L.gamma})
         if (ptr && (uintptr_t)ptr % 16 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: input, gamma and weights must be 16-byte aligned");
     return fa_launch_fused_qkv(ctx, L);
@@ -844,8 +849,9 @@ extern "C" fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_ten
         FA_NEED(r.t, r.name);
         if (!r.t->buffer) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: %s", r.name);
     }
-    bool q8 = false;
-    FA_TRY(weight_kind(b, b_scales, "b", p->n, p->k, q8));
+    int wbits = 16;
+    FA_TRY(weight_kind(b, b_scales, "b", p->n, p->k, wbits));
+    const bool q8 = wbits != 16;
     if (a->dtype != FA_DTYPE_F16 || output->dtype != FA_DTYPE_F16) return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "MatMul: a and output must be F16");
     if (p->transpose_a) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: transpose_a is not supported");
     if (p->activation != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: activation %u is not built", p->activation);
@@ -875,6 +881,7 @@ extern "C" fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_ten
     L.canonical = p->transpose_b == 0;
     L.residual = has_c ? half_ptr(c) : nullptr, L.alpha = p->alpha, L.beta = p->beta;
     if (q8) L.scales[0] = half_ptr(b_scales);
+    L.weight_bits = wbits;
     if ((uintptr_t)L.w[0] % 16 != 0 || (uintptr_t)L.x % 16 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: a and b must be 16-byte aligned");
     return fa_launch_fused_qkv(ctx, L);
 }

@@ -209,6 +209,7 @@ struct FusedQkvLaunch {
     float alpha = 1.0f, beta = 0.0f;
     // Q8_0: w[i] are int8 values in the same layouts, scales[i] f16 [rows, k_dim / 32]; nullptr = F16 weights
     const __half *scales[3] = {nullptr, nullptr, nullptr};
+    int weight_bits = 16;  // 16 = F16, 8 = Q8_0, 4 = Q4_0 (two weights per byte, element 2i in the low nibble of byte i)
 };
 fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l);
 fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l);  // fa_gemm.hip: many input rows

@@ -17,6 +17,7 @@
 // Q8_0 weights (src/metals/policies/policy_q8.metal: int8 values, one f16 scale per 32 weights of a row, separate
 // buffers) take the same route at half the bytes: 8 bytes per lane and block, converted to f16 exactly, one matrix
 // instruction per 32-weight block whose row sums are multiplied by the block's scales (staged in LDS) and added up.
+// Q4_0 weights (policy_q4_0.metal: nibble - 8, adjacent pairs per byte, the same scales) at a quarter: 4 bytes per lane.
 //
 // The same kernel with one matrix, no norm and the write stage's alpha / bias / beta * residual is the m = 1 path of
 // the MatMul op (src/metals/matmul.rs:190-239 -> GemvV2, write stage src/metals/gemv/stages.rs:200-224): the o_proj
@@ -54,8 +55,11 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-template <bool Q8>
+// WB: bits per weight - 16 (f16), 8 (Q8_0) or 4 (Q4_0)
+template <int WB>
 __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
+    constexpr bool Q8 = WB != 16;  // block-quantised: integer weights + one f16 scale per 32 of a row
+    constexpr bool Q4 = WB == 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, c = lane >> 4;
@@ -84,8 +88,8 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     // into place with LDS permutes was slower: 10.6 us against 9.5 on 31.5 MB of weights).
     // Per tile a lane keeps the address of its block 0 and its stride from block to block.
     // (Q8: the same element indices, one byte per element.)
-    typedef typename std::conditional<Q8, u2v_t, h8_t>::type wreg_t;
-    constexpr size_t WES = Q8 ? 1 : 2;  // weight element size in bytes
+    // (Q4: two elements per byte, element 2i in the low nibble of byte i.)
+    typedef typename std::conditional<Q4, uint32_t, typename std::conditional<Q8, u2v_t, h8_t>::type>::type wreg_t;
     auto tile_base = [&](uint32_t tile, const unsigned char *&p0, size_t &kb_stride, bool &ok) {
         const uint32_t gr = row_begin + tile * 16 + n;
         ok = gr < row_end;
@@ -95,8 +99,8 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
         const unsigned char *base = reinterpret_cast<const unsigned char *>(mat == 0 ? a.w[0] : mat == 1 ? a.w[1] : a.w[2]);
         const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
         // canonical (blocked by 32 features): (k % 32) + 32 * (row + (k / 32) * N); row-major: row * K + k
-        p0 = base + (a.canonical ? (size_t)lrow * 32 + c * 8 : (size_t)lrow * K + c * 8) * WES;
-        kb_stride = (a.canonical ? (size_t)N * 32 : 32) * WES;
+        p0 = base + (a.canonical ? (size_t)lrow * 32 + c * 8 : (size_t)lrow * K + c * 8) * WB / 8;
+        kb_stride = (a.canonical ? (size_t)N * 32 : 32) * WB / 8;
     };
 
     // A wave takes the feature blocks kb = wave, wave + 8, ... of every tile, in batches of QKV_UNITS; two batches
@@ -115,7 +119,8 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
         for (int i = 0; i < QKV_UNITS; ++i) {
             const uint32_t kb = (uint32_t)wave + (j0 + i) * QKV_NW;
             wreg_t z;
-            if constexpr (Q8) z = u2v_t{0u, 0u};
+            if constexpr (Q4) z = 0u;
+            else if constexpr (Q8) z = u2v_t{0u, 0u};
             else z = h8_t{0, 0, 0, 0, 0, 0, 0, 0};
             buf[i] = (ok && kb < nkb) ? *reinterpret_cast<const wreg_t *>(p0 + (size_t)kb * kb_stride) : z;
         }
@@ -240,13 +245,24 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
                 // per row (lane (n, c) of the result holds rows 4c..4c+3) and then accumulated
                 // int8 -> f16 without a conversion per element: s + 128 is a byte u, the f16 with bits 0x6400 | u is
                 // 1024 + u, and 1024 + u - 1152 = s exactly (two byte permutes and one packed subtraction per four)
-                const u2v_t raw = buf[i];
+                // Q4_0 (policy_q4_0.metal:70-86: value = nibble - 8): the eight nibbles first become two words of four
+                // bytes 0..15 in element order (two masks, a shift, two byte permutes), then the same route with
+                // 1024 + u - 1032
+                u2v_t raw;
+                if constexpr (Q4) {
+                    const uint32_t even = buf[i] & 0x0f0f0f0fu, odd = (buf[i] >> 4) & 0x0f0f0f0fu;
+                    raw[0] = __builtin_amdgcn_perm(odd, even, 0x05010400u);
+                    raw[1] = __builtin_amdgcn_perm(odd, even, 0x07030602u);
+                } else {
+                    raw = buf[i];
+                }
                 typedef _Float16 h2v_t __attribute__((ext_vector_type(2)));
                 h8_t wv;
 #pragma unroll
                 for (int hw = 0; hw < 2; ++hw) {
-                    const uint32_t u = raw[hw] ^ 0x80808080u;
-                    const h2v_t bias = {(_Float16)1152.0f, (_Float16)1152.0f};
+                    const uint32_t u = Q4 ? raw[hw] : raw[hw] ^ 0x80808080u;
+                    const _Float16 off = Q4 ? (_Float16)1032.0f : (_Float16)1152.0f;
+                    const h2v_t bias = {off, off};
                     const h2v_t lo = __builtin_bit_cast(h2v_t, __builtin_amdgcn_perm(0x64646464u, u, 0x05010400u)) - bias;
                     const h2v_t hi = __builtin_bit_cast(h2v_t, __builtin_amdgcn_perm(0x64646464u, u, 0x07030602u)) - bias;
                     wv[4 * hw + 0] = lo[0], wv[4 * hw + 1] = lo[1], wv[4 * hw + 2] = hi[0], wv[4 * hw + 3] = hi[1];
@@ -286,13 +302,14 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     a.residual = l.residual, a.alpha = l.alpha, a.beta = l.beta;
     for (int i = 0; i < 3; ++i) a.scales[i] = l.scales[i];
     const bool q8 = l.scales[0] != nullptr;
+    const bool q4 = l.weight_bits == 4;
     // More than a few input rows: no longer a weight stream but a GEMM (fa_gemm.hip). Measured on 5120 x 3072 with a
     // gamma, passes of this kernel against the GEMM (norm kernel, split-K GEMM, finish kernel): m = 8: 15.0 / 18.5 us,
     // m = 12 (from where only one workgroup's input rows fit a CU's LDS): 30.3 / 18.2, m = 16: 37.3 / 18.7,
     // m = 32: 76.8 / 19.8.
     constexpr uint32_t GEMM_MIN_M_DEFAULT = 12;
     auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
-    const bool gemm_ok = l.k_dim % (q8 ? 32 : 8) == 0 && aligned16(l.x) && aligned16(l.w[0]) && aligned16(l.w[1]) &&
+    const bool gemm_ok = !q4 && l.k_dim % (q8 ? 32 : 8) == 0 && aligned16(l.x) && aligned16(l.w[0]) && aligned16(l.w[1]) &&
                          aligned16(l.w[2]) && aligned16(l.gamma);
     if (gemm_ok && l.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : GEMM_MIN_M_DEFAULT)) return fa_launch_fused_qkv_gemm(ctx, l);
     const uint32_t total_rows = l.n_dim + 2 * l.n_kv;
@@ -318,9 +335,11 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
                        (q8 ? (size_t)tiles_per_wg * 16 * (l.k_dim / 32) * 2 : 0);
     static bool lds_allowed = false;
     if (!lds_allowed) {
-        FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)(lds_budget + 16 * 1024)));
-        FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)(lds_budget + 16 * 1024)));
+        FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)(lds_budget + 16 * 1024)));
         lds_allowed = true;
     }
@@ -328,7 +347,8 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     if (grid.y > 65535u) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv m %u needs %u passes", l.m, grid.y);
     FaLaunchScope scope(ctx, l.n_kv ? "fused_qkv_kernel" : "matmul_gemv_kernel", true);
     if (lds > lds_budget + 16 * 1024) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: k_dim %u needs %zu bytes of LDS", l.k_dim, lds);
-    if (q8) scope.launch(fused_qkv_kernel<true>, grid, dim3(QKV_NT), lds, a);
-    else scope.launch(fused_qkv_kernel<false>, grid, dim3(QKV_NT), lds, a);
+    if (q4) scope.launch(fused_qkv_kernel<4>, grid, dim3(QKV_NT), lds, a);
+    else if (q8) scope.launch(fused_qkv_kernel<8>, grid, dim3(QKV_NT), lds, a);
+    else scope.launch(fused_qkv_kernel<16>, grid, dim3(QKV_NT), lds, a);
     return scope.finish();
 }

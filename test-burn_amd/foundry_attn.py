@@ -19,6 +19,7 @@ STATUS_NAMES = {
     9: "InputNotFound",
 }
 DTYPE_F32, DTYPE_F16, DTYPE_BF16, DTYPE_I8, DTYPE_I32, DTYPE_U32 = 0, 1, 2, 15, 17, 20
+DTYPE_Q4_0, DTYPE_Q8_0, DTYPE_U8 = 3, 7, 18  # block-quantised weight policies (metallic-sdk's Dtype order), raw bytes
 ROPE_NEOX, ROPE_NORMAL = 0, 1
 
 
@@ -184,7 +185,7 @@ def check(status):
 
 
 _NP_DTYPE = {np.dtype(np.float16): DTYPE_F16, np.dtype(np.float32): DTYPE_F32, np.dtype(np.int8): DTYPE_I8,
-             np.dtype(np.int32): DTYPE_I32, np.dtype(np.uint32): DTYPE_U32}
+             np.dtype(np.int32): DTYPE_I32, np.dtype(np.uint32): DTYPE_U32, np.dtype(np.uint8): DTYPE_U8}
 
 
 class DevBuf:

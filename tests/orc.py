@@ -279,6 +279,33 @@ def quantize_q8_0(w, wpb=32):
     return q.reshape(n, k), scale
 
 
+def quantize_q4_0(w, wpb=32):
+    """Q4_0 of a row-major [n, k] matrix as the reference's test helper makes it (tests/gemm_v2_parity.rs:112-199): per 32
+    weights of a row, scale = max|w| / 7 stored as f16, q = round-half-away(w / scale) clamped to [-8, 7] (with the
+    unrounded scale). Returns (int8 [n, k] with values -8..7, f16 scales [n, k / wpb])."""
+    w = np.asarray(w, np.float16).astype(np.float32)
+    n, k = w.shape
+    blocks = w.reshape(n, k // wpb, wpb)
+    scale = (np.abs(blocks).max(axis=2) / np.float32(7.0)).astype(np.float32)
+    t = np.where(scale[:, :, None] > 0, blocks / np.where(scale == 0, np.float32(1), scale)[:, :, None], 0.0)
+    q = np.clip(np.sign(t) * np.floor(np.abs(t) + 0.5), -8, 7).astype(np.int8)
+    return q.reshape(n, k), scale.astype(np.float16)
+
+
+def pack_q4_0(q_flat):
+    """Integers -8..7 in the buffer's element order -> the policy's bytes: element 2i in the low nibble of byte i."""
+    u = (np.asarray(q_flat, np.int16).reshape(-1) + 8).astype(np.uint8)
+    return (u[0::2] | (u[1::2] << 4)).astype(np.uint8)
+
+
+def unpack_q4_0(packed):
+    """The oracle's reading of Q4_0 bytes (policy_q4_0.metal:70-98): int8 values in element order."""
+    packed = np.ascontiguousarray(packed, dtype=np.uint8).reshape(-1)
+    out = np.zeros(packed.size * 2, np.int8)
+    lib().orc_unpack_q4_0(packed.ctypes.data_as(C.c_void_p), C.c_size_t(out.size), out.ctypes.data_as(C.c_void_p))
+    return out
+
+
 def _i8(a):
     return np.ascontiguousarray(a, dtype=np.int8)
 

@@ -140,7 +140,7 @@ def test_fused_qkv_errors():
         f.fused_qkv(x.arg(), w8.arg(), wk.arg(), wv.arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1,
                     scales=(sc.arg(), fa.TensorArg(), fa.TensorArg()))
     assert e.value.variant == "UnsupportedDtype"
-    wq4 = wq.arg(dtype=3)  # Q4_0: not built
+    wq4 = wq.arg(dtype=4)  # Q4_1: not built
     with pytest.raises(fa.FoundryError) as e:
         f.fused_qkv(x.arg(), wq4, wk.arg(), wv.arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1)
     assert e.value.variant == "UnsupportedDtype"
@@ -236,8 +236,8 @@ def test_matmul_errors():
     with pytest.raises(fa.FoundryError) as e:  # Q8_0 weights without scales
         f.matmul(a.arg(), b8.arg(), o.arg(), 1, 32, 64)
     assert e.value.variant == "InputNotFound"
-    with pytest.raises(fa.FoundryError) as e:  # Q4_0: not built
-        f.matmul(a.arg(), b.arg(dtype=3), o.arg(), 1, 32, 64)
+    with pytest.raises(fa.FoundryError) as e:  # Q4_1: not built
+        f.matmul(a.arg(), b.arg(dtype=4), o.arg(), 1, 32, 64)
     assert e.value.variant == "UnsupportedDtype"
     f.synchronize()
     for z in (a, b, o, b8):
@@ -325,6 +325,69 @@ def test_matmul_q8_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta):
         f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, transpose_b=not canonical)
     assert e.value.variant == "InputNotFound"
     f.synchronize()
+    for z in (dx, dw, ds, db, dc, out):
+        z.free()
+
+
+# ---------------------------------------------------------------- Q4_0 weights
+
+@pytest.mark.parametrize("K,N,NK,m,norm,bias,layout", [
+    (1024, 1024, 128, 1, True, True, 1),
+    (3072, 3072, 1024, 1, True, False, 1),   # Llama-3.2-3B decode
+    (896, 896, 128, 5, True, True, 0),       # row-major bytes
+    (64, 40, 24, 3, True, True, 1),
+    (896, 896, 128, 20, False, True, 1),     # more than a few rows: passes of 16 (no GEMM for this policy)
+])
+def test_fused_qkv_q4_0_equals_oracle(K, N, NK, m, norm, bias, layout):
+    """Q4_0 weights (policy_q4_0.metal): the GPU reads the packed bytes, the oracle the integers its own reader makes of
+    the same bytes, through the Q8 block recurrence."""
+    announce("fused qkv q4_0", K, N, NK, m, norm, bias, layout)
+    f = ctx()
+    rng = np.random.default_rng(K + N + m + 4)
+    x, g, ws, bs = _data(rng, K, N, NK, m)
+    q4 = [orc.quantize_q4_0(w) for w in ws]
+    packed = [orc.pack_q4_0(orc.to_canonical(q) if layout == 1 else q.reshape(-1)) for q, _ in q4]
+    want = orc.fused_qkv_q8(x, [orc.unpack_q4_0(p) for p in packed], [s for _, s in q4], gamma=g if norm else None,
+                            biases=bs if bias else None, layout=layout)
+    dev_w = [f.array(p) for p in packed]
+    dev_s = [f.array(s) for _, s in q4]
+    dx, dg = f.array(x), f.array(g)
+    db = [f.array(b) for b in bs]
+    outs = [f.zeros((m, n)) for n in (N, NK, NK)]
+    wargs = [w.arg(dims=(n, K), dtype=fa.DTYPE_Q4_0) for w, n in zip(dev_w, (N, NK, NK))]
+    f.fused_qkv(dx.arg(), wargs[0], wargs[1], wargs[2], outs[0].arg(), outs[1].arg(), outs[2].arg(),
+                K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout,
+                scales=[s.arg() for s in dev_s])
+    for o, w, name in zip(outs, want, "qkv"):
+        got = o.download()
+        assert np.all(np.isfinite(got)), name
+        assert _close(got, w, K), (name, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
+    for b in dev_w + dev_s + [dx, dg] + db + outs:
+        b.free()
+
+
+@pytest.mark.parametrize("m,n,k,canonical,bias,resid,alpha,beta", [
+    (1, 128, 128, False, False, False, 1.0, 0.0),
+    (1, 3072, 3072, True, False, True, 1.0, 1.0),   # o_proj
+    (7, 896, 896, True, True, True, 0.5, 0.5),
+])
+def test_matmul_q4_0_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta):
+    announce("matmul q4_0", m, n, k, canonical, bias, resid, alpha, beta)
+    f = ctx()
+    rng = np.random.default_rng(m + n + k + 5)
+    x = rng.uniform(-1, 1, (m, k)).astype(np.float16)
+    q, sc = orc.quantize_q4_0(rng.uniform(-0.1, 0.1, (n, k)).astype(np.float16))
+    b = rng.uniform(-0.1, 0.1, n).astype(np.float16)
+    c = rng.uniform(-1, 1, (m, n)).astype(np.float16)
+    packed = orc.pack_q4_0(orc.to_canonical(q) if canonical else q.reshape(-1))
+    want = orc.matmul_gemv_q8(x, orc.unpack_q4_0(packed), sc, b if bias else None, c if resid else None, 1 if canonical else 0,
+                              32, alpha, beta)
+    dx, dw, ds = f.array(x), f.array(packed), f.array(sc)
+    db, dc, out = f.array(b), f.array(c), f.zeros((m, n))
+    f.matmul(dx.arg(), dw.arg(dims=(n, k), dtype=fa.DTYPE_Q4_0), out.arg(), m, n, k, bias=db.arg() if bias else None,
+             c=dc.arg() if resid else None, transpose_b=not canonical, alpha=alpha, beta=beta, b_scales=ds.arg())
+    g, wv = out.download().astype(np.float64), want.astype(np.float64)
+    assert np.all(np.abs(g - wv) <= 2 * np.maximum(np.abs(wv), 2.0 ** -10) * 2.0 ** -10 + 1e-4), float(np.max(np.abs(g - wv)))
     for z in (dx, dw, ds, db, dc, out):
         z.free()
 

@@ -691,3 +691,47 @@ def test_q8_0_projections_vs_float64_on_dequantised_weights():
     xn = (xf * inv * g.astype(np.float32)).astype(np.float16)
     assert np.array_equal(q, orc.matmul_gemv_q8(xn, w8, sc))
     assert np.array_equal(kk, orc.matmul_gemv_q8(xn, w8[:8], sc[:8])) and np.array_equal(v, orc.matmul_gemv_q8(xn, w8[8:16], sc[8:16]))
+
+
+# ---------------------------------------------------------------- Q4_0 weights
+
+def test_q4_0_nibble_order_is_the_loaders_adjacent_pairs():
+    """GGML stores weight j in the low and weight j + 16 in the high nibble of byte j of a block; the reference's loader
+    (and its test helper, tests/gemm_v2_parity.rs:141-196) de-interleaves that into adjacent pairs, which is the order
+    policy_q4_0.metal:70-98 reads. The transform below is that helper's loop; packing adjacent elements directly must
+    give the same bytes, and the oracle's reader must return the original integers."""
+    rng = np.random.default_rng(40)
+    q = rng.integers(-8, 8, 32).astype(np.int8)
+    u = (q + 8).astype(np.uint8)
+    ggml = np.array([(u[16 + j] << 4) | u[j] for j in range(16)], np.uint8)
+    block = np.zeros(16, np.uint8)
+    for i in range(8):
+        b0, b1 = ggml[2 * i], ggml[2 * i + 1]
+        block[i] = ((b1 & 0x0F) << 4) | (b0 & 0x0F)
+        block[i + 8] = (b1 & 0xF0) | (b0 >> 4)
+    assert np.array_equal(block, orc.pack_q4_0(q))
+    assert np.array_equal(orc.unpack_q4_0(block), q)
+    assert np.array_equal(orc.unpack_q4_0(np.array([0x00, 0xFF, 0x80, 0x7F], np.uint8)),
+                          np.array([-8, -8, 7, 7, -8, 0, 7, -1], np.int8))
+
+
+def test_q4_0_quantiser_and_dot_against_float64():
+    """scale = max|w| / 7, q = round(w / scale) in [-8, 7] (tests/gemm_v2_parity.rs:112-166); the dot product of the
+    oracle (the Q8 block recurrence on the unpacked integers) equals the float64 product with the dequantised weights."""
+    rng = np.random.default_rng(41)
+    n, k, m = 24, 96, 3
+    w = rng.uniform(-0.1, 0.1, (n, k)).astype(np.float16)
+    x = rng.uniform(-1, 1, (m, k)).astype(np.float16)
+    q, sc = orc.quantize_q4_0(w)
+    assert q.min() >= -8 and q.max() <= 7
+    blocks = w.astype(np.float32).reshape(n, k // 32, 32)
+    assert np.array_equal(sc, (np.abs(blocks).max(axis=2) / np.float32(7.0)).astype(np.float16))
+    amax = np.abs(blocks).argmax(axis=2)  # the largest weight of a block maps to +-7
+    assert np.all(np.abs(np.take_along_axis(q.reshape(n, k // 32, 32), amax[:, :, None], axis=2)) == 7)
+    deq = q.reshape(n, k // 32, 32).astype(np.float64) * sc.astype(np.float64)[:, :, None]
+    assert np.max(np.abs(deq.reshape(n, k) - w.astype(np.float64))) <= 0.5 * float(sc.astype(np.float64).max()) * 1.01
+    for layout in (0, 1):
+        stored = orc.to_canonical(q) if layout == 1 else q.reshape(-1)
+        got = orc.matmul_gemv_q8(x, orc.unpack_q4_0(orc.pack_q4_0(stored)), sc, layout=layout)
+        want = x.astype(np.float64) @ deq.reshape(n, k).T
+        assert np.max(np.abs(got.astype(np.float64) - want)) <= 2.0 ** -10 * np.maximum(np.abs(want), 2.0 ** -10).max() + 1e-5
