@@ -374,7 +374,7 @@ def bench_kv_growth(f, args):
     f.profile_enable(False)
 
 
-def bench_fused_qkv(f, args, q8=False):
+def bench_fused_qkv(f, args, q8=False, q4=False):
     """The step before the path at Llama-3.2-3B decode shape: RMSNorm + Q/K/V projections of one token, F16 (or Q8_0)
     weights in the reference's canonical blocked layout, one layer per step over 8 distinct layers' weights."""
     import orc
@@ -385,7 +385,12 @@ def bench_fused_qkv(f, args, q8=False):
     layers, host0 = [], None
     for i in range(NL):  # distinct weights so that no launch finds the previous one's in cache
         ws = [rng.uniform(-0.1, 0.1, (n, K)).astype(np.float16) for n in (N, NK, NK)]
-        if q8:
+        if q4:
+            ws = [orc.quantize_q4_0(w) for w in ws]
+            packed = [orc.pack_q4_0(fa.canonical_layout(w)) for w, _ in ws]
+            layers.append(([f.array(p) for p in packed], [f.array(sc) for _, sc in ws]))
+            ws = [(orc.unpack_q4_0(p), sc) for p, (_, sc) in zip(packed, ws)]
+        elif q8:
             ws = [orc.quantize_q8_0(w) for w in ws]
             layers.append(([f.array(fa.canonical_layout(w)) for w, _ in ws], [f.array(sc) for _, sc in ws]))
         else:
@@ -397,12 +402,15 @@ def bench_fused_qkv(f, args, q8=False):
 
     def step(i):
         w, sc = layers[i % NL]
-        f.fused_qkv(dx.arg(), w[0].arg(), w[1].arg(), w[2].arg(), oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1, gamma=dg.arg(),
+        wa = [t.arg(dims=(n, K), dtype=fa.DTYPE_Q4_0) for t, n in zip(w, (N, NK, NK))] if q4 else [t.arg() for t in w]
+        f.fused_qkv(dx.arg(), wa[0], wa[1], wa[2], oq.arg(), ok.arg(), ov.arg(), K, N, NK, 1, gamma=dg.arg(),
                     scales=[t.arg() for t in sc] if sc else None)
 
     step(0)
     f.synchronize()
-    if q8:
+    if q4:
+        want = orc.fused_qkv_q8(x, [w for w, _ in host0], [sc for _, sc in host0], gamma=g, layout=1)
+    elif q8:
         want = orc.fused_qkv_q8(x, [w for w, _ in host0], [sc for _, sc in host0], gamma=g)
     else:
         want = orc.fused_qkv(x, *host0, gamma=g)
@@ -417,11 +425,11 @@ def bench_fused_qkv(f, args, q8=False):
         step(i)
     f.synchronize()
     dt = time.perf_counter() - t0
-    wbytes = (1.0 + 2.0 / 32) if q8 else 2.0  # per weight: int8 + an f16 scale per 32, or f16
+    wbytes = (0.5 + 2.0 / 32) if q4 else (1.0 + 2.0 / 32) if q8 else 2.0  # per weight: nibble / int8 + an f16 scale per 32, or f16
     nbytes = wbytes * (N + 2 * NK) * K + 2 * K * 2 + 2 * (N + 2 * NK)  # weights, input + gamma, outputs
     _finish_secondary(f, args, "FusedQkv layer-steps/s + achieved HBM GB/s, Llama-3.2-3B decode shape",
                       "llama3.2-3b FusedQkv at decode: RMSNorm + Q/K/V projections of one token, k_dim 3072, n_dim 3072, "
-                      "n_kv 1024, %s canonical weights, eager launches (profiling events on)" % ("Q8_0" if q8 else "F16"),
+                      "n_kv 1024, %s canonical weights, eager launches (profiling events on)" % ("Q4_0" if q4 else "Q8_0" if q8 else "F16"),
                       "fused_qkv_kernel", nbytes, dt, {"qkv_max_abs_err": err})
     f.profile_enable(False)
 
@@ -852,6 +860,7 @@ SECONDARY = {"llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": be
              "llama3b_fused_qkv_q8_chunk32": lambda f, args: bench_fused_qkv_chunk(f, args, 32, q8=True),
              "llama3b_fused_qkv_q8_prefill_2k": lambda f, args: bench_fused_qkv_chunk(f, args, 2048, q8=True),
              "llama3b_fused_qkv_q8": lambda f, args: bench_fused_qkv(f, args, q8=True),
+             "llama3b_fused_qkv_q4": lambda f, args: bench_fused_qkv(f, args, q4=True),
              "llama3b_o_proj_q8": lambda f, args: bench_o_proj(f, args, q8=True)}
 
 

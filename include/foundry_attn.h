@@ -360,8 +360,8 @@ fa_status fa_paged_copy_blocks(fa_ctx *ctx, const fa_paged_kv *cache, const int3
  * the same element order, dtype FA_DTYPE_Q8_0 or FA_DTYPE_I8, plus a scale tensor s_* of f16 [rows, k_dim / 32],
  * row-major, weight = int8 * scale of its 32-block) or Q4_0 (PolicyQ4_0, src/metals/policies/policy_q4_0.metal: two
  * weights per byte in the same element order - element 2i in the low nibble of byte i, the loader's adjacent-pair
- * packing - dtype FA_DTYPE_Q4_0, weight = (nibble - 8) * scale, the same scale tensor; at decode sizes only: more than a
- * few input rows run as passes of 16 over the weight stream); the other block-quantised policies are refused with
+ * packing - dtype FA_DTYPE_Q4_0, weight = (nibble - 8) * scale, the same scale tensor); the other block-quantised
+ * policies are refused with
  * FA_ERR_UNSUPPORTED_DTYPE.
  *   out_q[b, r] = f16( sum_k xn[b, k] * W_q[r, k] + bias_q[r] ),  r < n_dim;  out_k, out_v likewise, r < n_kv
  *   xn[b, k]    = f16( x[b, k] * rsqrt(mean_k x[b, k]^2 + epsilon) * gamma[k] )  with gamma, else x[b, k]
@@ -405,8 +405,7 @@ fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_ar
  * layout (matmul.rs:199-207). transpose_a and activations other than none are not built
  * (FA_ERR_OPERATION_NOT_SUPPORTED). bias, c: NULL or NULL buffer = absent (the reference's "zero" placeholder).
  * Any m is accepted: up to fa_set_gemm_min_m() - 1 input rows run as passes of 16 over the weight stream; from there
- * on the op is a tiled GEMM on the matrix cores (F16 and Q8_0 weights; Q4_0 stays on the passes), the counterpart of
- * the reference's GEMM for large m (src/metals/mma).
+ * on the op is a tiled GEMM on the matrix cores, the counterpart of the reference's GEMM for large m (src/metals/mma).
  * ------------------------------------------------------------------------------------------- */
 typedef struct fa_matmul_params {
     uint32_t m, n, k;            /* k a multiple of 32 */
@@ -432,7 +431,7 @@ fa_status fa_set_gemm_min_m(fa_ctx *ctx, uint32_t min_m);
 
 /* Which GEMM kernel fa_fused_qkv / fa_matmul use (same tiling and arithmetic; results equal up to the f32 summation
  * order of the split-K partials, which does not depend on the kernel): 1 = operand tiles staged through registers (any
- * shape, F16 and Q8_0 weights); 2 = tiles loaded from memory straight into LDS in steps of 64 features, two workgroups
+ * shape, every weight policy); 2 = tiles loaded from memory straight into LDS in steps of 64 features, two workgroups
  * per compute unit; 3 = the same in steps of 32 features, four workgroups per compute unit; 0 (default) = 2 or 3 by
  * the number of output tiles. 2 and 3 need F16 weights, k_dim a multiple of 64 and operands below 2 GiB, and fall back
  * to 1 otherwise. No counterpart in the reference (a tuning switch like fa_set_prefill_variant).

@@ -1,4 +1,4 @@
-// FusedQkv and MatMul for many input rows (a prefill chunk): a tiled f16 GEMM on the matrix cores, F16 or Q8_0 weights.
+// FusedQkv and MatMul for many input rows (a prefill chunk): a tiled f16 GEMM on the matrix cores; F16, Q8_0 or Q4_0 weights.
 // Reference: the same ops as fa_qkv.hip - src/metals/gemv/qkv_step.rs:14-120 (FusedQkv), src/metals/matmul.rs:190-239
 // (MatMul; its large-m form is a GEMM, src/metals/mma) - with the write stage of src/metals/gemv/stages.rs:200-224.
 //
@@ -44,7 +44,7 @@ typedef float f4v_t __attribute__((ext_vector_type(4)));
 typedef float f16v_t __attribute__((ext_vector_type(16)));
 
 struct GemmDev {
-    const void *w[3];       // f16, or int8 (Q8_0) in the same element order
+    const void *w[3];       // f16, or int8 (Q8_0) / nibbles (Q4_0) in the same element order
     const __half *scales[3];  // Q8_0: f16 [rows, k_dim / 32] per matrix
     const __half *bias[3];
     __half *out[3];
@@ -201,12 +201,31 @@ __device__ __forceinline__ void q8_to_f16(const u4v_t raw, h8_t &p0, h8_t &p1) {
     }
 }
 
+// 8 Q4_0 weights (one word: element 2i in the low nibble of byte i, value = nibble - 8) -> one piece of 8 f16, exactly:
+// the nibbles become two words of four bytes 0..15 in element order, then 0x6400 | u is 1024 + u and 1024 + u - 1032.
+__device__ __forceinline__ h8_t q4_to_f16(uint32_t w) {
+    const uint32_t even = w & 0x0f0f0f0fu, odd = (w >> 4) & 0x0f0f0f0fu;
+    const uint32_t b[2] = {__builtin_amdgcn_perm(odd, even, 0x05010400u), __builtin_amdgcn_perm(odd, even, 0x07030602u)};
+    const h2v_t bias = {(_Float16)1032.0f, (_Float16)1032.0f};
+    h8_t r;
+#pragma unroll
+    for (int hw = 0; hw < 2; ++hw) {
+        const h2v_t lo = __builtin_bit_cast(h2v_t, __builtin_amdgcn_perm(0x64646464u, b[hw], 0x05010400u)) - bias;
+        const h2v_t hi = __builtin_bit_cast(h2v_t, __builtin_amdgcn_perm(0x64646464u, b[hw], 0x07030602u)) - bias;
+        r[4 * hw + 0] = lo[0], r[4 * hw + 1] = lo[1], r[4 * hw + 2] = hi[0], r[4 * hw + 3] = hi[1];
+    }
+    return r;
+}
+
 // Q8: the weights become exact f16 integers on their way into LDS; the matrix instructions of one 32-feature block
 // start from zero and their sums are multiplied by the block's scale of the weight row before they are added up (the
 // recurrence of tests/gemv_v2_parity.rs:95-116). For that the operands are swapped (input rows x weight rows), so that
 // a lane holds one weight row and needs one scale per block and tile.
-template <bool CANON, bool Q8>
+// WB: bits per weight - 16 (f16), 8 (Q8_0) or 4 (Q4_0: 16 bytes are the 32 features of a block = four f16 pieces).
+template <bool CANON, int WB>
 __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
+    constexpr bool Q8 = WB != 16;  // block-quantised: integer weights and block scales
+    constexpr bool Q4 = WB == 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr int W_STRIDE = CANON ? GM_STRIDE_CANONICAL : GM_STRIDE_ROWMAJOR;
     constexpr int X_STRIDE = GM_STRIDE_ROWMAJOR;
@@ -235,7 +254,9 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
     //   weights, row-major and input: piece p = (row p / 8, piece p % 8)
     //   Q8 weights: 16 bytes are 16 features = two f16 pieces; canonical (block i, row tid / 2, half tid % 2),
     //   row-major (row p / 4, quarter p % 4)
-    constexpr int W_LOADS = Q8 ? GM_LOADS / 2 : GM_LOADS;
+    //   Q4 weights: 16 bytes are the 32 features of one block = four f16 pieces; canonical (block tid / 128, row
+    //   tid % 128), row-major (row tid / 2, block tid % 2)
+    constexpr int W_LOADS = Q4 ? 1 : Q8 ? GM_LOADS / 2 : GM_LOADS;
     const unsigned char *wp[W_LOADS];
     const unsigned char *xp[GM_LOADS];
     uint32_t w_lds[W_LOADS], x_lds[GM_LOADS];
@@ -246,7 +267,15 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
     for (int i = 0; i < W_LOADS; ++i) {
         const uint32_t p = tid + GM_NT * i;
         uint32_t row, piece;
-        if constexpr (Q8) {
+        if constexpr (Q4) {
+            if (CANON) {
+                row = tid % GM_TN, piece = (tid / GM_TN) * 4;
+                wp[i] = W + ((size_t)(n0 + row) * 32 + (size_t)(tid / GM_TN) * N * 32) / 2;
+            } else {
+                row = tid / 2, piece = (tid % 2) * 4;
+                wp[i] = W + ((size_t)(n0 + row) * K + (tid % 2) * 32) / 2;
+            }
+        } else if constexpr (Q8) {
             if (CANON) {
                 row = tid / 2, piece = i * 4 + (tid % 2) * 2;
                 wp[i] = W + (size_t)(n0 + row) * 32 + (size_t)i * N * 32 + (tid % 2) * 16;
@@ -275,8 +304,7 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
         x_lds[i] = xpiece * X_STRIDE + xrow * 16;
         x_kpiece[i] = xpiece * 8;
     }
-    constexpr size_t WES = Q8 ? 1 : 2;  // bytes per weight
-    const size_t w_step = CANON ? (size_t)2 * N * 32 * WES : (size_t)GM_BK * WES;  // bytes between steps
+    const size_t w_step = (CANON ? (size_t)2 * N * 32 : (size_t)GM_BK) * WB / 8;  // bytes between steps
     const size_t x_step = (size_t)GM_BK * 2;
     // Q8: thread t fetches the scale of (weight row t % 128, block t / 128 of the step); scales are [row][k_dim / 32]
     const uint32_t nkb = K / 32;
@@ -317,7 +345,10 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
         unsigned char *base = smem + stage * GM_STAGE_BYTES;
 #pragma unroll
         for (int i = 0; i < W_LOADS; ++i) {
-            if constexpr (Q8) {
+            if constexpr (Q4) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) *reinterpret_cast<h8_t *>(base + w_lds[i] + q * W_STRIDE) = q4_to_f16(wr[i][q]);
+            } else if constexpr (Q8) {
                 h8_t p0, p1;
                 q8_to_f16(wr[i], p0, p1);
                 *reinterpret_cast<h8_t *>(base + w_lds[i]) = p0;
@@ -808,10 +839,12 @@ fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
     }
     static bool lds_allowed = false;
     if (!lds_allowed) {
-        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
-        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
-        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
-        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
+        FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
         lds_allowed = true;
     }
     FaLaunchScope scope(ctx, l.n_kv ? "fused_qkv_gemm_kernel" : "matmul_gemm_kernel", true);
@@ -836,12 +869,15 @@ fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
         }
         if (l.canonical) scope.launch(qkv_gemm_dma_kernel<true>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
         else scope.launch(qkv_gemm_dma_kernel<false>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+    } else if (l.weight_bits == 4) {
+        if (l.canonical) scope.launch(qkv_gemm_kernel<true, 4>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+        else scope.launch(qkv_gemm_kernel<false, 4>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
     } else if (q8) {
-        if (l.canonical) scope.launch(qkv_gemm_kernel<true, true>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
-        else scope.launch(qkv_gemm_kernel<false, true>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+        if (l.canonical) scope.launch(qkv_gemm_kernel<true, 8>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+        else scope.launch(qkv_gemm_kernel<false, 8>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
     } else {
-        if (l.canonical) scope.launch(qkv_gemm_kernel<true, false>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
-        else scope.launch(qkv_gemm_kernel<false, false>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+        if (l.canonical) scope.launch(qkv_gemm_kernel<true, 16>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
+        else scope.launch(qkv_gemm_kernel<false, 16>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
     }
     FA_TRY(scope.finish());
     if (a.k_splits > 1) {

@@ -309,7 +309,7 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     // m = 32: 76.8 / 19.8.
     constexpr uint32_t GEMM_MIN_M_DEFAULT = 12;
     auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
-    const bool gemm_ok = !q4 && l.k_dim % (q8 ? 32 : 8) == 0 && aligned16(l.x) && aligned16(l.w[0]) && aligned16(l.w[1]) &&
+    const bool gemm_ok = l.k_dim % (q8 ? 32 : 8) == 0 && aligned16(l.x) && aligned16(l.w[0]) && aligned16(l.w[1]) &&
                          aligned16(l.w[2]) && aligned16(l.gamma);
     if (gemm_ok && l.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : GEMM_MIN_M_DEFAULT)) return fa_launch_fused_qkv_gemm(ctx, l);
     const uint32_t total_rows = l.n_dim + 2 * l.n_kv;

@@ -336,7 +336,11 @@ def test_matmul_q8_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta):
     (3072, 3072, 1024, 1, True, False, 1),   # Llama-3.2-3B decode
     (896, 896, 128, 5, True, True, 0),       # row-major bytes
     (64, 40, 24, 3, True, True, 1),
-    (896, 896, 128, 20, False, True, 1),     # more than a few rows: passes of 16 (no GEMM for this policy)
+    (896, 896, 128, 20, False, True, 1),     # the split-K GEMM, and two passes of input rows
+    (896, 896, 128, 32, True, True, 0),      # a default prefill chunk, row-major bytes
+    (3072, 3072, 1024, 200, True, False, 1), # Llama-3.2-3B, ragged input tiles
+    (1056, 200, 72, 130, True, True, 0),     # k_dim = 16.5 steps, weight rows that do not fill tiles
+    (1056, 200, 72, 130, False, True, 1),
 ])
 def test_fused_qkv_q4_0_equals_oracle(K, N, NK, m, norm, bias, layout):
     """Q4_0 weights (policy_q4_0.metal): the GPU reads the packed bytes, the oracle the integers its own reader makes of
@@ -355,13 +359,22 @@ def test_fused_qkv_q4_0_equals_oracle(K, N, NK, m, norm, bias, layout):
     db = [f.array(b) for b in bs]
     outs = [f.zeros((m, n)) for n in (N, NK, NK)]
     wargs = [w.arg(dims=(n, K), dtype=fa.DTYPE_Q4_0) for w, n in zip(dev_w, (N, NK, NK))]
-    f.fused_qkv(dx.arg(), wargs[0], wargs[1], wargs[2], outs[0].arg(), outs[1].arg(), outs[2].arg(),
-                K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout,
-                scales=[s.arg() for s in dev_s])
-    for o, w, name in zip(outs, want, "qkv"):
-        got = o.download()
-        assert np.all(np.isfinite(got)), name
-        assert _close(got, w, K), (name, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
+    try:
+        for min_m, variant in _paths(m):
+            f.set_gemm_min_m(min_m)
+            f.set_gemm_variant(variant)
+            for o in outs:
+                o.upload(np.zeros(o.shape, np.float16))
+            f.fused_qkv(dx.arg(), wargs[0], wargs[1], wargs[2], outs[0].arg(), outs[1].arg(), outs[2].arg(),
+                        K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout,
+                        scales=[s.arg() for s in dev_s])
+            for o, w, name in zip(outs, want, "qkv"):
+                got = o.download()
+                assert np.all(np.isfinite(got)), (name, min_m, variant)
+                assert _close(got, w, K), (name, min_m, variant, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
+    finally:
+        f.set_gemm_min_m()
+        f.set_gemm_variant()
     for b in dev_w + dev_s + [dx, dg] + db + outs:
         b.free()
 
@@ -370,6 +383,8 @@ def test_fused_qkv_q4_0_equals_oracle(K, N, NK, m, norm, bias, layout):
     (1, 128, 128, False, False, False, 1.0, 0.0),
     (1, 3072, 3072, True, False, True, 1.0, 1.0),   # o_proj
     (7, 896, 896, True, True, True, 0.5, 0.5),
+    (40, 896, 896, False, True, True, 0.25, 0.75),   # the split-K GEMM
+    (256, 3072, 3072, True, False, True, 1.0, 1.0),  # o_proj of a 256-token prefill chunk
 ])
 def test_matmul_q4_0_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta):
     announce("matmul q4_0", m, n, k, canonical, bias, resid, alpha, beta)
