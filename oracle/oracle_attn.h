@@ -46,6 +46,12 @@
  *   orc_*_q8                  pinned: transcription of the reference test's Q8 CPU helper (tests/gemv_v2_parity.rs:82-125)
  *                             checked against float64 on the dequantised weights; the fused QKV form applies the same
  *                             per-8-chunk recurrence to the normalised input (no reference CPU helper combines them)
+ *   orc_unpack_q4_0           pinned: the nibble order against the reference test helper's GGML -> adjacent-pair transform
+ *                             (tests/gemm_v2_parity.rs:141-196) and known bytes; the Q4_0 dot is the Q8 recurrence on these
+ *                             integers (policy_q4_0.metal:45-66), checked against float64 on the dequantised weights. The
+ *                             reference holds no Q4_0 test of FusedQkv or of the GEMV path with a CPU helper of its own
+ *                             (its Q4_0 cases run MatMul against a dequantised f16 GEMM): that combination is pinned here
+ *                             by the float64 check only
  *   orc_fused_qkv             pinned: transcription of the reference test's CPU helpers (tests/qkv_parity_f16.rs:17-72)
  *                             checked against float64 matrix products; orc_weight_index pinned as a bijection that
  *                             reduces to the row-major index per 32-feature block (src/compound/stages/layout.rs:79-100)
