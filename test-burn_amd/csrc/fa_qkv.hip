@@ -161,7 +161,33 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     if (n_batches > 1) request(wbuf[1], 1);
 
     // Input rows of this pass into LDS, normalised: x * rsqrt(mean(x^2) + eps) * gamma in f32, rounded to f16.
-    for (uint32_t r = 0; r < cols; ++r) {
+    // Four rows or more: a wave takes whole rows (row r by wave r % 8) and needs no workgroup barrier for the sum of
+    // squares, so the rows are staged side by side instead of one after the other with two barriers each.
+    const bool rows_by_wave = cols >= 4;  // measured on 5120 x 3072: 2 rows 9.2 us row after row, 10.4 by wave; 4 rows 11.3 / 10.5; 8 rows 15.7 / 11.1
+    if (rows_by_wave) {
+        for (uint32_t r = wave; r < cols; r += QKV_NW) {
+            const __half *xr = a.x + (size_t)(m0 + r) * K;
+            unsigned char *dst = x_lds + (size_t)r * a.x_stride;
+            float ss = 0.0f;
+            for (uint32_t k8 = lane; k8 < K / 8; k8 += 64) {
+                const h8_t v = *reinterpret_cast<const h8_t *>(xr + k8 * 8);
+                *reinterpret_cast<h8_t *>(dst + k8 * 16) = v;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) ss += (float)v[i] * (float)v[i];
+            }
+            if (a.gamma) {
+                const float inv_rms = rsqrtf(wave_sum(ss) / (float)K + a.eps);
+                for (uint32_t k8 = lane; k8 < K / 8; k8 += 64) {  // each lane rewrites what it wrote
+                    h8_t v = *reinterpret_cast<const h8_t *>(dst + k8 * 16);
+                    const h8_t g = *reinterpret_cast<const h8_t *>(a.gamma + k8 * 8);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) v[i] = (_Float16)(((float)v[i] * inv_rms) * (float)g[i]);
+                    *reinterpret_cast<h8_t *>(dst + k8 * 16) = v;
+                }
+            }
+        }
+    }
+    for (uint32_t r = 0; r < (rows_by_wave ? 0u : cols); ++r) {
         const __half *xr = a.x + (size_t)(m0 + r) * K;
         unsigned char *dst = x_lds + (size_t)r * a.x_stride;
         float ss = 0.0f;
@@ -304,9 +330,9 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     const bool q8 = l.scales[0] != nullptr;
     const bool q4 = l.weight_bits == 4;
     // More than a few input rows: no longer a weight stream but a GEMM (fa_gemm.hip). Measured on 5120 x 3072 with a
-    // gamma, passes of this kernel against the GEMM (norm kernel, split-K GEMM, finish kernel): m = 8: 15.0 / 18.5 us,
-    // m = 12 (from where only one workgroup's input rows fit a CU's LDS): 30.3 / 18.2, m = 16: 37.3 / 18.7,
-    // m = 32: 76.8 / 19.8.
+    // gamma, this kernel against the GEMM (norm kernel, split-K GEMM, finish kernel): m = 4: 10.4 / 16.7 us, m = 10:
+    // 13.8 / 16.9, m = 12 (from where only one workgroup's input rows fit a CU's LDS): 18.8 / 17.0, m = 16: 19.7 / 17.5,
+    // m = 24 (two passes): 35.1 / 18.2.
     constexpr uint32_t GEMM_MIN_M_DEFAULT = 12;
     auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
     const bool gemm_ok = l.k_dim % (q8 ? 32 : 8) == 0 && aligned16(l.x) && aligned16(l.w[0]) && aligned16(l.w[1]) &&
