@@ -748,10 +748,22 @@ __global__ void __launch_bounds__(256) gemm_finish_kernel(GemmDev a) {
     const size_t o = (size_t)gm * N + gn;
     if (a.vec_store) {
         f4v_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
-        for (uint32_t sp = 0; sp < a.k_splits; ++sp) {
-            const float *src = a.partial + ((size_t)sp * a.m + gm) * a.n_total + col;
-            s0 += *reinterpret_cast<const f4v_t *>(src);
-            s1 += *reinterpret_cast<const f4v_t *>(src + 4);
+        const size_t split_stride = (size_t)a.m * a.n_total;
+        const float *src = a.partial + (size_t)gm * a.n_total + col;
+        uint32_t sp = 0;
+        for (; sp + 4 <= a.k_splits; sp += 4) {  // four splits' loads in flight, added in split order
+            f4v_t u[4], w[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                u[q] = *reinterpret_cast<const f4v_t *>(src + (sp + q) * split_stride);
+                w[q] = *reinterpret_cast<const f4v_t *>(src + (sp + q) * split_stride + 4);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; ++q) s0 += u[q], s1 += w[q];
+        }
+        for (; sp < a.k_splits; ++sp) {
+            s0 += *reinterpret_cast<const f4v_t *>(src + sp * split_stride);
+            s1 += *reinterpret_cast<const f4v_t *>(src + sp * split_stride + 4);
         }
         const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
         const h8_t bv = bias ? *reinterpret_cast<const h8_t *>(bias + gn) : z;
