@@ -406,6 +406,10 @@ fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_ar
  * (FA_ERR_OPERATION_NOT_SUPPORTED). bias, c: NULL or NULL buffer = absent (the reference's "zero" placeholder).
  * Any m is accepted: up to fa_set_gemm_min_m() - 1 input rows run as passes of 16 over the weight stream; from there
  * on the op is a tiled GEMM on the matrix cores, the counterpart of the reference's GEMM for large m (src/metals/mma).
+ * Block-quantised weights follow the arithmetic of the path that runs: the weight stream multiplies each 32-block's f32
+ * sum by the block scale (the GEMV policies, policy_q8.metal / policy_q4_0.metal), the GEMM works on f16(weight * scale)
+ * tiles like the reference's tile loader (src/metals/mma/tile_loader.metal:100-120); the two differ by the f16 rounding
+ * of the dequantised weights. The same holds for fa_fused_qkv.
  * ------------------------------------------------------------------------------------------- */
 typedef struct fa_matmul_params {
     uint32_t m, n, k;            /* k a multiple of 32 */

@@ -35,8 +35,7 @@ constexpr int GM_STRIDE_CANONICAL = GM_TN * 16 + 32;   // ... 16 rows x 4 pieces
 constexpr int GM_OPERAND_BYTES = GM_PIECES * GM_STRIDE_CANONICAL;  // the larger of the two
 constexpr int GM_STAGE_BYTES = 2 * GM_OPERAND_BYTES;
 constexpr int GM_T_STRIDE = GM_TN * 4 + 16;             // epilogue tile: bytes per input row
-constexpr int GM_LDS_BYTES = (2 * GM_STAGE_BYTES > GM_TM * GM_T_STRIDE ? 2 * GM_STAGE_BYTES : GM_TM * GM_T_STRIDE) +
-                             2 * 2 * GM_TN * 2;  // + Q8 block scales [stage][2 blocks][128 rows] f16
+constexpr int GM_LDS_BYTES = 2 * GM_STAGE_BYTES > GM_TM * GM_T_STRIDE ? 2 * GM_STAGE_BYTES : GM_TM * GM_T_STRIDE;
 constexpr int GM_LOADS = GM_TN * GM_PIECES / GM_NT;     // 16-byte pieces per thread, operand and step (4)
 
 typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
@@ -91,7 +90,7 @@ __global__ void __launch_bounds__(256) rmsnorm_rows_kernel(const __half *x, cons
 // The end of an output tile, shared by the GEMM kernels: accumulators -> LDS (f32, [input row][weight row]) -> either
 // the write stage and token-major f16 stores, or (split-K) the f32 partial tile. HALVES: the tile goes through LDS in
 // two halves of 64 input rows (tile j of every wave), for kernels that keep their LDS footprint at half a tile.
-template <bool Q8, bool HALVES>
+template <bool HALVES>
 __device__ __forceinline__ void gemm_epilogue(const GemmDev &a, unsigned char *smem, const f16v_t (&acc)[2][2], int tid,
                                               int lane, int wn, int wm, int mat, uint32_t N, uint32_t n0, uint32_t m0,
                                               uint32_t split) {
@@ -103,9 +102,8 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev &a, unsigned char *s
 #pragma unroll
     for (int half = 0; half < NH; ++half) {
         if (half) __syncthreads();  // the first half has been read out
-        // Accumulators -> LDS as f32 [input row][weight row]. Register r of lane l of a 32 x 32 tile is row
-        // 8 (r / 4) + 4 (l / 32) + r % 4 of the first operand and row l % 32 of the second: with the weights first, four
-        // consecutive weight rows per 16-byte write; with the input first (Q8), one float per register.
+        // Accumulators -> LDS as f32 [input row][weight row]. Register r of lane l of a 32 x 32 tile is weight row
+        // 8 (r / 4) + 4 (l / 32) + r % 4 and input row l % 32: four consecutive weight rows per 16-byte write.
 #pragma unroll
         for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -114,19 +112,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev &a, unsigned char *s
                 const uint32_t t0 = HALVES ? wm * 32 : wm * 64 + j * 32;  // LDS row of the tile's first input row
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    if constexpr (Q8) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const uint32_t trow = t0 + g * 8 + (lane >> 5) * 4 + e;
-                            const uint32_t nrow = wn * 64 + i * 32 + (lane & 31);
-                            *reinterpret_cast<float *>(smem + trow * GM_T_STRIDE + nrow * 4) = acc[i][j][g * 4 + e];
-                        }
-                    } else {
-                        const uint32_t nrow = wn * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
-                        const uint32_t trow = t0 + (lane & 31);
-                        const f4v_t q = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-                        *reinterpret_cast<f4v_t *>(smem + trow * GM_T_STRIDE + nrow * 4) = q;
-                    }
+                    const uint32_t nrow = wn * 64 + i * 32 + g * 8 + (lane >> 5) * 4;
+                    const uint32_t trow = t0 + (lane & 31);
+                    const f4v_t q = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+                    *reinterpret_cast<f4v_t *>(smem + trow * GM_T_STRIDE + nrow * 4) = q;
                 }
             }
         __syncthreads();
@@ -217,14 +206,17 @@ __device__ __forceinline__ h8_t q4_to_f16(uint32_t w) {
     return r;
 }
 
-// Q8: the weights become exact f16 integers on their way into LDS; the matrix instructions of one 32-feature block
-// start from zero and their sums are multiplied by the block's scale of the weight row before they are added up (the
-// recurrence of tests/gemv_v2_parity.rs:95-116). For that the operands are swapped (input rows x weight rows), so that
-// a lane holds one weight row and needs one scale per block and tile.
+// Block-quantised weights become f16 on their way into LDS as the reference's GEMM tile loader makes them
+// (src/metals/mma/tile_loader.metal:100-120: (half)(weight * (float)scale); the CPU reference of its tests dequantises
+// the same way, tests/gemm_v2_parity.rs:295-350): the integer is converted exactly, then multiplied by its block's scale
+// with one f16 rounding. From there on the GEMM is the F16 one. (The weight-stream kernel keeps the GEMV policies'
+// arithmetic instead - block sums in f32 times the scale; an earlier form of this kernel did that too, with 64 scaled
+// adds per block and wave beside 8 matrix instructions, and was bound by them: 152 us against 121 for F16 on 2048 x
+// 5120 x 3072.)
 // WB: bits per weight - 16 (f16), 8 (Q8_0) or 4 (Q4_0: 16 bytes are the 32 features of a block = four f16 pieces).
 template <bool CANON, int WB>
 __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
-    constexpr bool Q8 = WB != 16;  // block-quantised: integer weights and block scales
+    constexpr bool Q8 = WB != 16;  // block-quantised: integer weights with one f16 scale per 32 of a row
     constexpr bool Q4 = WB == 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr int W_STRIDE = CANON ? GM_STRIDE_CANONICAL : GM_STRIDE_ROWMAJOR;
@@ -262,6 +254,7 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
     uint32_t w_lds[W_LOADS], x_lds[GM_LOADS];
     bool w_ok[W_LOADS], x_ok[GM_LOADS];
     uint32_t w_kpiece[W_LOADS];  // first feature of the piece within the step, for the tail guard
+    uint32_t w_row[W_LOADS];
     uint32_t x_kpiece[GM_LOADS];
 #pragma unroll
     for (int i = 0; i < W_LOADS; ++i) {
@@ -294,6 +287,7 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
         w_ok[i] = n0 + row < N;
         w_lds[i] = piece * W_STRIDE + row * 16;
         w_kpiece[i] = piece * 8;
+        w_row[i] = row;
     }
 #pragma unroll
     for (int i = 0; i < GM_LOADS; ++i) {
@@ -306,22 +300,20 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
     }
     const size_t w_step = (CANON ? (size_t)2 * N * 32 : (size_t)GM_BK) * WB / 8;  // bytes between steps
     const size_t x_step = (size_t)GM_BK * 2;
-    // Q8: thread t fetches the scale of (weight row t % 128, block t / 128 of the step); scales are [row][k_dim / 32]
+    // Block-quantised weights: each 16-byte request lies within one 32-feature block of one row; its scale
+    // (scales[row][k_dim / 32]) is requested with it and folded into the f16 weights on their way into LDS.
     const uint32_t nkb = K / 32;
-    const __half *sc_src = nullptr;
-    bool sc_ok = false;
+    const __half *w_scale[W_LOADS];
     if constexpr (Q8) {
         const __half *sp = mat == 0 ? a.scales[0] : mat == 1 ? a.scales[1] : a.scales[2];
-        const uint32_t row = tid % GM_TN;
-        sc_ok = n0 + row < N;
-        sc_src = sp + (size_t)(n0 + row) * nkb + tid / GM_TN;
+#pragma unroll
+        for (int i = 0; i < W_LOADS; ++i) w_scale[i] = sp + (size_t)(n0 + w_row[i]) * nkb + w_kpiece[i] / 32;
     }
-    _Float16 *sc_lds = reinterpret_cast<_Float16 *>(smem + 2 * GM_STAGE_BYTES);  // [stage][2 blocks][128 rows]
 
     typedef typename std::conditional<Q8, u4v_t, h8_t>::type wreg_t;
     wreg_t wr[W_LOADS];
     h8_t xr[GM_LOADS];
-    _Float16 sr = (_Float16)0.0f;
+    _Float16 wsc[W_LOADS];
     auto fetch = [&](uint32_t ks) {
         const uint32_t k0 = ks * GM_BK;
 #pragma unroll
@@ -329,16 +321,14 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
             wreg_t z;
             if constexpr (Q8) z = u4v_t{0u, 0u, 0u, 0u};
             else z = h8_t{0, 0, 0, 0, 0, 0, 0, 0};
-            wr[i] = (w_ok[i] && k0 + w_kpiece[i] < K) ? *reinterpret_cast<const wreg_t *>(wp[i] + ks * w_step) : z;
+            const bool ok = w_ok[i] && k0 + w_kpiece[i] < K;
+            wr[i] = ok ? *reinterpret_cast<const wreg_t *>(wp[i] + ks * w_step) : z;
+            if constexpr (Q8) wsc[i] = ok ? *reinterpret_cast<const _Float16 *>(w_scale[i] + ks * 2) : (_Float16)0.0f;
         }
 #pragma unroll
         for (int i = 0; i < GM_LOADS; ++i) {
             const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
             xr[i] = (x_ok[i] && k0 + x_kpiece[i] < K) ? *reinterpret_cast<const h8_t *>(xp[i] + ks * x_step) : z;
-        }
-        if constexpr (Q8) {
-            const uint32_t kb = ks * 2 + tid / GM_TN;
-            sr = (sc_ok && kb < nkb) ? *reinterpret_cast<const _Float16 *>(sc_src + ks * 2) : (_Float16)0.0f;
         }
     };
     auto stash = [&](int stage) {
@@ -346,20 +336,21 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
 #pragma unroll
         for (int i = 0; i < W_LOADS; ++i) {
             if constexpr (Q4) {
+                const h8_t sc = {wsc[i], wsc[i], wsc[i], wsc[i], wsc[i], wsc[i], wsc[i], wsc[i]};
 #pragma unroll
-                for (int q = 0; q < 4; ++q) *reinterpret_cast<h8_t *>(base + w_lds[i] + q * W_STRIDE) = q4_to_f16(wr[i][q]);
+                for (int q = 0; q < 4; ++q) *reinterpret_cast<h8_t *>(base + w_lds[i] + q * W_STRIDE) = q4_to_f16(wr[i][q]) * sc;
             } else if constexpr (Q8) {
+                const h8_t sc = {wsc[i], wsc[i], wsc[i], wsc[i], wsc[i], wsc[i], wsc[i], wsc[i]};
                 h8_t p0, p1;
                 q8_to_f16(wr[i], p0, p1);
-                *reinterpret_cast<h8_t *>(base + w_lds[i]) = p0;
-                *reinterpret_cast<h8_t *>(base + w_lds[i] + W_STRIDE) = p1;
+                *reinterpret_cast<h8_t *>(base + w_lds[i]) = p0 * sc;
+                *reinterpret_cast<h8_t *>(base + w_lds[i] + W_STRIDE) = p1 * sc;
             } else {
                 *reinterpret_cast<h8_t *>(base + w_lds[i]) = wr[i];
             }
         }
 #pragma unroll
         for (int i = 0; i < GM_LOADS; ++i) *reinterpret_cast<h8_t *>(base + GM_OPERAND_BYTES + x_lds[i]) = xr[i];
-        if constexpr (Q8) sc_lds[stage * 2 * GM_TN + tid] = sr;
     };
 
     // Wave (wn, wm) owns weight rows 64 wn .. +63 and input rows 64 wm .. +63 of the tile.
@@ -385,42 +376,7 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
         if (more) fetch(ks + 1);
         const unsigned char *wa = smem + (ks & 1) * GM_STAGE_BYTES;
         const unsigned char *xa = wa + GM_OPERAND_BYTES;
-        if constexpr (Q8) {
-            // not unrolled: unrolled, the scheduler starts all eight block tiles before the first scaled add and their
-            // 128 result registers spill
-#pragma unroll 1
-            for (int blk = 0; blk < 2; ++blk) {
-                h8_t fb[2][2];  // [tile][16-feature half of the block]
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-#pragma unroll
-                    for (int h = 0; h < 2; ++h)
-                        fb[j][h] = *reinterpret_cast<const h8_t *>(xa + b_off + (blk * 2 + h) * 2 * X_STRIDE + j * 32 * 16);
-#pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    // two tiles' block sums at a time (the scheduling fences keep the rest out of the registers)
-                    h8_t fa[2];
-#pragma unroll
-                    for (int h = 0; h < 2; ++h)
-                        fa[h] = *reinterpret_cast<const h8_t *>(wa + a_off + (blk * 2 + h) * 2 * W_STRIDE + i * 32 * 16);
-                    const float sc = (float)sc_lds[((ks & 1) * 2 + blk) * GM_TN + wn * 64 + i * 32 + (lane & 31)];
-                    f16v_t t[2];
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) {
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) t[j][r] = 0.0f;
-                        t[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j][0], fa[0], t[j], 0, 0, 0);
-                    }
-#pragma unroll
-                    for (int j = 0; j < 2; ++j) t[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j][1], fa[1], t[j], 0, 0, 0);
-#pragma unroll
-                    for (int j = 0; j < 2; ++j)
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) acc[i][j][r] += t[j][r] * sc;
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
-        } else {
+        {
 #pragma unroll
             for (int kk = 0; kk < GM_BK / 16; ++kk) {
                 h8_t fa[2], fb[2];
@@ -439,7 +395,7 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_kernel(GemmDev a) {
         __syncthreads();
     }
 
-    gemm_epilogue<Q8, false>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
+    gemm_epilogue<false>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -604,7 +560,7 @@ __global__ void __launch_bounds__(GM_NT, 2) qkv_gemm_dma_kernel(GemmDev a) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
-    gemm_epilogue<false, false>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
+    gemm_epilogue<false>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
 }
 
 // The LDS-direct GEMM in steps of 32 features, two stages, with the output tile leaving through LDS in two halves: a
@@ -727,7 +683,7 @@ __global__ void __launch_bounds__(GM_NT, 4) qkv_gemm_dma32_kernel(GemmDev a) {
         }
     }
     __syncthreads();  // the stages are reused by the output tile
-    gemm_epilogue<false, true>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
+    gemm_epilogue<true>(a, smem, acc, tid, lane, wn, wm, mat, N, n0, m0, split);
 }
 
 // Adds the split-K partial tiles in split order and applies the write stage: one thread per 8 output columns.

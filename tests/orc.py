@@ -306,6 +306,17 @@ def unpack_q4_0(packed):
     return out
 
 
+def dequantize_blocks(q, scales, wpb=32):
+    """Block-quantised integers [n, k] (row-major) and their f16 scales [n, k / wpb] -> the f16 weights the reference's
+    GEMM works on: f16(q * scale), one rounding (src/metals/mma/tile_loader.metal:100-120; the CPU reference of
+    tests/gemm_v2_parity.rs:295-350 dequantises the same way). q * scale is exact in f32 (8-bit integer times an 11-bit
+    significand), so this is a single f32 -> f16 rounding."""
+    q = np.asarray(q)
+    n, k = q.shape
+    sf = np.asarray(scales, np.float16).astype(np.float32).reshape(n, k // wpb)
+    return (q.astype(np.float32).reshape(n, k // wpb, wpb) * sf[:, :, None]).reshape(n, k).astype(np.float16)
+
+
 def _i8(a):
     return np.ascontiguousarray(a, dtype=np.int8)
 

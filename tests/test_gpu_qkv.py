@@ -34,6 +34,13 @@ def _paths(m):
     return [(0, 0), (0, 1), (0, 2), (0, 3)]
 
 
+def _gemm_runs(m, min_m):
+    """Whether the library takes the GEMM for m input rows under the threshold override min_m (0 = its default of 12).
+    Block-quantised weights then follow the reference GEMM's arithmetic (f16(q * scale) weights, then the F16 product,
+    src/metals/mma/tile_loader.metal:100-120), the weight-stream kernel the GEMV policies' (block sums times scale)."""
+    return m >= (12 if min_m == 0 else min_m)
+
+
 def _close(got, want, K):
     g, w = got.astype(np.float64), want.astype(np.float64)
     ulp = np.maximum(np.abs(w), 2.0 ** -10) * 2.0 ** -10
@@ -264,7 +271,9 @@ def test_fused_qkv_q8_equals_oracle(K, N, NK, m, norm, bias, layout):
     rng = np.random.default_rng(K + N + m + 1)
     x, g, ws, bs = _data(rng, K, N, NK, m)
     q8 = [orc.quantize_q8_0(w) for w in ws]
-    want = orc.fused_qkv_q8(x, [q for q, _ in q8], [s for _, s in q8], gamma=g if norm else None, biases=bs if bias else None)
+    want_stream = orc.fused_qkv_q8(x, [q for q, _ in q8], [s for _, s in q8], gamma=g if norm else None, biases=bs if bias else None)
+    want_gemm = orc.fused_qkv(x, *[orc.dequantize_blocks(q, s) for q, s in q8], gamma=g if norm else None,
+                              biases=bs if bias else None, layout=0)
     dev_w = [f.array(orc.to_canonical(q) if layout == 1 else q.reshape(-1)) for q, _ in q8]
     dev_s = [f.array(s) for _, s in q8]
     dx, dg = f.array(x), f.array(g)
@@ -279,7 +288,7 @@ def test_fused_qkv_q8_equals_oracle(K, N, NK, m, norm, bias, layout):
             f.fused_qkv(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), outs[0].arg(), outs[1].arg(), outs[2].arg(),
                         K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout,
                         scales=[s.arg() for s in dev_s])
-            for o, w, name in zip(outs, want, "qkv"):
+            for o, w, name in zip(outs, want_gemm if _gemm_runs(m, min_m) else want_stream, "qkv"):
                 got = o.download()
                 assert np.all(np.isfinite(got)), (name, min_m, variant)
                 assert _close(got, w, K), (name, min_m, variant, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
@@ -306,7 +315,8 @@ def test_matmul_q8_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta):
     w8, sc = orc.quantize_q8_0(rng.uniform(-0.1, 0.1, (n, k)).astype(np.float16))
     b = rng.uniform(-0.1, 0.1, n).astype(np.float16)
     c = rng.uniform(-1, 1, (m, n)).astype(np.float16)
-    want = orc.matmul_gemv_q8(x, w8, sc, b if bias else None, c if resid else None, 0, 32, alpha, beta)
+    want_stream = orc.matmul_gemv_q8(x, w8, sc, b if bias else None, c if resid else None, 0, 32, alpha, beta)
+    want_gemm = orc.matmul_gemv(x, orc.dequantize_blocks(w8, sc), b if bias else None, c if resid else None, 0, 32, alpha, beta)
     dx, dw, ds = f.array(x), f.array(orc.to_canonical(w8) if canonical else w8.reshape(-1)), f.array(sc)
     db, dc, out = f.array(b), f.array(c), f.zeros((m, n))
     try:
@@ -316,7 +326,7 @@ def test_matmul_q8_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta):
             out.upload(np.zeros((m, n), np.float16))
             f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, bias=db.arg() if bias else None, c=dc.arg() if resid else None,
                      transpose_b=not canonical, alpha=alpha, beta=beta, b_scales=ds.arg())
-            g, wv = out.download().astype(np.float64), want.astype(np.float64)
+            g, wv = out.download().astype(np.float64), (want_gemm if _gemm_runs(m, min_m) else want_stream).astype(np.float64)
             assert np.all(np.abs(g - wv) <= 2 * np.maximum(np.abs(wv), 2.0 ** -10) * 2.0 ** -10 + 1e-4), (min_m, variant, float(np.max(np.abs(g - wv))))
     finally:
         f.set_gemm_min_m()
@@ -351,8 +361,10 @@ def test_fused_qkv_q4_0_equals_oracle(K, N, NK, m, norm, bias, layout):
     x, g, ws, bs = _data(rng, K, N, NK, m)
     q4 = [orc.quantize_q4_0(w) for w in ws]
     packed = [orc.pack_q4_0(orc.to_canonical(q) if layout == 1 else q.reshape(-1)) for q, _ in q4]
-    want = orc.fused_qkv_q8(x, [orc.unpack_q4_0(p) for p in packed], [s for _, s in q4], gamma=g if norm else None,
-                            biases=bs if bias else None, layout=layout)
+    want_stream = orc.fused_qkv_q8(x, [orc.unpack_q4_0(p) for p in packed], [s for _, s in q4], gamma=g if norm else None,
+                                   biases=bs if bias else None, layout=layout)
+    want_gemm = orc.fused_qkv(x, *[orc.dequantize_blocks(q, s) for q, s in q4], gamma=g if norm else None,
+                              biases=bs if bias else None, layout=0)
     dev_w = [f.array(p) for p in packed]
     dev_s = [f.array(s) for _, s in q4]
     dx, dg = f.array(x), f.array(g)
@@ -368,7 +380,7 @@ def test_fused_qkv_q4_0_equals_oracle(K, N, NK, m, norm, bias, layout):
             f.fused_qkv(dx.arg(), wargs[0], wargs[1], wargs[2], outs[0].arg(), outs[1].arg(), outs[2].arg(),
                         K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout,
                         scales=[s.arg() for s in dev_s])
-            for o, w, name in zip(outs, want, "qkv"):
+            for o, w, name in zip(outs, want_gemm if _gemm_runs(m, min_m) else want_stream, "qkv"):
                 got = o.download()
                 assert np.all(np.isfinite(got)), (name, min_m, variant)
                 assert _close(got, w, K), (name, min_m, variant, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
@@ -395,8 +407,11 @@ def test_matmul_q4_0_equals_oracle(m, n, k, canonical, bias, resid, alpha, beta)
     b = rng.uniform(-0.1, 0.1, n).astype(np.float16)
     c = rng.uniform(-1, 1, (m, n)).astype(np.float16)
     packed = orc.pack_q4_0(orc.to_canonical(q) if canonical else q.reshape(-1))
-    want = orc.matmul_gemv_q8(x, orc.unpack_q4_0(packed), sc, b if bias else None, c if resid else None, 1 if canonical else 0,
-                              32, alpha, beta)
+    if m >= 12:  # the GEMM's arithmetic
+        want = orc.matmul_gemv(x, orc.dequantize_blocks(q, sc), b if bias else None, c if resid else None, 0, 32, alpha, beta)
+    else:
+        want = orc.matmul_gemv_q8(x, orc.unpack_q4_0(packed), sc, b if bias else None, c if resid else None,
+                                  1 if canonical else 0, 32, alpha, beta)
     dx, dw, ds = f.array(x), f.array(packed), f.array(sc)
     db, dc, out = f.array(b), f.array(c), f.zeros((m, n))
     f.matmul(dx.arg(), dw.arg(dims=(n, k), dtype=fa.DTYPE_Q4_0), out.arg(), m, n, k, bias=db.arg() if bias else None,

@@ -735,3 +735,19 @@ def test_q4_0_quantiser_and_dot_against_float64():
         got = orc.matmul_gemv_q8(x, orc.unpack_q4_0(orc.pack_q4_0(stored)), sc, layout=layout)
         want = x.astype(np.float64) @ deq.reshape(n, k).T
         assert np.max(np.abs(got.astype(np.float64) - want)) <= 2.0 ** -10 * np.maximum(np.abs(want), 2.0 ** -10).max() + 1e-5
+
+
+def test_dequantize_blocks_is_one_rounding_of_the_exact_product():
+    """The GEMM form of block-quantised weights (src/metals/mma/tile_loader.metal:100-120; CPU reference of
+    tests/gemm_v2_parity.rs:295-350): w = f16(q * scale). q * scale is exact in f32 and f64, so the f32 route of
+    orc.dequantize_blocks must equal the float64 product rounded once - for Q8_0 and Q4_0 integers, subnormal scales
+    included."""
+    rng = np.random.default_rng(43)
+    n, k = 8, 128
+    for lo, hi in ((-127, 128), (-8, 8)):
+        q = rng.integers(lo, hi, (n, k)).astype(np.int8)
+        sc = rng.uniform(0, 0.02, (n, k // 32)).astype(np.float16)
+        sc[0, 0], sc[1, 1], sc[2, 2] = np.float16(6e-8), np.float16(3e-5), np.float16(0)  # subnormal, near the normal edge, zero
+        got = orc.dequantize_blocks(q, sc)
+        want = (q.astype(np.float64).reshape(n, k // 32, 32) * sc.astype(np.float64)[:, :, None]).reshape(n, k).astype(np.float16)
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
