@@ -464,8 +464,8 @@ def bench_fused_qkv_chunk(f, args, m, q8=False):
     step(0)
     f.synchronize()
     rows = min(m, 64)  # the oracle on the first rows (seconds of CPU time at most)
-    if q8:
-        want = orc.fused_qkv_q8(x[:rows], [w for w, _ in host0], [sc for _, sc in host0], gamma=g)
+    if q8:  # the GEMM's arithmetic for block-quantised weights: f16(q * scale), then the F16 product
+        want = orc.fused_qkv(x[:rows], *[orc.dequantize_blocks(w, sc) for w, sc in host0], gamma=g)
     else:
         want = orc.fused_qkv(x[:rows], *host0, gamma=g)
     err = max(float(np.max(np.abs(o.download()[:rows].astype(np.float64) - w.astype(np.float64)))) for o, w in zip((oq, ok, ov), want))
