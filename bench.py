@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload llama3b_decode_8k|...]
 
-Default workload = BASELINE config 2: Llama-3.2-3B-shaped decode attention, 28 layers, batch 1, 24 query heads,
+Default workload = benchmark configuration 2: Llama-3.2-3B-shaped decode attention, 28 layers, batch 1, 24 query heads,
 8 KV heads, head_dim 128, f16 KV cache at 8192 context (seeded N(0,1)), RoPE theta 5e5 ("normal" pairing), one token
 appended per layer then flash-decode SDPA. A "step" is one decode step = 28 x (fused RoPE + append, flash decode).
 Inputs are resident in HBM before the timed region. The K steps are recorded into HIP graphs of 16 steps each

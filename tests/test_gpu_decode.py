@@ -30,8 +30,8 @@ def gpu_decode(q, k, v, H, D, N, causal=True, query_offset=None, q_arg_dims=None
 
 
 @pytest.mark.parametrize("H,Hkv,D,N,cap", [
-    (14, 2, 64, 1025, 1152),    # BASELINE config 1 (Qwen2.5-0.5B shape)
-    (24, 8, 128, 8193, 8448),   # BASELINE config 2 (Llama-3.2-3B shape, one layer)
+    (14, 2, 64, 1025, 1152),    # benchmark configuration 1 (Qwen2.5-0.5B shape)
+    (24, 8, 128, 8193, 8448),   # benchmark configuration 2 (Llama-3.2-3B shape, one layer)
     (16, 2, 128, 3000, 3008),   # Qwen2.5-3B shape
     (16, 4, 128, 5000, 5120),   # SmolLM3 shape
     (32, 8, 128, 777, 1024),

@@ -11,7 +11,7 @@ pytestmark = pytest.mark.gpu
 
 SHAPES = [  # (seq, pos, cap, H, Hkv, D): first three are tests/kv_prep_fused.rs:249-267
     (1, 5, 16, 14, 2, 64), (4, 0, 16, 14, 2, 64), (2, 0, 64, 32, 8, 128),
-    (1, 1024, 1152, 14, 2, 64),      # Qwen2.5-0.5B decode step of BASELINE config 1
+    (1, 1024, 1152, 14, 2, 64),      # Qwen2.5-0.5B decode step of benchmark configuration 1
     (1, 8192, 8448, 24, 8, 128),     # Llama-3.2-3B decode step
     (33, 100, 256, 24, 8, 128), (7, 3, 32, 16, 4, 128), (5, 0, 8, 16, 2, 128),
 ]

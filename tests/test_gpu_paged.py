@@ -51,7 +51,7 @@ class Paged:
 
 
 @pytest.mark.parametrize("H,Hkv,D,bs,lens", [
-    (16, 2, 128, 16, [512, 777, 16, 1, 4095, 1000, 33, 2049]),   # Qwen2.5-3B shape (BASELINE config 3), ragged
+    (16, 2, 128, 16, [512, 777, 16, 1, 4095, 1000, 33, 2049]),   # Qwen2.5-3B shape (benchmark configuration 3), ragged
     (14, 2, 64, 16, [100, 5, 64]),
     (24, 8, 128, 32, [300, 31]),
     (8, 8, 64, 64, [129]),

@@ -117,7 +117,7 @@ def test_prefill_rows_equal_decode_and_first_row():
 
 
 def test_prefill_llama_shape_full_size_from_paged_cache():
-    """BASELINE config 4: 2048-token prompt, H24/Hkv8/D128, RoPE theta 5e5 on positions 0..2047, all rows
+    """benchmark configuration 4: 2048-token prompt, H24/Hkv8/D128, RoPE theta 5e5 on positions 0..2047, all rows
     appended into an empty paged cache, causal flash attention reading through the block table."""
     announce("prefill C4 full size")
     f = ctx()
