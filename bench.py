@@ -856,6 +856,7 @@ SECONDARY = {"llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": be
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
              "llama3b_o_proj": bench_o_proj,
              "llama3b_fused_qkv_chunk32": lambda f, args: bench_fused_qkv_chunk(f, args, 32),
+             "llama3b_fused_qkv_chunk512": lambda f, args: bench_fused_qkv_chunk(f, args, 512),
              "llama3b_fused_qkv_prefill_2k": lambda f, args: bench_fused_qkv_chunk(f, args, 2048),
              "llama3b_fused_qkv_q8_chunk32": lambda f, args: bench_fused_qkv_chunk(f, args, 32, q8=True),
              "llama3b_fused_qkv_q8_prefill_2k": lambda f, args: bench_fused_qkv_chunk(f, args, 2048, q8=True),
