@@ -6,17 +6,20 @@
 // 2 * m * n * k flops on m * k + n * k operands, so it runs as a GEMM:
 //   * a workgroup (4 waves) owns a 128 (weight rows) x 128 (input rows) output tile; a wave owns 64 x 64 of it as
 //     2 x 2 v_mfma_f32_32x32x16_f16 tiles (64 accumulator registers);
-//   * both operands move through LDS in steps of 64 features, two stages: the next step's 16-byte pieces are
-//     requested into registers before this step's matrix work and written after it, one barrier per step;
-//   * LDS layout per stage and operand: [16-byte piece of the 64 features][row], piece stride padded so that the
-//     writes (the global load's lane order) and the operand reads (32 consecutive rows per half wave) are both free of
-//     bank conflicts; the blocked ("canonical") weight layout is one contiguous 8 KiB per (tile, 32 features);
+//   * both operands move through LDS in steps of 64 (or 32) features, two stages, one barrier per step. Three
+//     kernels differ in how the tiles get there: through registers (qkv_gemm_kernel: any shape, and block-quantised
+//     weights, which become f16 on the way), or from memory straight into LDS (qkv_gemm_dma_kernel, 64 features per
+//     step, two workgroups per CU; qkv_gemm_dma32_kernel, 32 features, four per CU) - see the notes at each;
+//   * LDS layouts are chosen per kernel so that writes (served 8 lanes at a time) and operand reads (16 lanes at a
+//     time) are free of bank conflicts; the blocked ("canonical") weight layout is one contiguous 8 KiB per (tile, 32
+//     features);
 //   * the rows of W_q, W_k, W_v are tiled per matrix (a tile never straddles two); the workgroups of one XCD take
 //     consecutive tiles of the weight rows over all input rows, so a weight tile is fetched into one L2 only;
 //   * epilogue: accumulators to LDS as f32 [input row][weight row], then alpha * sum + bias + beta * residual, one
 //     rounding to f16 (as the GEMV path), 16-byte token-major stores.
 // RMSNorm: a small kernel in front writes the normalised input, rounded to f16 as qkv_project.metal:66-67 does, into
-// the context's workspace; the GEMM reads that.
+// the context's workspace; the GEMM reads that. Launches with few output tiles divide a tile's feature steps over
+// several workgroups (split-K: f32 partial tiles in the workspace, added in split order by gemm_finish_kernel).
 #include "fa_internal.h"
 #include <type_traits>
 
