@@ -786,11 +786,14 @@ fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
     const uint64_t n_wg = (uint64_t)a.n_tiles * a.m_tiles;
     if (n_wg > 0x7fffffffull) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %llu output tiles", (unsigned long long)n_wg);
     // Few output tiles (a short prefill chunk): the feature steps of a tile are divided over enough workgroups to
-    // give every CU a share of the weight stream, at least 4 steps each (a 32-row chunk of Llama-3.2-3B: 47.5 us
-    // unsplit, 19.2 us with the 48 steps over 6 to 12 workgroups per tile; 512 rows: 52.9 -> 38.8 us with 3).
+    // give every CU a share of the weight stream, at least 4 steps each (a 32-row chunk of Llama-3.2-3B: 36.9 us
+    // unsplit, 17.4 us with the 48 steps over 12 workgroups per tile; 512 rows: 42.9 -> 35.9 us with 3).
     const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
     const uint32_t all_steps = ceil_div_u32(l.k_dim, GM_BK);
-    const uint32_t target = 2 * n_cus;  // two workgroups are resident per CU
+    // Two workgroups per CU as the target. With the weights still in the last-level cache from the previous call (one
+    // layer in a loop) 1.5 per CU measures faster (256 rows: 26.7 us against 31.4), but with each call's weights coming
+    // from memory, as in a model, 2 per CU wins: 512 rows 26.5 + 6.2 us (GEMM + finish) against 32.0 + 5.0.
+    const uint32_t target = 2 * n_cus;
     uint32_t splits = (uint32_t)(target / n_wg);
     if (splits > all_steps / 4) splits = all_steps / 4;
     if (splits < 1) splits = 1;
