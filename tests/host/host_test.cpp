@@ -419,16 +419,17 @@ static void test_session_prefill_chunks_decode_loop_growth_snapshot(Foundry &fou
 
 // tests/qkv_parity_f16.rs:88-339: the fused QKV step at K 1024, N 1024, N_kv 128 with RMSNorm and biases against the
 // test's CPU helpers (here: the oracle's transcription of them), and the canonical weight layout the models use.
-static void test_fused_qkv_step(Foundry &foundry, WeightLayout layout) {
+// m = 1: the weight-stream kernel (a decode step); m = 32: a prefill chunk, which the library runs as a GEMM.
+static void test_fused_qkv_step(Foundry &foundry, WeightLayout layout, size_t m = 1) {
     const size_t K = 1024, N = 1024, NKV = 128;
     Rng rng{2024};
-    auto x = rng.fill(K, 1.0f), gamma = rng.fill(K, 0.5f);
+    auto x = rng.fill(m * K, 1.0f), gamma = rng.fill(K, 0.5f);
     for (auto &g : gamma) g = orc_f32_to_f16(orc_f16_to_f32(g) + 1.0f);  // 0.5 .. 1.5
     auto wq = rng.fill(N * K, 0.1f), wk = rng.fill(NKV * K, 0.1f), wv = rng.fill(NKV * K, 0.1f);
     auto bq = rng.fill(N, 0.1f), bk = rng.fill(NKV, 0.1f), bv = rng.fill(NKV, 0.1f);
-    std::vector<orc_f16> want_q(N), want_k(NKV), want_v(NKV);
+    std::vector<orc_f16> want_q(m * N), want_k(m * NKV), want_v(m * NKV);
     orc_fused_qkv(x.data(), wq.data(), wk.data(), wv.data(), gamma.data(), bq.data(), bk.data(), bv.data(), want_q.data(), want_k.data(),
-                  want_v.data(), (uint32_t)K, (uint32_t)N, (uint32_t)NKV, 1, 0, 32, 1e-6f, 4);
+                  want_v.data(), (uint32_t)K, (uint32_t)N, (uint32_t)NKV, (uint32_t)m, 0, 32, 1e-6f, 4);
     auto arrange = [&](const std::vector<orc_f16> &w, size_t rows) {
         if (layout == WeightLayout::RowMajor) return w;
         std::vector<orc_f16> c(w.size());
@@ -438,7 +439,7 @@ static void test_fused_qkv_step(Foundry &foundry, WeightLayout layout) {
     };
     TensorBindings b;
     b.set_int_global("i", 3);
-    b.insert("hidden", foundry.from_host(Dtype::F16, {1, K}, x.data()));
+    b.insert("hidden", foundry.from_host(Dtype::F16, {m, K}, x.data()));
     b.insert("layer.attn_norm_3", foundry.from_host(Dtype::F16, {K}, gamma.data()));
     b.insert("layer.wq_3", foundry.from_host(Dtype::F16, {N * K}, arrange(wq, N).data()));
     b.insert("layer.wk_3", foundry.from_host(Dtype::F16, {NKV * K}, arrange(wk, NKV).data()));
@@ -446,16 +447,16 @@ static void test_fused_qkv_step(Foundry &foundry, WeightLayout layout) {
     b.insert("layer.bq_3", foundry.from_host(Dtype::F16, {N}, bq.data()));
     b.insert("layer.bk_3", foundry.from_host(Dtype::F16, {NKV}, bk.data()));
     b.insert("layer.bv_3", foundry.from_host(Dtype::F16, {NKV}, bv.data()));
-    b.insert("q", foundry.zeros(Dtype::F16, {1, N}));
-    b.insert("k", foundry.zeros(Dtype::F16, {1, NKV}));
-    b.insert("v", foundry.zeros(Dtype::F16, {1, NKV}));
+    b.insert("q", foundry.zeros(Dtype::F16, {m, N}));
+    b.insert("k", foundry.zeros(Dtype::F16, {m, NKV}));
+    b.insert("v", foundry.zeros(Dtype::F16, {m, NKV}));
     FusedQkvStep step{"hidden", "layer.wq_{i}", "layer.wk_{i}", "layer.wv_{i}", "q", "k", "v"};
     step.gamma = "layer.attn_norm_{i}", step.bias_q = "layer.bq_{i}", step.bias_k = "layer.bk_{i}", step.bias_v = "layer.bv_{i}";
-    step.k_dim = (uint32_t)K, step.n_dim = (uint32_t)N, step.n_kv = (uint32_t)NKV, step.m = 0 /* treated as 1 */, step.layout = layout;
+    step.k_dim = (uint32_t)K, step.n_dim = (uint32_t)N, step.n_kv = (uint32_t)NKV, step.m = m == 1 ? 0 /* treated as 1 */ : (uint32_t)m, step.layout = layout;
     step.execute(foundry, b);
     foundry.synchronize();
     auto q = foundry.to_host<orc_f16>(*b.get("q")), k = foundry.to_host<orc_f16>(*b.get("k")), v = foundry.to_host<orc_f16>(*b.get("v"));
-    EXPECT(max_abs_diff(want_q, q, N) <= 8e-3f && max_abs_diff(want_k, k, NKV) <= 8e-3f && max_abs_diff(want_v, v, NKV) <= 8e-3f);
+    EXPECT(max_abs_diff(want_q, q, m * N) <= 8e-3f && max_abs_diff(want_k, k, m * NKV) <= 8e-3f && max_abs_diff(want_v, v, m * NKV) <= 8e-3f);
     FusedQkvStep missing = step;
     missing.bias_k = "not_bound";
     EXPECT(thrown_by([&] { missing.execute(foundry, b); }) == MetalError::InputNotFound);
@@ -514,6 +515,7 @@ int main(int argc, char **argv) {
         run_test("error variants", [&] { test_error_variants(foundry); });
         run_test("fused qkv step, row-major weights", [&] { test_fused_qkv_step(foundry, WeightLayout::RowMajor); });
         run_test("fused qkv step, canonical weights", [&] { test_fused_qkv_step(foundry, WeightLayout::Canonical); });
+        run_test("fused qkv step on a 32-token chunk (GEMM)", [&] { test_fused_qkv_step(foundry, WeightLayout::Canonical, 32); });
         run_test("matmul step as o_proj with residual", [&] { test_matmul_step_o_proj(foundry); });
         run_test("session: chunked prefill, snapshot, decode loop with growth, restore",
                  [&] { test_session_prefill_chunks_decode_loop_growth_snapshot(foundry); });
