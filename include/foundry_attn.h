@@ -433,8 +433,7 @@ fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b,
  * Environment: FOUNDRY_ATTN_GEMM_MIN_M (read at fa_ctx_create). */
 fa_status fa_set_gemm_min_m(fa_ctx *ctx, uint32_t min_m);
 
-/* Which GEMM kernel fa_fused_qkv / fa_matmul use (same tiling and arithmetic; results equal up to the f32 summation
- * order of the split-K partials, which does not depend on the kernel): 1 = operand tiles staged through registers (any
+/* Which GEMM kernel fa_fused_qkv / fa_matmul use (same tiling, step order and split points: bit-equal results): 1 = operand tiles staged through registers (any
  * shape, every weight policy); 2 = tiles loaded from memory straight into LDS in steps of 64 features, two workgroups
  * per compute unit; 3 = the same in steps of 32 features, four workgroups per compute unit; 0 (default) = 2 or 3 by
  * the number of output tiles. 2 and 3 need F16 weights, k_dim a multiple of 64 and operands below 2 GiB, and fall back

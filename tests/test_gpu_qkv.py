@@ -84,6 +84,7 @@ def test_fused_qkv_equals_oracle(K, N, NK, m, norm, bias, layout):
     outs = [f.zeros((m, n)) for n in (N, NK, NK)]
     # from 12 input rows on the library runs the GEMM; short chunks are also forced through the passes of 16 rows over
     # the weight stream, and shapes of a few rows through the GEMM
+    gemm_bits = None  # the GEMM kernels share tiling, step order and split points: their outputs are bit-equal
     try:
         for min_m, variant in _paths(m):
             f.set_gemm_min_m(min_m)
@@ -92,10 +93,16 @@ def test_fused_qkv_equals_oracle(K, N, NK, m, norm, bias, layout):
                 o.upload(np.zeros(o.shape, np.float16))
             f.fused_qkv(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), outs[0].arg(), outs[1].arg(), outs[2].arg(),
                         K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout)
-            for o, w, name in zip(outs, want, "qkv"):
-                got = o.download()
+            got_all = [o.download() for o in outs]
+            for got, w, name in zip(got_all, want, "qkv"):
                 assert np.all(np.isfinite(got)), (name, min_m, variant)
                 assert _close(got, w, K), (name, min_m, variant, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
+            if _gemm_runs(m, min_m):
+                bits_now = [g.view(np.uint16).copy() for g in got_all]
+                if gemm_bits is None:
+                    gemm_bits = bits_now
+                else:
+                    assert all(np.array_equal(a, b) for a, b in zip(gemm_bits, bits_now)), (min_m, variant)
     finally:
         f.set_gemm_min_m()
         f.set_gemm_variant()
