@@ -56,7 +56,10 @@ inline void check(fa_status s) {
 }
 
 // ---------------------------------------------------------------------------------------------- tensors
-enum class Dtype : uint32_t { F32 = FA_DTYPE_F32, F16 = FA_DTYPE_F16, BF16 = FA_DTYPE_BF16, I8 = FA_DTYPE_I8, I32 = FA_DTYPE_I32, U32 = FA_DTYPE_U32 };
+// Q8_0 tensors hold one int8 per weight. Q4_0 (two weights per byte) has no whole-byte element size and is not mirrored
+// here: it is reached through the C ABI directly (a fa_tensor_arg with dtype FA_DTYPE_Q4_0 over the packed bytes).
+enum class Dtype : uint32_t { F32 = FA_DTYPE_F32, F16 = FA_DTYPE_F16, BF16 = FA_DTYPE_BF16, Q8_0 = FA_DTYPE_Q8_0, I8 = FA_DTYPE_I8,
+                              I32 = FA_DTYPE_I32, U8 = FA_DTYPE_U8, U32 = FA_DTYPE_U32 };
 
 inline size_t dtype_size(Dtype d) {
     switch (d) {
