@@ -85,12 +85,19 @@ typedef struct fa_graph fa_graph;
 /* Foundry::new (src/lib.rs:57-61). Creates a stream on `device` and a 64 MiB scratch workspace. */
 fa_status fa_ctx_create(int device, fa_ctx **out);
 fa_status fa_ctx_destroy(fa_ctx *ctx);
-/* Foundry::synchronize (src/lib.rs:175-188). */
+/* Foundry::synchronize (src/lib.rs:175-188). Also reports what kernels flagged since the last call: a fused decode
+ * step whose device-side position was at or beyond its kv_len_bound or the cache capacity (the token was neither
+ * appended nor attended) -> FA_ERR_INVALID_OPERATION, once. Not callable during a capture; the same holds for the
+ * other calls that wait for the stream (fa_upload, fa_download, fa_device_free, fa_profile_reset, fa_profile_query):
+ * FA_ERR_OPERATION_FAILED, and the capture stays valid. */
 fa_status fa_synchronize(fa_ctx *ctx);
 /* The context's hipStream_t, for callers that enqueue their own work between the ops. */
 void *fa_ctx_stream(fa_ctx *ctx);
 /* Grows the scratch workspace to at least `bytes`. Must be called outside a capture; ops that need
- * more scratch than is reserved while capturing fail with FA_ERR_OPERATION_FAILED. */
+ * more scratch than is reserved while capturing fail with FA_ERR_OPERATION_FAILED. A recorded graph holds the
+ * address of the workspace it was captured against: when the workspace is outgrown later (by this call or by an
+ * eager op), the old buffer is kept alive until the last graph of the context is destroyed (or the context is), so
+ * replaying an older graph stays valid. */
 fa_status fa_ctx_reserve_workspace(fa_ctx *ctx, size_t bytes);
 
 /* Foundry::start_capture / end_capture (src/lib.rs:94-164). The reference batches dispatches into one
@@ -214,7 +221,9 @@ fa_status fa_flash_decode_dyn(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tens
  * row P of the caches and attended together with rows [0, P), where P = *d_position if d_position != NULL,
  * else params->position_offset. The cache rows and q_rot carry the same bits as after calling the two ops one
  * after the other and the attention reads the same f16 values (outputs agree up to f32 summation order). q_rot may have a NULL buffer
- * (then it is not written). kv_len_bound >= P + 1 as in fa_flash_decode_dyn. params->seq_len must be 1. */
+ * (then it is not written). kv_len_bound >= P + 1 as in fa_flash_decode_dyn; if a replayed graph's device position
+ * reaches P + 1 > min(kv_len_bound, capacity) the token is dropped (not appended, not attended) and the next
+ * fa_synchronize fails with FA_ERR_INVALID_OPERATION. params->seq_len must be 1. */
 fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
                                const fa_tensor_arg *q_rot, const fa_tensor_arg *k_cache,
                                const fa_tensor_arg *v_cache, const fa_tensor_arg *cos, const fa_tensor_arg *sin,

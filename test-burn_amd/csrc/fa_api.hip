@@ -110,8 +110,18 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     ctx->prefill_split_k = env_u32("FOUNDRY_ATTN_PREFILL_SPLIT_K", 0);
     ctx->prefill_variant = env_u32("FOUNDRY_ATTN_PREFILL_VARIANT", 0);
     if (ctx->prefill_variant > 2) ctx->prefill_variant = 0;
+    ctx->ledger = new FaGraphLedger();
     fa_status s = fa_ensure_workspace(ctx, (size_t)64 << 20);
     if (s == FA_OK) s = fa_ensure_counters(ctx, 4096);
+    if (s == FA_OK) {
+        // one word that kernels set bits in and the host reads after a synchronize: pinned host memory mapped into the device
+        hipError_t he = hipHostMalloc((void **)&ctx->h_status, sizeof(uint32_t), hipHostMallocMapped);
+        if (he == hipSuccess) {
+            *ctx->h_status = 0;
+            he = hipHostGetDevicePointer((void **)&ctx->d_status, ctx->h_status, 0);
+        }
+        if (he != hipSuccess) s = fa_fail(FA_ERR_OPERATION_FAILED, "status word allocation failed: %s", hipGetErrorString(he));
+    }
     if (s != FA_OK) {
         fa_ctx_destroy(ctx);
         return s;
@@ -131,6 +141,14 @@ extern "C" fa_status fa_ctx_destroy(fa_ctx *ctx) {
     for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->counters) (void)hipFree(ctx->counters);
+    if (ctx->h_status) (void)hipHostFree(ctx->h_status);
+    if (ctx->ledger) {
+        // graphs that outlive the context can no longer be launched (fa_graph_launch needs it); what they address goes now
+        for (void *p : ctx->ledger->retired) (void)hipFree(p);
+        ctx->ledger->retired.clear();
+        ctx->ledger->ctx_alive = false;
+        if (ctx->ledger->live_graphs == 0) delete ctx->ledger;
+    }
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return FA_OK;
@@ -142,6 +160,27 @@ extern "C" fa_status fa_synchronize(fa_ctx *ctx) {
     FA_NEED(ctx, "ctx");
     if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "cannot synchronize while a capture is active");
     FA_HIP(hipStreamSynchronize(ctx->stream));
+    if (ctx->h_status && *ctx->h_status) {
+        const uint32_t bits = *ctx->h_status;
+        *ctx->h_status = 0;
+        if (bits & FA_DEVSTAT_APPEND_DROPPED)
+            return fa_fail(FA_ERR_INVALID_OPERATION,
+                           "Invalid operation: a fused decode step ran at a position at or beyond its kv_len_bound or the cache "
+                           "capacity; its token was neither appended nor attended");
+        return fa_fail(FA_ERR_OPERATION_FAILED, "device status word 0x%x", bits);
+    }
+    return FA_OK;
+}
+
+// A buffer whose address may be baked into the kernel arguments of a recorded graph is parked while any graph of this
+// context is alive, and freed otherwise.
+static fa_status retire_or_free(fa_ctx *ctx, void *p) {
+    if (!p) return FA_OK;
+    if (ctx->ledger && ctx->ledger->live_graphs > 0) {
+        ctx->ledger->retired.push_back(p);
+        return FA_OK;
+    }
+    FA_HIP(hipFree(p));
     return FA_OK;
 }
 
@@ -153,7 +192,7 @@ fa_status fa_ensure_workspace(fa_ctx *ctx, size_t bytes) {
                        "fa_ctx_reserve_workspace before fa_start_capture",
                        bytes, ctx->workspace_bytes);
     FA_HIP(hipStreamSynchronize(ctx->stream));
-    if (ctx->workspace) FA_HIP(hipFree(ctx->workspace));
+    FA_TRY(retire_or_free(ctx, ctx->workspace));
     ctx->workspace = nullptr;
     ctx->workspace_bytes = 0;
     size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
@@ -168,7 +207,7 @@ fa_status fa_ensure_counters(fa_ctx *ctx, uint32_t n) {
         return fa_fail(FA_ERR_OPERATION_FAILED, "%u split counters needed during capture but only %u exist", n,
                        ctx->n_counters);
     FA_HIP(hipStreamSynchronize(ctx->stream));
-    if (ctx->counters) FA_HIP(hipFree(ctx->counters));
+    FA_TRY(retire_or_free(ctx, ctx->counters));
     ctx->counters = nullptr;
     ctx->n_counters = 0;
     uint32_t want = (n + 4095u) & ~4095u;
@@ -251,6 +290,8 @@ extern "C" fa_status fa_end_capture(fa_ctx *ctx, fa_graph **out) {
     fa_graph *gr = new fa_graph();
     gr->graph = g;
     gr->exec = ex;
+    gr->ledger = ctx->ledger;
+    ++ctx->ledger->live_graphs;
     *out = gr;
     return FA_OK;
 }
@@ -267,6 +308,14 @@ extern "C" fa_status fa_graph_destroy(fa_graph *graph) {
     if (!graph) return FA_OK;
     if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
     if (graph->graph) (void)hipGraphDestroy(graph->graph);
+    if (FaGraphLedger *lg = graph->ledger) {
+        if (--lg->live_graphs == 0) {
+            // hipFree waits for the device, so a replay still in flight has finished with these buffers
+            for (void *p : lg->retired) (void)hipFree(p);
+            lg->retired.clear();
+            if (!lg->ctx_alive) delete lg;
+        }
+    }
     delete graph;
     return FA_OK;
 }
@@ -290,6 +339,7 @@ extern "C" fa_status fa_profile_enable(fa_ctx *ctx, int on) {
 
 extern "C" fa_status fa_profile_reset(fa_ctx *ctx) {
     FA_NEED(ctx, "ctx");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "fa_profile_reset waits for the stream and cannot run while a capture is active");
     FA_HIP(hipStreamSynchronize(ctx->stream));
     prof_recycle(ctx);
     return FA_OK;
@@ -297,6 +347,7 @@ extern "C" fa_status fa_profile_reset(fa_ctx *ctx) {
 
 extern "C" fa_status fa_profile_query(fa_ctx *ctx, const char *prefix, uint64_t *launches, double *total_ms) {
     FA_NEED(ctx, "ctx");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "fa_profile_query waits for the stream and cannot run while a capture is active");
     FA_NEED(prefix, "kernel_prefix");
     FA_HIP(hipStreamSynchronize(ctx->stream));
     uint64_t n = 0;
@@ -328,6 +379,7 @@ extern "C" fa_status fa_device_alloc(fa_ctx *ctx, size_t bytes, void **out) {
 
 extern "C" fa_status fa_device_free(fa_ctx *ctx, void *ptr) {
     FA_NEED(ctx, "ctx");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "fa_device_free waits for the stream and cannot run while a capture is active");
     if (!ptr) return FA_OK;
     FA_HIP(hipStreamSynchronize(ctx->stream));
     FA_HIP(hipFree(ptr));
@@ -336,6 +388,7 @@ extern "C" fa_status fa_device_free(fa_ctx *ctx, void *ptr) {
 
 extern "C" fa_status fa_upload(fa_ctx *ctx, void *dst, size_t dst_offset, const void *src_host, size_t bytes) {
     FA_NEED(ctx, "ctx");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "fa_upload waits for the stream and cannot run while a capture is active");
     FA_NEED(dst, "dst");
     FA_NEED(src_host, "src_host");
     if (bytes == 0) return FA_OK;
@@ -346,6 +399,7 @@ extern "C" fa_status fa_upload(fa_ctx *ctx, void *dst, size_t dst_offset, const 
 
 extern "C" fa_status fa_download(fa_ctx *ctx, void *dst_host, const void *src, size_t src_offset, size_t bytes) {
     FA_NEED(ctx, "ctx");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "fa_download waits for the stream and cannot run while a capture is active");
     FA_NEED(dst_host, "dst_host");
     FA_NEED(src, "src");
     if (bytes == 0) return FA_OK;
@@ -1116,12 +1170,12 @@ static fa_status fused_common(const fa_tensor_arg *q, const fa_tensor_arg *k, co
     return FA_OK;
 }
 
-extern "C" fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
-                                          const fa_tensor_arg *v, const fa_tensor_arg *q_rot,
-                                          const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
-                                          const fa_tensor_arg *cos, const fa_tensor_arg *sin,
-                                          const fa_tensor_arg *output, const fa_kv_prep_fused_params *p,
-                                          const uint32_t *d_position, uint32_t kv_len_bound) {
+static fa_status decode_step_fused_impl(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                        const fa_tensor_arg *v, const fa_tensor_arg *q_rot,
+                                        const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
+                                        const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                        const fa_tensor_arg *output, const fa_kv_prep_fused_params *p,
+                                        const uint32_t *d_position, uint32_t kv_len_bound) {
     FA_NEED(ctx, "ctx");
     DecodeLaunch L;
     memset(&L, 0, sizeof(L));
@@ -1154,6 +1208,15 @@ extern "C" fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, c
         L.kv_len = p->position_offset + 1, L.kv_len_bound = L.kv_len;
     }
     return fa_launch_decode(ctx, L);
+}
+
+extern "C" fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                          const fa_tensor_arg *v, const fa_tensor_arg *q_rot,
+                                          const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
+                                          const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                          const fa_tensor_arg *output, const fa_kv_prep_fused_params *p,
+                                          const uint32_t *d_position, uint32_t kv_len_bound) {
+    return decode_step_fused_impl(ctx, q, k, v, q_rot, k_cache, v_cache, cos, sin, output, p, d_position, kv_len_bound);
 }
 
 extern "C" fa_status fa_decode_step_fused_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,

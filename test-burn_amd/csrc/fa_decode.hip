@@ -75,6 +75,7 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     a.k_in = L.k_in, a.v_in = L.v_in, a.cos_t = L.cos_t, a.sin_t = L.sin_t, a.q_rot_out = L.q_rot_out;
     a.qin_stride_b = L.qin_stride_b, a.kvin_stride_b = L.kvin_stride_b, a.qrot_stride_b = L.qrot_stride_b;
     a.rope_normal = L.rope_normal, a.apply_rope = L.apply_rope, a.table_rows = L.table_rows;
+    a.status = ctx->d_status;
     if (S > 1) {
         const size_t rows = (size_t)L.batch * ny * S * gt;
         const size_t acc_bytes = rows * L.head_dim * sizeof(float);

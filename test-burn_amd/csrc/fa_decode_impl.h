@@ -544,6 +544,9 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     if (!(FUSED && wave == 0)) n_raw = read_len();
     const uint32_t N = min(n_raw, min(a.capacity, a.kv_len_bound));
     const uint32_t nsplits = (N + a.chunk - 1) / a.chunk;
+    // A position at or past the launch bound / the capacity: the token is neither appended nor attended. The host
+    // finds the bit at its next synchronize.
+    if (FUSED && n_raw > N && tid == 0 && blockIdx.x == 0 && y == 0 && a.status) *a.status = FA_DEVSTAT_APPEND_DROPPED;
     if (split >= nsplits) return;  // uniform over the workgroup
     if (PAGED) {
         // Nothing has been requested yet (a paged cache needs the length first), so the partitions of this
@@ -824,7 +827,8 @@ fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
     const size_t lds = decode_lds_bytes<D>(a.gt);
     {
         // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
-        static bool lds_allowed = false;
+        static bool lds_allowed_on[64] = {};  // per device
+        bool &lds_allowed = lds_allowed_on[ctx->device & 63];
         if (!lds_allowed) {
             const int cap = (int)decode_lds_bytes<D>(MAX_GT);
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));

@@ -811,7 +811,8 @@ fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
         FA_TRY(norm.finish());
         a.x = (const __half *)ctx->workspace;
     }
-    static bool lds_allowed = false;
+    static bool lds_allowed_on[64] = {};  // per device
+    bool &lds_allowed = lds_allowed_on[ctx->device & 63];
     if (!lds_allowed) {
         FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
         FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
@@ -835,7 +836,8 @@ fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
         if (l.canonical) scope.launch(qkv_gemm_dma32_kernel<true>, dim3(grid), dim3(GM_NT), GR_LDS_BYTES, a);
         else scope.launch(qkv_gemm_dma32_kernel<false>, dim3(grid), dim3(GM_NT), GR_LDS_BYTES, a);
     } else if (dma_ok && ctx->gemm_variant != 1) {
-        static bool dma_lds_allowed = false;
+        static bool dma_lds_allowed_on[64] = {};  // per device
+        bool &dma_lds_allowed = dma_lds_allowed_on[ctx->device & 63];
         if (!dma_lds_allowed) {
             FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_dma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
             FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_dma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));

@@ -14,9 +14,18 @@
 
 #include "../../include/foundry_attn.h"
 
+// Shared by a context and the graphs recorded on it: while any graph is alive, scratch buffers whose addresses may be
+// baked into its kernel arguments are retired instead of freed. Outlives whichever of the two is destroyed first.
+struct FaGraphLedger {
+    int live_graphs = 0;
+    bool ctx_alive = true;
+    std::vector<void *> retired;  // outgrown buffers a live graph may still address; freed with the last graph or the context
+};
+
 struct fa_graph {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    FaGraphLedger *ledger = nullptr;
 };
 
 struct FaProfileRec {
@@ -34,6 +43,12 @@ struct fa_ctx {
     // per-(sequence, kv head) arrival counters for the in-kernel split merge; always zero between launches
     uint32_t *counters = nullptr;
     uint32_t n_counters = 0;
+    // Outgrown workspaces / counter arrays that a recorded graph may still reference are parked here: freed once no
+    // graph is alive, or with the context.
+    FaGraphLedger *ledger = nullptr;
+    // Sticky status word written by kernels (pinned host memory, mapped into the device): FA_DEVSTAT_* bits.
+    uint32_t *h_status = nullptr;  // host view
+    uint32_t *d_status = nullptr;  // device view of the same word
     fa_decode_variant decode_variant{0, 1};
     uint32_t decode_waves = 0;     // waves per decode workgroup: 0 = by launch size, 4 or 8
     uint32_t gemm_variant = 0;     // GEMM kernel: 0 = auto, 1 = tiles through registers, 2 / 3 = straight into LDS in steps of 64 / 32 features
@@ -163,6 +178,7 @@ struct FaDecodeDev {
     uint64_t qin_stride_b, kvin_stride_b, qrot_stride_b;
     uint32_t rope_normal, apply_rope, table_rows;
     uint32_t bf16;  // data tensors are bf16 (RoPE tables stay f16)
+    uint32_t *status;  // the context's device-written status word (FA_DEVSTAT_* bits)
 };
 
 
@@ -221,6 +237,9 @@ fa_status fa_launch_sage_quantize_k(fa_ctx *ctx, const void *k, const float *mea
                                     void *k_q, void *k_scale);
 fa_status fa_launch_sage_quantize_q(fa_ctx *ctx, const void *q, uint32_t n_heads, uint32_t head_dim, void *q_q,
                                     float *q_scale);
+
+// Bits of the context's device-written status word
+constexpr uint32_t FA_DEVSTAT_APPEND_DROPPED = 2u; // a fused decode step's position was beyond its launch bound / capacity
 
 fa_status fa_ensure_workspace(fa_ctx *ctx, size_t bytes);
 fa_status fa_ensure_counters(fa_ctx *ctx, uint32_t n);

@@ -359,7 +359,8 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     const uint32_t tiles_per_wg = ceil_div_u32(rows_per_wg, 16);
     const size_t lds = (size_t)cols * a.x_stride + (size_t)QKV_NW * 16 * 17 * sizeof(float) +
                        (q8 ? (size_t)tiles_per_wg * 16 * (l.k_dim / 32) * 2 : 0);
-    static bool lds_allowed = false;
+    static bool lds_allowed_on[64] = {};  // per device
+    bool &lds_allowed = lds_allowed_on[ctx->device & 63];
     if (!lds_allowed) {
         FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)(lds_budget + 16 * 1024)));

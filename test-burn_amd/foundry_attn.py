@@ -358,8 +358,8 @@ class Foundry:
         if q_rot is None:
             q_rot = TensorArg()
         a = [C.byref(x) for x in (q, k, v, q_rot, k_cache, v_cache, cos, sin, out)]
-        check(self.lib.fa_decode_step_fused(self.h, *a, C.byref(params), None if d_position is None else d_position.ptr,
-                                            kv_len_bound))
+        fn = self.lib.fa_decode_step_fused
+        check(fn(self.h, *a, C.byref(params), None if d_position is None else d_position.ptr, kv_len_bound))
 
     def decode_step_fused_paged(self, q, k, v, q_rot, cache, cos, sin, out, params, kv_len_bound):
         if q_rot is None:

@@ -271,10 +271,13 @@ def test_fused_step_errors_and_overflow_guard():
         f.decode_step_fused(q.arg(), k.arg(), v.arg(), None, kc.arg(), vc.arg(), cos.arg(), sin.arg(), out.arg(),
                             fa.KvPrepFusedParams.make(H, Hkv, D, 2, 0, cap))
     assert e.value.variant == "InvalidShape"
-    # a device position beyond the capacity appends nothing
+    # a device position beyond the capacity appends nothing, and the next synchronize reports the dropped token
     dpos = f.array(np.array([cap + 5], np.uint32))
     f.decode_step_fused(q.arg(), k.arg(), v.arg(), None, kc.arg(), vc.arg(), cos.arg(), sin.arg(), out.arg(),
                         fa.KvPrepFusedParams.make(H, Hkv, D, 1, 0, cap), d_position=dpos, kv_len_bound=cap)
+    with pytest.raises(fa.FoundryError) as e:
+        f.synchronize()
+    assert e.value.variant == "InvalidOperation"
     f.synchronize()
     assert not kc.download().any()
 

@@ -77,3 +77,117 @@ def test_per_kernel_profiling_counts_launches():
     finally:
         f.profile_enable(False)
         f.profile_reset()
+
+
+def _split_decode_state(f, rng, H, Hkv, D, cap, start):
+    cos, sin = fa.rope_tables(5e5, D, cap)
+    kc, vc = h16(rng.normal(size=(Hkv, cap, D))), h16(rng.normal(size=(Hkv, cap, D)))
+    q, k, v = (h16(rng.normal(size=(1, n * D))) for n in (H, Hkv, Hkv))
+    dev = dict(cos=f.array(cos), sin=f.array(sin), kc=f.array(kc), vc=f.array(vc), q=f.array(q), k=f.array(k),
+               v=f.array(v), out=f.zeros((1, H * D)), pos=f.array(np.array([start], np.uint32)))
+    return (cos, sin, kc, vc, q, k, v), dev
+
+
+@pytest.mark.parametrize("merge", [1, 0], ids=["merge_kernel", "merge_in_kernel"])
+def test_graph_survives_workspace_growth(merge):
+    """A recorded split decode addresses the workspace (and the arrival counters) it was captured against. Growing the
+    workspace afterwards must leave that buffer alive for the graph: replays before and after the growth equal the
+    oracle, and so does an eager call on the new workspace."""
+    announce("graph replay after the workspace has grown, merge", merge)
+    f = fa.Foundry(0)  # a context of its own: its workspace is the initial 64 MiB
+    rng = np.random.default_rng(81 + merge)
+    H, Hkv, D, cap, start = 24, 8, 128, 4096, 3000
+    (cos, sin, kc, vc, q, k, v), d = _split_decode_state(f, rng, H, Hkv, D, cap, start)
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, 1, 0, cap, fa.ROPE_NORMAL)
+    f.set_decode_variant(0, merge)
+    try:
+        def step():
+            f.decode_step_fused(d["q"].arg(), d["k"].arg(), d["v"].arg(), None, d["kc"].arg(), d["vc"].arg(),
+                                d["cos"].arg(), d["sin"].arg(), d["out"].arg(), p, d_position=d["pos"], kv_len_bound=cap)
+            f.u32_add(d["pos"], 1, 1)
+
+        f.start_capture()
+        step()
+        graph = f.end_capture()
+        ok, ov = kc.copy(), vc.copy()
+
+        def expect(t):
+            qr = orc.kv_prep_fused(q, k, v, ok, ov, cos, sin, orc.make_params(H, Hkv, D, 1, start + t, cap, rope_mode=1))
+            return orc.sdpa_decode(qr[:, 0].copy(), ok, ov, H, Hkv, D, cap, start + t + 1).reshape(-1)
+
+        graph.launch()
+        f.synchronize()
+        assert max_abs(d["out"].download().reshape(-1), expect(0)) <= 2e-3
+        # outgrow the workspace (64 MiB at first) while the graph is alive, then use the new one eagerly
+        grown = 160 << 20
+        f.reserve_workspace(grown)
+        step()
+        f.synchronize()
+        assert max_abs(d["out"].download().reshape(-1), expect(1)) <= 2e-3
+        for t in (2, 3):
+            graph.launch()
+            f.synchronize()
+            assert max_abs(d["out"].download().reshape(-1), expect(t)) <= 2e-3, t
+        assert np.array_equal(bits(d["kc"].download()), bits(ok))
+        f.reserve_workspace(grown + (64 << 20))  # a second retirement while the same graph lives
+        graph.launch()
+        f.synchronize()
+        assert max_abs(d["out"].download().reshape(-1), expect(4)) <= 2e-3
+        graph.destroy()  # frees the retired buffers
+        step()
+        f.synchronize()
+        assert max_abs(d["out"].download().reshape(-1), expect(5)) <= 2e-3
+    finally:
+        for b in d.values():
+            b.free()
+        f.close()
+
+
+def test_stream_waiting_calls_are_refused_during_capture():
+    announce("capture guards")
+    f = ctx()
+    buf = f.zeros((16,))
+    f.start_capture()
+    try:
+        for call in (lambda: buf.download(), lambda: buf.upload(np.zeros(16, np.float16)), lambda: f.synchronize(),
+                     lambda: f.profile_reset(), lambda: f.profile_query("x"), lambda: buf.free()):
+            with pytest.raises(fa.FoundryError) as e:
+                call()
+            assert e.value.variant == "OperationFailed" and "capture" in str(e.value)
+        f.u32_add(buf, 1, 0)  # the capture is still valid: record something and finish it
+    finally:
+        graph = f.end_capture()
+    graph.launch()
+    f.synchronize()
+    graph.destroy()
+    buf.free()
+
+
+def test_fused_step_past_its_bound_is_reported():
+    """A replayed fused step whose device position has moved past kv_len_bound (still inside the capacity) drops the
+    token; the next synchronize says so, once."""
+    announce("fused step beyond kv_len_bound")
+    f = ctx()
+    rng = np.random.default_rng(5)
+    H, Hkv, D, cap, start = 8, 2, 128, 512, 100
+    (cos, sin, kc, vc, q, k, v), d = _split_decode_state(f, rng, H, Hkv, D, cap, start)
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, 1, 0, cap, fa.ROPE_NEOX)
+    bound = start + 2  # room for positions start and start + 1
+
+    def step():
+        f.decode_step_fused(d["q"].arg(), d["k"].arg(), d["v"].arg(), None, d["kc"].arg(), d["vc"].arg(), d["cos"].arg(),
+                            d["sin"].arg(), d["out"].arg(), p, d_position=d["pos"], kv_len_bound=bound)
+        f.u32_add(d["pos"], 1, 1)
+
+    step()
+    step()
+    f.synchronize()  # both inside the bound
+    step()           # position start + 2: kv_len start + 3 > bound
+    with pytest.raises(fa.FoundryError) as e:
+        f.synchronize()
+    assert e.value.variant == "InvalidOperation" and "kv_len_bound" in str(e.value)
+    f.synchronize()  # reported once
+    got_k = d["kc"].download()
+    assert np.array_equal(bits(got_k[:, start + 2]), bits(kc[:, start + 2])), "the dropped token must not be stored"
+    for b in d.values():
+        b.free()
