@@ -230,6 +230,25 @@ fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_ten
                                const fa_tensor_arg *output, const fa_kv_prep_fused_params *params,
                                const uint32_t *d_position, uint32_t kv_len_bound);
 
+/* fa_decode_step_fused for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc). No counterpart in the reference. Same arguments, same kernels, same results bit for bit; the
+ * difference is where the partition partials live: in a static device array of fa_noalloc_scratch_bytes() (4 MiB) that
+ * every GPU the library runs on holds until the process ends, instead of the context's grow-only workspace. The call
+ * performs no hipMalloc / hipFree and no allocating library routine, at its first use on a device included (the array's
+ * address is looked up in fa_ctx_create). The partitions are always merged by the second launch (no arrival counters).
+ * Limits: partitions x batch x n_heads x (head_dim + 2) x 4 bytes must fit the array, else FA_ERR_INVALID_SHAPE
+ * (Llama-3.2-3B at 8K context needs 0.4 MiB); per-kernel profiling must be off (FA_ERR_OPERATION_FAILED otherwise: its
+ * events are created per launch). All calls on one GPU - from any context or thread - share that GPU's array, which
+ * keeps the last call's partials: calls that overlap in time on one GPU race. Calls on one context's stream, or
+ * replays of graphs recorded from them, are ordered and safe. */
+fa_status fa_decode_step_fused_noalloc(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                       const fa_tensor_arg *v, const fa_tensor_arg *q_rot,
+                                       const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
+                                       const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                       const fa_tensor_arg *output, const fa_kv_prep_fused_params *params,
+                                       const uint32_t *d_position, uint32_t kv_len_bound);
+size_t fa_noalloc_scratch_bytes(void);
+
 /* Tuning override, the counterpart of FlashDecodeVariant + METALLIC_FA_DECODE_* (src/metals/flashattention/
  * variants.rs:36-140). keys_per_split: context partition per workgroup (rounded up to the kernel's 16-key
  * block; 0 = auto: one partition per compute unit).

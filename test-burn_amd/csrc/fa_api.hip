@@ -113,6 +113,7 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     ctx->ledger = new FaGraphLedger();
     fa_status s = fa_ensure_workspace(ctx, (size_t)64 << 20);
     if (s == FA_OK) s = fa_ensure_counters(ctx, 4096);
+    if (s == FA_OK) s = fa_decode_static_scratch(device, &ctx->static_scratch, &ctx->static_scratch_bytes);
     if (s == FA_OK) {
         // one word that kernels set bits in and the host reads after a synchronize: pinned host memory mapped into the device
         hipError_t he = hipHostMalloc((void **)&ctx->h_status, sizeof(uint32_t), hipHostMallocMapped);
@@ -1175,10 +1176,11 @@ static fa_status decode_step_fused_impl(fa_ctx *ctx, const fa_tensor_arg *q, con
                                         const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
                                         const fa_tensor_arg *cos, const fa_tensor_arg *sin,
                                         const fa_tensor_arg *output, const fa_kv_prep_fused_params *p,
-                                        const uint32_t *d_position, uint32_t kv_len_bound) {
+                                        const uint32_t *d_position, uint32_t kv_len_bound, bool static_scratch) {
     FA_NEED(ctx, "ctx");
     DecodeLaunch L;
     memset(&L, 0, sizeof(L));
+    L.static_scratch = static_scratch;
     FA_NEED(p, "params");
     FA_TRY(fused_common(q, k, v, q_rot, cos, sin, p, 1, L));
     FA_TRY(check_tensor(k_cache, "k_cache", FA_DT(q), 0, 16));
@@ -1216,8 +1218,19 @@ extern "C" fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, c
                                           const fa_tensor_arg *cos, const fa_tensor_arg *sin,
                                           const fa_tensor_arg *output, const fa_kv_prep_fused_params *p,
                                           const uint32_t *d_position, uint32_t kv_len_bound) {
-    return decode_step_fused_impl(ctx, q, k, v, q_rot, k_cache, v_cache, cos, sin, output, p, d_position, kv_len_bound);
+    return decode_step_fused_impl(ctx, q, k, v, q_rot, k_cache, v_cache, cos, sin, output, p, d_position, kv_len_bound, false);
 }
+
+extern "C" fa_status fa_decode_step_fused_noalloc(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
+                                                  const fa_tensor_arg *v, const fa_tensor_arg *q_rot,
+                                                  const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
+                                                  const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                                  const fa_tensor_arg *output, const fa_kv_prep_fused_params *p,
+                                                  const uint32_t *d_position, uint32_t kv_len_bound) {
+    return decode_step_fused_impl(ctx, q, k, v, q_rot, k_cache, v_cache, cos, sin, output, p, d_position, kv_len_bound, true);
+}
+
+extern "C" size_t fa_noalloc_scratch_bytes(void) { return FA_STATIC_SCRATCH_BYTES; }
 
 extern "C" fa_status fa_decode_step_fused_paged(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k,
                                                 const fa_tensor_arg *v, const fa_tensor_arg *q_rot,

@@ -1,6 +1,33 @@
 // Host-side launch logic of the flash-decode kernels (partition sizing, scratch, kernel selection).
 #include "fa_decode_impl.h"
 
+#include <mutex>
+
+// Decode partials of the entry point that allocates nothing (fa_decode_step_fused_noalloc): every GPU the library runs
+// on holds its own copy of this array until the process ends. In host code the name is only a handle for
+// hipGetSymbolAddress: kernels are given the address that call returns, never the name.
+static __device__ __align__(256) unsigned char scratch[FA_STATIC_SCRATCH_BYTES];
+
+fa_status fa_decode_static_scratch(int device, void **ptr, size_t *bytes) {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex mu;
+    static void *per_device[MAX_DEVICES] = {};
+    if (device < 0 || device >= MAX_DEVICES)
+        return fa_fail(FA_ERR_DEVICE_NOT_FOUND, "Device not found (device %d: the static scratch table holds %d)", device, MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!per_device[device]) {
+        // the caller has made `device` current: the symbol resolves to that GPU's copy
+        void *p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fa_fail(FA_ERR_OPERATION_FAILED, "hipGetSymbolAddress(scratch) failed on device %d: %s", device, hipGetErrorString(e));
+        per_device[device] = p;
+    }
+    *ptr = per_device[device];
+    *bytes = FA_STATIC_SCRATCH_BYTES;
+    return FA_OK;
+}
+
 namespace {
 
 // Heads of a group served by one workgroup: the largest divisor of the group that fits the MFMA N dimension.
@@ -76,15 +103,32 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     a.qin_stride_b = L.qin_stride_b, a.kvin_stride_b = L.kvin_stride_b, a.qrot_stride_b = L.qrot_stride_b;
     a.rope_normal = L.rope_normal, a.apply_rope = L.apply_rope, a.table_rows = L.table_rows;
     a.status = ctx->d_status;
+    if (L.static_scratch) {
+        // Nothing may be allocated on this path: no workspace growth, no event creation. The partitions' partial
+        // states go to the static device array and a second launch merges them (no arrival counters to keep zero).
+        if (ctx->profiling)
+            return fa_fail(FA_ERR_OPERATION_FAILED, "the entry point that allocates nothing cannot run with per-kernel profiling enabled (events are created per launch)");
+        a.merge_in_kernel = 0;
+    }
     if (S > 1) {
         const size_t rows = (size_t)L.batch * ny * S * gt;
         const size_t acc_bytes = rows * L.head_dim * sizeof(float);
         const size_t ml_bytes = rows * 2 * sizeof(float);
-        FA_TRY(fa_ensure_workspace(ctx, acc_bytes + ml_bytes));
-        FA_TRY(fa_ensure_counters(ctx, L.batch * ny));
-        a.part_acc = (float *)ctx->workspace;
-        a.part_ml = (float *)((char *)ctx->workspace + acc_bytes);
-        a.counters = ctx->counters;
+        if (L.static_scratch) {
+            if (acc_bytes + ml_bytes > ctx->static_scratch_bytes || !ctx->static_scratch)
+                return fa_fail(FA_ERR_INVALID_SHAPE,
+                               "Invalid shape: this decode launch needs %zu bytes of partition partials (%u partitions x %u head rows), "
+                               "the static scratch of the entry point that allocates nothing holds %zu",
+                               acc_bytes + ml_bytes, S, (uint32_t)(L.batch * ny * gt), ctx->static_scratch_bytes);
+            a.part_acc = (float *)ctx->static_scratch;
+            a.part_ml = (float *)((char *)ctx->static_scratch + acc_bytes);
+        } else {
+            FA_TRY(fa_ensure_workspace(ctx, acc_bytes + ml_bytes));
+            FA_TRY(fa_ensure_counters(ctx, L.batch * ny));
+            a.part_acc = (float *)ctx->workspace;
+            a.part_ml = (float *)((char *)ctx->workspace + acc_bytes);
+            a.counters = ctx->counters;
+        }
     }
     int mode = MODE_PLAIN;
     if (L.q_scale)

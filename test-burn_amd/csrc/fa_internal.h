@@ -46,6 +46,9 @@ struct fa_ctx {
     // Outgrown workspaces / counter arrays that a recorded graph may still reference are parked here: freed once no
     // graph is alive, or with the context.
     FaGraphLedger *ledger = nullptr;
+    // The library's static device array on this device (decode partials of the entry point that allocates nothing)
+    void *static_scratch = nullptr;
+    size_t static_scratch_bytes = 0;
     // Sticky status word written by kernels (pinned host memory, mapped into the device): FA_DEVSTAT_* bits.
     uint32_t *h_status = nullptr;  // host view
     uint32_t *d_status = nullptr;  // device view of the same word
@@ -152,6 +155,7 @@ struct DecodeLaunch {
     uint64_t qin_stride_b, kvin_stride_b, qrot_stride_b;
     uint32_t rope_normal, apply_rope, table_rows;
     bool bf16;  // q, k, v, caches and out are bf16 instead of f16 (not with the int8 variant)
+    bool static_scratch;  // partials go to the library's static device array; nothing may be allocated
 };
 fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &a);
 
@@ -243,3 +247,8 @@ constexpr uint32_t FA_DEVSTAT_APPEND_DROPPED = 2u; // a fused decode step's posi
 
 fa_status fa_ensure_workspace(fa_ctx *ctx, size_t bytes);
 fa_status fa_ensure_counters(fa_ctx *ctx, uint32_t n);
+// Size of the static device array that holds the decode partials of fa_decode_step_fused_noalloc (per GPU, for the
+// life of the process).
+constexpr size_t FA_STATIC_SCRATCH_BYTES = (size_t)4 << 20;
+// Address and size of the static device array on the current device (looked up once per device).
+fa_status fa_decode_static_scratch(int device, void **ptr, size_t *bytes);

@@ -111,6 +111,8 @@ PROTOTYPES = {
     "fa_flash_attention": [_vp, _PT, _PT, _PT, _PT, _i, _u32, _u32, _u32, _u32, _u32, _i],
     "fa_flash_decode_dyn": [_vp, _PT, _PT, _PT, _PT, _u32, _u32, _vp, _u32, _u32],
     "fa_decode_step_fused": [_vp, _PT, _PT, _PT, _PT, _PT, _PT, _PT, _PT, _PT, C.POINTER(KvPrepFusedParams), _vp, _u32],
+    "fa_decode_step_fused_noalloc": [_vp, _PT, _PT, _PT, _PT, _PT, _PT, _PT, _PT, _PT, C.POINTER(KvPrepFusedParams), _vp, _u32],
+    "fa_noalloc_scratch_bytes": [],
     "fa_decode_step_fused_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _PT, _PT, _PT,
                                    C.POINTER(KvPrepFusedParams), _u32],
     "fa_set_decode_variant": [_vp, C.POINTER(DecodeVariant)],
@@ -138,7 +140,8 @@ PROTOTYPES = {
     "fa_device_info": [_vp, C.c_char_p, _sz, C.POINTER(_u32), C.POINTER(C.c_uint64)],
 }
 _RESTYPES = {"fa_status_name": C.c_char_p, "fa_last_error_string": C.c_char_p, "fa_version": C.c_char_p,
-             "fa_ctx_stream": _vp, "fa_is_capturing": _i, "fa_align_capacity": _sz, "fa_grown_capacity": _sz}
+             "fa_ctx_stream": _vp, "fa_is_capturing": _i, "fa_align_capacity": _sz, "fa_grown_capacity": _sz,
+             "fa_noalloc_scratch_bytes": _sz}
 
 _lib = None
 
@@ -354,11 +357,11 @@ class Foundry:
                                            d_position.ptr, kv_len_add, kv_len_bound))
 
     def decode_step_fused(self, q, k, v, q_rot, k_cache, v_cache, cos, sin, out, params, d_position=None,
-                          kv_len_bound=0):
+                          kv_len_bound=0, noalloc=False):
         if q_rot is None:
             q_rot = TensorArg()
         a = [C.byref(x) for x in (q, k, v, q_rot, k_cache, v_cache, cos, sin, out)]
-        fn = self.lib.fa_decode_step_fused
+        fn = self.lib.fa_decode_step_fused_noalloc if noalloc else self.lib.fa_decode_step_fused
         check(fn(self.h, *a, C.byref(params), None if d_position is None else d_position.ptr, kv_len_bound))
 
     def decode_step_fused_paged(self, q, k, v, q_rot, cache, cos, sin, out, params, kv_len_bound):
