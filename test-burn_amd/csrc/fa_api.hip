@@ -102,6 +102,7 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     }
     ctx->decode_variant.keys_per_split = env_u32("FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT", 0);
     ctx->decode_variant.merge = env_u32("FOUNDRY_ATTN_DECODE_MERGE", 1);
+    if (ctx->decode_variant.merge > 2) ctx->decode_variant.merge = 1;
     ctx->decode_waves = env_u32("FOUNDRY_ATTN_DECODE_WAVES", 0);
     if (ctx->decode_waves != 4 && ctx->decode_waves != 8) ctx->decode_waves = 0;
     ctx->gemm_min_m = env_u32("FOUNDRY_ATTN_GEMM_MIN_M", 0);
@@ -114,6 +115,15 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     fa_status s = fa_ensure_workspace(ctx, (size_t)64 << 20);
     if (s == FA_OK) s = fa_ensure_counters(ctx, 4096);
     if (s == FA_OK) s = fa_decode_static_scratch(device, &ctx->static_scratch, &ctx->static_scratch_bytes);
+    if (s == FA_OK) {
+        // Records of the polled merge: room for two workgroups per compute unit serving 16 heads of 128 dims each (32 B per float4 column)
+        ctx->poll_spin_us = env_u32("FOUNDRY_ATTN_DECODE_POLL_SPIN_US", 2000000);
+        const size_t bytes = (size_t)2 * (ctx->n_cus > 0 ? ctx->n_cus : 256) * (16 * 128 / 4) * 32;
+        hipError_t he = hipMalloc(&ctx->poll_ws, bytes);
+        if (he == hipSuccess) he = hipMemset(ctx->poll_ws, 0xff, bytes);
+        if (he != hipSuccess) s = fa_fail(FA_ERR_OUT_OF_MEMORY, "polled-merge buffer of %zu bytes: %s", bytes, hipGetErrorString(he));
+        else ctx->poll_ws_bytes = bytes;
+    }
     if (s == FA_OK) {
         // one word that kernels set bits in and the host reads after a synchronize: pinned host memory mapped into the device
         hipError_t he = hipHostMalloc((void **)&ctx->h_status, sizeof(uint32_t), hipHostMallocMapped);
@@ -143,6 +153,7 @@ extern "C" fa_status fa_ctx_destroy(fa_ctx *ctx) {
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->counters) (void)hipFree(ctx->counters);
     if (ctx->h_status) (void)hipHostFree(ctx->h_status);
+    if (ctx->poll_ws) (void)hipFree(ctx->poll_ws);
     if (ctx->ledger) {
         // graphs that outlive the context can no longer be launched (fa_graph_launch needs it); what they address goes now
         for (void *p : ctx->ledger->retired) (void)hipFree(p);
@@ -164,6 +175,13 @@ extern "C" fa_status fa_synchronize(fa_ctx *ctx) {
     if (ctx->h_status && *ctx->h_status) {
         const uint32_t bits = *ctx->h_status;
         *ctx->h_status = 0;
+        if (bits & FA_DEVSTAT_MERGE_TIMEOUT) {
+            // the buffer no longer holds the arrival pattern everywhere: restore it before anything else runs
+            (void)hipMemset(ctx->poll_ws, 0xff, ctx->poll_ws_bytes);
+            return fa_fail(FA_ERR_OPERATION_FAILED,
+                           "a decode launch's merging workgroup waited longer than %u us for the other partitions; the "
+                           "outputs of the decode calls since the last synchronize are invalid", ctx->poll_spin_us);
+        }
         if (bits & FA_DEVSTAT_APPEND_DROPPED)
             return fa_fail(FA_ERR_INVALID_OPERATION,
                            "Invalid operation: a fused decode step ran at a position at or beyond its kv_len_bound or the cache "
@@ -256,7 +274,7 @@ extern "C" fa_status fa_set_decode_variant(fa_ctx *ctx, const fa_decode_variant 
     if (v->keys_per_split % 64 != 0)
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "decode keys_per_split must be a multiple of 64 (or 0), got %u",
                        v->keys_per_split);
-    if (v->merge > 1) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "decode merge must be 0 or 1, got %u", v->merge);
+    if (v->merge > 2) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "decode merge must be 0, 1 or 2, got %u", v->merge);
     ctx->decode_variant = *v;
     return FA_OK;
 }

@@ -103,6 +103,20 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     a.qin_stride_b = L.qin_stride_b, a.kvin_stride_b = L.kvin_stride_b, a.qrot_stride_b = L.qrot_stride_b;
     a.rope_normal = L.rope_normal, a.apply_rope = L.apply_rope, a.table_rows = L.table_rows;
     a.status = ctx->d_status;
+    // The polled merge needs every workgroup of the launch resident at once (the merging workgroup of a head group
+    // occupies its compute unit while it waits) and its partials in the context's pattern-filled buffer.
+    bool polled = false;
+    if (ctx->decode_variant.merge == 2 && !L.static_scratch) {
+        const uint32_t n4 = (uint32_t)gt * L.head_dim / 4;  // records (float4 columns of all heads) per partition
+        const size_t need = (size_t)L.batch * ny * S * n4 * 32;
+        const uint64_t slots = waves == 4 ? 2 * n_cus : n_cus;
+        const uint32_t nt = waves * 64;
+        // a workgroup reads ceil(n4 / partitions) columns of every partition (fewer than n4 + partitions records for
+        // any partition count up to S), at most POLL_IPT records per thread
+        polled = S > 1 && groups * S <= slots && need <= ctx->poll_ws_bytes && (uint64_t)n4 + S <= (uint64_t)nt * POLL_IPT;
+        a.merge_in_kernel = polled ? 2u : 0u;
+        a.poll_ticks = (unsigned long long)ctx->poll_spin_us * 100ull;
+    }
     if (L.static_scratch) {
         // Nothing may be allocated on this path: no workspace growth, no event creation. The partitions' partial
         // states go to the static device array and a second launch merges them (no arrival counters to keep zero).
@@ -122,6 +136,9 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
                                acc_bytes + ml_bytes, S, (uint32_t)(L.batch * ny * gt), ctx->static_scratch_bytes);
             a.part_acc = (float *)ctx->static_scratch;
             a.part_ml = (float *)((char *)ctx->static_scratch + acc_bytes);
+        } else if (polled) {
+            a.part_acc = (float *)ctx->poll_ws;
+            a.part_ml = nullptr;
         } else {
             FA_TRY(fa_ensure_workspace(ctx, acc_bytes + ml_bytes));
             FA_TRY(fa_ensure_counters(ctx, L.batch * ny));

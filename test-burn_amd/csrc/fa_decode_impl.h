@@ -116,6 +116,27 @@ __device__ __forceinline__ float xor32(float x) {
     return __uint_as_float(((threadIdx.x >> 5) & 1) ? r.x : r.y);
 }
 
+// Reductions over aligned groups of 4, 8 or 32 consecutive lanes; every lane of the group gets the result. Lane
+// exchanges inside a 16-lane row are DPP moves (quad permutes, then the mirrors of a half row and of a row), the step
+// across rows is a lane swap. The order of the operands is fixed, so results are reproducible.
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+template <int G, bool MAX>
+__device__ __forceinline__ float group_reduce(float v) {
+    static_assert(G == 4 || G == 8 || G == 32, "group sizes in use");
+    auto op = [](float x, float y) { return MAX ? fmaxf(x, y) : x + y; };
+    v = op(v, dpp_mov<0xB1>(v));               // quad_perm [1,0,3,2]: lane ^ 1
+    v = op(v, dpp_mov<0x4E>(v));               // quad_perm [2,3,0,1]: lane ^ 2
+    if (G >= 8) v = op(v, dpp_mov<0x141>(v));  // row_half_mirror: the other quad of the 8 lanes
+    if (G >= 32) {
+        v = op(v, dpp_mov<0x140>(v));          // row_mirror: the other half of the row
+        v = op(v, xor16(v));
+    }
+    return v;
+}
+
 // Partial results written by one workgroup are read by another workgroup of the same launch, possibly through
 // a different L2 slice. They are therefore moved with buffer loads / stores that carry the sc0|sc1 cache
 // bits (write-through to, and read from, the device-wide coherence point) instead of a cache-wide
@@ -242,6 +263,133 @@ __device__ __forceinline__ void merge_and_store(const DecodeDev &a, uint32_t b, 
     }
 }
 
+// Cooperative polled merge (one launch, no ticket). Every partition's workgroup writes its partial state as records
+//   rec[group][partition][column] = {acc.x, acc.y, acc.z, acc.w, m, l, -, -}    column = head * D/4 + float4 column
+// and then merges a share of the columns itself: workgroup c of the group's `nsplits` owns columns c, c + nsplits, ...
+// and reads those columns' records of ALL partitions. What bounds a merge is how fast one compute unit can request
+// the partials (one unit pulling a head group's 50 KB needs about 2 us), so the reads are spread over all of them.
+// Nothing signals arrival: every word of the record buffer holds POLL_SENTINEL between launches and no record ever
+// stores that pattern, so a record whose six words all differ from it has arrived. A thread re-reads the records it
+// is still missing until they are there - or until `poll_ticks` of the 100 MHz clock have passed, in which case
+// nothing is stored and false is returned - and writes the pattern back over what it has consumed (each record is
+// read by exactly one thread of the launch). No workgroup waits for one that has not been started yet unless the
+// launch exceeds the resident capacity, which the host rules out.
+constexpr uint32_t POLL_SENTINEL = 0xffffffffu;
+constexpr int POLL_IPT = 4;  // records per thread, at most
+__device__ __forceinline__ float not_sentinel(float v) {  // the pattern is a NaN: a partial stores the canonical one instead
+    return __float_as_uint(v) == POLL_SENTINEL ? __uint_as_float(0x7fc00000u) : v;
+}
+template <int D>
+__device__ __forceinline__ bool coop_merge_and_store(const DecodeDev &a, uint32_t b, uint32_t y, uint32_t c,
+                                                     uint32_t nsplits, uint32_t S, int tid, float *sm) {
+    constexpr int CG = D / 4;
+    const uint32_t gt = a.gt, n4 = gt * CG;
+    const uint32_t my_cols = n4 > c ? (n4 - c + nsplits - 1) / nsplits : 0u;
+    const uint32_t items = my_cols * nsplits;  // <= NT * POLL_IPT (host)
+    const size_t g = (size_t)b * gridDim.y + y;
+    const float *rec = a.part_acc + g * S * n4 * 8;
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(rec);
+    f2_t *sm_ml = reinterpret_cast<f2_t *>(sm);                      // [items]
+    f4_t *sm_acc = reinterpret_cast<f4_t *>(sm + 2 * NT * POLL_IPT);  // [items]
+    const unsigned long long t_begin = wall_clock64();
+    bool timed_out = false;
+    u4_t x[POLL_IPT];
+    u2_t ml[POLL_IPT];
+    uint32_t off[POLL_IPT];  // byte offset of the record
+    uint32_t pend = 0;
+#pragma unroll
+    for (int j = 0; j < POLL_IPT; ++j) {
+        const uint32_t t = tid + j * NT;
+        if (t < items) {
+            const uint32_t i = t / nsplits, p = t - i * nsplits;
+            off[j] = ((p * n4) + c + i * nsplits) * 32u;
+            pend |= 1u << j;
+        } else {
+            off[j] = 0;
+        }
+    }
+    const uint32_t mine = pend;
+    for (;;) {
+#pragma unroll
+        for (int j = 0; j < POLL_IPT; ++j) {
+            if (pend >> j & 1u) {
+                x[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off[j], 0, CACHE_COHERENT);
+                ml[j] = __builtin_amdgcn_raw_buffer_load_b64(rs, (int)off[j] + 16, 0, CACHE_COHERENT);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < POLL_IPT; ++j) {
+            if (pend >> j & 1u) {
+                const bool ok = x[j].x != POLL_SENTINEL && x[j].y != POLL_SENTINEL && x[j].z != POLL_SENTINEL &&
+                                x[j].w != POLL_SENTINEL && ml[j].x != POLL_SENTINEL && ml[j].y != POLL_SENTINEL;
+                if (ok) pend &= ~(1u << j);
+            }
+        }
+        if (!__any(pend != 0)) break;
+        if (wall_clock64() - t_begin > a.poll_ticks) {
+            timed_out = true;
+            break;
+        }
+    }
+    if (!timed_out) {
+        const u4_t sent4 = {POLL_SENTINEL, POLL_SENTINEL, POLL_SENTINEL, POLL_SENTINEL};
+        const u2_t sent2 = {POLL_SENTINEL, POLL_SENTINEL};
+        // first everything that reads the loaded registers, then the stores: a wait for a load placed behind a store
+        // would wait for that store's acknowledgement as well
+#pragma unroll
+        for (int j = 0; j < POLL_IPT; ++j) {
+            if (mine >> j & 1u) {
+                const uint32_t t = tid + j * NT;
+                sm_ml[t] = __builtin_bit_cast(f2_t, ml[j]);
+                sm_acc[t] = __builtin_bit_cast(f4_t, x[j]);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < POLL_IPT; ++j) {
+            if (mine >> j & 1u) {
+                __builtin_amdgcn_raw_buffer_store_b128(sent4, rs, (int)off[j], 0, CACHE_COHERENT);
+                __builtin_amdgcn_raw_buffer_store_b64(sent2, rs, (int)off[j] + 16, 0, CACHE_COHERENT);
+            }
+        }
+    }
+    if (__syncthreads_or(timed_out ? 1 : 0)) return false;
+    // Column i of this workgroup: its partitions' states are sm[i * nsplits + p]. 32 lanes share a column: lane r takes
+    // partitions r, r + 32, ... in order, then the 32 running states are merged across the lanes.
+    for (uint32_t base = 0; base < my_cols * 32u; base += NT) {  // uniform over the workgroup
+        const uint32_t u = base + (uint32_t)tid, i = u >> 5, r = u & 31u;
+        const bool valid = i < my_cols;
+        float m_r = -1e30f, l_r = 0.0f;
+        f4_t acc_r = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (valid) {
+            const uint32_t t0 = i * nsplits;
+            for (uint32_t p = r; p < nsplits; p += 32u) {
+                const f2_t mlp = sm_ml[t0 + p];
+                const float mn = fmaxf(m_r, mlp.x);
+                const float e0 = fast_exp2(m_r - mn), e1 = fast_exp2(mlp.x - mn);
+                l_r = l_r * e0 + mlp.y * e1;
+                acc_r = acc_r * e0 + sm_acc[t0 + p] * e1;
+                m_r = mn;
+            }
+        }
+        const float mstar = group_reduce<32, true>(m_r);
+        const float w = fast_exp2(m_r - mstar);
+        const float L = group_reduce<32, false>(l_r * w);
+        f4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = group_reduce<32, false>(acc_r[e] * w);
+        if (valid && r == 0) {
+            const uint32_t col = c + i * nsplits, h = col / CG, c4 = col - h * CG;
+            const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 1.0f;
+            const uint32_t head = y * gt + h;
+            __half *op = a.out + (size_t)b * a.out_stride_b + (size_t)head * a.out_stride_h + c4 * 4;
+            const float ov[4] = {o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
+            store_out4(op, ov, a.bf16 != 0);
+        }
+    }
+    return true;
+}
+
 // RoPE of 8 elements (src/metals/kv_prep/kv_prep_fused.metal:66-82): products and sum are rounded separately
 // (no FMA contraction) and the result is rounded once to f16.
 //   normal: x = 8 consecutive dims (4 adjacent pairs), c/s = 4 values
@@ -285,6 +433,10 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ uint32_t sm_last;
+    // Number of waves that have put their part of the Q^T operand into LDS. A wave starts on its blocks once the
+    // count is complete instead of meeting the others at a barrier: a wave reaches that point only when all of its
+    // block requests have been accepted, which for the last one is most of the launch's streaming time.
+    __shared__ uint32_t sm_q_ready;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: tile addresses stay in SGPRs
@@ -473,6 +625,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                 kk[1][j].u = *reinterpret_cast<const uint4 *>(krow + (4 * j + c) * 8);
             }
             vv[1][0].u = *reinterpret_cast<const uint4 *>(vrow_in + (lane % VLPR) * 8);
+            if (lane == 0) sm_q_ready = 0;
             __builtin_amdgcn_sched_barrier(0);
             __syncthreads();  // releases the streaming waves
             __builtin_amdgcn_sched_barrier(0);
@@ -522,11 +675,15 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             }
 #pragma unroll
             for (int j = 0; j < KSTEPS; ++j) q_lds[j * 64 + lane] = qb[j].u;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+            if (lane == 0) __hip_atomic_store(&sm_q_ready, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             __builtin_amdgcn_s_setprio(0);
         } else {
             __syncthreads();  // wave 0 has queued its requests
         }
     } else {
+        if (tid == 0) sm_q_ready = 0;
+        __syncthreads();
         // wave j < KSTEPS fetches step j of the operand (requested before its K/V blocks, so it returns first)
         if (wave < KSTEPS && head_ok) {
             const unsigned char *qrow =
@@ -540,7 +697,11 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         issue_k(cur, m, 0);
         issue_v(cur, m, 0);
     }
-    if (!FUSED && wave < KSTEPS) q_lds[wave * 64 + lane] = qraw.u;
+    if (!FUSED && wave < KSTEPS) {
+        q_lds[wave * 64 + lane] = qraw.u;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        if (lane == 0) __hip_atomic_fetch_add(&sm_q_ready, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
     if (!(FUSED && wave == 0)) n_raw = read_len();
     const uint32_t N = min(n_raw, min(a.capacity, a.kv_len_bound));
     const uint32_t nsplits = (N + a.chunk - 1) / a.chunk;
@@ -574,7 +735,11 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         issue_v(cur, m, k1 - 1);
         if (cur + m < wbe) load_pages(cur + m, min((uint32_t)MBX, wbe - (cur + m)), pgn);
     }
-    __syncthreads();  // the Q^T operand is in LDS
+    {   // the Q^T operand is in LDS once every contributing wave has counted itself in
+        constexpr uint32_t Q_PARTS = FUSED ? 1u : (uint32_t)(KSTEPS < NW ? KSTEPS : NW);
+        while (__hip_atomic_load(&sm_q_ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < Q_PARTS) __builtin_amdgcn_s_sleep(1);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    }
 
     f4_t oacc[DBLK];
 #pragma unroll
@@ -736,28 +901,40 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     }
     __syncthreads();
 
-    const bool in_kernel = a.merge_in_kernel != 0;
+    const bool in_kernel = a.merge_in_kernel != 0, polled = a.merge_in_kernel == 2;
     const size_t gbase = ((size_t)b * gridDim.y + y) * S * gt;  // first row of this (sequence, head group)
     const uint32_t prow = split * gt;
     constexpr int CG = D / 4;
-    for (int idx = tid; idx < (int)gt * CG; idx += NT) {
-        const int h = idx / CG, c4 = idx % CG;
-        float ms = sm_ml[h * 2];
+    // NW consecutive lanes share a column (head h, float4 column c4): lane w reads wave w's state, the group merges,
+    // and its first lane owns the result.
+    const int wsel = tid % NW;
+    for (int base = 0; base < (int)gt * CG * NW; base += NT) {  // uniform over the workgroup
+        const int idx = (base + tid) / NW;
+        const bool valid = idx < (int)gt * CG;
+        const int h = valid ? idx / CG : 0, c4 = valid ? idx % CG : 0;
+        const float m_w = sm_ml[(wsel * gt + h) * 2], l_w = sm_ml[(wsel * gt + h) * 2 + 1];
+        const f4_t a_w = *reinterpret_cast<const f4_t *>(sm_acc + ((size_t)wsel * gt + h) * D + c4 * 4);
+        float ms = group_reduce<NW, true>(m_w);
+        const float e = fast_exp2(m_w - ms);
+        float L = group_reduce<NW, false>(l_w * e);
+        f4_t A;
 #pragma unroll
-        for (int w = 1; w < NW; ++w) ms = fmaxf(ms, sm_ml[(w * gt + h) * 2]);
-        float L = 0.0f;
-        f4_t A = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int w = 0; w < NW; ++w) {
-            const float e = fast_exp2(sm_ml[(w * gt + h) * 2] - ms);
-            L += sm_ml[(w * gt + h) * 2 + 1] * e;
-            A += *reinterpret_cast<const f4_t *>(sm_acc + ((size_t)w * gt + h) * D + c4 * 4) * e;
-        }
+        for (int i = 0; i < 4; ++i) A[i] = group_reduce<NW, false>(a_w[i] * e);
+        if (!valid || wsel != 0) continue;
         if (nsplits == 1) {
             const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 1.0f;
             __half *op = a.out + (size_t)b * a.out_stride_b + (size_t)(head0 + h) * a.out_stride_h + c4 * 4;
             const float ov[4] = {A[0] * inv, A[1] * inv, A[2] * inv, A[3] * inv};
             store_out4(op, ov, BF16);
+        } else if (polled) {
+            // record of (this partition, column idx); a word that equals the arrival pattern would never be seen as arrived
+            const u4_t r0 = {__float_as_uint(not_sentinel(A[0])), __float_as_uint(not_sentinel(A[1])),
+                             __float_as_uint(not_sentinel(A[2])), __float_as_uint(not_sentinel(A[3]))};
+            const u2_t r1 = {__float_as_uint(not_sentinel(ms)), __float_as_uint(not_sentinel(L))};
+            const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.part_acc + ((size_t)b * gridDim.y + y) * S * (gt * CG) * 8);
+            const uint32_t ro = (split * (gt * CG) + (uint32_t)idx) * 32u;
+            __builtin_amdgcn_raw_buffer_store_b128(r0, rs, (int)ro, 0, CACHE_COHERENT);
+            __builtin_amdgcn_raw_buffer_store_b64(r1, rs, (int)ro + 16, 0, CACHE_COHERENT);
         } else if (in_kernel) {
             float *pa = a.part_acc + gbase * D, *pm = a.part_ml + gbase * 2;
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, A), make_rsrc(pa),
@@ -773,6 +950,12 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         }
     }
     if (nsplits == 1 || !in_kernel) return;
+    if (polled) {
+        __syncthreads();  // the fold above read the LDS region that the merge reuses
+        if (!coop_merge_and_store<D>(a, b, y, split, nsplits, S, tid, reinterpret_cast<float *>(smem)) && tid == 0 && a.status)
+            *a.status = FA_DEVSTAT_MERGE_TIMEOUT;
+        return;
+    }
 
     // The last workgroup of this (sequence, head group) to arrive merges all partitions. The partials were
     // stored write-through; wait until those stores have completed (vmcnt(0)), then take a ticket. No
@@ -817,7 +1000,7 @@ size_t decode_lds_bytes(uint32_t gt) {
     // the per-wave V blocks + the Q^T operand + one RoPE table row
     const size_t v_tiles = (size_t)NW * MBX * BK * (D * 2 + 32) + (size_t)(D / 32) * 64 * 16 + 2 * D;
     const size_t fold = ((size_t)NW * gt * D + (size_t)NW * gt * 2) * sizeof(float);
-    const size_t merge = (size_t)NT * 6 * sizeof(float);
+    const size_t merge = (size_t)NT * 6 * sizeof(float) * POLL_IPT;  // the cooperative merge holds POLL_IPT records per thread
     size_t m = v_tiles > fold ? v_tiles : fold;
     return m > merge ? m : merge;
 }

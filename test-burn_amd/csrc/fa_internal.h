@@ -46,6 +46,11 @@ struct fa_ctx {
     // Outgrown workspaces / counter arrays that a recorded graph may still reference are parked here: freed once no
     // graph is alive, or with the context.
     FaGraphLedger *ledger = nullptr;
+    // Partials of the polled in-kernel partition merge (launches whose workgroups are all resident at once): a fixed
+    // buffer whose every word holds 0xffffffff between launches. Never reallocated, so recorded graphs may address it.
+    void *poll_ws = nullptr;
+    size_t poll_ws_bytes = 0;
+    uint32_t poll_spin_us = 2000000;  // bound of a merging workgroup's wait for the other partitions
     // The library's static device array on this device (decode partials of the entry point that allocates nothing)
     void *static_scratch = nullptr;
     size_t static_scratch_bytes = 0;
@@ -170,7 +175,8 @@ struct FaDecodeDev {
     float *part_ml;      // [batch][y][S][gt][2]
     uint32_t *counters;  // [batch][y]
     uint32_t kv_len, d_len_stride, kv_len_add, kv_len_bound, capacity, chunk, n_kv_heads, sub_per_kv, gt;
-    uint32_t bt_stride, block_size, block_shift /* log2(block_size), 32 if not a power of two */, merge_in_kernel;
+    uint32_t bt_stride, block_size, block_shift /* log2(block_size), 32 if not a power of two */;
+    uint32_t merge_in_kernel;  // 0 = a second launch merges, 1 = the last workgroup to arrive does, 2 = the last partition's workgroup polls
     float scale_log2e;
     // Sage-style int8 Q/K: q and k point at int8 data, scores are rescaled by q_scale[h] * k_scale[kvh][key/32]
     const float *q_scale;
@@ -183,6 +189,7 @@ struct FaDecodeDev {
     uint32_t rope_normal, apply_rope, table_rows;
     uint32_t bf16;  // data tensors are bf16 (RoPE tables stay f16)
     uint32_t *status;  // the context's device-written status word (FA_DEVSTAT_* bits)
+    unsigned long long poll_ticks;  // polled merge: how long the merging workgroup waits for partials, 100 MHz ticks
 };
 
 
@@ -243,6 +250,7 @@ fa_status fa_launch_sage_quantize_q(fa_ctx *ctx, const void *q, uint32_t n_heads
                                     float *q_scale);
 
 // Bits of the context's device-written status word
+constexpr uint32_t FA_DEVSTAT_MERGE_TIMEOUT = 1u;  // a merging workgroup gave up waiting for a partition's partial
 constexpr uint32_t FA_DEVSTAT_APPEND_DROPPED = 2u; // a fused decode step's position was beyond its launch bound / capacity
 
 fa_status fa_ensure_workspace(fa_ctx *ctx, size_t bytes);
