@@ -114,6 +114,9 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     ctx->ledger = new FaGraphLedger();
     fa_status s = fa_ensure_workspace(ctx, (size_t)64 << 20);
     if (s == FA_OK) s = fa_ensure_counters(ctx, 4096);
+    if (s == FA_OK) s = fa_decode_probe_xcd(ctx);
+    if (s == FA_OK && env_u32("FOUNDRY_ATTN_DECODE_XCD_LOCAL", 1) == 0) ctx->xcd_round_robin = false;
+    if (env_u32("FOUNDRY_ATTN_DEBUG", 0)) fprintf(stderr, "[foundry_attn] xcd round robin: %d\n", (int)ctx->xcd_round_robin);
     if (s == FA_OK) s = fa_decode_static_scratch(device, &ctx->static_scratch, &ctx->static_scratch_bytes);
     if (s == FA_OK) {
         // Records of the polled merge: room for two workgroups per compute unit serving 16 heads of 128 dims each (32 B per float4 column)

@@ -28,6 +28,34 @@ fa_status fa_decode_static_scratch(int device, void **ptr, size_t *bytes) {
     return FA_OK;
 }
 
+// One word per workgroup: the XCD it runs on.
+__global__ void xcd_probe_kernel(uint32_t *out) {
+    if (threadIdx.x == 0) out[blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)] = __builtin_amdgcn_s_getreg((4 - 1) << 11 | 0 << 6 | 20);
+}
+
+fa_status fa_decode_probe_xcd(fa_ctx *ctx) {
+    ctx->xcd_round_robin = false;
+    const dim3 grid(12, 4, 2);  // the 3-D shape of a decode launch
+    const uint32_t n = grid.x * grid.y * grid.z;
+    if (!ctx->workspace || ctx->workspace_bytes < n * sizeof(uint32_t)) return FA_OK;
+    uint32_t *d = (uint32_t *)ctx->workspace;
+    FA_HIP(hipMemsetAsync(d, 0xff, n * sizeof(uint32_t), ctx->stream));
+    hipLaunchKernelGGL(xcd_probe_kernel, grid, dim3(64), 0, ctx->stream, d);
+    std::vector<uint32_t> h(n);
+    FA_HIP(hipMemcpyAsync(h.data(), d, n * sizeof(uint32_t), hipMemcpyDeviceToHost, ctx->stream));
+    FA_HIP(hipStreamSynchronize(ctx->stream));
+    bool ok = true;
+    // the first workgroup of a launch continues where the previous launch stopped: only the step of one XCD per id matters
+    for (uint32_t i = 0; i < n; ++i) ok = ok && h[i] < 8u && h[i] == ((h[0] + i) & 7u);
+    ctx->xcd_round_robin = ok;
+    if (getenv("FOUNDRY_ATTN_DEBUG")) {
+        fprintf(stderr, "[foundry_attn] xcd of workgroups:");
+        for (uint32_t i = 0; i < n && i < 40; ++i) fprintf(stderr, " %u", h[i]);
+        fprintf(stderr, "\n");
+    }
+    return FA_OK;
+}
+
 namespace {
 
 // Heads of a group served by one workgroup: the largest divisor of the group that fits the MFMA N dimension.
@@ -115,6 +143,7 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
         // any partition count up to S), at most POLL_IPT records per thread
         polled = S > 1 && groups * S <= slots && need <= ctx->poll_ws_bytes && (uint64_t)n4 + S <= (uint64_t)nt * POLL_IPT;
         a.merge_in_kernel = polled ? 2u : 0u;
+        a.xcd_local = polled && ctx->xcd_round_robin && groups % 8 == 0 ? 1u : 0u;
         a.poll_ticks = (unsigned long long)ctx->poll_spin_us * 100ull;
     }
     if (L.static_scratch) {

@@ -279,9 +279,13 @@ constexpr int POLL_IPT = 4;  // records per thread, at most
 __device__ __forceinline__ float not_sentinel(float v) {  // the pattern is a NaN: a partial stores the canonical one instead
     return __float_as_uint(v) == POLL_SENTINEL ? __uint_as_float(0x7fc00000u) : v;
 }
-template <int D>
+// LOCAL: every workgroup of the head group runs on the same XCD. Records are then written with plain stores (they go
+// through to that XCD's L2) and read with device-scope loads (which pass the compute unit's own cache and hit the L2):
+// a quarter of a microsecond from store to load instead of a trip to memory and back.
+template <int D, bool LOCAL>
 __device__ __forceinline__ bool coop_merge_and_store(const DecodeDev &a, uint32_t b, uint32_t y, uint32_t c,
                                                      uint32_t nsplits, uint32_t S, int tid, float *sm) {
+    constexpr int LD_POLICY = LOCAL ? 0x10 /* sc1 */ : CACHE_COHERENT, ST_POLICY = LOCAL ? 0 : CACHE_COHERENT;
     constexpr int CG = D / 4;
     const uint32_t gt = a.gt, n4 = gt * CG;
     const uint32_t my_cols = n4 > c ? (n4 - c + nsplits - 1) / nsplits : 0u;
@@ -313,8 +317,8 @@ __device__ __forceinline__ bool coop_merge_and_store(const DecodeDev &a, uint32_
 #pragma unroll
         for (int j = 0; j < POLL_IPT; ++j) {
             if (pend >> j & 1u) {
-                x[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off[j], 0, CACHE_COHERENT);
-                ml[j] = __builtin_amdgcn_raw_buffer_load_b64(rs, (int)off[j] + 16, 0, CACHE_COHERENT);
+                x[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off[j], 0, LD_POLICY);
+                ml[j] = __builtin_amdgcn_raw_buffer_load_b64(rs, (int)off[j] + 16, 0, LD_POLICY);
             }
         }
 #pragma unroll
@@ -348,8 +352,8 @@ __device__ __forceinline__ bool coop_merge_and_store(const DecodeDev &a, uint32_
 #pragma unroll
         for (int j = 0; j < POLL_IPT; ++j) {
             if (mine >> j & 1u) {
-                __builtin_amdgcn_raw_buffer_store_b128(sent4, rs, (int)off[j], 0, CACHE_COHERENT);
-                __builtin_amdgcn_raw_buffer_store_b64(sent2, rs, (int)off[j] + 16, 0, CACHE_COHERENT);
+                __builtin_amdgcn_raw_buffer_store_b128(sent4, rs, (int)off[j], 0, ST_POLICY);
+                __builtin_amdgcn_raw_buffer_store_b64(sent2, rs, (int)off[j] + 16, 0, ST_POLICY);
             }
         }
     }
@@ -446,8 +450,16 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // and in a ragged batch the low partitions always exist while the high ones are mostly empty: some XCDs queue
     // work while others idle (measured: 62 us with 12 partitions per sequence, 55 us with 11). Rotating the index
     // by the head-group index spreads every sequence's partitions over all XCDs.
-    const uint32_t y = blockIdx.y, b = blockIdx.z;
-    const uint32_t split = (blockIdx.x + y + gridDim.y * b) % gridDim.x;
+    uint32_t y = blockIdx.y, b = blockIdx.z;
+    uint32_t split = (blockIdx.x + y + gridDim.y * b) % gridDim.x;
+    if (a.xcd_local) {
+        // All partitions of a head group on ONE XCD (workgroup id modulo 8), so that their partial states meet in that
+        // XCD's L2 instead of in memory: group = id % 8 + 8 (id / 8 / S), partition = id / 8 % S. The host selects this
+        // only when the number of head groups is a multiple of 8.
+        const uint32_t lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z), slot = lin >> 3;
+        const uint32_t g = (lin & 7u) + 8u * (slot / gridDim.x);
+        split = slot % gridDim.x, y = g % gridDim.y, b = g / gridDim.y;
+    }
     const uint32_t gt = a.gt;
     const uint32_t kvh = y / a.sub_per_kv;
     const uint32_t head0 = y * gt;
@@ -933,8 +945,13 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             const u2_t r1 = {__float_as_uint(not_sentinel(ms)), __float_as_uint(not_sentinel(L))};
             const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.part_acc + ((size_t)b * gridDim.y + y) * S * (gt * CG) * 8);
             const uint32_t ro = (split * (gt * CG) + (uint32_t)idx) * 32u;
-            __builtin_amdgcn_raw_buffer_store_b128(r0, rs, (int)ro, 0, CACHE_COHERENT);
-            __builtin_amdgcn_raw_buffer_store_b64(r1, rs, (int)ro + 16, 0, CACHE_COHERENT);
+            if (a.xcd_local) {
+                __builtin_amdgcn_raw_buffer_store_b128(r0, rs, (int)ro, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b64(r1, rs, (int)ro + 16, 0, 0);
+            } else {
+                __builtin_amdgcn_raw_buffer_store_b128(r0, rs, (int)ro, 0, CACHE_COHERENT);
+                __builtin_amdgcn_raw_buffer_store_b64(r1, rs, (int)ro + 16, 0, CACHE_COHERENT);
+            }
         } else if (in_kernel) {
             float *pa = a.part_acc + gbase * D, *pm = a.part_ml + gbase * 2;
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, A), make_rsrc(pa),
@@ -952,8 +969,13 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     if (nsplits == 1 || !in_kernel) return;
     if (polled) {
         __syncthreads();  // the fold above read the LDS region that the merge reuses
-        if (!coop_merge_and_store<D>(a, b, y, split, nsplits, S, tid, reinterpret_cast<float *>(smem)) && tid == 0 && a.status)
-            *a.status = FA_DEVSTAT_MERGE_TIMEOUT;
+        bool ok;
+        if (a.xcd_local) {
+            ok = coop_merge_and_store<D, true>(a, b, y, split, nsplits, S, tid, reinterpret_cast<float *>(smem));
+        } else {
+            ok = coop_merge_and_store<D, false>(a, b, y, split, nsplits, S, tid, reinterpret_cast<float *>(smem));
+        }
+        if (!ok && tid == 0 && a.status) *a.status = FA_DEVSTAT_MERGE_TIMEOUT;
         return;
     }
 

@@ -50,6 +50,7 @@ struct fa_ctx {
     // buffer whose every word holds 0xffffffff between launches. Never reallocated, so recorded graphs may address it.
     void *poll_ws = nullptr;
     size_t poll_ws_bytes = 0;
+    bool xcd_round_robin = false;  // workgroups whose ids are equal modulo 8 share an XCD on this device (probed at creation)
     uint32_t poll_spin_us = 2000000;  // bound of a merging workgroup's wait for the other partitions
     // The library's static device array on this device (decode partials of the entry point that allocates nothing)
     void *static_scratch = nullptr;
@@ -189,6 +190,7 @@ struct FaDecodeDev {
     uint32_t rope_normal, apply_rope, table_rows;
     uint32_t bf16;  // data tensors are bf16 (RoPE tables stay f16)
     uint32_t *status;  // the context's device-written status word (FA_DEVSTAT_* bits)
+    uint32_t xcd_local;  // polled merge: a head group's workgroups share an XCD and exchange partials through its L2
     unsigned long long poll_ticks;  // polled merge: how long the merging workgroup waits for partials, 100 MHz ticks
 };
 
@@ -251,7 +253,8 @@ fa_status fa_launch_sage_quantize_q(fa_ctx *ctx, const void *q, uint32_t n_heads
 
 // Bits of the context's device-written status word
 constexpr uint32_t FA_DEVSTAT_MERGE_TIMEOUT = 1u;  // a merging workgroup gave up waiting for a partition's partial
-constexpr uint32_t FA_DEVSTAT_APPEND_DROPPED = 2u; // a fused decode step's position was beyond its launch bound / capacity
+constexpr uint32_t FA_DEVSTAT_APPEND_DROPPED = 2u;
+constexpr uint32_t FA_DEVSTAT_XCD_PLACEMENT = 4u;  // a workgroup did not run on the XCD its id implies (L2-local merge) // a fused decode step's position was beyond its launch bound / capacity
 
 fa_status fa_ensure_workspace(fa_ctx *ctx, size_t bytes);
 fa_status fa_ensure_counters(fa_ctx *ctx, uint32_t n);
@@ -260,3 +263,6 @@ fa_status fa_ensure_counters(fa_ctx *ctx, uint32_t n);
 constexpr size_t FA_STATIC_SCRATCH_BYTES = (size_t)4 << 20;
 // Address and size of the static device array on the current device (looked up once per device).
 fa_status fa_decode_static_scratch(int device, void **ptr, size_t *bytes);
+// Finds out whether consecutive workgroup ids of a launch run on consecutive XCDs (8 of them, from any start): sets
+// ctx->xcd_round_robin.
+fa_status fa_decode_probe_xcd(fa_ctx *ctx);
