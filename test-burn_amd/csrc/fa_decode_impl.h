@@ -394,6 +394,81 @@ __device__ __forceinline__ bool coop_merge_and_store(const DecodeDev &a, uint32_
     return true;
 }
 
+// The same merge for up to 64 partitions, without LDS and without a barrier: a column's records are read by a group
+// of P2 consecutive lanes (P2 = the power of two that holds the partitions), one partition per lane, and the group
+// folds them with lane exchanges. A wave depends on no other wave.
+template <int D, bool LOCAL>
+__device__ __forceinline__ bool coop_merge_in_registers(const DecodeDev &a, uint32_t b, uint32_t y, uint32_t c,
+                                                        uint32_t nsplits, uint32_t S, int tid) {
+    constexpr int LD_POLICY = LOCAL ? 0x10 /* sc1 */ : CACHE_COHERENT, ST_POLICY = LOCAL ? 0 : CACHE_COHERENT;
+    constexpr int CG = D / 4;
+    const uint32_t gt = a.gt, n4 = gt * CG;
+    const uint32_t sh = 32u - (uint32_t)__builtin_clz(nsplits - 1u);  // 2 <= nsplits <= 64: 1 .. 6
+    const uint32_t p = (uint32_t)tid & ((1u << sh) - 1u), gi = (uint32_t)tid >> sh, gpw = (uint32_t)NT >> sh;
+    const size_t g = (size_t)b * gridDim.y + y;
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.part_acc + g * S * n4 * 8);
+    const unsigned long long t_begin = wall_clock64();
+    bool ok = true;
+    for (uint32_t base = 0; c + base * nsplits < n4; base += gpw) {  // uniform over the workgroup
+        const uint32_t col = c + (base + gi) * nsplits;
+        const bool valid = col < n4 && p < nsplits;
+        const uint32_t off = (p * n4 + col) * 32u;
+        u4_t x = {0u, 0u, 0u, 0u};
+        u2_t ml = {0u, 0u};
+        bool pend = valid;
+        for (;;) {
+            if (pend) {
+                x = __builtin_amdgcn_raw_buffer_load_b128(rs, (int)off, 0, LD_POLICY);
+                ml = __builtin_amdgcn_raw_buffer_load_b64(rs, (int)off + 16, 0, LD_POLICY);
+                pend = !(x.x != POLL_SENTINEL && x.y != POLL_SENTINEL && x.z != POLL_SENTINEL && x.w != POLL_SENTINEL &&
+                         ml.x != POLL_SENTINEL && ml.y != POLL_SENTINEL);
+            }
+            if (!__any(pend)) break;
+            if (wall_clock64() - t_begin > a.poll_ticks) {
+                ok = false;
+                break;
+            }
+        }
+        if (!ok) break;  // uniform over the wave
+        float m_r = valid ? __uint_as_float(ml.x) : -1e30f, l_r = valid ? __uint_as_float(ml.y) : 0.0f;
+        f4_t acc = valid ? __builtin_bit_cast(f4_t, x) : f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        if (valid) {  // consumed: back to the pattern for the next launch
+            const u4_t sent4 = {POLL_SENTINEL, POLL_SENTINEL, POLL_SENTINEL, POLL_SENTINEL};
+            const u2_t sent2 = {POLL_SENTINEL, POLL_SENTINEL};
+            __builtin_amdgcn_raw_buffer_store_b128(sent4, rs, (int)off, 0, ST_POLICY);
+            __builtin_amdgcn_raw_buffer_store_b64(sent2, rs, (int)off + 16, 0, ST_POLICY);
+        }
+        // the group's maximum, then the weighted sums; `sh` steps of lane exchanges each
+        float mstar = m_r;
+        if (sh >= 1) mstar = fmaxf(mstar, dpp_mov<0xB1>(mstar));
+        if (sh >= 2) mstar = fmaxf(mstar, dpp_mov<0x4E>(mstar));
+        if (sh >= 3) mstar = fmaxf(mstar, dpp_mov<0x141>(mstar));
+        if (sh >= 4) mstar = fmaxf(mstar, dpp_mov<0x140>(mstar));
+        if (sh >= 5) mstar = fmaxf(mstar, xor16(mstar));
+        if (sh >= 6) mstar = fmaxf(mstar, xor32(mstar));
+        const float w = fast_exp2(m_r - mstar);
+        float v[5] = {l_r * w, acc[0] * w, acc[1] * w, acc[2] * w, acc[3] * w};
+#pragma unroll
+        for (int e = 0; e < 5; ++e) {
+            if (sh >= 1) v[e] += dpp_mov<0xB1>(v[e]);
+            if (sh >= 2) v[e] += dpp_mov<0x4E>(v[e]);
+            if (sh >= 3) v[e] += dpp_mov<0x141>(v[e]);
+            if (sh >= 4) v[e] += dpp_mov<0x140>(v[e]);
+            if (sh >= 5) v[e] += xor16(v[e]);
+            if (sh >= 6) v[e] += xor32(v[e]);
+        }
+        if (col < n4 && p == 0) {
+            const uint32_t h = col / CG, c4 = col - h * CG;
+            const float L = v[0];
+            const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 1.0f;
+            __half *op = a.out + (size_t)b * a.out_stride_b + (size_t)(y * gt + h) * a.out_stride_h + c4 * 4;
+            const float ov[4] = {v[1] * inv, v[2] * inv, v[3] * inv, v[4] * inv};
+            store_out4(op, ov, a.bf16 != 0);
+        }
+    }
+    return ok;
+}
+
 // RoPE of 8 elements (src/metals/kv_prep/kv_prep_fused.metal:66-82): products and sum are rounded separately
 // (no FMA contraction) and the result is rounded once to f16.
 //   normal: x = 8 consecutive dims (4 adjacent pairs), c/s = 4 values
@@ -968,8 +1043,14 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     }
     if (nsplits == 1 || !in_kernel) return;
     if (polled) {
-        __syncthreads();  // the fold above read the LDS region that the merge reuses
         bool ok;
+        if (nsplits <= 64) {
+            ok = a.xcd_local ? coop_merge_in_registers<D, true>(a, b, y, split, nsplits, S, tid)
+                             : coop_merge_in_registers<D, false>(a, b, y, split, nsplits, S, tid);
+            if (!ok && lane == 0 && a.status) *a.status = FA_DEVSTAT_MERGE_TIMEOUT;
+            return;
+        }
+        __syncthreads();  // the fold above read the LDS region that the merge reuses
         if (a.xcd_local) {
             ok = coop_merge_and_store<D, true>(a, b, y, split, nsplits, S, tid, reinterpret_cast<float *>(smem));
         } else {
