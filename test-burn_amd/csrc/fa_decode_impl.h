@@ -125,10 +125,10 @@ __device__ __forceinline__ float dpp_mov(float v) {
 }
 template <int G, bool MAX>
 __device__ __forceinline__ float group_reduce(float v) {
-    static_assert(G == 4 || G == 8 || G == 32, "group sizes in use");
+    static_assert(G == 2 || G == 4 || G == 8 || G == 32, "group sizes in use");
     auto op = [](float x, float y) { return MAX ? fmaxf(x, y) : x + y; };
     v = op(v, dpp_mov<0xB1>(v));               // quad_perm [1,0,3,2]: lane ^ 1
-    v = op(v, dpp_mov<0x4E>(v));               // quad_perm [2,3,0,1]: lane ^ 2
+    if (G >= 4) v = op(v, dpp_mov<0x4E>(v));   // quad_perm [2,3,0,1]: lane ^ 2
     if (G >= 8) v = op(v, dpp_mov<0x141>(v));  // row_half_mirror: the other quad of the 8 lanes
     if (G >= 32) {
         v = op(v, dpp_mov<0x140>(v));          // row_mirror: the other half of the row
@@ -976,15 +976,20 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     l_run += xor16(l_run);
     l_run += xor32(l_run);
 
-    // fold the NW waves through LDS: sm_acc[wave][head][D], sm_ml[wave][head][2]
-    __syncthreads();  // every wave is done with its V region
-    float *sm_acc = reinterpret_cast<float *>(smem);
-    float *sm_ml = sm_acc + (size_t)NW * gt * D;
+    // Fold of the NW waves through LDS: sm_acc[wave][head][D] (+ 8 floats per wave, see below), sm_ml[wave][head][2].
+    // With up to 4 heads the states have a region of their own, so a wave writes its state as soon as it is done (the
+    // waves finish spread over the streaming time) and only the last wave's write is left before the barrier; with
+    // more heads the region would not fit beside the V tiles and reuses them once every wave is done with them.
+    const bool own_region = gt <= 4;
+    if (!own_region) __syncthreads();  // every wave is done with its V region
+    float *sm_acc = own_region ? reinterpret_cast<float *>(rope_lds + 2 * D) : reinterpret_cast<float *>(smem);
+    const uint32_t wstr = gt * D + 8;  // a wave pair is 2 wstr apart: 64 bytes off a multiple of the bank span
+    float *sm_ml = sm_acc + (size_t)NW * wstr;
     if ((uint32_t)n < gt) {
 #pragma unroll
         for (int blk = 0; blk < DBLK; ++blk)
-            *reinterpret_cast<f4_t *>(sm_acc + ((size_t)wave * gt + n) * D + blk * 16 + c * 4) = oacc[blk];
-        if (c == 0) sm_ml[(wave * gt + n) * 2] = m_run, sm_ml[(wave * gt + n) * 2 + 1] = l_run;
+            *reinterpret_cast<f4_t *>(sm_acc + (size_t)wave * wstr + n * D + blk * 16 + c * 4) = oacc[blk];
+        if (c == 0) *reinterpret_cast<f2_t *>(sm_ml + (wave * gt + n) * 2) = f2_t{m_run, l_run};
     }
     __syncthreads();
 
@@ -992,21 +997,25 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     const size_t gbase = ((size_t)b * gridDim.y + y) * S * gt;  // first row of this (sequence, head group)
     const uint32_t prow = split * gt;
     constexpr int CG = D / 4;
-    // NW consecutive lanes share a column (head h, float4 column c4): lane w reads wave w's state, the group merges,
-    // and its first lane owns the result.
-    const int wsel = tid % NW;
-    for (int base = 0; base < (int)gt * CG * NW; base += NT) {  // uniform over the workgroup
-        const int idx = (base + tid) / NW;
+    // LPC = NW / 2 consecutive lanes share a column (head h, float4 column c4): lane j merges the states of waves 2j and
+    // 2j + 1, the group merges its lanes' results, and its first lane owns the column's state. One pass for up to 4 heads.
+    constexpr int LPC = NW / 2;
+    const int wsel = tid % LPC;
+    for (int base = 0; base < (int)gt * CG * LPC; base += NT) {  // uniform over the workgroup
+        const int idx = (base + tid) / LPC;
         const bool valid = idx < (int)gt * CG;
         const int h = valid ? idx / CG : 0, c4 = valid ? idx % CG : 0;
-        const float m_w = sm_ml[(wsel * gt + h) * 2], l_w = sm_ml[(wsel * gt + h) * 2 + 1];
-        const f4_t a_w = *reinterpret_cast<const f4_t *>(sm_acc + ((size_t)wsel * gt + h) * D + c4 * 4);
-        float ms = group_reduce<NW, true>(m_w);
-        const float e = fast_exp2(m_w - ms);
-        float L = group_reduce<NW, false>(l_w * e);
+        const f2_t ml0 = *reinterpret_cast<const f2_t *>(sm_ml + ((2 * wsel) * gt + h) * 2);
+        const f2_t ml1 = *reinterpret_cast<const f2_t *>(sm_ml + ((2 * wsel + 1) * gt + h) * 2);
+        const f4_t a0 = *reinterpret_cast<const f4_t *>(sm_acc + (size_t)(2 * wsel) * wstr + h * D + c4 * 4);
+        const f4_t a1 = *reinterpret_cast<const f4_t *>(sm_acc + (size_t)(2 * wsel + 1) * wstr + h * D + c4 * 4);
+        const float m_w = fmaxf(ml0.x, ml1.x);
+        const float ms = group_reduce<LPC, true>(m_w);
+        const float e0 = fast_exp2(ml0.x - ms), e1 = fast_exp2(ml1.x - ms);
+        const float L = group_reduce<LPC, false>(ml0.y * e0 + ml1.y * e1);
         f4_t A;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) A[i] = group_reduce<NW, false>(a_w[i] * e);
+        for (int i = 0; i < 4; ++i) A[i] = group_reduce<LPC, false>(a0[i] * e0 + a1[i] * e1);
         if (!valid || wsel != 0) continue;
         if (nsplits == 1) {
             const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 1.0f;
@@ -1101,8 +1110,10 @@ enum Mode { MODE_PLAIN = 0, MODE_PAGED = 1, MODE_SAGE = 2, MODE_FUSED = 3, MODE_
 template <int D>
 size_t decode_lds_bytes(uint32_t gt) {
     // the per-wave V blocks + the Q^T operand + one RoPE table row
-    const size_t v_tiles = (size_t)NW * MBX * BK * (D * 2 + 32) + (size_t)(D / 32) * 64 * 16 + 2 * D;
-    const size_t fold = ((size_t)NW * gt * D + (size_t)NW * gt * 2) * sizeof(float);
+    // ... + the waves' states at the end of the block loop, for up to 4 heads (more heads reuse the V tiles)
+    const size_t v_tiles = (size_t)NW * MBX * BK * (D * 2 + 32) + (size_t)(D / 32) * 64 * 16 + 2 * D +
+                           (size_t)NW * (4 * D + 8) * sizeof(float) + (size_t)NW * 4 * 2 * sizeof(float);
+    const size_t fold = ((size_t)NW * (gt * D + 8) + (size_t)NW * gt * 2) * sizeof(float);
     const size_t merge = (size_t)NT * 6 * sizeof(float) * POLL_IPT;  // the cooperative merge holds POLL_IPT records per thread
     size_t m = v_tiles > fold ? v_tiles : fold;
     return m > merge ? m : merge;
