@@ -874,7 +874,7 @@ def main():
     ap.add_argument("--cpu-sample-seconds", type=float, default=12.0)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--keys-per-split", type=int, default=0)
-    ap.add_argument("--merge", type=int, default=1)
+    ap.add_argument("--merge", type=int, default=2)
     ap.add_argument("--unfused", action="store_true", help="two launches per layer (KvPrepFused, FlashAttention)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a copy kernel of known size (reference point for profiler HBM counters)")

@@ -231,8 +231,9 @@ fa_status fa_decode_step_fused(fa_ctx *ctx, const fa_tensor_arg *q, const fa_ten
                                const uint32_t *d_position, uint32_t kv_len_bound);
 
 /* fa_decode_step_fused for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
- * that forbid hipMalloc). No counterpart in the reference. Same arguments, same kernels, same results bit for bit; the
- * difference is where the partition partials live: in a static device array of fa_noalloc_scratch_bytes() (4 MiB) that
+ * that forbid hipMalloc). No counterpart in the reference. Same arguments, same kernels and the same results bit for bit
+ * as fa_decode_step_fused with the two-launch merge (fa_set_decode_variant merge = 1; within one f16 unit in the last
+ * place of the other merge forms); the difference is where the partition partials live: in a static device array of fa_noalloc_scratch_bytes() (4 MiB) that
  * every GPU the library runs on holds until the process ends, instead of the context's grow-only workspace. The call
  * performs no hipMalloc / hipFree and no allocating library routine, at its first use on a device included (the array's
  * address is looked up in fa_ctx_create). The partitions are always merged by the second launch (no arrival counters).
@@ -252,9 +253,18 @@ size_t fa_noalloc_scratch_bytes(void);
 /* Tuning override, the counterpart of FlashDecodeVariant + METALLIC_FA_DECODE_* (src/metals/flashattention/
  * variants.rs:36-140). keys_per_split: context partition per workgroup (rounded up to the kernel's 16-key
  * block; 0 = auto: one partition per compute unit).
- * merge: 0 = merged by the last workgroup to finish (one launch), 1 = separate merge kernel (the default of a
- * new context: measured slightly faster).
- * Environment: FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT, FOUNDRY_ATTN_DECODE_MERGE (read at fa_ctx_create). */
+ * merge: 0 = merged by the last workgroup to finish (one launch, an arrival ticket); 1 = separate merge kernel;
+ * 2 (the default of a new context) = polled: every partition's workgroup stores its partial state as records in a
+ * buffer whose words hold an arrival pattern between launches, then merges a share of the output columns itself as soon
+ * as the other partitions' records have arrived (one launch, no ticket, the reads spread over all compute units;
+ * a head group's workgroups are placed on one XCD where the launch allows, so the records meet in that XCD's L2). It
+ * applies to launches whose workgroups are all resident at once (at most one 8-wave or two 4-wave workgroups per compute
+ * unit; others take 1). A merging workgroup waits at most FOUNDRY_ATTN_DECODE_POLL_SPIN_US (default 2 s) for the other
+ * partitions; beyond that it stores nothing and the next fa_synchronize fails with FA_ERR_OPERATION_FAILED (the outputs
+ * of the decode calls since the previous synchronize are then invalid). The three forms fold the same partials in
+ * different f32 orders and agree to one f16 unit in the last place; each is deterministic.
+ * Environment: FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT, FOUNDRY_ATTN_DECODE_MERGE, FOUNDRY_ATTN_DECODE_POLL_SPIN_US,
+ * FOUNDRY_ATTN_DECODE_XCD_LOCAL (0 = records always through memory) (read at fa_ctx_create). */
 typedef struct fa_decode_variant {
     uint32_t keys_per_split;
     uint32_t merge;

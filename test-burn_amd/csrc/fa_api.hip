@@ -101,8 +101,8 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
         return fa_fail(FA_ERR_OPERATION_FAILED, "hipStreamCreate failed: %s", hipGetErrorString(e));
     }
     ctx->decode_variant.keys_per_split = env_u32("FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT", 0);
-    ctx->decode_variant.merge = env_u32("FOUNDRY_ATTN_DECODE_MERGE", 1);
-    if (ctx->decode_variant.merge > 2) ctx->decode_variant.merge = 1;
+    ctx->decode_variant.merge = env_u32("FOUNDRY_ATTN_DECODE_MERGE", 2);
+    if (ctx->decode_variant.merge > 2) ctx->decode_variant.merge = 2;
     ctx->decode_waves = env_u32("FOUNDRY_ATTN_DECODE_WAVES", 0);
     if (ctx->decode_waves != 4 && ctx->decode_waves != 8) ctx->decode_waves = 0;
     ctx->gemm_min_m = env_u32("FOUNDRY_ATTN_GEMM_MIN_M", 0);
@@ -116,7 +116,6 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     if (s == FA_OK) s = fa_ensure_counters(ctx, 4096);
     if (s == FA_OK) s = fa_decode_probe_xcd(ctx);
     if (s == FA_OK && env_u32("FOUNDRY_ATTN_DECODE_XCD_LOCAL", 1) == 0) ctx->xcd_round_robin = false;
-    if (env_u32("FOUNDRY_ATTN_DEBUG", 0)) fprintf(stderr, "[foundry_attn] xcd round robin: %d\n", (int)ctx->xcd_round_robin);
     if (s == FA_OK) s = fa_decode_static_scratch(device, &ctx->static_scratch, &ctx->static_scratch_bytes);
     if (s == FA_OK) {
         // Records of the polled merge: room for two workgroups per compute unit serving 16 heads of 128 dims each (32 B per float4 column)
@@ -180,7 +179,8 @@ extern "C" fa_status fa_synchronize(fa_ctx *ctx) {
         *ctx->h_status = 0;
         if (bits & FA_DEVSTAT_MERGE_TIMEOUT) {
             // the buffer no longer holds the arrival pattern everywhere: restore it before anything else runs
-            (void)hipMemset(ctx->poll_ws, 0xff, ctx->poll_ws_bytes);
+            (void)hipMemsetAsync(ctx->poll_ws, 0xff, ctx->poll_ws_bytes, ctx->stream);
+            (void)hipStreamSynchronize(ctx->stream);
             return fa_fail(FA_ERR_OPERATION_FAILED,
                            "a decode launch's merging workgroup waited longer than %u us for the other partitions; the "
                            "outputs of the decode calls since the last synchronize are invalid", ctx->poll_spin_us);

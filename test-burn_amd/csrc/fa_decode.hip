@@ -48,11 +48,6 @@ fa_status fa_decode_probe_xcd(fa_ctx *ctx) {
     // the first workgroup of a launch continues where the previous launch stopped: only the step of one XCD per id matters
     for (uint32_t i = 0; i < n; ++i) ok = ok && h[i] < 8u && h[i] == ((h[0] + i) & 7u);
     ctx->xcd_round_robin = ok;
-    if (getenv("FOUNDRY_ATTN_DEBUG")) {
-        fprintf(stderr, "[foundry_attn] xcd of workgroups:");
-        for (uint32_t i = 0; i < n && i < 40; ++i) fprintf(stderr, " %u", h[i]);
-        fprintf(stderr, "\n");
-    }
     return FA_OK;
 }
 

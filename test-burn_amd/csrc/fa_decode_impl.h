@@ -142,6 +142,12 @@ __device__ __forceinline__ float group_reduce(float v) {
 // bits (write-through to, and read from, the device-wide coherence point) instead of a cache-wide
 // write-back + invalidate around ordinary accesses.
 constexpr int CACHE_COHERENT = 0x11;  // sc0 | sc1
+// Cache rows are read once per launch: marked non-temporal, they do not push the kernel's code and the partial
+// records out of the L2.
+#ifndef FA_STREAM_POLICY
+#define FA_STREAM_POLICY 2
+#endif
+constexpr int STREAM_POLICY = FA_STREAM_POLICY;  // nt
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, 0xffffffff, 0x00020000);
 }
@@ -601,11 +607,12 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
 #pragma unroll
                 for (int j = 0; j < KSTEPS; ++j)
                     kk[mb][j].u = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                                krs, k_lane_off + j * 64, (int)(row0 * (uint32_t)(D * KES)), 0));
+                                                                krs, k_lane_off + j * 64, (int)(row0 * (uint32_t)(D * KES)), STREAM_POLICY));
             } else {
                 const unsigned char *blk0 = kbase + page_row(pgi[mb], row0) * KES;  // wave-uniform
 #pragma unroll
-                for (int j = 0; j < KSTEPS; ++j) kk[mb][j].u = *reinterpret_cast<const uint4 *>(blk0 + k_lane_off + j * 64);
+                for (int j = 0; j < KSTEPS; ++j)
+                    kk[mb][j].i = __builtin_nontemporal_load(reinterpret_cast<const i4_t *>(blk0 + k_lane_off + j * 64));
             }
         }
     };
@@ -619,10 +626,10 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                 if (!PAGED) {
                     vv[mb][i].u = __builtin_bit_cast(
                         uint4, __builtin_amdgcn_raw_buffer_load_b128(vrs, v_lane_off + i * VRPL * (D * 2),
-                                                                     (int)(row0 * (uint32_t)(D * 2)), 0));
+                                                                     (int)(row0 * (uint32_t)(D * 2)), STREAM_POLICY));
                 } else {
                     const unsigned char *blk0 = reinterpret_cast<const unsigned char *>(vbase + page_row(pgi[mb], row0));
-                    vv[mb][i].u = *reinterpret_cast<const uint4 *>(blk0 + v_lane_off + i * VRPL * (D * 2));
+                    vv[mb][i].i = __builtin_nontemporal_load(reinterpret_cast<const i4_t *>(blk0 + v_lane_off + i * VRPL * (D * 2)));
                 }
             }
         }
@@ -961,15 +968,20 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         __half *kw = const_cast<__half *>(reinterpret_cast<const __half *>(kbase)) + row_offset(p);
         __half *vw = const_cast<__half *>(vbase) + row_offset(p);
 #pragma unroll
-        for (int j = 0; j < KSTEPS; ++j) {
-            kk[0][j].u = n == 0 ? knew[j].u : make_uint4(0, 0, 0, 0);
-            if (writer && n == 0) *reinterpret_cast<uint4 *>(kw + (4 * j + c) * 8) = knew[j].u;
-        }
+        for (int j = 0; j < KSTEPS; ++j) kk[0][j].u = n == 0 ? knew[j].u : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < VLB; ++i) vv[0][i].u = make_uint4(0, 0, 0, 0);
-        vv[0][0] = vv[1][0];
-        if (writer && lane < VLPR) *reinterpret_cast<uint4 *>(vw + lane * 8) = vv[0][0].u;
+        const uint4 vnew = vv[1][0].u;
+        vv[0][0].u = vnew;
         consume(p, 1, p + 1, 0, 0);
+        // The cache rows are stored after the token has been attended: a wait for loaded registers inside the block
+        // code would otherwise wait for these stores' acknowledgements as well (microseconds while the launch streams).
+        __builtin_amdgcn_sched_barrier(0);
+        if (writer && n == 0) {
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j) *reinterpret_cast<uint4 *>(kw + (4 * j + c) * 8) = knew[j].u;
+        }
+        if (writer && lane < VLPR) *reinterpret_cast<uint4 *>(vw + lane * 8) = vnew;
     }
 
     // the head's sum over the four 16-lane rows (the running max is already common to them)

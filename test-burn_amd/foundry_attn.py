@@ -289,7 +289,7 @@ class Foundry:
     def reserve_workspace(self, nbytes):
         check(self.lib.fa_ctx_reserve_workspace(self.h, nbytes))
 
-    def set_decode_variant(self, keys_per_split=0, merge=1):
+    def set_decode_variant(self, keys_per_split=0, merge=2):
         """No arguments: the library's defaults (partition size by the launch rule, separate merge kernel)."""
         v = DecodeVariant(keys_per_split, merge)
         check(self.lib.fa_set_decode_variant(self.h, C.byref(v)))

@@ -62,7 +62,7 @@ def test_decode_ragged_lengths_and_splits(N, D, H, Hkv):
     k[:, N:], v[:, N:] = np.float16(np.nan), np.float16(np.nan)  # rows past kv_len must never contribute
     want = orc.sdpa_decode(q, k, v, H, Hkv, D, cap, N).reshape(H, D)
     try:
-        for kps, merge in [(0, 0), (64, 0), (64, 1), (128, 0), (1024, 1)]:
+        for kps, merge in [(0, 0), (64, 0), (64, 1), (128, 0), (1024, 1), (0, 2), (64, 2), (128, 2), (1024, 2)]:
             f.set_decode_variant(kps, merge)
             got = gpu_decode(q, k, v, H, D, N)
             assert np.all(np.isfinite(got)), (kps, merge)
@@ -316,3 +316,85 @@ def test_in_kernel_merge_equals_merge_kernel_over_many_launches():
                     assert np.all(np.abs(g - a) <= np.maximum(np.abs(a), 2.0 ** -14) * 2.0 ** -10), (kps, n)
     finally:
         f.set_decode_variant()
+
+
+def test_polled_merge_equals_merge_kernel_over_many_launches():
+    """The polled merge (every partition's workgroup merges a share of the columns as soon as the other partitions'
+    records have arrived in the pattern-filled buffer) against the two-launch merge: one f16 unit in the last place
+    (another f32 order), the same bits on every repetition, and the buffer is left ready for the next launch - a
+    record that was not reset, or one taken before it had arrived, would show in one of the checks. Launch shapes on
+    both sides of what the polled form takes (it needs all workgroups resident at once)."""
+    announce("polled merge stress")
+    f = ctx()
+    rng = np.random.default_rng(321)
+    for H, Hkv, D, cap in [(24, 8, 128, 4096), (14, 2, 64, 2048), (16, 4, 128, 8192), (32, 32, 128, 1024), (16, 1, 64, 4096)]:
+        q = h16(rng.normal(size=(H, D)))
+        k = h16(rng.normal(size=(Hkv, cap, D)))
+        v = h16(rng.normal(size=(Hkv, cap, D)))
+        dq, dk, dv = f.array(q), f.array(k), f.array(v)
+        oa, ob = f.zeros((1, H * D)), f.zeros((1, H * D))
+        lens = [int(x) for x in rng.integers(17, cap, size=12)] + [cap, min(cap, 64 * 17 + 1)]
+        try:
+            for kps in (0, 64, 256):
+                for n in lens:
+                    f.set_decode_variant(kps, 1)
+                    f.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), oa.arg(), True, n - 1, H, D, n, 1)
+                    f.set_decode_variant(kps, 2)
+                    a = oa.download().astype(np.float32)
+                    first = None
+                    for _ in range(3):
+                        f.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), ob.arg(), True, n - 1, H, D, n, 1)
+                        f.synchronize()
+                        got = ob.download()
+                        if first is None:
+                            first = bits(got)
+                        assert np.array_equal(bits(got), first), (H, Hkv, D, kps, n)
+                        g = got.astype(np.float32)
+                        assert np.all(np.abs(g - a) <= np.maximum(np.abs(a), 2.0 ** -14) * 2.0 ** -10), (H, Hkv, D, kps, n)
+        finally:
+            f.set_decode_variant()
+        for b in (dq, dk, dv, oa, ob):
+            b.free()
+
+
+def test_polled_merge_gives_up_cleanly():
+    """Failure handling of the polled merge, forced from the host: with a wait bound of zero a merging workgroup gives
+    up at its first look unless every record is already there. Every kernel still ends normally; the next synchronize
+    reports OperationFailed and restores the buffer; a context with the normal bound computes the right result."""
+    import os
+    announce("polled merge, zero wait bound")
+    H, Hkv, D, cap, n = 24, 8, 128, 4096, 4000
+    rng = np.random.default_rng(77)
+    q, k, v = h16(rng.normal(size=(H, D))), h16(rng.normal(size=(Hkv, cap, D))), h16(rng.normal(size=(Hkv, cap, D)))
+    want = orc.sdpa_decode(q, k, v, H, Hkv, D, cap, n).reshape(H, D)
+    os.environ["FOUNDRY_ATTN_DECODE_POLL_SPIN_US"] = "0"
+    try:
+        g = fa.Foundry(0)
+    finally:
+        del os.environ["FOUNDRY_ATTN_DECODE_POLL_SPIN_US"]
+    try:
+        g.set_decode_variant(0, 2)
+        dq, dk, dv, do = g.array(q), g.array(k), g.array(v), g.zeros((1, H * D))
+        failures = 0
+        for _ in range(4):
+            g.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), do.arg(), True, n - 1, H, D, n, 1)
+            try:
+                g.synchronize()
+                assert max_abs(do.download().reshape(H, D), want) <= TOL  # nobody had to wait: the result must be right
+            except fa.FoundryError as e:
+                failures += 1
+                assert e.variant == "OperationFailed" and "waited longer" in str(e)
+        # the two-launch merge of the same context is unaffected
+        g.set_decode_variant(0, 1)
+        g.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), do.arg(), True, n - 1, H, D, n, 1)
+        g.synchronize()
+        assert max_abs(do.download().reshape(H, D), want) <= TOL
+    finally:
+        g.close()
+    f = ctx()
+    f.set_decode_variant(0, 2)
+    try:
+        got = gpu_decode(q, k, v, H, D, n)
+    finally:
+        f.set_decode_variant()
+    assert max_abs(got, want) <= TOL

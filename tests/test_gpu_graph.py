@@ -88,7 +88,7 @@ def _split_decode_state(f, rng, H, Hkv, D, cap, start):
     return (cos, sin, kc, vc, q, k, v), dev
 
 
-@pytest.mark.parametrize("merge", [1, 0], ids=["merge_kernel", "merge_in_kernel"])
+@pytest.mark.parametrize("merge", [1, 0, 2], ids=["merge_kernel", "merge_in_kernel", "merge_polled"])
 def test_graph_survives_workspace_growth(merge):
     """A recorded split decode addresses the workspace (and the arrival counters) it was captured against. Growing the
     workspace afterwards must leave that buffer alive for the graph: replays before and after the growth equal the

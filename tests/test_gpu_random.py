@@ -22,7 +22,7 @@ def test_random_fused_decode_step(seed):
     pos = int(rng.integers(0, 3000))
     cap = (pos + 1 + int(rng.integers(0, 300)) + 15) // 16 * 16
     kps = int(rng.choice([0, 0, 64, 128, 256, 1024]))
-    merge = int(rng.integers(0, 2))
+    merge = int(rng.integers(0, 3))
     mode = int(rng.choice([fa.ROPE_NEOX, fa.ROPE_NORMAL]))
     step = int(rng.choice([0, 0, 4]))
     layer = int(rng.integers(0, 8))
