@@ -29,6 +29,17 @@ import foundry_attn as fa  # noqa: E402
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, AMD's published figure
 GRAPH_STEPS = 16
 
+_COLLECT = None  # a list while the default run gathers the other configurations' lines instead of printing them
+
+
+def emit(result):
+    """A workload's JSON line: printed, or kept for the default run's "configs" object."""
+    if _COLLECT is not None:
+        _COLLECT.append(result)
+    else:
+        print(json.dumps(result))
+
+
 
 def make_llama3b_decode(f, rng, start_ctx, room):
     """Allocates and fills the 28-layer Llama-3.2-3B-shaped decode state; returns a dict of device buffers."""
@@ -115,31 +126,44 @@ def run_steps(f, st, graph16, graph1, steps, room, history=None):
 
 def cpu_baseline(st, sample_seconds, room):
     """The oracle (scalar C restatement of the reference arithmetic, OpenMP over heads) on the same workload: decode
-    steps of the timed window over 2 of the 28 layers for about sample_seconds of wall time, scaled to 28 layers."""
+    steps of the timed window over 2 of the 28 layers, scaled to 28 layers; once on one thread and once on every host
+    core the process may use (about a third and two thirds of sample_seconds of wall time)."""
     import orc
 
-    threads = max(1, min(16, os.cpu_count() or 1, orc.lib().orc_max_threads()))
+    host_cpus = os.cpu_count() or 1
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        usable = host_cpus
+    all_threads = max(1, min(usable, orc.lib().orc_max_threads()))
     L, H, Hkv, D, cap, start = st["L"], st["H"], st["Hkv"], st["D"], st["cap"], st["start"]
     layers = len(st["host_kv"])
-    kv = [(k.copy(), v.copy()) for k, v in st["host_kv"]]
-    done = 0
-    t0 = time.perf_counter()
-    while True:
-        s = done % room
-        for i in range(layers):
-            k, v = kv[i]
-            qr = orc.kv_prep_fused(st["q_h"][s % GRAPH_STEPS, i:i + 1], st["k_h"][s % GRAPH_STEPS, i:i + 1],
-                                   st["v_h"][s % GRAPH_STEPS, i:i + 1], k, v, st["cos_h"], st["sin_h"],
-                                   orc.make_params(H, Hkv, D, 1, start + s, cap, rope_mode=1))
-            orc.sdpa_decode(qr[:, 0].copy(), k, v, H, Hkv, D, cap, start + s + 1, n_threads=threads)
-        done += 1
-        dt = time.perf_counter() - t0
-        if dt >= sample_seconds:
-            break
-    per_step = dt / done * (L / layers)
-    return {"value": 1.0 / per_step, "unit": "steps/s", "cores": threads, "kind": "port",
-            "sample": "%d decode steps x %d of %d layers from kv_len %d, scaled to %d layers (%.1f s wall on %d threads)"
-                      % (done, layers, L, start + 1, L, dt, threads)}
+
+    def sample(threads, seconds):
+        kv = [(k.copy(), v.copy()) for k, v in st["host_kv"]]
+        done = 0
+        t0 = time.perf_counter()
+        while True:
+            s = done % room
+            for i in range(layers):
+                k, v = kv[i]
+                qr = orc.kv_prep_fused(st["q_h"][s % GRAPH_STEPS, i:i + 1], st["k_h"][s % GRAPH_STEPS, i:i + 1],
+                                       st["v_h"][s % GRAPH_STEPS, i:i + 1], k, v, st["cos_h"], st["sin_h"],
+                                       orc.make_params(H, Hkv, D, 1, start + s, cap, rope_mode=1))
+                orc.sdpa_decode(qr[:, 0].copy(), k, v, H, Hkv, D, cap, start + s + 1, n_threads=threads)
+            done += 1
+            dt = time.perf_counter() - t0
+            if dt >= seconds:
+                break
+        per_step = dt / done * (L / layers)
+        return {"value": 1.0 / per_step, "unit": "steps/s", "cores": threads, "host_cpus": host_cpus, "kind": "port",
+                "sample": "%d decode steps x %d of %d layers from kv_len %d, scaled to %d layers (%.1f s wall on %d thread%s)"
+                          % (done, layers, L, start + 1, L, dt, threads, "" if threads == 1 else "s")}
+
+    one = sample(1, sample_seconds / 3.0)
+    many = sample(all_threads, sample_seconds * 2.0 / 3.0)
+    many["one_thread"] = one
+    return many
 
 
 def check_against_oracle(f, st, history):
@@ -161,10 +185,37 @@ def check_against_oracle(f, st, history):
     return cache_ok, err
 
 
-# HBM bytes per launch of the fused decode kernel from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
-# profiles/decode_llama3b_8k_hbm_counters.txt (scaled by the copy kernel of known size); a counter run cannot be made
-# from inside this script, so the figure is carried here and re-measured whenever the kernel changes.
-MEASURED_TRAFFIC_BYTES = 35.15e6
+# HBM bytes per launch of the fused decode kernel come from the FETCH_SIZE / WRITE_SIZE counter runs summarised in
+# profiles/decode_llama3b_8k_hbm_counters.txt (a counter run cannot be made from inside this script). The summary names
+# the hash of the kernel sources it was measured on: when those have changed since, the figure is reported as null.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "decode_llama3b_8k_hbm_counters.txt")
+KERNEL_SOURCES = ["fa_decode_impl.h", "fa_decode.hip", "fa_internal.h"]
+
+
+def kernel_source_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "test-burn_amd", "csrc", name), "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic():
+    """(bytes per launch or None, note) from the `traffic_bytes_per_launch=` / `kernel_source_sha256_16=` lines of the
+    committed counter summary."""
+    import re
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None, "no counter summary"
+    m_b = re.search(r"^traffic_bytes_per_launch=([0-9.eE+]+)", text, re.M)
+    m_h = re.search(r"^kernel_source_sha256_16=([0-9a-f]{16})", text, re.M)
+    if not m_b or not m_h:
+        return None, "counter summary carries no machine-readable figure"
+    if m_h.group(1) != kernel_source_hash():
+        return None, "counter summary is for kernel sources %s, these are %s" % (m_h.group(1), kernel_source_hash())
+    return float(m_b.group(1)), "profiles/decode_llama3b_8k_hbm_counters.txt"
 
 
 def calibration_copy(f, reps=3):
@@ -262,7 +313,7 @@ def bench_prefill(f, args):
                    "frac_of_hbm_peak": append_bytes / (ms_kp / 1e3 / max(1, n_kp)) / 1e9 / HBM_PEAK_GBPS},
         "parity": {"cache_bit_exact": bool(cache_ok), "prefill_max_abs_err_last64": err},
     }
-    print(json.dumps(result))
+    emit(result)
     if not cache_ok or err > 2e-3:
         sys.exit("parity check failed: cache_bit_exact=%s prefill_max_abs_err=%g" % (cache_ok, err))
 
@@ -282,7 +333,7 @@ def _finish_secondary(f, args, name, workload, kernel, bytes_per_launch, dt, par
     }
     if extra:
         result.update(extra)
-    print(json.dumps(result))
+    emit(result)
 
 
 def bench_small_decode(f, args):
@@ -494,7 +545,7 @@ def bench_fused_qkv_chunk(f, args, m, q8=False):
                 "frac": flops / total_s / 1e12 / MFMA_F16_PEAK_TFLOPS, "flops_per_step": flops}
     roof.update({"traffic": None, "kernel": "rmsnorm_rows_kernel + fused_qkv_gemm_kernel (+ gemm_finish_kernel)",
                  "avg_launch_us": us, "launches": kernels["fused_qkv_gemm_kernel"][0]})
-    print(json.dumps({
+    emit(({
         "metric": "FusedQkv chunk-steps/s, Llama-3.2-3B prefill chunk of %d tokens" % m, "value": args.steps / dt,
         "unit": "chunk-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
@@ -647,7 +698,7 @@ def bench_attn_block(f, args):
     finite = bool(np.all(np.isfinite(hid[0].download())))
     nbytes = L * (2.0 * (dm + 2 * kvd) * dm + 2.0 * dm * dm + 2.0 * 2 * Hkv * (pos + 1) * D)
     per_step = dt / args.steps
-    print(json.dumps({
+    emit(({
         "metric": "attention-block steps/s + achieved HBM GB/s, Llama-3.2-3B decode @8K ctx", "value": 1.0 / per_step,
         "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": per_step * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
@@ -709,7 +760,7 @@ def bench_prefill_block(f, args):
     finite = bool(np.all(np.isfinite(dout.download())))
     flops = 2.0 * M * (dm + 2 * kvd) * dm + 4.0 * D * H * M * (M + 1) / 2 + 2.0 * M * dm * dm
     total_s = sum(us.values()) * 1e-6
-    print(json.dumps({
+    emit(({
         "metric": "attention-block layer-steps/s, Llama-3.2-3B prefill of 2048 tokens", "value": args.steps / dt,
         "unit": "layer-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
@@ -851,7 +902,61 @@ def bench_sage_decode(f, args):
     f.profile_enable(False)
 
 
-SECONDARY = {"llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
+def bench_floors(f, args):
+    """What a launch of this size costs with the library's simplest kernels, for reading the decode figures against: an
+    (almost) empty launch, and plain copies that move as many bytes as one decode launch reads (Llama-3.2-3B layer at
+    8K: 33.6 MB) and as the paged batch's launch reads (240 MB). All through the C ABI, in HIP graphs, buffers rotated
+    so that nothing is served from the last-level cache."""
+    Hkv, D = 8, 128
+    out = {"metric": "launch and copy floors", "unit": "us", "n_gpus": 1, "config": {"workload": "floors"}, "floors": {}}
+    word = f.array(np.zeros(4, np.uint32))
+    n_launch = 256
+    f.start_capture()
+    for _ in range(n_launch):
+        f.u32_add(word, 1, 1)
+    g = f.end_capture()
+    for _ in range(3):
+        g.launch()
+    f.synchronize()
+    reps = 10
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        g.launch()
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    g.destroy()
+    out["floors"]["launch"] = {"kernel": "u32_add_kernel (one workgroup)", "us_per_launch": dt / (reps * n_launch) * 1e6,
+                               "what": "back-to-back dependent launches of a one-workgroup kernel in a HIP graph"}
+    for name, rows, n_rot in (("copy_33.6MB", 8192, 28), ("copy_240MB", 58594, 8)):
+        srcs = [f.zeros((Hkv, rows, D)) for _ in range(n_rot)]
+        dsts = [f.zeros((Hkv, rows, D)) for _ in range(n_rot)]
+        f.start_capture()
+        for s_, d_ in zip(srcs, dsts):
+            f.kv_prefix_copy(s_.arg(), d_.arg(), rows)
+        g = f.end_capture()
+        for _ in range(3):
+            g.launch()
+        f.synchronize()
+        reps = 20
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            g.launch()
+        f.synchronize()
+        dt = time.perf_counter() - t0
+        g.destroy()
+        moved = 2.0 * Hkv * rows * D * 2  # read + written
+        us = dt / (reps * n_rot) * 1e6
+        out["floors"][name] = {"kernel": "kv_prefix_copy_vec_kernel", "bytes_moved": moved, "us_per_launch": us,
+                               "gbps": moved / us / 1e3, "frac_of_hbm_peak": moved / us / 1e3 / HBM_PEAK_GBPS,
+                               "what": "fa_kv_prefix_copy of one [8, %d, 128] f16 tensor (half read, half written), %d "
+                                       "tensor pairs in rotation, HIP graph" % (rows, n_rot)}
+        for b in srcs + dsts:
+            b.free()
+    word.free()
+    emit(out)
+
+
+SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
              "llama3b_o_proj": bench_o_proj,
@@ -878,8 +983,8 @@ def main():
     ap.add_argument("--unfused", action="store_true", help="two launches per layer (KvPrepFused, FlashAttention)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run a copy kernel of known size (reference point for profiler HBM counters)")
-    ap.add_argument("--traffic-bytes", type=float, default=MEASURED_TRAFFIC_BYTES,
-                    help="measured HBM bytes per launch of the dominant kernel (from profiler counters) to report")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="only the headline workload: skip the other benchmark configurations and the floors")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path is built and measured on a single MI355X (--gpus 1); it uses no "
@@ -940,6 +1045,7 @@ def main():
     avg_n = st["start"] + (prof_steps + 1) / 2.0
     achieved = layer_bytes(st, avg_n) / avg_dec_s / 1e9
 
+    traffic, traffic_note = measured_traffic()
     ns = [st["start"] + 1 + (i % room) for i in range(args.steps)]
     bytes_total = sum(step_bytes(st, n) for n in ns)
     result = {
@@ -962,7 +1068,7 @@ def main():
         "whole_step_hbm_gbps": bytes_total / dt / 1e9,
         "whole_step_hbm_frac_of_peak": bytes_total / dt / 1e9 / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": args.traffic_bytes,
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_note,
                      "kernel": kernel, "avg_launch_us": avg_dec_s * 1e6, "launches": n_dec,
                      "bytes_per_launch": layer_bytes(st, avg_n),
                      "merge_kernel_avg_launch_us": (ms_mrg * 1e3 / n_mrg) if n_mrg else None},
@@ -970,11 +1076,38 @@ def main():
     }
     if args.calibration_copy:
         result["calibration_copy"] = calibration_copy(f)
+    graph16.destroy()
+    graph1.destroy()
+    for b in st["kc"] + st["vc"]:
+        b.free()
+    if not args.no_configs:
+        # the other benchmark configurations (one layer per step, a bounded number of steps each) and the floors, so that
+        # one run records them all; each is the same code as its --workload line
+        global _COLLECT
+        sub = argparse.Namespace(**vars(args))
+        sub.steps, sub.warmup = 100, 10
+        result["configs"], result["floors"] = {}, None
+        for tag, fn in (("C1_qwen05b_decode_1k", bench_small_decode), ("C3_qwen3b_paged_decode", bench_paged_decode),
+                        ("C4_llama3b_prefill_2k", bench_prefill), ("C5_smollm3_sage_decode_32k", bench_sage_decode),
+                        ("floors", bench_floors)):
+            _COLLECT = []
+            g = fa.Foundry(0)
+            try:
+                fn(g, sub)
+            finally:
+                g.close()
+            line, _COLLECT = _COLLECT[0], None
+            if tag == "floors":
+                result["floors"] = line["floors"]
+            else:
+                result["configs"][tag] = {k: line[k] for k in ("metric", "value", "unit", "steps", "ms_per_step", "dtype",
+                                                                "config", "roofline", "parity") if k in line}
+                for k in ("append",):
+                    if k in line:
+                        result["configs"][tag][k] = line[k]
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(st, args.cpu_sample_seconds, room)
     print(json.dumps(result))
-    graph16.destroy()
-    graph1.destroy()
     f.close()
     if not cache_ok or err > 2e-3:
         sys.exit("parity check failed: cache_bit_exact=%s decode_max_abs_err=%g" % (cache_ok, err))

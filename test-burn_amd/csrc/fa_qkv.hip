@@ -122,7 +122,8 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
             if constexpr (Q4) z = 0u;
             else if constexpr (Q8) z = u2v_t{0u, 0u};
             else z = h8_t{0, 0, 0, 0, 0, 0, 0, 0};
-            buf[i] = (ok && kb < nkb) ? *reinterpret_cast<const wreg_t *>(p0 + (size_t)kb * kb_stride) : z;
+            // weights are read once per launch: non-temporal, so that they do not push everything else out of the L2
+            buf[i] = (ok && kb < nkb) ? __builtin_nontemporal_load(reinterpret_cast<const wreg_t *>(p0 + (size_t)kb * kb_stride)) : z;
         }
     };
     // The first input row is requested before the weights (a CU's vector loads return in request order), then the
