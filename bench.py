@@ -837,9 +837,12 @@ def bench_paged_decode(f, args):
 
 
 def bench_sage_decode(f, args):
-    """SmolLM3-shaped decode with int8 Q/K (per-32-token scales, mean-smoothed K) at 32K context, one layer per step."""
+    """SmolLM3-shaped decode step with int8 Q/K (per-32-token scales, mean-smoothed K) at 32K context, one layer per
+    step: RoPE + append of the new token into the int8 cache (open block quantised anew) + int8 decode. Every 4th layer
+    skips RoPE (the model's rule); six layers' states in rotation."""
     import orc
     H, Hkv, D, N, NL = 16, 4, 128, 32768, 6
+    P = N - 1  # the new token's position
     rng = np.random.default_rng(0xF0DD + 5)
 
     def outliers(shape):
@@ -848,57 +851,78 @@ def bench_sage_decode(f, args):
         x[mask] = np.sign(x[mask]) * 8.0
         return x.astype(np.float16)
 
+    cos, sin = fa.rope_tables(5e6, D, N)
+    dcos, dsin = f.array(cos), f.array(sin)
     layers, host0 = [], None
     for i in range(NL):
         k, v = outliers((Hkv, N, D)), outliers((Hkv, N, D))
+        k[:, P:], v[:, P:] = 0, 0
         dk, dv = f.array(k), f.array(v)
-        dmean = f.zeros((Hkv, D), np.float32)
-        dkq, dks = f.zeros((Hkv, N, D), np.int8), f.zeros((Hkv, N // 32), np.float16)
-        f.sage_k_mean(dk, Hkv, N, D, N, dmean)
-        f.sage_quantize_k(dk, dmean, Hkv, N, D, 0, N, dkq, dks)
+        desc, bufs = fa.sage_cache(f, H, Hkv, N, D, dv)
+        f.sage_cache_build(dk, P, desc)
         f.synchronize()
         dk.free()
-        layers.append((dkq, dks, dv))
+        layers.append((desc, bufs))
         if i == 0:
             host0 = (k, v)
-    q = outliers((H, D))
-    dq, dqq, dqs, dout = f.array(q), f.zeros((H, D), np.int8), f.zeros((H,), np.float32), f.zeros((H * D,))
+    q, kn, vn = outliers((1, H * D)), outliers((1, Hkv * D)), outliers((1, Hkv * D))
+    dq, dkn, dvn, dout = f.array(q), f.array(kn), f.array(vn), f.zeros((H * D,))
+    params = [fa.KvPrepFusedParams.make(H, Hkv, D, 1, P, N, fa.ROPE_NEOX, layer_idx=i, no_rope_layer_step=4) for i in range(NL)]
 
     def step(i):
-        dkq, dks, dv = layers[i % NL]
-        f.sage_quantize_q(dq, H, D, dqq, dqs)
-        f.sage_decode(dqq, dqs, dkq, dks, dv, dout, H, Hkv, D, N, N)
+        f.sage_decode_step(dq.arg(), dkn.arg(), dvn.arg(), layers[i % NL][0], dcos.arg(), dsin.arg(), dout.arg(), params[i % NL])
 
     step(0)
     f.synchronize()
     got = dout.download().reshape(H, D).astype(np.float64)
-    kq, ks = layers[0][0].download(), layers[0][1].download()
-    qq, qs = orc.sage_quantize_q(q, H, D)
-    model = orc.sage_decode(qq, qs, kq, ks, host0[1], H, Hkv, D, N, N, n_threads=8).reshape(H, D).astype(np.float64)
+    # the checker: the oracle's f16 append, its quantiser with the state's mean, its int8 decode model
+    kc, vc = host0[0].copy(), host0[1].copy()
+    qr = orc.kv_prep_fused(q, kn, vn, kc, vc, cos, sin, orc.make_params(H, Hkv, D, 1, P, N, rope_mode=0, layer_idx=0, no_rope_layer_step=4))
+    mean = layers[0][1]["k_mean"].download()
+    want_kq, want_ks = orc.sage_quantize_k(kc, mean, Hkv, N, D, N)
+    state_ok = bool(np.array_equal(layers[0][1]["k_q"].download(), want_kq) and
+                    np.array_equal(layers[0][1]["k_scale"].download().view(np.uint16), want_ks.view(np.uint16)))
+    qq, qs = orc.sage_quantize_q(np.ascontiguousarray(qr[:, 0]), H, D)
+    model = orc.sage_decode(qq, qs, want_kq, want_ks, vc, H, Hkv, D, N, N, n_threads=8).reshape(H, D).astype(np.float64)
     err_model = float(np.max(np.abs(got - model)))
-    kf, vf, qf = host0[0].astype(np.float64), host0[1].astype(np.float64), q.astype(np.float64)
+    kf, vf, qf = kc.astype(np.float64), vc.astype(np.float64), qr[:, 0].astype(np.float64)
     full = np.zeros((H, D))
     for h in range(H):  # f16 SDPA on the unquantised tensors, in float64
         s_ = kf[h // (H // Hkv)] @ qf[h] / np.sqrt(D)
         w = np.exp(s_ - s_.max())
         full[h] = (w / w.sum()) @ vf[h // (H // Hkv)]
     err_full = float(np.max(np.abs(got - full)))
-    for i in range(args.warmup):
+    # timed as HIP-graph replays (two short launches per step: eager, the host's call overhead would be what is measured)
+    per_graph = 4 * NL
+    f.start_capture()
+    for i in range(per_graph):
         step(i)
+    graph = f.end_capture()
+    for _ in range(max(1, args.warmup // per_graph)):
+        graph.launch()
     f.synchronize()
+    reps = max(1, args.steps // per_graph)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        graph.launch()
+    f.synchronize()
+    dt = (time.perf_counter() - t0) * args.steps / (reps * per_graph)  # scaled to args.steps steps
+    graph.destroy()
+    # per-kernel times: an eager pass with events attached to the dispatches
     f.profile_reset()
     f.profile_enable(True)
-    t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(per_graph):
         step(i)
-    f.synchronize()
-    dt = time.perf_counter() - t0
+    n_ap, ms_ap = f.profile_query("sage_append_kernel")
     nbytes = float(Hkv * N * D + Hkv * (N // 32) * 2 + Hkv * N * D * 2 + 2 * H * D * 2)
     _finish_secondary(f, args, "int8-QK decode-attn layer-steps/s + achieved HBM GB/s, SmolLM3 shape @32K ctx",
-                      "smollm3 decode attention with int8 Q/K (K mean-smoothed, per-32-token f16 scales; f16 V), one layer per "
-                      "step, batch 1, H16/Hkv4/D128, kv_len 32768, 1% of entries at 8 sigma", "sage_decode_mfma_kernel",
-                      nbytes, dt, {"max_abs_err_vs_int8_cpu_model": err_model, "max_abs_err_vs_f16_sdpa_unquantised": err_full},
-                      {"dtype": "i8 (QK^T) / f16 (PV)"})
+                      "smollm3 decode step with int8 Q/K (K mean-smoothed with a fixed mean, per-32-token f16 scales; f16 V), one "
+                      "layer per step: RoPE (every 4th layer none) + append into the int8 cache + int8 decode, batch 1, "
+                      "H16/Hkv4/D128, kv_len 32768, 1% of entries at 8 sigma", "sage_decode_mfma_kernel",
+                      nbytes, dt, {"int8_state_bit_exact": state_ok, "max_abs_err_vs_int8_cpu_model": err_model,
+                                   "max_abs_err_vs_f16_sdpa_unquantised": err_full},
+                      {"dtype": "i8 (QK^T) / f16 (PV)",
+                       "append": {"kernel": "sage_append_kernel", "avg_launch_us": ms_ap * 1e3 / max(1, n_ap)}})
     f.profile_enable(False)
 
 
@@ -1102,7 +1126,7 @@ def main():
             else:
                 result["configs"][tag] = {k: line[k] for k in ("metric", "value", "unit", "steps", "ms_per_step", "dtype",
                                                                 "config", "roofline", "parity") if k in line}
-                for k in ("append",):
+                for k in ("append",):  # the append kernel of a configuration, where it is a launch of its own
                     if k in line:
                         result["configs"][tag][k] = line[k]
     if not args.no_cpu:

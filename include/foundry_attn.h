@@ -501,6 +501,43 @@ fa_status fa_sage_decode(fa_ctx *ctx, const void *q_q, const float *q_scale, con
                          const void *v, void *out, uint32_t n_heads, uint32_t n_kv_heads, uint32_t head_dim,
                          uint32_t capacity, uint32_t kv_len);
 
+/* The state of one layer for a decode session with int8 Q/K (all device memory, owned by the caller):
+ *   k_q      [n_kv_heads, capacity, head_dim] i8     k_scale [n_kv_heads, ceil(capacity / 32)] f16
+ *   k_tail   [n_kv_heads, 32, head_dim] f16          the exact (rotated) K rows of the open 32-row block
+ *   k_mean   [n_kv_heads, head_dim] f32              the smoothing offset, fixed when the state is built
+ *   v        [n_kv_heads, capacity, head_dim] f16    q_q [n_heads, head_dim] i8 and q_scale [n_heads] f32: the step's
+ *                                                    quantised query (scratch the step writes and reads) */
+typedef struct fa_sage_cache {
+    void *k_q, *k_scale, *k_tail, *v, *q_q;
+    float *k_mean, *q_scale;
+    uint32_t n_heads, n_kv_heads, capacity, head_dim;
+} fa_sage_cache;
+
+/* Builds the int8 state from an f16 K cache holding kv_len (rotated) rows, e.g. after the prompt's prefill: k_mean over
+ * rows [0, kv_len), k_q / k_scale for those rows, and the rows of the open block into k_tail. cache->v is the f16 V cache
+ * itself (not touched here). */
+fa_status fa_sage_cache_build(fa_ctx *ctx, const void *k_f16, uint32_t kv_len, const fa_sage_cache *cache);
+
+/* One decode step of one layer with int8 Q/K, the cache-write side of the sketch included (docs/SAGE.md:51-65: "quantise
+ * on the way into the cache"): the new token's k is rotated (KvPrepFused arithmetic: rope_mode, the no-RoPE layer rule,
+ * one rounding to f16) and appended at row P, v is appended raw, q is rotated, rounded to f16 and quantised per head;
+ * then rows [0, P] are attended as in fa_sage_decode. P = *d_position if d_position != NULL (kv_len_bound >= P + 1 as in
+ * fa_flash_decode_dyn), else params->position_offset. Two launches.
+ * The open block: a block scale covers 32 rows, so a row appended to a partly filled block can change the scale of the
+ * rows before it. The block's exact f16 rows are therefore kept in k_tail and the whole block is quantised anew at
+ * every append: k_q and k_scale always hold what quantising rows [0, P] from scratch gives. The smoothing mean stays
+ * the one the state was built with: subtracting ANY vector constant over the keys leaves softmax(q . k) unchanged
+ * (it shifts every score of a head by the same amount), so a fixed mean costs no accuracy in exact arithmetic and
+ * only moves the quantisation grid.
+ * q [1, n_heads*head_dim], k, v [1, n_kv_heads*head_dim] f16; cos/sin [>= P + 1, head_dim/2] f16; output
+ * [n_heads*head_dim] f16. params: n_heads, n_kv_heads, head_dim, rope_mode, layer_idx, no_rope_layer_step, seq_len = 1,
+ * max_seq_len = cache->capacity. A position at or beyond the capacity / the bound is dropped and reported by the next
+ * fa_synchronize like fa_decode_step_fused's. */
+fa_status fa_sage_decode_step(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                              const fa_sage_cache *cache, const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                              const fa_tensor_arg *output, const fa_kv_prep_fused_params *params,
+                              const uint32_t *d_position, uint32_t kv_len_bound);
+
 /* Library / device facts for harnesses. */
 const char *fa_version(void);
 fa_status fa_device_info(fa_ctx *ctx, char *name_out, size_t name_cap, uint32_t *compute_units,

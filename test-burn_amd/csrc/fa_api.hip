@@ -1412,3 +1412,87 @@ extern "C" fa_status fa_sage_decode(fa_ctx *ctx, const void *q_q, const float *q
     L.q_scale = q_scale, L.k_scale = (const __half *)k_scale, L.ks_stride = ceil_div_u32(capacity, FA_SAGE_BLOCK);
     return fa_launch_decode(ctx, L);
 }
+
+static fa_status check_sage_cache(const fa_sage_cache *c) {
+    FA_NEED(c, "cache");
+    if (!c->k_q || !c->k_scale || !c->k_tail || !c->v || !c->q_q || !c->k_mean || !c->q_scale)
+        return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: a buffer of the int8 cache state is null");
+    FA_TRY(sage_dims(c->head_dim));
+    if (c->n_kv_heads == 0 || c->n_heads == 0 || c->n_heads % c->n_kv_heads != 0 || c->capacity == 0)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: int8 cache state with %u heads, %u kv heads, capacity %u", c->n_heads,
+                       c->n_kv_heads, c->capacity);
+    if ((((uintptr_t)c->q_q) | ((uintptr_t)c->k_q)) % 8 != 0 || ((uintptr_t)c->v) % 16 != 0)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Sage decode needs 8-byte aligned int8 tensors and 16-byte aligned v");
+    return FA_OK;
+}
+
+extern "C" fa_status fa_sage_cache_build(fa_ctx *ctx, const void *k_f16, uint32_t kv_len, const fa_sage_cache *c) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(k_f16, "k_f16");
+    FA_TRY(check_sage_cache(c));
+    if (kv_len > c->capacity) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_len %u > capacity %u", kv_len, c->capacity);
+    FA_TRY(fa_launch_sage_k_mean(ctx, k_f16, c->n_kv_heads, c->capacity, c->head_dim, kv_len, c->k_mean));
+    FA_TRY(fa_launch_sage_quantize_k(ctx, k_f16, c->k_mean, c->n_kv_heads, c->capacity, c->head_dim, 0, kv_len, c->k_q, c->k_scale));
+    return fa_launch_sage_tail_copy(ctx, k_f16, c->n_kv_heads, c->capacity, c->head_dim, kv_len, c->k_tail);
+}
+
+extern "C" fa_status fa_sage_decode_step(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                                         const fa_sage_cache *c, const fa_tensor_arg *cos, const fa_tensor_arg *sin,
+                                         const fa_tensor_arg *output, const fa_kv_prep_fused_params *p,
+                                         const uint32_t *d_position, uint32_t kv_len_bound) {
+    FA_NEED(ctx, "ctx");
+    FA_TRY(check_sage_cache(c));
+    FA_TRY(check_kv_prep_params(p));
+    if (p->seq_len != 1) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: the int8 decode step takes 1 token, seq_len is %u", p->seq_len);
+    if (p->head_dim != c->head_dim || p->n_heads != c->n_heads || p->n_kv_heads != c->n_kv_heads)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: params (H %u, Hkv %u, D %u) do not match the int8 cache state (H %u, Hkv %u, D %u)",
+                       p->n_heads, p->n_kv_heads, p->head_dim, c->n_heads, c->n_kv_heads, c->head_dim);
+    if (p->max_seq_len != c->capacity)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: max_seq_len %u != cache capacity %u", p->max_seq_len, c->capacity);
+    FA_TRY(check_tensor(q, "q", FA_DTYPE_F16, p->d_model, 2));
+    FA_TRY(check_tensor(k, "k", FA_DTYPE_F16, p->kv_dim, 2));
+    FA_TRY(check_tensor(v, "v", FA_DTYPE_F16, p->kv_dim, 2));
+    FA_TRY(check_tensor(cos, "cos", FA_DTYPE_F16, 0, 2));
+    FA_TRY(check_tensor(sin, "sin", FA_DTYPE_F16, 0, 2));
+    FA_TRY(check_tensor(output, "output", FA_DTYPE_F16, p->d_model, 2));
+    const uint32_t half = p->head_dim / 2;
+    size_t rows = numel(cos) / half;
+    if (numel(sin) / half < rows) rows = numel(sin) / half;
+    if (cos->rank == 0 || sin->rank == 0) rows = 0xffffffffu;
+    if (rows == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: empty RoPE tables");
+    SageAppendLaunch A;
+    memset(&A, 0, sizeof(A));
+    A.q = tptr<const __half>(q), A.k = tptr<const __half>(k), A.v = tptr<const __half>(v);
+    A.cos_t = tptr<const __half>(cos), A.sin_t = tptr<const __half>(sin);
+    A.mean = c->k_mean, A.tail = (__half *)c->k_tail, A.k_scale = (__half *)c->k_scale, A.v_cache = (__half *)c->v;
+    A.k_q = (int8_t *)c->k_q, A.q_q = (int8_t *)c->q_q, A.q_scale = c->q_scale;
+    A.capacity = c->capacity, A.head_dim = c->head_dim, A.n_heads = c->n_heads, A.n_kv_heads = c->n_kv_heads;
+    A.rope_normal = p->rope_mode == FA_ROPE_MODE_NORMAL;
+    A.apply_rope = p->no_rope_layer_step == 0 || ((p->layer_idx + 1u) % p->no_rope_layer_step) != 0u;
+    A.table_rows = (uint32_t)(rows > 0xffffffffu ? 0xffffffffu : rows);
+    DecodeLaunch L;
+    memset(&L, 0, sizeof(L));
+    if (d_position) {
+        if (kv_len_bound == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: kv_len_bound is 0");
+        A.d_position = d_position, A.bound = kv_len_bound < c->capacity ? kv_len_bound : c->capacity;
+        L.d_len = d_position, L.d_len_stride = 0, L.kv_len_add = 1, L.kv_len_bound = A.bound;
+    } else {
+        if ((uint64_t)p->position_offset + 1 > c->capacity)
+            return fa_fail(FA_ERR_INVALID_OPERATION, "Invalid operation: position_offset %u + seq_len 1 exceeds max_seq_len %u",
+                           p->position_offset, c->capacity);
+        if ((uint64_t)p->position_offset + 1 > A.table_rows)
+            return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: RoPE tables hold %u rows, %u needed", A.table_rows, p->position_offset + 1);
+        A.position = p->position_offset, A.bound = p->position_offset + 1;
+        L.kv_len = p->position_offset + 1, L.kv_len_bound = L.kv_len;
+    }
+    FA_TRY(fa_launch_sage_append(ctx, A));
+    const size_t dm = (size_t)c->n_heads * c->head_dim;
+    L.q = c->q_q, L.k = c->k_q, L.v = (const __half *)c->v, L.out = tptr<__half>(output);
+    L.q_stride_b = dm, L.q_stride_h = c->head_dim, L.out_stride_b = dm, L.out_stride_h = c->head_dim;
+    L.k_stride_h = (uint64_t)c->capacity * c->head_dim, L.v_stride_h = (uint64_t)c->capacity * c->head_dim;
+    L.n_heads = c->n_heads, L.n_kv_heads = c->n_kv_heads, L.head_dim = c->head_dim, L.batch = 1;
+    L.capacity = c->capacity;
+    L.scale = 1.0f / sqrtf((float)c->head_dim);
+    L.q_scale = c->q_scale, L.k_scale = (const __half *)c->k_scale, L.ks_stride = ceil_div_u32(c->capacity, FA_SAGE_BLOCK);
+    return fa_launch_decode(ctx, L);
+}

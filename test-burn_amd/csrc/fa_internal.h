@@ -251,6 +251,20 @@ fa_status fa_launch_sage_quantize_k(fa_ctx *ctx, const void *k, const float *mea
 fa_status fa_launch_sage_quantize_q(fa_ctx *ctx, const void *q, uint32_t n_heads, uint32_t head_dim, void *q_q,
                                     float *q_scale);
 
+// The int8 decode step's append: RoPE + append of the new token into the quantised cache, query quantisation.
+struct SageAppendLaunch {
+    const __half *q, *k, *v, *cos_t, *sin_t;
+    const float *mean;
+    __half *tail, *k_scale, *v_cache;
+    int8_t *k_q, *q_q;
+    float *q_scale;
+    const uint32_t *d_position;
+    uint32_t position, bound, capacity, head_dim, n_heads, n_kv_heads, rope_normal, apply_rope, table_rows;
+};
+fa_status fa_launch_sage_append(fa_ctx *ctx, const SageAppendLaunch &l);
+fa_status fa_launch_sage_tail_copy(fa_ctx *ctx, const void *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim,
+                                   uint32_t kv_len, void *tail);
+
 // Bits of the context's device-written status word
 constexpr uint32_t FA_DEVSTAT_MERGE_TIMEOUT = 1u;  // a merging workgroup gave up waiting for a partition's partial
 constexpr uint32_t FA_DEVSTAT_APPEND_DROPPED = 2u;

@@ -66,6 +66,12 @@ class MatMulParams(C.Structure):
                 ("activation", C.c_uint32)]
 
 
+class SageCache(C.Structure):
+    _fields_ = [("k_q", C.c_void_p), ("k_scale", C.c_void_p), ("k_tail", C.c_void_p), ("v", C.c_void_p), ("q_q", C.c_void_p),
+                ("k_mean", C.c_void_p), ("q_scale", C.c_void_p), ("n_heads", C.c_uint32), ("n_kv_heads", C.c_uint32),
+                ("capacity", C.c_uint32), ("head_dim", C.c_uint32)]
+
+
 class DecodeVariant(C.Structure):
     _fields_ = [("keys_per_split", C.c_uint32), ("merge", C.c_uint32)]
 
@@ -137,6 +143,8 @@ PROTOTYPES = {
     "fa_sage_quantize_k": [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _vp, _vp],
     "fa_sage_quantize_q": [_vp, _vp, _u32, _u32, _vp, _vp],
     "fa_sage_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
+    "fa_sage_cache_build": [_vp, _vp, _u32, C.POINTER(SageCache)],
+    "fa_sage_decode_step": [_vp, _PT, _PT, _PT, C.POINTER(SageCache), _PT, _PT, _PT, C.POINTER(KvPrepFusedParams), _vp, _u32],
     "fa_device_info": [_vp, C.c_char_p, _sz, C.POINTER(_u32), C.POINTER(C.c_uint64)],
 }
 _RESTYPES = {"fa_status_name": C.c_char_p, "fa_last_error_string": C.c_char_p, "fa_version": C.c_char_p,
@@ -437,9 +445,29 @@ class Foundry:
     def sage_quantize_q(self, q, n_heads, head_dim, q_q, q_scale):
         check(self.lib.fa_sage_quantize_q(self.h, q.ptr, n_heads, head_dim, q_q.ptr, q_scale.ptr))
 
+    def sage_cache_build(self, k_f16, kv_len, cache):
+        check(self.lib.fa_sage_cache_build(self.h, k_f16.ptr, kv_len, C.byref(cache)))
+
+    def sage_decode_step(self, q, k, v, cache, cos, sin, out, params, d_position=None, kv_len_bound=0):
+        check(self.lib.fa_sage_decode_step(self.h, C.byref(q), C.byref(k), C.byref(v), C.byref(cache), C.byref(cos),
+                                           C.byref(sin), C.byref(out), C.byref(params),
+                                           None if d_position is None else d_position.ptr, kv_len_bound))
+
     def sage_decode(self, q_q, q_scale, k_q, k_scale, v, out, n_heads, n_kv_heads, head_dim, capacity, kv_len):
         check(self.lib.fa_sage_decode(self.h, q_q.ptr, q_scale.ptr, k_q.ptr, k_scale.ptr, v.ptr, out.ptr, n_heads,
                                       n_kv_heads, head_dim, capacity, kv_len))
+
+
+def sage_cache(ctx, n_heads, n_kv_heads, capacity, head_dim, v_buf):
+    """Allocates the int8 state of one layer around an existing f16 V cache buffer; returns (descriptor, buffers)."""
+    bufs = dict(k_q=ctx.zeros((n_kv_heads, capacity, head_dim), np.int8),
+                k_scale=ctx.zeros((n_kv_heads, (capacity + 31) // 32), np.float16),
+                k_tail=ctx.zeros((n_kv_heads, 32, head_dim), np.float16),
+                q_q=ctx.zeros((n_heads, head_dim), np.int8), k_mean=ctx.zeros((n_kv_heads, head_dim), np.float32),
+                q_scale=ctx.zeros((n_heads,), np.float32), v=v_buf)
+    d = SageCache(bufs["k_q"].ptr, bufs["k_scale"].ptr, bufs["k_tail"].ptr, v_buf.ptr, bufs["q_q"].ptr, bufs["k_mean"].ptr,
+                  bufs["q_scale"].ptr, n_heads, n_kv_heads, capacity, head_dim)
+    return d, bufs
 
 
 def rope_tables(rope_base, head_dim, n_pos, freq_factors=None, pos_begin=0):

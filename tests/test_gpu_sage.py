@@ -85,3 +85,97 @@ def test_sage_incremental_block_quantisation_and_errors():
         f.sage_k_mean(dk, Hkv, cap, 96, N, dmean)
     assert e.value.variant == "OperationNotSupported"
     f.synchronize()
+
+
+@pytest.mark.parametrize("H,Hkv,D,start,cap,steps,mode,layer,nope_step,dyn", [
+    (16, 4, 128, 90, 256, 40, fa.ROPE_NEOX, 0, 0, False),    # crosses the block boundaries at 96 and 128
+    (14, 2, 64, 64, 160, 34, fa.ROPE_NORMAL, 0, 0, True),    # starts on an empty open block, device-side position
+    (16, 4, 128, 37, 128, 6, fa.ROPE_NEOX, 3, 4, False),     # layer 3 of a model with every 4th layer un-rotated
+    (16, 4, 128, 32760, 32800, 12, fa.ROPE_NEOX, 0, 0, True)])  # SmolLM3 shape around the full 32K context
+def test_sage_decode_step_over_consecutive_tokens(H, Hkv, D, start, cap, steps, mode, layer, nope_step, dyn):
+    """fa_sage_decode_step: RoPE + append into the int8 cache (open block quantised anew from its exact rows, fixed
+    mean) + int8 decode, over consecutive positions. After every step the int8 rows and scales must be bit for bit what
+    the oracle's quantiser gives for the oracle's rotated f16 cache with the same mean, the V rows and the quantised
+    query bit-exact, and the output within tolerance of the oracle's int8 model; the error against f16 SDPA on the
+    unquantised cache is measured."""
+    announce("sage decode step", H, Hkv, D, start, cap, steps, mode, layer, nope_step, dyn)
+    f = ctx()
+    rng = np.random.default_rng(start + cap + D)
+    cos, sin = fa.rope_tables(1e6, D, cap)
+    kc, vc = np.zeros((Hkv, cap, D), np.float16), np.zeros((Hkv, cap, D), np.float16)
+    kc[:, :start] = outlier_normal(rng, (Hkv, start, D))
+    vc[:, :start] = outlier_normal(rng, (Hkv, start, D))
+    dk, dv = f.array(kc), f.array(vc)
+    desc, bufs = fa.sage_cache(f, H, Hkv, cap, D, dv)
+    f.sage_cache_build(dk, start, desc)
+    f.synchronize()
+    mean = bufs["k_mean"].download()
+    assert max_abs(mean, orc.sage_k_mean(kc, Hkv, cap, D, start)) <= 2e-5
+    dcos, dsin, dout = f.array(cos), f.array(sin), f.zeros((H * D,))
+    dpos = f.array(np.array([start], np.uint32)) if dyn else None
+    rope_mode = 0 if mode == fa.ROPE_NEOX else 1
+    worst_model, worst_full = 0.0, 0.0
+    for t in range(steps):
+        P = start + t
+        q, k, v = (outlier_normal(rng, (1, n * D)) for n in (H, Hkv, Hkv))
+        dq, dkn, dvn = f.array(q), f.array(k), f.array(v)
+        p = fa.KvPrepFusedParams.make(H, Hkv, D, 1, 0 if dyn else P, cap, mode, layer_idx=layer, no_rope_layer_step=nope_step)
+        f.sage_decode_step(dq.arg(), dkn.arg(), dvn.arg(), desc, dcos.arg(), dsin.arg(), dout.arg(), p, d_position=dpos,
+                           kv_len_bound=cap if dyn else 0)
+        if dyn:
+            f.u32_add(dpos, 1, 1)
+        f.synchronize()
+        # the oracle's f16 path appends the rotated row to its f16 cache; the int8 state is its quantisation
+        qr = orc.kv_prep_fused(q, k, v, kc, vc, cos, sin,
+                               orc.make_params(H, Hkv, D, 1, P, cap, rope_mode=rope_mode, layer_idx=layer, no_rope_layer_step=nope_step))
+        N = P + 1
+        check_state = t < 3 or t == steps - 1 or N % 32 in (0, 1)
+        if check_state:
+            want_kq, want_ks = orc.sage_quantize_k(kc, mean, Hkv, cap, D, N)
+            nb = (N + 31) // 32
+            assert np.array_equal(bits(bufs["k_scale"].download()[:, :nb]), bits(want_ks[:, :nb])), (t, "scales")
+            assert np.array_equal(bufs["k_q"].download()[:, :N], want_kq[:, :N]), (t, "int8 rows")
+            assert np.array_equal(bits(dv.download()[:, :N]), bits(vc[:, :N])), (t, "v rows")
+            want_qq, want_qs = orc.sage_quantize_q(np.ascontiguousarray(qr[:, 0]), H, D)
+            assert np.array_equal(bufs["q_q"].download(), want_qq) and np.array_equal(bufs["q_scale"].download(), want_qs)
+            got = dout.download().reshape(H, D)
+            model = orc.sage_decode(want_qq, want_qs, want_kq, want_ks, vc, H, Hkv, D, cap, N, n_threads=8).reshape(H, D)
+            # the bound scales with the outputs: at a few dozen keys with 8-sigma values they reach 2 .. 4, where one f16
+            # unit in the last place is already 2e-3 .. 4e-3
+            worst_model = max(worst_model, max_abs(got, model) / max(1.0, float(np.max(np.abs(model)))))
+            full = rm.gqa_decode_f64(np.ascontiguousarray(qr[:, 0]), kc, vc, H, Hkv, D, N)
+            worst_full = max(worst_full, max_abs(got, full))
+        for b in (dq, dkn, dvn):
+            b.free()
+    print("sage decode step: max abs err vs int8 model (relative to max(1, |out|)) %.2e, vs f16 sdpa %.4f" % (worst_model, worst_full), flush=True)
+    assert worst_model <= 2e-3
+    assert worst_full <= 0.2
+    # untouched rows past the last position stay zero
+    assert not bufs["k_q"].download()[:, start + steps:].any()
+    for b in list(bufs.values()) + [dk, dcos, dsin, dout] + ([dpos] if dyn else []):
+        b.free()
+
+
+def test_sage_decode_step_errors():
+    announce("sage decode step errors")
+    f = ctx()
+    H, Hkv, D, cap = 8, 2, 128, 64
+    dv = f.zeros((Hkv, cap, D))
+    desc, bufs = fa.sage_cache(f, H, Hkv, cap, D, dv)
+    q, k, v, out = f.zeros((1, H * D)), f.zeros((1, Hkv * D)), f.zeros((1, Hkv * D)), f.zeros((H * D,))
+    cos, sin = f.zeros((cap, D // 2)), f.zeros((cap, D // 2))
+    with pytest.raises(fa.FoundryError) as e:  # position at the capacity
+        f.sage_decode_step(q.arg(), k.arg(), v.arg(), desc, cos.arg(), sin.arg(), out.arg(), fa.KvPrepFusedParams.make(H, Hkv, D, 1, cap, cap))
+    assert e.value.variant == "InvalidOperation"
+    with pytest.raises(fa.FoundryError) as e:  # params of another shape
+        f.sage_decode_step(q.arg(), k.arg(), v.arg(), desc, cos.arg(), sin.arg(), out.arg(), fa.KvPrepFusedParams.make(H, Hkv, 64, 1, 0, cap))
+    assert e.value.variant == "InvalidShape"
+    dpos = f.array(np.array([cap + 3], np.uint32))  # a device position past the cache: dropped and reported
+    f.sage_decode_step(q.arg(), k.arg(), v.arg(), desc, cos.arg(), sin.arg(), out.arg(), fa.KvPrepFusedParams.make(H, Hkv, D, 1, 0, cap),
+                       d_position=dpos, kv_len_bound=cap)
+    with pytest.raises(fa.FoundryError) as e:
+        f.synchronize()
+    assert e.value.variant == "InvalidOperation"
+    f.synchronize()
+    for b in list(bufs.values()) + [q, k, v, out, cos, sin, dpos]:
+        b.free()
