@@ -538,6 +538,61 @@ fa_status fa_sage_decode_step(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tens
                               const fa_tensor_arg *output, const fa_kv_prep_fused_params *params,
                               const uint32_t *d_position, uint32_t kv_len_bound);
 
+/* ---------------------------------------------------------------------------------------------
+ * The un-fused chain around the cache (DSL ops Rope, KvCacheWrite, KvCacheWriteRepeatKvHeads, KvCacheRead, KvRearrange,
+ * RepeatKvHeads). The shipped model specs run KvPrepFused instead; these are thin per-element launches so that a spec
+ * which still names the old ops binds, with the reference kernels' index maps. Parameter structs = the reference's
+ * *ParamsResolved, field for field. All tensors f16; total_elements must equal the product it stands for
+ * (FA_ERR_INVALID_SHAPE); writes past max_seq_len -> FA_ERR_INVALID_OPERATION.
+ * ------------------------------------------------------------------------------------------- */
+/* RopeParams (src/metals/rope/mod.rs:13-22); kernel src/metals/rope/rope.metal:28-75: NeoX pairing (i, i + dim/2),
+ * position of row r = r % seq_len + position_offset, products rounded separately, one rounding to f16. */
+typedef struct fa_rope_params { uint32_t dim, seq_len, position_offset, total_elements; } fa_rope_params;
+fa_status fa_rope(fa_ctx *ctx, const fa_tensor_arg *input, const fa_tensor_arg *output, const fa_tensor_arg *cos,
+                  const fa_tensor_arg *sin, const fa_rope_params *params);
+/* KvCacheWriteParams (src/metals/kv_cache_write/mod.rs:63-78); kv_cache_write.metal:6-30: input [n_kv_heads,
+ * input_seq_len, head_dim] -> cache [n_kv_heads, max_seq_len, head_dim] at rows position_offset... layer_idx is unused. */
+typedef struct fa_kv_cache_write_params {
+    uint32_t n_kv_heads, head_dim, input_seq_len, position_offset, max_seq_len, total_elements, layer_idx;
+} fa_kv_cache_write_params;
+fa_status fa_kv_cache_write(fa_ctx *ctx, const fa_tensor_arg *input, const fa_tensor_arg *cache,
+                            const fa_kv_cache_write_params *params);
+/* KvCacheWriteRepeatKvHeadsParams (src/metals/kv_cache_write/mod.rs:16-35); kv_cache_write_repeat.metal:9-40: the same
+ * write into an expanded cache [n_heads, max_seq_len, head_dim], KV head h repeated into heads h*group_size .. +group_size-1. */
+typedef struct fa_kv_cache_write_repeat_params {
+    uint32_t n_kv_heads, n_heads, group_size, head_dim, input_seq_len, position_offset, max_seq_len, total_elements, layer_idx;
+} fa_kv_cache_write_repeat_params;
+fa_status fa_kv_cache_write_repeat_kv_heads(fa_ctx *ctx, const fa_tensor_arg *input, const fa_tensor_arg *cache,
+                                            const fa_kv_cache_write_repeat_params *params);
+/* KvCacheReadParams (src/metals/kv_cache_write/read.rs:15-26); kv_cache_read.metal:7-29: rows [0, seq_len) of every head
+ * of cache [n_kv_heads, max_seq_len, head_dim] -> output [n_kv_heads, seq_len, head_dim]. */
+typedef struct fa_kv_cache_read_params { uint32_t n_kv_heads, head_dim, seq_len, max_seq_len, total_elements; } fa_kv_cache_read_params;
+fa_status fa_kv_cache_read(fa_ctx *ctx, const fa_tensor_arg *cache, const fa_tensor_arg *output,
+                           const fa_kv_cache_read_params *params);
+/* KvRearrangeParams (src/metals/kv_rearrange/mod.rs:13-39); kv_rearrange.metal:10-47: input [batch*seq, row_stride]
+ * (kv_dim used) -> output [batch*n_heads, seq, head_dim], head h reading KV head h / (n_heads / n_kv_heads). */
+typedef struct fa_kv_rearrange_params {
+    uint32_t kv_dim, row_stride, kv_head_dim, n_heads, n_kv_heads, head_dim, seq, total_elements;
+} fa_kv_rearrange_params;
+fa_status fa_kv_rearrange(fa_ctx *ctx, const fa_tensor_arg *input, const fa_tensor_arg *output,
+                          const fa_kv_rearrange_params *params);
+/* RepeatKvHeadsParams (src/metals/repeat_kv_heads/mod.rs:16-40); repeat_kv_heads.metal:11-44: input [batch*n_kv_heads,
+ * cache_stride, head_dim] -> output [batch*n_heads, seq, head_dim]. */
+typedef struct fa_repeat_kv_heads_params {
+    uint32_t group_size, batch, n_kv_heads, n_heads, seq, head_dim, cache_stride, total_elements;
+} fa_repeat_kv_heads_params;
+fa_status fa_repeat_kv_heads(fa_ctx *ctx, const fa_tensor_arg *input, const fa_tensor_arg *output,
+                             const fa_repeat_kv_heads_params *params);
+
+/* The DSL op SdpaReference (src/metals/sdpa/step.rs:94-156; the materialized path :558-779 with
+ * softmax/softmax_sdpa_batched.metal:14-115). Same fields as FlashAttentionStep. There is no materialized path here: the
+ * op runs on the flash kernels with the same mask (key j visible to row r iff !causal or j <= query_offset + r). Numeric
+ * differences from the reference's fallback, all towards the exact result: scores and weights stay f32 (the fallback
+ * rounds both to f16), and K/V of a GQA model are read through the head map (the fallback lacks it). */
+fa_status fa_sdpa_reference(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
+                            const fa_tensor_arg *output, int causal, uint32_t query_offset, uint32_t n_heads,
+                            uint32_t head_dim, uint32_t kv_seq_len, uint32_t m, int kv_head_major);
+
 /* Library / device facts for harnesses. */
 const char *fa_version(void);
 fa_status fa_device_info(fa_ctx *ctx, char *name_out, size_t name_cap, uint32_t *compute_units,

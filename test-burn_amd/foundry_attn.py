@@ -145,6 +145,13 @@ PROTOTYPES = {
     "fa_sage_decode": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32],
     "fa_sage_cache_build": [_vp, _vp, _u32, C.POINTER(SageCache)],
     "fa_sage_decode_step": [_vp, _PT, _PT, _PT, C.POINTER(SageCache), _PT, _PT, _PT, C.POINTER(KvPrepFusedParams), _vp, _u32],
+    "fa_rope": [_vp, _PT, _PT, _PT, _PT, _vp],
+    "fa_kv_cache_write": [_vp, _PT, _PT, _vp],
+    "fa_kv_cache_write_repeat_kv_heads": [_vp, _PT, _PT, _vp],
+    "fa_kv_cache_read": [_vp, _PT, _PT, _vp],
+    "fa_kv_rearrange": [_vp, _PT, _PT, _vp],
+    "fa_repeat_kv_heads": [_vp, _PT, _PT, _vp],
+    "fa_sdpa_reference": [_vp, _PT, _PT, _PT, _PT, _i, _u32, _u32, _u32, _u32, _u32, _i],
     "fa_device_info": [_vp, C.c_char_p, _sz, C.POINTER(_u32), C.POINTER(C.c_uint64)],
 }
 _RESTYPES = {"fa_status_name": C.c_char_p, "fa_last_error_string": C.c_char_p, "fa_version": C.c_char_p,
@@ -444,6 +451,15 @@ class Foundry:
 
     def sage_quantize_q(self, q, n_heads, head_dim, q_q, q_scale):
         check(self.lib.fa_sage_quantize_q(self.h, q.ptr, n_heads, head_dim, q_q.ptr, q_scale.ptr))
+
+    def legacy_op(self, name, tensors, params):
+        """One of the un-fused ops (fa_rope, fa_kv_cache_write, ...): `params` is the tuple of u32 fields of its struct."""
+        arr = (C.c_uint32 * len(params))(*params)
+        check(getattr(self.lib, name)(self.h, *[C.byref(t) for t in tensors], C.cast(arr, C.c_void_p)))
+
+    def sdpa_reference(self, q, k, v, out, causal, query_offset, n_heads, head_dim, kv_seq_len, m, kv_head_major=True):
+        check(self.lib.fa_sdpa_reference(self.h, C.byref(q), C.byref(k), C.byref(v), C.byref(out), int(causal), query_offset,
+                                         n_heads, head_dim, kv_seq_len, m, int(kv_head_major)))
 
     def sage_cache_build(self, k_f16, kv_len, cache):
         check(self.lib.fa_sage_cache_build(self.h, k_f16.ptr, kv_len, C.byref(cache)))
