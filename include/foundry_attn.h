@@ -119,6 +119,12 @@ fa_status fa_profile_enable(fa_ctx *ctx, int on);
 fa_status fa_profile_reset(fa_ctx *ctx);
 fa_status fa_profile_query(fa_ctx *ctx, const char *kernel_prefix, uint64_t *launches, double *total_ms);
 
+/* Clock readings from inside the prefill kernel (its LDS-direct variant): while a buffer of n_workgroups x 2 u64 is set,
+ * every prefill launch of at most n_workgroups workgroups leaves per workgroup {shader-clock ticks, 100 MHz wall-clock
+ * ticks} between its first instruction and the end of its key loop; ticks / wall x 100 = the MHz the kernel really ran
+ * at (the matrix peak scales with it). NULL switches it off. */
+fa_status fa_profile_clock_buffer(fa_ctx *ctx, void *d_buffer, uint32_t n_workgroups);
+
 /* Device memory, the executor's buffer management (src/model/executor.rs:2286-2328, src/lib.rs:317-377).
  * fa_upload/fa_download are synchronous with respect to the context's stream. */
 fa_status fa_device_alloc(fa_ctx *ctx, size_t bytes, void **out);
@@ -592,6 +598,13 @@ fa_status fa_repeat_kv_heads(fa_ctx *ctx, const fa_tensor_arg *input, const fa_t
 fa_status fa_sdpa_reference(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
                             const fa_tensor_arg *output, int causal, uint32_t query_offset, uint32_t n_heads,
                             uint32_t head_dim, uint32_t kv_seq_len, uint32_t m, int kv_head_major);
+
+/* Measures the shader clock the device sustains under a given load, for reading utilisation figures against: every
+ * compute unit runs 8 waves of back-to-back v_mfma_f32_32x32x16_f16 (matrix_load != 0) or of dependent FMAs
+ * (matrix_load == 0) for `iterations` rounds, and each wave's shader-clock ticks are divided by its 100 MHz wall-clock
+ * ticks. *busy_ms (nullable) is how long the waves ran: run long enough (tens of milliseconds) for the power
+ * management to settle. A harness facility without a counterpart in the reference; synchronises the stream. */
+fa_status fa_measure_clock(fa_ctx *ctx, int matrix_load, uint32_t iterations, float *shader_mhz, float *busy_ms);
 
 /* Library / device facts for harnesses. */
 const char *fa_version(void);

@@ -387,6 +387,14 @@ extern "C" fa_status fa_profile_query(fa_ctx *ctx, const char *prefix, uint64_t 
     return FA_OK;
 }
 
+extern "C" fa_status fa_profile_clock_buffer(fa_ctx *ctx, void *d_buffer, uint32_t n_workgroups) {
+    FA_NEED(ctx, "ctx");
+    if (d_buffer && ((uintptr_t)d_buffer % 8) != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "the clock buffer must be 8-byte aligned");
+    ctx->clock_buf = (unsigned long long *)d_buffer;
+    ctx->clock_buf_workgroups = d_buffer ? n_workgroups : 0;
+    return FA_OK;
+}
+
 // memory ----------------------------------------------------------------------------------------
 
 extern "C" fa_status fa_device_alloc(fa_ctx *ctx, size_t bytes, void **out) {

@@ -64,6 +64,9 @@ struct fa_ctx {
     uint32_t gemm_min_m = 0;       // FusedQkv / MatMul: input rows from which the GEMM runs (0 = default)
     uint32_t prefill_split_k = 0;  // 0 = auto
     uint32_t prefill_variant = 0;  // 0 = auto, 1 = tiles staged through registers, 2 = tiles straight into LDS, two-phase loop
+    // optional: the prefill kernel leaves {shader-clock ticks, wall ticks} per workgroup here (fa_profile_clock_buffer)
+    unsigned long long *clock_buf = nullptr;
+    uint32_t clock_buf_workgroups = 0;
     // per-kernel profiling
     bool profiling = false;
     std::vector<FaProfileRec> prof;

@@ -50,6 +50,8 @@ struct PrefillDev {
     uint32_t splits;             // > 1: the key tiles of a query tile are divided over `splits` workgroups
     float *part_acc, *part_ml;   // [head][query tile][split][BM][D] unnormalised sums, [..][BM][2] (max, sum)
     float scale_log2e;
+    uint32_t out_aligned16;         // output base and strides are multiples of 16 bytes: rows leave as whole 16-byte pieces
+    unsigned long long *clock_out;  // nullable: per workgroup {shader-clock ticks, 100 MHz wall ticks} from start to end
 };
 
 constexpr int BM = 128;  // query rows per workgroup
@@ -511,6 +513,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     typedef __attribute__((address_space(3))) void *lds_ptr;
     __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * GRP_LDS];  // [group]{K[2], V[2]}
 
+    const unsigned long long clk0 = a.clock_out ? __builtin_readcyclecounter() : 0ull, wall0 = a.clock_out ? wall_clock64() : 0ull;
     const int lane = threadIdx.x & 63;
     const int wave8 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int grp = wave8 >> 2, wave = wave8 & 3;
@@ -807,6 +810,10 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         m_run = m;
     }
     const float l_tot = lacc[0];
+    if (a.clock_out && threadIdx.x == 0) {
+        a.clock_out[(size_t)blockIdx.x * 2] = __builtin_readcyclecounter() - clk0;
+        a.clock_out[(size_t)blockIdx.x * 2 + 1] = wall_clock64() - wall0;
+    }
     if (S > 1) {  // unnormalised partial state for the merge kernel (flash_prefill.metal:592-617)
         if (q_row >= a.q_len) return;
         const size_t prow = (((size_t)head * n_qt + q_tile) * S + split) * BM + wave * 32 + n;
@@ -822,6 +829,37 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         return;
     }
     const float inv_l = (isfinite(l_tot) && fabsf(l_tot) > 1e-6f) ? (1.0f / l_tot) : 0.0f;  // flash_prefill.metal:255-261
+    if (a.out_aligned16) {
+        // A lane holds one row's values in 8-byte pieces, 64 rows' pieces per store instruction: written like that, every
+        // instruction touches 64 cache lines and the L2 is left with half-written lines to flush at the kernel's end
+        // (measured: 5 us of a 47 us launch at 2048 tokens, 39 of 454 at 8192). So the wave's 32 rows go through its own
+        // corner of LDS (past what the group merge used; LDS runs a wave's accesses in order, no barrier) and leave as
+        // whole 256-byte rows, 16 bytes per lane.
+        constexpr int ORS = ROWB + 16, RPI = 1024 / ROWB;  // LDS row stride; rows per store instruction
+        unsigned char *ot = lds + 2 * GRP_LDS - 4 * 32 * ORS + wave * (32 * ORS);
+#pragma unroll
+        for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+            for (int gi = 0; gi < 4; ++gi) {  // accumulators 4gi..4gi+3 are d = 32b + 8gi + 4hi + 0..3
+                h4_t o;
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) o[jj] = to_elem<BF16>(oacc[b][gi * 4 + jj] * inv_l);
+                *reinterpret_cast<h4_t *>(ot + n * ORS + (b * 32 + gi * 8 + hi * 4) * 2) = o;
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+        const int rl = lane / (ROWB / 16), ch = lane % (ROWB / 16);
+        __half *ob = a.out + (size_t)head * a.out_stride_h + ch * 8;
+#pragma unroll
+        for (int it = 0; it < 32 / RPI; ++it) {
+            const int row = it * RPI + rl;
+            const uint32_t qr = q0 + wave * 32 + row;
+            const uint4 val = *reinterpret_cast<const uint4 *>(ot + row * ORS + ch * 16);
+            if (qr < a.q_len) __builtin_nontemporal_store(__builtin_bit_cast(u4_t, val), reinterpret_cast<u4_t *>(ob + (size_t)qr * a.out_stride_m));
+        }
+        return;
+    }
     if (q_row < a.q_len) {
         __half *op = a.out + (size_t)head * a.out_stride_h + (size_t)q_row * a.out_stride_m;
 #pragma unroll
@@ -898,6 +936,8 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
     if (!L.paged && (uint64_t)L.kv_len * L.head_dim * 2 >= (1ull << 32))
         return fa_fail(FA_ERR_INVALID_SHAPE, "prefill: one KV head of the contiguous cache must stay below 4 GiB");
     a.scale_log2e = L.scale * 1.4426950408889634f;
+    a.clock_out = nullptr;
+    a.out_aligned16 = ((uintptr_t)L.out % 16 == 0 && L.out_stride_h % 8 == 0 && L.out_stride_m % 8 == 0) ? 1u : 0u;
     if (L.q_len == 0) return FA_OK;
     if (L.head_dim != 128 && L.head_dim != 64)
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill only supports head_dim=64 or 128, got %u", L.head_dim);
@@ -924,6 +964,7 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
         a.part_ml = (float *)((char *)ctx->workspace + acc_bytes);
     }
     dim3 grid(base_wgs * splits, 1, 1);
+    if (ctx->clock_buf && grid.x <= ctx->clock_buf_workgroups) a.clock_out = ctx->clock_buf;
     {
         // the LDS-direct kernel (measured faster at every size) addresses the query rows of a head with 32-bit offsets
         const bool lds_direct = ctx->prefill_variant != 1 && ((uint64_t)(L.q_len - 1) * L.q_stride_m + L.head_dim) * 2 < (1ull << 32);

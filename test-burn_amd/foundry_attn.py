@@ -104,6 +104,7 @@ PROTOTYPES = {
     "fa_profile_enable": [_vp, _i],
     "fa_profile_reset": [_vp],
     "fa_profile_query": [_vp, C.c_char_p, C.POINTER(C.c_uint64), C.POINTER(C.c_double)],
+    "fa_profile_clock_buffer": [_vp, _vp, _u32],
     "fa_device_alloc": [_vp, _sz, C.POINTER(_vp)],
     "fa_device_free": [_vp, _vp],
     "fa_upload": [_vp, _vp, _sz, _vp, _sz],
@@ -152,6 +153,7 @@ PROTOTYPES = {
     "fa_kv_rearrange": [_vp, _PT, _PT, _vp],
     "fa_repeat_kv_heads": [_vp, _PT, _PT, _vp],
     "fa_sdpa_reference": [_vp, _PT, _PT, _PT, _PT, _i, _u32, _u32, _u32, _u32, _u32, _i],
+    "fa_measure_clock": [_vp, _i, _u32, C.POINTER(C.c_float), C.POINTER(C.c_float)],
     "fa_device_info": [_vp, C.c_char_p, _sz, C.POINTER(_u32), C.POINTER(C.c_uint64)],
 }
 _RESTYPES = {"fa_status_name": C.c_char_p, "fa_last_error_string": C.c_char_p, "fa_version": C.c_char_p,
@@ -451,6 +453,15 @@ class Foundry:
 
     def sage_quantize_q(self, q, n_heads, head_dim, q_q, q_scale):
         check(self.lib.fa_sage_quantize_q(self.h, q.ptr, n_heads, head_dim, q_q.ptr, q_scale.ptr))
+
+    def profile_clock_buffer(self, buf, n_workgroups):
+        check(self.lib.fa_profile_clock_buffer(self.h, None if buf is None else buf.ptr, n_workgroups))
+
+    def measure_clock(self, matrix_load, iterations):
+        """(shader MHz, milliseconds the waves ran) under back-to-back MFMAs (matrix_load) or dependent FMAs."""
+        mhz, ms = C.c_float(), C.c_float()
+        check(self.lib.fa_measure_clock(self.h, int(matrix_load), iterations, C.byref(mhz), C.byref(ms)))
+        return mhz.value, ms.value
 
     def legacy_op(self, name, tensors, params):
         """One of the un-fused ops (fa_rope, fa_kv_cache_write, ...): `params` is the tuple of u32 fields of its struct."""
