@@ -18,6 +18,8 @@
 // FLOPs per (query row, visible key, head): 4 * D.
 #include "fa_internal.h"
 
+#include <type_traits>
+
 namespace {
 
 typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
@@ -47,7 +49,8 @@ struct PrefillDev {
     uint64_t q_stride_h, q_stride_m, k_stride_h, v_stride_h, out_stride_h, out_stride_m;
     const int32_t *block_table;
     uint32_t n_heads, group_size, q_len, kv_len, query_offset, causal, block_size, block_shift, n_kv_heads, paged;
-    uint32_t splits;             // > 1: the key tiles of a query tile are divided over `splits` workgroups
+    uint32_t splits;             // > 1: the key tiles of a query tile are divided over `splits` items
+    uint32_t n_qt, n_items, n_workgroups;  // query tiles; (query tile, head, split) items; workgroups that share them out
     float *part_acc, *part_ml;   // [head][query tile][split][BM][D] unnormalised sums, [..][BM][2] (max, sum)
     float scale_log2e;
     uint32_t out_aligned16;         // output base and strides are multiples of 16 bytes: rows leave as whole 16-byte pieces
@@ -510,8 +513,9 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     constexpr int RG_BYTES = 4 * ROWB;   // one 4-row group of a V tile
     constexpr int K_DMA = CHK / 4, V_DMA = 16 * ROWB / 1024;  // instructions per wave per tile
     constexpr int K_AHEAD = 6, V_AHEAD = 6;
+    constexpr int Q_STAGE = BM * ROWB;  // the query rows of the coming item, in the K tile's layout
     typedef __attribute__((address_space(3))) void *lds_ptr;
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * GRP_LDS];  // [group]{K[2], V[2]}
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * GRP_LDS + Q_STAGE];  // [group]{K[2], V[2]}, Q
 
     const unsigned long long clk0 = a.clock_out ? __builtin_readcyclecounter() : 0ull, wall0 = a.clock_out ? wall_clock64() : 0ull;
     const int lane = threadIdx.x & 63;
@@ -519,28 +523,39 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     const int grp = wave8 >> 2, wave = wave8 & 3;
     unsigned char *k_base = lds + grp * GRP_LDS, *v_base = k_base + 2 * K_TILE;
     const uint32_t k_lds_addr = (uint32_t)(uintptr_t)(lds_ptr)lds + grp * GRP_LDS, v_lds_addr = k_lds_addr + 2 * K_TILE;
+    const uint32_t q_lds_addr = (uint32_t)(uintptr_t)(lds_ptr)lds + 2 * GRP_LDS;
     const int n = lane & 31, hi = lane >> 5;
-    const uint32_t S = a.splits;
-    const uint32_t n_qt = gridDim.x / (a.n_heads * S);
-    const uint32_t q_tile = n_qt - 1 - blockIdx.x / (a.n_heads * S);  // heaviest query tiles first
-    const uint32_t head = (blockIdx.x / S) % a.n_heads;
-    const uint32_t split = blockIdx.x % S;
-    const uint32_t kvh = head / a.group_size;
-    const uint32_t q0 = q_tile * BM;
-    const uint32_t q_row = q0 + wave * 32 + n;
-    const uint32_t q_row_c = min(q_row, a.q_len - 1);
-    uint32_t kv_end = a.kv_len;
-    if (a.causal) {
-        const uint64_t last = (uint64_t)min(q0 + BM - 1, a.q_len - 1) + a.query_offset + 1;
-        kv_end = (uint32_t)min((uint64_t)a.kv_len, last);
-    }
-    const int all_tiles = (int)((kv_end + BN - 1) / BN);
-    const int per_split = (all_tiles + (int)S - 1) / (int)S;
-    const int t_lo = min(all_tiles, (int)split * per_split);
-    const int n_tiles = min(all_tiles, t_lo + per_split);
-    const int t0 = t_lo + grp;                                  // group g attends tiles t0, t0 + 2, ...
-    const int ntg = t0 < n_tiles ? (n_tiles - t0 + 1) / 2 : 0;  // how many
-    const int iters = (n_tiles - t_lo + 1) / 2;                 // of group 0: the barriers are workgroup-wide
+    const uint32_t S = a.splits, n_qt = a.n_qt, n_items = a.n_items, n_wgs = a.n_workgroups;
+
+    // ---- the items of this workgroup. An item is one (query tile, head, split), numbered heaviest query tile first;
+    // round r hands items r n_wgs .. (r + 1) n_wgs - 1 to the workgroups in rising order when r is even and in
+    // falling order when it is odd, so the workgroup with the heaviest item of one round gets the lightest of the next.
+    auto item_of = [&](uint32_t r) -> uint32_t { return r * n_wgs + ((r & 1) ? n_wgs - 1 - blockIdx.x : blockIdx.x); };
+    uint32_t q_tile = 0, head = 0, split = 0, kvh = 0, q0 = 0, kv_end = 0;
+    int t0 = 0, ntg = 0, iters = 0;
+    rsrc_words krs = make_rsrc_words(nullptr, 0), vrs = krs;
+    auto enter_item = [&](uint32_t item) {
+        const uint32_t qi = item / (a.n_heads * S), rest = item - qi * (a.n_heads * S);
+        q_tile = n_qt - 1 - qi, head = rest / S, split = rest - head * S;
+        kvh = head / a.group_size;
+        q0 = q_tile * BM;
+        kv_end = a.kv_len;
+        if (a.causal) {
+            const uint64_t last = (uint64_t)min(q0 + BM - 1, a.q_len - 1) + a.query_offset + 1;
+            kv_end = (uint32_t)min((uint64_t)a.kv_len, last);
+        }
+        const int all_tiles = (int)((kv_end + BN - 1) / BN);
+        const int per_split = (all_tiles + (int)S - 1) / (int)S;
+        const int t_lo = min(all_tiles, (int)split * per_split);
+        const int n_tiles = min(all_tiles, t_lo + per_split);
+        t0 = t_lo + grp;                                  // group g attends tiles t0, t0 + 2, ...
+        ntg = t0 < n_tiles ? (n_tiles - t0 + 1) / 2 : 0;  // how many
+        iters = (n_tiles - t_lo + 1) / 2;                 // of group 0: the barriers are workgroup-wide
+        if (!PAGED) {
+            krs = make_rsrc_words(a.k + (size_t)kvh * a.k_stride_h, kv_end * (uint32_t)ROWB);
+            vrs = make_rsrc_words(a.v + (size_t)kvh * a.v_stride_h, kv_end * (uint32_t)ROWB);
+        }
+    };
 
     U4H8 qreg[DSTEPS];
 
@@ -549,11 +564,6 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     constexpr int CBR = ROWB / 64;
     const int k_lane_src = (lane & 15) * ROWB + (lane >> 4) * 16;
     const int v_lane_src = ((lane / (16 * CBR)) * 4 + ((lane & 15) >> 2)) * ROWB + ((lane >> 4) % CBR) * 64 + (lane & 3) * 16;
-    rsrc_words krs = make_rsrc_words(nullptr, 0), vrs = krs;
-    if (!PAGED) {
-        krs = make_rsrc_words(a.k + (size_t)kvh * a.k_stride_h, kv_end * (uint32_t)ROWB);
-        vrs = make_rsrc_words(a.v + (size_t)kvh * a.v_stride_h, kv_end * (uint32_t)ROWB);
-    }
     typedef const int32_t __attribute__((address_space(4))) *const_i32p;
     const const_i32p bt = (const_i32p)a.block_table;
     const uint32_t bs_shift = a.block_shift;
@@ -583,70 +593,40 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
             buffer_to_lds_b128<V_DMA, 1024, 1024>(rs, v_lds_addr + buf * V_TILE + wave * (4 * RG_BYTES), v_lane_src, so);
         }
     };
+    // The query rows take the same road: into LDS in the K tile's layout (wave w of the eight moves rows 16w..16w+15
+    // as one 16-row block; rows past the last query come out of the descriptor's bound check as zeros), then each lane
+    // picks its operand pieces out of them. (Loading the pieces straight from memory, 16 bytes from each of 64 places
+    // per instruction, cost every workgroup 2.6 us.)
+    const size_t q_bytes = ((size_t)(a.q_len - 1) * a.q_stride_m + D) * 2;
+    auto q_dma = [&](uint32_t item) {
+        int ql = lane;
+        asm volatile("" : "+v"(ql));  // the lane's source offset is worked out here, not kept in a register across the loop
+        const int q_lane_src = (ql & 15) * (int)(a.q_stride_m * 2) + (ql >> 4) * 16;
+        const uint32_t qi = item / (a.n_heads * S), hd = (item - qi * (a.n_heads * S)) / S;
+        const uint32_t row0 = (n_qt - 1 - qi) * BM + 16 * wave8;
+        const rsrc_words qrs = make_rsrc_words(a.q + (size_t)hd * a.q_stride_h, (uint32_t)q_bytes);
+        buffer_to_lds_b128<K_DMA, 64, 1024>(qrs, q_lds_addr + wave8 * RB_BYTES, q_lane_src, (int)(row0 * (uint32_t)(a.q_stride_m * 2)));
+    };
 
     f16_t oacc[DBLKS];
-#pragma unroll
-    for (int b = 0; b < DBLKS; ++b)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[b][i] = 0.0f;
     // Row sums ride on the matrix pipe: an all-ones A operand against P^T leaves, in every accumulator of a lane,
     // the sum of that lane's query row over the keys of the step (both lane halves included) - 4 more MFMAs a tile
     // instead of 32 more additions in the VALU phase, which is the longer one. Only element 0 is ever read.
     f16_t lacc;
+    float m_run;
+    auto clear_state = [&]() {
 #pragma unroll
-    for (int i = 0; i < 16; ++i) lacc[i] = 0.0f;
+        for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) oacc[b][i] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) lacc[i] = 0.0f;
+        m_run = -1e30f;
+    };
     h8_t ones;
 #pragma unroll
     for (int i = 0; i < 8; ++i) ones[i] = to_elem<BF16>(1.0f);
-    float m_run = -1e30f;
     const float c = a.scale_log2e;
-    const uint32_t q_abs = q_row_c + a.query_offset;
-    const uint32_t wave_min_limit = a.causal ? (min(q0 + wave * 32, a.q_len - 1) + a.query_offset) : 0xffffffffu;
-
-    // On entry to MFMA phase j the LDS holds K_{j+1} in K[(j+1)&1] and V_j in V[j&1]. VALU phase j starts by
-    // requesting K_{j+2} into K[j&1] and V_{j+1} into V[(j+1)&1] (both buffers were last read in MFMA phase j-1);
-    // the requests are complete (vmcnt) before the barrier that ends MFMA phase j, two phases later, so VALU phase
-    // j+1 may already fetch the first operands of MFMA phase j+1 ahead of its barrier.
-    // The query rows take the same road once: into LDS in the K tile's layout (wave w moves rows 16w..16w+15 as one
-    // 16-row block; rows past the last query come out of the descriptor's bound check as zeros), then each lane
-    // picks its operand pieces out of them. (Loading the pieces straight from memory, 16 bytes from each of 64
-    // places per instruction, cost every workgroup 2.6 us.) The 8 blocks are parked in the two groups' second V
-    // buffers, which no tile needs yet.
-    {
-        const size_t q_bytes = ((size_t)(a.q_len - 1) * a.q_stride_m + D) * 2;
-        const rsrc_words qrs = make_rsrc_words(a.q + (size_t)head * a.q_stride_h, (uint32_t)q_bytes);
-        const int q_lane_src = (lane & 15) * (int)(a.q_stride_m * 2) + (lane >> 4) * 16;
-        const uint32_t dst = (uint32_t)(uintptr_t)(lds_ptr)lds + (wave8 >> 2) * GRP_LDS + 2 * K_TILE + V_TILE + (wave8 & 3) * RB_BYTES;
-        buffer_to_lds_b128<K_DMA, 64, 1024>(qrs, dst, q_lane_src, (int)((q0 + 16 * wave8) * (uint32_t)(a.q_stride_m * 2)));
-    }
-    int32_t pg_k = 0, pg_v = 0, pg_next = 0;  // pages of the K tile / V tile requested next, and of the K tile after
-    if (ntg > 0) {
-        const int32_t p0 = page_of(0), p1 = page_of(1);
-        pg_k = page_of(2), pg_next = page_of(3), pg_v = p1;
-        dma(true, 0, 0, p0);
-        if (ntg > 1) dma(true, 1, 1, p1);
-        dma(false, 0, 0, p0);
-    }
-    // Q, K_0 (for S_0) and K_1 (whose first operands the first VALU phase reads ahead) must be there now; V_0,
-    // requested last (loads complete in order), has until the first MFMA phase. A CU pulls about 25 GB/s on its
-    // own, so every 16 KB not waited for here is worth half a microsecond.
-    constexpr int VMCNT_V = 0x0F70 | V_DMA, VMCNT_KV = 0x0F70 | (V_DMA + K_DMA);
-    if (ntg > 0) __builtin_amdgcn_s_waitcnt(VMCNT_V);
-    else __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    {
-        const int rb = wave * 2 + (n >> 4);  // 16-row block of this lane's row; both groups hold the same 128 rows
-        const unsigned char *qp = lds + (rb >> 2) * GRP_LDS + 2 * K_TILE + V_TILE + (rb & 3) * RB_BYTES + hi * 256 + (n & 15) * 16;
-#pragma unroll
-        for (int s = 0; s < DSTEPS; ++s) qreg[s].u = *reinterpret_cast<const uint4 *>(qp + s * 512);
-#pragma unroll
-        for (int s = 0; s < DSTEPS; ++s) {  // arrived: keep the wait out of the loop
-            u4_t t = __builtin_bit_cast(u4_t, qreg[s].u);
-            asm volatile("" : "+v"(t));
-            qreg[s].u = __builtin_bit_cast(uint4, t);
-        }
-    }
-    __syncthreads();  // before the buffers the rows were parked in receive their first V tiles
 
     const int k_lane = (n >> 4) * RB_BYTES + hi * 256 + (n & 15) * 16;
     const int v_lane = hi * RG_BYTES + ((lane & 15) >> 2) * 64 + ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
@@ -659,7 +639,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         for (int i = 0; i < K_AHEAD; ++i)
             kpre[i].u = *reinterpret_cast<const uint4 *>(k_lds + (i / DSTEPS) * (2 * RB_BYTES) + (i % DSTEPS) * 512);
     };
-    auto s_tile = [&](int buf, bool own_pipeline) {
+    auto s_tile = [&](int buf) {  // S_0 of an item, outside the phases
         const unsigned char *k_lds = k_base + buf * K_TILE + k_lane;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
@@ -674,203 +654,321 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
                                 : __builtin_amdgcn_mfma_f32_32x32x16_f16(kk.h, qreg[s].h, sacc[kb], 0, 0, 0);
             }
         }
-        if (!own_pipeline) return;
 #pragma unroll
         for (int i = 0; i < 2 * DSTEPS; ++i) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
     };
-    // One scheduling region, nothing conditional. (After the group's last tile S_{j+1} is computed from whatever the
-    // buffer holds and never used: cheaper than a second copy of this code, which also made the register allocator
-    // shuffle the 64 accumulator registers between two homes on every iteration.)
+    // The MFMA phase, nothing conditional. (After the group's last tile S_{j+1} is computed from whatever the buffer
+    // holds and never used: cheaper than a second copy of this code.) Its 36 MFMAs are written in the order they are
+    // to issue, each preceded by the LDS reads of operands needed K_AHEAD MFMAs later, and nothing may move across the
+    // scheduling barriers between them: left to the scheduler, the reads end up directly in front of their MFMAs
+    // whenever it judges the register pressure of the function too high, and the pipe then idles through every read.
     auto mfma_phase = [&](int j) {
-        s_tile((j + 1) & 1, false);
+        constexpr int NS = 2 * DSTEPS, NG = 4, NV = NG * DBLKS;  // S MFMAs; (key block, k-step) pairs; V operands
+        const unsigned char *k_lds = k_base + ((j + 1) & 1) * K_TILE + k_lane;
         const unsigned char *v_lds = v_base + (j & 1) * V_TILE + v_lane;
-        // k-slot jj of k-step ks <-> key 32 kb + 16 ks + ... = accumulator 8 ks + jj of block kb, for both operands
+        U4H8 kop[NS];
+        union {
+            fp16x4_t f[2];
+            h8_t h;
+        } vop[NV];
+#pragma unroll
+        for (int i = 0; i < K_AHEAD; ++i) kop[i] = kpre[i];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                lacc = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, ones), __builtin_bit_cast(bf8_t, pb[kb][ks]), lacc, 0, 0, 0)
-                            : __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pb[kb][ks], lacc, 0, 0, 0);
+            for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.0f;
 #pragma unroll
-                for (int b = 0; b < DBLKS; ++b) {
-                    const unsigned char *p0 = v_lds + (kb * 8 + ks * 4) * RG_BYTES + b * 256;
-                    const unsigned char *p1 = p0 + 2 * RG_BYTES;
-                    union {
-                        fp16x4_t f[2];
-                        h8_t h;
-                    } va;
-                    va.f[0] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p0));
-                    va.f[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p1));
-                    oacc[b] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, va.h),
+        for (int i = 0; i < NS + NG * (DBLKS + 1); ++i) {
+            if (i + K_AHEAD < NS) {  // K operand i + K_AHEAD
+                const int t = i + K_AHEAD;
+                kop[t].u = *reinterpret_cast<const uint4 *>(k_lds + (t / DSTEPS) * (2 * RB_BYTES) + (t % DSTEPS) * 512);
+            }
+            const int pv = i - (NS - V_AHEAD);  // V operand pv: k-slot jj of k-step ks <-> key 32 kb + 16 ks + ... =
+            if (pv >= 0 && pv < NV) {           // accumulator 8 ks + jj of block kb, for both operands
+                const int g = pv / DBLKS, b = pv % DBLKS, kb = g / 2, ks = g % 2;
+                const unsigned char *p0 = v_lds + (kb * 8 + ks * 4) * RG_BYTES + b * 256;
+                vop[pv].f[0] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p0));
+                vop[pv].f[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p0 + 2 * RG_BYTES));
+            }
+            if (i < NS) {
+                const int kb = i / DSTEPS, st = i % DSTEPS;
+                sacc[kb] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop[i].b, qreg[st].b, sacc[kb], 0, 0, 0)
+                                : __builtin_amdgcn_mfma_f32_32x32x16_f16(kop[i].h, qreg[st].h, sacc[kb], 0, 0, 0);
+            } else {
+                const int g = (i - NS) / (DBLKS + 1), r = (i - NS) % (DBLKS + 1), kb = g / 2, ks = g % 2;
+                if (r == 0) {
+                    lacc = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, ones), __builtin_bit_cast(bf8_t, pb[kb][ks]), lacc, 0, 0, 0)
+                                : __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pb[kb][ks], lacc, 0, 0, 0);
+                } else {
+                    const int b = r - 1;
+                    oacc[b] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, vop[g * DBLKS + b].h),
                                                                            __builtin_bit_cast(bf8_t, pb[kb][ks]), oacc[b], 0, 0, 0)
-                                   : __builtin_amdgcn_mfma_f32_32x32x16_f16(va.h, pb[kb][ks], oacc[b], 0, 0, 0);
+                                   : __builtin_amdgcn_mfma_f32_32x32x16_f16(vop[g * DBLKS + b].h, pb[kb][ks], oacc[b], 0, 0, 0);
                 }
             }
-        // operand reads run K_AHEAD / V_AHEAD MFMAs ahead across both contractions
-        constexpr int NS = 2 * DSTEPS, NPV = 4 * DBLKS + 4, VR = 8 * DBLKS, V_EARLY = 2 * V_AHEAD;
-#pragma unroll
-        for (int i = 0; i < NS; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 2);
-            if (i < NS - K_AHEAD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 2);
-            else __builtin_amdgcn_sched_group_barrier(0x100, 2, 2);
-        }
-#pragma unroll
-        for (int i = 0; i < NPV; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 2);
-            if (V_EARLY + 2 * i < VR) __builtin_amdgcn_sched_group_barrier(0x100, 2, 2);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
-    if (ntg > 0) {
-        k_prefetch(0);
-        s_tile(0, true);
-    }
-    if (grp == 1) phase_barrier();  // one phase behind group 0
-    for (int j = 0; j < iters; ++j) {
-        if (j < ntg) {  // ---- VALU phase: P_j = 2^(c S_j - m), running max and sum
-            if (j + 2 < ntg) dma(true, j + 2, j & 1, pg_k);
-            if (j + 1 < ntg) dma(false, j + 1, (j + 1) & 1, pg_v);
-            pg_v = pg_k, pg_k = pg_next;
-            if (PAGED && j + 4 < ntg) pg_next = page_of(j + 4);
-            const uint32_t key0 = (uint32_t)(t0 + 2 * j) * BN;
-            const bool need_mask = (key0 + BN - 1 > wave_min_limit) || (key0 + BN > kv_end);
-            if (need_mask) {  // accumulator i of block kb is key key0 + 32 kb + 8 (i / 4) + 4 hi + i % 4
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const uint32_t key = key0 + kb * 32 + (i / 4) * 8 + hi * 4 + (i % 4);
-                        const bool vis = key < kv_end && (!a.causal || key <= q_abs);
-                        sacc[kb][i] = vis ? sacc[kb][i] : -INFINITY;
-                    }
-            }
-            float part[4] = {sacc[0][0], sacc[0][1], sacc[0][2], sacc[0][3]};  // four short chains, not one long
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) part[i & 3] = fmaxf(part[i & 3], sacc[kb][i]);
-            const float mloc = max_with_other_half(fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]))) * c;
-            // lazy rescale: only when a row maximum has grown by more than 2^8 (weights up to 256 until then; the
-            // final division by l removes the common factor)
-            if (__any(mloc > m_run + 8.0f)) {
-                const float m_new = fmaxf(m_run, mloc);
-                const float alpha = fast_exp2(m_run - m_new);
-                lacc[0] *= alpha;
-                m_run = m_new;
-#pragma unroll
-                for (int b = 0; b < DBLKS; ++b)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
-            }
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                    for (int jj = 0; jj < 8; ++jj)
-                        pb[kb][ks][jj] = to_elem<BF16>(fast_exp2(fmaf(sacc[kb][8 * ks + jj], c, -m_run)));
-            k_prefetch((j + 1) & 1);
-            if (j == 0) {  // V_0 has landed: everything but what this phase requested (K_2, V_1)
-                if (ntg > 2) __builtin_amdgcn_s_waitcnt(VMCNT_KV);
-                else if (ntg > 1) __builtin_amdgcn_s_waitcnt(VMCNT_V);
-                else __builtin_amdgcn_s_waitcnt(0x0F70);
-            }
-        }
-        phase_barrier();
-        if (j < ntg) mfma_phase(j);  // ---- MFMA phase
-        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the rows requested in the last VALU phase have landed
-        phase_barrier();
-    }
-    if (grp == 0) phase_barrier();  // same number of barriers for both groups
 
-    // merge the two groups' states: group 1 parks (m, l, acc) in LDS as [value][wave][lane], group 0 folds them in
-    {
-        float *mx = reinterpret_cast<float *>(lds);
-        const int slot = wave * 64 + lane;
-        if (grp == 1) {
-            mx[slot] = m_run;
-            mx[256 + slot] = lacc[0];
+    // ---- what a group does with a finished item. After the exchange below group g holds the merged accumulators of
+    // its half of the head dimension (blocks g DBLKS/2 ..) and the merged (m, l) of every row: it writes that half of
+    // the rows of query tile o_q0 of head o_head, normalised by 1 / l, or, with splits, the unnormalised state for the
+    // merge kernel.
+    constexpr int HB = DBLKS / 2;
+    auto write_item = [&](uint32_t o_item, auto G) {
+        constexpr int g = decltype(G)::value;
+        // (lane-derived values are worked out afresh from an opaque copy of the lane number: hoisted out of the item
+        // loop they would sit in registers through the tile loop, which has none to spare)
+        int lo = lane;
+        asm volatile("" : "+v"(lo));
+        const int n = lo & 31, hi = lo >> 5, lane = lo;
+        const uint32_t o_qi = o_item / (a.n_heads * S), o_rest = o_item - o_qi * (a.n_heads * S);
+        const uint32_t o_head = o_rest / S, o_q0 = (n_qt - 1 - o_qi) * BM;
+        const float o_m = m_run, o_l = lacc[0];  // untouched since the exchange
+        const uint32_t q_row = o_q0 + wave * 32 + n;
+        if (S > 1) {  // flash_prefill.metal:592-617
+            if (q_row < a.q_len) {
+                const size_t prow = (size_t)((o_head * n_qt + (n_qt - 1 - o_qi)) * S + (o_rest - o_head * S)) * BM + wave * 32 + n;
+                float *pa = a.part_acc + prow * D;
 #pragma unroll
-            for (int b = 0; b < DBLKS; ++b)
+                for (int b = g * HB; b < (g + 1) * HB; ++b)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) mx[(2 + b * 16 + i) * 256 + slot] = oacc[b][i];
+                    for (int gi = 0; gi < 4; ++gi) {
+                        float4 v = make_float4(oacc[b][gi * 4], oacc[b][gi * 4 + 1], oacc[b][gi * 4 + 2], oacc[b][gi * 4 + 3]);
+                        *reinterpret_cast<float4 *>(pa + b * 32 + gi * 8 + hi * 4) = v;
+                    }
+                if (g == 0 && hi == 0) a.part_ml[prow * 2] = o_m, a.part_ml[prow * 2 + 1] = o_l;
+            }
+            return;
         }
-        __syncthreads();
-        if (grp == 1) return;
-        const float m1 = mx[slot], l1 = mx[256 + slot];
+        const float inv_l = (isfinite(o_l) && fabsf(o_l) > 1e-6f) ? (1.0f / o_l) : 0.0f;  // flash_prefill.metal:255-261
+        if (a.out_aligned16) {
+            // A lane holds one row's values in 8-byte pieces, 64 rows' pieces per store instruction: written like that,
+            // every instruction touches 64 cache lines and the L2 is left with half-written lines to flush (measured:
+            // 5 us of a 47 us launch at 2048 tokens, 39 of 454 at 8192). So the wave's 32 half rows go through the part
+            // of the group's second V buffer that only this wave's loads fill (LDS runs a wave's accesses in order: no
+            // barrier), 16-byte chunks exchanged by row number against bank conflicts, and leave D bytes at a time.
+            constexpr int HROW = ROWB / 2, CPR = HROW / 16, RPI = 64 / CPR;  // half row; its 16-byte chunks; rows per store
+            unsigned char *ot = v_base + V_TILE + wave * (16 * ROWB);
+            // byte offsets inside the slice as exclusive-ors of a lane part and a constant part (the row, the chunk and
+            // the 8-byte half occupy separate bits)
+            int w_off = n * HROW + (n & (CPR - 1)) * 16 + hi * 8;                                // ^ chunk * 16
+            int r_off = (lane / CPR) * HROW + (((lane % CPR) ^ ((lane / CPR) & (CPR - 1))) * 16);  // ^ (row and chunk bits of it * RPI)
+            asm volatile("" : "+v"(w_off), "+v"(r_off));
+#pragma unroll
+            for (int bb = 0; bb < HB; ++bb)
+#pragma unroll
+                for (int gi = 0; gi < 4; ++gi) {  // accumulators 4gi..4gi+3 of block b are d = 32b + 8gi + 4hi + 0..3
+                    h4_t o;
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) o[jj] = to_elem<BF16>(oacc[g * HB + bb][gi * 4 + jj] * inv_l);
+                    *reinterpret_cast<h4_t *>(ot + (w_off ^ ((bb * 4 + gi) * 16))) = o;
+                }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+            __half *ob = a.out + (size_t)o_head * a.out_stride_h + g * (D / 2) + (lane % CPR) * 8;
+#pragma unroll
+            for (int it = 0; it < 32 / RPI; ++it) {
+                const int row = it * RPI + lane / CPR;
+                const uint32_t qr = o_q0 + wave * 32 + row;
+                const uint4 val = *reinterpret_cast<const uint4 *>(ot + (r_off ^ (it * RPI * HROW + ((it * RPI) & (CPR - 1)) * 16)));
+                if (qr < a.q_len) __builtin_nontemporal_store(__builtin_bit_cast(u4_t, val), reinterpret_cast<u4_t *>(ob + (size_t)qr * a.out_stride_m));
+            }
+            return;
+        }
+        if (q_row < a.q_len) {
+            __half *op = a.out + (size_t)o_head * a.out_stride_h + (size_t)q_row * a.out_stride_m;
+#pragma unroll
+            for (int b = g * HB; b < (g + 1) * HB; ++b)
+#pragma unroll
+                for (int gi = 0; gi < 4; ++gi) {  // accumulators 4gi..4gi+3 are d = 32b + 8gi + 4hi + 0..3
+                    h4_t o;
+#pragma unroll
+                    for (int jj = 0; jj < 4; ++jj) o[jj] = to_elem<BF16>(oacc[b][gi * 4 + jj] * inv_l);
+                    *reinterpret_cast<h4_t *>(op + b * 32 + gi * 8 + hi * 4) = o;
+                }
+        }
+    };
+    // The exchange: a group parks (m, l) and the accumulators of the OTHER group's half in its own, now idle, tile
+    // buffers as [value][wave][lane]; after a barrier it folds what the other group parked into its own half.
+    auto park = [&](auto G) {
+        constexpr int g = decltype(G)::value;
+        int lo = lane;
+        asm volatile("" : "+v"(lo));  // (see write_item)
+        float *mx = reinterpret_cast<float *>(lds + g * GRP_LDS) + wave * 64 + lo;
+        mx[0] = m_run;
+        mx[256] = lacc[0];
+#pragma unroll
+        for (int bb = 0; bb < HB; ++bb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) mx[(2 + bb * 16 + i) * 256] = oacc[(1 - g) * HB + bb][i];
+    };
+    auto fold = [&](auto G) {
+        constexpr int g = decltype(G)::value;
+        int lo = lane;
+        asm volatile("" : "+v"(lo));  // (see write_item)
+        const float *mx = reinterpret_cast<const float *>(lds + (1 - g) * GRP_LDS) + wave * 64 + lo;
+        const float m1 = mx[0], l1 = mx[256];
         const float m = fmaxf(m_run, m1);
         const float e0 = fast_exp2(m_run - m), e1 = fast_exp2(m1 - m);
         lacc[0] = lacc[0] * e0 + l1 * e1;
 #pragma unroll
-        for (int b = 0; b < DBLKS; ++b)
+        for (int bb = 0; bb < HB; ++bb)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) oacc[b][i] = oacc[b][i] * e0 + mx[(2 + b * 16 + i) * 256 + slot] * e1;
+            for (int i = 0; i < 16; ++i) oacc[g * HB + bb][i] = oacc[g * HB + bb][i] * e0 + mx[(2 + bb * 16 + i) * 256] * e1;
         m_run = m;
+    };
+
+    // On entry to MFMA phase j the LDS holds K_{j+1} in K[(j+1)&1] and V_j in V[j&1]. VALU phase j starts by
+    // requesting K_{j+2} into K[j&1] and V_{j+1} into V[(j+1)&1] (both buffers were last read in MFMA phase j-1);
+    // the requests are complete (vmcnt) before the barrier that ends MFMA phase j, two phases later, so VALU phase
+    // j+1 may already fetch the first operands of MFMA phase j+1 ahead of its barrier.
+    //
+    // Items follow one another inside the workgroup, and what an item costs beyond its tiles is kept off the matrix
+    // pipe's path where it can be: the next item's query rows are requested during the first MFMA phase of the
+    // current one (their own 32 KB of LDS); group 0, which ends one phase before group 1, parks its state while group
+    // 1 runs its last phase; group 1 folds it in and writes the rows out after both groups have requested the next
+    // item's first tiles. Nothing but scalars lives from one item to the next: with accumulators alive across the
+    // item loop the register allocator ran out inside the tile loop and gave up the operand read-ahead there.
+    constexpr int VMCNT_V = 0x0F70 | V_DMA, VMCNT_KV = 0x0F70 | (V_DMA + K_DMA), VMCNT_Q = 0x0F70 | K_DMA;
+    uint32_t round = 0, item = blockIdx.x;
+    int32_t pg_k = 0, pg_v = 0, pg_next = 0;  // pages of the K tile / V tile requested next, and of the K tile after
+    auto first_tiles = [&]() {
+        if (ntg > 0) {
+            const int32_t p0 = page_of(0), p1 = page_of(1);
+            pg_k = page_of(2), pg_next = page_of(3), pg_v = p1;
+            dma(true, 0, 0, p0);
+            if (ntg > 1) dma(true, 1, 1, p1);
+            dma(false, 0, 0, p0);
+        }
+    };
+    enter_item(item);
+    q_dma(item);
+    first_tiles();
+    while (true) {
+        const uint32_t next_item = item_of(round + 1);
+        const bool has_next = next_item < n_items;
+        // Q, K_0 (for S_0) and K_1 (whose first operands the first VALU phase reads ahead) must be there now; V_0,
+        // requested last (loads complete in order), has until the first MFMA phase. A CU pulls about 25 GB/s on its
+        // own, so every 16 KB not waited for here is worth half a microsecond.
+        if (ntg > 0) __builtin_amdgcn_s_waitcnt(VMCNT_V);
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        {
+            int lo = lane;
+            asm volatile("" : "+v"(lo));  // (see write_item)
+            const int rb = wave * 2 + ((lo & 31) >> 4);  // 16-row block of this lane's row; both groups hold the same 128 rows
+            const unsigned char *qp = lds + 2 * GRP_LDS + rb * RB_BYTES + (lo >> 5) * 256 + (lo & 15) * 16;
+#pragma unroll
+            for (int s = 0; s < DSTEPS; ++s) qreg[s].u = *reinterpret_cast<const uint4 *>(qp + s * 512);
+#pragma unroll
+            for (int s = 0; s < DSTEPS; ++s) {  // arrived: keep the wait out of the loop
+                u4_t t = __builtin_bit_cast(u4_t, qreg[s].u);
+                asm volatile("" : "+v"(t));
+                qreg[s].u = __builtin_bit_cast(uint4, t);
+            }
+        }
+        clear_state();
+        const uint32_t q_row_c = min(q0 + wave * 32 + n, a.q_len - 1);
+        const uint32_t q_abs = q_row_c + a.query_offset;
+        const uint32_t wave_min_limit = a.causal ? (min(q0 + wave * 32, a.q_len - 1) + a.query_offset) : 0xffffffffu;
+        if (ntg > 0) {
+            k_prefetch(0);
+            s_tile(0);
+        }
+        if (grp == 1) phase_barrier();  // one phase behind group 0
+        for (int j = 0; j < iters; ++j) {
+            if (j < ntg) {  // ---- VALU phase: P_j = 2^(c S_j - m), running max and sum
+                if (j + 2 < ntg) dma(true, j + 2, j & 1, pg_k);
+                if (j + 1 < ntg) dma(false, j + 1, (j + 1) & 1, pg_v);
+                pg_v = pg_k, pg_k = pg_next;
+                if (PAGED && j + 4 < ntg) pg_next = page_of(j + 4);
+                const uint32_t key0 = (uint32_t)(t0 + 2 * j) * BN;
+                const bool need_mask = (key0 + BN - 1 > wave_min_limit) || (key0 + BN > kv_end);
+                if (need_mask) {  // accumulator i of block kb is key key0 + 32 kb + 8 (i / 4) + 4 hi + i % 4
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            const uint32_t key = key0 + kb * 32 + (i / 4) * 8 + hi * 4 + (i % 4);
+                            const bool vis = key < kv_end && (!a.causal || key <= q_abs);
+                            sacc[kb][i] = vis ? sacc[kb][i] : -INFINITY;
+                        }
+                }
+                float part[4] = {sacc[0][0], sacc[0][1], sacc[0][2], sacc[0][3]};  // four short chains, not one long
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) part[i & 3] = fmaxf(part[i & 3], sacc[kb][i]);
+                const float mloc = max_with_other_half(fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3]))) * c;
+                // lazy rescale: only when a row maximum has grown by more than 2^8 (weights up to 256 until then; the
+                // final division by l removes the common factor)
+                if (__any(mloc > m_run + 8.0f)) {
+                    const float m_new = fmaxf(m_run, mloc);
+                    const float alpha = fast_exp2(m_run - m_new);
+                    lacc[0] *= alpha;
+                    m_run = m_new;
+#pragma unroll
+                    for (int b = 0; b < DBLKS; ++b)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
+                }
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                        for (int jj = 0; jj < 8; ++jj)
+                            pb[kb][ks][jj] = to_elem<BF16>(fast_exp2(fmaf(sacc[kb][8 * ks + jj], c, -m_run)));
+                k_prefetch((j + 1) & 1);
+                if (j == 0) {  // V_0 has landed: everything but what this phase requested (K_2, V_1)
+                    if (ntg > 2) __builtin_amdgcn_s_waitcnt(VMCNT_KV);
+                    else if (ntg > 1) __builtin_amdgcn_s_waitcnt(VMCNT_V);
+                    else __builtin_amdgcn_s_waitcnt(0x0F70);
+                }
+            }
+            phase_barrier();
+            // every wave has taken its query rows out of LDS (each passed a barrier since): the next item's may come
+            const bool stage_now = j == 0 && has_next;
+            if (stage_now) q_dma(next_item);
+            if (j < ntg) mfma_phase(j);  // ---- MFMA phase
+            // the rows requested in the last VALU phase have landed (the query rows just requested may take longer)
+            if (stage_now) __builtin_amdgcn_s_waitcnt(VMCNT_Q);
+            else __builtin_amdgcn_s_waitcnt(0x0F70);
+            phase_barrier();
+        }
+        const bool q_staged = has_next && iters > 0;
+
+        // merge the two groups' states: group 0 parks while group 1 runs its last phase
+        if (grp == 0) {
+            park(std::integral_constant<int, 0>());
+            phase_barrier();  // same number of barriers for both groups
+        } else {
+            park(std::integral_constant<int, 1>());
+        }
+        __syncthreads();
+        if (grp == 0) fold(std::integral_constant<int, 0>());
+        else fold(std::integral_constant<int, 1>());
+        __syncthreads();  // the parked states have been read: the buffers may receive the next item's tiles
+        // the next item's first tiles are requested before this one's rows are written out
+        const uint32_t o_item = item;
+        if (has_next) {
+            item = next_item, ++round;
+            enter_item(item);
+            if (!q_staged) q_dma(item);
+            first_tiles();
+        }
+        if (grp == 0) write_item(o_item, std::integral_constant<int, 0>());
+        else write_item(o_item, std::integral_constant<int, 1>());
+        if (!has_next) break;
     }
-    const float l_tot = lacc[0];
     if (a.clock_out && threadIdx.x == 0) {
         a.clock_out[(size_t)blockIdx.x * 2] = __builtin_readcyclecounter() - clk0;
         a.clock_out[(size_t)blockIdx.x * 2 + 1] = wall_clock64() - wall0;
-    }
-    if (S > 1) {  // unnormalised partial state for the merge kernel (flash_prefill.metal:592-617)
-        if (q_row >= a.q_len) return;
-        const size_t prow = (((size_t)head * n_qt + q_tile) * S + split) * BM + wave * 32 + n;
-        float *pa = a.part_acc + prow * D;
-#pragma unroll
-        for (int b = 0; b < DBLKS; ++b)
-#pragma unroll
-            for (int gi = 0; gi < 4; ++gi) {
-                float4 v = make_float4(oacc[b][gi * 4], oacc[b][gi * 4 + 1], oacc[b][gi * 4 + 2], oacc[b][gi * 4 + 3]);
-                *reinterpret_cast<float4 *>(pa + b * 32 + gi * 8 + hi * 4) = v;
-            }
-        if (hi == 0) a.part_ml[prow * 2] = m_run, a.part_ml[prow * 2 + 1] = l_tot;
-        return;
-    }
-    const float inv_l = (isfinite(l_tot) && fabsf(l_tot) > 1e-6f) ? (1.0f / l_tot) : 0.0f;  // flash_prefill.metal:255-261
-    if (a.out_aligned16) {
-        // A lane holds one row's values in 8-byte pieces, 64 rows' pieces per store instruction: written like that, every
-        // instruction touches 64 cache lines and the L2 is left with half-written lines to flush at the kernel's end
-        // (measured: 5 us of a 47 us launch at 2048 tokens, 39 of 454 at 8192). So the wave's 32 rows go through its own
-        // corner of LDS (past what the group merge used; LDS runs a wave's accesses in order, no barrier) and leave as
-        // whole 256-byte rows, 16 bytes per lane.
-        constexpr int ORS = ROWB + 16, RPI = 1024 / ROWB;  // LDS row stride; rows per store instruction
-        unsigned char *ot = lds + 2 * GRP_LDS - 4 * 32 * ORS + wave * (32 * ORS);
-#pragma unroll
-        for (int b = 0; b < DBLKS; ++b)
-#pragma unroll
-            for (int gi = 0; gi < 4; ++gi) {  // accumulators 4gi..4gi+3 are d = 32b + 8gi + 4hi + 0..3
-                h4_t o;
-#pragma unroll
-                for (int jj = 0; jj < 4; ++jj) o[jj] = to_elem<BF16>(oacc[b][gi * 4 + jj] * inv_l);
-                *reinterpret_cast<h4_t *>(ot + n * ORS + (b * 32 + gi * 8 + hi * 4) * 2) = o;
-            }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-        const int rl = lane / (ROWB / 16), ch = lane % (ROWB / 16);
-        __half *ob = a.out + (size_t)head * a.out_stride_h + ch * 8;
-#pragma unroll
-        for (int it = 0; it < 32 / RPI; ++it) {
-            const int row = it * RPI + rl;
-            const uint32_t qr = q0 + wave * 32 + row;
-            const uint4 val = *reinterpret_cast<const uint4 *>(ot + row * ORS + ch * 16);
-            if (qr < a.q_len) __builtin_nontemporal_store(__builtin_bit_cast(u4_t, val), reinterpret_cast<u4_t *>(ob + (size_t)qr * a.out_stride_m));
-        }
-        return;
-    }
-    if (q_row < a.q_len) {
-        __half *op = a.out + (size_t)head * a.out_stride_h + (size_t)q_row * a.out_stride_m;
-#pragma unroll
-        for (int b = 0; b < DBLKS; ++b)
-#pragma unroll
-            for (int gi = 0; gi < 4; ++gi) {  // accumulators 4gi..4gi+3 are d = 32b + 8gi + 4hi + 0..3
-                h4_t o;
-#pragma unroll
-                for (int jj = 0; jj < 4; ++jj) o[jj] = to_elem<BF16>(oacc[b][gi * 4 + jj] * inv_l);
-                *reinterpret_cast<h4_t *>(op + b * 32 + gi * 8 + hi * 4) = o;
-            }
     }
 }
 
@@ -963,11 +1061,14 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
         a.part_acc = (float *)ctx->workspace;
         a.part_ml = (float *)((char *)ctx->workspace + acc_bytes);
     }
-    dim3 grid(base_wgs * splits, 1, 1);
+    // the LDS-direct kernel (measured faster at every size) addresses the query rows of a head with 32-bit offsets
+    const bool lds_direct = ctx->prefill_variant != 1 && ((uint64_t)(L.q_len - 1) * L.q_stride_m + L.head_dim) * 2 < (1ull << 32);
+    // Its workgroups (one fits a CU) stay and share out the (query tile, head, split) items among themselves.
+    a.n_qt = ceil_div_u32(L.q_len, BM), a.n_items = base_wgs * splits;
+    a.n_workgroups = lds_direct ? (a.n_items < n_cus ? a.n_items : n_cus) : a.n_items;
+    dim3 grid(a.n_workgroups, 1, 1);
     if (ctx->clock_buf && grid.x <= ctx->clock_buf_workgroups) a.clock_out = ctx->clock_buf;
     {
-        // the LDS-direct kernel (measured faster at every size) addresses the query rows of a head with 32-bit offsets
-        const bool lds_direct = ctx->prefill_variant != 1 && ((uint64_t)(L.q_len - 1) * L.q_stride_m + L.head_dim) * 2 < (1ull << 32);
         FaLaunchScope scope(ctx, lds_direct ? "flash_prefill_dma_kernel" : "flash_prefill_mfma_kernel", true);
         if (lds_direct) {
             auto kern = flash_prefill_dma_kernel<128, false, false>;
