@@ -609,23 +609,19 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     };
 
     f16_t oacc[DBLKS];
-    // Row sums ride on the matrix pipe: an all-ones A operand against P^T leaves, in every accumulator of a lane,
-    // the sum of that lane's query row over the keys of the step (both lane halves included) - 4 more MFMAs a tile
-    // instead of 32 more additions in the VALU phase, which is the longer one. Only element 0 is ever read.
-    f16_t lacc;
+    // Row sums are added up in the VALU phase, each lane over the keys it holds (the other half of the row's keys is
+    // in lane ^ 32 and joins at the end of the item). On the matrix pipe (an all-ones operand against P^T: 4 more MFMAs
+    // a tile) they cost 16 registers and a ninth of the pipe's energy, and the part is power-limited on this kernel.
+    float l_run;
     float m_run;
     auto clear_state = [&]() {
 #pragma unroll
         for (int b = 0; b < DBLKS; ++b)
 #pragma unroll
             for (int i = 0; i < 16; ++i) oacc[b][i] = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) lacc[i] = 0.0f;
+        l_run = 0.0f;
         m_run = -1e30f;
     };
-    h8_t ones;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) ones[i] = to_elem<BF16>(1.0f);
     const float c = a.scale_log2e;
 
     const int k_lane = (n >> 4) * RB_BYTES + hi * 256 + (n & 15) * 16;
@@ -661,7 +657,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         }
     };
     // The MFMA phase, nothing conditional. (After the group's last tile S_{j+1} is computed from whatever the buffer
-    // holds and never used: cheaper than a second copy of this code.) Its 36 MFMAs are written in the order they are
+    // holds and never used: cheaper than a second copy of this code.) Its 32 MFMAs are written in the order they are
     // to issue, each preceded by the LDS reads of operands needed K_AHEAD MFMAs later, and nothing may move across the
     // scheduling barriers between them: left to the scheduler, the reads end up directly in front of their MFMAs
     // whenever it judges the register pressure of the function too high, and the pipe then idles through every read.
@@ -681,7 +677,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
 #pragma unroll
             for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.0f;
 #pragma unroll
-        for (int i = 0; i < NS + NG * (DBLKS + 1); ++i) {
+        for (int i = 0; i < NS + NV; ++i) {
             if (i + K_AHEAD < NS) {  // K operand i + K_AHEAD
                 const int t = i + K_AHEAD;
                 kop[t].u = *reinterpret_cast<const uint4 *>(k_lds + (t / DSTEPS) * (2 * RB_BYTES) + (t % DSTEPS) * 512);
@@ -698,16 +694,10 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
                 sacc[kb] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop[i].b, qreg[st].b, sacc[kb], 0, 0, 0)
                                 : __builtin_amdgcn_mfma_f32_32x32x16_f16(kop[i].h, qreg[st].h, sacc[kb], 0, 0, 0);
             } else {
-                const int g = (i - NS) / (DBLKS + 1), r = (i - NS) % (DBLKS + 1), kb = g / 2, ks = g % 2;
-                if (r == 0) {
-                    lacc = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, ones), __builtin_bit_cast(bf8_t, pb[kb][ks]), lacc, 0, 0, 0)
-                                : __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pb[kb][ks], lacc, 0, 0, 0);
-                } else {
-                    const int b = r - 1;
-                    oacc[b] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, vop[g * DBLKS + b].h),
-                                                                           __builtin_bit_cast(bf8_t, pb[kb][ks]), oacc[b], 0, 0, 0)
-                                   : __builtin_amdgcn_mfma_f32_32x32x16_f16(vop[g * DBLKS + b].h, pb[kb][ks], oacc[b], 0, 0, 0);
-                }
+                const int g = (i - NS) / DBLKS, b = (i - NS) % DBLKS, kb = g / 2, ks = g % 2;
+                oacc[b] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, vop[g * DBLKS + b].h),
+                                                                       __builtin_bit_cast(bf8_t, pb[kb][ks]), oacc[b], 0, 0, 0)
+                               : __builtin_amdgcn_mfma_f32_32x32x16_f16(vop[g * DBLKS + b].h, pb[kb][ks], oacc[b], 0, 0, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -727,7 +717,10 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         const int n = lo & 31, hi = lo >> 5, lane = lo;
         const uint32_t o_qi = o_item / (a.n_heads * S), o_rest = o_item - o_qi * (a.n_heads * S);
         const uint32_t o_head = o_rest / S, o_q0 = (n_qt - 1 - o_qi) * BM;
-        const float o_m = m_run, o_l = lacc[0];  // untouched since the exchange
+        const float o_m = m_run;  // untouched since the exchange, like l_run: this lane's half of the row's keys
+        typedef unsigned int u2v __attribute__((ext_vector_type(2)));
+        const u2v lsw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
+        const float o_l = __uint_as_float(lsw.x) + __uint_as_float(lsw.y);
         const uint32_t q_row = o_q0 + wave * 32 + n;
         if (S > 1) {  // flash_prefill.metal:592-617
             if (q_row < a.q_len) {
@@ -801,7 +794,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         asm volatile("" : "+v"(lo));  // (see write_item)
         float *mx = reinterpret_cast<float *>(lds + g * GRP_LDS) + wave * 64 + lo;
         mx[0] = m_run;
-        mx[256] = lacc[0];
+        mx[256] = l_run;
 #pragma unroll
         for (int bb = 0; bb < HB; ++bb)
 #pragma unroll
@@ -815,7 +808,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         const float m1 = mx[0], l1 = mx[256];
         const float m = fmaxf(m_run, m1);
         const float e0 = fast_exp2(m_run - m), e1 = fast_exp2(m1 - m);
-        lacc[0] = lacc[0] * e0 + l1 * e1;
+        l_run = l_run * e0 + l1 * e1;
 #pragma unroll
         for (int bb = 0; bb < HB; ++bb)
 #pragma unroll
@@ -910,20 +903,25 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
                 if (__any(mloc > m_run + 8.0f)) {
                     const float m_new = fmaxf(m_run, mloc);
                     const float alpha = fast_exp2(m_run - m_new);
-                    lacc[0] *= alpha;
+                    l_run *= alpha;
                     m_run = m_new;
 #pragma unroll
                     for (int b = 0; b < DBLKS; ++b)
 #pragma unroll
                         for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
                 }
+                float psum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                     for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                        for (int jj = 0; jj < 8; ++jj)
-                            pb[kb][ks][jj] = to_elem<BF16>(fast_exp2(fmaf(sacc[kb][8 * ks + jj], c, -m_run)));
+                        for (int jj = 0; jj < 8; ++jj) {
+                            const float e = fast_exp2(fmaf(sacc[kb][8 * ks + jj], c, -m_run));
+                            psum[jj & 3] += e;
+                            pb[kb][ks][jj] = to_elem<BF16>(e);
+                        }
+                l_run += (psum[0] + psum[1]) + (psum[2] + psum[3]);
                 k_prefetch((j + 1) & 1);
                 if (j == 0) {  // V_0 has landed: everything but what this phase requested (K_2, V_1)
                     if (ntg > 2) __builtin_amdgcn_s_waitcnt(VMCNT_KV);
