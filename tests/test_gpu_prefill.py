@@ -116,6 +116,37 @@ def test_prefill_rows_equal_decode_and_first_row():
         assert max_abs(do.download().reshape(H, D), got[:, r]) <= 1.5e-3
 
 
+@pytest.mark.parametrize("H,Hkv,D,M", [(24, 8, 128, 4133), (14, 2, 64, 5000)])
+def test_prefill_many_items_per_workgroup_rows_equal_decode(H, Hkv, D, M):
+    """More (query tile, head) items than three times the CUs, the last tile ragged: every resident workgroup works
+    through several items in turn. Sampled rows (tile edges, the ragged end) against the decode kernel's answer for the
+    same row, which the oracle tests pin; rows of the output nobody should have touched stay as they were."""
+    announce("prefill, several items per workgroup", H, Hkv, D, M)
+    f = ctx()
+    rng = np.random.default_rng(M)
+    q, k, v = h16(rng.normal(size=(H, M, D))), h16(rng.normal(size=(Hkv, M, D))), h16(rng.normal(size=(Hkv, M, D)))
+    dq, dk, dv = f.array(q), f.array(k), f.array(v)
+    guard = 3
+    sentinel = np.float16(-7.5)
+    dout = f.array(np.full((M + guard, H * D), sentinel, np.float16))
+    f.flash_attention(dq.arg((H, M, D)), dk.arg(), dv.arg(), dout.arg((M, H * D)), True, 0, H, D, M, M)
+    f.synchronize()
+    got = dout.download()
+    assert np.all(got[M:] == sentinel), "rows past the last query were written"
+    got = got[:M].reshape(M, H, D)
+    assert np.isfinite(got.astype(np.float32)).all()
+    rows = sorted({0, 1, 127, 128, 129, 2047, 2048, 3000, M - 130, M - 2, M - 1} | set(rng.integers(0, M, 6).tolist()))
+    d1 = f.zeros((1, H * D))
+    for r in rows:
+        dqr = f.array(np.ascontiguousarray(q[:, r]))
+        f.flash_attention(dqr.arg((1, H * D)), dk.arg(), dv.arg(), d1.arg(), True, r, H, D, r + 1, 1)
+        f.synchronize()
+        assert max_abs(d1.download().reshape(H, D), got[r]) <= 1.5e-3, r
+        dqr.free()
+    for b in (dq, dk, dv, dout, d1):
+        b.free()
+
+
 def test_prefill_llama_shape_full_size_from_paged_cache():
     """benchmark configuration 4: 2048-token prompt, H24/Hkv8/D128, RoPE theta 5e5 on positions 0..2047, all rows
     appended into an empty paged cache, causal flash attention reading through the block table."""
