@@ -239,10 +239,10 @@ def calibration_copy(f, reps=3):
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense f16 / bf16 matrix peak
 
 
-def bench_prefill(f, args):
-    """Llama-3.2-3B-shaped prefill of one layer: 2048 tokens, RoPE + append into an empty paged cache, then causal
-    flash prefill from the paged cache. One step = both launches."""
-    H, Hkv, D, M, bs = 24, 8, 128, 2048, 16
+def bench_prefill(f, args, tokens=2048):
+    """Llama-3.2-3B-shaped prefill of one layer: `tokens` tokens (2048 = benchmark configuration 4), RoPE + append into an
+    empty paged cache, then causal flash prefill from the paged cache. One step = both launches."""
+    H, Hkv, D, M, bs = 24, 8, 128, tokens, 16
     rng = np.random.default_rng(0xF0DD + 4)
     nblk = M // bs
     perm = rng.permutation(nblk).astype(np.int32).reshape(1, nblk)
@@ -299,12 +299,12 @@ def bench_prefill(f, args):
     achieved = flops / avg_pf_s / 1e12
     append_bytes = 2.0 * M * (H + 2 * Hkv) * D * 2  # read q, k, v; write q_rot and the cache rows
     result = {
-        "metric": "prefill-attn steps/s + achieved f16 MFMA TFLOP/s (% peak), Llama-3.2-3B shape, 2048 tokens",
+        "metric": "prefill-attn steps/s + achieved f16 MFMA TFLOP/s (%% peak), Llama-3.2-3B shape, %d tokens" % M,
         "value": args.steps / dt, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "llama3.2-3b prefill attention, one layer: RoPE + append of 2048 tokens into an empty paged "
-                               "f16 cache (16-token blocks, permuted block table), then causal flash prefill, H24/Hkv8/D128"},
+        "config": {"workload": "llama3.2-3b prefill attention, one layer: RoPE + append of %d tokens into an empty paged "
+                               "f16 cache (16-token blocks, permuted block table), then causal flash prefill, H24/Hkv8/D128" % M},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_F16_PEAK_TFLOPS, "traffic": None, "kernel": pf_kernel,
                      "avg_launch_us": avg_pf_s * 1e6, "launches": n_pf, "flops_per_launch": flops},
@@ -977,10 +977,38 @@ def bench_floors(f, args):
         for b in srcs + dsts:
             b.free()
     word.free()
+    # Shader clock the board sustains: under back-to-back MFMAs on every CU (fa_measure_clock), and inside the prefill
+    # kernel itself (fa_profile_clock_buffer: each resident workgroup's shader-clock ticks over its 100 MHz wall ticks)
+    # on random and on all-zero inputs. The published matrix peak is the figure at 2.4 GHz.
+    clocks = {}
+    mhz, busy = f.measure_clock(True, 200000)
+    clocks["mfma_probe"] = {"shader_mhz": mhz, "busy_ms": busy, "what": "fa_measure_clock: 8 waves of dependent-free v_mfma_f32_32x32x16_f16 per CU"}
+    H = 24
+    rng = np.random.default_rng(11)
+    for M in (2048, 8192):
+        for data in ("random", "zero"):
+            mk = (lambda n: f.array(rng.standard_normal((n, M, D), dtype=np.float32).astype(np.float16))) if data == "random" else (lambda n: f.zeros((n, M, D)))
+            q, k, v, o = mk(H), mk(Hkv), mk(Hkv), f.zeros((M, H * D))
+            n_wg = min(f.n_cus(), -(-M // 128) * H)
+            buf = fa.DevBuf(f, (n_wg, 2), np.int64)
+            for rep in range(24):  # long enough for the power management to settle; the last launch's readings count
+                if rep == 23:
+                    f.profile_clock_buffer(buf, n_wg)
+                f.flash_attention(q.arg(), k.arg(), v.arg(), o.arg(), True, 0, H, D, M, M)
+            f.synchronize()
+            f.profile_clock_buffer(None, 0)
+            h = buf.download().astype(np.float64)
+            clocks["prefill_%d_%s" % (M, data)] = {"shader_mhz": float(np.mean(h[:, 0] / h[:, 1]) * 100.0),
+                                                    "cycles_per_workgroup_median": float(np.median(h[:, 0])),
+                                                    "what": "flash_prefill_dma_kernel, Llama-3.2-3B shape, %d tokens, %s inputs" % (M, data)}
+            for b in (q, k, v, o, buf):
+                b.free()
+    out["floors"]["clock"] = clocks
     emit(out)
 
 
-SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill, "qwen05b_decode_1k": bench_small_decode,
+SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill,
+             "llama3b_prefill_8k": lambda f, args: bench_prefill(f, args, 8192), "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
              "llama3b_o_proj": bench_o_proj,

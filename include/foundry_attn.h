@@ -121,9 +121,13 @@ fa_status fa_profile_query(fa_ctx *ctx, const char *kernel_prefix, uint64_t *lau
 
 /* Clock readings from inside the prefill kernel (its LDS-direct variant): while a buffer of n_workgroups x 2 u64 is set,
  * every prefill launch of at most n_workgroups workgroups leaves per workgroup {shader-clock ticks, 100 MHz wall-clock
- * ticks} between its first instruction and the end of its key loop; ticks / wall x 100 = the MHz the kernel really ran
- * at (the matrix peak scales with it). NULL switches it off. */
+ * ticks} between its first instruction and its last (that kernel launches min(items, compute units) workgroups, each
+ * of which works through several (query tile, head) items); ticks / wall x 100 = the MHz the kernel really ran at (the
+ * matrix peak scales with it). NULL switches it off. */
 fa_status fa_profile_clock_buffer(fa_ctx *ctx, void *d_buffer, uint32_t n_workgroups);
+
+/* Compute units of the context's device (what the launch-sizing rules count in). */
+fa_status fa_compute_units(fa_ctx *ctx, uint32_t *n);
 
 /* Device memory, the executor's buffer management (src/model/executor.rs:2286-2328, src/lib.rs:317-377).
  * fa_upload/fa_download are synchronous with respect to the context's stream. */

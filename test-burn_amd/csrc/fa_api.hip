@@ -395,6 +395,13 @@ extern "C" fa_status fa_profile_clock_buffer(fa_ctx *ctx, void *d_buffer, uint32
     return FA_OK;
 }
 
+extern "C" fa_status fa_compute_units(fa_ctx *ctx, uint32_t *n) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(n, "n");
+    *n = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 0u;
+    return FA_OK;
+}
+
 // memory ----------------------------------------------------------------------------------------
 
 extern "C" fa_status fa_device_alloc(fa_ctx *ctx, size_t bytes, void **out) {
@@ -1344,6 +1351,7 @@ extern "C" fa_status fa_flash_prefill_paged(fa_ctx *ctx, const fa_tensor_arg *q,
     P.bf16 = FA_IS_BF16(q);
     P.paged = true, P.block_table = cache->block_table + (size_t)seq_index * cache->max_blocks_per_seq;
     P.block_size = cache->block_size, P.n_kv_heads = cache->n_kv_heads;
+    P.pool_bytes = (uint64_t)cache->n_blocks * cache->n_kv_heads * cache->block_size * D * 2;
     return fa_launch_prefill(ctx, P);
 }
 

@@ -208,6 +208,7 @@ struct PrefillLaunch {
     bool paged;
     const int32_t *block_table;
     uint32_t block_size, n_kv_heads;
+    uint64_t pool_bytes;  // paged: size of each pool (0 = unknown)
     bool bf16;  // q, k, v and out are bf16 instead of f16
 };
 fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &a);

@@ -51,6 +51,7 @@ struct PrefillDev {
     uint32_t n_heads, group_size, q_len, kv_len, query_offset, causal, block_size, block_shift, n_kv_heads, paged;
     uint32_t splits;             // > 1: the key tiles of a query tile are divided over `splits` items
     uint32_t n_qt, n_items, n_workgroups;  // query tiles; (query tile, head, split) items; workgroups that share them out
+    uint32_t pool_bytes32;       // paged: size of each pool when below 4 GiB (whole pages then go by a 32-bit offset), else 0
     float *part_acc, *part_ml;   // [head][query tile][split][BM][D] unnormalised sums, [..][BM][2] (max, sum)
     float scale_log2e;
     uint32_t out_aligned16;         // output base and strides are multiples of 16 bytes: rows leave as whole 16-byte pieces
@@ -534,6 +535,8 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     uint32_t q_tile = 0, head = 0, split = 0, kvh = 0, q0 = 0, kv_end = 0;
     int t0 = 0, ntg = 0, iters = 0;
     rsrc_words krs = make_rsrc_words(nullptr, 0), vrs = krs;
+    if (PAGED) krs = make_rsrc_words(a.k, a.pool_bytes32), vrs = make_rsrc_words(a.v, a.pool_bytes32);  // the whole pools
+    const uint32_t page_bytes = a.n_kv_heads * a.block_size * (uint32_t)ROWB;  // of one page, all heads
     auto enter_item = [&](uint32_t item) {
         const uint32_t qi = item / (a.n_heads * S), rest = item - qi * (a.n_heads * S);
         q_tile = n_qt - 1 - qi, head = rest / S, split = rest - head * S;
@@ -578,12 +581,17 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         rsrc_words rs = is_k ? krs : vrs;
         int so = (int)(key * (uint32_t)ROWB);
         if (PAGED) {
-            const uint32_t valid = key < kv_end ? min(16u, kv_end - key) : 0u;
             const uint32_t rip = bs_shift < 32 ? key & (a.block_size - 1) : key % a.block_size;
-            const size_t base = (((size_t)page * a.n_kv_heads + kvh) * a.block_size + rip) * (size_t)ROWB;
-            const unsigned char *pool = reinterpret_cast<const unsigned char *>(is_k ? a.k : a.v);
-            rs = make_rsrc_words(pool + base, valid * ROWB);
-            so = 0;
+            if (a.pool_bytes32 != 0 && key + 16 <= kv_end) {
+                // all 16 rows exist: the pool's descriptor and a 32-bit offset to the rows
+                so = (int)((uint32_t)page * page_bytes + (kvh * a.block_size + rip) * (uint32_t)ROWB);
+            } else {  // a descriptor that ends with the last visible row (rows past it come out as zeros)
+                const uint32_t valid = key < kv_end ? min(16u, kv_end - key) : 0u;
+                const size_t base = (((size_t)page * a.n_kv_heads + kvh) * a.block_size + rip) * (size_t)ROWB;
+                const unsigned char *pool = reinterpret_cast<const unsigned char *>(is_k ? a.k : a.v);
+                rs = make_rsrc_words(pool + base, valid * ROWB);
+                so = 0;
+            }
         }
         if (is_k) {
             // chunk quads: 64 bytes apart in a row, 1 KB apart in LDS
@@ -1027,6 +1035,7 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
     a.n_heads = L.n_heads, a.group_size = L.group_size, a.q_len = L.q_len, a.kv_len = L.kv_len;
     a.query_offset = L.query_offset, a.causal = L.causal ? 1u : 0u, a.block_size = L.block_size;
     a.n_kv_heads = L.n_kv_heads, a.paged = L.paged ? 1u : 0u;
+    a.pool_bytes32 = (L.paged && L.pool_bytes > 0 && L.pool_bytes < (1ull << 32)) ? (uint32_t)L.pool_bytes : 0u;
     a.block_shift = 32;
     if (L.paged && L.block_size && (L.block_size & (L.block_size - 1)) == 0) a.block_shift = (uint32_t)__builtin_ctz(L.block_size);
     if (!L.paged && (uint64_t)L.kv_len * L.head_dim * 2 >= (1ull << 32))

@@ -105,6 +105,7 @@ PROTOTYPES = {
     "fa_profile_reset": [_vp],
     "fa_profile_query": [_vp, C.c_char_p, C.POINTER(C.c_uint64), C.POINTER(C.c_double)],
     "fa_profile_clock_buffer": [_vp, _vp, _u32],
+    "fa_compute_units": [_vp, C.POINTER(_u32)],
     "fa_device_alloc": [_vp, _sz, C.POINTER(_vp)],
     "fa_device_free": [_vp, _vp],
     "fa_upload": [_vp, _vp, _sz, _vp, _sz],
@@ -456,6 +457,11 @@ class Foundry:
 
     def profile_clock_buffer(self, buf, n_workgroups):
         check(self.lib.fa_profile_clock_buffer(self.h, None if buf is None else buf.ptr, n_workgroups))
+
+    def n_cus(self):
+        n = C.c_uint32()
+        check(self.lib.fa_compute_units(self.h, C.byref(n)))
+        return n.value
 
     def measure_clock(self, matrix_load, iterations):
         """(shader MHz, milliseconds the waves ran) under back-to-back MFMAs (matrix_load) or dependent FMAs."""
