@@ -519,4 +519,122 @@ inline void CompiledMatMulStep::execute(Foundry &foundry, const FastBindings &fa
     check(fa_matmul(foundry.ctx(), a.c(), b.c(), b_scales.c(), output.c(), bias.c(), c.c(), &p));
 }
 
+// ---------------------------------------------------------------------------------------------- SdpaReference
+// src/metals/sdpa/step.rs:94-156: the same fields as FlashAttentionStep; runs on the flash kernels (fa_sdpa_reference).
+struct SdpaReferenceStep;
+struct CompiledSdpaReferenceStep : CompiledStep {
+    const SdpaReferenceStep *step;
+    size_t q_idx, k_idx, v_idx, output_idx;
+    void execute(Foundry &foundry, const FastBindings &fast, const TensorBindings &bindings, const SymbolTable &) const override;
+    const char *name() const override { return "SdpaReference"; }
+};
+
+struct SdpaReferenceStep {
+    Ref q, k, v, output;
+    bool causal = false;
+    DynamicU32 query_offset, n_heads, head_dim, kv_seq_len, m;
+    bool kv_head_major = false;
+    std::vector<std::unique_ptr<CompiledStep>> compile(TensorBindings &b, SymbolTable &s) const {
+        auto c = std::make_unique<CompiledSdpaReferenceStep>();
+        c->step = this;
+        c->q_idx = s.get_or_create(b.interpolate(q)), c->k_idx = s.get_or_create(b.interpolate(k));
+        c->v_idx = s.get_or_create(b.interpolate(v)), c->output_idx = s.get_or_create(b.interpolate(output));
+        std::vector<std::unique_ptr<CompiledStep>> out;
+        out.push_back(std::move(c));
+        return out;
+    }
+    void execute(Foundry &foundry, TensorBindings &bindings) const { execute_step(*this, foundry, bindings); }
+    const char *name() const { return "SdpaReference"; }
+};
+
+inline void CompiledSdpaReferenceStep::execute(Foundry &foundry, const FastBindings &fast, const TensorBindings &bindings,
+                                               const SymbolTable &) const {
+    const TensorArg q = TensorArg::from_tensor(need(fast, q_idx, "q")), k = TensorArg::from_tensor(need(fast, k_idx, "k"));
+    const TensorArg v = TensorArg::from_tensor(need(fast, v_idx, "v")), out = TensorArg::from_tensor(need(fast, output_idx, "output"));
+    const SdpaReferenceStep &s = *step;
+    uint32_t m = s.m.resolve(bindings);
+    if (m == 0) m = 1;  // serde default, src/metals/sdpa/step.rs:179-180
+    check(fa_sdpa_reference(foundry.ctx(), q.c(), k.c(), v.c(), out.c(), s.causal ? 1 : 0, s.query_offset.resolve(bindings),
+                            s.n_heads.resolve(bindings), s.head_dim.resolve(bindings), s.kv_seq_len.resolve(bindings), m,
+                            s.kv_head_major ? 1 : 0));
+}
+
+// ---------------------------------------------------------------------------------------------- the un-fused chain
+// The kernel structs of the older DSL ops: tensors as TensorArg, parameters with DynamicValue fields resolved against
+// the bindings, run with `kernel.run(foundry)` (the reference's `foundry.run(&kernel)`).
+struct RopeParams {  // src/metals/rope/mod.rs:13-22
+    uint32_t dim = 0;
+    DynamicU32 seq_len, position_offset, total_elements;
+    fa_rope_params resolve(const TensorBindings &b) const { return {dim, seq_len.resolve(b), position_offset.resolve(b), total_elements.resolve(b)}; }
+};
+struct Rope {  // src/metals/rope/mod.rs:36-48
+    TensorArg input, output, cos, sin;
+    fa_rope_params params;
+    void run(Foundry &f) const { check(fa_rope(f.ctx(), input.c(), output.c(), cos.c(), sin.c(), &params)); }
+};
+struct KvCacheWriteParams {  // src/metals/kv_cache_write/mod.rs:63-78
+    uint32_t n_kv_heads = 0, head_dim = 0;
+    DynamicU32 input_seq_len, position_offset, max_seq_len, total_elements, layer_idx;
+    fa_kv_cache_write_params resolve(const TensorBindings &b) const {
+        return {n_kv_heads, head_dim, input_seq_len.resolve(b), position_offset.resolve(b), max_seq_len.resolve(b),
+                total_elements.resolve(b), layer_idx.resolve(b)};
+    }
+};
+struct KvCacheWrite {  // src/metals/kv_cache_write/mod.rs:92-100
+    TensorArg input, cache;
+    fa_kv_cache_write_params params;
+    void run(Foundry &f) const { check(fa_kv_cache_write(f.ctx(), input.c(), cache.c(), &params)); }
+};
+struct KvCacheWriteRepeatKvHeadsParams {  // src/metals/kv_cache_write/mod.rs:16-35
+    uint32_t n_kv_heads = 0, n_heads = 0, group_size = 0, head_dim = 0;
+    DynamicU32 input_seq_len, position_offset, max_seq_len, total_elements, layer_idx;
+    fa_kv_cache_write_repeat_params resolve(const TensorBindings &b) const {
+        return {n_kv_heads, n_heads, group_size, head_dim, input_seq_len.resolve(b), position_offset.resolve(b),
+                max_seq_len.resolve(b), total_elements.resolve(b), layer_idx.resolve(b)};
+    }
+};
+struct KvCacheWriteRepeatKvHeads {  // src/metals/kv_cache_write/mod.rs:50-58
+    TensorArg input, cache;
+    fa_kv_cache_write_repeat_params params;
+    void run(Foundry &f) const { check(fa_kv_cache_write_repeat_kv_heads(f.ctx(), input.c(), cache.c(), &params)); }
+};
+struct KvCacheReadParams {  // src/metals/kv_cache_write/read.rs:15-26
+    uint32_t n_kv_heads = 0, head_dim = 0;
+    DynamicU32 seq_len, max_seq_len, total_elements;
+    fa_kv_cache_read_params resolve(const TensorBindings &b) const {
+        return {n_kv_heads, head_dim, seq_len.resolve(b), max_seq_len.resolve(b), total_elements.resolve(b)};
+    }
+};
+struct KvCacheRead {  // src/metals/kv_cache_write/read.rs:39-47
+    TensorArg cache, output;
+    fa_kv_cache_read_params params;
+    void run(Foundry &f) const { check(fa_kv_cache_read(f.ctx(), cache.c(), output.c(), &params)); }
+};
+struct KvRearrangeParams {  // src/metals/kv_rearrange/mod.rs:13-39
+    DynamicU32 kv_dim, row_stride, kv_head_dim, n_heads, n_kv_heads, head_dim, seq, total_elements;
+    fa_kv_rearrange_params resolve(const TensorBindings &b) const {
+        return {kv_dim.resolve(b), row_stride.resolve(b), kv_head_dim.resolve(b), n_heads.resolve(b), n_kv_heads.resolve(b),
+                head_dim.resolve(b), seq.resolve(b), total_elements.resolve(b)};
+    }
+};
+struct KvRearrange {  // src/metals/kv_rearrange/mod.rs:51-59
+    TensorArg input, output;
+    fa_kv_rearrange_params params;
+    void run(Foundry &f) const { check(fa_kv_rearrange(f.ctx(), input.c(), output.c(), &params)); }
+};
+struct RepeatKvHeadsParams {  // src/metals/repeat_kv_heads/mod.rs:16-40
+    uint32_t group_size = 0, batch = 0, n_kv_heads = 0, n_heads = 0;
+    DynamicU32 seq;
+    uint32_t head_dim = 0;
+    DynamicU32 cache_stride, total_elements;
+    fa_repeat_kv_heads_params resolve(const TensorBindings &b) const {
+        return {group_size, batch, n_kv_heads, n_heads, seq.resolve(b), head_dim, cache_stride.resolve(b), total_elements.resolve(b)};
+    }
+};
+struct RepeatKvHeads {  // src/metals/repeat_kv_heads/mod.rs:53-61
+    TensorArg input, output;
+    fa_repeat_kv_heads_params params;
+    void run(Foundry &f) const { check(fa_repeat_kv_heads(f.ctx(), input.c(), output.c(), &params)); }
+};
+
 }  // namespace metallic_foundry

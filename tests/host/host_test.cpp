@@ -208,6 +208,100 @@ static void run_fused_parity(Foundry &foundry, size_t seq_len, size_t position_o
     EXPECT(std::memcmp(v_ref.data(), v_fused.data(), v_ref.size() * 2) == 0);
 }
 
+// tests/kv_prep_fused.rs:28-247 as the reference runs it: the un-fused chain (KvRearrange -> Rope -> KvCacheWrite per
+// tensor) on the device next to KvPrepFused, q_rot and both caches bit for bit; then SdpaReference next to FlashAttention
+// on the result.
+static void run_fused_against_unfused_chain(Foundry &foundry, size_t seq_len, size_t position_offset, size_t max_seq_len,
+                                            size_t n_heads, size_t n_kv_heads, size_t head_dim) {
+    const size_t d_model = n_heads * head_dim, kv_dim = n_kv_heads * head_dim;
+    Rng rng{(uint32_t)(seq_len * 977 + head_dim + position_offset)};
+    auto q = rng.fill(seq_len * d_model, 1.0f), k = rng.fill(seq_len * kv_dim, 1.0f), v = rng.fill(seq_len * kv_dim, 1.0f);
+    std::vector<orc_f16> cos(max_seq_len * head_dim / 2), sin(cos.size());
+    orc_rope_tables(10000.0f, (uint32_t)head_dim, 0, (uint32_t)max_seq_len, nullptr, cos.data(), sin.data());
+    auto prior = rng.fill(n_kv_heads * max_seq_len * head_dim, 1.0f);  // rows before position_offset: an earlier prefix
+
+    TensorBindings b;
+    b.insert("q", foundry.from_host(Dtype::F16, {seq_len, d_model}, q.data()));
+    b.insert("k", foundry.from_host(Dtype::F16, {seq_len, kv_dim}, k.data()));
+    b.insert("v", foundry.from_host(Dtype::F16, {seq_len, kv_dim}, v.data()));
+    b.insert("q_rot", foundry.zeros(Dtype::F16, {n_heads, seq_len, head_dim}));
+    b.insert("k_cache", foundry.from_host(Dtype::F16, {n_kv_heads, max_seq_len, head_dim}, prior.data()));
+    b.insert("v_cache", foundry.from_host(Dtype::F16, {n_kv_heads, max_seq_len, head_dim}, prior.data()));
+    b.insert("rope_cos", foundry.from_host(Dtype::F16, {max_seq_len, head_dim / 2}, cos.data()));
+    b.insert("rope_sin", foundry.from_host(Dtype::F16, {max_seq_len, head_dim / 2}, sin.data()));
+    b.set_int_global("m", seq_len);
+    b.set_int_global("position_offset", position_offset);
+    KvPrepFusedStep fused{"q", "k", "v", "q_rot", "k_cache", "v_cache", "rope_cos", "rope_sin", {}};
+    fused.params.d_model = (uint32_t)d_model, fused.params.kv_dim = (uint32_t)kv_dim, fused.params.head_dim = (uint32_t)head_dim;
+    fused.params.n_heads = (uint32_t)n_heads, fused.params.n_kv_heads = (uint32_t)n_kv_heads;
+    fused.params.group_size = (uint32_t)(n_heads / n_kv_heads);
+    fused.params.seq_len = DynamicU32::var("m"), fused.params.position_offset = DynamicU32::var("position_offset");
+    fused.params.max_seq_len = (uint32_t)max_seq_len, fused.params.total_elements = (uint32_t)(n_heads * seq_len * head_dim);
+    fused.execute(foundry, b);
+
+    // the chain, one tensor at a time
+    Tensor q_heads = foundry.zeros(Dtype::F16, {n_heads, seq_len, head_dim}), q_rot2 = foundry.zeros(Dtype::F16, {n_heads, seq_len, head_dim});
+    Tensor k_heads = foundry.zeros(Dtype::F16, {n_kv_heads, seq_len, head_dim}), k_rot = foundry.zeros(Dtype::F16, {n_kv_heads, seq_len, head_dim});
+    Tensor v_heads = foundry.zeros(Dtype::F16, {n_kv_heads, seq_len, head_dim});
+    Tensor k_cache2 = foundry.from_host(Dtype::F16, {n_kv_heads, max_seq_len, head_dim}, prior.data());
+    Tensor v_cache2 = foundry.from_host(Dtype::F16, {n_kv_heads, max_seq_len, head_dim}, prior.data());
+    auto arg = [](const Tensor &t) { return TensorArg::from_tensor(t); };
+    auto rearrange = [&](const char *src, const Tensor &dst, size_t dim, size_t heads) {
+        KvRearrangeParams p;
+        p.kv_dim = (uint32_t)dim, p.row_stride = (uint32_t)dim, p.kv_head_dim = (uint32_t)head_dim, p.n_heads = (uint32_t)heads;
+        p.n_kv_heads = (uint32_t)heads, p.head_dim = (uint32_t)head_dim, p.seq = DynamicU32::var("m");
+        p.total_elements = (uint32_t)(heads * seq_len * head_dim);
+        KvRearrange{arg(*b.get(src)), arg(dst), p.resolve(b)}.run(foundry);
+    };
+    auto rope = [&](const Tensor &src, const Tensor &dst, size_t heads) {
+        RopeParams p;
+        p.dim = (uint32_t)head_dim, p.seq_len = DynamicU32::var("m"), p.position_offset = DynamicU32::var("position_offset");
+        p.total_elements = (uint32_t)(heads * seq_len * head_dim);
+        Rope{arg(src), arg(dst), arg(*b.get("rope_cos")), arg(*b.get("rope_sin")), p.resolve(b)}.run(foundry);
+    };
+    auto cache_write = [&](const Tensor &src, const Tensor &cache) {
+        KvCacheWriteParams p;
+        p.n_kv_heads = (uint32_t)n_kv_heads, p.head_dim = (uint32_t)head_dim, p.input_seq_len = DynamicU32::var("m");
+        p.position_offset = DynamicU32::var("position_offset"), p.max_seq_len = (uint32_t)max_seq_len;
+        p.total_elements = (uint32_t)(n_kv_heads * seq_len * head_dim), p.layer_idx = 0;
+        KvCacheWrite{arg(src), arg(cache), p.resolve(b)}.run(foundry);
+    };
+    rearrange("q", q_heads, d_model, n_heads), rope(q_heads, q_rot2, n_heads);
+    rearrange("k", k_heads, kv_dim, n_kv_heads), rope(k_heads, k_rot, n_kv_heads), cache_write(k_rot, k_cache2);
+    rearrange("v", v_heads, kv_dim, n_kv_heads), cache_write(v_heads, v_cache2);
+    foundry.synchronize();
+    auto same = [&](const Tensor &x, const Tensor &y) {
+        auto hx = foundry.to_host<orc_f16>(x), hy = foundry.to_host<orc_f16>(y);
+        return hx.size() == hy.size() && std::memcmp(hx.data(), hy.data(), hx.size() * 2) == 0;
+    };
+    EXPECT(same(q_rot2, *b.get("q_rot")));
+    EXPECT(same(k_cache2, *b.get("k_cache")));
+    EXPECT(same(v_cache2, *b.get("v_cache")));
+
+    // attention over what is now in the cache, through both step names
+    const size_t kv_len = position_offset + seq_len;
+    b.insert("out_flash", foundry.zeros(Dtype::F16, {seq_len, d_model}));
+    b.insert("out_reference", foundry.zeros(Dtype::F16, {seq_len, d_model}));
+    b.set_int_global("kv_seq_len", kv_len);
+    FlashAttentionStep flash{"q_rot", "k_cache", "v_cache", "out_flash"};
+    flash.causal = true, flash.kv_head_major = true, flash.query_offset = DynamicU32::var("position_offset");
+    flash.n_heads = (uint32_t)n_heads, flash.head_dim = (uint32_t)head_dim, flash.kv_seq_len = DynamicU32::var("kv_seq_len");
+    flash.m = DynamicU32::var("m");
+    SdpaReferenceStep ref{"q_rot", "k_cache", "v_cache", "out_reference"};
+    ref.causal = true, ref.kv_head_major = true, ref.query_offset = DynamicU32::var("position_offset");
+    ref.n_heads = (uint32_t)n_heads, ref.head_dim = (uint32_t)head_dim, ref.kv_seq_len = DynamicU32::var("kv_seq_len");
+    ref.m = DynamicU32::var("m");
+    flash.execute(foundry, b), ref.execute(foundry, b);
+    foundry.synchronize();
+    EXPECT(same(*b.get("out_flash"), *b.get("out_reference")));
+    std::vector<orc_f16> want(seq_len * d_model);
+    auto q_host = foundry.to_host<orc_f16>(*b.get("q_rot")), k_host = foundry.to_host<orc_f16>(*b.get("k_cache")), v_host = foundry.to_host<orc_f16>(*b.get("v_cache"));
+    orc_sdpa_prefill(q_host.data(), k_host.data(), v_host.data(), want.data(), (uint32_t)n_heads, (uint32_t)(n_heads / n_kv_heads), (uint32_t)head_dim,
+                     (uint32_t)seq_len, (uint32_t)kv_len, (uint32_t)position_offset, 1, 1.0f / std::sqrt((float)head_dim), seq_len * head_dim,
+                     head_dim, max_seq_len * head_dim, head_dim, max_seq_len * head_dim, head_dim, head_dim, d_model, 32, 1);
+    EXPECT(max_abs_diff(want, foundry.to_host<orc_f16>(*b.get("out_reference")), want.size()) <= 2e-3f);
+}
+
 // tests/flashattention_decode_parity.rs: decode through the FlashAttention step at several kv lengths and seeds.
 static void run_decode_parity(Foundry &foundry, uint32_t seed, size_t n_heads, size_t n_kv_heads, size_t head_dim, size_t kv_len,
                               size_t capacity) {
@@ -512,6 +606,10 @@ int main(int argc, char **argv) {
                 });
             }
         run_test("closed-form prefill H2 N15 D64", [&] { test_closed_form_prefill(foundry); });
+        run_test("un-fused chain == KvPrepFused, SdpaReference == FlashAttention (decode row)",
+                 [&] { run_fused_against_unfused_chain(foundry, 1, 37, 64, 14, 2, 64); });
+        run_test("un-fused chain == KvPrepFused, SdpaReference == FlashAttention (chunk after a prefix)",
+                 [&] { run_fused_against_unfused_chain(foundry, 5, 20, 64, 8, 2, 128); });
         run_test("error variants", [&] { test_error_variants(foundry); });
         run_test("fused qkv step, row-major weights", [&] { test_fused_qkv_step(foundry, WeightLayout::RowMajor); });
         run_test("fused qkv step, canonical weights", [&] { test_fused_qkv_step(foundry, WeightLayout::Canonical); });
