@@ -126,6 +126,13 @@ fa_status fa_profile_query(fa_ctx *ctx, const char *kernel_prefix, uint64_t *lau
  * matrix peak scales with it). NULL switches it off. */
 fa_status fa_profile_clock_buffer(fa_ctx *ctx, void *d_buffer, uint32_t n_workgroups);
 
+/* Device-side stopwatch on the context's stream: _start records an event behind everything enqueued so far, _stop
+ * records a second one behind everything enqueued since, waits for it and returns the time between the two (what the
+ * work enqueued in between took on the device, launch gaps included). Not during a capture (graph launches in between
+ * are fine). */
+fa_status fa_stream_timer_start(fa_ctx *ctx);
+fa_status fa_stream_timer_stop(fa_ctx *ctx, float *elapsed_ms);
+
 /* Compute units of the context's device (what the launch-sizing rules count in). */
 fa_status fa_compute_units(fa_ctx *ctx, uint32_t *n);
 

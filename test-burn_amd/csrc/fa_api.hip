@@ -152,6 +152,8 @@ extern "C" fa_status fa_ctx_destroy(fa_ctx *ctx) {
         (void)hipEventDestroy(r.stop);
     }
     for (auto e : ctx->event_pool) (void)hipEventDestroy(e);
+    if (ctx->timer_start) (void)hipEventDestroy(ctx->timer_start);
+    if (ctx->timer_stop) (void)hipEventDestroy(ctx->timer_stop);
     if (ctx->workspace) (void)hipFree(ctx->workspace);
     if (ctx->counters) (void)hipFree(ctx->counters);
     if (ctx->h_status) (void)hipHostFree(ctx->h_status);
@@ -392,6 +394,30 @@ extern "C" fa_status fa_profile_clock_buffer(fa_ctx *ctx, void *d_buffer, uint32
     if (d_buffer && ((uintptr_t)d_buffer % 8) != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "the clock buffer must be 8-byte aligned");
     ctx->clock_buf = (unsigned long long *)d_buffer;
     ctx->clock_buf_workgroups = d_buffer ? n_workgroups : 0;
+    return FA_OK;
+}
+
+extern "C" fa_status fa_stream_timer_start(fa_ctx *ctx) {
+    FA_NEED(ctx, "ctx");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "fa_stream_timer_start during a capture");
+    if (!ctx->timer_start) {
+        FA_HIP(hipEventCreate(&ctx->timer_start));
+        FA_HIP(hipEventCreate(&ctx->timer_stop));
+    }
+    FA_HIP(hipEventRecord(ctx->timer_start, ctx->stream));
+    ctx->timer_running = true;
+    return FA_OK;
+}
+
+extern "C" fa_status fa_stream_timer_stop(fa_ctx *ctx, float *elapsed_ms) {
+    FA_NEED(ctx, "ctx");
+    FA_NEED(elapsed_ms, "elapsed_ms");
+    if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "fa_stream_timer_stop during a capture");
+    if (!ctx->timer_running) return fa_fail(FA_ERR_INVALID_OPERATION, "fa_stream_timer_stop without fa_stream_timer_start");
+    FA_HIP(hipEventRecord(ctx->timer_stop, ctx->stream));
+    FA_HIP(hipEventSynchronize(ctx->timer_stop));
+    FA_HIP(hipEventElapsedTime(elapsed_ms, ctx->timer_start, ctx->timer_stop));
+    ctx->timer_running = false;
     return FA_OK;
 }
 

@@ -67,6 +67,8 @@ struct fa_ctx {
     // optional: the prefill kernel leaves {shader-clock ticks, wall ticks} per workgroup here (fa_profile_clock_buffer)
     unsigned long long *clock_buf = nullptr;
     uint32_t clock_buf_workgroups = 0;
+    hipEvent_t timer_start = nullptr, timer_stop = nullptr;  // fa_stream_timer_start / _stop
+    bool timer_running = false;
     // per-kernel profiling
     bool profiling = false;
     std::vector<FaProfileRec> prof;

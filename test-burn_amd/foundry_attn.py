@@ -106,6 +106,8 @@ PROTOTYPES = {
     "fa_profile_query": [_vp, C.c_char_p, C.POINTER(C.c_uint64), C.POINTER(C.c_double)],
     "fa_profile_clock_buffer": [_vp, _vp, _u32],
     "fa_compute_units": [_vp, C.POINTER(_u32)],
+    "fa_stream_timer_start": [_vp],
+    "fa_stream_timer_stop": [_vp, C.POINTER(C.c_float)],
     "fa_device_alloc": [_vp, _sz, C.POINTER(_vp)],
     "fa_device_free": [_vp, _vp],
     "fa_upload": [_vp, _vp, _sz, _vp, _sz],
@@ -457,6 +459,14 @@ class Foundry:
 
     def profile_clock_buffer(self, buf, n_workgroups):
         check(self.lib.fa_profile_clock_buffer(self.h, None if buf is None else buf.ptr, n_workgroups))
+
+    def timer_start(self):
+        check(self.lib.fa_stream_timer_start(self.h))
+
+    def timer_stop(self):
+        ms = C.c_float()
+        check(self.lib.fa_stream_timer_stop(self.h, C.byref(ms)))
+        return ms.value
 
     def n_cus(self):
         n = C.c_uint32()
