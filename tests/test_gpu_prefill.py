@@ -87,6 +87,32 @@ def test_prefill_layouts_and_noncausal():
     assert max_abs(off, orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, 3, cap, causal=True, out_layout="head_major")) <= TOL
 
 
+@pytest.mark.parametrize("D", [64, 128])
+def test_prefill_output_view_that_is_only_8_byte_aligned(D):
+    """The output tensor starts 8 bytes into its buffer: whole-row 16-byte stores are not possible and each group writes its
+    half of every row in 8-byte pieces. Same bits as the aligned output; the bytes around the view stay untouched."""
+    announce("prefill, 8-byte aligned output view", D)
+    f = ctx()
+    rng = np.random.default_rng(17 + D)
+    H, Hkv, M = 6, 2, 333
+    q, k, v = h16(rng.normal(size=(H, M, D))), h16(rng.normal(size=(Hkv, M, D))), h16(rng.normal(size=(Hkv, M, D)))
+    dq, dk, dv = f.array(q), f.array(k), f.array(v)
+    aligned = f.zeros((M, H * D))
+    f.flash_attention(dq.arg((H, M, D)), dk.arg(), dv.arg(), aligned.arg(), True, 0, H, D, M, M)
+    pad = 4  # elements = 8 bytes
+    sentinel = np.float16(3.25)
+    shifted = f.array(np.full((M * H * D + 2 * pad,), sentinel, np.float16))
+    f.flash_attention(dq.arg((H, M, D)), dk.arg(), dv.arg(), shifted.arg((M, H * D), offset=pad * 2), True, 0, H, D, M, M)
+    f.synchronize()
+    got = shifted.download()
+    assert np.all(got[:pad] == sentinel) and np.all(got[-pad:] == sentinel)
+    assert np.array_equal(bits(got[pad:-pad].reshape(M, H * D)), bits(aligned.download()))
+    want = orc.sdpa_prefill(q, k, v, H, Hkv, D, M, M, 0, M, causal=True)
+    assert max_abs(got[pad:-pad].reshape(M, H * D), want) <= TOL
+    for b in (dq, dk, dv, aligned, shifted):
+        b.free()
+
+
 def test_prefill_known_answer_fixture_noncausal():
     announce("prefill fixture")
     g = np.load(os.path.join(GOLD, "known_answer_sdpa.npz"))
