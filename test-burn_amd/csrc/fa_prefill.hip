@@ -978,463 +978,6 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     }
 }
 
-// 64 query rows per wave (variant 3). Same tiling of an item (128 query rows of one head, the key tiles split between two
-// groups), same memory -> LDS road, same resident workgroups as the kernel above, but a workgroup has FOUR waves, one per
-// SIMD, and each owns 64 rows: every K and V operand read from LDS feeds two MFMAs instead of one (half the LDS bytes and
-// operand reads per FLOP), and a wave has the SIMD's whole register file (~380 registers: 128 + 64 + 64 accumulators
-// of O^T, S^T_j, S^T_{j+1}, 64 of Q^T). With no second wave on the SIMD the softmax cannot hide behind another wave's
-// MFMAs; it is interleaved into the wave's own MFMA stream instead:
-//   (C)  S_{j+1} = K_{j+1} Q^T   (32 MFMAs)  between them: P_j = 2^(c S_j - m), row sums      (2 elements per MFMA)
-//   (D)  O^T += V_j^T P_j        (32 MFMAs)  between them: mask and row maxima of S_{j+1}
-// one workgroup barrier per tile; K_{j+2} and V_{j+1} are requested right after it.
-template <bool BF16, bool PAGED>
-__global__ void __launch_bounds__(256, 1) __attribute__((amdgpu_waves_per_eu(1, 1))) flash_prefill_w64_kernel(PrefillDev a) {
-    constexpr int D = 128, DSTEPS = D / 16, DBLKS = D / 32, ROWB = D * 2, CHK = D / 8, HB = DBLKS / 2;
-    constexpr int K_TILE = BN * ROWB, V_TILE = BN * ROWB, GRP_LDS = 2 * K_TILE + 2 * V_TILE;
-    constexpr int RB_BYTES = CHK * 256;  // one 16-row block of a K tile
-    constexpr int RG_BYTES = 4 * ROWB;   // one 4-row group of a V tile
-    constexpr int K_DMA = CHK / 4, V_DMA = 16 * ROWB / 1024;  // instructions per 16 rows of a tile
-    constexpr int AHEAD = 6;             // operand reads in flight ahead of their MFMA
-    constexpr int Q_STAGE = BM * ROWB;
-    typedef __attribute__((address_space(3))) void *lds_ptr;
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[2 * GRP_LDS + Q_STAGE];  // [group]{K[2], V[2]}, Q
-
-    const unsigned long long clk0 = a.clock_out ? __builtin_readcyclecounter() : 0ull, wall0 = a.clock_out ? wall_clock64() : 0ull;
-    const int lane = threadIdx.x & 63;
-    const int wave4 = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int grp = wave4 >> 1, w2 = wave4 & 1;  // group; which 64 rows of the item
-    unsigned char *k_base = lds + grp * GRP_LDS, *v_base = k_base + 2 * K_TILE;
-    const uint32_t k_lds_addr = (uint32_t)(uintptr_t)(lds_ptr)lds + grp * GRP_LDS, v_lds_addr = k_lds_addr + 2 * K_TILE;
-    const uint32_t q_lds_addr = (uint32_t)(uintptr_t)(lds_ptr)lds + 2 * GRP_LDS;
-    const int n = lane & 31, hi = lane >> 5;
-    const uint32_t S = a.splits, n_qt = a.n_qt, n_items = a.n_items, n_wgs = a.n_workgroups;
-
-    auto item_of = [&](uint32_t r) -> uint32_t { return r * n_wgs + ((r & 1) ? n_wgs - 1 - blockIdx.x : blockIdx.x); };
-    uint32_t q_tile = 0, head = 0, split = 0, kvh = 0, q0 = 0, kv_end = 0;
-    int t0 = 0, ntg = 0, iters = 0;
-    rsrc_words krs = make_rsrc_words(nullptr, 0), vrs = krs;
-    if (PAGED) krs = make_rsrc_words(a.k, a.pool_bytes32), vrs = make_rsrc_words(a.v, a.pool_bytes32);
-    const uint32_t page_bytes = a.n_kv_heads * a.block_size * (uint32_t)ROWB;
-    auto enter_item = [&](uint32_t item) {
-        const uint32_t qi = item / (a.n_heads * S), rest = item - qi * (a.n_heads * S);
-        q_tile = n_qt - 1 - qi, head = rest / S, split = rest - head * S;
-        kvh = head / a.group_size;
-        q0 = q_tile * BM;
-        kv_end = a.kv_len;
-        if (a.causal) {
-            const uint64_t last = (uint64_t)min(q0 + BM - 1, a.q_len - 1) + a.query_offset + 1;
-            kv_end = (uint32_t)min((uint64_t)a.kv_len, last);
-        }
-        const int all_tiles = (int)((kv_end + BN - 1) / BN);
-        const int per_split = (all_tiles + (int)S - 1) / (int)S;
-        const int t_lo = min(all_tiles, (int)split * per_split);
-        const int n_tiles = min(all_tiles, t_lo + per_split);
-        t0 = t_lo + grp;
-        ntg = t0 < n_tiles ? (n_tiles - t0 + 1) / 2 : 0;
-        iters = (n_tiles - t_lo + 1) / 2;
-        if (!PAGED) {
-            krs = make_rsrc_words(a.k + (size_t)kvh * a.k_stride_h, kv_end * (uint32_t)ROWB);
-            vrs = make_rsrc_words(a.v + (size_t)kvh * a.v_stride_h, kv_end * (uint32_t)ROWB);
-        }
-    };
-
-    constexpr int CBR = ROWB / 64;
-    const int k_lane_src = (lane & 15) * ROWB + (lane >> 4) * 16;
-    const int v_lane_src = ((lane / (16 * CBR)) * 4 + ((lane & 15) >> 2)) * ROWB + ((lane >> 4) % CBR) * 64 + (lane & 3) * 16;
-    typedef const int32_t __attribute__((address_space(4))) *const_i32p;
-    const const_i32p bt = (const_i32p)a.block_table;
-    const uint32_t bs_shift = a.block_shift;
-    // 16-row block `blk` (0..3) of group-local tile i of one tensor into LDS buffer `buf`; a wave moves blocks 2 w2, 2 w2 + 1
-    auto dma16 = [&](bool is_k, int i, int buf, int blk) {
-        const uint32_t key = (uint32_t)(t0 + 2 * i) * BN + 16 * blk;
-        rsrc_words rs = is_k ? krs : vrs;
-        int so = (int)(key * (uint32_t)ROWB);
-        if (PAGED) {
-            const int32_t page = key < kv_end ? bt[bs_shift < 32 ? key >> bs_shift : key / a.block_size] : 0;
-            const uint32_t rip = bs_shift < 32 ? key & (a.block_size - 1) : key % a.block_size;
-            if (a.pool_bytes32 != 0 && key + 16 <= kv_end) {
-                so = (int)((uint32_t)page * page_bytes + (kvh * a.block_size + rip) * (uint32_t)ROWB);
-            } else {
-                const uint32_t valid = key < kv_end ? min(16u, kv_end - key) : 0u;
-                const size_t base = (((size_t)page * a.n_kv_heads + kvh) * a.block_size + rip) * (size_t)ROWB;
-                const unsigned char *pool = reinterpret_cast<const unsigned char *>(is_k ? a.k : a.v);
-                rs = make_rsrc_words(pool + base, valid * ROWB);
-                so = 0;
-            }
-        }
-        if (is_k) buffer_to_lds_b128<K_DMA, 64, 1024>(rs, k_lds_addr + buf * K_TILE + blk * RB_BYTES, k_lane_src, so);
-        else buffer_to_lds_b128<V_DMA, 1024, 1024>(rs, v_lds_addr + buf * V_TILE + blk * (4 * RG_BYTES), v_lane_src, so);
-    };
-    auto dma = [&](bool is_k, int i, int buf) {
-        dma16(is_k, i, buf, 2 * w2);
-        dma16(is_k, i, buf, 2 * w2 + 1);
-    };
-    constexpr int TILE_DMA = 2 * K_DMA;  // instructions per wave per tile (K_DMA == V_DMA)
-    const size_t q_bytes = ((size_t)(a.q_len - 1) * a.q_stride_m + D) * 2;
-    auto q_dma = [&](uint32_t item) {
-        int ql = lane;
-        asm volatile("" : "+v"(ql));
-        const int q_lane_src = (ql & 15) * (int)(a.q_stride_m * 2) + (ql >> 4) * 16;
-        const uint32_t qi = item / (a.n_heads * S), hd = (item - qi * (a.n_heads * S)) / S;
-        const rsrc_words qrs = make_rsrc_words(a.q + (size_t)hd * a.q_stride_h, (uint32_t)q_bytes);
-#pragma unroll
-        for (int h2 = 0; h2 < 2; ++h2) {
-            const int blk = 2 * wave4 + h2;
-            const uint32_t row0 = (n_qt - 1 - qi) * BM + 16 * blk;
-            buffer_to_lds_b128<K_DMA, 64, 1024>(qrs, q_lds_addr + blk * RB_BYTES, q_lane_src, (int)(row0 * (uint32_t)(a.q_stride_m * 2)));
-        }
-    };
-
-    U4H8 qreg[2][DSTEPS];
-    f16_t oacc[2][DBLKS];
-    float l_run[2], m_run[2];
-    auto clear_state = [&]() {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb) {
-#pragma unroll
-            for (int b = 0; b < DBLKS; ++b)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) oacc[rb][b][i] = 0.0f;
-            l_run[rb] = 0.0f, m_run[rb] = -1e30f;
-        }
-    };
-    const float c = a.scale_log2e;
-    const int k_lane = (n >> 4) * RB_BYTES + hi * 256 + (n & 15) * 16;
-    const int v_lane = hi * RG_BYTES + ((lane & 15) >> 2) * 64 + ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
-    h8_t pb[2][2][2];  // [row block][key block][k-step]
-    uint32_t q_abs[2], wave_min_limit = 0;
-
-    auto mfma = [&](const U4H8 &x, const U4H8 &y, f16_t acc) -> f16_t {
-        return BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(x.b, y.b, acc, 0, 0, 0) : __builtin_amdgcn_mfma_f32_32x32x16_f16(x.h, y.h, acc, 0, 0, 0);
-    };
-    // S = K_buf Q^T into s (both row blocks), optionally with a piece of other work after every MFMA
-    auto s_tile = [&](int buf, f16_t (&s)[2][2], auto &&between) {
-        const unsigned char *k_lds = k_base + buf * K_TILE + k_lane;
-        constexpr int NK = 2 * DSTEPS;
-        U4H8 kop[NK];
-#pragma unroll
-        for (int t = 0; t < AHEAD; ++t) kop[t].u = *reinterpret_cast<const uint4 *>(k_lds + (t / DSTEPS) * (2 * RB_BYTES) + (t % DSTEPS) * 512);
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) s[rb][kb][i] = 0.0f;
-#pragma unroll
-        for (int t = 0; t < NK; ++t) {
-            if (t + AHEAD < NK) {
-                const int u = t + AHEAD;
-                kop[u].u = *reinterpret_cast<const uint4 *>(k_lds + (u / DSTEPS) * (2 * RB_BYTES) + (u % DSTEPS) * 512);
-            }
-            const int kb = t / DSTEPS, st = t % DSTEPS;
-#pragma unroll
-            for (int rb = 0; rb < 2; ++rb) {
-                s[rb][kb] = mfma(kop[t], qreg[rb][st], s[rb][kb]);
-                between(2 * t + rb);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    };
-    // O^T += V_buf^T P (both row blocks)
-    auto pv_tile = [&](int buf, auto &&between) {
-        const unsigned char *v_lds = v_base + buf * V_TILE + v_lane;
-        constexpr int NV = 4 * DBLKS;  // (key block, k-step, d block)
-        union VOp {
-            fp16x4_t f[2];
-            h8_t h;
-            U4H8 u;
-        };
-        VOp vop[NV];
-        auto read_v = [&](int p) {
-            const int g = p / DBLKS, b = p % DBLKS, kb = g / 2, ks = g % 2;
-            const unsigned char *p0 = v_lds + (kb * 8 + ks * 4) * RG_BYTES + b * 256;
-            vop[p].f[0] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p0));
-            vop[p].f[1] = __builtin_amdgcn_ds_read_tr16_b64_v4f16((fp16x4_t __attribute__((address_space(3))) *)(p0 + 2 * RG_BYTES));
-        };
-#pragma unroll
-        for (int p = 0; p < AHEAD; ++p) read_v(p);
-#pragma unroll
-        for (int p = 0; p < NV; ++p) {
-            if (p + AHEAD < NV) read_v(p + AHEAD);
-            const int g = p / DBLKS, b = p % DBLKS, kb = g / 2, ks = g % 2;
-#pragma unroll
-            for (int rb = 0; rb < 2; ++rb) {
-                U4H8 pp;
-                pp.h = pb[rb][kb][ks];
-                oacc[rb][b] = mfma(vop[p].u, pp, oacc[rb][b]);
-                between(2 * p + rb);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    };
-    auto nothing = [](int) {};
-
-    // ---- end of an item: exchange of halves between the groups and the rows out (see the kernel above)
-    auto write_item = [&](uint32_t o_item, auto G) {
-        constexpr int g = decltype(G)::value;
-        int lo = lane;
-        asm volatile("" : "+v"(lo));
-        const int n = lo & 31, hi = lo >> 5, lane = lo;
-        const uint32_t o_qi = o_item / (a.n_heads * S), o_rest = o_item - o_qi * (a.n_heads * S);
-        const uint32_t o_head = o_rest / S, o_q0 = (n_qt - 1 - o_qi) * BM;
-        typedef unsigned int u2v __attribute__((ext_vector_type(2)));
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb) {
-            const float o_m = m_run[rb];
-            const u2v lsw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run[rb]), __float_as_uint(l_run[rb]), false, false);
-            const float o_l = __uint_as_float(lsw.x) + __uint_as_float(lsw.y);
-            const uint32_t row_in_tile = w2 * 64 + rb * 32 + n;
-            const uint32_t q_row = o_q0 + row_in_tile;
-            if (S > 1) {
-                if (q_row < a.q_len) {
-                    const size_t prow = (size_t)((o_head * n_qt + (n_qt - 1 - o_qi)) * S + (o_rest - o_head * S)) * BM + row_in_tile;
-                    float *pa = a.part_acc + prow * D;
-#pragma unroll
-                    for (int b = g * HB; b < (g + 1) * HB; ++b)
-#pragma unroll
-                        for (int gi = 0; gi < 4; ++gi) {
-                            float4 v = make_float4(oacc[rb][b][gi * 4], oacc[rb][b][gi * 4 + 1], oacc[rb][b][gi * 4 + 2], oacc[rb][b][gi * 4 + 3]);
-                            *reinterpret_cast<float4 *>(pa + b * 32 + gi * 8 + hi * 4) = v;
-                        }
-                    if (g == 0 && hi == 0) a.part_ml[prow * 2] = o_m, a.part_ml[prow * 2 + 1] = o_l;
-                }
-                continue;
-            }
-            const float inv_l = (isfinite(o_l) && fabsf(o_l) > 1e-6f) ? (1.0f / o_l) : 0.0f;
-            if (a.out_aligned16) {
-                constexpr int HROW = ROWB / 2, CPR = HROW / 16, RPI = 64 / CPR;
-                unsigned char *ot = v_base + V_TILE + (2 * w2 + rb) * (16 * ROWB);  // 4 KB of this wave's part of the second V buffer
-                int w_off = n * HROW + (n & (CPR - 1)) * 16 + hi * 8;
-                int r_off = (lane / CPR) * HROW + (((lane % CPR) ^ ((lane / CPR) & (CPR - 1))) * 16);
-                asm volatile("" : "+v"(w_off), "+v"(r_off));
-#pragma unroll
-                for (int bb = 0; bb < HB; ++bb)
-#pragma unroll
-                    for (int gi = 0; gi < 4; ++gi) {
-                        h4_t o;
-#pragma unroll
-                        for (int jj = 0; jj < 4; ++jj) o[jj] = to_elem<BF16>(oacc[rb][g * HB + bb][gi * 4 + jj] * inv_l);
-                        *reinterpret_cast<h4_t *>(ot + (w_off ^ ((bb * 4 + gi) * 16))) = o;
-                    }
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
-                __builtin_amdgcn_wave_barrier();
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-                __half *ob = a.out + (size_t)o_head * a.out_stride_h + g * (D / 2) + (lane % CPR) * 8;
-#pragma unroll
-                for (int it = 0; it < 32 / RPI; ++it) {
-                    const int row = it * RPI + lane / CPR;
-                    const uint32_t qr = o_q0 + w2 * 64 + rb * 32 + row;
-                    const uint4 val = *reinterpret_cast<const uint4 *>(ot + (r_off ^ (it * RPI * HROW + ((it * RPI) & (CPR - 1)) * 16)));
-                    if (qr < a.q_len) __builtin_nontemporal_store(__builtin_bit_cast(u4_t, val), reinterpret_cast<u4_t *>(ob + (size_t)qr * a.out_stride_m));
-                }
-                continue;
-            }
-            if (q_row < a.q_len) {
-                __half *op = a.out + (size_t)o_head * a.out_stride_h + (size_t)q_row * a.out_stride_m;
-#pragma unroll
-                for (int b = g * HB; b < (g + 1) * HB; ++b)
-#pragma unroll
-                    for (int gi = 0; gi < 4; ++gi) {
-                        h4_t o;
-#pragma unroll
-                        for (int jj = 0; jj < 4; ++jj) o[jj] = to_elem<BF16>(oacc[rb][b][gi * 4 + jj] * inv_l);
-                        *reinterpret_cast<h4_t *>(op + b * 32 + gi * 8 + hi * 4) = o;
-                    }
-            }
-        }
-    };
-    // [value][row block][wave of the group][lane]: 2 + HB * 16 values of 256 floats
-    auto park = [&](auto G) {
-        constexpr int g = decltype(G)::value;
-        int lo = lane;
-        asm volatile("" : "+v"(lo));
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb) {
-            float *mx = reinterpret_cast<float *>(lds + g * GRP_LDS) + rb * 128 + w2 * 64 + lo;
-            mx[0] = m_run[rb];
-            mx[256] = l_run[rb];
-#pragma unroll
-            for (int bb = 0; bb < HB; ++bb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) mx[(2 + bb * 16 + i) * 256] = oacc[rb][(1 - g) * HB + bb][i];
-        }
-    };
-    auto fold = [&](auto G) {
-        constexpr int g = decltype(G)::value;
-        int lo = lane;
-        asm volatile("" : "+v"(lo));
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb) {
-            const float *mx = reinterpret_cast<const float *>(lds + (1 - g) * GRP_LDS) + rb * 128 + w2 * 64 + lo;
-            const float m1 = mx[0], l1 = mx[256];
-            const float m = fmaxf(m_run[rb], m1);
-            const float e0 = fast_exp2(m_run[rb] - m), e1 = fast_exp2(m1 - m);
-            l_run[rb] = l_run[rb] * e0 + l1 * e1;
-#pragma unroll
-            for (int bb = 0; bb < HB; ++bb)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) oacc[rb][g * HB + bb][i] = oacc[rb][g * HB + bb][i] * e0 + mx[(2 + bb * 16 + i) * 256] * e1;
-            m_run[rb] = m;
-        }
-    };
-
-    // softmax, first part, of S tile `tile` of the group (group-local index) held in s: mask, row maxima -> mloc
-    float mloc[2];
-    auto mask_tile = [&](f16_t (&s)[2][2], int jt) {
-        const uint32_t key0 = (uint32_t)(t0 + 2 * jt) * BN;
-        const bool need_mask = (key0 + BN - 1 > wave_min_limit) || (key0 + BN > kv_end);
-        if (need_mask) {
-#pragma unroll
-            for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const uint32_t key = key0 + kb * 32 + (i / 4) * 8 + hi * 4 + (i % 4);
-                        const bool vis = key < kv_end && (!a.causal || key <= q_abs[rb]);
-                        s[rb][kb][i] = vis ? s[rb][kb][i] : -INFINITY;
-                    }
-        }
-    };
-    auto max_piece = [&](f16_t (&s)[2][2], float (&part)[2][4], int piece) {  // piece 0..15: four elements each
-        const int rb = piece / 8, kb = (piece % 8) / 4, i0 = (piece % 4) * 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) part[rb][i] = fmaxf(part[rb][i], s[rb][kb][i0 + i]);
-    };
-    auto finish_max = [&](float (&part)[2][4]) {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-            mloc[rb] = max_with_other_half(fmaxf(fmaxf(part[rb][0], part[rb][1]), fmaxf(part[rb][2], part[rb][3]))) * c;
-    };
-    // lazy rescale: only when a row maximum has grown by more than 2^8
-    auto rescale = [&]() {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-            if (__any(mloc[rb] > m_run[rb] + 8.0f)) {
-                const float m_new = fmaxf(m_run[rb], mloc[rb]);
-                const float alpha = fast_exp2(m_run[rb] - m_new);
-                l_run[rb] *= alpha;
-                m_run[rb] = m_new;
-#pragma unroll
-                for (int b = 0; b < DBLKS; ++b)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) oacc[rb][b][i] *= alpha;
-            }
-    };
-    // second part: two elements of P = 2^(c S - m) and their share of the row sum
-    float psum[2][2];
-    auto exp_piece = [&](f16_t (&s)[2][2], int piece) {  // piece 0..31
-        const int rb = piece / 16, kb = (piece % 16) / 8, i0 = (piece % 8) * 2;
-        const float e0 = fast_exp2(fmaf(s[rb][kb][i0], c, -m_run[rb])), e1 = fast_exp2(fmaf(s[rb][kb][i0 + 1], c, -m_run[rb]));
-        psum[rb][0] += e0, psum[rb][1] += e1;
-        pb[rb][kb][i0 / 8][i0 % 8] = to_elem<BF16>(e0);
-        pb[rb][kb][i0 / 8][i0 % 8 + 1] = to_elem<BF16>(e1);
-    };
-
-    constexpr int VMCNT_V = 0x0F70 | TILE_DMA;
-    uint32_t round = 0, item = blockIdx.x;
-    auto first_tiles = [&]() {
-        if (ntg > 0) {
-            dma(true, 0, 0);
-            if (ntg > 1) dma(true, 1, 1);
-            dma(false, 0, 0);
-        }
-    };
-    enter_item(item);
-    q_dma(item);
-    first_tiles();
-    f16_t sA[2][2], sB[2][2];
-    while (true) {
-        const uint32_t next_item = item_of(round + 1);
-        const bool has_next = next_item < n_items;
-        if (ntg > 0) __builtin_amdgcn_s_waitcnt(VMCNT_V);  // Q, K_0, K_1 are there; V_0 has until the first tile's second half
-        else __builtin_amdgcn_s_waitcnt(0x0F70);
-        __syncthreads();
-        {
-            int lo = lane;
-            asm volatile("" : "+v"(lo));
-#pragma unroll
-            for (int rb = 0; rb < 2; ++rb) {
-                const int blk = 4 * w2 + 2 * rb + ((lo & 31) >> 4);
-                const unsigned char *qp = lds + 2 * GRP_LDS + blk * RB_BYTES + (lo >> 5) * 256 + (lo & 15) * 16;
-#pragma unroll
-                for (int s = 0; s < DSTEPS; ++s) qreg[rb][s].u = *reinterpret_cast<const uint4 *>(qp + s * 512);
-            }
-        }
-        clear_state();
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb) q_abs[rb] = min(q0 + w2 * 64 + rb * 32 + n, a.q_len - 1) + a.query_offset;
-        wave_min_limit = a.causal ? (min(q0 + w2 * 64, a.q_len - 1) + a.query_offset) : 0xffffffffu;
-        // S_0 and its maxima, nothing to hide behind yet
-        if (ntg > 0) {
-            s_tile(0, sA, nothing);
-            mask_tile(sA, 0);
-            float part[2][4];
-#pragma unroll
-            for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) part[rb][i] = -INFINITY;
-#pragma unroll
-            for (int pc = 0; pc < 16; ++pc) max_piece(sA, part, pc);
-            finish_max(part);
-            rescale();
-        }
-        // one iteration: scur holds S_j (maxima taken, m_run covers it), snext receives S_{j+1}
-        auto iteration = [&](int j, f16_t (&scur)[2][2], f16_t (&snext)[2][2]) {
-            __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): K_{j+1} and V_j, requested one iteration ago, have landed
-            __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_barrier();        // ... in every wave; and every wave is done with K_j and V_{j-1}
-            __builtin_amdgcn_sched_barrier(0);
-            if (j + 2 < ntg) dma(true, j + 2, j & 1);
-            if (j + 1 < ntg) dma(false, j + 1, (j + 1) & 1);
-            if (j == 0 && has_next) q_dma(next_item);  // every wave has taken its query rows out of LDS
-            if (j < ntg) {
-                psum[0][0] = psum[0][1] = psum[1][0] = psum[1][1] = 0.0f;
-                s_tile((j + 1) & 1, snext, [&](int i) { if (i < 32) exp_piece(scur, i); });  // (C)
-                l_run[0] += psum[0][0] + psum[0][1], l_run[1] += psum[1][0] + psum[1][1];
-                mask_tile(snext, j + 1);
-                float part[2][4];
-#pragma unroll
-                for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) part[rb][i] = -INFINITY;
-                pv_tile(j & 1, [&](int i) { if (i >= 8 && i < 24) max_piece(snext, part, i - 8); });      // (D)
-                if (j + 1 < ntg) {
-                    finish_max(part);
-                    rescale();
-                }
-            }
-        };
-        for (int j = 0; j < iters; j += 2) {
-            iteration(j, sA, sB);
-            if (j + 1 < iters) iteration(j + 1, sB, sA);
-        }
-        const bool q_staged = has_next && iters > 0;
-
-        __syncthreads();  // the other wave of the group may still be reading the V tile the parked state overwrites
-        if (grp == 0) park(std::integral_constant<int, 0>());
-        else park(std::integral_constant<int, 1>());
-        __syncthreads();
-        if (grp == 0) fold(std::integral_constant<int, 0>());
-        else fold(std::integral_constant<int, 1>());
-        __syncthreads();
-        const uint32_t o_item = item;
-        if (has_next) {
-            item = next_item, ++round;
-            enter_item(item);
-            if (!q_staged) q_dma(item);
-            first_tiles();
-        }
-        if (grp == 0) write_item(o_item, std::integral_constant<int, 0>());
-        else write_item(o_item, std::integral_constant<int, 1>());
-        if (!has_next) break;
-    }
-    if (a.clock_out && threadIdx.x == 0) {
-        a.clock_out[(size_t)blockIdx.x * 2] = __builtin_readcyclecounter() - clk0;
-        a.clock_out[(size_t)blockIdx.x * 2 + 1] = wall_clock64() - wall0;
-    }
-}
-
 // Merge of the per-split states (flash_prefill.metal:843-888): m* = max m_s, L = sum l_s 2^(m_s - m*) over the
 // splits with l_s > 0, out = sum acc_s 2^(m_s - m*) / L (0 when L is unusable). m is kept in the exp2 domain.
 template <int D, bool BF16>
@@ -1533,12 +1076,8 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
     dim3 grid(a.n_workgroups, 1, 1);
     if (ctx->clock_buf && grid.x <= ctx->clock_buf_workgroups) a.clock_out = ctx->clock_buf;
     {
-        FaLaunchScope scope(ctx, !lds_direct ? "flash_prefill_mfma_kernel" : (ctx->prefill_variant == 3 && L.head_dim == 128) ? "flash_prefill_w64_kernel" : "flash_prefill_dma_kernel", true);
-        if (lds_direct && ctx->prefill_variant == 3 && L.head_dim == 128) {
-            auto kern = L.bf16 ? (L.paged ? flash_prefill_w64_kernel<true, true> : flash_prefill_w64_kernel<true, false>)
-                               : (L.paged ? flash_prefill_w64_kernel<false, true> : flash_prefill_w64_kernel<false, false>);
-            scope.launch(kern, grid, dim3(256), 0, a);
-        } else if (lds_direct) {
+        FaLaunchScope scope(ctx, lds_direct ? "flash_prefill_dma_kernel" : "flash_prefill_mfma_kernel", true);
+        if (lds_direct) {
             auto kern = flash_prefill_dma_kernel<128, false, false>;
             if (L.head_dim == 128) {
                 kern = L.bf16 ? (L.paged ? flash_prefill_dma_kernel<128, true, true> : flash_prefill_dma_kernel<128, true, false>)

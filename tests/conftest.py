@@ -12,7 +12,7 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
-@pytest.fixture(params=[1, 2, 3], ids=["staged", "lds_direct", "rows64"])
+@pytest.fixture(params=[1, 2], ids=["staged", "lds_direct"])
 def prefill_variant(request):
     """Runs a GPU test once per prefill kernel variant (fa_set_prefill_variant) and restores the default."""
     from gpu_util import ctx
