@@ -191,3 +191,27 @@ def test_fused_step_past_its_bound_is_reported():
     assert np.array_equal(bits(got_k[:, start + 2]), bits(kc[:, start + 2])), "the dropped token must not be stored"
     for b in d.values():
         b.free()
+
+
+def test_stream_timer_and_compute_units():
+    announce("stream timer")
+    f = ctx()
+    assert f.n_cus() >= 1
+    with pytest.raises(fa.FoundryError) as e:
+        f.timer_stop()  # nothing started
+    assert e.value.variant == "InvalidOperation"
+    word = f.array(np.zeros(4, np.uint32))
+    f.start_capture()
+    with pytest.raises(fa.FoundryError):
+        f.timer_start()  # not during a capture
+    for _ in range(64):
+        f.u32_add(word, 1, 1)
+    g = f.end_capture()
+    f.timer_start()
+    for _ in range(4):
+        g.launch()
+    ms = f.timer_stop()
+    assert 0.0 < ms < 100.0
+    assert int(word.download()[0]) == 256
+    g.destroy()
+    word.free()
