@@ -726,10 +726,11 @@ def bench_attn_block(f, args):
         "parity": {"outputs_finite": finite, "note": "stage-by-stage parity of this chain: tests/test_gpu_block.py"}}))
 
 
-def bench_prefill_block(f, args):
+def bench_prefill_block(f, args, fused=False):
     """The attention block of one Llama-3.2-3B layer on a 2048-token prompt in one chunk (models/llama.json:509-585):
     FusedQkv (norm kernel + GEMM) -> KvPrepFused (RoPE + append of 2048 rows) -> FlashAttention (causal prefill) -> o_proj
-    MatMul with residual (GEMM); F16 canonical weights, contiguous cache, eager launches, 4 layers' buffers in rotation."""
+    MatMul with residual (GEMM); F16 canonical weights, contiguous cache, eager launches, 4 layers' buffers in rotation.
+    fused: the first two as one op (fa_fused_qkv_kv_prep: KvPrepFused is the GEMM's write stage)."""
     L, H, Hkv, D, M = 4, 24, 8, 128, 2048
     dm, kvd, cap = H * D, Hkv * D, 2048
     rng = np.random.default_rng(0xF0DD + 12)
@@ -749,9 +750,13 @@ def bench_prefill_block(f, args):
 
     def step(i):
         ly = layers[i % L]
-        f.fused_qkv(hid.arg(), ly["wq"].arg(), ly["wk"].arg(), ly["wv"].arg(), dq.arg(), dk.arg(), dv.arg(), dm, dm, kvd, M,
-                    gamma=ly["g"].arg())
-        f.kv_prep_fused(dq.arg(), dk.arg(), dv.arg(), dqr.arg(), ly["kc"].arg(), ly["vc"].arg(), dcos.arg(), dsin.arg(), p)
+        if fused:
+            f.fused_qkv_kv_prep(hid.arg(), ly["wq"].arg(), ly["wk"].arg(), ly["wv"].arg(), dm, dqr.arg(), dcos.arg(), dsin.arg(), p,
+                                k_cache=ly["kc"].arg(), v_cache=ly["vc"].arg(), gamma=ly["g"].arg())
+        else:
+            f.fused_qkv(hid.arg(), ly["wq"].arg(), ly["wk"].arg(), ly["wv"].arg(), dq.arg(), dk.arg(), dv.arg(), dm, dm, kvd, M,
+                        gamma=ly["g"].arg())
+            f.kv_prep_fused(dq.arg(), dk.arg(), dv.arg(), dqr.arg(), ly["kc"].arg(), ly["vc"].arg(), dcos.arg(), dsin.arg(), p)
         f.flash_attention(dqr.arg(), ly["kc"].arg(), ly["vc"].arg(), dattn.arg(), True, 0, H, D, M, M)
         f.matmul(dattn.arg(), ly["wo"].arg(), dout.arg(), M, dm, dm, c=hid.arg(), transpose_b=False, alpha=1.0, beta=1.0)
 
@@ -780,8 +785,9 @@ def bench_prefill_block(f, args):
         "metric": "attention-block layer-steps/s, Llama-3.2-3B prefill of 2048 tokens", "value": args.steps / dt,
         "unit": "layer-steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "llama3.2-3b attention block on a 2048-token prompt, one layer per step: FusedQkv, KvPrepFused, "
-                               "causal FlashAttention, o_proj with residual; eager launches (profiling events on)"},
+        "config": {"workload": "llama3.2-3b attention block on a 2048-token prompt, one layer per step: "
+                               + ("FusedQkv with KvPrepFused as its write stage (one op), " if fused else "FusedQkv, KvPrepFused, ")
+                               + "causal FlashAttention, o_proj with residual; eager launches (profiling events on)"},
         "roofline": {"bound": "mfma", "achieved": flops / total_s / 1e12, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops / total_s / 1e12 / MFMA_F16_PEAK_TFLOPS, "traffic": None, "kernel": "sum of the block's kernels",
                      "avg_launch_us": us, "flops_per_step": flops},
@@ -1023,7 +1029,7 @@ def bench_floors(f, args):
     emit(out)
 
 
-SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill,
+SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill,
              "llama3b_prefill_8k": lambda f, args: bench_prefill(f, args, 8192), "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,

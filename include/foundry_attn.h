@@ -451,6 +451,31 @@ fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_ar
                        const fa_tensor_arg *out_v, const fa_tensor_arg *bias_q, const fa_tensor_arg *bias_k,
                        const fa_tensor_arg *bias_v, const fa_tensor_arg *gamma, const fa_fused_qkv_params *params);
 
+/* FusedQkv and KvPrepFused as one op (a prefill chunk: m = params->seq_len input rows). The two ops it joins are
+ * src/metals/gemv/qkv_step.rs:14-120 and src/metals/kv_prep/kv_prep_fused.metal:26-123; the reference runs them as two
+ * dispatches with the token-major q, k, v tensors between them and names their fusion as future work
+ * (LATEST_FOUNDRY.md:211). Arguments: those of fa_fused_qkv without out_q / out_k / out_v, then those of
+ * fa_kv_prep_fused (fa_kv_prep_fused_paged) without q / k / v. The result is bit for bit that of fa_fused_qkv followed
+ * by fa_kv_prep_fused on the same context: every projection is rounded to f16 as FusedQkv stores it, then rotated and
+ * placed as KvPrepFused does. qkv_params->m must equal params->seq_len, n_dim = params->d_model, n_kv = params->kv_dim;
+ * head_dim 64 or 128; f16 only; q_rot, caches / pools, biases and tables 16-byte aligned. From fa_set_gemm_min_m() rows
+ * on it is the GEMM's write stage (no q / k / v round trip, one launch fewer); with fewer rows the weight-stream
+ * kernel writes q, k, v into the context's workspace and the KvPrepFused kernel follows (m = 1 belongs to
+ * fa_decode_step_fused, which takes the raw projections). Workspace rule under capture as for fa_fused_qkv. */
+fa_status fa_fused_qkv_kv_prep(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
+                               const fa_tensor_arg *s_k, const fa_tensor_arg *w_v, const fa_tensor_arg *s_v,
+                               const fa_tensor_arg *input, const fa_tensor_arg *bias_q, const fa_tensor_arg *bias_k,
+                               const fa_tensor_arg *bias_v, const fa_tensor_arg *gamma, const fa_fused_qkv_params *qkv_params,
+                               const fa_tensor_arg *q_rot, const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
+                               const fa_tensor_arg *cos, const fa_tensor_arg *sin, const fa_kv_prep_fused_params *params);
+fa_status fa_fused_qkv_kv_prep_paged(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
+                                     const fa_tensor_arg *s_k, const fa_tensor_arg *w_v, const fa_tensor_arg *s_v,
+                                     const fa_tensor_arg *input, const fa_tensor_arg *bias_q, const fa_tensor_arg *bias_k,
+                                     const fa_tensor_arg *bias_v, const fa_tensor_arg *gamma,
+                                     const fa_fused_qkv_params *qkv_params, const fa_tensor_arg *q_rot,
+                                     const fa_paged_kv *cache, uint32_t seq_index, const fa_tensor_arg *cos,
+                                     const fa_tensor_arg *sin, const fa_kv_prep_fused_params *params);
+
 /* ---------------------------------------------------------------------------------------------
  * MatMul, weight-stream form: the step after the path (o_proj: `attn_out [m, H*D]` x W_o, residual `hidden`,
  * models/llama.json:566-585; op src/metals/matmul.rs:11-239, which runs GemvV2 for m == 1 and for canonical

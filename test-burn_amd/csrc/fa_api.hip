@@ -7,6 +7,7 @@
 #include <cstring>
 
 #include "fa_internal.h"
+#include "fa_qkv_rope.h"
 
 // ------------------------------------------------------------------------------------------------ errors
 
@@ -613,6 +614,33 @@ static fa_status check_kv_prep_params(const fa_kv_prep_fused_params *p) {
     return FA_OK;
 }
 
+// The outputs and tables of a KvPrepFused call (everything but its q, k, v inputs); `dt` is the data type of the call.
+static fa_status kv_prep_outputs(fa_ctx *ctx, fa_dtype dt, const fa_tensor_arg *q_rot, const fa_tensor_arg *cos,
+                                 const fa_tensor_arg *sin, const fa_kv_prep_fused_params *p, KvPrepLaunch &L) {
+    FA_NEED(ctx, "ctx");
+    FA_TRY(check_kv_prep_params(p));
+    const int al = p->head_dim % 16 == 0 ? 16 : 2;
+    const size_t nq = (size_t)p->seq_len * p->d_model;
+    FA_TRY(check_tensor(q_rot, "q_rot", dt, nq, al));
+    FA_TRY(check_tensor(cos, "cos", FA_DTYPE_F16, 0, al));
+    FA_TRY(check_tensor(sin, "sin", FA_DTYPE_F16, 0, al));
+    const uint32_t half = p->head_dim / 2;
+    size_t rows = numel(cos) / half;
+    const size_t rows_s = numel(sin) / half;
+    if (rows_s < rows) rows = rows_s;
+    if (cos->rank == 0 || sin->rank == 0) rows = 0xffffffffu;  // metadata-free tables: trust the caller
+    if (rows == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: empty RoPE tables");
+    L.q = L.k = L.v = nullptr;
+    L.q_rot = tptr<__half>(q_rot);
+    L.cos_t = tptr<const __half>(cos), L.sin_t = tptr<const __half>(sin);
+    L.p = *p;
+    L.d_position = nullptr, L.block_table = nullptr, L.seq_lens = nullptr;
+    L.bt_stride = 0, L.block_size = 1;
+    L.table_rows = (uint32_t)(rows > 0xffffffffu ? 0xffffffffu : rows);
+    L.bf16 = dt == FA_DTYPE_BF16;
+    return FA_OK;
+}
+
 static fa_status kv_prep_common(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tensor_arg *k, const fa_tensor_arg *v,
                                 const fa_tensor_arg *q_rot, const fa_tensor_arg *cos, const fa_tensor_arg *sin,
                                 const fa_kv_prep_fused_params *p, KvPrepLaunch &L) {
@@ -623,23 +651,8 @@ static fa_status kv_prep_common(fa_ctx *ctx, const fa_tensor_arg *q, const fa_te
     FA_TRY(check_tensor(q, "q", FA_DT(q), nq, al));
     FA_TRY(check_tensor(k, "k", FA_DT(q), nkv, al));
     FA_TRY(check_tensor(v, "v", FA_DT(q), nkv, al));
-    FA_TRY(check_tensor(q_rot, "q_rot", FA_DT(q), nq, al));
-    FA_TRY(check_tensor(cos, "cos", FA_DTYPE_F16, 0, al));
-    FA_TRY(check_tensor(sin, "sin", FA_DTYPE_F16, 0, al));
-    const uint32_t half = p->head_dim / 2;
-    size_t rows = numel(cos) / half;
-    const size_t rows_s = numel(sin) / half;
-    if (rows_s < rows) rows = rows_s;
-    if (cos->rank == 0 || sin->rank == 0) rows = 0xffffffffu;  // metadata-free tables: trust the caller
-    if (rows == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: empty RoPE tables");
+    FA_TRY(kv_prep_outputs(ctx, FA_DT(q), q_rot, cos, sin, p, L));
     L.q = tptr<const __half>(q), L.k = tptr<const __half>(k), L.v = tptr<const __half>(v);
-    L.q_rot = tptr<__half>(q_rot);
-    L.cos_t = tptr<const __half>(cos), L.sin_t = tptr<const __half>(sin);
-    L.p = *p;
-    L.d_position = nullptr, L.block_table = nullptr, L.seq_lens = nullptr;
-    L.bt_stride = 0, L.block_size = 1;
-    L.table_rows = (uint32_t)(rows > 0xffffffffu ? 0xffffffffu : rows);
-    L.bf16 = FA_IS_BF16(q);
     return FA_OK;
 }
 
@@ -890,16 +903,20 @@ static fa_status weight_kind(const fa_tensor_arg *w, const fa_tensor_arg *scales
     return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "%s: weight dtype %u: F16, Q8_0 and Q4_0 weights are built, no other block-quantised policy", what, w->dtype);
 }
 
-extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
+// Checks a FusedQkv call and fills its launch. with_outputs = false: the three token-major outputs are not part of the
+// call (the KvPrepFused write stage takes their place) and L.out stays empty.
+static fa_status fused_qkv_common(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
                                   const fa_tensor_arg *s_k, const fa_tensor_arg *w_v, const fa_tensor_arg *s_v,
-                                  const fa_tensor_arg *input, const fa_tensor_arg *out_q, const fa_tensor_arg *out_k,
-                                  const fa_tensor_arg *out_v, const fa_tensor_arg *bias_q, const fa_tensor_arg *bias_k,
-                                  const fa_tensor_arg *bias_v, const fa_tensor_arg *gamma, const fa_fused_qkv_params *p) {
+                                  const fa_tensor_arg *input, bool with_outputs, const fa_tensor_arg *out_q,
+                                  const fa_tensor_arg *out_k, const fa_tensor_arg *out_v, const fa_tensor_arg *bias_q,
+                                  const fa_tensor_arg *bias_k, const fa_tensor_arg *bias_v, const fa_tensor_arg *gamma,
+                                  const fa_fused_qkv_params *p, FusedQkvLaunch &L) {
     FA_NEED(ctx, "ctx");
     FA_NEED(p, "params");
     const struct { const fa_tensor_arg *t; const char *name; } req[] = {{input, "input"}, {w_q, "w_q"}, {w_k, "w_k"}, {w_v, "w_v"},
                                                                          {out_q, "out_q"}, {out_k, "out_k"}, {out_v, "out_v"}};
     for (const auto &r : req) {
+        if (!with_outputs && r.name[0] == 'o') continue;
         FA_NEED(r.t, r.name);
         if (!r.t->buffer) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: %s", r.name);
     }
@@ -911,7 +928,8 @@ extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const f
     if (wbits != wbits_k || wbits != wbits_v)  // the reference falls back to three separate projections there (qkv_step.rs:243-259)
         return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: mixed weight dtypes are not supported");
     for (const fa_tensor_arg *t : {input, out_q, out_k, out_v})
-        if (t->dtype != FA_DTYPE_F16) return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: activations must be F16, got dtype %u", t->dtype);
+        if ((t == input || with_outputs) && t->dtype != FA_DTYPE_F16)
+            return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: activations must be F16, got dtype %u", t->dtype);
     const uint32_t m = p->m ? p->m : 1;
     if (p->k_dim == 0 || p->n_dim == 0 || p->n_kv == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv k_dim %u n_dim %u n_kv %u", p->k_dim, p->n_dim, p->n_kv);
     if (p->k_dim % 32 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: k_dim %u must be a multiple of 32", p->k_dim);
@@ -929,7 +947,7 @@ extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const f
     }
     if (numel(w_q) < (size_t)p->n_dim * p->k_dim || numel(w_k) < (size_t)p->n_kv * p->k_dim || numel(w_v) < (size_t)p->n_kv * p->k_dim)
         return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv weights smaller than rows * k_dim");
-    if (numel(out_q) < (size_t)m * p->n_dim || numel(out_k) < (size_t)m * p->n_kv || numel(out_v) < (size_t)m * p->n_kv)
+    if (with_outputs && (numel(out_q) < (size_t)m * p->n_dim || numel(out_k) < (size_t)m * p->n_kv || numel(out_v) < (size_t)m * p->n_kv))
         return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv outputs smaller than m * rows");
     const bool has_norm = present(gamma), has_bias = present(bias_q);
     if (has_norm && (gamma->dtype != FA_DTYPE_F16 || numel(gamma) < p->k_dim))
@@ -940,12 +958,14 @@ extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const f
             numel(bias_k) < p->n_kv || numel(bias_v) < p->n_kv)
             return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv biases must be F16 [n_dim], [n_kv], [n_kv]");
     }
-    FusedQkvLaunch L;
     L.w[0] = half_ptr(w_q), L.w[1] = half_ptr(w_k), L.w[2] = half_ptr(w_v);
     L.bias[0] = has_bias ? half_ptr(bias_q) : nullptr, L.bias[1] = has_bias ? half_ptr(bias_k) : nullptr;
     L.bias[2] = has_bias ? half_ptr(bias_v) : nullptr;
-    L.out[0] = const_cast<__half *>(half_ptr(out_q)), L.out[1] = const_cast<__half *>(half_ptr(out_k));
-    L.out[2] = const_cast<__half *>(half_ptr(out_v));
+    L.out[0] = L.out[1] = L.out[2] = nullptr;
+    if (with_outputs) {
+        L.out[0] = const_cast<__half *>(half_ptr(out_q)), L.out[1] = const_cast<__half *>(half_ptr(out_k));
+        L.out[2] = const_cast<__half *>(half_ptr(out_v));
+    }
     L.x = half_ptr(input), L.gamma = has_norm ? half_ptr(gamma) : nullptr;
     L.k_dim = p->k_dim, L.n_dim = p->n_dim, L.n_kv = p->n_kv, L.m = m, L.eps = p->epsilon;
     L.canonical = p->layout == FA_WEIGHT_LAYOUT_CANONICAL;
@@ -953,7 +973,106 @@ extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const f
     L.weight_bits = wbits;
     for (const void *ptr : {(const void *)L.w[0], (const void *)L.w[1], (const void *)L.w[2], (const void *)L.x, (const void *)L.gamma})
         if (ptr && (uintptr_t)ptr % 16 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: input, gamma and weights must be 16-byte aligned");
+    return FA_OK;
+}
+
+extern "C" fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
+                                  const fa_tensor_arg *s_k, const fa_tensor_arg *w_v, const fa_tensor_arg *s_v,
+                                  const fa_tensor_arg *input, const fa_tensor_arg *out_q, const fa_tensor_arg *out_k,
+                                  const fa_tensor_arg *out_v, const fa_tensor_arg *bias_q, const fa_tensor_arg *bias_k,
+                                  const fa_tensor_arg *bias_v, const fa_tensor_arg *gamma, const fa_fused_qkv_params *p) {
+    FusedQkvLaunch L;
+    FA_TRY(fused_qkv_common(ctx, w_q, s_q, w_k, s_k, w_v, s_v, input, true, out_q, out_k, out_v, bias_q, bias_k, bias_v, gamma, p, L));
     return fa_launch_fused_qkv(ctx, L);
+}
+
+// FusedQkv followed by KvPrepFused as one op. From gemm_min_m input rows on the GEMM's write stage does the KvPrepFused
+// work; below, the weight-stream kernel writes q, k, v into the workspace and the KvPrepFused kernel follows.
+static fa_status fused_qkv_kv_prep(fa_ctx *ctx, FusedQkvLaunch &Q, KvPrepLaunch &K) {
+    const fa_kv_prep_fused_params &kp = K.p;
+    if (Q.m != kp.seq_len) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv m %u != KvPrepFused seq_len %u", Q.m, kp.seq_len);
+    if (Q.n_dim != kp.d_model || Q.n_kv != kp.kv_dim)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv n_dim %u / n_kv %u != KvPrepFused d_model %u / kv_dim %u", Q.n_dim, Q.n_kv,
+                       kp.d_model, kp.kv_dim);
+    if (!(kp.head_dim == 64 || kp.head_dim == 128))
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv + KvPrepFused supports head_dim 64 or 128, got %u", kp.head_dim);
+    if (Q.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : FA_GEMM_MIN_M_DEFAULT)) {  // the row count from which fa_launch_fused_qkv takes the GEMM
+        QkvRopeLaunch R;
+        R.cos_t = K.cos_t, R.sin_t = K.sin_t, R.q_rot = K.q_rot, R.k_cache = K.k_cache, R.v_cache = K.v_cache;
+        R.block_table = K.mode == 1 ? K.block_table : nullptr;
+        R.head_dim = kp.head_dim, R.n_heads = kp.n_heads, R.n_kv_heads = kp.n_kv_heads, R.position_offset = kp.position_offset;
+        R.max_seq_len = kp.max_seq_len, R.block_size = K.block_size, R.capacity = K.capacity, R.table_rows = K.table_rows;
+        R.rope_normal = kp.rope_mode == FA_ROPE_MODE_NORMAL;
+        R.apply_rope = kp.no_rope_layer_step == 0 || ((kp.layer_idx + 1u) % kp.no_rope_layer_step) != 0u;
+        return fa_launch_fused_qkv_gemm_rope(ctx, Q, R);
+    }
+    const size_t nq = ((size_t)Q.m * Q.n_dim * sizeof(__half) + 255) & ~(size_t)255;
+    const size_t nkv = ((size_t)Q.m * Q.n_kv * sizeof(__half) + 255) & ~(size_t)255;
+    FA_TRY(fa_ensure_workspace(ctx, nq + 2 * nkv));
+    char *ws = (char *)ctx->workspace;
+    Q.out[0] = (__half *)ws, Q.out[1] = (__half *)(ws + nq), Q.out[2] = (__half *)(ws + nq + nkv);
+    const uint32_t min_m = ctx->gemm_min_m;
+    ctx->gemm_min_m = 0xffffffffu;  // the weight-stream kernel: its outputs are in the workspace the GEMM would use
+    const fa_status st = fa_launch_fused_qkv(ctx, Q);
+    ctx->gemm_min_m = min_m;
+    FA_TRY(st);
+    K.q = Q.out[0], K.k = Q.out[1], K.v = Q.out[2];
+    return fa_launch_kv_prep(ctx, K);
+}
+
+extern "C" fa_status fa_fused_qkv_kv_prep(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
+                                          const fa_tensor_arg *s_k, const fa_tensor_arg *w_v, const fa_tensor_arg *s_v,
+                                          const fa_tensor_arg *input, const fa_tensor_arg *bias_q, const fa_tensor_arg *bias_k,
+                                          const fa_tensor_arg *bias_v, const fa_tensor_arg *gamma, const fa_fused_qkv_params *qkv_params,
+                                          const fa_tensor_arg *q_rot, const fa_tensor_arg *k_cache, const fa_tensor_arg *v_cache,
+                                          const fa_tensor_arg *cos, const fa_tensor_arg *sin, const fa_kv_prep_fused_params *p) {
+    FusedQkvLaunch Q;
+    FA_TRY(fused_qkv_common(ctx, w_q, s_q, w_k, s_k, w_v, s_v, input, false, nullptr, nullptr, nullptr, bias_q, bias_k, bias_v, gamma,
+                            qkv_params, Q));
+    KvPrepLaunch K;
+    FA_TRY(kv_prep_outputs(ctx, FA_DTYPE_F16, q_rot, cos, sin, p, K));
+    const size_t ncache = (size_t)p->n_kv_heads * p->max_seq_len * p->head_dim;
+    FA_TRY(check_tensor(k_cache, "k_cache", FA_DTYPE_F16, ncache, 16));
+    FA_TRY(check_tensor(v_cache, "v_cache", FA_DTYPE_F16, ncache, 16));
+    if ((uint64_t)p->position_offset + p->seq_len > p->max_seq_len)
+        return fa_fail(FA_ERR_INVALID_OPERATION, "Invalid operation: position_offset %u + seq_len %u exceeds max_seq_len %u",
+                       p->position_offset, p->seq_len, p->max_seq_len);
+    if ((uint64_t)p->position_offset + p->seq_len > K.table_rows)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: RoPE tables hold %u rows, %u needed", K.table_rows, p->position_offset + p->seq_len);
+    K.k_cache = tptr<__half>(k_cache), K.v_cache = tptr<__half>(v_cache);
+    K.mode = 0, K.capacity = p->max_seq_len;
+    return fused_qkv_kv_prep(ctx, Q, K);
+}
+
+extern "C" fa_status fa_fused_qkv_kv_prep_paged(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
+                                                const fa_tensor_arg *s_k, const fa_tensor_arg *w_v, const fa_tensor_arg *s_v,
+                                                const fa_tensor_arg *input, const fa_tensor_arg *bias_q, const fa_tensor_arg *bias_k,
+                                                const fa_tensor_arg *bias_v, const fa_tensor_arg *gamma,
+                                                const fa_fused_qkv_params *qkv_params, const fa_tensor_arg *q_rot,
+                                                const fa_paged_kv *cache, uint32_t seq_index, const fa_tensor_arg *cos,
+                                                const fa_tensor_arg *sin, const fa_kv_prep_fused_params *p) {
+    FusedQkvLaunch Q;
+    FA_TRY(fused_qkv_common(ctx, w_q, s_q, w_k, s_k, w_v, s_v, input, false, nullptr, nullptr, nullptr, bias_q, bias_k, bias_v, gamma,
+                            qkv_params, Q));
+    FA_TRY(check_paged(cache));
+    KvPrepLaunch K;
+    FA_TRY(kv_prep_outputs(ctx, FA_DTYPE_F16, q_rot, cos, sin, p, K));
+    if (p->head_dim != cache->head_dim || p->n_kv_heads != cache->n_kv_heads)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: params (Hkv %u, D %u) do not match the paged cache (Hkv %u, D %u)",
+                       p->n_kv_heads, p->head_dim, cache->n_kv_heads, cache->head_dim);
+    if (seq_index >= cache->n_seqs) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: seq_index %u >= n_seqs %u", seq_index, cache->n_seqs);
+    const uint64_t cap = (uint64_t)cache->max_blocks_per_seq * cache->block_size;
+    if ((uint64_t)p->position_offset + p->seq_len > cap)
+        return fa_fail(FA_ERR_INVALID_OPERATION, "Invalid operation: position_offset %u + seq_len %u exceeds paged capacity %llu",
+                       p->position_offset, p->seq_len, (unsigned long long)cap);
+    if ((uint64_t)p->position_offset + p->seq_len > K.table_rows)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: RoPE tables hold %u rows, %u needed", K.table_rows, p->position_offset + p->seq_len);
+    K.k_cache = (__half *)cache->k_pool, K.v_cache = (__half *)cache->v_pool;
+    K.mode = 1;
+    K.block_table = cache->block_table + (size_t)seq_index * cache->max_blocks_per_seq;
+    K.bt_stride = cache->max_blocks_per_seq, K.block_size = cache->block_size;
+    K.capacity = (uint32_t)cap;
+    return fused_qkv_kv_prep(ctx, Q, K);
 }
 
 extern "C" fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_tensor_arg *b, const fa_tensor_arg *b_scales,

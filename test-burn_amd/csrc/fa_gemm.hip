@@ -16,11 +16,13 @@
 //   * the rows of W_q, W_k, W_v are tiled per matrix (a tile never straddles two); the workgroups of one XCD take
 //     consecutive tiles of the weight rows over all input rows, so a weight tile is fetched into one L2 only;
 //   * epilogue: accumulators to LDS as f32 [input row][weight row], then alpha * sum + bias + beta * residual, one
-//     rounding to f16 (as the GEMV path), 16-byte token-major stores.
+//     rounding to f16 (as the GEMV path), 16-byte token-major stores - or, with a RoPE write stage, the KvPrepFused
+//     arithmetic on those f16 values and stores to q_rot and the cache rows (rope_store_piece).
 // RMSNorm: a small kernel in front writes the normalised input, rounded to f16 as qkv_project.metal:66-67 does, into
 // the context's workspace; the GEMM reads that. Launches with few output tiles divide a tile's feature steps over
 // several workgroups (split-K: f32 partial tiles in the workspace, added in split order by gemm_finish_kernel).
 #include "fa_internal.h"
+#include "fa_qkv_rope.h"
 #include <type_traits>
 
 namespace {
@@ -45,6 +47,13 @@ typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef float f4v_t __attribute__((ext_vector_type(4)));
 typedef float f16v_t __attribute__((ext_vector_type(16)));
 
+// KvPrepFused as the write stage (kv_prep_fused.metal:45-122): out[0] is q_rot [H, m, D], out[1] / out[2] the K / V cache.
+struct RopeDev {
+    const __half *cos_t, *sin_t;
+    const int32_t *block_table;  // paged: the sequence's table row
+    uint32_t on, head_dim, n_kv_heads, position_offset, max_seq_len, block_size, capacity, table_rows, normal, apply;
+};
+
 struct GemmDev {
     const void *w[3];       // f16, or int8 (Q8_0) / nibbles (Q4_0) in the same element order
     const __half *scales[3];  // Q8_0: f16 [rows, k_dim / 32] per matrix
@@ -60,7 +69,61 @@ struct GemmDev {
     // [split][m][n_total]; gemm_finish_kernel adds them up in split order and applies the write stage
     uint32_t k_splits, steps_per_split, n_total;
     float *partial;
+    RopeDev rope;
 };
+
+// Rotation of one element: products and sum rounded separately (kv_prep_fused.metal:74-82), as fa_kvprep.hip.
+__device__ __forceinline__ float rope_one(float x, float mate, float c, float s, bool first) {
+#pragma clang fp contract(off)
+    const float p0 = x * c, p1 = mate * s;
+    return first ? p0 - p1 : p0 + p1;
+}
+
+// Write stage of one piece: y = the projections of token gm, columns gn .. gn + 7 of matrix mat (0 Q, 1 K, 2 V),
+// already rounded to f16 as FusedQkv stores them; mate = the piece half a head away (NeoX pairing; unused otherwise).
+// Q goes to q_rot[h][gm][hd], K (rotated) and V (as is) to cache row position_offset + gm of KV head h.
+__device__ __forceinline__ void rope_store_piece(const GemmDev &a, int mat, uint32_t gm, uint32_t gn, h8_t y, const h8_t mate) {
+    const RopeDev &r = a.rope;
+    const uint32_t D = r.head_dim, half = D >> 1, h = gn / D, hd = gn - h * D;
+    const uint32_t pos = r.position_offset + gm;
+    __half *dst;
+    if (mat == 0) {
+        dst = a.out[0] + ((size_t)h * a.m + gm) * D + hd;
+    } else {
+        if (pos >= r.capacity) return;  // never outside the cache
+        size_t row;
+        if (!r.block_table) {
+            row = ((size_t)h * r.max_seq_len + pos) * D;
+        } else {
+            const size_t blk = (size_t)r.block_table[pos / r.block_size];
+            row = ((blk * r.n_kv_heads + h) * r.block_size + pos % r.block_size) * D;
+        }
+        dst = (mat == 1 ? a.out[1] : a.out[2]) + row + hd;
+    }
+    if (mat != 2 && r.apply) {
+        const uint32_t tp = pos < r.table_rows ? pos : r.table_rows - 1;  // stay inside the tables
+        if (r.normal) {  // pairs (hd + 2i, hd + 2i + 1), table columns hd / 2 + i
+            typedef _Float16 h4v_t __attribute__((ext_vector_type(4)));
+            const h4v_t c4 = *reinterpret_cast<const h4v_t *>(r.cos_t + (size_t)tp * half + (hd >> 1));
+            const h4v_t s4 = *reinterpret_cast<const h4v_t *>(r.sin_t + (size_t)tp * half + (hd >> 1));
+            h8_t o;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                o[2 * i] = (_Float16)rope_one((float)y[2 * i], (float)y[2 * i + 1], (float)c4[i], (float)s4[i], true);
+                o[2 * i + 1] = (_Float16)rope_one((float)y[2 * i + 1], (float)y[2 * i], (float)c4[i], (float)s4[i], false);
+            }
+            y = o;
+        } else {  // pairs (hd, hd + D / 2), table column hd mod D / 2
+            const bool first = hd < half;
+            const uint32_t pc = first ? hd : hd - half;
+            const h8_t c8 = *reinterpret_cast<const h8_t *>(r.cos_t + (size_t)tp * half + pc);
+            const h8_t s8 = *reinterpret_cast<const h8_t *>(r.sin_t + (size_t)tp * half + pc);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) y[e] = (_Float16)rope_one((float)y[e], (float)mate[e], (float)c8[e], (float)s8[e], first);
+        }
+    }
+    *reinterpret_cast<h8_t *>(dst) = y;
+}
 
 // inv_rms of each input row, then (x * inv_rms) * gamma in f32, rounded to f16 (rmsnorm.metal:17-96).
 __global__ void __launch_bounds__(256) rmsnorm_rows_kernel(const __half *x, const __half *gamma, __half *y, uint32_t K,
@@ -160,7 +223,26 @@ __device__ __forceinline__ void gemm_epilogue(const GemmDev &a, unsigned char *s
                     if (a.residual) v += a.beta * (float)rv[e];
                     y[e] = (_Float16)v;
                 }
-                *reinterpret_cast<h8_t *>(out + o) = y;
+                if (a.rope.on) {
+                    // the mate piece of a NeoX pair lies half a head away in the same LDS row (a tile holds whole heads)
+                    h8_t mate = z;
+                    if (!a.rope.normal && a.rope.apply && mat != 2) {
+                        const uint32_t hp = a.rope.head_dim >> 4;  // pieces in half a head
+                        const uint32_t m8 = ((n8 * 8) & (a.rope.head_dim - 1)) < (a.rope.head_dim >> 1) ? n8 + hp : n8 - hp;
+                        const f4v_t t0 = *reinterpret_cast<const f4v_t *>(smem + t * GM_T_STRIDE + m8 * 32);
+                        const f4v_t t1 = *reinterpret_cast<const f4v_t *>(smem + t * GM_T_STRIDE + m8 * 32 + 16);
+                        const h8_t bm = bias ? *reinterpret_cast<const h8_t *>(bias + n0 + m8 * 8) : z;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            float v = (e < 4 ? t0[e & 3] : t1[e & 3]) * a.alpha;
+                            if (bias) v += (float)bm[e];
+                            mate[e] = (_Float16)v;
+                        }
+                    }
+                    rope_store_piece(a, mat, gm, gn, y, mate);
+                } else {
+                    *reinterpret_cast<h8_t *>(out + o) = y;
+                }
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
@@ -706,36 +788,51 @@ __global__ void __launch_bounds__(256) gemm_finish_kernel(GemmDev a) {
     __half *out = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
     const size_t o = (size_t)gm * N + gn;
     if (a.vec_store) {
-        f4v_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
         const size_t split_stride = (size_t)a.m * a.n_total;
-        const float *src = a.partial + (size_t)gm * a.n_total + col;
-        uint32_t sp = 0;
-        for (; sp + 4 <= a.k_splits; sp += 4) {  // four splits' loads in flight, added in split order
-            f4v_t u[4], w[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                u[q] = *reinterpret_cast<const f4v_t *>(src + (sp + q) * split_stride);
-                w[q] = *reinterpret_cast<const f4v_t *>(src + (sp + q) * split_stride + 4);
-            }
-#pragma unroll
-            for (int q = 0; q < 4; ++q) s0 += u[q], s1 += w[q];
-        }
-        for (; sp < a.k_splits; ++sp) {
-            s0 += *reinterpret_cast<const f4v_t *>(src + sp * split_stride);
-            s1 += *reinterpret_cast<const f4v_t *>(src + sp * split_stride + 4);
-        }
         const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-        const h8_t bv = bias ? *reinterpret_cast<const h8_t *>(bias + gn) : z;
-        const h8_t rv = a.residual ? *reinterpret_cast<const h8_t *>(a.residual + o) : z;
-        h8_t y;
+        // the write stage's value of the 8 columns from column c of the concatenated list (column g of the matrix)
+        auto piece = [&](uint32_t c, uint32_t g) -> h8_t {
+            f4v_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = s0;
+            const float *src = a.partial + (size_t)gm * a.n_total + c;
+            uint32_t sp = 0;
+            for (; sp + 4 <= a.k_splits; sp += 4) {  // four splits' loads in flight, added in split order
+                f4v_t u[4], w[4];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            float t = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
-            if (bias) t += (float)bv[e];
-            if (a.residual) t += a.beta * (float)rv[e];
-            y[e] = (_Float16)t;
+                for (int q = 0; q < 4; ++q) {
+                    u[q] = *reinterpret_cast<const f4v_t *>(src + (sp + q) * split_stride);
+                    w[q] = *reinterpret_cast<const f4v_t *>(src + (sp + q) * split_stride + 4);
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) s0 += u[q], s1 += w[q];
+            }
+            for (; sp < a.k_splits; ++sp) {
+                s0 += *reinterpret_cast<const f4v_t *>(src + sp * split_stride);
+                s1 += *reinterpret_cast<const f4v_t *>(src + sp * split_stride + 4);
+            }
+            const h8_t bv = bias ? *reinterpret_cast<const h8_t *>(bias + g) : z;
+            const h8_t rv = a.residual ? *reinterpret_cast<const h8_t *>(a.residual + (size_t)gm * N + g) : z;
+            h8_t y;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float t = (e < 4 ? s0[e & 3] : s1[e & 3]) * a.alpha;
+                if (bias) t += (float)bv[e];
+                if (a.residual) t += a.beta * (float)rv[e];
+                y[e] = (_Float16)t;
+            }
+            return y;
+        };
+        const h8_t y = piece(col, gn);
+        if (a.rope.on) {
+            h8_t mate = z;
+            if (!a.rope.normal && a.rope.apply && mat != 2) {  // NeoX: the piece half a head away
+                const uint32_t half = a.rope.head_dim >> 1;
+                const bool first = (gn & (a.rope.head_dim - 1)) < half;
+                mate = first ? piece(col + half, gn + half) : piece(col - half, gn - half);
+            }
+            rope_store_piece(a, mat, gm, gn, y, mate);
+        } else {
+            *reinterpret_cast<h8_t *>(out + o) = y;
         }
-        *reinterpret_cast<h8_t *>(out + o) = y;
     } else {
         // a group of 8 columns of the concatenated list may straddle two matrices: element by element
         for (uint32_t e = 0; e < 8 && col + e < a.n_total; ++e) {
@@ -760,11 +857,26 @@ __global__ void __launch_bounds__(256) gemm_finish_kernel(GemmDev a) {
 
 }  // namespace
 
-fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
+static fa_status launch_gemm(fa_ctx *ctx, const FusedQkvLaunch &l, const QkvRopeLaunch *rope) {
     if (l.k_dim % 8 != 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: k_dim %u must be a multiple of 8", l.k_dim);
     GemmDev a;
     memset(&a, 0, sizeof(a));
     for (int i = 0; i < 3; ++i) a.w[i] = l.w[i], a.bias[i] = l.bias[i], a.out[i] = l.out[i], a.scales[i] = l.scales[i];
+    if (rope) {
+        const QkvRopeLaunch &r = *rope;
+        // a 128-row tile of a weight matrix must hold whole heads (the NeoX mate of a column lies in the same tile)
+        if (!(r.head_dim == 64 || r.head_dim == 128))
+            return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv with the KvPrepFused write stage supports head_dim 64 or 128, got %u", r.head_dim);
+        if (l.n_dim != r.n_heads * r.head_dim || l.n_kv != r.n_kv_heads * r.head_dim)
+            return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_dim %u / n_kv %u are not n_heads %u / n_kv_heads %u x head_dim %u", l.n_dim,
+                           l.n_kv, r.n_heads, r.n_kv_heads, r.head_dim);
+        if (l.residual) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "the KvPrepFused write stage takes no residual");
+        a.out[0] = r.q_rot, a.out[1] = r.k_cache, a.out[2] = r.v_cache;
+        a.rope.cos_t = r.cos_t, a.rope.sin_t = r.sin_t, a.rope.block_table = r.block_table;
+        a.rope.on = 1, a.rope.head_dim = r.head_dim, a.rope.n_kv_heads = r.n_kv_heads, a.rope.position_offset = r.position_offset;
+        a.rope.max_seq_len = r.max_seq_len, a.rope.block_size = r.block_size ? r.block_size : 1, a.rope.capacity = r.capacity;
+        a.rope.table_rows = r.table_rows, a.rope.normal = r.rope_normal ? 1u : 0u, a.rope.apply = r.apply_rope ? 1u : 0u;
+    }
     const bool q8 = l.scales[0] != nullptr;
     a.rows[0] = l.n_dim, a.rows[1] = l.n_kv, a.rows[2] = l.n_kv;
     a.n_tiles = 0;
@@ -780,6 +892,8 @@ fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
     }
     vec = vec && (!a.residual || aligned16(a.residual));
     a.vec_store = vec ? 1u : 0u;
+    if (rope && (!vec || !aligned16(rope->cos_t) || !aligned16(rope->sin_t)))
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv with the KvPrepFused write stage needs 16-byte aligned q_rot, caches, biases and tables");
     if (!aligned16(l.x) || !aligned16(l.w[0]) || (l.w[1] && !aligned16(l.w[1])) || (l.w[2] && !aligned16(l.w[2])) ||
         (l.gamma && !aligned16(l.gamma)))
         return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: the GEMM path needs 16-byte aligned input and weights");
@@ -804,7 +918,7 @@ fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
     const size_t partial_bytes = a.k_splits > 1 ? (size_t)a.k_splits * l.m * a.n_total * sizeof(float) : 0;
     if (norm_bytes + partial_bytes) FA_TRY(fa_ensure_workspace(ctx, norm_bytes + partial_bytes));
     a.partial = (float *)((char *)ctx->workspace + norm_bytes);
-    if (a.k_splits > 1 && a.n_total % 8 != 0) a.vec_store = 0;
+    if (a.k_splits > 1 && a.n_total % 8 != 0) a.vec_store = 0;  // (never with a RoPE write stage: whole heads of 64 or 128)
     if (l.gamma) {
         FaLaunchScope norm(ctx, "rmsnorm_rows_kernel", true);
         norm.launch(rmsnorm_rows_kernel, dim3(l.m), dim3(256), 0, l.x, l.gamma, (__half *)ctx->workspace, l.k_dim, l.eps);
@@ -863,3 +977,7 @@ fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) {
     }
     return FA_OK;
 }
+
+fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l) { return launch_gemm(ctx, l, nullptr); }
+
+fa_status fa_launch_fused_qkv_gemm_rope(fa_ctx *ctx, const FusedQkvLaunch &l, const QkvRopeLaunch &r) { return launch_gemm(ctx, l, &r); }

@@ -23,6 +23,7 @@
 // the MatMul op (src/metals/matmul.rs:190-239 -> GemvV2, write stage src/metals/gemv/stages.rs:200-224): the o_proj
 // consumer of the attention output.
 #include "fa_internal.h"
+#include "fa_qkv_rope.h"
 #include <type_traits>
 
 namespace {
@@ -334,7 +335,7 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     // gamma, this kernel against the GEMM (norm kernel, split-K GEMM, finish kernel): m = 4: 10.4 / 16.7 us, m = 10:
     // 13.8 / 16.9, m = 12 (from where only one workgroup's input rows fit a CU's LDS): 18.8 / 17.0, m = 16: 19.7 / 17.5,
     // m = 24 (two passes): 35.1 / 18.2.
-    constexpr uint32_t GEMM_MIN_M_DEFAULT = 12;
+    constexpr uint32_t GEMM_MIN_M_DEFAULT = FA_GEMM_MIN_M_DEFAULT;
     auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
     const bool gemm_ok = l.k_dim % (q8 ? 32 : 8) == 0 && aligned16(l.x) && aligned16(l.w[0]) && aligned16(l.w[1]) &&
                          aligned16(l.w[2]) && aligned16(l.gamma);

@@ -138,6 +138,9 @@ PROTOTYPES = {
     "fa_paged_gather": [_vp, C.POINTER(PagedKv), _u32, _u32, _vp, _vp, _u32],
     "fa_paged_copy_blocks": [_vp, C.POINTER(PagedKv), _vp, _vp, _u32],
     "fa_fused_qkv": [_vp] + [_PT] * 14 + [C.POINTER(FusedQkvParams)],
+    "fa_fused_qkv_kv_prep": [_vp] + [_PT] * 11 + [C.POINTER(FusedQkvParams)] + [_PT] * 5 + [C.POINTER(KvPrepFusedParams)],
+    "fa_fused_qkv_kv_prep_paged": [_vp] + [_PT] * 11 + [C.POINTER(FusedQkvParams), _PT, C.POINTER(PagedKv), _u32, _PT, _PT,
+                                   C.POINTER(KvPrepFusedParams)],
     "fa_matmul": [_vp] + [_PT] * 6 + [C.POINTER(MatMulParams)],
     "fa_kv_prefix_copy": [_vp, _PT, _PT, _sz],
     "fa_kv_prefix_copy_batch": [_vp, _PT, _PT, _u32, _sz],
@@ -422,6 +425,24 @@ class Foundry:
         check(self.lib.fa_fused_qkv(self.h, C.byref(w_q), C.byref(sq), C.byref(w_k), C.byref(sk), C.byref(w_v), C.byref(sv),
                                     C.byref(x), C.byref(out_q), C.byref(out_k), C.byref(out_v), C.byref(bq), C.byref(bk),
                                     C.byref(bv), C.byref(g), C.byref(p)))
+
+    def fused_qkv_kv_prep(self, x, w_q, w_k, w_v, k_dim, q_rot, cos, sin, params, k_cache=None, v_cache=None, paged=None,
+                          seq_index=0, gamma=None, biases=None, layout=WEIGHT_LAYOUT_CANONICAL, weights_per_block=32,
+                          epsilon=1e-6, scales=None):
+        """FusedQkv + KvPrepFused in one op (params: KvPrepFusedParams; m = params.seq_len). Either k_cache and v_cache
+        (contiguous) or paged (a PagedKv) and seq_index."""
+        p = FusedQkvParams(k_dim, params.d_model, params.kv_dim, params.seq_len, weights_per_block, layout, epsilon)
+        none = TensorArg()
+        g = gamma if gamma is not None else none
+        bq, bk, bv = biases if biases is not None else (none, none, none)
+        sq, sk, sv = scales if scales is not None else (none, none, none)
+        head = [C.byref(t) for t in (w_q, sq, w_k, sk, w_v, sv, x, bq, bk, bv, g)] + [C.byref(p), C.byref(q_rot)]
+        if paged is None:
+            check(self.lib.fa_fused_qkv_kv_prep(self.h, *head, C.byref(k_cache), C.byref(v_cache), C.byref(cos), C.byref(sin),
+                                                C.byref(params)))
+        else:
+            check(self.lib.fa_fused_qkv_kv_prep_paged(self.h, *head, C.byref(paged), seq_index, C.byref(cos), C.byref(sin),
+                                                      C.byref(params)))
 
     def matmul(self, a, b, output, m, n, k, bias=None, c=None, transpose_b=True, alpha=1.0, beta=0.0, transpose_a=False,
                weights_per_block=32, activation=0, b_scales=None):

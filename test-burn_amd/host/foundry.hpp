@@ -466,6 +466,65 @@ inline void CompiledFusedQkvStep::execute(Foundry &foundry, const FastBindings &
                        b_q.c(), b_k.c(), b_v.c(), gamma.c(), &p));
 }
 
+// ---------------------------------------------------------------------------------------------- FusedQkv + KvPrepFused
+// A FusedQkv step whose three outputs feed the KvPrepFused step that follows it and nothing else (the pair of
+// models/llama.json:509-548), run as one op: fa_fused_qkv_kv_prep. The reference has no such step (it names the fusion as
+// future work, LATEST_FOUNDRY.md:211); an executor would form it from the two adjacent steps when `fusable` holds. The
+// tensors named by qkv.out_* / prep.q, k, v need not be bound: they are never written.
+struct FusedQkvKvPrepStep;
+struct CompiledFusedQkvKvPrepStep : CompiledStep {
+    const FusedQkvKvPrepStep *step;
+    size_t input_idx, w_q_idx, w_k_idx, w_v_idx, q_rot_idx, k_cache_idx, v_cache_idx, cos_idx, sin_idx;
+    std::optional<size_t> gamma_idx, bias_q_idx, bias_k_idx, bias_v_idx, s_q_idx, s_k_idx, s_v_idx;
+    void execute(Foundry &foundry, const FastBindings &fast, const TensorBindings &bindings, const SymbolTable &) const override;
+    const char *name() const override { return "FusedQkvKvPrep"; }
+};
+
+struct FusedQkvKvPrepStep {
+    FusedQkvStep qkv;
+    KvPrepFusedStep prep;
+    static bool fusable(const FusedQkvStep &a, const KvPrepFusedStep &b) { return a.out_q == b.q && a.out_k == b.k && a.out_v == b.v; }
+    std::vector<std::unique_ptr<CompiledStep>> compile(TensorBindings &b, SymbolTable &s) const {
+        if (!fusable(qkv, prep)) throw MetalError(MetalError::InvalidOperation, "FusedQkvKvPrep: KvPrepFused does not read FusedQkv's outputs");
+        auto c = std::make_unique<CompiledFusedQkvKvPrepStep>();
+        c->step = this;
+        auto idx = [&](const Ref &r) { return s.get_or_create(b.interpolate(r)); };
+        auto opt = [&](const std::optional<Ref> &r) -> std::optional<size_t> {
+            if (!r) return std::nullopt;
+            return idx(*r);
+        };
+        c->input_idx = idx(qkv.input), c->w_q_idx = idx(qkv.w_q), c->w_k_idx = idx(qkv.w_k), c->w_v_idx = idx(qkv.w_v);
+        c->gamma_idx = opt(qkv.gamma), c->bias_q_idx = opt(qkv.bias_q), c->bias_k_idx = opt(qkv.bias_k), c->bias_v_idx = opt(qkv.bias_v);
+        c->s_q_idx = opt(qkv.s_q), c->s_k_idx = opt(qkv.s_k), c->s_v_idx = opt(qkv.s_v);
+        c->q_rot_idx = idx(prep.q_rot), c->k_cache_idx = idx(prep.k_cache), c->v_cache_idx = idx(prep.v_cache);
+        c->cos_idx = idx(prep.cos), c->sin_idx = idx(prep.sin);
+        std::vector<std::unique_ptr<CompiledStep>> out;
+        out.push_back(std::move(c));
+        return out;
+    }
+    void execute(Foundry &foundry, TensorBindings &bindings) const { execute_step(*this, foundry, bindings); }
+    const char *name() const { return "FusedQkvKvPrep"; }
+};
+
+inline void CompiledFusedQkvKvPrepStep::execute(Foundry &foundry, const FastBindings &fast, const TensorBindings &bindings,
+                                                const SymbolTable &) const {
+    const FusedQkvStep &s = step->qkv;
+    auto arg = [&](size_t idx, const char *what) { return TensorArg::from_tensor(need(fast, idx, what)); };
+    auto opt = [&](const std::optional<size_t> &idx, const char *what) { return idx ? arg(*idx, what) : TensorArg(); };
+    const TensorArg input = arg(input_idx, "input"), w_q = arg(w_q_idx, "w_q"), w_k = arg(w_k_idx, "w_k"), w_v = arg(w_v_idx, "w_v");
+    const TensorArg gamma = opt(gamma_idx, "gamma"), b_q = opt(bias_q_idx, "bias_q"), b_k = opt(bias_k_idx, "bias_k"), b_v = opt(bias_v_idx, "bias_v");
+    const TensorArg s_q = opt(s_q_idx, "s_q"), s_k = opt(s_k_idx, "s_k"), s_v = opt(s_v_idx, "s_v");
+    const TensorArg q_rot = arg(q_rot_idx, "q_rot"), kc = arg(k_cache_idx, "k_cache"), vc = arg(v_cache_idx, "v_cache");
+    const TensorArg cos = arg(cos_idx, "cos"), sin = arg(sin_idx, "sin");
+    fa_fused_qkv_params p;
+    p.k_dim = s.k_dim.resolve(bindings), p.n_dim = s.n_dim.resolve(bindings), p.n_kv = s.n_kv.resolve(bindings);
+    p.m = std::max<uint32_t>(s.m.resolve(bindings), 1);
+    p.weights_per_block = s.weights_per_block.resolve(bindings), p.layout = (uint32_t)s.layout, p.epsilon = s.rms_eps;
+    const fa_kv_prep_fused_params kp = step->prep.params.resolve(bindings);
+    check(fa_fused_qkv_kv_prep(foundry.ctx(), w_q.c(), s_q.c(), w_k.c(), s_k.c(), w_v.c(), s_v.c(), input.c(), b_q.c(), b_k.c(), b_v.c(),
+                               gamma.c(), &p, q_rot.c(), kc.c(), vc.c(), cos.c(), sin.c(), &kp));
+}
+
 // ---------------------------------------------------------------------------------------------- MatMul
 struct MatMulStep;
 struct CompiledMatMulStep : CompiledStep {

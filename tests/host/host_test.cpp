@@ -557,6 +557,74 @@ static void test_fused_qkv_step(Foundry &foundry, WeightLayout layout, size_t m 
     foundry.synchronize();
 }
 
+// FusedQkv then KvPrepFused as two steps against the pair as one step: q_rot and both caches bit for bit.
+static void test_fused_qkv_kv_prep_step(Foundry &foundry, size_t m, RopeMode mode) {
+    const size_t H = 8, HKV = 2, D = 64, K = 512, N = H * D, NKV = HKV * D, CAP = 96, POS = 11;
+    Rng rng{(uint32_t)(77 + m)};
+    auto x = rng.fill(m * K, 1.0f), gamma = rng.fill(K, 0.5f);
+    for (auto &g : gamma) g = orc_f32_to_f16(orc_f16_to_f32(g) + 1.0f);
+    auto wq = rng.fill(N * K, 0.1f), wk = rng.fill(NKV * K, 0.1f), wv = rng.fill(NKV * K, 0.1f);
+    auto bq = rng.fill(N, 0.1f), bk = rng.fill(NKV, 0.1f), bv = rng.fill(NKV, 0.1f);
+    auto cache0 = rng.fill(HKV * CAP * D, 1.0f);
+    std::vector<orc_f16> cos(CAP * D / 2), sin(cos.size());
+    orc_rope_tables(10000.0f, (uint32_t)D, 0, (uint32_t)CAP, nullptr, cos.data(), sin.data());
+    TensorBindings b;
+    b.set_int_global("i", 0);
+    b.set_int_global("m", m);
+    b.set_int_global("position_offset", POS);
+    b.insert("hidden", foundry.from_host(Dtype::F16, {m, K}, x.data()));
+    b.insert("norm", foundry.from_host(Dtype::F16, {K}, gamma.data()));
+    b.insert("wq", foundry.from_host(Dtype::F16, {N * K}, wq.data()));
+    b.insert("wk", foundry.from_host(Dtype::F16, {NKV * K}, wk.data()));
+    b.insert("wv", foundry.from_host(Dtype::F16, {NKV * K}, wv.data()));
+    b.insert("bq", foundry.from_host(Dtype::F16, {N}, bq.data()));
+    b.insert("bk", foundry.from_host(Dtype::F16, {NKV}, bk.data()));
+    b.insert("bv", foundry.from_host(Dtype::F16, {NKV}, bv.data()));
+    b.insert("q", foundry.zeros(Dtype::F16, {m, N}));
+    b.insert("k", foundry.zeros(Dtype::F16, {m, NKV}));
+    b.insert("v", foundry.zeros(Dtype::F16, {m, NKV}));
+    b.insert("rope_cos", foundry.from_host(Dtype::F16, {CAP, D / 2}, cos.data()));
+    b.insert("rope_sin", foundry.from_host(Dtype::F16, {CAP, D / 2}, sin.data()));
+    for (const char *suffix : {"two", "one"}) {
+        b.insert(std::string("q_rot_") + suffix, foundry.zeros(Dtype::F16, {H, m, D}));
+        b.insert(std::string("k_cache_") + suffix, foundry.from_host(Dtype::F16, {HKV, CAP, D}, cache0.data()));
+        b.insert(std::string("v_cache_") + suffix, foundry.from_host(Dtype::F16, {HKV, CAP, D}, cache0.data()));
+    }
+    FusedQkvStep qkv{"hidden", "wq", "wk", "wv", "q", "k", "v"};
+    qkv.gamma = "norm", qkv.bias_q = "bq", qkv.bias_k = "bk", qkv.bias_v = "bv";
+    qkv.k_dim = (uint32_t)K, qkv.n_dim = (uint32_t)N, qkv.n_kv = (uint32_t)NKV, qkv.m = DynamicU32::var("m"), qkv.layout = WeightLayout::RowMajor;
+    KvPrepFusedStep prep{"q", "k", "v", "q_rot_two", "k_cache_two", "v_cache_two", "rope_cos", "rope_sin", {}};
+    prep.params.d_model = (uint32_t)N, prep.params.kv_dim = (uint32_t)NKV, prep.params.head_dim = (uint32_t)D;
+    prep.params.n_heads = (uint32_t)H, prep.params.n_kv_heads = (uint32_t)HKV, prep.params.group_size = (uint32_t)(H / HKV);
+    prep.params.seq_len = DynamicU32::var("m"), prep.params.position_offset = DynamicU32::var("position_offset");
+    prep.params.max_seq_len = (uint32_t)CAP, prep.params.total_elements = (uint32_t)(H * m * D), prep.params.rope_mode = mode;
+    qkv.execute(foundry, b);
+    prep.execute(foundry, b);
+    FusedQkvKvPrepStep both{qkv, prep};
+    both.qkv.out_q = both.prep.q = "q_unbound", both.qkv.out_k = both.prep.k = "k_unbound", both.qkv.out_v = both.prep.v = "v_unbound";
+    both.prep.q_rot = "q_rot_one", both.prep.k_cache = "k_cache_one", both.prep.v_cache = "v_cache_one";
+    both.execute(foundry, b);
+    foundry.synchronize();
+    for (const char *t : {"q_rot_", "k_cache_", "v_cache_"}) {
+        auto two = foundry.to_host<orc_f16>(*b.get(std::string(t) + "two")), one = foundry.to_host<orc_f16>(*b.get(std::string(t) + "one"));
+        EXPECT(two.size() == one.size() && std::memcmp(two.data(), one.data(), two.size() * 2) == 0);
+    }
+    // and the two-step result is the oracle's KvPrepFused of the device's own projections
+    auto q = foundry.to_host<orc_f16>(*b.get("q")), k = foundry.to_host<orc_f16>(*b.get("k")), v = foundry.to_host<orc_f16>(*b.get("v"));
+    std::vector<orc_f16> q_ref(H * m * D), k_ref = cache0, v_ref = cache0;
+    orc_kv_prep_params p = {(uint32_t)N, (uint32_t)NKV, (uint32_t)D, (uint32_t)H, (uint32_t)HKV, (uint32_t)(H / HKV), (uint32_t)m, (uint32_t)POS,
+                            (uint32_t)CAP, (uint32_t)(H * m * D), (uint32_t)mode, 0, 0};
+    orc_kv_prep_fused(q.data(), k.data(), v.data(), q_ref.data(), k_ref.data(), v_ref.data(), cos.data(), sin.data(), &p);
+    auto q_one = foundry.to_host<orc_f16>(*b.get("q_rot_one")), k_one = foundry.to_host<orc_f16>(*b.get("k_cache_one"));
+    auto v_one = foundry.to_host<orc_f16>(*b.get("v_cache_one"));
+    EXPECT(std::memcmp(q_ref.data(), q_one.data(), q_ref.size() * 2) == 0);
+    EXPECT(std::memcmp(k_ref.data(), k_one.data(), k_ref.size() * 2) == 0);
+    EXPECT(std::memcmp(v_ref.data(), v_one.data(), v_ref.size() * 2) == 0);
+    FusedQkvKvPrepStep mismatched = both;
+    mismatched.prep.q = "something_else";
+    EXPECT(thrown_by([&] { mismatched.execute(foundry, b); }) == MetalError::InvalidOperation);
+}
+
 // The o_proj step of models/llama.json:566-585: MatMul with transpose_b, c = hidden, alpha = beta = 1, bias "zero".
 static void test_matmul_step_o_proj(Foundry &foundry) {
     const size_t K = 512, N = 384;
@@ -614,6 +682,8 @@ int main(int argc, char **argv) {
         run_test("fused qkv step, row-major weights", [&] { test_fused_qkv_step(foundry, WeightLayout::RowMajor); });
         run_test("fused qkv step, canonical weights", [&] { test_fused_qkv_step(foundry, WeightLayout::Canonical); });
         run_test("fused qkv step on a 32-token chunk (GEMM)", [&] { test_fused_qkv_step(foundry, WeightLayout::Canonical, 32); });
+        run_test("fused qkv + kv prep as one step, 48-token chunk, NeoX", [&] { test_fused_qkv_kv_prep_step(foundry, 48, RopeMode::Neox); });
+        run_test("fused qkv + kv prep as one step, 3 rows, adjacent pairs", [&] { test_fused_qkv_kv_prep_step(foundry, 3, RopeMode::Normal); });
         run_test("matmul step as o_proj with residual", [&] { test_matmul_step_o_proj(foundry); });
         run_test("session: chunked prefill, snapshot, decode loop with growth, restore",
                  [&] { test_session_prefill_chunks_decode_loop_growth_snapshot(foundry); });
