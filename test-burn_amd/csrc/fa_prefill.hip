@@ -680,12 +680,22 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         } vop[NV];
 #pragma unroll
         for (int i = 0; i < K_AHEAD; ++i) kop[i] = kpre[i];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.0f;
+        // S_j of the tile's second 32 keys is still in sacc[1]: its weights P_j are made between the MFMAs of the first
+        // chain (which accumulates into sacc[0]), EPS of them per MFMA, before the second chain starts over in sacc[1]
+        constexpr int EPS = 16 / DSTEPS;
+        float psum2[2] = {0.0f, 0.0f};
+        const f16_t zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
         for (int i = 0; i < NS + NV; ++i) {
+            if (i < DSTEPS) {
+#pragma unroll
+                for (int e = i * EPS; e < (i + 1) * EPS; ++e) {
+                    const float w = fast_exp2(fmaf(sacc[1][e], c, -m_run));
+                    psum2[e & 1] += w;
+                    pb[1][e / 8][e % 8] = to_elem<BF16>(w);
+                }
+            }
+            if (i == DSTEPS) l_run += psum2[0] + psum2[1];
             if (i + K_AHEAD < NS) {  // K operand i + K_AHEAD
                 const int t = i + K_AHEAD;
                 kop[t].u = *reinterpret_cast<const uint4 *>(k_lds + (t / DSTEPS) * (2 * RB_BYTES) + (t % DSTEPS) * 512);
@@ -699,8 +709,9 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
             }
             if (i < NS) {
                 const int kb = i / DSTEPS, st = i % DSTEPS;
-                sacc[kb] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop[i].b, qreg[st].b, sacc[kb], 0, 0, 0)
-                                : __builtin_amdgcn_mfma_f32_32x32x16_f16(kop[i].h, qreg[st].h, sacc[kb], 0, 0, 0);
+                const f16_t acc = st == 0 ? zero16 : sacc[kb];  // a chain starts from zero
+                sacc[kb] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(kop[i].b, qreg[st].b, acc, 0, 0, 0)
+                                : __builtin_amdgcn_mfma_f32_32x32x16_f16(kop[i].h, qreg[st].h, acc, 0, 0, 0);
             } else {
                 const int g = (i - NS) / DBLKS, b = (i - NS) % DBLKS, kb = g / 2, ks = g % 2;
                 oacc[b] = BF16 ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf8_t, vop[g * DBLKS + b].h),
@@ -918,17 +929,17 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
 #pragma unroll
                         for (int i = 0; i < 16; ++i) oacc[b][i] *= alpha;
                 }
+                // the weights of the tile's first 32 keys; those of the other 32 are made in the MFMA phase, between the
+                // MFMAs of the first accumulation chain (this phase is the longer of the two)
                 float psum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-                    for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                        for (int jj = 0; jj < 8; ++jj) {
-                            const float e = fast_exp2(fmaf(sacc[kb][8 * ks + jj], c, -m_run));
-                            psum[jj & 3] += e;
-                            pb[kb][ks][jj] = to_elem<BF16>(e);
-                        }
+                    for (int jj = 0; jj < 8; ++jj) {
+                        const float e = fast_exp2(fmaf(sacc[0][8 * ks + jj], c, -m_run));
+                        psum[jj & 3] += e;
+                        pb[0][ks][jj] = to_elem<BF16>(e);
+                    }
                 l_run += (psum[0] + psum[1]) + (psum[2] + psum[3]);
                 k_prefetch((j + 1) & 1);
                 if (j == 0) {  // V_0 has landed: everything but what this phase requested (K_2, V_1)
