@@ -914,7 +914,7 @@ def bench_sage_decode(f, args):
         w = np.exp(s_ - s_.max())
         full[h] = (w / w.sum()) @ vf[h // (H // Hkv)]
     err_full = float(np.max(np.abs(got - full)))
-    # timed as HIP-graph replays (two short launches per step: eager, the host's call overhead would be what is measured)
+    # timed as HIP-graph replays (short launches: eager, the host's call overhead would be what is measured)
     per_graph = 4 * NL
     f.start_capture()
     for i in range(per_graph):
@@ -936,15 +936,17 @@ def bench_sage_decode(f, args):
     for i in range(per_graph):
         step(i)
     n_ap, ms_ap = f.profile_query("sage_append_kernel")
+    one_launch = n_ap == 0  # the default: append and attention in one kernel (FOUNDRY_ATTN_SAGE_FUSED=0: two)
     nbytes = float(Hkv * N * D + Hkv * (N // 32) * 2 + Hkv * N * D * 2 + 2 * H * D * 2)
     _finish_secondary(f, args, "int8-QK decode-attn layer-steps/s + achieved HBM GB/s, SmolLM3 shape @32K ctx",
                       "smollm3 decode step with int8 Q/K (K mean-smoothed with a fixed mean, per-32-token f16 scales; f16 V), one "
                       "layer per step: RoPE (every 4th layer none) + append into the int8 cache + int8 decode, batch 1, "
-                      "H16/Hkv4/D128, kv_len 32768, 1% of entries at 8 sigma", "sage_decode_mfma_kernel",
+                      "H16/Hkv4/D128, kv_len 32768, 1% of entries at 8 sigma" + (", one launch per step" if one_launch else ", two launches per step"),
+                      "sage_fused_append_decode_kernel" if one_launch else "sage_decode_mfma_kernel",
                       nbytes, dt, {"int8_state_bit_exact": state_ok, "max_abs_err_vs_int8_cpu_model": err_model,
                                    "max_abs_err_vs_f16_sdpa_unquantised": err_full},
                       {"dtype": "i8 (QK^T) / f16 (PV)",
-                       "append": {"kernel": "sage_append_kernel", "avg_launch_us": ms_ap * 1e3 / max(1, n_ap)}})
+                       "append": None if one_launch else {"kernel": "sage_append_kernel", "avg_launch_us": ms_ap * 1e3 / max(1, n_ap)}})
     f.profile_enable(False)
 
 

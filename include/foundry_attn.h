@@ -298,9 +298,9 @@ fa_status fa_set_prefill_split_k(fa_ctx *ctx, uint32_t split_k);
 /* Prefill kernel variant, in the spirit of the reference's per-kernel variant overrides
  * (src/metals/flashattention/variants.rs): 1 = K/V tiles staged through registers, one barrier per key tile;
  * 2 = K/V tiles loaded straight into LDS, softmax and MFMA work of the two wave groups alternating in two
- * barrier-separated phases, row sums on the matrix pipe (measured 3 % faster at 2048 tokens, 14 % at 8192 and on
- * a paged cache); 0 (default) = 2. Same contract; variant 2 normalises by the sum of the f16-rounded weights that
- * enter the PV product, variant 1 by the sum of the unrounded ones (outputs agree to one f16 ulp).
+ * barrier-separated phases, resident workgroups that share out the (query tile, head) items (measured 10 % faster at
+ * 2048 tokens, 14 % at 8192 and on a paged cache); 0 (default) = 2. Same contract; the two differ in the order in which
+ * a row's weights are summed (outputs agree to one f16 ulp).
  * Environment: FOUNDRY_ATTN_PREFILL_VARIANT (read at fa_ctx_create). */
 fa_status fa_set_prefill_variant(fa_ctx *ctx, uint32_t variant);
 
@@ -564,7 +564,7 @@ fa_status fa_sage_cache_build(fa_ctx *ctx, const void *k_f16, uint32_t kv_len, c
  * on the way into the cache"): the new token's k is rotated (KvPrepFused arithmetic: rope_mode, the no-RoPE layer rule,
  * one rounding to f16) and appended at row P, v is appended raw, q is rotated, rounded to f16 and quantised per head;
  * then rows [0, P] are attended as in fa_sage_decode. P = *d_position if d_position != NULL (kv_len_bound >= P + 1 as in
- * fa_flash_decode_dyn), else params->position_offset. Two launches.
+ * fa_flash_decode_dyn), else params->position_offset. One launch (fa_set_sage_step_variant).
  * The open block: a block scale covers 32 rows, so a row appended to a partly filled block can change the scale of the
  * rows before it. The block's exact f16 rows are therefore kept in k_tail and the whole block is quantised anew at
  * every append: k_q and k_scale always hold what quantising rows [0, P] from scratch gives. The smoothing mean stays
@@ -579,6 +579,13 @@ fa_status fa_sage_decode_step(fa_ctx *ctx, const fa_tensor_arg *q, const fa_tens
                               const fa_sage_cache *cache, const fa_tensor_arg *cos, const fa_tensor_arg *sin,
                               const fa_tensor_arg *output, const fa_kv_prep_fused_params *params,
                               const uint32_t *d_position, uint32_t kv_len_bound);
+
+/* How fa_sage_decode_step runs: 1 (and 0, the default) = one launch - every workgroup of the decode kernel rotates and
+ * quantises its head group's query, and the workgroup whose partition holds row P quantises the open block anew, stores
+ * it and attends it from the registers it was made in; 2 = an append kernel followed by the decode kernel. Same
+ * int8 state bit for bit; the outputs differ by the order in which partial sums are folded. No counterpart in the reference.
+ * Environment: FOUNDRY_ATTN_SAGE_FUSED = 0 selects 2 (read at fa_ctx_create). */
+fa_status fa_set_sage_step_variant(fa_ctx *ctx, uint32_t variant);
 
 /* ---------------------------------------------------------------------------------------------
  * The un-fused chain around the cache (DSL ops Rope, KvCacheWrite, KvCacheWriteRepeatKvHeads, KvCacheRead, KvRearrange,

@@ -111,6 +111,7 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     if (ctx->gemm_variant > 3) ctx->gemm_variant = 0;
     ctx->prefill_split_k = env_u32("FOUNDRY_ATTN_PREFILL_SPLIT_K", 0);
     ctx->prefill_variant = env_u32("FOUNDRY_ATTN_PREFILL_VARIANT", 0);
+    ctx->sage_fused_step = env_u32("FOUNDRY_ATTN_SAGE_FUSED", 1);
     if (ctx->prefill_variant > 2) ctx->prefill_variant = 0;
     ctx->ledger = new FaGraphLedger();
     fa_status s = fa_ensure_workspace(ctx, (size_t)64 << 20);
@@ -264,6 +265,13 @@ extern "C" fa_status fa_set_gemm_variant(fa_ctx *ctx, uint32_t variant) {
 extern "C" fa_status fa_set_gemm_min_m(fa_ctx *ctx, uint32_t min_m) {
     FA_NEED(ctx, "ctx");
     ctx->gemm_min_m = min_m;
+    return FA_OK;
+}
+
+extern "C" fa_status fa_set_sage_step_variant(fa_ctx *ctx, uint32_t variant) {
+    FA_NEED(ctx, "ctx");
+    if (variant > 2) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "the int8 decode step has variants 0 (default), 1 (one launch) and 2 (two launches), got %u", variant);
+    ctx->sage_fused_step = variant == 2 ? 0u : 1u;
     return FA_OK;
 }
 
@@ -1646,14 +1654,27 @@ extern "C" fa_status fa_sage_decode_step(fa_ctx *ctx, const fa_tensor_arg *q, co
         A.position = p->position_offset, A.bound = p->position_offset + 1;
         L.kv_len = p->position_offset + 1, L.kv_len_bound = L.kv_len;
     }
-    FA_TRY(fa_launch_sage_append(ctx, A));
     const size_t dm = (size_t)c->n_heads * c->head_dim;
-    L.q = c->q_q, L.k = c->k_q, L.v = (const __half *)c->v, L.out = tptr<__half>(output);
+    const bool one_launch = ctx->sage_fused_step != 0 && c->head_dim % 16 == 0;
+    if (one_launch) {
+        // append and attention in one launch: every workgroup rotates and quantises its head group's query, the workgroup
+        // whose partition holds row P quantises the open block anew and attends it from registers
+        L.sage_fused = true, L.fused = true;
+        L.q = A.q, L.k_in = A.k, L.v_in = A.v, L.cos_t = A.cos_t, L.sin_t = A.sin_t;
+        L.qin_stride_b = dm, L.kvin_stride_b = (uint64_t)c->n_kv_heads * c->head_dim;
+        L.rope_normal = A.rope_normal, L.apply_rope = A.apply_rope, L.table_rows = A.table_rows;
+        L.sage_tail = A.tail, L.sage_mean = A.mean, L.q_q_out = A.q_q, L.q_scale_out = A.q_scale;
+        L.q_scale = nullptr;
+    } else {
+        FA_TRY(fa_launch_sage_append(ctx, A));
+        L.q = c->q_q, L.q_scale = c->q_scale;
+    }
+    L.k = c->k_q, L.v = (const __half *)c->v, L.out = tptr<__half>(output);
     L.q_stride_b = dm, L.q_stride_h = c->head_dim, L.out_stride_b = dm, L.out_stride_h = c->head_dim;
     L.k_stride_h = (uint64_t)c->capacity * c->head_dim, L.v_stride_h = (uint64_t)c->capacity * c->head_dim;
     L.n_heads = c->n_heads, L.n_kv_heads = c->n_kv_heads, L.head_dim = c->head_dim, L.batch = 1;
     L.capacity = c->capacity;
     L.scale = 1.0f / sqrtf((float)c->head_dim);
-    L.q_scale = c->q_scale, L.k_scale = (const __half *)c->k_scale, L.ks_stride = ceil_div_u32(c->capacity, FA_SAGE_BLOCK);
+    L.k_scale = (const __half *)c->k_scale, L.ks_stride = ceil_div_u32(c->capacity, FA_SAGE_BLOCK);
     return fa_launch_decode(ctx, L);
 }

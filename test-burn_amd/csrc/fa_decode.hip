@@ -101,6 +101,8 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     }
     if (chunk == 0) chunk = waves == 4 ? auto_chunk(4, 2 * n_cus) : auto_chunk(8, n_cus);
     chunk = (chunk + BK - 1) / BK * BK;
+    // the int8 step in one launch: the open 32-row block must lie inside one partition
+    if (L.sage_fused) chunk = (chunk + FA_SAGE_BLOCK - 1) / FA_SAGE_BLOCK * FA_SAGE_BLOCK;
     const uint32_t S = ceil_div_u32(bound, chunk);
     // a contiguous cache slab is addressed with 32-bit byte offsets (tile base included)
     if (!L.paged && ((uint64_t)L.capacity + chunk + MBX * BK) * L.head_dim * 2 >= (1ull << 32))
@@ -126,6 +128,7 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
     a.qin_stride_b = L.qin_stride_b, a.kvin_stride_b = L.kvin_stride_b, a.qrot_stride_b = L.qrot_stride_b;
     a.rope_normal = L.rope_normal, a.apply_rope = L.apply_rope, a.table_rows = L.table_rows;
     a.status = ctx->d_status;
+    a.sage_tail = L.sage_tail, a.sage_mean = L.sage_mean, a.q_q_out = L.q_q_out, a.q_scale_out = L.q_scale_out;
     // The polled merge needs every workgroup of the launch resident at once (the merging workgroup of a head group
     // occupies its compute unit while it waits) and its partials in the context's pattern-filled buffer.
     bool polled = false;
@@ -172,7 +175,9 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
         }
     }
     int mode = MODE_PLAIN;
-    if (L.q_scale)
+    if (L.sage_fused)
+        mode = MODE_SAGE_FUSED;
+    else if (L.q_scale)
         mode = MODE_SAGE;
     else if (L.fused)
         mode = L.paged ? MODE_FUSED_PAGED : MODE_FUSED;

@@ -75,6 +75,14 @@ union U4H {
     _Float16 e[8];
 };
 
+// The int8 quantiser of fa_sage.hip: rint(x / scale) clamped to +-127, 0 for a zero scale.
+__device__ __forceinline__ int sage_quant_i8(float x, float scale) {
+    if (!(scale > 0.0f)) return 0;
+    float r = rintf(x / scale);
+    r = fminf(fmaxf(r, -127.0f), 127.0f);
+    return (int)r;
+}
+
 constexpr int NW = FA_DECODE_NW;  // waves per workgroup; two per SIMD in all: 8 = one workgroup per CU, 4 = two, at <= 256 VGPRs
 constexpr int NT = NW * 64;  // threads per workgroup
 constexpr int BK = 16;       // keys per block (MFMA M dimension)
@@ -512,7 +520,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     constexpr int DBLK = D / 16;                    // 16-row blocks of O^T
     constexpr int VRS = D * 2 + 32;                 // LDS row stride of the V tile (bank spread for the transpose loads)
     constexpr int KES = SAGE ? 1 : 2;               // K element size in bytes
-    static_assert(!(SAGE && FUSED), "the fused append is f16 only");
+    static_assert(!(SAGE && PAGED), "the int8 variant has a contiguous cache");
     static_assert(!(SAGE && BF16), "the int8 variant keeps V in f16");
     static_assert(KSTEPS * 4 == SEGS, "a K row is KSTEPS x 4 segments");
 
@@ -522,6 +530,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // count is complete instead of meeting the others at a barrier: a wave reaches that point only when all of its
     // block requests have been accepted, which for the last one is most of the launch's streaming time.
     __shared__ uint32_t sm_q_ready;
+    __shared__ float sm_qscale[MAX_GT];  // SAGE + FUSED: the per-head scales of the query quantised in this workgroup
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: tile addresses stay in SGPRs
@@ -703,7 +712,129 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     uint32_t n_raw = 0;
     U4H qraw;
     qraw.u = make_uint4(0, 0, 0, 0);
-    if (FUSED) {
+    // SAGE + FUSED, wave 0's staging area (its own V region, unused until it attends the open block): the raw rows of the
+    // group's query heads and of the new K, their rotated forms, the smoothing mean.
+    __half *st_qraw = reinterpret_cast<__half *>(smem), *st_kraw = st_qraw + MAX_GT * D, *st_qrot = st_kraw + D;
+    __half *st_krot = st_qrot + MAX_GT * D;
+    float *st_mean = reinterpret_cast<float *>(st_krot + D);
+    static_assert(!(SAGE && FUSED) || (2 * MAX_GT * D + 2 * D) * 2 + D * 4 <= MBX * BK * VRS, "staging fits a wave's V region");
+    uint4 sage_vnew = make_uint4(0, 0, 0, 0);
+    if constexpr (SAGE && FUSED) {
+        if (wave == 0) {
+            // As below: the requests that do not depend on the length go out before any other wave may request anything.
+            __builtin_amdgcn_s_setprio(3);
+            constexpr int QV = MAX_GT * D / 8 / 64;  // 16-byte pieces of the group's query rows per lane
+            uint4 qv[QV], kv4 = make_uint4(0, 0, 0, 0), mv4 = make_uint4(0, 0, 0, 0);
+            const __half *qrow = a.q + (size_t)b * a.qin_stride_b + (size_t)head0 * D;
+#pragma unroll
+            for (int i = 0; i < QV; ++i) {
+                const uint32_t e = lane + 64 * i;
+                qv[i] = e < gt * (D / 8) ? *reinterpret_cast<const uint4 *>(qrow + e * 8) : make_uint4(0, 0, 0, 0);
+            }
+            if (lane < D / 8) kv4 = *reinterpret_cast<const uint4 *>(a.k_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D + lane * 8);
+            if (lane < D / 4) mv4 = *reinterpret_cast<const uint4 *>(a.sage_mean + (size_t)kvh * D + lane * 4);
+            sage_vnew = *reinterpret_cast<const uint4 *>(a.v_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D + (lane % VLPR) * 8);
+            if (lane == 0) sm_q_ready = 0;
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();  // releases the streaming waves
+            __builtin_amdgcn_sched_barrier(0);
+            n_raw = read_len();
+            const uint32_t p0 = min(n_raw, min(a.capacity, a.kv_len_bound)) - 1;
+            const bool rope_q = rope_on;
+            if (rope_q) {  // the table row through the scalar cache, as below
+                const uint32_t tp = min(p0, a.table_rows - 1);
+                const __half *ct = a.cos_t + (size_t)tp * (D / 2), *st = a.sin_t + (size_t)tp * (D / 2);
+                if constexpr (D == 128) {
+                    u16_t c0, c1, s0, s1;
+                    asm volatile(
+                        "s_load_dwordx16 %0, %4, 0x0\n\ts_load_dwordx16 %1, %4, 0x40\n\t"
+                        "s_load_dwordx16 %2, %5, 0x0\n\ts_load_dwordx16 %3, %5, 0x40\n\ts_waitcnt lgkmcnt(0)"
+                        : "=&s"(c0), "=&s"(c1), "=&s"(s0), "=&s"(s1)
+                        : "s"(ct), "s"(st)
+                        : "memory");
+                    if (lane == 0) {
+                        u16_t *dst = reinterpret_cast<u16_t *>(rope_lds);
+                        dst[0] = c0, dst[1] = c1, dst[2] = s0, dst[3] = s1;
+                    }
+                } else {
+                    u16_t c0, s0;
+                    asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                                 : "=&s"(c0), "=&s"(s0)
+                                 : "s"(ct), "s"(st)
+                                 : "memory");
+                    if (lane == 0) {
+                        u16_t *dst = reinterpret_cast<u16_t *>(rope_lds);
+                        dst[0] = c0, dst[1] = s0;
+                    }
+                }
+            }
+            // raw rows and the mean into the staging area
+#pragma unroll
+            for (int i = 0; i < QV; ++i) {
+                const uint32_t e = lane + 64 * i;
+                if (e < gt * (D / 8)) *reinterpret_cast<uint4 *>(st_qraw + e * 8) = qv[i];
+            }
+            if (lane < D / 8) *reinterpret_cast<uint4 *>(st_kraw + lane * 8) = kv4;
+            if (lane < D / 4) *reinterpret_cast<uint4 *>(st_mean + lane * 4) = mv4;
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+            __builtin_amdgcn_wave_barrier();  // LDS executes a wave's accesses in order
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+            // Rotation, one element at a time with the arithmetic of the append kernel (products and sum rounded
+            // separately, one rounding to f16: kv_prep_fused.metal:66-82)
+            const __half *cosr = reinterpret_cast<const __half *>(rope_lds), *sinr = cosr + D / 2;
+            auto rotate = [&](const __half *row, uint32_t d) -> __half {
+#pragma clang fp contract(off)
+                if (!rope_on) return row[d];
+                constexpr uint32_t half = D / 2;
+                const uint32_t pair = rope_normal ? (d >> 1) : (d < half ? d : d - half);
+                const bool first = rope_normal ? ((d & 1u) == 0u) : (d < half);
+                const uint32_t mate = rope_normal ? (first ? d + 1 : d - 1) : (first ? d + half : d - half);
+                const float cc = __half2float(cosr[pair]), sn = __half2float(sinr[pair]);
+                const float p0f = __half2float(row[d]) * cc, p1f = __half2float(row[mate]) * sn;
+                return __float2half_rn(first ? p0f - p1f : p0f + p1f);
+            };
+            for (uint32_t e = lane; e < gt * D; e += 64) st_qrot[e] = rotate(st_qraw + (e / D) * D, e % D);
+            for (uint32_t d = lane; d < (uint32_t)D; d += 64) st_krot[d] = rotate(st_kraw, d);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+            // The query operand: lane (n, c) of step j holds int8 segment 4j + c (16 values) of head n, quantised with
+            // the head's own scale max|q| / 127 (f32), as sage_append_kernel does it.
+            float qx[KSTEPS][16];
+            float amax = 0.0f;
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    qx[j][i] = head_ok ? __half2float(st_qrot[n * D + (4 * j + c) * 16 + i]) : 0.0f;
+                    amax = fmaxf(amax, fabsf(qx[j][i]));
+                }
+            amax = fmaxf(amax, xor16(amax));
+            amax = fmaxf(amax, xor32(amax));
+            const float qs = amax / 127.0f;
+#pragma unroll
+            for (int j = 0; j < KSTEPS; ++j) {
+                union {
+                    uint4 u;
+                    int8_t e[16];
+                } o;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o.e[i] = (int8_t)sage_quant_i8(qx[j][i], qs);
+                q_lds[j * 64 + lane] = o.u;
+                if (head_ok && split == 0 && a.q_q_out)
+                    *reinterpret_cast<uint4 *>(a.q_q_out + (size_t)(head0 + n) * D + (4 * j + c) * 16) = o.u;
+            }
+            if (head_ok && c == 0) {
+                sm_qscale[n] = qs;
+                if (split == 0 && a.q_scale_out) a.q_scale_out[head0 + n] = qs;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+            if (lane == 0) __hip_atomic_store(&sm_q_ready, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __builtin_amdgcn_s_setprio(0);
+        } else {
+            __syncthreads();  // wave 0 has queued its requests
+        }
+    } else if (FUSED) {
         if (wave == 0) {
             // First everything that does not depend on the length: the raw query rows and the new token's
             // raw K / V row (parked in the block registers that this wave does not otherwise use). All lanes load
@@ -820,7 +951,8 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // cache rows of its partition end before it, and it is attended as a one-key block of its own.
     const uint32_t p = N - 1;
     const bool owns_new = FUSED && n_raw == N && p >= k0 && p < k1;
-    const uint32_t kend = owns_new ? k1 - 1 : k1;
+    // (int8: the whole open 32-row block is left to wave 0, which quantises it anew; partitions are multiples of 32 rows)
+    const uint32_t kend = owns_new ? (SAGE ? (p & ~(uint32_t)(FA_SAGE_BLOCK - 1)) : k1 - 1) : k1;
     const uint32_t wbe = min(wb1, (kend - k0 + BK - 1) / BK);  // this wave's blocks that hold a valid key end here
     if (PAGED && cur < wbe) {
         const uint32_t m = min((uint32_t)MBX, wbe - cur);
@@ -834,6 +966,8 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         while (__hip_atomic_load(&sm_q_ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < Q_PARTS) __builtin_amdgcn_s_sleep(1);
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     }
+    if (SAGE && FUSED && head_ok) qsc = sm_qscale[n] * a.scale_log2e;
+    float ks_open = -1.0f;  // SAGE + FUSED: the scale of the open block while wave 0 attends it from registers
 
     f4_t oacc[DBLK];
 #pragma unroll
@@ -861,7 +995,8 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                         si = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk[mb][j].i, q_op(j).i, si, 0, 0, 0);
                     // a block lies inside one 32-key scale block
                     const uint32_t key = min(tbase + BK * mb, kend - 1);
-                    const float ks = __half2float(a.k_scale[(size_t)kvh * a.ks_stride + key / FA_SAGE_BLOCK]);
+                    const float ks = (FUSED && ks_open >= 0.0f) ? ks_open
+                                                                : __half2float(a.k_scale[(size_t)kvh * a.ks_stride + key / FA_SAGE_BLOCK]);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) s[mb * 4 + i] = (float)si[i] * (qsc * ks);
                 } else {
@@ -957,7 +1092,84 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         cur = nblk;
     }
 
-    if (FUSED && owns_new && wave == 0) {
+    if constexpr (SAGE && FUSED) {
+        if (owns_new && wave == 0) {
+            // The open block, rows b0 .. p: its earlier rows are exact in the tail, the new row is in the staging area.
+            // All of them are quantised anew (a block has one scale, and the new row may raise it), stored, and attended
+            // from the registers they were made in; rows past p carry no weight.
+            const bool writer = y % a.sub_per_kv == 0;
+            const uint32_t r = p & (FA_SAGE_BLOCK - 1), b0 = p - r, nsb = r / BK + 1;
+            __half *tail = a.sage_tail + (size_t)kvh * FA_SAGE_BLOCK * D;
+            // V rows of the block (the new row is patched in below)
+            issue_v((b0 - k0) / BK, nsb, 0);
+            float kx[2][KSTEPS][16];
+            float amax = 0.0f;
+#pragma unroll
+            for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+                for (int j = 0; j < KSTEPS; ++j) {
+                    const uint32_t row = sb * BK + n, col = (4 * j + c) * 16;
+                    U4H t0, t1;
+                    t0.u = make_uint4(0, 0, 0, 0), t1.u = t0.u;
+                    if (row < r) {
+                        t0.u = *reinterpret_cast<const uint4 *>(tail + (size_t)row * D + col);
+                        t1.u = *reinterpret_cast<const uint4 *>(tail + (size_t)row * D + col + 8);
+                    } else if (row == r) {
+                        t0.u = *reinterpret_cast<const uint4 *>(st_krot + col);
+                        t1.u = *reinterpret_cast<const uint4 *>(st_krot + col + 8);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const float v = (float)(i < 8 ? t0.e[i] : t1.e[i - 8]) - st_mean[col + i];
+                        kx[sb][j][i] = row <= r ? v : 0.0f;
+                        amax = fmaxf(amax, fabsf(kx[sb][j][i]));
+                    }
+                }
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+            const __half sc16 = __float2half_rn(amax / 127.0f);
+            const float sc = __half2float(sc16);
+            int8_t *kq = const_cast<int8_t *>(reinterpret_cast<const int8_t *>(kbase)) + (size_t)b0 * D;
+#pragma unroll
+            for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+                for (int j = 0; j < KSTEPS; ++j) {
+                    union {
+                        uint4 u;
+                        int8_t e[16];
+                    } o;
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) o.e[i] = (int8_t)sage_quant_i8(kx[sb][j][i], sc);
+                    kk[sb][j].u = o.u;
+                }
+            // the new V row into its place among the block's rows (load i holds rows i VRPL .. of a 16-row block)
+            {
+                const uint32_t rr = r % BK, sbn = r / BK;
+#pragma unroll
+                for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+                    for (int i = 0; i < VLB; ++i)
+                        if ((uint32_t)sb == sbn && (uint32_t)(i * VRPL + lane / VLPR) == rr) vv[sb][i].u = sage_vnew;
+            }
+            // (the V blocks go through this wave's LDS region, which is the staging area: take the rotated row out first)
+            const uint4 krot16 = *reinterpret_cast<const uint4 *>(st_krot + (lane % (D / 8)) * 8);
+            ks_open = sc;
+            consume(b0, nsb, p + 1, 0, 0);
+            ks_open = -1.0f;
+            __builtin_amdgcn_sched_barrier(0);
+            if (writer) {  // after the block has been attended (see below): the int8 rows, the scale, the tail row, the V row
+#pragma unroll
+                for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+                    for (int j = 0; j < KSTEPS; ++j)
+                        if ((uint32_t)(sb * BK + n) <= r)
+                            *reinterpret_cast<uint4 *>(kq + (size_t)(sb * BK + n) * D + (4 * j + c) * 16) = kk[sb][j].u;
+                if (lane == 0) const_cast<__half *>(a.k_scale)[(size_t)kvh * a.ks_stride + b0 / FA_SAGE_BLOCK] = sc16;
+                if (lane < D / 8) *reinterpret_cast<uint4 *>(tail + (size_t)r * D + lane * 8) = krot16;
+                if (lane < VLPR) *reinterpret_cast<uint4 *>(const_cast<__half *>(vbase) + (size_t)p * D + lane * 8) = sage_vnew;
+            }
+        }
+    } else if (FUSED && owns_new && wave == 0) {
         // The new row is not in the cache: rotate K / copy V from the raw projections (kv_prep_fused.metal:89-122),
         // attend it as a block whose only valid key is row 0, and let one workgroup of the KV head store it.
         const bool writer = y % a.sub_per_kv == 0;
@@ -1116,7 +1328,7 @@ __global__ void __launch_bounds__(NT_MERGE) flash_decode_merge_kernel(DecodeDev 
     merge_and_store<D, false, NT_MERGE>(a, b, y, nsplits, S, threadIdx.x, sm, (int)blockIdx.x, 1);
 }
 
-enum Mode { MODE_PLAIN = 0, MODE_PAGED = 1, MODE_SAGE = 2, MODE_FUSED = 3, MODE_FUSED_PAGED = 4 };
+enum Mode { MODE_PLAIN = 0, MODE_PAGED = 1, MODE_SAGE = 2, MODE_FUSED = 3, MODE_FUSED_PAGED = 4, MODE_SAGE_FUSED = 5 };
 
 // Dynamic LDS: the per-wave V tiles during the main loop, then the wave fold / the partition merge.
 template <int D>
@@ -1143,6 +1355,7 @@ fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, true, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
+            FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, true, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, false, false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
@@ -1153,7 +1366,8 @@ fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
         }
     }
     {
-        const char *name = mode == MODE_SAGE ? "sage_decode_mfma_kernel"
+        const char *name = mode == MODE_SAGE_FUSED ? "sage_fused_append_decode_kernel"
+                           : mode == MODE_SAGE ? "sage_decode_mfma_kernel"
                            : (mode == MODE_FUSED || mode == MODE_FUSED_PAGED) ? "fused_rope_append_decode_kernel"
                                                                               : "flash_decode_mfma_kernel";
         FaLaunchScope scope(ctx, name, true);
@@ -1172,6 +1386,9 @@ fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
                 break;
             case MODE_SAGE:
                 scope.launch((flash_decode_mfma_kernel<D, false, true, false>), grid, dim3(NT), lds, a);
+                break;
+            case MODE_SAGE_FUSED:
+                scope.launch((flash_decode_mfma_kernel<D, false, true, true>), grid, dim3(NT), lds, a);
                 break;
             case MODE_FUSED:
                 if (a.bf16)

@@ -63,6 +63,7 @@ struct fa_ctx {
     uint32_t gemm_variant = 0;     // GEMM kernel: 0 = auto, 1 = tiles through registers, 2 / 3 = straight into LDS in steps of 64 / 32 features
     uint32_t gemm_min_m = 0;       // FusedQkv / MatMul: input rows from which the GEMM runs (0 = default)
     uint32_t prefill_split_k = 0;  // 0 = auto
+    uint32_t sage_fused_step = 1;  // the int8 decode step as one launch (env FOUNDRY_ATTN_SAGE_FUSED=0: append kernel + decode kernel)
     uint32_t prefill_variant = 0;  // 0 = auto, 1 = tiles staged through registers, 2 = tiles straight into LDS, two-phase loop
     // optional: the prefill kernel leaves {shader-clock ticks, wall ticks} per workgroup here (fa_profile_clock_buffer)
     unsigned long long *clock_buf = nullptr;
@@ -167,6 +168,12 @@ struct DecodeLaunch {
     uint32_t rope_normal, apply_rope, table_rows;
     bool bf16;  // q, k, v, caches and out are bf16 instead of f16 (not with the int8 variant)
     bool static_scratch;  // partials go to the library's static device array; nothing may be allocated
+    // int8 step in one launch (fused, q_scale == nullptr, k = the int8 cache, k_scale written): see FaDecodeDev
+    bool sage_fused;
+    __half *sage_tail;
+    const float *sage_mean;
+    int8_t *q_q_out;
+    float *q_scale_out;
 };
 fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &a);
 
@@ -197,6 +204,12 @@ struct FaDecodeDev {
     uint32_t *status;  // the context's device-written status word (FA_DEVSTAT_* bits)
     uint32_t xcd_local;  // polled merge: a head group's workgroups share an XCD and exchange partials through its L2
     unsigned long long poll_ticks;  // polled merge: how long the merging workgroup waits for partials, 100 MHz ticks
+    // SAGE + FUSED (the int8 decode step in one launch): q is the raw f16 projection, k the int8 cache (written: the open
+    // block's rows), k_scale is written too; the exact rows of the open block, the smoothing mean, the step's quantised query
+    __half *sage_tail;       // [Hkv, 32, D]
+    const float *sage_mean;  // [Hkv, D]
+    int8_t *q_q_out;         // [H, D]
+    float *q_scale_out;      // [H]
 };
 
 

@@ -128,6 +128,7 @@ PROTOTYPES = {
     "fa_set_decode_variant": [_vp, C.POINTER(DecodeVariant)],
     "fa_set_prefill_split_k": [_vp, C.c_uint32],
     "fa_set_prefill_variant": [_vp, C.c_uint32],
+    "fa_set_sage_step_variant": [_vp, C.c_uint32],
     "fa_set_gemm_min_m": [_vp, C.c_uint32],
     "fa_set_gemm_variant": [_vp, C.c_uint32],
     "fa_kv_prep_fused_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _u32, _PT, _PT,
@@ -511,6 +512,10 @@ class Foundry:
 
     def sage_cache_build(self, k_f16, kv_len, cache):
         check(self.lib.fa_sage_cache_build(self.h, k_f16.ptr, kv_len, C.byref(cache)))
+
+    def set_sage_step_variant(self, variant=0):
+        """1 (default) = the int8 decode step as one launch, 2 = append kernel + decode kernel."""
+        check(self.lib.fa_set_sage_step_variant(self.h, variant))
 
     def sage_decode_step(self, q, k, v, cache, cos, sin, out, params, d_position=None, kv_len_bound=0):
         check(self.lib.fa_sage_decode_step(self.h, C.byref(q), C.byref(k), C.byref(v), C.byref(cache), C.byref(cos),

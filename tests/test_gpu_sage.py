@@ -87,19 +87,21 @@ def test_sage_incremental_block_quantisation_and_errors():
     f.synchronize()
 
 
+@pytest.mark.parametrize("launches", [1, 2], ids=["one_launch", "two_launches"])
 @pytest.mark.parametrize("H,Hkv,D,start,cap,steps,mode,layer,nope_step,dyn", [
     (16, 4, 128, 90, 256, 40, fa.ROPE_NEOX, 0, 0, False),    # crosses the block boundaries at 96 and 128
     (14, 2, 64, 64, 160, 34, fa.ROPE_NORMAL, 0, 0, True),    # starts on an empty open block, device-side position
     (16, 4, 128, 37, 128, 6, fa.ROPE_NEOX, 3, 4, False),     # layer 3 of a model with every 4th layer un-rotated
     (16, 4, 128, 32760, 32800, 12, fa.ROPE_NEOX, 0, 0, True)])  # SmolLM3 shape around the full 32K context
-def test_sage_decode_step_over_consecutive_tokens(H, Hkv, D, start, cap, steps, mode, layer, nope_step, dyn):
+def test_sage_decode_step_over_consecutive_tokens(H, Hkv, D, start, cap, steps, mode, layer, nope_step, dyn, launches):
     """fa_sage_decode_step: RoPE + append into the int8 cache (open block quantised anew from its exact rows, fixed
     mean) + int8 decode, over consecutive positions. After every step the int8 rows and scales must be bit for bit what
     the oracle's quantiser gives for the oracle's rotated f16 cache with the same mean, the V rows and the quantised
     query bit-exact, and the output within tolerance of the oracle's int8 model; the error against f16 SDPA on the
     unquantised cache is measured."""
-    announce("sage decode step", H, Hkv, D, start, cap, steps, mode, layer, nope_step, dyn)
+    announce("sage decode step", H, Hkv, D, start, cap, steps, mode, layer, nope_step, dyn, launches)
     f = ctx()
+    f.set_sage_step_variant(launches)
     rng = np.random.default_rng(start + cap + D)
     cos, sin = fa.rope_tables(1e6, D, cap)
     kc, vc = np.zeros((Hkv, cap, D), np.float16), np.zeros((Hkv, cap, D), np.float16)
@@ -147,6 +149,7 @@ def test_sage_decode_step_over_consecutive_tokens(H, Hkv, D, start, cap, steps, 
             worst_full = max(worst_full, max_abs(got, full))
         for b in (dq, dkn, dvn):
             b.free()
+    f.set_sage_step_variant()
     print("sage decode step: max abs err vs int8 model (relative to max(1, |out|)) %.2e, vs f16 sdpa %.4f" % (worst_model, worst_full), flush=True)
     assert worst_model <= 2e-3
     assert worst_full <= 0.2
