@@ -583,6 +583,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // ahead (`pgn`), and the rows are addressed as page base (SGPRs) + the same lane offset. Rows of the page past
     // the sequence end exist, so nothing needs a clamp there either.
     U4H kk[MBX][KSTEPS], vv[MBX][VLB];
+    _Float16 ksr[MBX] = {};  // int8: the scale of each block in flight, requested with the block (a block lies inside one 32-key scale block)
     typedef const int32_t __attribute__((address_space(4))) *const_i32p;
     const const_i32p btc = (const_i32p)bt;
     int32_t pgi[MBX] = {}, pgn[MBX] = {};  // page ids of the round being requested / of the one after
@@ -612,6 +613,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         for (int mb = 0; mb < MBX; ++mb) {
             if ((uint32_t)mb >= m) break;
             const uint32_t row0 = k0 + (blk + mb) * BK;
+            if (SAGE) ksr[mb] = reinterpret_cast<const _Float16 *>(a.k_scale)[(size_t)kvh * a.ks_stride + row0 / FA_SAGE_BLOCK];
             if (!PAGED) {
 #pragma unroll
                 for (int j = 0; j < KSTEPS; ++j)
@@ -712,12 +714,12 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     uint32_t n_raw = 0;
     U4H qraw;
     qraw.u = make_uint4(0, 0, 0, 0);
-    // SAGE + FUSED, wave 0's staging area (its own V region, unused until it attends the open block): the raw rows of the
-    // group's query heads and of the new K, their rotated forms, the smoothing mean.
-    __half *st_qraw = reinterpret_cast<__half *>(smem), *st_kraw = st_qraw + MAX_GT * D, *st_qrot = st_kraw + D;
-    __half *st_krot = st_qrot + MAX_GT * D;
+    // SAGE + FUSED, wave 0's staging area (its own V region, unused until it attends the open block): the quantised rows
+    // of the group's query heads, the rotated new K row, the smoothing mean.
+    __half *st_qraw = reinterpret_cast<__half *>(smem);  // int8 [MAX_GT][D]
+    __half *st_krot = st_qraw + MAX_GT * D / 2;
     float *st_mean = reinterpret_cast<float *>(st_krot + D);
-    static_assert(!(SAGE && FUSED) || (2 * MAX_GT * D + 2 * D) * 2 + D * 4 <= MBX * BK * VRS, "staging fits a wave's V region");
+    static_assert(!(SAGE && FUSED) || MAX_GT * D + D * 2 + D * 4 <= MBX * BK * VRS, "staging fits a wave's V region");
     uint4 sage_vnew = make_uint4(0, 0, 0, 0);
     if constexpr (SAGE && FUSED) {
         if (wave == 0) {
@@ -768,66 +770,69 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                     }
                 }
             }
-            // raw rows and the mean into the staging area
+            if (lane < D / 4) *reinterpret_cast<uint4 *>(st_mean + lane * 4) = mv4;
+            __builtin_amdgcn_wave_barrier();  // LDS executes a wave's accesses in order: the table row is there
+            // Rotation in the layout the rows were fetched in: lane l holds piece l % (D / 8) (8 dims) of row l / (D / 8)
+            // (+ 64 i / (D / 8)); a NeoX mate piece is D / 16 lanes away. Arithmetic of the append kernel (rope8: products
+            // and sum rounded separately, one rounding to f16: kv_prep_fused.metal:66-82).
+            constexpr int PPR = D / 8;  // pieces per row
+            const int sgm = lane % PPR;
+            auto rotate_piece = [&](const uint4 raw) -> uint4 {
+                if (!rope_on) return raw;
+                U4H x, mate, cu, su;
+                x.u = raw;
+                const unsigned char *cp = rope_lds, *sp = rope_lds + D;
+                if (rope_normal) {
+                    const uint2 c4 = *reinterpret_cast<const uint2 *>(cp + sgm * 8), s4 = *reinterpret_cast<const uint2 *>(sp + sgm * 8);
+                    cu.u = make_uint4(c4.x, c4.y, 0, 0), su.u = make_uint4(s4.x, s4.y, 0, 0);
+                    return rope8(x, x, cu, su, true, true, false).u;
+                }
+                mate.u = make_uint4(__shfl_xor(raw.x, PPR / 2), __shfl_xor(raw.y, PPR / 2), __shfl_xor(raw.z, PPR / 2), __shfl_xor(raw.w, PPR / 2));
+                const int pc = sgm % (PPR / 2);
+                cu.u = *reinterpret_cast<const uint4 *>(cp + pc * 16), su.u = *reinterpret_cast<const uint4 *>(sp + pc * 16);
+                return rope8(x, mate, cu, su, false, sgm < PPR / 2, false).u;
+            };
+            // the new K row (lanes 0 .. D/8 - 1 hold it; the others rotate zeros along so that the exchange is uniform)
+            {
+                const uint4 kr = rotate_piece(kv4);
+                if (lane < PPR) *reinterpret_cast<uint4 *>(st_krot + lane * 8) = kr;
+            }
+            // The query: rotated, then quantised per head with the head's own scale max|q| / 127 (f32), as
+            // sage_append_kernel does it - here 8 values per lane (the operand layout would make every lane divide 16
+            // KSTEPS values, most of them for heads the group does not have) - and handed over as int8 rows in LDS.
+            int8_t *st_q8 = reinterpret_cast<int8_t *>(st_qraw);
 #pragma unroll
             for (int i = 0; i < QV; ++i) {
-                const uint32_t e = lane + 64 * i;
-                if (e < gt * (D / 8)) *reinterpret_cast<uint4 *>(st_qraw + e * 8) = qv[i];
+                if ((uint32_t)(64 * i) >= gt * PPR) break;  // uniform: no rows left
+                const uint32_t e = lane + 64 * i, row = e / PPR;
+                U4H o;
+                o.u = rotate_piece(qv[i]);
+                float amax = 0.0f;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) amax = fmaxf(amax, fabsf((float)o.e[t]));
+#pragma unroll
+                for (int off = 1; off < PPR; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+                const float qs = amax / 127.0f;
+                union {
+                    uint2 u;
+                    int8_t b[8];
+                } q8;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) q8.b[t] = (int8_t)sage_quant_i8((float)o.e[t], qs);
+                if (row < gt) {
+                    *reinterpret_cast<uint2 *>(st_q8 + row * D + sgm * 8) = q8.u;
+                    if (sgm == 0) sm_qscale[row] = qs;
+                    if (split == 0 && a.q_q_out) *reinterpret_cast<uint2 *>(a.q_q_out + (size_t)(head0 + row) * D + sgm * 8) = q8.u;
+                    if (split == 0 && sgm == 0 && a.q_scale_out) a.q_scale_out[head0 + row] = qs;
+                }
             }
-            if (lane < D / 8) *reinterpret_cast<uint4 *>(st_kraw + lane * 8) = kv4;
-            if (lane < D / 4) *reinterpret_cast<uint4 *>(st_mean + lane * 4) = mv4;
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
-            __builtin_amdgcn_wave_barrier();  // LDS executes a wave's accesses in order
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-            // Rotation, one element at a time with the arithmetic of the append kernel (products and sum rounded
-            // separately, one rounding to f16: kv_prep_fused.metal:66-82)
-            const __half *cosr = reinterpret_cast<const __half *>(rope_lds), *sinr = cosr + D / 2;
-            auto rotate = [&](const __half *row, uint32_t d) -> __half {
-#pragma clang fp contract(off)
-                if (!rope_on) return row[d];
-                constexpr uint32_t half = D / 2;
-                const uint32_t pair = rope_normal ? (d >> 1) : (d < half ? d : d - half);
-                const bool first = rope_normal ? ((d & 1u) == 0u) : (d < half);
-                const uint32_t mate = rope_normal ? (first ? d + 1 : d - 1) : (first ? d + half : d - half);
-                const float cc = __half2float(cosr[pair]), sn = __half2float(sinr[pair]);
-                const float p0f = __half2float(row[d]) * cc, p1f = __half2float(row[mate]) * sn;
-                return __float2half_rn(first ? p0f - p1f : p0f + p1f);
-            };
-            for (uint32_t e = lane; e < gt * D; e += 64) st_qrot[e] = rotate(st_qraw + (e / D) * D, e % D);
-            for (uint32_t d = lane; d < (uint32_t)D; d += 64) st_krot[d] = rotate(st_kraw, d);
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
-            // The query operand: lane (n, c) of step j holds int8 segment 4j + c (16 values) of head n, quantised with
-            // the head's own scale max|q| / 127 (f32), as sage_append_kernel does it.
-            float qx[KSTEPS][16];
-            float amax = 0.0f;
+            // the operand: lane (n, c) of step j holds int8 segment 4j + c (16 values) of head n
 #pragma unroll
             for (int j = 0; j < KSTEPS; ++j)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    qx[j][i] = head_ok ? __half2float(st_qrot[n * D + (4 * j + c) * 16 + i]) : 0.0f;
-                    amax = fmaxf(amax, fabsf(qx[j][i]));
-                }
-            amax = fmaxf(amax, xor16(amax));
-            amax = fmaxf(amax, xor32(amax));
-            const float qs = amax / 127.0f;
-#pragma unroll
-            for (int j = 0; j < KSTEPS; ++j) {
-                union {
-                    uint4 u;
-                    int8_t e[16];
-                } o;
-#pragma unroll
-                for (int i = 0; i < 16; ++i) o.e[i] = (int8_t)sage_quant_i8(qx[j][i], qs);
-                q_lds[j * 64 + lane] = o.u;
-                if (head_ok && split == 0 && a.q_q_out)
-                    *reinterpret_cast<uint4 *>(a.q_q_out + (size_t)(head0 + n) * D + (4 * j + c) * 16) = o.u;
-            }
-            if (head_ok && c == 0) {
-                sm_qscale[n] = qs;
-                if (split == 0 && a.q_scale_out) a.q_scale_out[head0 + n] = qs;
-            }
+                q_lds[j * 64 + lane] = head_ok ? *reinterpret_cast<const uint4 *>(st_q8 + n * D + (4 * j + c) * 16) : make_uint4(0, 0, 0, 0);
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
             if (lane == 0) __hip_atomic_store(&sm_q_ready, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             __builtin_amdgcn_s_setprio(0);
@@ -967,7 +972,6 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     }
     if (SAGE && FUSED && head_ok) qsc = sm_qscale[n] * a.scale_log2e;
-    float ks_open = -1.0f;  // SAGE + FUSED: the scale of the open block while wave 0 attends it from registers
 
     f4_t oacc[DBLK];
 #pragma unroll
@@ -993,10 +997,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
 #pragma unroll
                     for (int j = 0; j < KSTEPS; ++j)
                         si = __builtin_amdgcn_mfma_i32_16x16x64_i8(kk[mb][j].i, q_op(j).i, si, 0, 0, 0);
-                    // a block lies inside one 32-key scale block
-                    const uint32_t key = min(tbase + BK * mb, kend - 1);
-                    const float ks = (FUSED && ks_open >= 0.0f) ? ks_open
-                                                                : __half2float(a.k_scale[(size_t)kvh * a.ks_stride + key / FA_SAGE_BLOCK]);
+                    const float ks = (float)ksr[mb];
 #pragma unroll
                     for (int i = 0; i < 4; ++i) s[mb * 4 + i] = (float)si[i] * (qsc * ks);
                 } else {
@@ -1153,9 +1154,8 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             }
             // (the V blocks go through this wave's LDS region, which is the staging area: take the rotated row out first)
             const uint4 krot16 = *reinterpret_cast<const uint4 *>(st_krot + (lane % (D / 8)) * 8);
-            ks_open = sc;
+            ksr[0] = ksr[1] = (_Float16)sc16;
             consume(b0, nsb, p + 1, 0, 0);
-            ks_open = -1.0f;
             __builtin_amdgcn_sched_barrier(0);
             if (writer) {  // after the block has been attended (see below): the int8 rows, the scale, the tail row, the V row
 #pragma unroll
