@@ -92,7 +92,8 @@ def test_sage_incremental_block_quantisation_and_errors():
     (16, 4, 128, 90, 256, 40, fa.ROPE_NEOX, 0, 0, False),    # crosses the block boundaries at 96 and 128
     (14, 2, 64, 64, 160, 34, fa.ROPE_NORMAL, 0, 0, True),    # starts on an empty open block, device-side position
     (16, 4, 128, 37, 128, 6, fa.ROPE_NEOX, 3, 4, False),     # layer 3 of a model with every 4th layer un-rotated
-    (16, 4, 128, 32760, 32800, 12, fa.ROPE_NEOX, 0, 0, True)])  # SmolLM3 shape around the full 32K context
+    (16, 4, 128, 32760, 32800, 12, fa.ROPE_NEOX, 0, 0, True),   # SmolLM3 shape around the full 32K context
+    (32, 8, 128, 49980, 50016, 5, fa.ROPE_NORMAL, 0, 0, True)])  # more partitions than compute units: 4-wave workgroups, merge kernel
 def test_sage_decode_step_over_consecutive_tokens(H, Hkv, D, start, cap, steps, mode, layer, nope_step, dyn, launches):
     """fa_sage_decode_step: RoPE + append into the int8 cache (open block quantised anew from its exact rows, fixed
     mean) + int8 decode, over consecutive positions. After every step the int8 rows and scales must be bit for bit what
