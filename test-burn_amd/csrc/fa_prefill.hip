@@ -1006,9 +1006,13 @@ __global__ void __launch_bounds__(256) flash_prefill_merge_kernel(PrefillDev a) 
     if (q_row >= a.q_len) return;
     const size_t base = (((size_t)head * n_qt + q_tile) * S) * BM + r;
     float mstar = -1e30f;
-    for (uint32_t s = 0; s < S; ++s) {
-        const float *ml = a.part_ml + (base + (size_t)s * BM) * 2;
-        if (ml[1] > 0.0f) mstar = fmaxf(mstar, ml[0]);
+    for (uint32_t s0 = 0; s0 < S; s0 += PB) {  // PB loads in flight (one after the other they cost a memory latency each)
+        float2 ml[PB];
+#pragma unroll
+        for (int k = 0; k < PB; ++k) ml[k] = *reinterpret_cast<const float2 *>(a.part_ml + (base + (size_t)min(s0 + k, S - 1) * BM) * 2);
+#pragma unroll
+        for (int k = 0; k < PB; ++k)
+            if (s0 + k < S && ml[k].y > 0.0f) mstar = fmaxf(mstar, ml[k].x);
     }
     float L = 0.0f;
     float4 o = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
