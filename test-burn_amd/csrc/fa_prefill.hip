@@ -52,7 +52,13 @@ struct PrefillDev {
     uint32_t splits;             // > 1: the key tiles of a query tile are divided over `splits` items
     uint32_t n_qt, n_items, n_workgroups;  // query tiles; (query tile, head, split) items; workgroups that share them out
     uint32_t pool_bytes32;       // paged: size of each pool when below 4 GiB (whole pages then go by a 32-bit offset), else 0
-    float *part_acc, *part_ml;   // [head][query tile][split][BM][D] unnormalised sums, [..][BM][2] (max, sum)
+    // A chunk of at most 32 query rows (the reference's default prefill chunk): the four 32-row blocks of an item are the
+    // rows of up to four query heads of one KV group instead of 128 rows of one head (three quarters of which would be
+    // empty), so the group's heads share every K/V tile. pack_heads = heads per item (0 = off), pack_blocks = such
+    // items per KV head.
+    uint32_t pack_heads, pack_blocks;
+    uint32_t part_rows;          // rows per (head, query tile, split) in the partial buffers: BM, or 32 when heads are packed
+    float *part_acc, *part_ml;   // [head][query tile][split][part_rows][D] unnormalised sums, [..][part_rows][2] (max, sum)
     float scale_log2e;
     uint32_t out_aligned16;         // output base and strides are multiples of 16 bytes: rows leave as whole 16-byte pieces
     unsigned long long *clock_out;  // nullable: per workgroup {shader-clock ticks, 100 MHz wall ticks} from start to end
@@ -537,10 +543,37 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     rsrc_words krs = make_rsrc_words(nullptr, 0), vrs = krs;
     if (PAGED) krs = make_rsrc_words(a.k, a.pool_bytes32), vrs = make_rsrc_words(a.v, a.pool_bytes32);  // the whole pools
     const uint32_t page_bytes = a.n_kv_heads * a.block_size * (uint32_t)ROWB;  // of one page, all heads
+    // this wave's 32 rows: query rows w_row0 .. of head w_head (w_ok: such a head exists)
+    uint32_t w_row0 = 0;
+    struct WaveRows {
+        uint32_t head, row0, ok;
+    };
+    auto wave_rows = [&](uint32_t item, uint32_t w) __attribute__((always_inline)) -> WaveRows {
+        WaveRows r;
+        if (a.pack_heads) {
+            const uint32_t hb = item / S, kv = hb / a.pack_blocks, h_in = (hb - kv * a.pack_blocks) * a.pack_heads + w;
+            r.head = kv * a.group_size + min(h_in, a.group_size - 1), r.row0 = 0;
+            r.ok = (w < a.pack_heads && h_in < a.group_size) ? 1u : 0u;
+        } else {
+            const uint32_t qi = item / (a.n_heads * S);
+            r.head = (item - qi * (a.n_heads * S)) / S, r.row0 = (n_qt - 1 - qi) * BM + 32 * w, r.ok = 1u;
+        }
+        return r;
+    };
     auto enter_item = [&](uint32_t item) {
-        const uint32_t qi = item / (a.n_heads * S), rest = item - qi * (a.n_heads * S);
-        q_tile = n_qt - 1 - qi, head = rest / S, split = rest - head * S;
-        kvh = head / a.group_size;
+        if (a.pack_heads) {
+            const uint32_t hb = item / S;
+            q_tile = 0, split = item - hb * S, kvh = hb / a.pack_blocks;
+            head = kvh * a.group_size + (hb - kvh * a.pack_blocks) * a.pack_heads;
+        } else {
+            const uint32_t qi = item / (a.n_heads * S), rest = item - qi * (a.n_heads * S);
+            q_tile = n_qt - 1 - qi, head = rest / S, split = rest - head * S;
+            kvh = head / a.group_size;
+        }
+        // (uniform values that come out of a branch and end up in the scalar operands of the DMA instructions)
+        kvh = (uint32_t)__builtin_amdgcn_readfirstlane((int)kvh), head = (uint32_t)__builtin_amdgcn_readfirstlane((int)head);
+        split = (uint32_t)__builtin_amdgcn_readfirstlane((int)split), q_tile = (uint32_t)__builtin_amdgcn_readfirstlane((int)q_tile);
+        w_row0 = wave_rows(item, (uint32_t)wave).row0;
         q0 = q_tile * BM;
         kv_end = a.kv_len;
         if (a.causal) {
@@ -610,9 +643,10 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         int ql = lane;
         asm volatile("" : "+v"(ql));  // the lane's source offset is worked out here, not kept in a register across the loop
         const int q_lane_src = (ql & 15) * (int)(a.q_stride_m * 2) + (ql >> 4) * 16;
-        const uint32_t qi = item / (a.n_heads * S), hd = (item - qi * (a.n_heads * S)) / S;
-        const uint32_t row0 = (n_qt - 1 - qi) * BM + 16 * wave8;
-        const rsrc_words qrs = make_rsrc_words(a.q + (size_t)hd * a.q_stride_h, (uint32_t)q_bytes);
+        // the 16 rows this wave moves are half of the 32 rows of wave (wave8 / 2) of either group
+        const WaveRows wr = wave_rows(item, (uint32_t)wave8 >> 1);
+        const uint32_t row0 = wr.row0 + 16 * ((uint32_t)wave8 & 1);
+        const rsrc_words qrs = make_rsrc_words(a.q + (size_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)wr.head) * a.q_stride_h, (uint32_t)q_bytes * (uint32_t)__builtin_amdgcn_readfirstlane((int)wr.ok));
         buffer_to_lds_b128<K_DMA, 64, 1024>(qrs, q_lds_addr + wave8 * RB_BYTES, q_lane_src, (int)(row0 * (uint32_t)(a.q_stride_m * 2)));
     };
 
@@ -734,16 +768,18 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         int lo = lane;
         asm volatile("" : "+v"(lo));
         const int n = lo & 31, hi = lo >> 5, lane = lo;
-        const uint32_t o_qi = o_item / (a.n_heads * S), o_rest = o_item - o_qi * (a.n_heads * S);
-        const uint32_t o_head = o_rest / S, o_q0 = (n_qt - 1 - o_qi) * BM;
+        const WaveRows owr = wave_rows(o_item, (uint32_t)wave);  // this wave's rows of the item
+        if (!owr.ok) return;  // (a packed item with fewer heads than waves)
+        const uint32_t o_head = owr.head, o_row0 = owr.row0;
+        const uint32_t o_split = a.pack_heads ? o_item % S : (o_item % (a.n_heads * S)) % S;
         const float o_m = m_run;  // untouched since the exchange, like l_run: this lane's half of the row's keys
         typedef unsigned int u2v __attribute__((ext_vector_type(2)));
         const u2v lsw = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run), __float_as_uint(l_run), false, false);
         const float o_l = __uint_as_float(lsw.x) + __uint_as_float(lsw.y);
-        const uint32_t q_row = o_q0 + wave * 32 + n;
+        const uint32_t q_row = o_row0 + n;
         if (S > 1) {  // flash_prefill.metal:592-617
             if (q_row < a.q_len) {
-                const size_t prow = (size_t)((o_head * n_qt + (n_qt - 1 - o_qi)) * S + (o_rest - o_head * S)) * BM + wave * 32 + n;
+                const size_t prow = (size_t)((o_head * n_qt + q_row / BM) * S + o_split) * a.part_rows + q_row % BM;
                 float *pa = a.part_acc + prow * D;
 #pragma unroll
                 for (int b = g * HB; b < (g + 1) * HB; ++b)
@@ -786,7 +822,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
 #pragma unroll
             for (int it = 0; it < 32 / RPI; ++it) {
                 const int row = it * RPI + lane / CPR;
-                const uint32_t qr = o_q0 + wave * 32 + row;
+                const uint32_t qr = o_row0 + row;
                 const uint4 val = *reinterpret_cast<const uint4 *>(ot + (r_off ^ (it * RPI * HROW + ((it * RPI) & (CPR - 1)) * 16)));
                 if (qr < a.q_len) __builtin_nontemporal_store(__builtin_bit_cast(u4_t, val), reinterpret_cast<u4_t *>(ob + (size_t)qr * a.out_stride_m));
             }
@@ -885,9 +921,9 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
             }
         }
         clear_state();
-        const uint32_t q_row_c = min(q0 + wave * 32 + n, a.q_len - 1);
+        const uint32_t q_row_c = min(w_row0 + n, a.q_len - 1);
         const uint32_t q_abs = q_row_c + a.query_offset;
-        const uint32_t wave_min_limit = a.causal ? (min(q0 + wave * 32, a.q_len - 1) + a.query_offset) : 0xffffffffu;
+        const uint32_t wave_min_limit = a.causal ? (min(w_row0, a.q_len - 1) + a.query_offset) : 0xffffffffu;
         if (ntg > 0) {
             k_prefetch(0);
             s_tile(0);
@@ -995,21 +1031,21 @@ template <int D, bool BF16>
 __global__ void __launch_bounds__(256) flash_prefill_merge_kernel(PrefillDev a) {
     constexpr int CG = D / 4;           // float4 columns per row
     constexpr int ROWS = 256 / CG;      // rows per workgroup (8 at D = 128, 16 at D = 64)
-    constexpr int SLABS = BM / ROWS;    // workgroups per query tile
     constexpr int PB = 8;               // splits loaded per batch
-    const uint32_t S = a.splits;
+    const uint32_t S = a.splits, PR = a.part_rows;
+    const uint32_t SLABS = PR / ROWS;   // workgroups per query tile
     const uint32_t n_qt = gridDim.x / (a.n_heads * SLABS);
     const uint32_t slab = blockIdx.x % SLABS, qh = blockIdx.x / SLABS;
     const uint32_t q_tile = qh / a.n_heads, head = qh % a.n_heads;
     const int r = slab * ROWS + threadIdx.x / CG, c4 = threadIdx.x % CG;
     const uint32_t q_row = q_tile * BM + r;
     if (q_row >= a.q_len) return;
-    const size_t base = (((size_t)head * n_qt + q_tile) * S) * BM + r;
+    const size_t base = (((size_t)head * n_qt + q_tile) * S) * PR + r;
     float mstar = -1e30f;
     for (uint32_t s0 = 0; s0 < S; s0 += PB) {  // PB loads in flight (one after the other they cost a memory latency each)
         float2 ml[PB];
 #pragma unroll
-        for (int k = 0; k < PB; ++k) ml[k] = *reinterpret_cast<const float2 *>(a.part_ml + (base + (size_t)min(s0 + k, S - 1) * BM) * 2);
+        for (int k = 0; k < PB; ++k) ml[k] = *reinterpret_cast<const float2 *>(a.part_ml + (base + (size_t)min(s0 + k, S - 1) * PR) * 2);
 #pragma unroll
         for (int k = 0; k < PB; ++k)
             if (s0 + k < S && ml[k].y > 0.0f) mstar = fmaxf(mstar, ml[k].x);
@@ -1022,8 +1058,8 @@ __global__ void __launch_bounds__(256) flash_prefill_merge_kernel(PrefillDev a) 
 #pragma unroll
         for (int k = 0; k < PB; ++k) {
             const uint32_t s = min(s0 + k, S - 1);  // clamped; masked below
-            v[k] = *reinterpret_cast<const float4 *>(a.part_acc + (base + (size_t)s * BM) * D + c4 * 4);
-            ml[k] = *reinterpret_cast<const float2 *>(a.part_ml + (base + (size_t)s * BM) * 2);
+            v[k] = *reinterpret_cast<const float4 *>(a.part_acc + (base + (size_t)s * PR) * D + c4 * 4);
+            ml[k] = *reinterpret_cast<const float2 *>(a.part_ml + (base + (size_t)s * PR) * 2);
         }
 #pragma unroll
         for (int k = 0; k < PB; ++k) {
@@ -1064,7 +1100,17 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
     // Split-K (src/metals/flashattention/step.rs:849-864): few query tiles against a long context (a prefill chunk
     // after a long prefix) would leave most CUs idle, so the key tiles of each query tile are divided over several
     // workgroups, at least 4 tiles each, up to one workgroup per CU.
-    const uint32_t base_wgs = ceil_div_u32(L.q_len, BM) * L.n_heads;
+    // the LDS-direct kernel (measured faster at every size) addresses the query rows of a head with 32-bit offsets
+    const bool lds_direct = ctx->prefill_variant != 1 && ((uint64_t)(L.q_len - 1) * L.q_stride_m + L.head_dim) * 2 < (1ull << 32);
+    // A chunk of at most 32 rows (the reference's default prefill chunk, src/model/executor.rs:232-250): an item is the
+    // rows of up to four heads of a KV group, which then share every K/V tile (see PrefillDev).
+    a.pack_heads = 0, a.pack_blocks = 1, a.part_rows = BM;
+    if (lds_direct && L.q_len <= 32 && L.group_size >= 2) {
+        a.pack_heads = L.group_size < 4 ? L.group_size : 4;
+        a.pack_blocks = ceil_div_u32(L.group_size, a.pack_heads);
+        a.part_rows = 32;
+    }
+    const uint32_t base_wgs = a.pack_heads ? L.n_kv_heads * a.pack_blocks : ceil_div_u32(L.q_len, BM) * L.n_heads;
     const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
     const uint32_t key_tiles = ceil_div_u32(L.kv_len, BN);
     uint32_t splits = ctx->prefill_split_k;
@@ -1072,19 +1118,20 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
         splits = 1;
         if (base_wgs * 2 <= n_cus) splits = n_cus / base_wgs;  // all workgroups resident at once, one per CU
         if (splits > key_tiles / 4) splits = key_tiles / 4;
+        // (packed heads: every split is one more partial per row for the merge, so beyond 16 splits each should have 16
+        // tiles. A 32-row chunk after 2K / 8K / 32K tokens measured best with 8 / 16 / 24-32 splits.)
+        if (a.pack_heads && splits > 16 && key_tiles / splits < 16) splits = key_tiles / 16 > 16 ? key_tiles / 16 : 16;
     }
     if (splits > key_tiles) splits = key_tiles;
     if (splits < 1) splits = 1;
     a.splits = splits, a.part_acc = nullptr, a.part_ml = nullptr;
     if (splits > 1) {
-        const size_t rows = (size_t)base_wgs * splits * BM;
+        const size_t rows = (size_t)L.n_heads * ceil_div_u32(L.q_len, BM) * splits * a.part_rows;
         const size_t acc_bytes = rows * L.head_dim * sizeof(float);
         FA_TRY(fa_ensure_workspace(ctx, acc_bytes + rows * 2 * sizeof(float)));
         a.part_acc = (float *)ctx->workspace;
         a.part_ml = (float *)((char *)ctx->workspace + acc_bytes);
     }
-    // the LDS-direct kernel (measured faster at every size) addresses the query rows of a head with 32-bit offsets
-    const bool lds_direct = ctx->prefill_variant != 1 && ((uint64_t)(L.q_len - 1) * L.q_stride_m + L.head_dim) * 2 < (1ull << 32);
     // Its workgroups (one fits a CU) stay and share out the (query tile, head, split) items among themselves.
     a.n_qt = ceil_div_u32(L.q_len, BM), a.n_items = base_wgs * splits;
     a.n_workgroups = lds_direct ? (a.n_items < n_cus ? a.n_items : n_cus) : a.n_items;
@@ -1113,15 +1160,16 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
         FA_TRY(scope.finish());
     }
     if (splits > 1) {
+        const uint32_t merge_tiles = L.n_heads * ceil_div_u32(L.q_len, BM);  // (head, query tile) pairs
         FaLaunchScope scope(ctx, "flash_prefill_merge_kernel", true);
         if (L.head_dim == 128 && L.bf16)
-            scope.launch(flash_prefill_merge_kernel<128, true>, dim3(base_wgs * (BM / 8)), dim3(256), 0, a);
+            scope.launch(flash_prefill_merge_kernel<128, true>, dim3(merge_tiles * (a.part_rows / 8)), dim3(256), 0, a);
         else if (L.head_dim == 128)
-            scope.launch(flash_prefill_merge_kernel<128, false>, dim3(base_wgs * (BM / 8)), dim3(256), 0, a);
+            scope.launch(flash_prefill_merge_kernel<128, false>, dim3(merge_tiles * (a.part_rows / 8)), dim3(256), 0, a);
         else if (L.bf16)
-            scope.launch(flash_prefill_merge_kernel<64, true>, dim3(base_wgs * (BM / 16)), dim3(256), 0, a);
+            scope.launch(flash_prefill_merge_kernel<64, true>, dim3(merge_tiles * (a.part_rows / 16)), dim3(256), 0, a);
         else
-            scope.launch(flash_prefill_merge_kernel<64, false>, dim3(base_wgs * (BM / 16)), dim3(256), 0, a);
+            scope.launch(flash_prefill_merge_kernel<64, false>, dim3(merge_tiles * (a.part_rows / 16)), dim3(256), 0, a);
         FA_TRY(scope.finish());
     }
     return FA_OK;

@@ -263,6 +263,8 @@ def test_paged_decode_full_batch_of_32_ragged_sequences():
     (14, 2, 64, 48, 70, 37),      # block size not a power of two, head_dim 64
     (8, 8, 128, 32, 0, 129),      # no prefix, one row into a second query tile
     (4, 2, 128, 16, 2000, 32),    # a 32-row chunk after a long prefix: few query tiles, split over the keys
+    (24, 8, 128, 16, 1111, 32),   # the same at the Llama-3.2-3B shape: the three heads of a KV group share an item
+    (14, 2, 64, 32, 500, 9),      # nine rows, groups of seven heads
 ])
 def test_paged_prefill_chunk_after_prefix(H, Hkv, D, bs, prefix, M):
     """A prefill chunk attending a paged cache that already holds a prefix (sequence 1 of 3, random block

@@ -229,6 +229,37 @@ def test_prefill_errors():
     f.synchronize()
 
 
+@pytest.mark.parametrize("split_k", [0, 1, 5])
+@pytest.mark.parametrize("H,Hkv,D,M,prefix,layout", [
+    (24, 8, 128, 32, 4000, "head_major"),   # the reference's default chunk at the Llama-3.2-3B shape: 3 heads per item
+    (16, 2, 128, 20, 3000, "token_major"),  # a group of 8: two items of 4 heads per KV head, rows past the chunk's end
+    (14, 2, 64, 32, 2500, "head_major"),    # a group of 7: items of 4 and of 3 heads
+    (8, 4, 64, 5, 1500, "token_major"),     # a group of 2: two of the four waves of a group have no head
+    (12, 3, 128, 2, 900, "head_major"),     # two rows
+    (6, 2, 128, 31, 0, "head_major"),       # no prefix: one key tile, nothing to split
+])
+def test_prefill_chunk_of_at_most_32_rows_packs_the_heads_of_a_kv_group(H, Hkv, D, M, prefix, layout, split_k, prefill_variant):
+    """A chunk of at most 32 query rows (the reference's default prefill chunk size, src/model/executor.rs:232-250) runs
+    with the rows of up to four heads of a KV group in one item. Same contract as every other prefill launch: the oracle
+    and float64 within the tolerance, for the automatic split count, no split and a forced one."""
+    announce("prefill, short chunk", H, Hkv, D, M, prefix, layout, split_k, prefill_variant)
+    f = ctx()
+    rng = np.random.default_rng(H * 100 + M + prefix)
+    N = prefix + M
+    cap = N + 3
+    q, k, v = h16(rng.normal(size=(H, M, D))), h16(rng.normal(size=(Hkv, cap, D))), h16(rng.normal(size=(Hkv, cap, D)))
+    k[:, N:], v[:, N:] = np.float16(np.nan), np.float16(np.nan)
+    want = orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, prefix, cap, causal=True, out_layout="head_major", n_threads=8)
+    f.set_prefill_split_k(split_k)
+    try:
+        got = gpu_prefill(q, k, v, H, D, M, N, prefix, q_layout=layout)
+    finally:
+        f.set_prefill_split_k(0)
+    assert np.all(np.isfinite(got))
+    assert max_abs(got, want) <= TOL
+    assert max_abs(got, rm.gqa_prefill_f64(q, k, v, H, Hkv, D, N, prefix)) <= TOL
+
+
 @pytest.mark.parametrize("split_k", [0, 1, 2, 3, 4, 8])
 def test_prefill_split_k_independent_of_split_count(split_k):
     """A prefill chunk after a long prefix, key tiles divided over split_k workgroups + merge kernel
