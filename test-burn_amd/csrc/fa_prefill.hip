@@ -52,12 +52,12 @@ struct PrefillDev {
     uint32_t splits;             // > 1: the key tiles of a query tile are divided over `splits` items
     uint32_t n_qt, n_items, n_workgroups;  // query tiles; (query tile, head, split) items; workgroups that share them out
     uint32_t pool_bytes32;       // paged: size of each pool when below 4 GiB (whole pages then go by a 32-bit offset), else 0
-    // A chunk of at most 32 query rows (the reference's default prefill chunk): the four 32-row blocks of an item are the
-    // rows of up to four query heads of one KV group instead of 128 rows of one head (three quarters of which would be
-    // empty), so the group's heads share every K/V tile. pack_heads = heads per item (0 = off), pack_blocks = such
-    // items per KV head.
-    uint32_t pack_heads, pack_blocks;
-    uint32_t part_rows;          // rows per (head, query tile, split) in the partial buffers: BM, or 32 when heads are packed
+    // A chunk of at most 64 query rows (the reference's default prefill chunk is 32): the four 32-row blocks of an item
+    // are (head, 32 rows) pairs of one KV group - its heads' first rows, then (when there are more than 32 rows) their
+    // second 32 - instead of 128 rows of one head, half or three quarters of which would be empty; the group's heads
+    // share every K/V tile. pack_heads != 0 = on, pack_nb = 32-row blocks per head (1 or 2), pack_blocks = items per KV head.
+    uint32_t pack_heads, pack_nb, pack_blocks;
+    uint32_t part_rows;          // rows per (head, query tile, split) in the partial buffers: BM, or 32 pack_nb when heads are packed
     float *part_acc, *part_ml;   // [head][query tile][split][part_rows][D] unnormalised sums, [..][part_rows][2] (max, sum)
     float scale_log2e;
     uint32_t out_aligned16;         // output base and strides are multiples of 16 bytes: rows leave as whole 16-byte pieces
@@ -551,9 +551,11 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     auto wave_rows = [&](uint32_t item, uint32_t w) __attribute__((always_inline)) -> WaveRows {
         WaveRows r;
         if (a.pack_heads) {
-            const uint32_t hb = item / S, kv = hb / a.pack_blocks, h_in = (hb - kv * a.pack_blocks) * a.pack_heads + w;
-            r.head = kv * a.group_size + min(h_in, a.group_size - 1), r.row0 = 0;
-            r.ok = (w < a.pack_heads && h_in < a.group_size) ? 1u : 0u;
+            // pair p of the KV group = (head p % G, rows 32 (p / G) ..); this item holds pairs 4 (item's index) .. + 3
+            const uint32_t hb = item / S, kv = hb / a.pack_blocks, pr = (hb - kv * a.pack_blocks) * 4 + w;
+            const uint32_t rb = pr / a.group_size, h_in = pr - rb * a.group_size;
+            r.ok = rb < a.pack_nb ? 1u : 0u;
+            r.head = kv * a.group_size + (r.ok ? h_in : 0u), r.row0 = r.ok ? rb * 32 : 0u;
         } else {
             const uint32_t qi = item / (a.n_heads * S);
             r.head = (item - qi * (a.n_heads * S)) / S, r.row0 = (n_qt - 1 - qi) * BM + 32 * w, r.ok = 1u;
@@ -564,7 +566,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
         if (a.pack_heads) {
             const uint32_t hb = item / S;
             q_tile = 0, split = item - hb * S, kvh = hb / a.pack_blocks;
-            head = kvh * a.group_size + (hb - kvh * a.pack_blocks) * a.pack_heads;
+            head = kvh * a.group_size;
         } else {
             const uint32_t qi = item / (a.n_heads * S), rest = item - qi * (a.n_heads * S);
             q_tile = n_qt - 1 - qi, head = rest / S, split = rest - head * S;
@@ -1102,13 +1104,13 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
     // workgroups, at least 4 tiles each, up to one workgroup per CU.
     // the LDS-direct kernel (measured faster at every size) addresses the query rows of a head with 32-bit offsets
     const bool lds_direct = ctx->prefill_variant != 1 && ((uint64_t)(L.q_len - 1) * L.q_stride_m + L.head_dim) * 2 < (1ull << 32);
-    // A chunk of at most 32 rows (the reference's default prefill chunk, src/model/executor.rs:232-250): an item is the
-    // rows of up to four heads of a KV group, which then share every K/V tile (see PrefillDev).
-    a.pack_heads = 0, a.pack_blocks = 1, a.part_rows = BM;
-    if (lds_direct && L.q_len <= 32 && L.group_size >= 2) {
-        a.pack_heads = L.group_size < 4 ? L.group_size : 4;
-        a.pack_blocks = ceil_div_u32(L.group_size, a.pack_heads);
-        a.part_rows = 32;
+    // A chunk of at most 64 rows (the reference's default prefill chunk is 32, src/model/executor.rs:232-250): an item is
+    // four (head, 32 rows) pairs of a KV group, which then share every K/V tile (see PrefillDev).
+    a.pack_heads = 0, a.pack_nb = 1, a.pack_blocks = 1, a.part_rows = BM;
+    if (lds_direct && L.q_len <= 64 && L.group_size >= 2) {
+        a.pack_heads = 1, a.pack_nb = ceil_div_u32(L.q_len, 32);
+        a.pack_blocks = ceil_div_u32(L.group_size * a.pack_nb, 4);
+        a.part_rows = 32 * a.pack_nb;
     }
     const uint32_t base_wgs = a.pack_heads ? L.n_kv_heads * a.pack_blocks : ceil_div_u32(L.q_len, BM) * L.n_heads;
     const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;

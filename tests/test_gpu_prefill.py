@@ -237,11 +237,14 @@ def test_prefill_errors():
     (8, 4, 64, 5, 1500, "token_major"),     # a group of 2: two of the four waves of a group have no head
     (12, 3, 128, 2, 900, "head_major"),     # two rows
     (6, 2, 128, 31, 0, "head_major"),       # no prefix: one key tile, nothing to split
+    (24, 8, 128, 64, 4000, "head_major"),   # 64 rows: six (head, 32 rows) pairs per KV group in items of four and two
+    (14, 2, 64, 40, 700, "token_major"),    # 40 rows, groups of seven heads: fourteen pairs, the second blocks ragged
+    (4, 2, 128, 33, 300, "head_major"),     # one row into the second block, groups of two: exactly one item per KV head
 ])
-def test_prefill_chunk_of_at_most_32_rows_packs_the_heads_of_a_kv_group(H, Hkv, D, M, prefix, layout, split_k, prefill_variant):
-    """A chunk of at most 32 query rows (the reference's default prefill chunk size, src/model/executor.rs:232-250) runs
-    with the rows of up to four heads of a KV group in one item. Same contract as every other prefill launch: the oracle
-    and float64 within the tolerance, for the automatic split count, no split and a forced one."""
+def test_prefill_short_chunk_packs_the_heads_of_a_kv_group(H, Hkv, D, M, prefix, layout, split_k, prefill_variant):
+    """A chunk of at most 64 query rows (the reference's default prefill chunk size is 32, src/model/executor.rs:232-250)
+    runs with four (head, 32 rows) pairs of a KV group in one item. Same contract as every other prefill launch: the
+    oracle and float64 within the tolerance, for the automatic split count, no split and a forced one."""
     announce("prefill, short chunk", H, Hkv, D, M, prefix, layout, split_k, prefill_variant)
     f = ctx()
     rng = np.random.default_rng(H * 100 + M + prefix)
