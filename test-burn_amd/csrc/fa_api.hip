@@ -1019,11 +1019,7 @@ static fa_status fused_qkv_kv_prep(fa_ctx *ctx, FusedQkvLaunch &Q, KvPrepLaunch 
     FA_TRY(fa_ensure_workspace(ctx, nq + 2 * nkv));
     char *ws = (char *)ctx->workspace;
     Q.out[0] = (__half *)ws, Q.out[1] = (__half *)(ws + nq), Q.out[2] = (__half *)(ws + nq + nkv);
-    const uint32_t min_m = ctx->gemm_min_m;
-    ctx->gemm_min_m = 0xffffffffu;  // the weight-stream kernel: its outputs are in the workspace the GEMM would use
-    const fa_status st = fa_launch_fused_qkv(ctx, Q);
-    ctx->gemm_min_m = min_m;
-    FA_TRY(st);
+    FA_TRY(fa_launch_fused_qkv(ctx, Q, true));  // the weight-stream kernel: the outputs are in the workspace the GEMM would use
     K.q = Q.out[0], K.k = Q.out[1], K.v = Q.out[2];
     return fa_launch_kv_prep(ctx, K);
 }

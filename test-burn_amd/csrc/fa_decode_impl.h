@@ -716,8 +716,8 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     qraw.u = make_uint4(0, 0, 0, 0);
     // SAGE + FUSED, wave 0's staging area (its own V region, unused until it attends the open block): the quantised rows
     // of the group's query heads, the rotated new K row, the smoothing mean.
-    __half *st_qraw = reinterpret_cast<__half *>(smem);  // int8 [MAX_GT][D]
-    __half *st_krot = st_qraw + MAX_GT * D / 2;
+    int8_t *st_q8 = reinterpret_cast<int8_t *>(smem);  // [MAX_GT][D]
+    __half *st_krot = reinterpret_cast<__half *>(smem + MAX_GT * D);
     float *st_mean = reinterpret_cast<float *>(st_krot + D);
     static_assert(!(SAGE && FUSED) || MAX_GT * D + D * 2 + D * 4 <= MBX * BK * VRS, "staging fits a wave's V region");
     uint4 sage_vnew = make_uint4(0, 0, 0, 0);
@@ -742,8 +742,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             __builtin_amdgcn_sched_barrier(0);
             n_raw = read_len();
             const uint32_t p0 = min(n_raw, min(a.capacity, a.kv_len_bound)) - 1;
-            const bool rope_q = rope_on;
-            if (rope_q) {  // the table row through the scalar cache, as below
+            if (rope_on) {  // the table row through the scalar cache, as below
                 const uint32_t tp = min(p0, a.table_rows - 1);
                 const __half *ct = a.cos_t + (size_t)tp * (D / 2), *st = a.sin_t + (size_t)tp * (D / 2);
                 if constexpr (D == 128) {
@@ -800,7 +799,6 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             // The query: rotated, then quantised per head with the head's own scale max|q| / 127 (f32), as
             // sage_append_kernel does it - here 8 values per lane (the operand layout would make every lane divide 16
             // KSTEPS values, most of them for heads the group does not have) - and handed over as int8 rows in LDS.
-            int8_t *st_q8 = reinterpret_cast<int8_t *>(st_qraw);
 #pragma unroll
             for (int i = 0; i < QV; ++i) {
                 if ((uint32_t)(64 * i) >= gt * PPR) break;  // uniform: no rows left

@@ -259,7 +259,8 @@ struct FusedQkvLaunch {
     const __half *scales[3] = {nullptr, nullptr, nullptr};
     int weight_bits = 16;  // 16 = F16, 8 = Q8_0, 4 = Q4_0 (two weights per byte, element 2i in the low nibble of byte i)
 };
-fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l);
+// weight_stream_only: never the GEMM (whose scratch is the context's workspace), whatever the number of input rows
+fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l, bool weight_stream_only = false);
 fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l);  // fa_gemm.hip: many input rows
 
 fa_status fa_launch_sage_k_mean(fa_ctx *ctx, const void *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim,

@@ -322,7 +322,7 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
 
 }  // namespace
 
-fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
+fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l, bool weight_stream_only) {
     QkvDev a;
     for (int i = 0; i < 3; ++i) a.w[i] = l.w[i], a.bias[i] = l.bias[i], a.out[i] = l.out[i];
     a.rows[0] = l.n_dim, a.rows[1] = l.n_kv, a.rows[2] = l.n_kv;
@@ -339,7 +339,7 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l) {
     auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
     const bool gemm_ok = l.k_dim % (q8 ? 32 : 8) == 0 && aligned16(l.x) && aligned16(l.w[0]) && aligned16(l.w[1]) &&
                          aligned16(l.w[2]) && aligned16(l.gamma);
-    if (gemm_ok && l.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : GEMM_MIN_M_DEFAULT)) return fa_launch_fused_qkv_gemm(ctx, l);
+    if (!weight_stream_only && gemm_ok && l.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : GEMM_MIN_M_DEFAULT)) return fa_launch_fused_qkv_gemm(ctx, l);
     const uint32_t total_rows = l.n_dim + 2 * l.n_kv;
     const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
     // Workgroups: a multiple of the CU count, enough of them that a workgroup's rows fit one 16-row tile where the
