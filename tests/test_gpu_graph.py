@@ -215,3 +215,52 @@ def test_stream_timer_and_compute_units():
     assert int(word.download()[0]) == 256
     g.destroy()
     word.free()
+
+
+def test_captured_prefill_chunks_with_the_fused_qkv_write_stage_replay():
+    """A prefill chunk of one layer as a captured graph - FusedQkv with KvPrepFused as its write stage (norm kernel, split-K
+    GEMM, finish kernel), then the chunk's attention over the cache (split-K prefill + merge) - replayed several times
+    with eager work and synchronisations between the replays; every replay must reproduce the eager result bit for bit."""
+    announce("graph replay, fused qkv + kv prep + prefill chunk")
+    f = ctx()
+    rng = np.random.default_rng(21)
+    H, Hkv, D, K, m, prefix, cap = 24, 8, 128, 1024, 32, 1000, 1280
+    N, NK = H * D, Hkv * D
+    x = rng.uniform(-1, 1, (m, K)).astype(np.float16)
+    g = rng.uniform(0.5, 1.5, K).astype(np.float16)
+    ws = [rng.uniform(-0.1, 0.1, (n, K)).astype(np.float16) for n in (N, NK, NK)]
+    kc0, vc0 = h16(rng.normal(size=(Hkv, cap, D))), h16(rng.normal(size=(Hkv, cap, D)))
+    cos, sin = fa.rope_tables(5e5, D, cap)
+    dev_w = [f.array(orc.to_canonical(w)) for w in ws]
+    dx, dg, dcos, dsin = f.array(x), f.array(g), f.array(cos), f.array(sin)
+    dkc, dvc = f.array(kc0), f.array(vc0)
+    dqr, dout = f.zeros((H, m, D)), f.zeros((m, H * D))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, m, prefix, cap, fa.ROPE_NORMAL)
+
+    def enqueue():
+        f.fused_qkv_kv_prep(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), K, dqr.arg(), dcos.arg(), dsin.arg(), p,
+                            k_cache=dkc.arg(), v_cache=dvc.arg(), gamma=dg.arg())
+        f.flash_attention(dqr.arg(), dkc.arg(), dvc.arg(), dout.arg(), True, prefix, H, D, prefix + m, m)
+
+    enqueue()  # eager: the reference result, and the workspace at its final size before the capture
+    f.synchronize()
+    want_out, want_k, want_qr = bits(dout.download()), bits(dkc.download()), bits(dqr.download())
+    f.start_capture()
+    enqueue()
+    graph = f.end_capture()
+    scratch = f.zeros((64, 64))
+    for t in range(4):
+        for d, src in ((dkc, kc0), (dvc, vc0)):
+            d.upload(src)
+        dout.upload(np.zeros((m, H * D), np.float16))
+        dqr.upload(np.zeros((H, m, D), np.float16))
+        graph.launch()
+        f.synchronize()
+        assert np.array_equal(bits(dout.download()), want_out), t
+        assert np.array_equal(bits(dkc.download()), want_k), t
+        assert np.array_equal(bits(dqr.download()), want_qr), t
+        scratch.upload(np.full((64, 64), t, np.float16))  # eager work between the replays
+        f.synchronize()
+    graph.destroy()
+    for b in dev_w + [dx, dg, dcos, dsin, dkc, dvc, dqr, dout, scratch]:
+        b.free()
