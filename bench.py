@@ -726,6 +726,68 @@ def bench_attn_block(f, args):
         "parity": {"outputs_finite": finite, "note": "stage-by-stage parity of this chain: tests/test_gpu_block.py"}}))
 
 
+def bench_prefill_chunk(f, args, m=32, prefix=8160):
+    """One prefill chunk of m rows (32 = the reference's default chunk, src/model/executor.rs:232-250) attending a contiguous
+    Llama-3.2-3B-shaped cache that already holds `prefix` tokens: the split-K prefill kernel + its merge kernel, timed as
+    graph replays over 4 layers' caches in rotation. HBM-bound: every launch reads the whole prefix once."""
+    H, Hkv, D, L = 24, 8, 128, 4
+    N, cap = prefix + m, prefix + 512
+    rng = np.random.default_rng(0xF0DD + 14)
+    caches = [(f.array(rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16)),
+               f.array(rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16))) for _ in range(L)]
+    q = rng.standard_normal((H, m, D), dtype=np.float32).astype(np.float16)
+    dq, dout = f.array(q), f.zeros((m, H * D))
+
+    def step(i):
+        kc, vc = caches[i % L]
+        f.flash_attention(dq.arg(), kc.arg(), vc.arg(), dout.arg(), True, prefix, H, D, N, m)
+
+    step(0)
+    f.synchronize()
+    import orc  # the CPU oracle is only the checker here
+    want = orc.sdpa_prefill(q, caches[0][0].download(), caches[0][1].download(), H, Hkv, D, m, N, prefix, cap, causal=True,
+                            out_layout="head_major", n_threads=max(1, min(16, os.cpu_count() or 1, orc.lib().orc_max_threads())))
+    got = dout.download().reshape(m, H, D).transpose(1, 0, 2)
+    err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64))))
+    per_graph = 4 * L
+    f.start_capture()
+    for i in range(per_graph):
+        step(i)
+    graph = f.end_capture()
+    for _ in range(max(1, args.warmup // per_graph)):
+        graph.launch()
+    f.synchronize()
+    reps = max(1, args.steps // per_graph)
+    f.timer_start()
+    for _ in range(reps):
+        graph.launch()
+    per_step = f.timer_stop() / 1e3 / (reps * per_graph)
+    graph.destroy()
+    f.profile_reset()
+    f.profile_enable(True)
+    for i in range(per_graph):
+        step(i)
+    us = {}
+    for kname in ("flash_prefill_dma_kernel", "flash_prefill_mfma_kernel", "flash_prefill_merge_kernel"):
+        n, ms = f.profile_query(kname)
+        if n:
+            us[kname] = ms * 1e3 / n
+    f.profile_enable(False)
+    nbytes = 2.0 * Hkv * N * D * 2 + 2.0 * H * m * D * 2  # K and V once per KV head, q in, out
+    emit({
+        "metric": "prefill-chunk steps/s + achieved HBM GB/s, Llama-3.2-3B shape, %d rows after %d tokens" % (m, prefix),
+        "value": 1.0 / per_step, "unit": "steps/s", "n_gpus": 1, "steps": reps * per_graph, "warmup": args.warmup,
+        "ms_per_step": per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "llama3.2-3b prefill chunk of %d rows after a %d-token prefix, one layer per step: causal attention "
+                               "(split over the keys) + merge, contiguous cache, graph replays" % (m, prefix)},
+        "roofline": {"bound": "hbm", "achieved": nbytes / per_step / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": nbytes / per_step / 1e9 / HBM_PEAK_GBPS, "traffic": None, "kernel": "prefill kernel + merge kernel (one step)",
+                     "avg_launch_us": us, "bytes_per_step": nbytes,
+                     "timing": "HIP events on the stream around the graph replays / steps in them"},
+        "parity": {"max_abs_err_vs_oracle": err}})
+
+
 def bench_prefill_block(f, args, fused=False):
     """The attention block of one Llama-3.2-3B layer on a 2048-token prompt in one chunk (models/llama.json:509-585):
     FusedQkv (norm kernel + GEMM) -> KvPrepFused (RoPE + append of 2048 rows) -> FlashAttention (causal prefill) -> o_proj
@@ -1031,7 +1093,7 @@ def bench_floors(f, args):
     emit(out)
 
 
-SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill,
+SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_chunk32_8k": bench_prefill_chunk, "llama3b_prefill_chunk32_32k": lambda f, args: bench_prefill_chunk(f, args, 32, 32736), "llama3b_prefill_chunk64_8k": lambda f, args: bench_prefill_chunk(f, args, 64, 8128), "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill,
              "llama3b_prefill_8k": lambda f, args: bench_prefill(f, args, 8192), "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
