@@ -95,11 +95,20 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
         return c;
     };
     uint32_t waves = ctx->decode_waves;  // 0 = by the rule above
+    bool short_context = false;
     if (waves == 0) {
         const uint32_t c8 = chunk ? chunk : auto_chunk(8, n_cus);
         waves = groups * ceil_div_u32(bound, (c8 + BK - 1) / BK * BK) > n_cus ? 4u : 8u;
+        // A context so short that even four waves get at most one block each (at most 64 keys per compute unit's
+        // share): 4-wave workgroups, still one per CU - half the waves to start, fold and keep in step. Measured,
+        // H24 / Hkv8 / D128: 512 keys 6.86 -> 6.61 us, 1024 6.90 -> 6.69, 2048 7.12 -> 6.90; H14 / Hkv2 / D64 at 1025: 6.40 -> 6.28.
+        if (waves == 8 && !chunk) {
+            const uint32_t s_max = groups >= n_cus ? 1u : (uint32_t)(n_cus / groups);
+            short_context = ceil_div_u32(bound, s_max) <= 4u * BK;
+            if (short_context) waves = 4;
+        }
     }
-    if (chunk == 0) chunk = waves == 4 ? auto_chunk(4, 2 * n_cus) : auto_chunk(8, n_cus);
+    if (chunk == 0) chunk = waves == 4 ? auto_chunk(4, short_context ? n_cus : 2 * n_cus) : auto_chunk(8, n_cus);
     chunk = (chunk + BK - 1) / BK * BK;
     // the int8 step in one launch: the open 32-row block must lie inside one partition
     if (L.sage_fused) chunk = (chunk + FA_SAGE_BLOCK - 1) / FA_SAGE_BLOCK * FA_SAGE_BLOCK;
