@@ -668,6 +668,61 @@ def bench_long_decode(f, args):
     f.profile_enable(False)
 
 
+def bench_short_decode(f, args, pos=2047):
+    """Llama-3.2-3B-shaped single-layer decode step at a short context (pos + 1 keys): where a launch is mostly its fixed
+    cost. Eight layers' caches in rotation, a graph of 32 launches replayed, two events on the stream.
+    FOUNDRY_ATTN_DECODE_WAVES=8 forces the 8-wave workgroups that longer contexts use."""
+    import orc
+    H, Hkv, D, NL = 24, 8, 128, 8
+    cap = pos + 1 + 64
+    rng = np.random.default_rng(0xF0DD + 15)
+    cos, sin = fa.rope_tables(5e5, D, cap)
+    dcos, dsin = f.array(cos), f.array(sin)
+    host = [(rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16),
+             rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16)) for _ in range(NL)]
+    caches = [(f.array(kc), f.array(vc)) for kc, vc in host]
+    q, k, v = (rng.standard_normal((1, n * D), dtype=np.float32).astype(np.float16) for n in (H, Hkv, Hkv))
+    dq, dk, dv, dout = f.array(q), f.array(k), f.array(v), f.zeros((1, H * D))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, 1, pos, cap, fa.ROPE_NORMAL)
+
+    def step(i):
+        kc, vc = caches[i % NL]
+        f.decode_step_fused(dq.arg(), dk.arg(), dv.arg(), None, kc.arg(), vc.arg(), dcos.arg(), dsin.arg(), dout.arg(), p)
+
+    step(0)
+    f.synchronize()
+    want_qr = orc.kv_prep_fused(q, k, v, host[0][0], host[0][1], cos, sin, orc.make_params(H, Hkv, D, 1, pos, cap, rope_mode=1))
+    want = orc.sdpa_decode(want_qr[:, 0].copy(), host[0][0], host[0][1], H, Hkv, D, cap, pos + 1, n_threads=8)
+    err = float(np.max(np.abs(dout.download().reshape(-1).astype(np.float64) - want.reshape(-1).astype(np.float64))))
+    per_graph = 4 * NL
+    f.start_capture()
+    for i in range(per_graph):
+        step(i)
+    graph = f.end_capture()
+    for _ in range(max(1, args.warmup // per_graph)):
+        graph.launch()
+    f.synchronize()
+    reps = max(1, args.steps // per_graph)
+    f.timer_start()
+    for _ in range(reps):
+        graph.launch()
+    per_step = f.timer_stop() / 1e3 / (reps * per_graph)
+    graph.destroy()
+    nbytes = 2.0 * Hkv * (pos + 1) * D * 2 + 2 * Hkv * D * 2 + 2 * H * D * 2 + 2 * Hkv * D * 2 + 2 * D
+    emit({
+        "metric": "decode-attn layer-steps/s + achieved HBM GB/s, Llama-3.2-3B shape @%d keys" % (pos + 1),
+        "value": 1.0 / per_step, "unit": "layer-steps/s", "n_gpus": 1, "steps": reps * per_graph, "warmup": args.warmup,
+        "ms_per_step": per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "llama3.2-3b single-layer decode step at a short context: RoPE + KV append + flash decode, batch 1, "
+                               "H24/Hkv8/D128, kv_len %d, graph replays" % (pos + 1)},
+        "roofline": {"bound": "hbm", "achieved": nbytes / per_step / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": nbytes / per_step / 1e9 / HBM_PEAK_GBPS, "traffic": None, "kernel": "fused_rope_append_decode_kernel",
+                     "avg_launch_us": per_step * 1e6, "bytes_per_launch": nbytes,
+                     "timing": "HIP events on the stream around the graph replays / launches in them"},
+        "parity": {"decode_max_abs_err": err}})
+
+
 def bench_attn_block(f, args):
     """The attention block of a Llama-3.2-3B decode step, all 28 layers, as the reference's graph runs it
     (models/llama.json:509-585): FusedQkv (RMSNorm + projections) -> RoPE + KV append + flash decode -> o_proj MatMul
@@ -1093,7 +1148,7 @@ def bench_floors(f, args):
     emit(out)
 
 
-SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_chunk32_8k": bench_prefill_chunk, "llama3b_prefill_chunk32_32k": lambda f, args: bench_prefill_chunk(f, args, 32, 32736), "llama3b_prefill_chunk64_8k": lambda f, args: bench_prefill_chunk(f, args, 64, 8128), "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_prefill_2k": bench_prefill,
+SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_chunk32_8k": bench_prefill_chunk, "llama3b_prefill_chunk32_32k": lambda f, args: bench_prefill_chunk(f, args, 32, 32736), "llama3b_prefill_chunk64_8k": lambda f, args: bench_prefill_chunk(f, args, 64, 8128), "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_decode_2k": bench_short_decode, "llama3b_decode_512": lambda f, args: bench_short_decode(f, args, 511), "llama3b_prefill_2k": bench_prefill,
              "llama3b_prefill_8k": lambda f, args: bench_prefill(f, args, 8192), "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
