@@ -902,10 +902,11 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
     while (true) {
         const uint32_t next_item = item_of(round + 1);
         const bool has_next = next_item < n_items;
-        // Q, K_0 (for S_0) and K_1 (whose first operands the first VALU phase reads ahead) must be there now; V_0,
-        // requested last (loads complete in order), has until the first MFMA phase. A CU pulls about 25 GB/s on its
-        // own, so every 16 KB not waited for here is worth half a microsecond.
-        if (ntg > 0) __builtin_amdgcn_s_waitcnt(VMCNT_V);
+        // Q and K_0 (for S_0) must be there now; K_1 and V_0, requested after them (loads complete in order), have until
+        // the first MFMA phase. A CU pulls about 25 GB/s on its own, so every 16 KB not waited for here is worth half a
+        // microsecond.
+        if (ntg > 1) __builtin_amdgcn_s_waitcnt(VMCNT_KV);
+        else if (ntg > 0) __builtin_amdgcn_s_waitcnt(VMCNT_V);
         else __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
         {
@@ -979,8 +980,9 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
                         pb[0][ks][jj] = to_elem<BF16>(e);
                     }
                 l_run += (psum[0] + psum[1]) + (psum[2] + psum[3]);
-                k_prefetch((j + 1) & 1);
-                if (j == 0) {  // V_0 has landed: everything but what this phase requested (K_2, V_1)
+                // (K_1 may still be on its way during an item's first phase: its first operands are read after the barrier)
+                if (j > 0) k_prefetch((j + 1) & 1);
+                if (j == 0) {  // K_1 and V_0 have landed: everything but what this phase requested (K_2, V_1)
                     if (ntg > 2) __builtin_amdgcn_s_waitcnt(VMCNT_KV);
                     else if (ntg > 1) __builtin_amdgcn_s_waitcnt(VMCNT_V);
                     else __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -990,6 +992,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a)
             // every wave has taken its query rows out of LDS (each passed a barrier since): the next item's may come
             const bool stage_now = j == 0 && has_next;
             if (stage_now) q_dma(next_item);
+            if (j == 0 && ntg > 0) k_prefetch(1);
             if (j < ntg) mfma_phase(j);  // ---- MFMA phase
             // the rows requested in the last VALU phase have landed (the query rows just requested may take longer)
             if (stage_now) __builtin_amdgcn_s_waitcnt(VMCNT_Q);
