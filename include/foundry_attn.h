@@ -58,6 +58,9 @@ typedef enum fa_status {
 const char *fa_status_name(fa_status s);
 /* Message of the last failing call on this thread ("" if none). Valid until the next failing call. */
 const char *fa_last_error_string(void);
+/* The fa_dtype that the last FA_ERR_UNSUPPORTED_DTYPE of this thread refused (0xffffffff if none yet): the `dtype`
+ * field of MetalError::UnsupportedDtype { operation, dtype } (src/error.rs:22-75). */
+uint32_t fa_last_error_dtype(void);
 
 /* Dtype, same order as metallic-sdk's enum (crates/metallic-sdk/src/tensor.rs:7-30). */
 typedef enum fa_dtype {
@@ -85,11 +88,14 @@ typedef struct fa_graph fa_graph;
 /* Foundry::new (src/lib.rs:57-61). Creates a stream on `device` and a 64 MiB scratch workspace. */
 fa_status fa_ctx_create(int device, fa_ctx **out);
 fa_status fa_ctx_destroy(fa_ctx *ctx);
-/* Foundry::synchronize (src/lib.rs:175-188). Also reports what kernels flagged since the last call: a fused decode
- * step whose device-side position was at or beyond its kv_len_bound or the cache capacity (the token was neither
- * appended nor attended) -> FA_ERR_INVALID_OPERATION, once. Not callable during a capture; the same holds for the
- * other calls that wait for the stream (fa_upload, fa_download, fa_device_free, fa_profile_reset, fa_profile_query):
- * FA_ERR_OPERATION_FAILED, and the capture stays valid. */
+/* Foundry::synchronize (src/lib.rs:175-188). Also reports what kernels flagged since the last report: a polled decode
+ * merge that gave up (FA_ERR_OPERATION_FAILED, see fa_set_decode_variant; it takes precedence and its message names the
+ * other condition when both were raised) or a fused decode step whose device-side position was at or beyond its
+ * kv_len_bound or the cache capacity (the token was neither appended nor attended; FA_ERR_INVALID_OPERATION), once.
+ * Every call that waits for the stream makes the same report - fa_upload, fa_download, fa_device_free (the buffer is
+ * freed all the same), fa_profile_reset, fa_profile_query, fa_stream_timer_stop - so a caller that reads results with
+ * fa_download alone cannot miss it. None of them is callable during a capture: FA_ERR_OPERATION_FAILED, and the capture
+ * stays valid. */
 fa_status fa_synchronize(fa_ctx *ctx);
 /* The context's hipStream_t, for callers that enqueue their own work between the ops. */
 void *fa_ctx_stream(fa_ctx *ctx);
@@ -276,10 +282,18 @@ size_t fa_noalloc_scratch_bytes(void);
  * as the other partitions' records have arrived (one launch, no ticket, the reads spread over all compute units;
  * a head group's workgroups are placed on one XCD where the launch allows, so the records meet in that XCD's L2). It
  * applies to launches whose workgroups are all resident at once (at most one 8-wave or two 4-wave workgroups per compute
- * unit; others take 1). A merging workgroup waits at most FOUNDRY_ATTN_DECODE_POLL_SPIN_US (default 2 s) for the other
- * partitions; beyond that it stores nothing and the next fa_synchronize fails with FA_ERR_OPERATION_FAILED (the outputs
- * of the decode calls since the previous synchronize are then invalid). The three forms fold the same partials in
- * different f32 orders and agree to one f16 unit in the last place; each is deterministic.
+ * unit; others take 1).
+ * Form 2 ASSUMES THAT THE CONTEXT HAS THE GPU'S COMPUTE UNITS TO ITSELF while a decode launch runs: residency is counted
+ * per launch against all compute units of the device. Work of another stream, context or process (or a compute-unit
+ * mask) can hold part of them, and two polled launches can then each wait for workgroups the other keeps from
+ * starting. A merging workgroup therefore waits at most FOUNDRY_ATTN_DECODE_POLL_SPIN_US / fa_set_decode_poll_spin_us
+ * (default 5 ms, hundreds of launch times) for the other partitions; beyond that it stores nothing, every kernel still
+ * ends, and the next call that waits for the stream fails with FA_ERR_OPERATION_FAILED: the outputs of the decode
+ * calls since the previous wait are invalid, the record buffer is restored, and the context switches itself to
+ * merge = 1 until fa_set_decode_variant selects form 2 again. Callers that run several contexts or streams on one GPU
+ * at the same time should set merge = 1 (FOUNDRY_ATTN_DECODE_MERGE=1) from the start.
+ * The three forms fold the same partials in different f32 orders and agree to one f16 unit in the last place; each is
+ * deterministic.
  * Environment: FOUNDRY_ATTN_DECODE_KEYS_PER_SPLIT, FOUNDRY_ATTN_DECODE_MERGE, FOUNDRY_ATTN_DECODE_POLL_SPIN_US,
  * FOUNDRY_ATTN_DECODE_XCD_LOCAL (0 = records always through memory) (read at fa_ctx_create). */
 typedef struct fa_decode_variant {
@@ -287,6 +301,9 @@ typedef struct fa_decode_variant {
     uint32_t merge;
 } fa_decode_variant;
 fa_status fa_set_decode_variant(fa_ctx *ctx, const fa_decode_variant *variant);
+/* The polled merge's wait bound in microseconds (see above; 0 = give up at the first look unless every record is there,
+ * which is how the tests force the give-up path from the host). No counterpart in the reference. */
+fa_status fa_set_decode_poll_spin_us(fa_ctx *ctx, uint32_t spin_us);
 
 /* Prefill split-K override, the counterpart of the reference's prefill split-K selector and its environment
  * override (src/metals/flashattention/step.rs:849-864): the key tiles of every query tile are divided over
@@ -653,6 +670,9 @@ fa_status fa_measure_clock(fa_ctx *ctx, int matrix_load, uint32_t iterations, fl
 const char *fa_version(void);
 fa_status fa_device_info(fa_ctx *ctx, char *name_out, size_t name_cap, uint32_t *compute_units,
                          uint64_t *global_mem_bytes);
+/* Free and total bytes of the context's device memory right now (hipMemGetInfo), for harnesses that check what a call
+ * allocates. Either pointer may be NULL. */
+fa_status fa_device_mem_info(fa_ctx *ctx, uint64_t *free_bytes, uint64_t *total_bytes);
 
 #ifdef __cplusplus
 }

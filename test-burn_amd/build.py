@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libfoundry_attn.so")
 SOURCES = ["fa_api.hip", "fa_kvprep.hip", "fa_decode.hip", "fa_decode_d64.hip", "fa_decode_d128.hip", "fa_decode_d64_w4.hip", "fa_decode_d128_w4.hip", "fa_prefill.hip",
-           "fa_sage.hip", "fa_kvcopy.hip", "fa_qkv.hip", "fa_gemm.hip", "fa_legacy.hip"]
+           "fa_sage.hip", "fa_kvcopy.hip", "fa_qkv.hip", "fa_gemm.hip", "fa_legacy.hip", "fa_probe.hip"]
 HEADERS = [os.path.join(CSRC, "fa_internal.h"), os.path.join(CSRC, "fa_decode_impl.h"), os.path.join(CSRC, "fa_qkv_rope.h"),
            os.path.join(HERE, "..", "include", "foundry_attn.h")]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

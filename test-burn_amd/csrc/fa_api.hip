@@ -21,7 +21,20 @@ fa_status fa_fail(fa_status s, const char *fmt, ...) {
     return s;
 }
 
+// dtype named by the last FA_ERR_UNSUPPORTED_DTYPE of this thread
+static thread_local uint32_t g_err_dtype = 0xffffffffu;
+
+fa_status fa_fail_dtype(uint32_t dtype, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    g_err_dtype = dtype;
+    return FA_ERR_UNSUPPORTED_DTYPE;
+}
+
 extern "C" const char *fa_last_error_string(void) { return g_err; }
+extern "C" uint32_t fa_last_error_dtype(void) { return g_err_dtype; }
 
 extern "C" const char *fa_status_name(fa_status s) {
     switch (s) {
@@ -121,7 +134,7 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     if (s == FA_OK) s = fa_decode_static_scratch(device, &ctx->static_scratch, &ctx->static_scratch_bytes);
     if (s == FA_OK) {
         // Records of the polled merge: room for two workgroups per compute unit serving 16 heads of 128 dims each (32 B per float4 column)
-        ctx->poll_spin_us = env_u32("FOUNDRY_ATTN_DECODE_POLL_SPIN_US", 2000000);
+        ctx->poll_spin_us = env_u32("FOUNDRY_ATTN_DECODE_POLL_SPIN_US", ctx->poll_spin_us);
         const size_t bytes = (size_t)2 * (ctx->n_cus > 0 ? ctx->n_cus : 256) * (16 * 128 / 4) * 32;
         hipError_t he = hipMalloc(&ctx->poll_ws, bytes);
         if (he == hipSuccess) he = hipMemset(ctx->poll_ws, 0xff, bytes);
@@ -129,10 +142,10 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
         else ctx->poll_ws_bytes = bytes;
     }
     if (s == FA_OK) {
-        // one word that kernels set bits in and the host reads after a synchronize: pinned host memory mapped into the device
-        hipError_t he = hipHostMalloc((void **)&ctx->h_status, sizeof(uint32_t), hipHostMallocMapped);
+        // words that kernels raise and the host reads after a wait for the stream: pinned host memory mapped into the device
+        hipError_t he = hipHostMalloc((void **)&ctx->h_status, FA_DEVSTAT_WORDS * sizeof(uint32_t), hipHostMallocMapped);
         if (he == hipSuccess) {
-            *ctx->h_status = 0;
+            memset(ctx->h_status, 0, FA_DEVSTAT_WORDS * sizeof(uint32_t));
             he = hipHostGetDevicePointer((void **)&ctx->d_status, ctx->h_status, 0);
         }
         if (he != hipSuccess) s = fa_fail(FA_ERR_OPERATION_FAILED, "status word allocation failed: %s", hipGetErrorString(he));
@@ -174,28 +187,41 @@ extern "C" fa_status fa_ctx_destroy(fa_ctx *ctx) {
 
 extern "C" void *fa_ctx_stream(fa_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
 
+fa_status fa_check_device_status(fa_ctx *ctx) {
+    if (!ctx->h_status) return FA_OK;
+    volatile uint32_t *w = ctx->h_status;
+    const bool timeout = w[FA_DEVSTAT_MERGE_TIMEOUT] != 0, dropped = w[FA_DEVSTAT_APPEND_DROPPED] != 0;
+    if (!timeout && !dropped) return FA_OK;
+    for (uint32_t i = 0; i < FA_DEVSTAT_WORDS; ++i) w[i] = 0;
+    if (timeout) {
+        // The record buffer no longer holds the arrival pattern everywhere: restore it before anything else runs. The
+        // wait can only run out when this context did not have the GPU's compute units to itself (another stream,
+        // context or process held part of them, or workgroups were not placed as probed), and that may well happen
+        // again: from here on the context merges with the second launch, until fa_set_decode_variant says otherwise.
+        (void)hipMemsetAsync(ctx->poll_ws, 0xff, ctx->poll_ws_bytes, ctx->stream);
+        (void)hipStreamSynchronize(ctx->stream);
+        if (ctx->decode_variant.merge == 2) ctx->decode_variant.merge = 1;
+        return fa_fail(FA_ERR_OPERATION_FAILED,
+                       "a decode launch's merging workgroup waited longer than %u us for the other partitions; the "
+                       "outputs of the decode calls since the last wait for the stream are invalid%s. The context now merges "
+                       "partitions with a second launch (decode merge = 1); fa_set_decode_variant re-enables the polled form",
+                       ctx->poll_spin_us, dropped ? " (a fused decode step was also dropped: position beyond its bound)" : "");
+    }
+    return fa_fail(FA_ERR_INVALID_OPERATION,
+                   "Invalid operation: a fused decode step ran at a position at or beyond its kv_len_bound or the cache "
+                   "capacity; its token was neither appended nor attended");
+}
+
+// hipStreamSynchronize + the report of what kernels flagged
+static fa_status fa_wait_stream(fa_ctx *ctx) {
+    FA_HIP(hipStreamSynchronize(ctx->stream));
+    return fa_check_device_status(ctx);
+}
+
 extern "C" fa_status fa_synchronize(fa_ctx *ctx) {
     FA_NEED(ctx, "ctx");
     if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "cannot synchronize while a capture is active");
-    FA_HIP(hipStreamSynchronize(ctx->stream));
-    if (ctx->h_status && *ctx->h_status) {
-        const uint32_t bits = *ctx->h_status;
-        *ctx->h_status = 0;
-        if (bits & FA_DEVSTAT_MERGE_TIMEOUT) {
-            // the buffer no longer holds the arrival pattern everywhere: restore it before anything else runs
-            (void)hipMemsetAsync(ctx->poll_ws, 0xff, ctx->poll_ws_bytes, ctx->stream);
-            (void)hipStreamSynchronize(ctx->stream);
-            return fa_fail(FA_ERR_OPERATION_FAILED,
-                           "a decode launch's merging workgroup waited longer than %u us for the other partitions; the "
-                           "outputs of the decode calls since the last synchronize are invalid", ctx->poll_spin_us);
-        }
-        if (bits & FA_DEVSTAT_APPEND_DROPPED)
-            return fa_fail(FA_ERR_INVALID_OPERATION,
-                           "Invalid operation: a fused decode step ran at a position at or beyond its kv_len_bound or the cache "
-                           "capacity; its token was neither appended nor attended");
-        return fa_fail(FA_ERR_OPERATION_FAILED, "device status word 0x%x", bits);
-    }
-    return FA_OK;
+    return fa_wait_stream(ctx);
 }
 
 // A buffer whose address may be baked into the kernel arguments of a recorded graph is parked while any graph of this
@@ -293,6 +319,12 @@ extern "C" fa_status fa_set_decode_variant(fa_ctx *ctx, const fa_decode_variant 
     return FA_OK;
 }
 
+extern "C" fa_status fa_set_decode_poll_spin_us(fa_ctx *ctx, uint32_t spin_us) {
+    FA_NEED(ctx, "ctx");
+    ctx->poll_spin_us = spin_us;
+    return FA_OK;
+}
+
 // capture ---------------------------------------------------------------------------------------
 
 extern "C" int fa_is_capturing(fa_ctx *ctx) { return ctx && ctx->capturing ? 1 : 0; }
@@ -375,7 +407,7 @@ extern "C" fa_status fa_profile_reset(fa_ctx *ctx) {
     if (ctx->capturing) return fa_fail(FA_ERR_OPERATION_FAILED, "fa_profile_reset waits for the stream and cannot run while a capture is active");
     FA_HIP(hipStreamSynchronize(ctx->stream));
     prof_recycle(ctx);
-    return FA_OK;
+    return fa_check_device_status(ctx);
 }
 
 extern "C" fa_status fa_profile_query(fa_ctx *ctx, const char *prefix, uint64_t *launches, double *total_ms) {
@@ -395,7 +427,7 @@ extern "C" fa_status fa_profile_query(fa_ctx *ctx, const char *prefix, uint64_t 
     }
     if (launches) *launches = n;
     if (total_ms) *total_ms = ms;
-    return FA_OK;
+    return fa_check_device_status(ctx);
 }
 
 extern "C" fa_status fa_profile_clock_buffer(fa_ctx *ctx, void *d_buffer, uint32_t n_workgroups) {
@@ -427,7 +459,7 @@ extern "C" fa_status fa_stream_timer_stop(fa_ctx *ctx, float *elapsed_ms) {
     FA_HIP(hipEventSynchronize(ctx->timer_stop));
     FA_HIP(hipEventElapsedTime(elapsed_ms, ctx->timer_start, ctx->timer_stop));
     ctx->timer_running = false;
-    return FA_OK;
+    return fa_check_device_status(ctx);
 }
 
 extern "C" fa_status fa_compute_units(fa_ctx *ctx, uint32_t *n) {
@@ -455,7 +487,7 @@ extern "C" fa_status fa_device_free(fa_ctx *ctx, void *ptr) {
     if (!ptr) return FA_OK;
     FA_HIP(hipStreamSynchronize(ctx->stream));
     FA_HIP(hipFree(ptr));
-    return FA_OK;
+    return fa_check_device_status(ctx);
 }
 
 extern "C" fa_status fa_upload(fa_ctx *ctx, void *dst, size_t dst_offset, const void *src_host, size_t bytes) {
@@ -465,8 +497,7 @@ extern "C" fa_status fa_upload(fa_ctx *ctx, void *dst, size_t dst_offset, const 
     FA_NEED(src_host, "src_host");
     if (bytes == 0) return FA_OK;
     FA_HIP(hipMemcpyAsync((char *)dst + dst_offset, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
-    FA_HIP(hipStreamSynchronize(ctx->stream));
-    return FA_OK;
+    return fa_wait_stream(ctx);
 }
 
 extern "C" fa_status fa_download(fa_ctx *ctx, void *dst_host, const void *src, size_t src_offset, size_t bytes) {
@@ -476,8 +507,7 @@ extern "C" fa_status fa_download(fa_ctx *ctx, void *dst_host, const void *src, s
     FA_NEED(src, "src");
     if (bytes == 0) return FA_OK;
     FA_HIP(hipMemcpyAsync(dst_host, (const char *)src + src_offset, bytes, hipMemcpyDeviceToHost, ctx->stream));
-    FA_HIP(hipStreamSynchronize(ctx->stream));
-    return FA_OK;
+    return fa_wait_stream(ctx);
 }
 
 extern "C" fa_status fa_device_memset(fa_ctx *ctx, void *dst, int value, size_t bytes) {
@@ -516,6 +546,16 @@ extern "C" fa_status fa_device_info(fa_ctx *ctx, char *name_out, size_t name_cap
     }
     if (compute_units) *compute_units = (uint32_t)prop.multiProcessorCount;
     if (global_mem_bytes) *global_mem_bytes = (uint64_t)prop.totalGlobalMem;
+    return FA_OK;
+}
+
+extern "C" fa_status fa_device_mem_info(fa_ctx *ctx, uint64_t *free_bytes, uint64_t *total_bytes) {
+    FA_NEED(ctx, "ctx");
+    size_t f = 0, t = 0;
+    FA_HIP(hipSetDevice(ctx->device));
+    FA_HIP(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = (uint64_t)f;
+    if (total_bytes) *total_bytes = (uint64_t)t;
     return FA_OK;
 }
 
@@ -583,7 +623,7 @@ static fa_status check_tensor(const fa_tensor_arg *t, const char *name, fa_dtype
     if (!t->buffer) return fa_fail(FA_ERR_INPUT_NOT_FOUND, "Input not found: %s", name);
     if (t->rank > 4) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %s has rank %u > 4", name, t->rank);
     if (t->dtype != (uint32_t)want)
-        return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "Unsupported dtype %u for %s (expected %u)", t->dtype, name, (unsigned)want);
+        return fa_fail_dtype(t->dtype, "Unsupported dtype %u for %s (expected %u)", t->dtype, name, (unsigned)want);
     if (t->rank > 0 && numel(t) < need_elems)
         return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %s holds %zu elements, %zu needed", name, numel(t), need_elems);
     if (align > 1 && (((uintptr_t)t->buffer + t->offset) % (size_t)align) != 0)
@@ -802,7 +842,7 @@ static fa_status kv_copy_shape(const fa_tensor_arg *t, const char *name, size_t 
     if (t->strides[0] != t->dims[1] * t->dims[2] || t->strides[1] != t->dims[2] || t->strides[2] != 1)
         return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: KV tensor '%s' has unsupported strides [%zu, %zu, %zu], expected [%zu, %zu, 1]",
                        name, t->strides[0], t->strides[1], t->strides[2], t->dims[1] * t->dims[2], t->dims[2]);
-    if (dtype_bytes(t->dtype) == 0) return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "Unsupported dtype %u for KV tensor '%s'", t->dtype, name);
+    if (dtype_bytes(t->dtype) == 0) return fa_fail_dtype(t->dtype, "Unsupported dtype %u for KV tensor '%s'", t->dtype, name);
     return FA_OK;
 }
 
@@ -903,12 +943,12 @@ static fa_status weight_kind(const fa_tensor_arg *w, const fa_tensor_arg *scales
         const size_t need = rows * (k / 32);
         const size_t have = scales->dtype == FA_DTYPE_F16 ? numel(scales) : numel(scales) / 2;  // f16, or the scale bytes
         if (scales->dtype != FA_DTYPE_F16 && scales->dtype != FA_DTYPE_U8 && scales->dtype != FA_DTYPE_I8)
-            return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "%s: %s scales must be f16 values (F16, or their bytes as U8)", what, policy);
+            return fa_fail_dtype(scales->dtype, "%s: %s scales must be f16 values (F16, or their bytes as U8)", what, policy);
         if (scales->rank > 0 && have < need) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: %s holds %zu scales, %zu needed", what, have, need);
         if ((uintptr_t)half_ptr(scales) % 2 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "%s: scales must be 2-byte aligned", what);
         return FA_OK;
     }
-    return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "%s: weight dtype %u: F16, Q8_0 and Q4_0 weights are built, no other block-quantised policy", what, w->dtype);
+    return fa_fail_dtype(w->dtype, "%s: weight dtype %u: F16, Q8_0 and Q4_0 weights are built, no other block-quantised policy", what, w->dtype);
 }
 
 // Checks a FusedQkv call and fills its launch. with_outputs = false: the three token-major outputs are not part of the
@@ -934,10 +974,10 @@ static fa_status fused_qkv_common(fa_ctx *ctx, const fa_tensor_arg *w_q, const f
     FA_TRY(weight_kind(w_v, s_v, "w_v", p->n_kv, p->k_dim, wbits_v));
     const bool q8 = wbits != 16;  // block-quantised (scales present)
     if (wbits != wbits_k || wbits != wbits_v)  // the reference falls back to three separate projections there (qkv_step.rs:243-259)
-        return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: mixed weight dtypes are not supported");
+        return fa_fail_dtype(wbits != wbits_k ? w_k->dtype : w_v->dtype, "FusedQkv: mixed weight dtypes are not supported");
     for (const fa_tensor_arg *t : {input, out_q, out_k, out_v})
         if ((t == input || with_outputs) && t->dtype != FA_DTYPE_F16)
-            return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "FusedQkv: activations must be F16, got dtype %u", t->dtype);
+            return fa_fail_dtype(t->dtype, "FusedQkv: activations must be F16, got dtype %u", t->dtype);
     const uint32_t m = p->m ? p->m : 1;
     if (p->k_dim == 0 || p->n_dim == 0 || p->n_kv == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv k_dim %u n_dim %u n_kv %u", p->k_dim, p->n_dim, p->n_kv);
     if (p->k_dim % 32 != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv: k_dim %u must be a multiple of 32", p->k_dim);
@@ -1092,7 +1132,7 @@ extern "C" fa_status fa_matmul(fa_ctx *ctx, const fa_tensor_arg *a, const fa_ten
     int wbits = 16;
     FA_TRY(weight_kind(b, b_scales, "b", p->n, p->k, wbits));
     const bool q8 = wbits != 16;
-    if (a->dtype != FA_DTYPE_F16 || output->dtype != FA_DTYPE_F16) return fa_fail(FA_ERR_UNSUPPORTED_DTYPE, "MatMul: a and output must be F16");
+    if (a->dtype != FA_DTYPE_F16 || output->dtype != FA_DTYPE_F16) return fa_fail_dtype(a->dtype != FA_DTYPE_F16 ? a->dtype : output->dtype, "MatMul: a and output must be F16");
     if (p->transpose_a) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: transpose_a is not supported");
     if (p->activation != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "MatMul: activation %u is not built", p->activation);
     const uint32_t m = p->m ? p->m : 1;

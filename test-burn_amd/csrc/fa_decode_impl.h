@@ -43,6 +43,7 @@
 // with several rounds of workgroups, where one workgroup's start and end overlap the other's stream.
 #pragma once
 #include "fa_internal.h"
+#include <mutex>
 #include <type_traits>
 
 #ifndef FA_DECODE_NW
@@ -935,7 +936,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     const uint32_t nsplits = (N + a.chunk - 1) / a.chunk;
     // A position at or past the launch bound / the capacity: the token is neither appended nor attended. The host
     // finds the bit at its next synchronize.
-    if (FUSED && n_raw > N && tid == 0 && blockIdx.x == 0 && y == 0 && a.status) *a.status = FA_DEVSTAT_APPEND_DROPPED;
+    if (FUSED && n_raw > N && tid == 0 && blockIdx.x == 0 && y == 0 && a.status) a.status[FA_DEVSTAT_APPEND_DROPPED] = 1u;
     if (split >= nsplits) return;  // uniform over the workgroup
     if (PAGED) {
         // Nothing has been requested yet (a paged cache needs the length first), so the partitions of this
@@ -1278,7 +1279,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         if (nsplits <= 64) {
             ok = a.xcd_local ? coop_merge_in_registers<D, true>(a, b, y, split, nsplits, S, tid)
                              : coop_merge_in_registers<D, false>(a, b, y, split, nsplits, S, tid);
-            if (!ok && lane == 0 && a.status) *a.status = FA_DEVSTAT_MERGE_TIMEOUT;
+            if (!ok && lane == 0 && a.status) a.status[FA_DEVSTAT_MERGE_TIMEOUT] = 1u;
             return;
         }
         __syncthreads();  // the fold above read the LDS region that the merge reuses
@@ -1287,7 +1288,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         } else {
             ok = coop_merge_and_store<D, false>(a, b, y, split, nsplits, S, tid, reinterpret_cast<float *>(smem));
         }
-        if (!ok && tid == 0 && a.status) *a.status = FA_DEVSTAT_MERGE_TIMEOUT;
+        if (!ok && tid == 0 && a.status) a.status[FA_DEVSTAT_MERGE_TIMEOUT] = 1u;
         return;
     }
 
@@ -1345,8 +1346,11 @@ template <int D>
 fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
     const size_t lds = decode_lds_bytes<D>(a.gt);
     {
-        // more than 64 KiB of dynamic LDS has to be allowed per kernel, once
-        static bool lds_allowed_on[64] = {};  // per device
+        // more than 64 KiB of dynamic LDS has to be allowed per kernel, once per device (contexts of several threads
+        // may get here together)
+        static std::mutex lds_mu;
+        static bool lds_allowed_on[64] = {};
+        std::lock_guard<std::mutex> lds_lock(lds_mu);
         bool &lds_allowed = lds_allowed_on[ctx->device & 63];
         if (!lds_allowed) {
             const int cap = (int)decode_lds_bytes<D>(MAX_GT);

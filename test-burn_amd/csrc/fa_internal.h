@@ -51,13 +51,14 @@ struct fa_ctx {
     void *poll_ws = nullptr;
     size_t poll_ws_bytes = 0;
     bool xcd_round_robin = false;  // workgroups whose ids are equal modulo 8 share an XCD on this device (probed at creation)
-    uint32_t poll_spin_us = 2000000;  // bound of a merging workgroup's wait for the other partitions
+    uint32_t poll_spin_us = 5000;  // bound of a merging workgroup's wait for the other partitions (hundreds of launch times)
     // The library's static device array on this device (decode partials of the entry point that allocates nothing)
     void *static_scratch = nullptr;
     size_t static_scratch_bytes = 0;
-    // Sticky status word written by kernels (pinned host memory, mapped into the device): FA_DEVSTAT_* bits.
-    uint32_t *h_status = nullptr;  // host view
-    uint32_t *d_status = nullptr;  // device view of the same word
+    // Sticky status words written by kernels (pinned host memory, mapped into the device): one word per condition
+    // (FA_DEVSTAT_*), so that a kernel raises one with a plain store and no store can erase another condition.
+    uint32_t *h_status = nullptr;  // host view, FA_DEVSTAT_WORDS words
+    uint32_t *d_status = nullptr;  // device view of the same words
     fa_decode_variant decode_variant{0, 1};
     uint32_t decode_waves = 0;     // waves per decode workgroup: 0 = by launch size, 4 or 8
     uint32_t gemm_variant = 0;     // GEMM kernel: 0 = auto, 1 = tiles through registers, 2 / 3 = straight into LDS in steps of 64 / 32 features
@@ -79,6 +80,8 @@ struct fa_ctx {
 
 // Error plumbing --------------------------------------------------------------------------------
 fa_status fa_fail(fa_status s, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+// FA_ERR_UNSUPPORTED_DTYPE with the offending dtype kept for fa_last_error_dtype()
+fa_status fa_fail_dtype(uint32_t dtype, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 
 #define FA_HIP(expr)                                                                                       \
     do {                                                                                                   \
@@ -201,7 +204,7 @@ struct FaDecodeDev {
     uint64_t qin_stride_b, kvin_stride_b, qrot_stride_b;
     uint32_t rope_normal, apply_rope, table_rows;
     uint32_t bf16;  // data tensors are bf16 (RoPE tables stay f16)
-    uint32_t *status;  // the context's device-written status word (FA_DEVSTAT_* bits)
+    uint32_t *status;  // the context's device-written status words (one per FA_DEVSTAT_* condition)
     uint32_t xcd_local;  // polled merge: a head group's workgroups share an XCD and exchange partials through its L2
     unsigned long long poll_ticks;  // polled merge: how long the merging workgroup waits for partials, 100 MHz ticks
     // SAGE + FUSED (the int8 decode step in one launch): q is the raw f16 projection, k the int8 cache (written: the open
@@ -285,10 +288,14 @@ fa_status fa_launch_sage_append(fa_ctx *ctx, const SageAppendLaunch &l);
 fa_status fa_launch_sage_tail_copy(fa_ctx *ctx, const void *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim,
                                    uint32_t kv_len, void *tail);
 
-// Bits of the context's device-written status word
-constexpr uint32_t FA_DEVSTAT_MERGE_TIMEOUT = 1u;  // a merging workgroup gave up waiting for a partition's partial
-constexpr uint32_t FA_DEVSTAT_APPEND_DROPPED = 2u;
-constexpr uint32_t FA_DEVSTAT_XCD_PLACEMENT = 4u;  // a workgroup did not run on the XCD its id implies (L2-local merge) // a fused decode step's position was beyond its launch bound / capacity
+// The context's device-written status words: a kernel stores 1 into the word of the condition it met.
+constexpr uint32_t FA_DEVSTAT_MERGE_TIMEOUT = 0u;   // a merging workgroup gave up waiting for a partition's partial
+constexpr uint32_t FA_DEVSTAT_APPEND_DROPPED = 1u;  // a fused decode step's position was beyond its launch bound / capacity
+constexpr uint32_t FA_DEVSTAT_WORDS = 4u;
+// Reads and clears the status words after the stream has been waited for; restores what a reported condition left
+// behind (the polled merge's record buffer) and returns the condition as an error. Every entry point that waits for the
+// stream ends with it.
+fa_status fa_check_device_status(fa_ctx *ctx);
 
 fa_status fa_ensure_workspace(fa_ctx *ctx, size_t bytes);
 fa_status fa_ensure_counters(fa_ctx *ctx, uint32_t n);

@@ -124,7 +124,7 @@ __global__ void __launch_bounds__(256) sage_append_kernel(SageAppendDev a) {
     const uint32_t n_raw = (a.d_position ? *a.d_position : a.position) + 1;
     const uint32_t lim = a.bound < a.capacity ? a.bound : a.capacity;
     if (n_raw > lim) {  // beyond the launch bound or the cache: nothing is appended (reported at the next synchronize)
-        if (blockIdx.x == 0 && tid == 0 && a.status) *a.status = FA_DEVSTAT_APPEND_DROPPED;
+        if (blockIdx.x == 0 && tid == 0 && a.status) a.status[FA_DEVSTAT_APPEND_DROPPED] = 1u;
         return;
     }
     const uint32_t P = n_raw - 1;

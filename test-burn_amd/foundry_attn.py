@@ -29,6 +29,7 @@ class FoundryError(RuntimeError):
     def __init__(self, status, message):
         self.status = status
         self.variant = STATUS_NAMES.get(status, "Unknown")
+        self.dtype = load().fa_last_error_dtype() if status == 7 else None  # UnsupportedDtype names the refused dtype
         super().__init__("%s: %s" % (self.variant, message))
 
 
@@ -90,6 +91,7 @@ _vp, _u32, _sz, _i = C.c_void_p, C.c_uint32, C.c_size_t, C.c_int
 PROTOTYPES = {
     "fa_status_name": [_i],
     "fa_last_error_string": [],
+    "fa_last_error_dtype": [],
     "fa_version": [],
     "fa_ctx_create": [_i, C.POINTER(_vp)],
     "fa_ctx_destroy": [_vp],
@@ -126,6 +128,7 @@ PROTOTYPES = {
     "fa_decode_step_fused_paged": [_vp, _PT, _PT, _PT, _PT, C.POINTER(PagedKv), _PT, _PT, _PT,
                                    C.POINTER(KvPrepFusedParams), _u32],
     "fa_set_decode_variant": [_vp, C.POINTER(DecodeVariant)],
+    "fa_set_decode_poll_spin_us": [_vp, C.c_uint32],
     "fa_set_prefill_split_k": [_vp, C.c_uint32],
     "fa_set_prefill_variant": [_vp, C.c_uint32],
     "fa_set_sage_step_variant": [_vp, C.c_uint32],
@@ -162,10 +165,11 @@ PROTOTYPES = {
     "fa_sdpa_reference": [_vp, _PT, _PT, _PT, _PT, _i, _u32, _u32, _u32, _u32, _u32, _i],
     "fa_measure_clock": [_vp, _i, _u32, C.POINTER(C.c_float), C.POINTER(C.c_float)],
     "fa_device_info": [_vp, C.c_char_p, _sz, C.POINTER(_u32), C.POINTER(C.c_uint64)],
+    "fa_device_mem_info": [_vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
 }
 _RESTYPES = {"fa_status_name": C.c_char_p, "fa_last_error_string": C.c_char_p, "fa_version": C.c_char_p,
              "fa_ctx_stream": _vp, "fa_is_capturing": _i, "fa_align_capacity": _sz, "fa_grown_capacity": _sz,
-             "fa_noalloc_scratch_bytes": _sz}
+             "fa_noalloc_scratch_bytes": _sz, "fa_last_error_dtype": _u32}
 
 _lib = None
 
@@ -318,6 +322,10 @@ class Foundry:
         v = DecodeVariant(keys_per_split, merge)
         check(self.lib.fa_set_decode_variant(self.h, C.byref(v)))
 
+    def set_decode_poll_spin_us(self, spin_us):
+        """How long a merging workgroup of the polled decode merge waits for the other partitions' records."""
+        check(self.lib.fa_set_decode_poll_spin_us(self.h, spin_us))
+
     def set_gemm_variant(self, variant=0):
         """0 = auto; 1 = GEMM operand tiles through registers; 2 / 3 = straight into LDS in steps of 64 / 32 features."""
         check(self.lib.fa_set_gemm_variant(self.h, variant))
@@ -348,6 +356,12 @@ class Foundry:
         cus, mem = _u32(), C.c_uint64()
         check(self.lib.fa_device_info(self.h, name, 256, C.byref(cus), C.byref(mem)))
         return name.value.decode(), cus.value, mem.value
+
+    def device_mem_info(self):
+        """(free, total) bytes of device memory right now."""
+        free, total = C.c_uint64(), C.c_uint64()
+        check(self.lib.fa_device_mem_info(self.h, C.byref(free), C.byref(total)))
+        return free.value, total.value
 
     # -- memory
     def empty(self, shape, dtype=np.float16):

@@ -43,16 +43,21 @@ class MetalError : public std::runtime_error {
         OperationFailed = FA_ERR_OPERATION_FAILED,
         InputNotFound = FA_ERR_INPUT_NOT_FOUND,
     };
-    MetalError(Variant v, const std::string &msg) : std::runtime_error(std::string(variant_name(v)) + ": " + msg), variant_(v) {}
+    MetalError(Variant v, const std::string &msg, uint32_t dtype = 0xffffffffu)
+        : std::runtime_error(std::string(variant_name(v)) + ": " + msg), variant_(v), dtype_(dtype) {}
     Variant variant() const { return variant_; }
+    // UnsupportedDtype { operation, dtype } (src/error.rs:22-75): the fa_dtype that was refused, 0xffffffff for other variants
+    uint32_t dtype() const { return dtype_; }
     static const char *variant_name(Variant v) { return fa_status_name((fa_status)v); }
 
   private:
     Variant variant_;
+    uint32_t dtype_;
 };
 
 inline void check(fa_status s) {
-    if (s != FA_OK) throw MetalError((MetalError::Variant)s, fa_last_error_string());
+    if (s != FA_OK)
+        throw MetalError((MetalError::Variant)s, fa_last_error_string(), s == FA_ERR_UNSUPPORTED_DTYPE ? fa_last_error_dtype() : 0xffffffffu);
 }
 
 // ---------------------------------------------------------------------------------------------- tensors

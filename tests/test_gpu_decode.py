@@ -359,42 +359,52 @@ def test_polled_merge_equals_merge_kernel_over_many_launches():
 
 def test_polled_merge_gives_up_cleanly():
     """Failure handling of the polled merge, forced from the host: with a wait bound of zero a merging workgroup gives
-    up at its first look unless every record is already there. Every kernel still ends normally; the next synchronize
-    reports OperationFailed and restores the buffer; a context with the normal bound computes the right result."""
-    import os
+    up at its first look unless every record is already there. Every kernel still ends normally. The give-up is
+    reported by whichever call waits for the stream next (here a download, with no synchronize in between), the record
+    buffer is restored, and the context falls back to the two-launch merge until the polled form is selected again -
+    which, with the normal bound, is then right on the SAME context."""
     announce("polled merge, zero wait bound")
     H, Hkv, D, cap, n = 24, 8, 128, 4096, 4000
     rng = np.random.default_rng(77)
     q, k, v = h16(rng.normal(size=(H, D))), h16(rng.normal(size=(Hkv, cap, D))), h16(rng.normal(size=(Hkv, cap, D)))
     want = orc.sdpa_decode(q, k, v, H, Hkv, D, cap, n).reshape(H, D)
-    os.environ["FOUNDRY_ATTN_DECODE_POLL_SPIN_US"] = "0"
+    g = fa.Foundry(0)
     try:
-        g = fa.Foundry(0)
-    finally:
-        del os.environ["FOUNDRY_ATTN_DECODE_POLL_SPIN_US"]
-    try:
-        g.set_decode_variant(0, 2)
         dq, dk, dv, do = g.array(q), g.array(k), g.array(v), g.zeros((1, H * D))
+        dropped = g.array(np.array([cap + 5], np.uint32))
+        kc, vc = g.zeros((Hkv, cap, D)), g.zeros((Hkv, cap, D))
+        cos, sin, raw = g.zeros((cap, D // 2)), g.zeros((cap, D // 2)), g.zeros((1, H * D))
         failures = 0
-        for _ in range(4):
+        for it in range(4):
+            g.set_decode_variant(0, 2)
+            g.set_decode_poll_spin_us(0)
             g.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), do.arg(), True, n - 1, H, D, n, 1)
+            if it == 0:
+                # a second condition raised behind the first (a fused step at a position past its cache) must not erase it
+                g.decode_step_fused(raw.arg(), raw.arg((1, Hkv * D)), raw.arg((1, Hkv * D)), None, kc.arg(), vc.arg(), cos.arg(),
+                                    sin.arg(), raw.arg(), fa.KvPrepFusedParams.make(H, Hkv, D, 1, 0, cap), d_position=dropped,
+                                    kv_len_bound=cap)
             try:
-                g.synchronize()
-                assert max_abs(do.download().reshape(H, D), want) <= TOL  # nobody had to wait: the result must be right
+                got = do.download().reshape(H, D)  # waits for the stream: the report comes from here
+                assert it > 0, "the dropped step of the first iteration was not reported"
+                assert max_abs(got, want) <= TOL   # nobody had to wait: the result must be right
             except fa.FoundryError as e:
+                if it == 0 and "waited longer" not in str(e):
+                    assert e.variant == "InvalidOperation"  # only the dropped step was flagged (nobody had to wait)
+                    continue
                 failures += 1
                 assert e.variant == "OperationFailed" and "waited longer" in str(e)
-        # the two-launch merge of the same context is unaffected
-        g.set_decode_variant(0, 1)
-        g.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), do.arg(), True, n - 1, H, D, n, 1)
+                assert it > 0 or "also dropped" in str(e)  # both conditions of the first iteration survive
+                # the context has fallen back to the two-launch merge
+                g.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), do.arg(), True, n - 1, H, D, n, 1)
+                assert max_abs(do.download().reshape(H, D), want) <= TOL
+            g.synchronize()  # nothing is left over
+        # the polled form again on the same context, normal bound: right, repeatedly (the record buffer was restored)
+        g.set_decode_poll_spin_us(5000)
+        g.set_decode_variant(0, 2)
+        for _ in range(3):
+            g.flash_attention(dq.arg((1, H * D)), dk.arg(), dv.arg(), do.arg(), True, n - 1, H, D, n, 1)
+            assert max_abs(do.download().reshape(H, D), want) <= TOL
         g.synchronize()
-        assert max_abs(do.download().reshape(H, D), want) <= TOL
     finally:
         g.close()
-    f = ctx()
-    f.set_decode_variant(0, 2)
-    try:
-        got = gpu_decode(q, k, v, H, D, n)
-    finally:
-        f.set_decode_variant()
-    assert max_abs(got, want) <= TOL

@@ -120,7 +120,7 @@ def test_kv_prep_errors():
     assert e.value.variant == "InputNotFound" and "k" in str(e.value)
     with pytest.raises(fa.FoundryError) as e:
         call(good, q=bufs["q"].arg(dtype=fa.DTYPE_F32))
-    assert e.value.variant == "UnsupportedDtype"
+    assert e.value.variant == "UnsupportedDtype" and e.value.dtype == fa.DTYPE_F32  # the refused dtype travels with the error
     with pytest.raises(fa.FoundryError) as e:
         call(good, kc=bufs["kc"].arg((Hkv, cap // 2, D)))
     assert e.value.variant == "InvalidShape"

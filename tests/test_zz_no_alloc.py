@@ -108,3 +108,32 @@ def test_noalloc_rejects_what_does_not_fit():
         f.set_decode_variant(0, 1)
     for b in (dkc, dvc, dq, dk, dv, dcos, dsin, dout, dq2, dout2):
         b.free()
+
+
+def test_noalloc_leaves_device_memory_untouched():
+    """The property the entry point is named for: between two readings of the device's free memory, a call of it (and the
+    wait for its kernels) allocates and frees nothing. The allocating entry point runs the same shape first, so that the
+    kernels' code is resident before the first reading."""
+    f = ctx()
+    announce("noalloc decode step: free device memory before and after")
+    rng = np.random.default_rng(11)
+    H, Hkv, D, cap, pos = 24, 8, 128, 4096, 4000
+    cos, sin = fa.rope_tables(5e5, D, cap)
+    dkc, dvc = f.array(h16(rng.normal(size=(Hkv, cap, D)))), f.array(h16(rng.normal(size=(Hkv, cap, D))))
+    dq, dk, dv = (f.array(h16(rng.normal(size=(1, n * D)))) for n in (H, Hkv, Hkv))
+    dcos, dsin, dout = f.array(cos), f.array(sin), f.zeros((1, H * D))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, 1, pos, cap, fa.ROPE_NORMAL)
+    args = (dq.arg(), dk.arg(), dv.arg(), None, dkc.arg(), dvc.arg(), dcos.arg(), dsin.arg(), dout.arg(), p)
+    f.set_decode_variant(0, 1)
+    try:
+        f.decode_step_fused(*args)
+        f.synchronize()
+        before = f.device_mem_info()[0]
+        for _ in range(3):
+            f.decode_step_fused(*args, noalloc=True)
+        f.synchronize()
+        assert f.device_mem_info()[0] == before
+    finally:
+        f.set_decode_variant()
+    for b in (dkc, dvc, dq, dk, dv, dcos, dsin, dout):
+        b.free()
