@@ -259,14 +259,10 @@ def bench_prefill(f, args, tokens=2048):
         f.kv_prep_fused_paged(dq.arg(), dk.arg(), dv.arg(), dqr.arg(), desc, 0, dcos.arg(), dsin.arg(), p)
         f.flash_prefill_paged(dqr.arg(), desc, 0, dout.arg(), True, 0, H, M, M)
 
-    for _ in range(args.warmup):
-        step()
+    step()
     f.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    f.synchronize()
-    dt = time.perf_counter() - t0
+    # a step's device time: (append, attention) pairs recorded into a HIP graph and replayed between two events on the stream
+    per_step, n_timed = graph_replay_seconds(f, lambda i: step(), 8 if M <= 2048 else 2, args.warmup, min(args.steps, 80 if M <= 2048 else 8))
 
     # parity: cache bit-exact against the oracle's append; the last 64 query rows against the oracle's prefill
     import orc  # the CPU oracle is only the checker here
@@ -314,11 +310,13 @@ def bench_prefill(f, args, tokens=2048):
     append_bytes = 2.0 * M * (H + 2 * Hkv) * D * 2  # read q, k, v; write q_rot and the cache rows
     result = {
         "metric": "prefill-attn steps/s + achieved f16 MFMA TFLOP/s (%% peak), Llama-3.2-3B shape, %d tokens" % M,
-        "value": args.steps / dt, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": 1.0 / per_step, "unit": "steps/s", "n_gpus": 1, "steps": n_timed, "warmup": args.warmup,
+        "ms_per_step": per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
+        "timing": "ms_per_step = device time per step: HIP graph replays between two events on the kernels' stream",
         "config": {"workload": "llama3.2-3b prefill attention, one layer: RoPE + append of %d tokens into an empty paged "
-                               "f16 cache (16-token blocks, permuted block table), then causal flash prefill, H24/Hkv8/D128" % M},
+                               "f16 cache (16-token blocks, permuted block table), then causal flash prefill, H24/Hkv8/D128, "
+                               "graph replays" % M},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_F16_PEAK_TFLOPS, "traffic": None, "kernel": pf_kernel,
                      "avg_launch_us": avg_pf_s * 1e6, "launches": n_pf, "flops_per_launch": flops,
@@ -334,21 +332,74 @@ def bench_prefill(f, args, tokens=2048):
         sys.exit("parity check failed: cache_bit_exact=%s prefill_max_abs_err=%g" % (cache_ok, err))
 
 
-def _finish_secondary(f, args, name, workload, kernel, bytes_per_launch, dt, parity, extra=None, unit="layer-steps/s"):
+def graph_replay_seconds(f, step, per_graph, warmup, steps):
+    """Device seconds per step of `step(i)` recorded `per_graph` times into one HIP graph and replayed: two events on the
+    kernels' stream around the replays (per-dispatch profiling off), divided by the steps in them. Returns (seconds per
+    step, steps timed)."""
+    f.start_capture()
+    for i in range(per_graph):
+        step(i)
+    graph = f.end_capture()
+    for _ in range(max(1, warmup // per_graph)):
+        graph.launch()
+    f.synchronize()
+    reps = max(1, steps // per_graph)
+    f.timer_start()
+    for _ in range(reps):
+        graph.launch()
+    per_step = f.timer_stop() / 1e3 / (reps * per_graph)
+    graph.destroy()
+    return per_step, reps * per_graph
+
+
+def eager_kernel_us(f, step, n_steps, kernels):
+    """{kernel: (launches, average us)} from an eager pass with HIP events attached to every dispatch (the events add a few
+    tenths of a microsecond to what they measure)."""
+    f.profile_reset()
+    f.profile_enable(True)
+    for i in range(n_steps):
+        step(i)
+    out = {}
+    for k in kernels:
+        n, ms = f.profile_query(k)
+        if n:
+            out[k] = (n, ms * 1e3 / n)
+    f.profile_enable(False)
+    f.profile_reset()
+    return out
+
+
+def _finish_secondary(f, args, name, workload, kernel, bytes_per_launch, dt, parity, extra=None, unit="layer-steps/s",
+                      graph=None):
+    """graph = (device seconds per step from graph replays, steps timed): then `value` and `ms_per_step` are device time per
+    step, and - when the step is that one kernel - so is the roofline's launch duration; the eager per-dispatch event
+    figure stays as a sub-field. Without it (legacy lines) the host's wall time over eager launches is reported."""
     n, ms = f.profile_query(kernel)
-    avg_s = ms / 1e3 / max(1, n)
+    eager_s = ms / 1e3 / max(1, n)
+    steps = args.steps
+    if graph is not None:
+        per_step, steps = graph
+        dt = per_step * steps
+    one_kernel_step = graph is not None and (extra or {}).get("kernels_per_step", 1) == 1
+    avg_s = graph[0] if one_kernel_step else eager_s
     achieved = bytes_per_launch / avg_s / 1e9
     result = {
-        "metric": name, "value": args.steps / dt, "unit": unit, "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True, "scaling": "weak",
+        "metric": name, "value": steps / dt, "unit": unit, "n_gpus": 1, "steps": steps,
+        "warmup": args.warmup, "ms_per_step": dt / steps * 1e3, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic", "config": {"workload": workload},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": kernel, "avg_launch_us": avg_s * 1e6,
-                     "launches": n, "bytes_per_launch": bytes_per_launch},
+                     "launches": steps if one_kernel_step else n, "bytes_per_launch": bytes_per_launch,
+                     "timing": ("HIP events on the stream around the graph replays / launches in them" if one_kernel_step
+                                else "HIP events around each eager dispatch"),
+                     "eager_dispatch_avg_launch_us": eager_s * 1e6, "eager_dispatch_launches": n},
         "parity": parity,
     }
+    if graph is not None:
+        result["timing"] = "ms_per_step = device time per step: HIP graph replays between two events on the kernels' stream"
+        result["whole_step_hbm_frac_of_peak"] = bytes_per_launch / graph[0] / 1e9 / HBM_PEAK_GBPS
     if extra:
-        result.update(extra)
+        result.update({k: v for k, v in extra.items() if k != "kernels_per_step"})
     emit(result)
 
 
@@ -382,21 +433,16 @@ def bench_small_decode(f, args):
     want = orc.sdpa_decode(want_qr[:, 0].copy(), host[0], host[1], H, Hkv, D, cap, pos + 1)
     err = float(np.max(np.abs(dout.download().reshape(-1).astype(np.float64) - want.reshape(-1).astype(np.float64))))
     ok = bool(np.array_equal(caches[0][0].download().view(np.uint16), host[0].view(np.uint16)))
-    for i in range(args.warmup):
-        step(i)
-    f.synchronize()
+    graph = graph_replay_seconds(f, step, 4 * NL, args.warmup, args.steps)
     f.profile_reset()
     f.profile_enable(True)
-    t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(2 * NL):
         step(i)
-    f.synchronize()
-    dt = time.perf_counter() - t0
     nbytes = 2.0 * Hkv * (pos + 1) * D * 2 + 2 * Hkv * D * 2 + 2 * H * D * 2 + 2 * D
     _finish_secondary(f, args, "decode-attn layer-steps/s + achieved HBM GB/s, Qwen2.5-0.5B shape @1K ctx",
                       "qwen2.5-0.5b single-layer decode step: RoPE + KV append + flash decode, batch 1, H14/Hkv2/D64, "
-                      "kv_len 1025, eager launches (profiling events on)", "fused_rope_append_decode_kernel", nbytes, dt,
-                      {"cache_bit_exact": ok, "decode_max_abs_err": err})
+                      "kv_len 1025, graph replays over 16 layers' caches", "fused_rope_append_decode_kernel", nbytes, 0.0,
+                      {"cache_bit_exact": ok, "decode_max_abs_err": err}, graph=graph)
     f.profile_enable(False)
 
 
@@ -955,23 +1001,22 @@ def bench_paged_decode(f, args):
                                orc.make_params(H, Hkv, D, 1, n, n + 1, rope_mode=0))
         want = orc.sdpa_decode(qr[:, 0].copy(), kc, vc, H, Hkv, D, n + 1, n + 1, n_threads=8).reshape(H, D)
         err = max(err, float(np.max(np.abs(got[b_].astype(np.float64) - want.astype(np.float64)))))
-    for i in range(args.warmup):
-        step(i)
-    f.synchronize()
+    graph = graph_replay_seconds(f, step, 4 * NL, args.warmup, args.steps)
     f.profile_reset()
     f.profile_enable(True)
-    t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(4 * NL):
         step(i)
-    f.synchronize()
-    dt = time.perf_counter() - t0
+    n_mrg, ms_mrg = f.profile_query("flash_decode_merge_kernel")
     total = float(np.sum(lens.astype(np.float64) + 1))
     nbytes = 2.0 * Hkv * total * D * 2 + B * (2 * Hkv * D * 2 + 2 * H * D * 2 + 2 * D + 4) + 4.0 * sum(need)
     _finish_secondary(f, args, "paged decode-attn layer-steps/s + achieved HBM GB/s, Qwen2.5-3B shape, 32 ragged sequences",
                       "qwen2.5-3b batched paged decode, one layer per step: 32 sequences of %d..%d tokens (sum %d), "
                       "H16/Hkv2/D128, 16-token blocks with a permuted block table, RoPE + append + flash decode in one "
-                      "launch + merge" % (int(lens.min()), int(lens.max()), int(lens.sum())),
-                      "fused_rope_append_decode_kernel", nbytes, dt, {"decode_max_abs_err_3_sequences": err})
+                      "launch%s, graph replays over 4 layers' pools" % (int(lens.min()), int(lens.max()), int(lens.sum()),
+                                                                       " + merge launch" if n_mrg else ", merge inside"),
+                      "fused_rope_append_decode_kernel", nbytes, 0.0, {"decode_max_abs_err_3_sequences": err},
+                      {"kernels_per_step": 2 if n_mrg else 1,
+                       "merge_kernel_avg_launch_us": (ms_mrg * 1e3 / n_mrg) if n_mrg else None}, graph=graph)
     f.profile_enable(False)
 
 
@@ -1116,6 +1161,30 @@ def bench_floors(f, args):
                                "what": "fa_kv_prefix_copy of one [8, %d, 128] f16 tensor (half read, half written), %d "
                                        "tensor pairs in rotation, HIP graph" % (rows, n_rot)}
         for b in srcs + dsts:
+            b.free()
+    # Launches that only READ as many bytes: the column-sum kernel behind fa_sage_k_mean (it streams its input once with
+    # 16-byte non-temporal loads and stores a few KB of partial sums; a second, tiny launch finishes the mean), over
+    # [16, rows, 128] f16 tensors in rotation. The read-only launch by itself is timed with events attached to its eager
+    # dispatches; the pair as graph replays.
+    for name, rows, n_rot in (("read_33.6MB", 8200, 28), ("read_240MB", 58594, 8)):
+        heads = 16
+        srcs = [f.zeros((heads, rows, D)) for _ in range(n_rot)]
+        mean = f.zeros((heads, D), np.float32)
+
+        def read_step(i):
+            f.sage_k_mean(srcs[i % n_rot], heads, rows, D, rows, mean)
+
+        pair_s, _ = graph_replay_seconds(f, read_step, n_rot, 3 * n_rot, 20 * n_rot)
+        ev = eager_kernel_us(f, read_step, 4 * n_rot, ("sage_k_colsum_kernel", "sage_k_mean_finish_kernel"))
+        us = ev["sage_k_colsum_kernel"][1]
+        nread = float(heads * rows * D * 2)
+        out["floors"][name] = {"kernel": "sage_k_colsum_kernel", "bytes_read": nread, "us_per_launch": us,
+                               "gbps": nread / us / 1e3, "frac_of_hbm_peak": nread / us / 1e3 / HBM_PEAK_GBPS,
+                               "finish_kernel_us": ev["sage_k_mean_finish_kernel"][1], "graph_us_per_call_both_kernels": pair_s * 1e6,
+                               "what": "the streaming launch of fa_sage_k_mean over one [16, %d, 128] f16 tensor (read once, "
+                                       "%d tensors in rotation): HIP events attached to its eager dispatches; "
+                                       "graph_us_per_call_both_kernels = that launch + the finish launch as graph replays" % (rows, n_rot)}
+        for b in srcs + [mean]:
             b.free()
     word.free()
     # Shader clock the board sustains: under back-to-back MFMAs on every CU (fa_measure_clock), and inside the prefill

@@ -12,15 +12,19 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-OBJ = os.path.join(HERE, "build")
-LIB = os.path.join(HERE, "libfoundry_attn.so")
+# FOUNDRY_ATTN_BUILD_FLAGS (extra hipcc flags) and FOUNDRY_ATTN_BUILD_TAG (suffix of the object directory and of the
+# library name) make a second, differently configured library next to the product one, e.g. a development build with
+# -DFA_DECODE_TRACE; foundry_attn.py loads it when FOUNDRY_ATTN_LIB names it.
+TAG = os.environ.get("FOUNDRY_ATTN_BUILD_TAG", "")
+OBJ = os.path.join(HERE, "build" + TAG)
+LIB = os.path.join(HERE, "libfoundry_attn%s.so" % TAG)
 SOURCES = ["fa_api.hip", "fa_kvprep.hip", "fa_decode.hip", "fa_decode_d64.hip", "fa_decode_d128.hip", "fa_decode_d64_w4.hip", "fa_decode_d128_w4.hip", "fa_prefill.hip",
            "fa_sage.hip", "fa_kvcopy.hip", "fa_qkv.hip", "fa_gemm.hip", "fa_legacy.hip", "fa_probe.hip"]
 HEADERS = [os.path.join(CSRC, "fa_internal.h"), os.path.join(CSRC, "fa_decode_impl.h"), os.path.join(CSRC, "fa_qkv_rope.h"),
            os.path.join(HERE, "..", "include", "foundry_attn.h")]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Wall", "-Wno-unused-function",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"] + os.environ.get("FOUNDRY_ATTN_BUILD_FLAGS", "").split()
 
 
 def _stale(src, obj):

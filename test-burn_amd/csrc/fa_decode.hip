@@ -183,6 +183,9 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
             a.counters = ctx->counters;
         }
     }
+#ifdef FA_DECODE_TRACE
+    a.trace = (ctx->clock_buf && (uint64_t)S * ny * L.batch * (waves * 16 / 2) <= ctx->clock_buf_workgroups) ? ctx->clock_buf : nullptr;
+#endif
     int mode = MODE_PLAIN;
     if (L.sage_fused)
         mode = MODE_SAGE_FUSED;

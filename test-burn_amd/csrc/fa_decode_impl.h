@@ -536,6 +536,30 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: tile addresses stay in SGPRs
     const int n = lane & 15, c = lane >> 4;  // MFMA column (head slot / key row) and 16-lane row
+#ifdef FA_DECODE_TRACE
+    // Development builds (-DFA_DECODE_TRACE): every wave keeps 16 wall-clock stamps (100 MHz) of its phases in scalar
+    // registers and leaves them in the buffer set with fa_profile_clock_buffer when it ends.
+    unsigned long long tstamp[16] = {};
+#define FA_TR(i)                                   \
+    do {                                           \
+        __builtin_amdgcn_sched_barrier(0);         \
+        tstamp[i] = wall_clock64();                \
+        __builtin_amdgcn_sched_barrier(0);         \
+    } while (0)
+#define FA_TR_FLUSH()                                                                                               \
+    do {                                                                                                            \
+        if (a.trace && lane < 16) {                                                                                 \
+            const size_t wg = blockIdx.x + gridDim.x * (blockIdx.y + (size_t)gridDim.y * blockIdx.z);               \
+            unsigned long long v = 0;                                                                               \
+            for (int i = 0; i < 16; ++i) v = lane == i ? tstamp[i] : v;                                             \
+            a.trace[(wg * NW + wave) * 16 + lane] = v;                                                              \
+        }                                                                                                           \
+    } while (0)
+    FA_TR(0);
+#else
+#define FA_TR(i) do { } while (0)
+#define FA_TR_FLUSH() do { } while (0)
+#endif
     // Consecutive workgroup ids go to consecutive XCDs (8). With the partition index taken straight from blockIdx.x
     // and a partition count that is a multiple of 8 (or 4), partition p of EVERY sequence lands on the same XCD -
     // and in a ragged batch the low partitions always exist while the high ones are mostly empty: some XCDs queue
@@ -858,6 +882,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             __builtin_amdgcn_sched_barrier(0);
             __syncthreads();  // releases the streaming waves
             __builtin_amdgcn_sched_barrier(0);
+            FA_TR(1);
             n_raw = read_len();
             const uint32_t p0 = min(n_raw, min(a.capacity, a.kv_len_bound)) - 1;
             if (rope_on) {
@@ -907,8 +932,10 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
             if (lane == 0) __hip_atomic_store(&sm_q_ready, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             __builtin_amdgcn_s_setprio(0);
+            FA_TR(2);
         } else {
             __syncthreads();  // wave 0 has queued its requests
+            FA_TR(1);
         }
     } else {
         if (tid == 0) sm_q_ready = 0;
@@ -925,6 +952,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         const uint32_t m = min((uint32_t)MBX, wb1 - cur);
         issue_k(cur, m, 0);
         issue_v(cur, m, 0);
+        FA_TR(2);
     }
     if (!FUSED && wave < KSTEPS) {
         q_lds[wave * 64 + lane] = qraw.u;
@@ -937,7 +965,10 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // A position at or past the launch bound / the capacity: the token is neither appended nor attended. The host
     // finds the bit at its next synchronize.
     if (FUSED && n_raw > N && tid == 0 && blockIdx.x == 0 && y == 0 && a.status) a.status[FA_DEVSTAT_APPEND_DROPPED] = 1u;
-    if (split >= nsplits) return;  // uniform over the workgroup
+    if (split >= nsplits) {  // uniform over the workgroup
+        FA_TR_FLUSH();
+        return;
+    }
     if (PAGED) {
         // Nothing has been requested yet (a paged cache needs the length first), so the partitions of this
         // sequence can still be made equal: the same number of them, none a few keys long. A short tail partition
@@ -971,6 +1002,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     }
     if (SAGE && FUSED && head_ok) qsc = sm_qscale[n] * a.scale_log2e;
+    FA_TR(3);
 
     f4_t oacc[DBLK];
 #pragma unroll
@@ -1030,6 +1062,9 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         }
         mt = fmaxf(mt, xor16(mt));
         mt = fmaxf(mt, xor32(mt));
+#ifdef FA_DECODE_TRACE
+        if (tstamp[4] == 0) FA_TR(4);  // the first round's K blocks have arrived and S is there
+#endif
         const float mn = fmaxf(m_run, mt);
         const float al = fast_exp2(m_run - mn);
         // P^T operand of block mb: k-slot i of lane (n, c) is key 4c + i of the block, the order the accumulators
@@ -1065,6 +1100,9 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         // The V registers are free as soon as the blocks are in LDS: the next round's V is requested before this
         // round's second contraction, not after it (the wait for V was the exposed latency of every round).
         if (mnext) issue_v(nblk, mnext, k1 - 1);
+#ifdef FA_DECODE_TRACE
+        if (tstamp[5] == 0) FA_TR(5);  // the first round's V blocks have arrived and are in LDS
+#endif
         // O^T += V^T . P^T : a transpose load hands lane (n, c) keys 4c..4c+3 of dim 16*blk + n
 #pragma unroll
         for (int mb = 0; mb < MBX; ++mb) {
@@ -1195,6 +1233,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         if (writer && lane < VLPR) *reinterpret_cast<uint4 *>(vw + lane * 8) = vnew;
     }
 
+    FA_TR(6);
     // the head's sum over the four 16-lane rows (the running max is already common to them)
     l_run += xor16(l_run);
     l_run += xor32(l_run);
@@ -1214,7 +1253,9 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             *reinterpret_cast<f4_t *>(sm_acc + (size_t)wave * wstr + n * D + blk * 16 + c * 4) = oacc[blk];
         if (c == 0) *reinterpret_cast<f2_t *>(sm_ml + (wave * gt + n) * 2) = f2_t{m_run, l_run};
     }
+    FA_TR(7);
     __syncthreads();
+    FA_TR(8);
 
     const bool in_kernel = a.merge_in_kernel != 0, polled = a.merge_in_kernel == 2;
     const size_t gbase = ((size_t)b * gridDim.y + y) * S * gt;  // first row of this (sequence, head group)
@@ -1273,13 +1314,19 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             if (c4 == 0) a.part_ml[(gbase + prow + h) * 2] = ms, a.part_ml[(gbase + prow + h) * 2 + 1] = L;
         }
     }
-    if (nsplits == 1 || !in_kernel) return;
+    FA_TR(9);
+    if (nsplits == 1 || !in_kernel) {
+        FA_TR_FLUSH();
+        return;
+    }
     if (polled) {
         bool ok;
         if (nsplits <= 64) {
             ok = a.xcd_local ? coop_merge_in_registers<D, true>(a, b, y, split, nsplits, S, tid)
                              : coop_merge_in_registers<D, false>(a, b, y, split, nsplits, S, tid);
             if (!ok && lane == 0 && a.status) a.status[FA_DEVSTAT_MERGE_TIMEOUT] = 1u;
+            FA_TR(10);
+            FA_TR_FLUSH();
             return;
         }
         __syncthreads();  // the fold above read the LDS region that the merge reuses

@@ -213,6 +213,11 @@ struct FaDecodeDev {
     const float *sage_mean;  // [Hkv, D]
     int8_t *q_q_out;         // [H, D]
     float *q_scale_out;      // [H]
+#ifdef FA_DECODE_TRACE
+    // development builds only (-DFA_DECODE_TRACE): every wave leaves 16 wall-clock stamps (100 MHz) of its phases here,
+    // [workgroup][wave][16]; the buffer is the one set with fa_profile_clock_buffer
+    unsigned long long *trace;
+#endif
 };
 
 

@@ -6,41 +6,85 @@
 
 namespace {
 
-constexpr int MEAN_PARTS = 64;
+typedef float sg_f4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int sg_u4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int sg_u2_t __attribute__((ext_vector_type(2)));
 
-// partial[h][part][d] = sum over the part's rows of K[h][row][d]; blockDim = head_dim threads x 256/head_dim row lanes
+__device__ __forceinline__ float h_lo(unsigned w) { return __half2float(__ushort_as_half((unsigned short)(w & 0xffffu))); }
+__device__ __forceinline__ float h_hi(unsigned w) { return __half2float(__ushort_as_half((unsigned short)(w >> 16))); }
+
+// Column sums of K over the sequence, as a streaming reduction: the kernel only reads (and stores a few KB of partial
+// sums), 16 bytes per lane and request, MEAN_UNROLL requests per lane in flight before the first is used (non-temporal:
+// the rows are read once). A workgroup of 256 threads owns `rows_per_part` consecutive rows of one head; thread t reads
+// dims 8 (t % CPR) .. of rows t / CPR, + RPI, ... (CPR = D / 8 chunks per row, RPI = 256 / CPR rows per pass) and keeps
+// 8 f32 sums; the RPI row lanes of a column are then added through LDS in lane order. A second, small launch adds the
+// parts in part order and divides (tickets that let the last workgroup of a head finish inside the first launch were
+// measured: a thousand device-scope atomics on a handful of counters cost more than the second launch).
+constexpr int MEAN_UNROLL = 8;
+constexpr uint32_t MEAN_MAX_PARTS = 1024;
+
+template <int D>
 __global__ void __launch_bounds__(256)
-sage_k_colsum_kernel(const __half *k, uint32_t capacity, uint32_t head_dim, uint32_t kv_len, float *partial) {
-    __shared__ float sm[256];
-    const uint32_t h = blockIdx.y, part = blockIdx.x;
-    const uint32_t d = threadIdx.x % head_dim, rl = threadIdx.x / head_dim, nrl = 256 / head_dim;
-    const uint32_t rows_per_part = (kv_len + MEAN_PARTS - 1) / MEAN_PARTS;
+sage_k_colsum_kernel(const __half *k, uint32_t capacity, uint32_t kv_len, uint32_t rows_per_part, uint32_t n_parts,
+                     float *partial) {
+    constexpr int CPR = D / 8, RPI = 256 / CPR;
+    __shared__ float sm[256 * 8];
+    const uint32_t h = blockIdx.y, part = blockIdx.x, tid = threadIdx.x;
+    const uint32_t ch = tid % CPR, rl = tid / CPR;
     const uint32_t r0 = part * rows_per_part, r1 = min(kv_len, r0 + rows_per_part);
-    float s = 0.0f;
-    for (uint32_t r = r0 + rl; r < r1; r += nrl) s += __half2float(k[((size_t)h * capacity + r) * head_dim + d]);
-    sm[threadIdx.x] = s;
+    const __half *base = k + ((size_t)h * capacity) * D + ch * 8;
+    float s[8] = {};
+    for (uint32_t r = r0 + rl; r < r1; r += RPI * MEAN_UNROLL) {
+        sg_u4_t x[MEAN_UNROLL];
+#pragma unroll
+        for (int u = 0; u < MEAN_UNROLL; ++u) {
+            const uint32_t row = r + u * RPI;
+            x[u] = row < r1 ? __builtin_nontemporal_load(reinterpret_cast<const sg_u4_t *>(base + (size_t)row * D)) : sg_u4_t{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int u = 0; u < MEAN_UNROLL; ++u) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) s[2 * w] += h_lo(x[u][w]), s[2 * w + 1] += h_hi(x[u][w]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sm[i * 256 + tid] = s[i];
     __syncthreads();
-    if (rl == 0) {
-        for (uint32_t j = 1; j < nrl; ++j) s += sm[j * head_dim + d];
-        partial[((size_t)h * MEAN_PARTS + part) * head_dim + d] = s;
+    if (tid < D) {
+        // column d = tid: chunk d / 8, element d % 8, the RPI row lanes in order
+        const uint32_t c = tid / 8, e = tid % 8;
+        float t = 0.0f;
+        for (uint32_t j = 0; j < (uint32_t)RPI; ++j) t += sm[e * 256 + j * CPR + c];
+        partial[((size_t)h * n_parts + part) * D + tid] = t;
     }
 }
 
-__global__ void sage_k_mean_finish_kernel(const float *partial, uint32_t head_dim, uint32_t kv_len, float *mean) {
-    const uint32_t h = blockIdx.x, d = threadIdx.x;
-    if (d >= head_dim) return;
-    float s = 0.0f;
-    for (int p = 0; p < MEAN_PARTS; ++p) s += partial[((size_t)h * MEAN_PARTS + p) * head_dim + d];
-    mean[(size_t)h * head_dim + d] = kv_len ? s / (float)kv_len : 0.0f;
-}
-
-__device__ __forceinline__ float block_max_256(float v, float *sm) {
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = v;
+// One workgroup of 256 threads per head: column d = tid % D, part lanes tid / D take parts pl, pl + 256 / D, ... (eight
+// loads in flight at a time), then the lanes in order.
+template <int D>
+__global__ void __launch_bounds__(256)
+sage_k_mean_finish_kernel(const float *partial, uint32_t n_parts, uint32_t kv_len, float *mean) {
+    __shared__ float sm[256];
+    const uint32_t h = blockIdx.x, tid = threadIdx.x;
+    const uint32_t d = tid % D, pl = tid / D, npl = 256 / D;
+    const float *hp = partial + (size_t)h * n_parts * D + d;
+    float t = 0.0f;
+    for (uint32_t p0 = pl; p0 < n_parts; p0 += npl * 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const uint32_t p = p0 + u * npl;
+            v[u] = p < n_parts ? hp[(size_t)p * D] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) t += v[u];
+    }
+    sm[tid] = t;
     __syncthreads();
-    v = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
-    __syncthreads();
-    return v;
+    if (pl == 0) {
+        for (uint32_t j = 1; j < npl; ++j) t += sm[j * D + d];
+        mean[(size_t)h * D + d] = kv_len ? t / (float)kv_len : 0.0f;
+    }
 }
 
 __device__ __forceinline__ int quant_i8(float x, float scale) {
@@ -50,30 +94,60 @@ __device__ __forceinline__ int quant_i8(float x, float scale) {
     return (int)r;
 }
 
-// One workgroup per (32-row block, kv head).
+// One wave per 32-row block of one head (four blocks per workgroup): the block is read ONCE - 16 bytes per lane and
+// request, all of a lane's requests in flight together - held in registers as f32 differences from the mean, reduced to
+// the block's scale with lane exchanges, quantised and stored 8 bytes per lane and row. Lane l owns dims 8 (l % CPR) ..
+// of rows l / CPR + RPP i.
+template <int D>
 __global__ void __launch_bounds__(256)
-sage_quantize_k_kernel(const __half *k, const float *mean, uint32_t capacity, uint32_t head_dim, uint32_t row_begin,
-                       uint32_t row_end, int8_t *k_q, __half *k_scale, uint32_t n_scale_blocks) {
-    __shared__ float sm[4];
-    const uint32_t h = blockIdx.y;
-    const uint32_t b0 = row_begin + blockIdx.x * FA_SAGE_BLOCK;
-    const uint32_t b1 = min(row_end, b0 + FA_SAGE_BLOCK);
-    const uint32_t n = (b1 - b0) * head_dim;
-    float amax = 0.0f;
-    for (uint32_t i = threadIdx.x; i < n; i += 256) {
-        const uint32_t r = b0 + i / head_dim, d = i % head_dim;
-        const float x = __half2float(k[((size_t)h * capacity + r) * head_dim + d]) - mean[(size_t)h * head_dim + d];
-        amax = fmaxf(amax, fabsf(x));
+sage_quantize_k_kernel(const __half *k, const float *mean, uint32_t capacity, uint32_t row_begin, uint32_t row_end,
+                       uint32_t n_blocks, int8_t *k_q, __half *k_scale, uint32_t n_scale_blocks) {
+    constexpr int CPR = D / 8, RPP = 64 / CPR, NI = 32 / RPP;  // chunks per row, rows per pass of the wave, passes
+    const uint32_t h = blockIdx.y, lane = threadIdx.x & 63u;
+    const uint32_t blk = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (blk >= n_blocks) return;  // uniform over the wave
+    const uint32_t b0 = row_begin + blk * FA_SAGE_BLOCK, b1 = min(row_end, b0 + FA_SAGE_BLOCK);
+    const uint32_t ch = lane % CPR, rl = lane / CPR;
+    const __half *src = k + ((size_t)h * capacity + b0) * D + ch * 8;
+    sg_u4_t raw[NI];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const uint32_t row = rl + i * RPP;
+        raw[i] = b0 + row < b1 ? __builtin_nontemporal_load(reinterpret_cast<const sg_u4_t *>(src + (size_t)row * D)) : sg_u4_t{0u, 0u, 0u, 0u};
     }
-    amax = block_max_256(amax, sm);
+    const sg_f4_t m0 = *reinterpret_cast<const sg_f4_t *>(mean + (size_t)h * D + ch * 8);
+    const sg_f4_t m1 = *reinterpret_cast<const sg_f4_t *>(mean + (size_t)h * D + ch * 8 + 4);
+    const float mu[8] = {m0[0], m0[1], m0[2], m0[3], m1[0], m1[1], m1[2], m1[3]};
+    float x[NI][8];
+    float amax = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const bool live = b0 + rl + i * RPP < b1;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            x[i][2 * w] = live ? h_lo(raw[i][w]) - mu[2 * w] : 0.0f;
+            x[i][2 * w + 1] = live ? h_hi(raw[i][w]) - mu[2 * w + 1] : 0.0f;
+            amax = fmaxf(amax, fmaxf(fabsf(x[i][2 * w]), fabsf(x[i][2 * w + 1])));
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
     const __half sc16 = __float2half_rn(amax / 127.0f);
     const float sc = __half2float(sc16);
-    if (threadIdx.x == 0) k_scale[(size_t)h * n_scale_blocks + b0 / FA_SAGE_BLOCK] = sc16;
-    for (uint32_t i = threadIdx.x; i < n; i += 256) {
-        const uint32_t r = b0 + i / head_dim, d = i % head_dim;
-        const size_t idx = ((size_t)h * capacity + r) * head_dim + d;
-        const float x = __half2float(k[idx]) - mean[(size_t)h * head_dim + d];
-        k_q[idx] = (int8_t)quant_i8(x, sc);
+    if (lane == 0) k_scale[(size_t)h * n_scale_blocks + b0 / FA_SAGE_BLOCK] = sc16;
+    int8_t *dst = k_q + ((size_t)h * capacity + b0) * D + ch * 8;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const uint32_t row = rl + i * RPP;
+        if (b0 + row >= b1) continue;
+        sg_u2_t o;
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+            const unsigned q0 = (unsigned)quant_i8(x[i][4 * w], sc) & 0xffu, q1 = (unsigned)quant_i8(x[i][4 * w + 1], sc) & 0xffu;
+            const unsigned q2 = (unsigned)quant_i8(x[i][4 * w + 2], sc) & 0xffu, q3 = (unsigned)quant_i8(x[i][4 * w + 3], sc) & 0xffu;
+            o[w] = q0 | (q1 << 8) | (q2 << 16) | (q3 << 24);
+        }
+        *reinterpret_cast<sg_u2_t *>(dst + (size_t)row * D) = o;
     }
 }
 
@@ -236,17 +310,34 @@ fa_status fa_launch_sage_append(fa_ctx *ctx, const SageAppendLaunch &l) {
 
 fa_status fa_launch_sage_k_mean(fa_ctx *ctx, const void *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim,
                                 uint32_t kv_len, float *mean_out) {
-    FA_TRY(fa_ensure_workspace(ctx, (size_t)n_kv_heads * MEAN_PARTS * head_dim * sizeof(float)));
+    if (((uintptr_t)k & 15u) != 0) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "the K tensor must be 16-byte aligned");
+    // Parts: about eight workgroups per compute unit over all heads (a workgroup has all of a pass - 256 threads x
+    // MEAN_UNROLL requests of 16 bytes = 32 KiB - in flight at once, and eight of them fit a compute unit), each a whole
+    // number of passes, at most MEAN_MAX_PARTS per head.
+    const uint32_t rows_per_pass = (256u / (head_dim / 8u)) * MEAN_UNROLL;
+    const uint64_t n_cus = (uint64_t)(ctx->n_cus > 0 ? ctx->n_cus : 256);
+    uint32_t want = (uint32_t)((8 * n_cus + n_kv_heads - 1) / n_kv_heads);
+    if (want > MEAN_MAX_PARTS) want = MEAN_MAX_PARTS;
+    if (want == 0) want = 1;
+    uint32_t rows_per_part = ceil_div_u32(ceil_div_u32(kv_len ? kv_len : 1u, want), rows_per_pass) * rows_per_pass;
+    const uint32_t n_parts = ceil_div_u32(kv_len ? kv_len : 1u, rows_per_part);
+    FA_TRY(fa_ensure_workspace(ctx, (size_t)n_kv_heads * n_parts * head_dim * sizeof(float)));
     float *partial = (float *)ctx->workspace;
     {
         FaLaunchScope scope(ctx, "sage_k_colsum_kernel", true);
-        scope.launch(sage_k_colsum_kernel, dim3(MEAN_PARTS, n_kv_heads), dim3(256), 0,
-                           (const __half *)k, capacity, head_dim, kv_len, partial);
+        if (head_dim == 128)
+            scope.launch(sage_k_colsum_kernel<128>, dim3(n_parts, n_kv_heads), dim3(256), 0, (const __half *)k, capacity, kv_len,
+                         rows_per_part, n_parts, partial);
+        else
+            scope.launch(sage_k_colsum_kernel<64>, dim3(n_parts, n_kv_heads), dim3(256), 0, (const __half *)k, capacity, kv_len,
+                         rows_per_part, n_parts, partial);
         FA_TRY(scope.finish());
     }
     FaLaunchScope scope(ctx, "sage_k_mean_finish_kernel", true);
-    scope.launch(sage_k_mean_finish_kernel, dim3(n_kv_heads), dim3(head_dim), 0, partial, head_dim,
-                       kv_len, mean_out);
+    if (head_dim == 128)
+        scope.launch(sage_k_mean_finish_kernel<128>, dim3(n_kv_heads), dim3(256), 0, partial, n_parts, kv_len, mean_out);
+    else
+        scope.launch(sage_k_mean_finish_kernel<64>, dim3(n_kv_heads), dim3(256), 0, partial, n_parts, kv_len, mean_out);
     return scope.finish();
 }
 
@@ -254,11 +345,16 @@ fa_status fa_launch_sage_quantize_k(fa_ctx *ctx, const void *k, const float *mea
                                     uint32_t capacity, uint32_t head_dim, uint32_t row_begin, uint32_t row_end,
                                     void *k_q, void *k_scale) {
     if (row_end <= row_begin) return FA_OK;
+    if ((((uintptr_t)k | (uintptr_t)mean) & 15u) != 0 || ((uintptr_t)k_q & 7u) != 0)
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "K and the mean must be 16-byte aligned, the int8 cache 8-byte aligned");
     const uint32_t nblk = ceil_div_u32(row_end - row_begin, FA_SAGE_BLOCK);
     FaLaunchScope scope(ctx, "sage_quantize_k_kernel", true);
-    scope.launch(sage_quantize_k_kernel, dim3(nblk, n_kv_heads), dim3(256), 0, (const __half *)k, mean,
-                       capacity, head_dim, row_begin, row_end, (int8_t *)k_q, (__half *)k_scale,
-                       ceil_div_u32(capacity, FA_SAGE_BLOCK));
+    if (head_dim == 128)
+        scope.launch(sage_quantize_k_kernel<128>, dim3(ceil_div_u32(nblk, 4), n_kv_heads), dim3(256), 0, (const __half *)k, mean,
+                     capacity, row_begin, row_end, nblk, (int8_t *)k_q, (__half *)k_scale, ceil_div_u32(capacity, FA_SAGE_BLOCK));
+    else
+        scope.launch(sage_quantize_k_kernel<64>, dim3(ceil_div_u32(nblk, 4), n_kv_heads), dim3(256), 0, (const __half *)k, mean,
+                     capacity, row_begin, row_end, nblk, (int8_t *)k_q, (__half *)k_scale, ceil_div_u32(capacity, FA_SAGE_BLOCK));
     return scope.finish();
 }
 

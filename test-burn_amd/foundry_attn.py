@@ -10,7 +10,7 @@ import os
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libfoundry_attn.so")
+LIB_PATH = os.environ.get("FOUNDRY_ATTN_LIB") or os.path.join(HERE, "libfoundry_attn.so")  # the override is for development builds
 
 FA_OK = 0
 STATUS_NAMES = {
