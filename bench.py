@@ -869,7 +869,7 @@ def bench_prefill_chunk(f, args, m=32, prefix=8160):
     for i in range(per_graph):
         step(i)
     us = {}
-    for kname in ("flash_prefill_dma_kernel", "flash_prefill_mfma_kernel", "flash_prefill_merge_kernel"):
+    for kname in ("flash_chunk_kernel", "flash_prefill_dma_kernel", "flash_prefill_mfma_kernel", "flash_prefill_merge_kernel"):
         n, ms = f.profile_query(kname)
         if n:
             us[kname] = ms * 1e3 / n
@@ -881,9 +881,11 @@ def bench_prefill_chunk(f, args, m=32, prefix=8160):
         "ms_per_step": per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "llama3.2-3b prefill chunk of %d rows after a %d-token prefix, one layer per step: causal attention "
-                               "(split over the keys) + merge, contiguous cache, graph replays" % (m, prefix)},
+                               "split over the keys, merge %s, contiguous cache, graph replays"
+                               % (m, prefix, "inside the launch" if "flash_chunk_kernel" in us else "as a second launch")},
         "roofline": {"bound": "hbm", "achieved": nbytes / per_step / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": nbytes / per_step / 1e9 / HBM_PEAK_GBPS, "traffic": None, "kernel": "prefill kernel + merge kernel (one step)",
+                     "frac": nbytes / per_step / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "flash_chunk_kernel" if "flash_chunk_kernel" in us else "prefill kernel + merge kernel (one step)",
                      "avg_launch_us": us, "bytes_per_step": nbytes,
                      "timing": "HIP events on the stream around the graph replays / steps in them"},
         "parity": {"max_abs_err_vs_oracle": err}})

@@ -316,8 +316,13 @@ fa_status fa_set_prefill_split_k(fa_ctx *ctx, uint32_t split_k);
  * (src/metals/flashattention/variants.rs): 1 = K/V tiles staged through registers, one barrier per key tile;
  * 2 = K/V tiles loaded straight into LDS, softmax and MFMA work of the two wave groups alternating in two
  * barrier-separated phases, resident workgroups that share out the (query tile, head) items (measured 10 % faster at
- * 2048 tokens, 14 % at 8192 and on a paged cache); 0 (default) = 2. Same contract; the two differ in the order in which
- * a row's weights are summed (outputs agree to one f16 ulp).
+ * 2048 tokens, 14 % at 8192 and on a paged cache); 3 = 2, and every launch of at most 64 query rows (head_dim 64 or
+ * 128) goes to the short-chunk kernel: one workgroup per (KV head, context partition) that reads its share of the
+ * prefix once, like a decode step, and merges the partitions inside the launch (same residency assumption, wait bound
+ * and reporting as the polled decode merge above; its partial states use the context's workspace, which cannot grow
+ * inside a capture); 0 (default) = 2, with the short-chunk kernel where it is measured to win: at most 64 rows, at
+ * least 2048 visible keys, group_size * ceil(rows / 32) <= 4, and no split-K override. Same contract; the variants
+ * differ in the order in which a row's weights are summed (outputs agree to one f16 ulp).
  * Environment: FOUNDRY_ATTN_PREFILL_VARIANT (read at fa_ctx_create). */
 fa_status fa_set_prefill_variant(fa_ctx *ctx, uint32_t variant);
 

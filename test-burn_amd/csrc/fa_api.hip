@@ -125,7 +125,7 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     ctx->prefill_split_k = env_u32("FOUNDRY_ATTN_PREFILL_SPLIT_K", 0);
     ctx->prefill_variant = env_u32("FOUNDRY_ATTN_PREFILL_VARIANT", 0);
     ctx->sage_fused_step = env_u32("FOUNDRY_ATTN_SAGE_FUSED", 1);
-    if (ctx->prefill_variant > 2) ctx->prefill_variant = 0;
+    if (ctx->prefill_variant > 3) ctx->prefill_variant = 0;
     ctx->ledger = new FaGraphLedger();
     fa_status s = fa_ensure_workspace(ctx, (size_t)64 << 20);
     if (s == FA_OK) s = fa_ensure_counters(ctx, 4096);
@@ -303,7 +303,7 @@ extern "C" fa_status fa_set_sage_step_variant(fa_ctx *ctx, uint32_t variant) {
 
 extern "C" fa_status fa_set_prefill_variant(fa_ctx *ctx, uint32_t variant) {
     FA_NEED(ctx, "ctx");
-    if (variant > 2) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "prefill variant must be 0, 1 or 2, got %u", variant);
+    if (variant > 3) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "prefill variant must be 0 ... 3, got %u", variant);
     ctx->prefill_variant = variant;
     return FA_OK;
 }

@@ -65,7 +65,7 @@ struct fa_ctx {
     uint32_t gemm_min_m = 0;       // FusedQkv / MatMul: input rows from which the GEMM runs (0 = default)
     uint32_t prefill_split_k = 0;  // 0 = auto
     uint32_t sage_fused_step = 1;  // the int8 decode step as one launch (env FOUNDRY_ATTN_SAGE_FUSED=0: append kernel + decode kernel)
-    uint32_t prefill_variant = 0;  // 0 = auto, 1 = tiles staged through registers, 2 = tiles straight into LDS, two-phase loop
+    uint32_t prefill_variant = 0;  // 0 = auto, 1 = tiles staged through registers, 2 = tiles straight into LDS, two-phase loop, 3 = as 0 with the chunk kernel wherever it applies
     // optional: the prefill kernel leaves {shader-clock ticks, wall ticks} per workgroup here (fa_profile_clock_buffer)
     unsigned long long *clock_buf = nullptr;
     uint32_t clock_buf_workgroups = 0;
@@ -235,6 +235,9 @@ struct PrefillLaunch {
     bool bf16;  // q, k, v and out are bf16 instead of f16
 };
 fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &a);
+// fa_chunk.hip: a chunk of at most 64 rows against a long prefix as one memory-bound launch (merge inside). *taken says
+// whether it took the launch; `force`: also where the tiled kernel would normally be preferred (short contexts).
+fa_status fa_launch_prefill_chunk(fa_ctx *ctx, const PrefillLaunch &a, bool force, bool *taken);
 
 fa_status fa_launch_u32_add(fa_ctx *ctx, uint32_t *vals, uint32_t n, uint32_t delta);
 fa_status fa_launch_paged_gather(fa_ctx *ctx, const fa_paged_kv *c, uint32_t seq_index, uint32_t seq_len, void *k_out,

@@ -17,10 +17,15 @@
 //                                A = V^T fetched with ds_read_b64_tr_b16 (LDS transpose load)
 // FLOPs per (query row, visible key, head): 4 * D.
 #include "fa_internal.h"
+#include "fa_lds_dma.h"
 
 #include <type_traits>
 
 namespace {
+
+using fa_lds_dma::buffer_to_lds_b128;
+using fa_lds_dma::make_rsrc_words;
+using fa_lds_dma::rsrc_words;
 
 typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
@@ -420,75 +425,6 @@ __device__ __forceinline__ void phase_barrier() {
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-}
-
-// 16 bytes per lane from a buffer straight into LDS: lane l's bytes land at lds_addr + imm + 16 l, read from
-// base + voff + soff + imm; out-of-range lanes deliver zeros. Written as assembly so that the compiler does not
-// serialise every later LDS read behind it (it cannot tell which LDS bytes such a load writes); completion is
-// tracked by vmcnt, and the waits are placed by hand.
-typedef unsigned int rsrc_words __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ rsrc_words make_rsrc_words(const void *base, uint32_t bytes) {
-    const uint64_t b = reinterpret_cast<uint64_t>(base);
-    rsrc_words r;
-    r.x = (uint32_t)b, r.y = (uint32_t)(b >> 32) & 0xffffu, r.z = bytes, r.w = 0x00020000u;
-    return r;
-}
-// N such loads whose sources are SRC_STEP bytes apart and whose destinations are DST_STEP bytes apart. When the two
-// steps are equal the instruction's immediate offset (which moves source and destination alike) does the stepping.
-template <int N, int SRC_STEP, int DST_STEP>
-__device__ __forceinline__ void buffer_to_lds_b128(rsrc_words rs, uint32_t lds_addr, int voff, int soff) {
-    static_assert(N == 1 || N == 2 || N == 4, "1, 2 or 4 loads");
-    if constexpr (SRC_STEP == DST_STEP) {
-        static_assert((N - 1) * SRC_STEP < 4096, "12-bit immediate");
-        if constexpr (N == 4)
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-                         "buffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
-                         "buffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds\n\t"
-                         "buffer_load_dwordx4 %1, %2, %3 offen offset:%5 lds\n\t"
-                         "buffer_load_dwordx4 %1, %2, %3 offen offset:%6 lds"
-                         :
-                         : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff), "n"(SRC_STEP), "n"(2 * SRC_STEP), "n"(3 * SRC_STEP)
-                         : "memory");
-        else if constexpr (N == 2)
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-                         "buffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
-                         "buffer_load_dwordx4 %1, %2, %3 offen offset:%4 lds"
-                         :
-                         : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff), "n"(SRC_STEP)
-                         : "memory");
-        else
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                         :
-                         : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
-                         : "memory");
-    } else {  // (the source-offset update sits between the m0 write and the load that needs it)
-        int so = soff;
-        if constexpr (N == 4)
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\t"
-                         "buffer_load_dwordx4 %2, %3, %0 offen lds\n\t"
-                         "s_add_i32 m0, %1, %5\n\ts_add_i32 %0, %0, %4\n\t"
-                         "buffer_load_dwordx4 %2, %3, %0 offen lds\n\t"
-                         "s_add_i32 m0, %1, %6\n\ts_add_i32 %0, %0, %4\n\t"
-                         "buffer_load_dwordx4 %2, %3, %0 offen lds\n\t"
-                         "s_add_i32 m0, %1, %7\n\ts_add_i32 %0, %0, %4\n\t"
-                         "buffer_load_dwordx4 %2, %3, %0 offen lds"
-                         : "+s"(so)
-                         : "s"(lds_addr), "v"(voff), "s"(rs), "n"(SRC_STEP), "n"(DST_STEP), "n"(2 * DST_STEP), "n"(3 * DST_STEP)
-                         : "memory", "scc");
-        else if constexpr (N == 2)
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\t"
-                         "buffer_load_dwordx4 %2, %3, %0 offen lds\n\t"
-                         "s_add_i32 m0, %1, %5\n\ts_add_i32 %0, %0, %4\n\t"
-                         "buffer_load_dwordx4 %2, %3, %0 offen lds"
-                         : "+s"(so)
-                         : "s"(lds_addr), "v"(voff), "s"(rs), "n"(SRC_STEP), "n"(DST_STEP)
-                         : "memory", "scc");
-        else
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                         :
-                         : "s"(lds_addr), "v"(voff), "s"(rs), "s"(soff)
-                         : "memory");
-    }
 }
 
 // Two-phase variant of the kernel above (same tiling and arithmetic; results differ only by the order in which a
@@ -1102,6 +1038,13 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
     if (L.q_len == 0) return FA_OK;
     if (L.head_dim != 128 && L.head_dim != 64)
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill only supports head_dim=64 or 128, got %u", L.head_dim);
+    // A chunk of at most 64 rows after a long prefix is a memory-bound launch: fa_chunk.hip (unless a kernel or a split
+    // count has been asked for by name)
+    if ((ctx->prefill_variant == 0 && ctx->prefill_split_k == 0) || ctx->prefill_variant == 3) {
+        bool taken = false;
+        FA_TRY(fa_launch_prefill_chunk(ctx, L, ctx->prefill_variant == 3, &taken));
+        if (taken) return FA_OK;
+    }
     // Split-K (src/metals/flashattention/step.rs:849-864): few query tiles against a long context (a prefill chunk
     // after a long prefix) would leave most CUs idle, so the key tiles of each query tile are divided over several
     // workgroups, at least 4 tiles each, up to one workgroup per CU.

@@ -320,3 +320,52 @@ def test_prefill_chunk_after_long_prefix_auto_split():
     want = orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, prefix, cap, causal=True, out_layout="head_major", n_threads=8)
     got = gpu_prefill(q, k, v, H, D, M, N, prefix)
     assert max_abs(got, want) <= TOL
+
+
+def test_prefill_chunk_after_32k_prefix_ring_wraps():
+    """32 rows against a 32K prefix: every workgroup of the chunk kernel takes its partition through the LDS ring
+    several times over (1024 keys = 16 rounds of 64 in 4 slots), with the last partition shorter than the others."""
+    announce("prefill chunk 32 @ 32k")
+    rng = np.random.default_rng(14)
+    H, Hkv, D, M, prefix = 24, 8, 128, 32, 32768 - 32 - 40
+    N, cap = M + prefix, 32768
+    q = h16(rng.normal(size=(H, M, D)))
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    v = h16(rng.normal(size=(Hkv, cap, D)))
+    want = orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, prefix, cap, causal=True, out_layout="head_major", n_threads=8)
+    got = gpu_prefill(q, k, v, H, D, M, N, prefix)
+    assert max_abs(got, want) <= TOL
+
+
+def test_prefill_chunk_kernel_gives_up_cleanly():
+    """Failure handling of the chunk kernel's waits (LDS ring and merge), forced from the host: with a wait bound of
+    zero a wave gives up at its first look at anything that is not there yet. Every kernel still ends normally, the
+    next stream wait reports it, and with the normal bound the same context is right again (the arrival pattern of
+    the partial buffer was restored)."""
+    announce("prefill chunk kernel, zero wait bound")
+    rng = np.random.default_rng(15)
+    H, Hkv, D, M, prefix = 24, 8, 128, 32, 4000
+    N, cap = M + prefix, 4096
+    q, k, v = h16(rng.normal(size=(H, M, D))), h16(rng.normal(size=(Hkv, cap, D))), h16(rng.normal(size=(Hkv, cap, D)))
+    want = orc.sdpa_prefill(q, k, v, H, Hkv, D, M, N, prefix, cap, causal=True, out_layout="token_major", n_threads=8)
+    g = fa.Foundry(0)
+    try:
+        dq, dk, dv, do = g.array(q), g.array(k), g.array(v), g.zeros((M, H * D))
+        g.set_prefill_variant(3)
+        g.set_decode_poll_spin_us(0)
+        reported = 0
+        for _ in range(3):
+            g.flash_attention(dq.arg((H, M, D)), dk.arg(), dv.arg(), do.arg(), True, prefix, H, D, N, M)
+            try:
+                g.synchronize()
+            except fa.FoundryError as e:
+                reported += 1
+                assert e.variant == "OperationFailed" and "waited longer" in str(e)
+        assert reported >= 1  # (a wave cannot find a whole round in LDS at its first look)
+        g.set_decode_poll_spin_us(5000)
+        for _ in range(3):
+            g.flash_attention(dq.arg((H, M, D)), dk.arg(), dv.arg(), do.arg(), True, prefix, H, D, N, M)
+            assert max_abs(do.download().reshape(M, H * D), want.reshape(M, H * D)) <= TOL
+        g.synchronize()
+    finally:
+        g.close()
