@@ -829,13 +829,17 @@ def bench_attn_block(f, args):
 
 def bench_prefill_chunk(f, args, m=32, prefix=8160):
     """One prefill chunk of m rows (32 = the reference's default chunk, src/model/executor.rs:232-250) attending a contiguous
-    Llama-3.2-3B-shaped cache that already holds `prefix` tokens: the split-K prefill kernel + its merge kernel, timed as
-    graph replays over 4 layers' caches in rotation. HBM-bound: every launch reads the whole prefix once."""
-    H, Hkv, D, L = 24, 8, 128, 4
+    Llama-3.2-3B-shaped cache that already holds `prefix` tokens: the short-chunk kernel (partitions merged inside the
+    launch) or, under another prefill variant, the split-K prefill kernel + its merge kernel; timed as graph replays over
+    as many layers' caches in rotation as take about 1 GB (28 at 8K tokens), so that no replay finds its rows in a cache.
+    HBM-bound: every launch reads the whole prefix once."""
+    H, Hkv, D = 24, 8, 128
     N, cap = prefix + m, prefix + 512
+    L = max(4, min(28, int(np.ceil(0.94e9 / (2.0 * Hkv * N * D * 2)))))
     rng = np.random.default_rng(0xF0DD + 14)
-    caches = [(f.array(rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16)),
-               f.array(rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16))) for _ in range(L)]
+    k0 = rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16)
+    v0 = rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16)
+    caches = [(f.array(k0), f.array(v0)) for _ in range(L)]  # (the same rows in every layer's buffers)
     q = rng.standard_normal((H, m, D), dtype=np.float32).astype(np.float16)
     dq, dout = f.array(q), f.zeros((m, H * D))
 
@@ -850,7 +854,7 @@ def bench_prefill_chunk(f, args, m=32, prefix=8160):
                             out_layout="head_major", n_threads=max(1, min(16, os.cpu_count() or 1, orc.lib().orc_max_threads())))
     got = dout.download().reshape(m, H, D).transpose(1, 0, 2)
     err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64))))
-    per_graph = 4 * L
+    per_graph = 2 * L
     f.start_capture()
     for i in range(per_graph):
         step(i)
@@ -881,8 +885,8 @@ def bench_prefill_chunk(f, args, m=32, prefix=8160):
         "ms_per_step": per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "llama3.2-3b prefill chunk of %d rows after a %d-token prefix, one layer per step: causal attention "
-                               "split over the keys, merge %s, contiguous cache, graph replays"
-                               % (m, prefix, "inside the launch" if "flash_chunk_kernel" in us else "as a second launch")},
+                               "split over the keys, merge %s, contiguous cache, %d layers' caches in rotation, graph replays"
+                               % (m, prefix, "inside the launch" if "flash_chunk_kernel" in us else "as a second launch", L)},
         "roofline": {"bound": "hbm", "achieved": nbytes / per_step / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": nbytes / per_step / 1e9 / HBM_PEAK_GBPS, "traffic": None,
                      "kernel": "flash_chunk_kernel" if "flash_chunk_kernel" in us else "prefill kernel + merge kernel (one step)",
@@ -1364,7 +1368,7 @@ def main():
         result["configs"], result["floors"] = {}, None
         for tag, fn in (("C1_qwen05b_decode_1k", bench_small_decode), ("C3_qwen3b_paged_decode", bench_paged_decode),
                         ("C4_llama3b_prefill_2k", bench_prefill), ("C5_smollm3_sage_decode_32k", bench_sage_decode),
-                        ("floors", bench_floors)):
+                        ("llama3b_prefill_chunk32_8k", bench_prefill_chunk), ("floors", bench_floors)):
             _COLLECT = []
             g = fa.Foundry(0)
             try:
@@ -1376,7 +1380,9 @@ def main():
                 result["floors"] = line["floors"]
             else:
                 result["configs"][tag] = {k: line[k] for k in ("metric", "value", "unit", "steps", "ms_per_step", "dtype",
-                                                                "config", "roofline", "parity") if k in line}
+                                                                "config", "roofline", "parity", "timing",
+                                                                "whole_step_hbm_frac_of_peak", "eager_dispatch_avg_launch_us",
+                                                                "merge_kernel_avg_launch_us") if k in line}
                 for k in ("append",):  # the append kernel of a configuration, where it is a launch of its own
                     if k in line:
                         result["configs"][tag][k] = line[k]
