@@ -20,7 +20,7 @@ OBJ = os.path.join(HERE, "build" + TAG)
 LIB = os.path.join(HERE, "libfoundry_attn%s.so" % TAG)
 SOURCES = ["fa_api.hip", "fa_kvprep.hip", "fa_decode.hip", "fa_decode_d64.hip", "fa_decode_d128.hip", "fa_decode_d64_w4.hip", "fa_decode_d128_w4.hip", "fa_prefill.hip", "fa_chunk.hip",
            "fa_sage.hip", "fa_kvcopy.hip", "fa_qkv.hip", "fa_gemm.hip", "fa_legacy.hip", "fa_probe.hip"]
-HEADERS = [os.path.join(CSRC, "fa_internal.h"), os.path.join(CSRC, "fa_decode_impl.h"), os.path.join(CSRC, "fa_qkv_rope.h"), os.path.join(CSRC, "fa_lds_dma.h"),
+HEADERS = [os.path.join(CSRC, "fa_internal.h"), os.path.join(CSRC, "fa_decode_impl.h"), os.path.join(CSRC, "fa_qkv_rope.h"), os.path.join(CSRC, "fa_lds_dma.h"), os.path.join(CSRC, "fa_sage_quant.h"),
            os.path.join(HERE, "..", "include", "foundry_attn.h")]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950", "-Wall", "-Wno-unused-function",

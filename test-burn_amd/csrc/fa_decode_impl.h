@@ -43,6 +43,7 @@
 // with several rounds of workgroups, where one workgroup's start and end overlap the other's stream.
 #pragma once
 #include "fa_internal.h"
+#include "fa_sage_quant.h"
 #include <mutex>
 #include <type_traits>
 
@@ -761,12 +762,38 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             if (lane < D / 8) kv4 = *reinterpret_cast<const uint4 *>(a.k_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D + lane * 8);
             if (lane < D / 4) mv4 = *reinterpret_cast<const uint4 *>(a.sage_mean + (size_t)kvh * D + lane * 4);
             sage_vnew = *reinterpret_cast<const uint4 *>(a.v_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D + (lane % VLPR) * 8);
+            // The exact rows of the open 32-row block, all 32 of them whatever the position turns out to be (the rows at
+            // and past it are not used): the workgroup that owns the new token quantises the block anew, which is the
+            // longest thing any wave of the launch does, and a request made after the barrier would queue behind the
+            // other waves' blocks. Lane (n, c) takes the two halves of segment 4j + c of rows n and 16 + n; they are
+            // parked in block registers that this wave does not otherwise use until then.
+            static_assert(2 * KSTEPS <= VLB && MBX >= 3, "the open block's rows are parked in kk[0..1] and vv[2]");
+            {
+                const __half *tail_rows = a.sage_tail + (size_t)kvh * FA_SAGE_BLOCK * D;
+#pragma unroll
+                for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+                    for (int j = 0; j < KSTEPS; ++j) {
+                        const __half *src = tail_rows + (size_t)(sb * BK + n) * D + (4 * j + c) * 16;
+                        kk[sb][j].u = *reinterpret_cast<const uint4 *>(src);
+                        vv[2][sb * KSTEPS + j].u = *reinterpret_cast<const uint4 *>(src + 8);
+                    }
+            }
             if (lane == 0) sm_q_ready = 0;
             __builtin_amdgcn_sched_barrier(0);
             __syncthreads();  // releases the streaming waves
             __builtin_amdgcn_sched_barrier(0);
+            FA_TR(1);
             n_raw = read_len();
             const uint32_t p0 = min(n_raw, min(a.capacity, a.kv_len_bound)) - 1;
+            {
+                // ... and the block's V rows as soon as the position says where they are (same conditions as below)
+                const uint32_t N0 = p0 + 1;
+                if (n_raw == N0 && N0 > 0 && p0 >= k0 && p0 < k0 + chunk && split < (N0 + a.chunk - 1) / a.chunk) {
+                    const uint32_t r0 = p0 & (FA_SAGE_BLOCK - 1);
+                    issue_v((p0 - r0 - k0) / BK, r0 / BK + 1, 0);
+                }
+            }
             if (rope_on) {  // the table row through the scalar cache, as below
                 const uint32_t tp = min(p0, a.table_rows - 1);
                 const __half *ct = a.cos_t + (size_t)tp * (D / 2), *st = a.sin_t + (size_t)tp * (D / 2);
@@ -795,6 +822,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                 }
             }
             if (lane < D / 4) *reinterpret_cast<uint4 *>(st_mean + lane * 4) = mv4;
+            FA_TR(11);
             __builtin_amdgcn_wave_barrier();  // LDS executes a wave's accesses in order: the table row is there
             // Rotation in the layout the rows were fetched in: lane l holds piece l % (D / 8) (8 dims) of row l / (D / 8)
             // (+ 64 i / (D / 8)); a NeoX mate piece is D / 16 lanes away. Arithmetic of the append kernel (rope8: products
@@ -1138,8 +1166,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             const bool writer = y % a.sub_per_kv == 0;
             const uint32_t r = p & (FA_SAGE_BLOCK - 1), b0 = p - r, nsb = r / BK + 1;
             __half *tail = a.sage_tail + (size_t)kvh * FA_SAGE_BLOCK * D;
-            // V rows of the block (the new row is patched in below)
-            issue_v((b0 - k0) / BK, nsb, 0);
+            // (the V rows of the block were requested when the position was read; the new row is patched in below)
             float kx[2][KSTEPS][16];
             float amax = 0.0f;
 #pragma unroll
@@ -1150,8 +1177,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                     U4H t0, t1;
                     t0.u = make_uint4(0, 0, 0, 0), t1.u = t0.u;
                     if (row < r) {
-                        t0.u = *reinterpret_cast<const uint4 *>(tail + (size_t)row * D + col);
-                        t1.u = *reinterpret_cast<const uint4 *>(tail + (size_t)row * D + col + 8);
+                        t0 = kk[sb][j], t1 = vv[2][sb * KSTEPS + j];  // requested before the first barrier
                     } else if (row == r) {
                         t0.u = *reinterpret_cast<const uint4 *>(st_krot + col);
                         t1.u = *reinterpret_cast<const uint4 *>(st_krot + col + 8);
@@ -1165,8 +1191,9 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                 }
 #pragma unroll
             for (int off = 1; off < 64; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
+            FA_TR(12);
             const __half sc16 = __float2half_rn(amax / 127.0f);
-            const float sc = __half2float(sc16);
+            const SageDivisor dv = sage_divisor(__half2float(sc16));
             int8_t *kq = const_cast<int8_t *>(reinterpret_cast<const int8_t *>(kbase)) + (size_t)b0 * D;
 #pragma unroll
             for (int sb = 0; sb < 2; ++sb)
@@ -1177,7 +1204,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                         int8_t e[16];
                     } o;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) o.e[i] = (int8_t)sage_quant_i8(kx[sb][j][i], sc);
+                    for (int i = 0; i < 16; ++i) o.e[i] = (int8_t)sage_quant_i8_block(kx[sb][j][i], dv);
                     kk[sb][j].u = o.u;
                 }
             // the new V row into its place among the block's rows (load i holds rows i VRPL .. of a 16-row block)
@@ -1192,7 +1219,9 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             // (the V blocks go through this wave's LDS region, which is the staging area: take the rotated row out first)
             const uint4 krot16 = *reinterpret_cast<const uint4 *>(st_krot + (lane % (D / 8)) * 8);
             ksr[0] = ksr[1] = (_Float16)sc16;
+            FA_TR(13);
             consume(b0, nsb, p + 1, 0, 0);
+            FA_TR(14);
             __builtin_amdgcn_sched_barrier(0);
             if (writer) {  // after the block has been attended (see below): the int8 rows, the scale, the tail row, the V row
 #pragma unroll

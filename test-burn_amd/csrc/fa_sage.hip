@@ -3,6 +3,7 @@
 // Every step is elementwise f32 with IEEE division and round-half-even, so results are reproducible
 // bit for bit on the host given the same mean.
 #include "fa_internal.h"
+#include "fa_sage_quant.h"
 
 namespace {
 
@@ -133,7 +134,7 @@ sage_quantize_k_kernel(const __half *k, const float *mean, uint32_t capacity, ui
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off));
     const __half sc16 = __float2half_rn(amax / 127.0f);
-    const float sc = __half2float(sc16);
+    const SageDivisor dv = sage_divisor(__half2float(sc16));
     if (lane == 0) k_scale[(size_t)h * n_scale_blocks + b0 / FA_SAGE_BLOCK] = sc16;
     int8_t *dst = k_q + ((size_t)h * capacity + b0) * D + ch * 8;
 #pragma unroll
@@ -143,8 +144,8 @@ sage_quantize_k_kernel(const __half *k, const float *mean, uint32_t capacity, ui
         sg_u2_t o;
 #pragma unroll
         for (int w = 0; w < 2; ++w) {
-            const unsigned q0 = (unsigned)quant_i8(x[i][4 * w], sc) & 0xffu, q1 = (unsigned)quant_i8(x[i][4 * w + 1], sc) & 0xffu;
-            const unsigned q2 = (unsigned)quant_i8(x[i][4 * w + 2], sc) & 0xffu, q3 = (unsigned)quant_i8(x[i][4 * w + 3], sc) & 0xffu;
+            const unsigned q0 = (unsigned)sage_quant_i8_block(x[i][4 * w], dv) & 0xffu, q1 = (unsigned)sage_quant_i8_block(x[i][4 * w + 1], dv) & 0xffu;
+            const unsigned q2 = (unsigned)sage_quant_i8_block(x[i][4 * w + 2], dv) & 0xffu, q3 = (unsigned)sage_quant_i8_block(x[i][4 * w + 3], dv) & 0xffu;
             o[w] = q0 | (q1 << 8) | (q2 << 16) | (q3 << 24);
         }
         *reinterpret_cast<sg_u2_t *>(dst + (size_t)row * D) = o;
@@ -253,7 +254,7 @@ __global__ void __launch_bounds__(256) sage_append_kernel(SageAppendDev a) {
         }
         amax = wg_max(amax);
         const __half sc16 = __float2half_rn(amax / 127.0f);
-        const float sc = __half2float(sc16);
+        const SageDivisor dv = sage_divisor(__half2float(sc16));
         if (tid == 0) a.k_scale[(size_t)h * ((a.capacity + FA_SAGE_BLOCK - 1) / FA_SAGE_BLOCK) + b0 / FA_SAGE_BLOCK] = sc16;
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
@@ -264,7 +265,7 @@ __global__ void __launch_bounds__(256) sage_append_kernel(SageAppendDev a) {
                     int8_t b[8];
                 } o;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) o.b[i] = (int8_t)quant_i8(x[it][i], sc);
+                for (int i = 0; i < 8; ++i) o.b[i] = (int8_t)sage_quant_i8_block(x[it][i], dv);
                 *reinterpret_cast<uint2 *>(a.k_q + ((size_t)h * a.capacity + b0 + j) * D + ch * 8) = o.u;
             }
         }
