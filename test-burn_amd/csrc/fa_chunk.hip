@@ -29,7 +29,7 @@
 
 namespace {
 
-using fa_lds_dma::buffer_to_lds_b128;
+using fa_lds_dma::buffer_to_lds_b128_nt;
 using fa_lds_dma::make_rsrc_words;
 using fa_lds_dma::rsrc_words;
 
@@ -64,6 +64,8 @@ struct ChunkDev {
     const int32_t *block_table;
     uint32_t n_kv_heads, group_size, q_len, kv_len, query_offset, causal, block_size, block_shift;
     uint32_t part_len;  // keys per partition (a multiple of 32)
+    uint32_t kv_end;    // keys anyone in the chunk can see: kv_len, or min(kv_len, q_len + query_offset) when causal
+    uint32_t nsplits;   // partitions that hold any of them = ceil(kv_end / part_len) = the grid's x dimension
     uint32_t pairs;     // (head of the group, 32-row block) pairs of a KV head: group_size * ceil(q_len / 32)
     uint32_t ncols;     // pairs * 32: columns of a KV head in the partial buffers
     float *part_acc;    // [kv head][partition][column][D] unnormalised sums
@@ -138,7 +140,7 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
     } while (0)
 #define FC_TR_FLUSH()                                                                                               \
     do {                                                                                                            \
-        if (a.trace && lane < 16) {                                                                                 \
+        if (a.trace && lane < 12) {                                                                                 \
             const size_t wg = blockIdx.x + gridDim.x * (blockIdx.y + (size_t)gridDim.y * blockIdx.z);               \
             unsigned long long v = 0;                                                                               \
             for (int i = 0; i < 16; ++i) v = lane == i ? tstamp[i] : v;                                             \
@@ -160,22 +162,8 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
         const uint32_t g = (lin & 7u) + 8u * (slot / gridDim.x);
         split = slot % gridDim.x, kvh = g % gridDim.y, cgrp = g / gridDim.y;
     }
-    const uint32_t G = a.group_size;
-    // this workgroup's column blocks: pairs [8 cgrp, 8 cgrp + pairs_here); wave -> (column block, tile parity)
-    const uint32_t pairs_here = min(8u, a.pairs - cgrp * 8u);
-    const bool halves = pairs_here <= 4u;  // the 8 waves also split each round's 32-key tiles in two sets (even, odd)
-    const uint32_t cb = halves ? (uint32_t)(wave8 & 3) : (uint32_t)wave8;
-    const uint32_t kh = halves ? (uint32_t)(wave8 >> 2) : 0u;
-    const bool active = cb < pairs_here;
-    const uint32_t pair = cgrp * 8u + (active ? cb : 0u);
-    const uint32_t head = kvh * G + pair % G, rb = pair / G;
-    const uint32_t q_row = rb * 32u + (uint32_t)n;  // the query row this lane's column belongs to
-    const uint32_t q_row_c = min(q_row, a.q_len - 1);
-
     // keys anyone in the chunk can see, and this workgroup's partition of them
-    uint32_t kv_end = a.kv_len;
-    if (a.causal) kv_end = (uint32_t)min((uint64_t)a.kv_len, (uint64_t)a.q_len + a.query_offset);
-    const uint32_t nsplits = (kv_end + a.part_len - 1) / a.part_len;
+    const uint32_t kv_end = a.kv_end, nsplits = a.nsplits;
     if (split >= nsplits) return;  // uniform over the workgroup (the mergers count nsplits partitions, too)
     const uint32_t k_lo = split * a.part_len, k_hi = min(kv_end, k_lo + a.part_len);
     // The partition goes through LDS in rounds of RBLKS 16-row blocks (64 keys), round r in slot r % RING of the ring.
@@ -188,18 +176,23 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
     // partition's end come out of the descriptor's bound check as zeros (no memory access), so every block of a round is
     // written whether it holds keys or not.
     // A wave that makes requests faster than memory serves them stalls at the request: that is why the waves that compute
-    // make none. Producers and consumers meet through two counters in LDS, not at barriers (a barrier per round would make
-    // every round as slow as the slower side was in THAT round): `landed` counts (producer, round) parts that are in LDS,
-    // `freed` counts (consumer wave, round) pairs that have been read. A producer keeps up to RING - 1 rounds in flight
-    // and reuses a slot when all 8 consumer waves have read the round that was in it. Every wait is bounded like the
+    // make none. Producers and consumers meet through counters in LDS, not at barriers (a barrier per round would make
+    // every round as slow as the slower side was in THAT round). Each slot of the ring has two: `landed` counts the
+    // producers whose part of the slot's round is in LDS, `freed` the consumer waves that have read it; neither is ever
+    // reset, so round r is complete in its slot at NPROD (r / RING + 1) and read at 8 (r / RING + 1). (One counter for
+    // all rounds would not do: waves of one side run up to RING - 1 rounds apart, and a sum cannot tell four producers
+    // done with round r from two of them done with round r + 1.) A producer keeps up to RING - 1 rounds in flight and
+    // reuses a slot when all 8 consumer waves have read the round that was in it. Every wait is bounded like the
     // merge's; a wave that gives up says so in the status word and runs on without waiting (the launch ends, its output
     // is not valid, the next stream wait reports it).
-    __shared__ uint32_t ring_count[2];  // landed, freed
-    if (tid == 0) ring_count[0] = 0u, ring_count[1] = 0u;
+    __shared__ uint32_t ring_count[2][RING];  // landed, freed
+    if (tid < 2 * RING) ring_count[tid / RING][tid % RING] = 0u;
     const unsigned long long t_ring = wall_clock64();
     bool gave_up = false;
-    auto wait_count = [&](int which, uint32_t target) __attribute__((always_inline)) {
-        while (!gave_up && __hip_atomic_load(&ring_count[which], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
+    // (which: 0 landed, 1 freed) of round r's slot: has everybody on that side done round r?
+    auto wait_count = [&](int which, int r, uint32_t per_round) __attribute__((always_inline)) {
+        const uint32_t target = per_round * (uint32_t)(r / RING + 1);
+        while (!gave_up && __hip_atomic_load(&ring_count[which][r % RING], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
             __builtin_amdgcn_s_sleep(1);
             if (wall_clock64() - t_ring > a.poll_ticks) {
                 gave_up = true;
@@ -208,11 +201,12 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
         }
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
     };
-    auto bump_count = [&](int which) __attribute__((always_inline)) {
+    auto bump_count = [&](int which, int r) __attribute__((always_inline)) {
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
-        if (lane == 0) __hip_atomic_fetch_add(&ring_count[which], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (lane == 0) __hip_atomic_fetch_add(&ring_count[which][r % RING], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     };
     if (wave8 >= 8) {
+        FC_TR(13);
         constexpr int CBR = ROWB / 64;
         const int blk = wave8 - 8;
         const int k_lane_src = (lane & 15) * ROWB + (lane >> 4) * 16;
@@ -243,8 +237,8 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
                 so = 0;
             }
             // K: chunk quads, 64 bytes apart in a row, 1 KB apart in LDS; V: 1 KB of rows after 1 KB of rows
-            buffer_to_lds_b128<K_DMA, 64, 1024>(kr, k_lds_addr + (uint32_t)slot * RB_BYTES, k_lane_src, so);
-            buffer_to_lds_b128<V_DMA, 1024, 1024>(vr, v_lds_addr + (uint32_t)slot * (4 * RG_BYTES), v_lane_src, so);
+            buffer_to_lds_b128_nt<K_DMA, 64, 1024>(kr, k_lds_addr + (uint32_t)slot * RB_BYTES, k_lane_src, so);
+            buffer_to_lds_b128_nt<V_DMA, 1024, 1024>(vr, v_lds_addr + (uint32_t)slot * (4 * RG_BYTES), v_lane_src, so);
         };
         // at most `ahead` rounds' requests of this wave may still be out (they complete in order)
         auto wait_rounds = [&](int ahead) __attribute__((always_inline)) {
@@ -253,21 +247,54 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
             else if (ahead == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | BLK_DMA);
             else __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * BLK_DMA) & 15) | (((2 * BLK_DMA) >> 4) << 14));
         };
+        // (Spacing the first rounds' requests in time, one round of the whole launch per interval at the memory's rate,
+        // was tried so that round 0 would not share the queues with the later rounds: it lands 4.3 - 4.8 us after the
+        // launch either way - 0.9 us until the workgroup knows its partition, 1.1 us until the requests are out, 2.5 us
+        // until the rows are there.)
         int issued = 0, told = 0;
-        for (; issued < min(rounds, RING - 1); ++issued) dma_round(issued);
-        __builtin_amdgcn_s_barrier();  // the counters are zero
+        for (; issued < min(rounds, RING - 1); ++issued) {
+            dma_round(issued);
+#ifdef FA_DECODE_TRACE
+            if (issued == 0) FC_TR(14);
+#endif
+            if (issued == 0) __builtin_amdgcn_s_barrier();  // the counters are zero
+        }
+        if (issued == 0) __builtin_amdgcn_s_barrier();
         while (told < rounds) {
             wait_rounds(issued - told - 1);  // this wave's part of round `told` is in LDS
-            bump_count(0);
+#ifdef FA_DECODE_TRACE
+            if (told == 0) FC_TR(15);
+            if (told == rounds - 1) {
+                if (a.trace && blk == 0 && lane >= 12 && lane < 16) {
+                    const size_t wg = blockIdx.x + gridDim.x * (blockIdx.y + (size_t)gridDim.y * blockIdx.z);
+                    unsigned long long v = 0;
+                    for (int i = 13; i < 16; ++i) v = lane == i ? tstamp[i] : v;
+                    if (lane == 12) v = tstamp[0];
+                    a.trace[(wg * 8 + 3) * 16 + lane] = v;
+                }
+            }
+#endif
+            bump_count(0, told);
             ++told;
             if (issued < rounds) {
-                if (issued >= RING) wait_count(1, 8u * (uint32_t)(issued - RING + 1));  // the slot's last round has been read
+                if (issued >= RING) wait_count(1, issued - RING, 8u);  // the slot's last round has been read
                 dma_round(issued++);
             }
         }
         return;  // (a wave that has ended no longer counts at the workgroup's barriers)
     }
 
+    const uint32_t G = a.group_size;
+    // this workgroup's column blocks: pairs [8 cgrp, 8 cgrp + pairs_here); wave -> (column block, tile parity)
+    const uint32_t pairs_here = min(8u, a.pairs - cgrp * 8u);
+    const bool halves = pairs_here <= 4u;  // the 8 waves also split each round's 32-key tiles in two sets (even, odd)
+    const uint32_t cb = halves ? (uint32_t)(wave8 & 3) : (uint32_t)wave8;
+    const uint32_t kh = halves ? (uint32_t)(wave8 >> 2) : 0u;
+    const bool active = cb < pairs_here;
+    const uint32_t pair = cgrp * 8u + (active ? cb : 0u);
+    const uint32_t head = kvh * G + pair % G, rb = pair / G;
+    const uint32_t q_row = rb * 32u + (uint32_t)n;  // the query row this lane's column belongs to
+    const uint32_t q_row_c = min(q_row, a.q_len - 1);
     // ---- The 8 waves that attend. Q^T operand: lane (n, hi) keeps Q[q_row][16 s + 8 hi .. +8] for every k-step s.
     U4H8 qreg[DSTEPS];
     {
@@ -373,14 +400,14 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
     FC_TR(1);
     __syncthreads();  // the counters are zero
     for (int r = 0; r < rounds; ++r) {
-        wait_count(0, (uint32_t)NPROD * (uint32_t)(r + 1));  // round r is in LDS
+        wait_count(0, r, (uint32_t)NPROD);  // round r is in LDS
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 #ifdef FA_DECODE_TRACE
         if (r == 0) FC_TR(3);
 #endif
         attend_round(r);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // (this wave's reads of the round have completed)
-        bump_count(1);
+        bump_count(1, r);
     }
     FC_TR(4);
     __syncthreads();  // every wave is done with the tiles: the LDS below is reused
@@ -617,6 +644,7 @@ fa_status fa_launch_prefill_chunk(fa_ctx *ctx, const PrefillLaunch &L, bool forc
     a.block_shift = 32;
     if (L.paged && L.block_size && (L.block_size & (L.block_size - 1)) == 0) a.block_shift = (uint32_t)__builtin_ctz(L.block_size);
     a.part_len = part_len, a.pairs = pairs, a.ncols = pairs * 32;
+    a.kv_end = kv_end, a.nsplits = S;
     a.scale_log2e = L.scale * 1.4426950408889634f;
     a.status = ctx->d_status;
     a.poll_ticks = (unsigned long long)ctx->poll_spin_us * 100ull;
