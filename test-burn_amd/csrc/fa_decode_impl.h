@@ -572,12 +572,24 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         // All partitions of a head group on ONE XCD (workgroup id modulo 8), so that their partial states meet in that
         // XCD's L2 instead of in memory: group = id % 8 + 8 (id / 8 / S), partition = id / 8 % S. The host selects this
         // only when the number of head groups is a multiple of 8.
+        // (The quotients by the grid's dimensions are products with reciprocals the host worked out - exact for the
+        // few thousand workgroups a launch of this form can have: a division is two dozen dependent instructions, and
+        // the whole workgroup waits for these values before its first request.)
         const uint32_t lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z), slot = lin >> 3;
-        const uint32_t g = (lin & 7u) + 8u * (slot / gridDim.x);
-        split = slot % gridDim.x, y = g % gridDim.y, b = g / gridDim.y;
+        const uint32_t sq = __umulhi(slot, a.rcp_gx);  // slot / gridDim.x
+        const uint32_t g = (lin & 7u) + 8u * sq;
+        split = slot - sq * gridDim.x;
+        b = __umulhi(g, a.rcp_gy);                     // g / gridDim.y
+        y = g - b * gridDim.y;
     }
+    // A head group that only pads the grid (see the host): its workgroups address the last real group's rows, so that
+    // nothing they request before they leave - with the workgroups of empty partitions, below - is out of range. (Leaving
+    // here, before the first barrier, cost every launch of the kernel 0.4 us, and even these few instructions cost the
+    // 8-wave form 0.09 us per launch at 8K context: only the 4-wave form, which the small launches use, has them.)
+    const bool pad_wg = NW == 4 && a.ny_real != 0 && y >= a.ny_real;
+    if (pad_wg) y = a.ny_real - 1;
     const uint32_t gt = a.gt;
-    const uint32_t kvh = y / a.sub_per_kv;
+    const uint32_t kvh = a.sub_per_kv == 1u ? y : y / a.sub_per_kv;  // (the division off the common path: see the reciprocals above)
     const uint32_t head0 = y * gt;
     const uint32_t S = gridDim.x;
     uint32_t chunk = a.chunk, k0 = split * chunk;  // (a paged launch evens its partitions out once the length is known)
@@ -993,7 +1005,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // A position at or past the launch bound / the capacity: the token is neither appended nor attended. The host
     // finds the bit at its next synchronize.
     if (FUSED && n_raw > N && tid == 0 && blockIdx.x == 0 && y == 0 && a.status) a.status[FA_DEVSTAT_APPEND_DROPPED] = 1u;
-    if (split >= nsplits) {  // uniform over the workgroup
+    if (split >= nsplits || pad_wg) {  // uniform over the workgroup
         FA_TR_FLUSH();
         return;
     }

@@ -206,6 +206,8 @@ struct FaDecodeDev {
     uint32_t bf16;  // data tensors are bf16 (RoPE tables stay f16)
     uint32_t *status;  // the context's device-written status words (one per FA_DEVSTAT_* condition)
     uint32_t xcd_local;  // polled merge: a head group's workgroups share an XCD and exchange partials through its L2
+    uint32_t rcp_gx, rcp_gy;  // xcd_local: floor(2^32 / d) + 1 for the grid's x and y dimensions (exact quotients of numbers below 2^16 by d < 2^16)
+    uint32_t ny_real;    // != 0: the grid's y dimension is padded (to a multiple of 8 head groups) and only y < ny_real exist
     unsigned long long poll_ticks;  // polled merge: how long the merging workgroup waits for partials, 100 MHz ticks
     // SAGE + FUSED (the int8 decode step in one launch): q is the raw f16 projection, k the int8 cache (written: the open
     // block's rows), k_scale is written too; the exact rows of the open block, the smoothing mean, the step's quantised query
