@@ -321,7 +321,7 @@ fa_status fa_set_prefill_split_k(fa_ctx *ctx, uint32_t split_k);
  * prefix once, like a decode step, and merges the partitions inside the launch (same residency assumption, wait bound
  * and reporting as the polled decode merge above; its partial states use the context's workspace, which cannot grow
  * inside a capture); 0 (default) = 2, with the short-chunk kernel where it is measured to win: at most 64 rows, at
- * least 2048 visible keys, group_size * ceil(rows / 32) <= 4, and no split-K override. Same contract; the variants
+ * least 2048 visible keys, group_size * ceil(rows / 32) <= 8, and no split-K override. Same contract; the variants
  * differ in the order in which a row's weights are summed (outputs agree to one f16 ulp).
  * Environment: FOUNDRY_ATTN_PREFILL_VARIANT (read at fa_ctx_create). */
 fa_status fa_set_prefill_variant(fa_ctx *ctx, uint32_t variant);

@@ -15,8 +15,9 @@
 // do nothing else - and each of the other 8 waves attends them for its own column block with v_mfma_f32_32x32x16
 // (S^T = K Q^T with Q^T resident in registers, P^T straight from the S^T accumulators, V^T through ds_read_b64_tr_b16:
 // the tiling of the prefill kernel, fa_prefill.hip). With at most 4 column blocks the 8 waves split each round's keys in
-// two halves as well; that is the case the host routes here by default (with more column blocks every wave attends
-// every key and the launch is bound by arithmetic, where the tiled kernel is as good).
+// two halves as well; with 5 to 8 every wave attends every key and the launch is bound by arithmetic (64 rows x 3 heads
+// after 8K tokens: 26.0 us against 27.0 us for the tiled kernel and its merge launch). The host routes chunks of up to
+// 8 column blocks here by default.
 //
 // Merge: every workgroup stores its unnormalised state - acc [column][D] f32, then, once those stores have completed,
 // (m, l) per column into a buffer whose words hold an all-ones pattern between launches - and then merges ITS share of the
@@ -624,7 +625,8 @@ fa_status fa_launch_prefill_chunk(fa_ctx *ctx, const PrefillLaunch &L, bool forc
     // below a few hundred keys per compute unit's share the launch is all fixed cost either way: the tiled kernel keeps it
     if (!force && kv_end < 2048) return FA_OK;
     const uint32_t nb = ceil_div_u32(L.q_len, 32), pairs = L.group_size * nb, cgroups = ceil_div_u32(pairs, 8);
-    if (!force && pairs > 4) return FA_OK;  // (measured: 64 rows x 3 heads after 8K tokens is no faster here than tiled)
+    // (with more than 8 column blocks a KV head's keys would be read once per group of 8: the tiled kernel keeps those)
+    if (!force && pairs > 8) return FA_OK;
     const uint32_t groups = L.n_kv_heads * cgroups;
     if (groups > n_cus) return FA_OK;
     if (!L.paged && (uint64_t)L.kv_len * L.head_dim * 2 >= (1ull << 32)) return FA_OK;  // (the tiled kernel reports it)
