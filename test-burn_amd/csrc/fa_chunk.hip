@@ -282,6 +282,11 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
                 dma_round(issued++);
             }
         }
+        // (Tried: one producer staying on through the other waves' barriers to ask for the write-back of the partial
+        // sums while the others merge. They are megabytes of modified L2 lines when the exchange is XCD-local, and the
+        // suspicion was that writing them back at the end of the launch is why launches of a graph follow one another
+        // 2 us apart here against 0.4 us after a decode launch. An agent-scope release from every workgroup: 26.8 us per
+        // launch instead of 19.3; from one workgroup per XCD: no gain.)
         return;  // (a wave that has ended no longer counts at the workgroup's barriers)
     }
 
