@@ -319,7 +319,8 @@ fa_status fa_set_prefill_split_k(fa_ctx *ctx, uint32_t split_k);
  * 2048 tokens, 14 % at 8192 and on a paged cache); 3 = 2, and every launch of at most 64 query rows (head_dim 64 or
  * 128) goes to the short-chunk kernel: one workgroup per (KV head, context partition) that reads its share of the
  * prefix once, like a decode step, and merges the partitions inside the launch (same residency assumption, wait bound
- * and reporting as the polled decode merge above; its partial states use the context's workspace, which cannot grow
+ * and reporting as the polled decode merge above - after a give-up the context leaves this kernel out until
+ * fa_set_prefill_variant is called again -; its partial states use the context's workspace, which cannot grow
  * inside a capture); 0 (default) = 2, with the short-chunk kernel where it is measured to win: at most 64 rows, at
  * least 2048 visible keys, group_size * ceil(rows / 32) <= 8, and no split-K override. Same contract; the variants
  * differ in the order in which a row's weights are summed (outputs agree to one f16 ulp).

@@ -201,10 +201,15 @@ fa_status fa_check_device_status(fa_ctx *ctx) {
         (void)hipMemsetAsync(ctx->poll_ws, 0xff, ctx->poll_ws_bytes, ctx->stream);
         (void)hipStreamSynchronize(ctx->stream);
         if (ctx->decode_variant.merge == 2) ctx->decode_variant.merge = 1;
+        // (the short-chunk prefill kernel merges inside its launch under the same assumption, and its waits raise the
+        // same word: it is left out, too, until fa_set_prefill_variant selects a variant again)
+        ctx->prefill_chunk_off = true;
+        if (ctx->prefill_variant == 3) ctx->prefill_variant = 2;
         return fa_fail(FA_ERR_OPERATION_FAILED,
-                       "a decode launch's merging workgroup waited longer than %u us for the other partitions; the "
-                       "outputs of the decode calls since the last wait for the stream are invalid%s. The context now merges "
-                       "partitions with a second launch (decode merge = 1); fa_set_decode_variant re-enables the polled form",
+                       "a decode or short-chunk prefill launch's workgroup waited longer than %u us for the other partitions; the "
+                       "outputs of the attention calls since the last wait for the stream are invalid%s. The context now merges "
+                       "partitions with a second launch (decode merge = 1, tiled prefill kernel for short chunks); "
+                       "fa_set_decode_variant and fa_set_prefill_variant re-enable the forms that merge inside the launch",
                        ctx->poll_spin_us, dropped ? " (a fused decode step was also dropped: position beyond its bound)" : "");
     }
     return fa_fail(FA_ERR_INVALID_OPERATION,
@@ -305,6 +310,7 @@ extern "C" fa_status fa_set_prefill_variant(fa_ctx *ctx, uint32_t variant) {
     FA_NEED(ctx, "ctx");
     if (variant > 3) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "prefill variant must be 0 ... 3, got %u", variant);
     ctx->prefill_variant = variant;
+    ctx->prefill_chunk_off = false;  // (set by a give-up of the short-chunk kernel: a new selection starts afresh)
     return FA_OK;
 }
 

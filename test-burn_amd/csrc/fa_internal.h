@@ -65,6 +65,7 @@ struct fa_ctx {
     uint32_t gemm_min_m = 0;       // FusedQkv / MatMul: input rows from which the GEMM runs (0 = default)
     uint32_t prefill_split_k = 0;  // 0 = auto
     uint32_t sage_fused_step = 1;  // the int8 decode step as one launch (env FOUNDRY_ATTN_SAGE_FUSED=0: append kernel + decode kernel)
+    bool prefill_chunk_off = false;  // a wait inside the short-chunk prefill kernel (or the polled decode merge) has run out: not routed to until fa_set_prefill_variant
     uint32_t prefill_variant = 0;  // 0 = auto, 1 = tiles staged through registers, 2 = tiles straight into LDS, two-phase loop, 3 = as 0 with the chunk kernel wherever it applies
     // optional: the prefill kernel leaves {shader-clock ticks, wall ticks} per workgroup here (fa_profile_clock_buffer)
     unsigned long long *clock_buf = nullptr;

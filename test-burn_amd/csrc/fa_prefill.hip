@@ -1040,7 +1040,7 @@ fa_status fa_launch_prefill(fa_ctx *ctx, const PrefillLaunch &L) {
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "Prefill only supports head_dim=64 or 128, got %u", L.head_dim);
     // A chunk of at most 64 rows after a long prefix is a memory-bound launch: fa_chunk.hip (unless a kernel or a split
     // count has been asked for by name)
-    if ((ctx->prefill_variant == 0 && ctx->prefill_split_k == 0) || ctx->prefill_variant == 3) {
+    if (!ctx->prefill_chunk_off && ((ctx->prefill_variant == 0 && ctx->prefill_split_k == 0) || ctx->prefill_variant == 3)) {
         bool taken = false;
         FA_TRY(fa_launch_prefill_chunk(ctx, L, ctx->prefill_variant == 3, &taken));
         if (taken) return FA_OK;

@@ -355,6 +355,7 @@ def test_prefill_chunk_kernel_gives_up_cleanly():
         g.set_decode_poll_spin_us(0)
         reported = 0
         for _ in range(3):
+            g.set_prefill_variant(3)  # (a give-up takes the kernel out until it is selected again)
             g.flash_attention(dq.arg((H, M, D)), dk.arg(), dv.arg(), do.arg(), True, prefix, H, D, N, M)
             try:
                 g.synchronize()
@@ -362,6 +363,11 @@ def test_prefill_chunk_kernel_gives_up_cleanly():
                 reported += 1
                 assert e.variant == "OperationFailed" and "waited longer" in str(e)
         assert reported >= 1  # (a wave cannot find a whole round in LDS at its first look)
+        # after a give-up the context leaves the kernel out: right again at once, zero bound or not (tiled kernel + merge launch)
+        g.flash_attention(dq.arg((H, M, D)), dk.arg(), dv.arg(), do.arg(), True, prefix, H, D, N, M)
+        assert max_abs(do.download().reshape(M, H * D), want.reshape(M, H * D)) <= TOL
+        # ... and selecting the variant again brings the kernel back, which with the normal bound is right
+        g.set_prefill_variant(3)
         g.set_decode_poll_spin_us(5000)
         for _ in range(3):
             g.flash_attention(dq.arg((H, M, D)), dk.arg(), dv.arg(), do.arg(), True, prefix, H, D, N, M)
