@@ -895,6 +895,108 @@ def bench_prefill_chunk(f, args, m=32, prefix=8160):
         "parity": {"max_abs_err_vs_oracle": err}})
 
 
+def bench_phase_timeline(f, args, which="decode_8k"):
+    """Where a launch's time goes, from clock stamps the kernels take themselves: only a development build of the
+    library has them (python test-burn_amd/build.py with FOUNDRY_ATTN_BUILD_TAG=_trace and
+    FOUNDRY_ATTN_BUILD_FLAGS=-DFA_DECODE_TRACE in the environment builds libfoundry_attn_trace.so beside the product library;
+    FOUNDRY_ATTN_LIB selects it). Every wave stamps the 100 MHz wall clock at the kernel's phase boundaries and leaves the
+    stamps in the clock buffer; the workload is replayed as a HIP graph and the phases are reported in microseconds after
+    the first workgroup's entry, as min / median / 90th percentile / max over the waves that reached them.
+    which: decode_8k (the fused decode step of the main configuration), sage_32k (the int8 step, wave 0 of every workgroup
+    = the wave that prepares the query and owns the open block), chunk32_8k (the short-chunk prefill kernel)."""
+    rng = np.random.default_rng(0xF0DD + 21)
+    if which == "decode_8k":
+        st = make_llama3b_decode(f, rng, 8192, 64)
+        per_graph, waves, rows = 2 * 28, 8, 256 * 8
+        names = ["entry", "start barrier released", "block requests issued", "query operand ready", "first round: S done",
+                 "first round: V in LDS", "block loop done", "state in LDS", "fold starts", "records stored", "merge done"]
+
+    elif which == "sage_32k":
+        H, Hkv, D, N, NL = 16, 4, 128, 32768, 6
+        P = N - 1
+        cos, sin = fa.rope_tables(5e6, D, N)
+        dcos, dsin = f.array(cos), f.array(sin)
+        k = rng.standard_normal((Hkv, N, D), dtype=np.float32).astype(np.float16)
+        v = rng.standard_normal((Hkv, N, D), dtype=np.float32).astype(np.float16)
+        k[:, P:], v[:, P:] = 0, 0
+        layers = []
+        for _ in range(NL):
+            dk, dv = f.array(k), f.array(v)
+            desc, bufs = fa.sage_cache(f, H, Hkv, N, D, dv)
+            f.sage_cache_build(dk, P, desc)
+            f.synchronize()
+            dk.free()
+            layers.append((desc, bufs))
+        q, kn, vn = (rng.standard_normal((1, n * D), dtype=np.float32).astype(np.float16) for n in (H, Hkv, Hkv))
+        dq, dkn, dvn, dout = f.array(q), f.array(kn), f.array(vn), f.zeros((H * D,))
+        params = [fa.KvPrepFusedParams.make(H, Hkv, D, 1, P, N, fa.ROPE_NEOX, layer_idx=i, no_rope_layer_step=4) for i in range(NL)]
+        per_graph, waves, rows = 2 * NL, 8, 256 * 8
+        names = ["entry", "start barrier released", "block requests issued", "query operand ready", "first round: S done",
+                 "first round: V in LDS", "block loop done", "state in LDS", "fold starts", "records stored", "merge done",
+                 "wave 0: table row and mean in LDS", "wave 0: open block's scale known", "wave 0: open block quantised",
+                 "wave 0: open block attended"]
+
+        def step(i):
+            f.sage_decode_step(dq.arg(), dkn.arg(), dvn.arg(), layers[i % NL][0], dcos.arg(), dsin.arg(), dout.arg(), params[i % NL])
+    else:
+        H, Hkv, D, L, m, prefix = 24, 8, 128, 28, 32, 8160
+        N, cap = prefix + m, prefix + 512
+        k0 = rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16)
+        v0 = rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16)
+        caches = [(f.array(k0), f.array(v0)) for _ in range(L)]
+        dq, dout = f.array(rng.standard_normal((H, m, D), dtype=np.float32).astype(np.float16)), f.zeros((m, H * D))
+        per_graph, waves, rows = L, 8, 256 * 8
+        names = ["entry", "query rows requested", None, "round 0 in LDS (seen by this wave)", "last tile attended", "after the barrier",
+                 "key halves folded", "state stored", "merge starts", "rows written", "all (m, l) of the first batch seen",
+                 "sums of the first pass folded", "producer 0: entry", "producer 0: in its branch", "producer 0: round 0 requested",
+                 "producer 0: round 0 landed"]
+
+        def step(i):
+            kc, vc = caches[i % L]
+            f.flash_attention(dq.arg(), kc.arg(), vc.arg(), dout.arg(), True, prefix, H, D, N, m)
+    if which == "decode_8k":
+        def run(n):  # (the decode bench's own step: 28 layers per call)
+            for s_ in range(n // 28):
+                enqueue_step(f, st, s_, True)
+    else:
+        def run(n):
+            for i in range(n):
+                step(i)
+    run(per_graph)
+    f.synchronize()
+    buf = fa.DevBuf(f, (rows * 16,), np.uint64)
+    buf.upload(np.zeros((rows * 16,), np.uint64))
+    f.profile_clock_buffer(buf, rows * 8)
+    f.start_capture()
+    run(per_graph)
+    graph = f.end_capture()
+    phases, span = {}, None
+    for rep in range(4):
+        graph.launch()
+        f.synchronize()
+    t = buf.download().reshape(rows, 16).astype(np.float64)  # the last launch of the last replay
+    f.profile_clock_buffer(None, 0)
+    graph.destroy()
+    live = t[:, 0] > 0
+    if not live.any():
+        sys.exit("no stamps in the clock buffer: this library was built without -DFA_DECODE_TRACE (see the workload's description)")
+    t0 = t[live, 0].min()
+    for i, nm in enumerate(names):
+        if nm is None:
+            continue
+        col = t[:, i][t[:, i] > 0]
+        if col.size:
+            us = (col - t0) / 100.0
+            phases[nm] = {"waves": int(col.size), "min": round(float(us.min()), 2), "p50": round(float(np.median(us)), 2),
+                          "p90": round(float(np.percentile(us, 90)), 2), "max": round(float(us.max()), 2)}
+    emit({"metric": "phase timeline of one launch, us after the first workgroup's entry (%s)" % which, "value": max(p["max"] for p in phases.values()),
+          "unit": "us", "n_gpus": 1, "steps": per_graph, "warmup": per_graph, "ms_per_step": None, "higher_is_better": False,
+          "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+          "config": {"workload": "clock stamps inside the kernel, development build of the library; graph replays, the stamps of "
+                                 "the last launch of the last replay"},
+          "phases": phases})
+
+
 def bench_prefill_block(f, args, fused=False):
     """The attention block of one Llama-3.2-3B layer on a 2048-token prompt in one chunk (models/llama.json:509-585):
     FusedQkv (norm kernel + GEMM) -> KvPrepFused (RoPE + append of 2048 rows) -> FlashAttention (causal prefill) -> o_proj
@@ -1223,7 +1325,7 @@ def bench_floors(f, args):
     emit(out)
 
 
-SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_chunk32_8k": bench_prefill_chunk, "llama3b_prefill_chunk32_32k": lambda f, args: bench_prefill_chunk(f, args, 32, 32736), "llama3b_prefill_chunk64_8k": lambda f, args: bench_prefill_chunk(f, args, 64, 8128), "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_decode_2k": bench_short_decode, "llama3b_decode_512": lambda f, args: bench_short_decode(f, args, 511), "llama3b_prefill_2k": bench_prefill,
+SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_chunk32_8k": bench_prefill_chunk, "llama3b_prefill_chunk32_32k": lambda f, args: bench_prefill_chunk(f, args, 32, 32736), "llama3b_prefill_chunk64_8k": lambda f, args: bench_prefill_chunk(f, args, 64, 8128), "timeline_decode_8k": bench_phase_timeline, "timeline_sage_32k": lambda f, args: bench_phase_timeline(f, args, "sage_32k"), "timeline_chunk32_8k": lambda f, args: bench_phase_timeline(f, args, "chunk32_8k"), "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_decode_2k": bench_short_decode, "llama3b_decode_512": lambda f, args: bench_short_decode(f, args, 511), "llama3b_prefill_2k": bench_prefill,
              "llama3b_prefill_8k": lambda f, args: bench_prefill(f, args, 8192), "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,
