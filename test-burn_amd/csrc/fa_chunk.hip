@@ -70,7 +70,8 @@ struct ChunkDev {
     uint32_t pairs;     // (head of the group, 32-row block) pairs of a KV head: group_size * ceil(q_len / 32)
     uint32_t ncols;     // pairs * 32: columns of a KV head in the partial buffers
     float *part_acc;    // [kv head][partition][column][D] unnormalised sums
-    float *part_ml;     // [kv head][partition][column][2] (max, sum); every word 0xffffffff between launches
+    float *part_ml;     // [kv head][partition][column][D / 32][2] (max, sum), one copy for each wave that merges a piece of the
+                        // column; every word 0xffffffff between launches
     float scale_log2e;
     uint32_t xcd_local;            // the workgroups of a KV head share an XCD: partials meet in its L2
     unsigned long long poll_ticks; // bound of a merging thread's wait for the other partitions, 100 MHz ticks
@@ -478,7 +479,7 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
     const __amdgpu_buffer_rsrc_t rs_acc =
         __builtin_amdgcn_make_buffer_rsrc(a.part_acc + grp_rows * D, 0, (int)0xffffffffu, 0x00020000);
     const __amdgpu_buffer_rsrc_t rs_ml =
-        __builtin_amdgcn_make_buffer_rsrc(a.part_ml + grp_rows * 2, 0, (int)0xffffffffu, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(a.part_ml + grp_rows * (2 * (CG / 8)), 0, (int)0xffffffffu, 0x00020000);
     if (owner && q_row < a.q_len) {
         const uint32_t prow = split * ncols + pair * 32u + (uint32_t)n;
 #pragma unroll
@@ -494,32 +495,38 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
         if (hi == 0) {
             const u2_t mlv = {__float_as_uint(not_pattern(m_run)), __float_as_uint(not_pattern(l_tot))};
-            __builtin_amdgcn_raw_buffer_store_b64(mlv, rs_ml, (int)(prow * 2u * 4u), 0, ST_POLICY);
+#pragma unroll
+            for (int cp = 0; cp < CG / 8; ++cp)  // (a copy per merging wave: each consumes and clears its own)
+                __builtin_amdgcn_raw_buffer_store_b64(mlv, rs_ml, (int)((prow * (CG / 8) + cp) * 2u * 4u), 0, ST_POLICY);
         }
     }
     FC_TR(7);
     __syncthreads();  // every wave is done with the LDS it parked in: the merge below folds through it
     FC_TR(8);
 
-    // Merge of this workgroup's columns: split, split + nsplits, ... Thread (c4 = tid % CG, r = tid / CG): float4 column c4;
-    // the RL = 512 / CG row lanes are dealt to the columns of a pass, lph lanes per column, and a column's lanes take its
-    // partitions q, q + lph, ... in order; an LDS pass then folds the lanes in lane order.
-    constexpr int RL = NTC / CG;
+    // Merge of this workgroup's columns: split, split + nsplits, ... A wave holds 8 float4 columns (c4) x 8 row lanes: lane
+    // l is column 8 (wave % (CG / 8)) + l % 8, row lane 8 (wave / (CG / 8)) + l / 8; 8 lanes read one 128-byte line. The
+    // RL = 512 / CG row lanes are dealt to the columns of a pass, lph = 1, 2, 4 or 8 lanes per column, so that a column's
+    // lanes are lanes of ONE wave: each takes the column's partitions q, q + lph, ... in order, and lane exchanges
+    // (lanes 8, 16 and 32 apart) fold them - no LDS, no barrier, and no wave waits for another wave's partitions.
+    constexpr int RL = NTC / CG, CGW = CG / 8;
     constexpr int PB = 8;  // partitions per thread and batch: all loads of a batch in flight together
     // (the columns of this workgroup's own column group: col0 .. col0 + 32 pairs_here)
     const uint32_t col0 = cgrp * 256u, gcols = pairs_here * 32u;
     const uint32_t nmy = gcols > split ? (gcols - split + nsplits - 1) / nsplits : 0u;
-    const int c4 = tid % CG, rl = tid / CG;
+    const int c4 = (wave8 % CGW) * 8 + (lane & 7), rl = (wave8 / CGW) * 8 + (lane >> 3);
     const unsigned long long t_begin = wall_clock64();
     bool timed_out = false;
-    float *sm = reinterpret_cast<float *>(lds);  // [NTC][6]: m, l, acc
-    for (uint32_t j0 = 0; j0 < nmy; j0 += RL) {  // uniform over the workgroup
-        const uint32_t hpp = min(nmy - j0, (uint32_t)RL), lph = (uint32_t)RL / hpp;
+    uint32_t hpp = 0;
+    for (uint32_t j0 = 0; j0 < nmy; j0 += hpp) {  // uniform over the workgroup
+        uint32_t lph = 8;
+        while (lph > 1 && (uint32_t)RL / lph < nmy - j0) lph >>= 1;
+        hpp = (uint32_t)RL / lph;  // columns of this pass (not all of them need exist)
         const uint32_t jl = (uint32_t)rl / lph, q = (uint32_t)rl % lph;
         const uint32_t col = col0 + split + (j0 + jl) * nsplits;
         // column -> (pair, row in block) -> (head, query row)
         const uint32_t cpair = col / 32u, crow = (cpair / G) * 32u + col % 32u, chead = kvh * G + cpair % G;
-        const bool mine = jl < hpp && col < col0 + gcols && crow < a.q_len;
+        const bool mine = j0 + jl < nmy && col < col0 + gcols && crow < a.q_len;
         MergeState st = {-1e30f, 0.0f, {0.0f, 0.0f, 0.0f, 0.0f}};
         // Every load of a batch is issued whether its lane wants it or not (an unwanted one reads row 0): a load inside a
         // branch makes the compiler wait for all earlier ones first, and the batch would take one round trip per partition.
@@ -539,7 +546,7 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
                 u2_t got[PB];
 #pragma unroll
                 for (int kk = 0; kk < PB; ++kk)
-                    got[kk] = __builtin_amdgcn_raw_buffer_load_b64(rs_ml, (int)(rowi[kk] * 2u * 4u), 0, LD_POLICY);
+                    got[kk] = __builtin_amdgcn_raw_buffer_load_b64(rs_ml, (int)((rowi[kk] * CGW + (uint32_t)(wave8 % CGW)) * 2u * 4u), 0, LD_POLICY);
 #pragma unroll
                 for (int kk = 0; kk < PB; ++kk) {
                     const bool fresh = (pend >> kk & 1u) && got[kk].x != CHUNK_SENTINEL && got[kk].y != CHUNK_SENTINEL;
@@ -564,42 +571,42 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
 #pragma unroll
             for (int kk = 0; kk < PB; ++kk)
                 merge_in(st, (want >> kk & 1u) != 0, __uint_as_float(ml[kk].x), __uint_as_float(ml[kk].y), x[kk]);
-            // consumed: the pattern goes back for the next launch (one lane of the 32 that read the same pair)
-            if (c4 == 0) {
+            // consumed: the pattern goes back for the next launch (this wave's own copy of the pair; one lane of the 8 that read it)
+            if ((lane & 7) == 0) {
                 const u2_t pat = {CHUNK_SENTINEL, CHUNK_SENTINEL};
 #pragma unroll
                 for (int kk = 0; kk < PB; ++kk)
-                    if (want >> kk & 1u) __builtin_amdgcn_raw_buffer_store_b64(pat, rs_ml, (int)(rowi[kk] * 2u * 4u), 0, ST_POLICY);
+                    if (want >> kk & 1u)
+                        __builtin_amdgcn_raw_buffer_store_b64(pat, rs_ml, (int)((rowi[kk] * CGW + (uint32_t)(wave8 % CGW)) * 2u * 4u), 0, ST_POLICY);
             }
         }
 #ifdef FA_DECODE_TRACE
         asm volatile("" ::"v"(st.acc[0] + st.l));
         if (tstamp[11] == 0) FC_TR(11);
 #endif
-        // fold the lph lanes of a column in lane order
-        *reinterpret_cast<f2_t *>(sm + (size_t)tid * 2) = f2_t{st.m, st.l};
-        *reinterpret_cast<f4_t *>(sm + 2 * NTC + (size_t)tid * 4) = st.acc;
-        const int any_timeout = __syncthreads_or(timed_out ? 1 : 0);
+        if (__any(timed_out ? 1 : 0)) {  // (the whole wave leaves: nothing it would write can be trusted)
+            if (lane == 0 && a.status) a.status[FA_DEVSTAT_MERGE_TIMEOUT] = 1u;
+            break;
+        }
+        // fold the lph lanes of a column: partners 8, 16, 32 lanes away (every lane takes part; an idle one carries an
+        // empty state, which counts for nothing)
+#pragma unroll
+        for (uint32_t off = 8; off < 64; off <<= 1) {
+            if (off >= 8u * lph) break;  // uniform
+            const float pm = __shfl_xor(st.m, (int)off), pl = __shfl_xor(st.l, (int)off);
+            const f4_t pa = {__shfl_xor(st.acc[0], (int)off), __shfl_xor(st.acc[1], (int)off), __shfl_xor(st.acc[2], (int)off),
+                             __shfl_xor(st.acc[3], (int)off)};
+            merge_in(st, true, pm, pl, pa);
+        }
 #ifdef FA_DECODE_TRACE
         if (tstamp[12] == 0) FC_TR(12);
 #endif
-        if (mine && q == 0 && !any_timeout) {
-            MergeState tot = {-1e30f, 0.0f, {0.0f, 0.0f, 0.0f, 0.0f}};
-            for (uint32_t jj = 0; jj < lph; ++jj) {
-                const size_t t = (size_t)(rl + jj) * CG + c4;
-                const f2_t mlj = *reinterpret_cast<const f2_t *>(sm + t * 2);
-                merge_in(tot, true, mlj.x, mlj.y, *reinterpret_cast<const f4_t *>(sm + 2 * NTC + t * 4));
-            }
-            const float inv = (isfinite(tot.l) && fabsf(tot.l) > 1e-6f) ? (1.0f / tot.l) : 0.0f;
+        if (mine && q == 0) {
+            const float inv = (isfinite(st.l) && fabsf(st.l) > 1e-6f) ? (1.0f / st.l) : 0.0f;
             h4_t h;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) h[e] = to_elem<BF16>(tot.acc[e] * inv);
+            for (int e = 0; e < 4; ++e) h[e] = to_elem<BF16>(st.acc[e] * inv);
             *reinterpret_cast<h4_t *>(a.out + (size_t)chead * a.out_stride_h + (size_t)crow * a.out_stride_m + c4 * 4) = h;
-        }
-        __syncthreads();
-        if (any_timeout) {
-            if (tid == 0 && a.status) a.status[FA_DEVSTAT_MERGE_TIMEOUT] = 1u;
-            return;
         }
     }
     FC_TR(9);
@@ -660,7 +667,7 @@ fa_status fa_launch_prefill_chunk(fa_ctx *ctx, const PrefillLaunch &L, bool forc
 #endif
     if (S > 1) {
         const size_t rows = (size_t)L.n_kv_heads * S * a.ncols;
-        const size_t acc_bytes = rows * L.head_dim * sizeof(float), ml_bytes = rows * 2 * sizeof(float);
+        const size_t acc_bytes = rows * L.head_dim * sizeof(float), ml_bytes = rows * 2 * sizeof(float) * (L.head_dim / 32);  // (a copy per merging wave: see the kernel)
         if (acc_bytes >= (1ull << 31) || ml_bytes > ctx->poll_ws_bytes || !ctx->poll_ws) return FA_OK;
         FA_TRY(fa_ensure_workspace(ctx, acc_bytes));
         a.part_acc = (float *)ctx->workspace;
