@@ -420,75 +420,94 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
     __syncthreads();  // every wave is done with the tiles: the LDS below is reused
     FC_TR(5);
 
-    // With split tiles: the odd tiles' waves park their state in LDS - (m, l) as [column block][lane], the sums as
-    // [accumulator quad][column block][lane] float4 - and the even tiles' waves fold it in
+    // With split tiles the two waves of a column block share what is left: the wave of the even tiles keeps the lower half
+    // of the head dimension (32-dim blocks 0 .. DBLKS / 2 - 1), the wave of the odd tiles the upper half. Each parks (m, l)
+    // - as [half][column block][lane] - and the blocks it gives away - [half][accumulator quad][column block][lane] float4 -
+    // in LDS, and after a barrier folds what the other parked into the blocks it keeps.
+    constexpr int HB = DBLKS / 2;
+    const int b_lo = halves ? (int)kh * HB : 0, b_n = halves ? HB : DBLKS;  // this wave's blocks from here on
     if (halves) {
-        f2_t *mx_ml = reinterpret_cast<f2_t *>(lds);
-        f4_t *mx_acc = reinterpret_cast<f4_t *>(lds + 256 * sizeof(f2_t));
+        f2_t *mx_ml = reinterpret_cast<f2_t *>(lds);                              // [2][256]
+        f4_t *mx_acc = reinterpret_cast<f4_t *>(lds + 2 * 256 * sizeof(f2_t));    // [2][HB * 4][256]
         const int slot = (int)cb * 64 + lane;
-        if (kh == 1 && active) {
-            mx_ml[slot] = f2_t{m_run, l_run};
+        if (active) {
+            mx_ml[kh * 256 + slot] = f2_t{m_run, l_run};
 #pragma unroll
-            for (int b = 0; b < DBLKS; ++b)
+            for (int bb = 0; bb < HB; ++bb)
 #pragma unroll
-                for (int gi = 0; gi < 4; ++gi)
-                    mx_acc[(b * 4 + gi) * 256 + slot] = f4_t{oacc[b][gi * 4], oacc[b][gi * 4 + 1], oacc[b][gi * 4 + 2], oacc[b][gi * 4 + 3]};
+                for (int gi = 0; gi < 4; ++gi) {
+                    // (constant register indices: the give-away half is chosen by a select, not by an index)
+                    f4_t v;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] = kh == 0 ? oacc[HB + bb][gi * 4 + e] : oacc[bb][gi * 4 + e];
+                    mx_acc[((int)kh * HB * 4 + bb * 4 + gi) * 256 + slot] = v;
+                }
         }
         __syncthreads();
-        if (kh == 0 && active) {
-            const f2_t ml1 = mx_ml[slot];
+        if (active) {
+            const int oh = 1 - (int)kh;
+            const f2_t ml1 = mx_ml[oh * 256 + slot];
             const float m = fmaxf(m_run, ml1.x);
             const float e0 = fast_exp2(m_run - m), e1 = fast_exp2(ml1.x - m);
             l_run = l_run * e0 + ml1.y * e1;
+            // the kept blocks move to registers 0 .. HB - 1 of the accumulator array (constant indices again)
 #pragma unroll
-            for (int b = 0; b < DBLKS; ++b)
+            for (int bb = 0; bb < HB; ++bb)
 #pragma unroll
                 for (int gi = 0; gi < 4; ++gi) {
-                    const f4_t o1 = mx_acc[(b * 4 + gi) * 256 + slot];
+                    const f4_t o1 = mx_acc[(oh * HB * 4 + bb * 4 + gi) * 256 + slot];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) oacc[b][gi * 4 + e] = oacc[b][gi * 4 + e] * e0 + o1[e] * e1;
+                    for (int e = 0; e < 4; ++e) {
+                        const float mine_v = kh == 0 ? oacc[bb][gi * 4 + e] : oacc[HB + bb][gi * 4 + e];
+                        oacc[bb][gi * 4 + e] = mine_v * e0 + o1[e] * e1;
+                    }
                 }
             m_run = m;
         }
     }
     FC_TR(6);
-    const bool owner = active && kh == 0;  // this wave holds the partition's state of its 32 columns
+    // (from here on accumulator block bb of this wave is 32-dim block b_lo + bb of its 32 columns, bb < b_n)
     const float l_tot = l_run + __shfl_xor(l_run, 32);
 
     if (nsplits == 1) {  // finalise, flash_prefill.metal:255-261
-        if (owner && q_row < a.q_len) {
+        if (active && q_row < a.q_len) {
             const float inv_l = (isfinite(l_tot) && fabsf(l_tot) > 1e-6f) ? (1.0f / l_tot) : 0.0f;
             __half *op = a.out + (size_t)head * a.out_stride_h + (size_t)q_row * a.out_stride_m;
 #pragma unroll
-            for (int b = 0; b < DBLKS; ++b)
+            for (int bb = 0; bb < DBLKS; ++bb)
 #pragma unroll
                 for (int gi = 0; gi < 4; ++gi) {
-                    // accumulators 4 gi .. 4 gi + 3 are d = 32 b + 8 gi + 4 hi + 0..3
+                    if (bb >= b_n) break;  // uniform
+                    // accumulators 4 gi .. 4 gi + 3 of block b are d = 32 b + 8 gi + 4 hi + 0..3
                     h4_t o;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) o[j] = to_elem<BF16>(oacc[b][gi * 4 + j] * inv_l);
-                    *reinterpret_cast<h4_t *>(op + b * 32 + gi * 8 + hi * 4) = o;
+                    for (int j = 0; j < 4; ++j) o[j] = to_elem<BF16>(oacc[bb][gi * 4 + j] * inv_l);
+                    *reinterpret_cast<h4_t *>(op + (b_lo + bb) * 32 + gi * 8 + hi * 4) = o;
                 }
         }
         return;
     }
 
-    // The partition's state: the sums first, then - once those stores have completed - (m, l), whose arrival says so.
+    // The partition's state: a wave stores the sums of its blocks and then - once those stores have completed - (m, l), whose
+    // arrival says so. There is one copy of (m, l) per 32-dim block, because a merging wave reads one block of a column
+    // (8 float4 pieces) and its own copy of the pair: the copy of block b follows the sums of block b, whoever stored them.
+    static_assert(CG / 8 == DBLKS, "one copy of (m, l) per 32-dim block");
     const uint32_t ncols = a.ncols;
     const size_t grp_rows = ((size_t)kvh * S) * ncols;  // first (partition, column) row of this KV head
     const __amdgpu_buffer_rsrc_t rs_acc =
         __builtin_amdgcn_make_buffer_rsrc(a.part_acc + grp_rows * D, 0, (int)0xffffffffu, 0x00020000);
     const __amdgpu_buffer_rsrc_t rs_ml =
         __builtin_amdgcn_make_buffer_rsrc(a.part_ml + grp_rows * (2 * (CG / 8)), 0, (int)0xffffffffu, 0x00020000);
-    if (owner && q_row < a.q_len) {
+    if (active && q_row < a.q_len) {
         const uint32_t prow = split * ncols + pair * 32u + (uint32_t)n;
 #pragma unroll
-        for (int b = 0; b < DBLKS; ++b)
+        for (int bb = 0; bb < DBLKS; ++bb)
 #pragma unroll
             for (int gi = 0; gi < 4; ++gi) {
-                const f4_t v = {oacc[b][gi * 4], oacc[b][gi * 4 + 1], oacc[b][gi * 4 + 2], oacc[b][gi * 4 + 3]};
+                if (bb >= b_n) break;  // uniform
+                const f4_t v = {oacc[bb][gi * 4], oacc[bb][gi * 4 + 1], oacc[bb][gi * 4 + 2], oacc[bb][gi * 4 + 3]};
                 __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, v), rs_acc,
-                                                       (int)((prow * D + b * 32 + gi * 8 + hi * 4) * 4u), 0, ST_POLICY);
+                                                       (int)((prow * D + (b_lo + bb) * 32 + gi * 8 + hi * 4) * 4u), 0, ST_POLICY);
             }
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the sums are where the readers will look
@@ -496,12 +515,13 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
         if (hi == 0) {
             const u2_t mlv = {__float_as_uint(not_pattern(m_run)), __float_as_uint(not_pattern(l_tot))};
 #pragma unroll
-            for (int cp = 0; cp < CG / 8; ++cp)  // (a copy per merging wave: each consumes and clears its own)
-                __builtin_amdgcn_raw_buffer_store_b64(mlv, rs_ml, (int)((prow * (CG / 8) + cp) * 2u * 4u), 0, ST_POLICY);
+            for (int bb = 0; bb < DBLKS; ++bb) {
+                if (bb >= b_n) break;  // uniform
+                __builtin_amdgcn_raw_buffer_store_b64(mlv, rs_ml, (int)((prow * (CG / 8) + (uint32_t)(b_lo + bb)) * 2u * 4u), 0, ST_POLICY);
+            }
         }
     }
     FC_TR(7);
-    __syncthreads();  // every wave is done with the LDS it parked in: the merge below folds through it
     FC_TR(8);
 
     // Merge of this workgroup's columns: split, split + nsplits, ... A wave holds 8 float4 columns (c4) x 8 row lanes: lane
