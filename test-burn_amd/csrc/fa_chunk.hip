@@ -19,10 +19,11 @@
 // after 8K tokens: 26.0 us against 27.0 us for the tiled kernel and its merge launch). The host routes chunks of up to
 // 8 column blocks here by default.
 //
-// Merge: every workgroup stores its unnormalised state - acc [column][D] f32, then, once those stores have completed,
-// (m, l) per column into a buffer whose words hold an all-ones pattern between launches - and then merges ITS share of the
-// columns (column c belongs to workgroup c mod partitions): it polls the (m, l) pairs of all partitions of a column until
-// none is the pattern, reads the sums, folds them in partition order and writes the rows. When the workgroups of a KV
+// Merge: every workgroup stores its unnormalised state - acc [column][D] f32, then, once a wave's stores have completed,
+// (m, l) per column and 32-dim block into a buffer whose words hold an all-ones pattern between launches - and then merges
+// ITS share of the columns (column c belongs to workgroup c mod partitions): its waves poll the (m, l) pairs of all
+// partitions of a column until none is the pattern, read the sums, fold them (partitions in order within a lane, lanes by
+// exchanges within the wave) and write the rows. When the workgroups of a KV
 // head sit on one XCD the exchange goes through that XCD's L2 (plain stores, L2-scope loads), otherwise through
 // device-coherent accesses. Same residency assumption and the same bounded wait as the decode kernel's polled merge.
 #include "fa_internal.h"
