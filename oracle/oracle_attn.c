@@ -760,8 +760,9 @@ void orc_sage_k_mean(const orc_f16 *k, uint32_t n_kv_heads, uint32_t capacity, u
 static inline int8_t quant_i8(float x, float scale) {
     if (!(scale > 0.0f)) return 0;
     float r = nearbyintf(x / scale); /* round half to even, as the GPU's rint does */
-    if (r > 127.0f) r = 127.0f;
-    if (r < -127.0f) r = -127.0f;
+    /* clamp with maxNum / minNum, which pass over a NaN operand: a NaN quotient (a NaN key, or an infinite key over the
+     * infinite scale it makes) becomes -127 instead of an undefined conversion */
+    r = fminf(fmaxf(r, -127.0f), 127.0f);
     return (int8_t)r;
 }
 

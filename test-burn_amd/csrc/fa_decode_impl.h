@@ -1211,13 +1211,9 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
                 for (int j = 0; j < KSTEPS; ++j) {
-                    union {
-                        uint4 u;
-                        int8_t e[16];
-                    } o;
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) o.e[i] = (int8_t)sage_quant_i8_block(kx[sb][j][i], dv);
-                    kk[sb][j].u = o.u;
+                    const float *kv = kx[sb][j];
+                    kk[sb][j].u = make_uint4(sage_quant4_i8(kv[0], kv[1], kv[2], kv[3], dv), sage_quant4_i8(kv[4], kv[5], kv[6], kv[7], dv),
+                                             sage_quant4_i8(kv[8], kv[9], kv[10], kv[11], dv), sage_quant4_i8(kv[12], kv[13], kv[14], kv[15], dv));
                 }
             // the new V row into its place among the block's rows (load i holds rows i VRPL .. of a 16-row block)
             {

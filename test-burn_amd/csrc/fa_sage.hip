@@ -144,9 +144,7 @@ sage_quantize_k_kernel(const __half *k, const float *mean, uint32_t capacity, ui
         sg_u2_t o;
 #pragma unroll
         for (int w = 0; w < 2; ++w) {
-            const unsigned q0 = (unsigned)sage_quant_i8_block(x[i][4 * w], dv) & 0xffu, q1 = (unsigned)sage_quant_i8_block(x[i][4 * w + 1], dv) & 0xffu;
-            const unsigned q2 = (unsigned)sage_quant_i8_block(x[i][4 * w + 2], dv) & 0xffu, q3 = (unsigned)sage_quant_i8_block(x[i][4 * w + 3], dv) & 0xffu;
-            o[w] = q0 | (q1 << 8) | (q2 << 16) | (q3 << 24);
+            o[w] = sage_quant4_i8(x[i][4 * w], x[i][4 * w + 1], x[i][4 * w + 2], x[i][4 * w + 3], dv);
         }
         *reinterpret_cast<sg_u2_t *>(dst + (size_t)row * D) = o;
     }
@@ -260,13 +258,9 @@ __global__ void __launch_bounds__(256) sage_append_kernel(SageAppendDev a) {
         for (int it = 0; it < 2; ++it) {
             const uint32_t item = tid + it * 256, j = item / cpr, ch = item % cpr;
             if (j <= r) {
-                union {
-                    uint2 u;
-                    int8_t b[8];
-                } o;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) o.b[i] = (int8_t)sage_quant_i8_block(x[it][i], dv);
-                *reinterpret_cast<uint2 *>(a.k_q + ((size_t)h * a.capacity + b0 + j) * D + ch * 8) = o.u;
+                const uint2 o = make_uint2(sage_quant4_i8(x[it][0], x[it][1], x[it][2], x[it][3], dv),
+                                           sage_quant4_i8(x[it][4], x[it][5], x[it][6], x[it][7], dv));
+                *reinterpret_cast<uint2 *>(a.k_q + ((size_t)h * a.capacity + b0 + j) * D + ch * 8) = o;
             }
         }
     } else {

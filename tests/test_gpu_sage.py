@@ -87,6 +87,40 @@ def test_sage_incremental_block_quantisation_and_errors():
     f.synchronize()
 
 
+def test_sage_quantiser_special_blocks_match_the_oracle_bit_for_bit():
+    """The quantiser divides a block by its one scale through a shared reciprocal, which holds for a finite positive
+    scale; other blocks take the plain division. Blocks of every kind against the oracle: all rows equal to the mean
+    (scale 0), one infinity (scale infinite: finite values quantise to 0, the infinity - a NaN quotient - to -127, which is
+    what a clamp with maxNum / minNum makes of a NaN), one NaN (ignored by the block's maximum, -127 itself), tiny values (a scale that is a subnormal f16), the largest f16 values, and
+    values exactly half way between two steps of the grid."""
+    announce("sage quantiser special blocks")
+    f = ctx()
+    rng = np.random.default_rng(7)
+    Hkv, D, cap = 2, 128, 32 * 8
+    k = h16(rng.normal(size=(Hkv, cap, D)))
+    k[:, 0:32] = 0                                       # block 0: zeros (the mean below is zero, too)
+    k[:, 40, 5] = np.float16(np.inf)                     # block 1: an infinity
+    k[:, 70, 9] = np.float16(np.nan)                     # block 2: a NaN
+    k[:, 96:128] = h16(rng.normal(size=(Hkv, 32, D)) * 1e-7)   # block 3: subnormal-scale values
+    k[:, 128:160] = h16(rng.uniform(-65504, 65504, size=(Hkv, 32, D)))  # block 4: the f16 range
+    half = (np.arange(D) % 255 - 127).astype(np.float32) + 0.5          # block 5: k / scale = n + 1/2 with scale 1: max |k| = 127
+    k[:, 160:192] = h16(np.clip(half, -126.5, 126.5))[None, None, :]
+    k[:, 160, 0] = np.float16(127.0)
+    mean = np.zeros((Hkv, D), np.float32)
+    dk, dmean = f.array(k), f.array(mean)
+    dkq, dks = f.zeros((Hkv, cap, D), np.int8), f.zeros((Hkv, cap // 32), np.float16)
+    f.sage_quantize_k(dk, dmean, Hkv, cap, D, 0, cap, dkq, dks)
+    f.synchronize()
+    with np.errstate(all="ignore"):
+        want_kq, want_ks = orc.sage_quantize_k(k, mean, Hkv, cap, D, cap)
+    got_q, got_s = dkq.download(), dks.download()
+    assert np.array_equal(bits(got_s), bits(want_ks))
+    assert np.array_equal(got_q, want_kq)
+    assert not got_q[:, 0:32].any() and got_q[0, 40, 5] == -127 and got_q[0, 41, 5] == 0 and got_q[0, 70, 9] == -127
+    for b in (dk, dmean, dkq, dks):
+        b.free()
+
+
 @pytest.mark.parametrize("launches", [1, 2], ids=["one_launch", "two_launches"])
 @pytest.mark.parametrize("H,Hkv,D,start,cap,steps,mode,layer,nope_step,dyn", [
     (16, 4, 128, 90, 256, 40, fa.ROPE_NEOX, 0, 0, False),    # crosses the block boundaries at 96 and 128
