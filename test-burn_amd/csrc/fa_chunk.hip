@@ -125,8 +125,14 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
     constexpr int CG = D / 4;            // float4 columns per row
     constexpr int ST_POLICY = LOCAL ? 0 : COHERENT, LD_POLICY = LOCAL ? L2_SCOPE : COHERENT;
     typedef __attribute__((address_space(3))) void *lds_ptr;
-    // NBLK 16-row blocks of K, then of V: a ring of RING rounds
-    __shared__ __attribute__((aligned(1024))) unsigned char lds[NBLK * (RB_BYTES + 4 * RG_BYTES)];
+    // NBLK 16-row blocks of K, then of V: a ring of RING rounds. After the tiles the same bytes hold what the two waves
+    // of a column block park for each other (PARK_BYTES) and, behind that, a region per wave in which the sums are turned
+    // from the accumulator layout into rows (TP_WAVE bytes each: 32 rows x the wave's share of the head dimension).
+    constexpr int PARK_BYTES = 2 * 256 * 8 + 2 * (DBLKS / 2) * 4 * 256 * 16, TP_WAVE = 32 * (D / 2) * 4;
+    constexpr int RING_BYTES = NBLK * (RB_BYTES + 4 * RG_BYTES);
+    constexpr int LDS_BYTES = RING_BYTES > PARK_BYTES + 8 * TP_WAVE ? RING_BYTES : PARK_BYTES + 8 * TP_WAVE;
+    static_assert(8 * 2 * TP_WAVE <= LDS_BYTES, "without parking, a wave's region is twice as large and starts at 0");
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[LDS_BYTES];
     unsigned char *k_area = lds, *v_area = lds + NBLK * RB_BYTES;
     const uint32_t k_lds_addr = (uint32_t)(uintptr_t)(lds_ptr)lds, v_lds_addr = k_lds_addr + NBLK * RB_BYTES;
 
@@ -499,17 +505,41 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
         __builtin_amdgcn_make_buffer_rsrc(a.part_acc + grp_rows * D, 0, (int)0xffffffffu, 0x00020000);
     const __amdgpu_buffer_rsrc_t rs_ml =
         __builtin_amdgcn_make_buffer_rsrc(a.part_ml + grp_rows * (2 * (CG / 8)), 0, (int)0xffffffffu, 0x00020000);
-    if (active && q_row < a.q_len) {
-        const uint32_t prow = split * ncols + pair * 32u + (uint32_t)n;
+    if (active) {
+        // A lane holds 16-byte pieces of ONE row: stored as they are, an instruction would touch 64 cache lines, 32 bytes of
+        // each. So the wave's rows go through LDS - a region of its own, LDS runs a wave's
+        // accesses in order: no barrier -, 16-byte chunks exchanged by row number against bank conflicts, and leave as whole
+        // 128-byte lines, 8 lanes per line.
+        unsigned char *tp = lds + (halves ? PARK_BYTES + wave8 * TP_WAVE : wave8 * 2 * TP_WAVE);
+        const int row_bytes = b_n * 128, xm = (b_n * 8 - 1) & 15;  // (a row holds 8 b_n chunks: the exchange stays inside it)
 #pragma unroll
         for (int bb = 0; bb < DBLKS; ++bb)
 #pragma unroll
             for (int gi = 0; gi < 4; ++gi) {
                 if (bb >= b_n) break;  // uniform
                 const f4_t v = {oacc[bb][gi * 4], oacc[bb][gi * 4 + 1], oacc[bb][gi * 4 + 2], oacc[bb][gi * 4 + 3]};
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, v), rs_acc,
-                                                       (int)((prow * D + (b_lo + bb) * 32 + gi * 8 + hi * 4) * 4u), 0, ST_POLICY);
+                const int chunk = bb * 8 + gi * 2 + hi;  // accumulators 4 gi .. + 3 of block bb are dims 32 bb + 8 gi + 4 hi ..
+                *reinterpret_cast<f4_t *>(tp + n * row_bytes + ((chunk ^ (n & xm)) * 16)) = v;
             }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront", "local");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront", "local");
+        const uint32_t prow0 = split * ncols + pair * 32u;
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            const int row = it * 8 + (lane >> 3), piece = lane & 7;
+#pragma unroll
+            for (int bb = 0; bb < DBLKS; ++bb) {
+                if (bb >= b_n) break;  // uniform
+                const f4_t v = *reinterpret_cast<const f4_t *>(tp + row * row_bytes + (((bb * 8 + piece) ^ (row & xm)) * 16));
+                if (rb * 32u + (uint32_t)row < a.q_len)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, v), rs_acc,
+                                                           (int)(((prow0 + (uint32_t)row) * D + (b_lo + bb) * 32 + piece * 4) * 4u), 0, ST_POLICY);
+            }
+        }
+    }
+    if (active && q_row < a.q_len) {
+        const uint32_t prow = split * ncols + pair * 32u + (uint32_t)n;
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the sums are where the readers will look
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
