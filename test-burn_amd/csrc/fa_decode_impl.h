@@ -566,6 +566,16 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // and in a ragged batch the low partitions always exist while the high ones are mostly empty: some XCDs queue
     // work while others idle (measured: 62 us with 12 partitions per sequence, 55 us with 11). Rotating the index
     // by the head-group index spreads every sequence's partitions over all XCDs.
+    // The f16 fused step in 8-wave workgroups starts without the barrier that holds the streaming waves until wave 0 has
+    // queued its requests (below): its streaming waves spend a microsecond at their own requests anyway, and wave 0's few
+    // get in among their first ones (measured at 8K context: 10.58 -> 10.48 us per launch; the 4-wave workgroups of the small
+    // launches lose by it - 6.0 -> 6.1 us at 1K context, 6.6 -> 7.0 us at 512 - and keep the barrier). The operand counter is
+    // then cleared here, behind a barrier that costs the waves' entry skew only.
+    constexpr bool EARLY_START = FUSED && !SAGE && NW == 8;
+    if constexpr (EARLY_START) {
+        if (tid == 0) sm_q_ready = 0;
+        __syncthreads();
+    }
     uint32_t y = blockIdx.y, b = blockIdx.z;
     uint32_t split = (blockIdx.x + y + gridDim.y * b) % gridDim.x;
     if (a.xcd_local) {
@@ -918,9 +928,11 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                 kk[1][j].u = *reinterpret_cast<const uint4 *>(krow + (4 * j + c) * 8);
             }
             vv[1][0].u = *reinterpret_cast<const uint4 *>(vrow_in + (lane % VLPR) * 8);
-            if (lane == 0) sm_q_ready = 0;
-            __builtin_amdgcn_sched_barrier(0);
-            __syncthreads();  // releases the streaming waves
+            if constexpr (!EARLY_START) {
+                if (lane == 0) sm_q_ready = 0;
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();  // releases the streaming waves
+            }
             __builtin_amdgcn_sched_barrier(0);
             FA_TR(1);
             n_raw = read_len();
@@ -974,7 +986,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             __builtin_amdgcn_s_setprio(0);
             FA_TR(2);
         } else {
-            __syncthreads();  // wave 0 has queued its requests
+            if constexpr (!EARLY_START) __syncthreads();  // wave 0 has queued its requests
             FA_TR(1);
         }
     } else {
