@@ -711,6 +711,14 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // (a barrier holds them until then), rotates, and publishes the MFMA operand through LDS while the blocks
     // are in flight. A contiguous cache is allocated up to `capacity`, so the blocks can be requested before the
     // length is known; a paged cache needs the length to stay inside its block table.
+    // With the early start the streaming waves' first requests come here, ahead of wave 0's preparation in the program
+    // as well: they used to sit behind it, a jump of several KB into instructions nobody had fetched yet.
+    if (EARLY_START && !PAGED && cur < wb1) {
+        const uint32_t m = min((uint32_t)MBX, wb1 - cur);
+        issue_k(cur, m, 0);
+        issue_v(cur, m, 0);
+        FA_TR(2);
+    }
     const bool rope_normal = a.rope_normal != 0, rope_on = a.apply_rope != 0;
     const bool head_ok = (uint32_t)n < gt;
     // Q^T operand [KSTEPS][64], shared by the workgroup through LDS: reading it per MFMA step instead of holding
@@ -1000,7 +1008,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         }
         if (SAGE && head_ok) qsc = a.q_scale[head0 + n] * a.scale_log2e;
     }
-    if (!PAGED && cur < wb1) {
+    if (!EARLY_START && !PAGED && cur < wb1) {
         const uint32_t m = min((uint32_t)MBX, wb1 - cur);
         issue_k(cur, m, 0);
         issue_v(cur, m, 0);
