@@ -569,7 +569,8 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // The f16 fused step in 8-wave workgroups starts without the barrier that holds the streaming waves until wave 0 has
     // queued its requests (below): its streaming waves spend a microsecond at their own requests anyway, and wave 0's few
     // get in among their first ones (measured at 8K context: 10.58 -> 10.48 us per launch; the 4-wave workgroups of the small
-    // launches lose by it - 6.0 -> 6.1 us at 1K context, 6.6 -> 7.0 us at 512 - and keep the barrier). The operand counter is
+    // launches lose by it - 6.0 -> 6.1 us at 1K context, 6.6 -> 7.0 us at 512 - and keep the barrier, and so does the int8
+    // step, whose wave 0 has four times the requests: 15.8 -> 16.9 us at 32K context). The operand counter is
     // then cleared here, behind a barrier that costs the waves' entry skew only.
     constexpr bool EARLY_START = FUSED && !SAGE && NW == 8;
     if constexpr (EARLY_START) {
