@@ -513,7 +513,12 @@ __device__ __forceinline__ U4H rope8(const U4H &x, const U4H &mate, const U4H &c
 }
 
 template <int D, bool PAGED, bool SAGE, bool FUSED, bool BF16 = false>
-__global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(DecodeDev a) {
+__global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(DecodeDev a_by_value) {
+    // The arguments are read where the program needs them, straight from the launch's argument block (the struct is its
+    // first and only member): a by-value struct is copied field by field at the kernel's entry, which puts every field
+    // the kernel ever uses - four dozen scalar registers, half of them spilled at once - ahead of the first request.
+    const DecodeDev &a = *(const DecodeDev *)__builtin_amdgcn_kernarg_segment_ptr();
+    (void)a_by_value;
     constexpr int KSTEPS = SAGE ? D / 64 : D / 32;  // MFMA steps over head_dim for S^T; 16 B per lane each
     constexpr int SEGS = SAGE ? D / 16 : D / 8;     // 16-byte segments per K row
     constexpr int VLB = D / 32;                     // 1 KiB V loads per block
@@ -573,6 +578,12 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // step, whose wave 0 has four times the requests: 15.8 -> 16.9 us at 32K context). The operand counter is
     // then cleared here, behind a barrier that costs the waves' entry skew only.
     constexpr bool EARLY_START = FUSED && !SAGE && NW == 8;
+    if constexpr (!PAGED) {
+        // ... and those on the way to the first request in ONE trip through the scalar cache, not one trip per use.
+        asm volatile("" ::"s"(a.k), "s"(a.v), "s"(a.k_stride_b), "s"(a.k_stride_h), "s"(a.v_stride_b), "s"(a.v_stride_h),
+                     "s"(a.capacity), "s"(a.chunk), "s"(a.sub_per_kv), "s"(a.gt), "s"(a.xcd_local), "s"(a.rcp_gx),
+                     "s"(a.rcp_gy), "s"(gridDim.x), "s"(gridDim.y));
+    }
     if constexpr (EARLY_START) {
         if (tid == 0) sm_q_ready = 0;
         __syncthreads();
