@@ -75,6 +75,8 @@ struct ChunkDev {
                         // column; every word 0xffffffff between launches
     float scale_log2e;
     uint32_t xcd_local;            // the workgroups of a KV head share an XCD: partials meet in its L2
+    uint32_t rcp_gx, rcp_gy;       // xcd_local: floor(2^32 / d) + 1 for the grid's x and y dimensions (0 for d = 1): exact
+                                   // quotients of numbers below 2^16
     unsigned long long poll_ticks; // bound of a merging thread's wait for the other partitions, 100 MHz ticks
     uint32_t *status;              // the context's device-written status words
 #ifdef FA_DECODE_TRACE
@@ -114,7 +116,14 @@ __device__ __forceinline__ void merge_in(MergeState &s, bool counts, float m_p, 
 }
 
 template <int D, bool BF16, bool PAGED, bool LOCAL>
-__global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
+__global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a_by_value) {
+    // The arguments are read where the program needs them, straight from the launch's argument block (the struct is its
+    // only member): a by-value struct is copied field by field at the kernel's entry, every field the kernel ever uses
+    // ahead of the first request. Those that the first request does need come in one trip through the scalar cache.
+    const ChunkDev &a = *(const ChunkDev *)__builtin_amdgcn_kernarg_segment_ptr();
+    (void)a_by_value;
+    asm volatile("" ::"s"(a.k), "s"(a.v), "s"(a.k_stride_h), "s"(a.v_stride_h), "s"(a.part_len), "s"(a.kv_end), "s"(a.nsplits),
+                 "s"(a.rcp_gx), "s"(a.rcp_gy), "s"(a.poll_ticks), "s"(gridDim.x), "s"(gridDim.y));
     constexpr int DSTEPS = D / 16;  // MFMA k-steps over head_dim for S^T
     constexpr int DBLKS = D / 32;   // 32-row blocks of O^T
     constexpr int ROWB = D * 2, CHK = D / 8;
@@ -168,8 +177,13 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
         // so that their partial states meet in that XCD's L2: group = id % 8 + 8 (id / 8 / S), partition = id / 8 % S.
         // The host selects this only when the number of groups is a multiple of 8.
         const uint32_t lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z), slot = lin >> 3;
-        const uint32_t g = (lin & 7u) + 8u * (slot / gridDim.x);
-        split = slot % gridDim.x, kvh = g % gridDim.y, cgrp = g / gridDim.y;
+        // (The quotients are products with reciprocals from the host: a division is two dozen dependent instructions,
+        // four of them 0.4 us in which the workgroup does not yet know what to ask for.)
+        const uint32_t sq = a.rcp_gx ? __umulhi(slot, a.rcp_gx) : slot;
+        const uint32_t g = (lin & 7u) + 8u * sq;
+        split = slot - sq * gridDim.x;
+        cgrp = a.rcp_gy ? __umulhi(g, a.rcp_gy) : g;
+        kvh = g - cgrp * gridDim.y;
     }
     // keys anyone in the chunk can see, and this workgroup's partition of them
     const uint32_t kv_end = a.kv_end, nsplits = a.nsplits;
@@ -196,14 +210,14 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
     // is not valid, the next stream wait reports it).
     __shared__ uint32_t ring_count[2][RING];  // landed, freed
     if (tid < 2 * RING) ring_count[tid / RING][tid % RING] = 0u;
-    const unsigned long long t_ring = wall_clock64();
+    const unsigned long long t_ring = wall_clock64(), poll_ticks = a.poll_ticks;
     bool gave_up = false;
     // (which: 0 landed, 1 freed) of round r's slot: has everybody on that side done round r?
     auto wait_count = [&](int which, int r, uint32_t per_round) __attribute__((always_inline)) {
         const uint32_t target = per_round * (uint32_t)(r / RING + 1);
         while (!gave_up && __hip_atomic_load(&ring_count[which][r % RING], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < target) {
             __builtin_amdgcn_s_sleep(1);
-            if (wall_clock64() - t_ring > a.poll_ticks) {
+            if (wall_clock64() - t_ring > poll_ticks) {
                 gave_up = true;
                 if (lane == 0 && a.status) a.status[FA_DEVSTAT_MERGE_TIMEOUT] = 1u;
             }
@@ -298,6 +312,9 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
         return;  // (a wave that has ended no longer counts at the workgroup's barriers)
     }
 
+    // (read once: the waits and fences of the loops below would have each use fetch them again)
+    const bool causal = a.causal != 0;
+    const uint32_t q_len = a.q_len;
     const uint32_t G = a.group_size;
     // this workgroup's column blocks: pairs [8 cgrp, 8 cgrp + pairs_here); wave -> (column block, tile parity)
     const uint32_t pairs_here = min(8u, a.pairs - cgrp * 8u);
@@ -308,7 +325,7 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
     const uint32_t pair = cgrp * 8u + (active ? cb : 0u);
     const uint32_t head = kvh * G + pair % G, rb = pair / G;
     const uint32_t q_row = rb * 32u + (uint32_t)n;  // the query row this lane's column belongs to
-    const uint32_t q_row_c = min(q_row, a.q_len - 1);
+    const uint32_t q_row_c = min(q_row, q_len - 1);
     // ---- The 8 waves that attend. Q^T operand: lane (n, hi) keeps Q[q_row][16 s + 8 hi .. +8] for every k-step s.
     U4H8 qreg[DSTEPS];
     {
@@ -327,7 +344,7 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
     const float c = a.scale_log2e;
     const uint32_t q_abs = q_row_c + a.query_offset;  // last visible key of this lane's row when causal
     // first key index that some row of this wave cannot see
-    const uint32_t wave_min_limit = a.causal ? (min(rb * 32u, a.q_len - 1) + a.query_offset) : 0xffffffffu;
+    const uint32_t wave_min_limit = causal ? (min(rb * 32u, q_len - 1) + a.query_offset) : 0xffffffffu;
     const int k_lane = (n >> 4) * RB_BYTES + hi * 256 + (n & 15) * 16;
     const int v_lane = hi * RG_BYTES + ((lane & 15) >> 2) * 64 + ((lane >> 4) & 1) * 32 + (lane & 3) * 8;
 
@@ -350,7 +367,7 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const uint32_t key = key0 + (i / 4) * 8 + hi * 4 + (i % 4);
-                const bool vis = key < k_hi && (!a.causal || key <= q_abs);
+                const bool vis = key < k_hi && (!causal || key <= q_abs);
                 sacc[i] = vis ? sacc[i] : -INFINITY;
             }
         }
@@ -477,7 +494,7 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
     const float l_tot = l_run + __shfl_xor(l_run, 32);
 
     if (nsplits == 1) {  // finalise, flash_prefill.metal:255-261
-        if (active && q_row < a.q_len) {
+        if (active && q_row < q_len) {
             const float inv_l = (isfinite(l_tot) && fabsf(l_tot) > 1e-6f) ? (1.0f / l_tot) : 0.0f;
             __half *op = a.out + (size_t)head * a.out_stride_h + (size_t)q_row * a.out_stride_m;
 #pragma unroll
@@ -532,13 +549,13 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
             for (int bb = 0; bb < DBLKS; ++bb) {
                 if (bb >= b_n) break;  // uniform
                 const f4_t v = *reinterpret_cast<const f4_t *>(tp + row * row_bytes + (((bb * 8 + piece) ^ (row & xm)) * 16));
-                if (rb * 32u + (uint32_t)row < a.q_len)
+                if (rb * 32u + (uint32_t)row < q_len)
                     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, v), rs_acc,
                                                            (int)(((prow0 + (uint32_t)row) * D + (b_lo + bb) * 32 + piece * 4) * 4u), 0, ST_POLICY);
             }
         }
     }
-    if (active && q_row < a.q_len) {
+    if (active && q_row < q_len) {
         const uint32_t prow = split * ncols + pair * 32u + (uint32_t)n;
         __atomic_signal_fence(__ATOMIC_SEQ_CST);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the sums are where the readers will look
@@ -577,7 +594,7 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
         const uint32_t col = col0 + split + (j0 + jl) * nsplits;
         // column -> (pair, row in block) -> (head, query row)
         const uint32_t cpair = col / 32u, crow = (cpair / G) * 32u + col % 32u, chead = kvh * G + cpair % G;
-        const bool mine = j0 + jl < nmy && col < col0 + gcols && crow < a.q_len;
+        const bool mine = j0 + jl < nmy && col < col0 + gcols && crow < q_len;
         MergeState st = {-1e30f, 0.0f, {0.0f, 0.0f, 0.0f, 0.0f}};
         // Every load of a batch is issued whether its lane wants it or not (an unwanted one reads row 0): a load inside a
         // branch makes the compiler wait for all earlier ones first, and the batch would take one round trip per partition.
@@ -606,7 +623,7 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a) {
                     pend &= fresh ? ~(1u << kk) : ~0u;
                 }
                 if (!__any(pend != 0)) break;
-                if (wall_clock64() - t_begin > a.poll_ticks) {
+                if (wall_clock64() - t_begin > poll_ticks) {
                     timed_out = true;
                     break;
                 }
@@ -724,6 +741,9 @@ fa_status fa_launch_prefill_chunk(fa_ctx *ctx, const PrefillLaunch &L, bool forc
         a.part_acc = (float *)ctx->workspace;
         a.part_ml = (float *)ctx->poll_ws;  // all-ones between launches; the mergers put the pattern back
         a.xcd_local = ctx->xcd_round_robin && groups % 8 == 0 ? 1u : 0u;
+        // (a launch has at most one workgroup per compute unit, so every number divided in the kernel is far below 2^16)
+        a.rcp_gx = S > 1 ? (uint32_t)((1ull << 32) / S) + 1u : 0u;
+        a.rcp_gy = L.n_kv_heads > 1 ? (uint32_t)((1ull << 32) / L.n_kv_heads) + 1u : 0u;
     }
     dim3 grid(S, L.n_kv_heads, cgroups);
     FaLaunchScope scope(ctx, "flash_chunk_kernel", true);

@@ -206,6 +206,10 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
         mode = L.paged ? MODE_FUSED_PAGED : MODE_FUSED;
     else if (L.paged)
         mode = MODE_PAGED;
+    {   // (divisions that every wave would otherwise do before its first request)
+        const uint32_t streaming = (mode == MODE_FUSED || mode == MODE_FUSED_PAGED || mode == MODE_SAGE_FUSED) ? waves - 1 : waves;
+        a.nb_q = (chunk / BK) / streaming, a.nb_r = (chunk / BK) % streaming;
+    }
     dim3 grid(S, ny_grid, L.batch);
     if (a.xcd_local) {
         // the kernel's reciprocals (see there): every workgroup index and both divisors stay below 2^16

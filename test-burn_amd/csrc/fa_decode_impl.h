@@ -582,14 +582,18 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         // ... and those on the way to the first request in ONE trip through the scalar cache, not one trip per use.
         asm volatile("" ::"s"(a.k), "s"(a.v), "s"(a.k_stride_b), "s"(a.k_stride_h), "s"(a.v_stride_b), "s"(a.v_stride_h),
                      "s"(a.capacity), "s"(a.chunk), "s"(a.sub_per_kv), "s"(a.gt), "s"(a.xcd_local), "s"(a.rcp_gx),
-                     "s"(a.rcp_gy), "s"(gridDim.x), "s"(gridDim.y));
+                     "s"(a.rcp_gy), "s"(a.nb_q), "s"(a.nb_r), "s"(gridDim.x), "s"(gridDim.y));
+        // (In the 4-wave form also what reading the length takes, one more trip later instead of three: 6.28 -> 6.24 us
+        // per launch at 512 tokens of context. The 8-wave form loses by it, 10.12 -> 10.19 us at 8K.)
+        if constexpr (NW == 4)
+            asm volatile("" ::"s"(a.d_len), "s"(a.d_len_stride), "s"(a.kv_len_add), "s"(a.kv_len), "s"(a.kv_len_bound));
     }
     if constexpr (EARLY_START) {
         if (tid == 0) sm_q_ready = 0;
         __syncthreads();
     }
     uint32_t y = blockIdx.y, b = blockIdx.z;
-    uint32_t split = (blockIdx.x + y + gridDim.y * b) % gridDim.x;
+    uint32_t split;
     if (a.xcd_local) {
         // All partitions of a head group on ONE XCD (workgroup id modulo 8), so that their partial states meet in that
         // XCD's L2 instead of in memory: group = id % 8 + 8 (id / 8 / S), partition = id / 8 % S. The host selects this
@@ -603,6 +607,11 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         split = slot - sq * gridDim.x;
         b = __umulhi(g, a.rcp_gy);                     // g / gridDim.y
         y = g - b * gridDim.y;
+    } else {
+        // (the empty statement keeps the compiler from working the remainder out ahead of the branch, for both forms)
+        uint32_t d = gridDim.x;
+        asm volatile("" : "+s"(d));
+        split = (blockIdx.x + y + gridDim.y * b) % d;
     }
     // A head group that only pads the grid (see the host): its workgroups address the last real group's rows, so that
     // nothing they request before they leave - with the workgroups of empty partitions, below - is out of range. (Leaving
@@ -710,9 +719,11 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // FUSED, wave 0 streams no blocks: it prepares the query operand and attends the new token.
     constexpr int KW = FUSED ? NW - 1 : NW;  // streaming waves
     const int sw = FUSED ? wave - 1 : wave;  // index among them (-1: none)
+    // (A contiguous cache's partitions are the host's, and so is the division: nb_q blocks each, one more for the first
+    // nb_r waves. A paged launch sizes its partitions below, once it knows the length.)
     uint32_t nb = chunk / BK;
-    uint32_t wb0 = sw >= 0 ? nb - ((uint32_t)(KW - sw) * nb) / KW : 0u;
-    uint32_t wb1 = sw >= 0 ? nb - ((uint32_t)(KW - 1 - sw) * nb) / KW : 0u;
+    uint32_t wb0 = sw >= 0 ? (uint32_t)sw * a.nb_q + min((uint32_t)sw, a.nb_r) : 0u;
+    uint32_t wb1 = sw >= 0 ? wb0 + a.nb_q + ((uint32_t)sw < a.nb_r ? 1u : 0u) : 0u;
     uint32_t cur = wb0;
 
     // A CU accepts vector memory requests in order and only as fast as its earlier ones complete, so anything
@@ -1068,6 +1079,12 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         issue_v(cur, m, k1 - 1);
         if (cur + m < wbe) load_pages(cur + m, min((uint32_t)MBX, wbe - (cur + m)), pgn);
     }
+    // The arguments of the fold and the merge, as a copy of their own made here, in one trip, while the wave waits for
+    // its first rows anyway: read where they are used they cost the end of the launch a trip each, eight or so in a row.
+    const DecodeDev tl = a;
+    const uint32_t GY = gridDim.y;
+    asm volatile("" ::"s"(tl.merge_in_kernel), "s"(tl.part_acc), "s"(tl.part_ml), "s"(tl.counters), "s"(tl.out), "s"(tl.out_stride_b),
+                 "s"(tl.out_stride_h), "s"(tl.bf16), "s"(tl.status), "s"(tl.poll_ticks), "s"(tl.xcd_local), "s"(GY));
     {   // the Q^T operand is in LDS once every contributing wave has counted itself in
         constexpr uint32_t Q_PARTS = FUSED ? 1u : (uint32_t)(KSTEPS < NW ? KSTEPS : NW);
         while (__hip_atomic_load(&sm_q_ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < Q_PARTS) __builtin_amdgcn_s_sleep(1);
@@ -1326,8 +1343,8 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     __syncthreads();
     FA_TR(8);
 
-    const bool in_kernel = a.merge_in_kernel != 0, polled = a.merge_in_kernel == 2;
-    const size_t gbase = ((size_t)b * gridDim.y + y) * S * gt;  // first row of this (sequence, head group)
+    const bool in_kernel = tl.merge_in_kernel != 0, polled = tl.merge_in_kernel == 2;
+    const size_t gbase = ((size_t)b * GY + y) * S * gt;  // first row of this (sequence, head group)
     const uint32_t prow = split * gt;
     constexpr int CG = D / 4;
     // LPC = NW / 2 consecutive lanes share a column (head h, float4 column c4): lane j merges the states of waves 2j and
@@ -1352,7 +1369,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         if (!valid || wsel != 0) continue;
         if (nsplits == 1) {
             const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 1.0f;
-            __half *op = a.out + (size_t)b * a.out_stride_b + (size_t)(head0 + h) * a.out_stride_h + c4 * 4;
+            __half *op = tl.out + (size_t)b * tl.out_stride_b + (size_t)(head0 + h) * tl.out_stride_h + c4 * 4;
             const float ov[4] = {A[0] * inv, A[1] * inv, A[2] * inv, A[3] * inv};
             store_out4(op, ov, BF16);
         } else if (polled) {
@@ -1360,9 +1377,9 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             const u4_t r0 = {__float_as_uint(not_sentinel(A[0])), __float_as_uint(not_sentinel(A[1])),
                              __float_as_uint(not_sentinel(A[2])), __float_as_uint(not_sentinel(A[3]))};
             const u2_t r1 = {__float_as_uint(not_sentinel(ms)), __float_as_uint(not_sentinel(L))};
-            const __amdgpu_buffer_rsrc_t rs = make_rsrc(a.part_acc + ((size_t)b * gridDim.y + y) * S * (gt * CG) * 8);
+            const __amdgpu_buffer_rsrc_t rs = make_rsrc(tl.part_acc + ((size_t)b * GY + y) * S * (gt * CG) * 8);
             const uint32_t ro = (split * (gt * CG) + (uint32_t)idx) * 32u;
-            if (a.xcd_local) {
+            if (tl.xcd_local) {
                 __builtin_amdgcn_raw_buffer_store_b128(r0, rs, (int)ro, 0, 0);
                 __builtin_amdgcn_raw_buffer_store_b64(r1, rs, (int)ro + 16, 0, 0);
             } else {
@@ -1370,7 +1387,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                 __builtin_amdgcn_raw_buffer_store_b64(r1, rs, (int)ro + 16, 0, CACHE_COHERENT);
             }
         } else if (in_kernel) {
-            float *pa = a.part_acc + gbase * D, *pm = a.part_ml + gbase * 2;
+            float *pa = tl.part_acc + gbase * D, *pm = tl.part_ml + gbase * 2;
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u4_t, A), make_rsrc(pa),
                                                    (int)(((prow + h) * D + c4 * 4) * 4u), 0, CACHE_COHERENT);
             if (c4 == 0) {
@@ -1379,8 +1396,8 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
                                                       (int)((prow + h) * 2 * 4u), 0, CACHE_COHERENT);
             }
         } else {
-            *reinterpret_cast<f4_t *>(a.part_acc + (gbase + prow + h) * D + c4 * 4) = A;
-            if (c4 == 0) a.part_ml[(gbase + prow + h) * 2] = ms, a.part_ml[(gbase + prow + h) * 2 + 1] = L;
+            *reinterpret_cast<f4_t *>(tl.part_acc + (gbase + prow + h) * D + c4 * 4) = A;
+            if (c4 == 0) tl.part_ml[(gbase + prow + h) * 2] = ms, tl.part_ml[(gbase + prow + h) * 2 + 1] = L;
         }
     }
     FA_TR(9);
@@ -1391,20 +1408,20 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     if (polled) {
         bool ok;
         if (nsplits <= 64) {
-            ok = a.xcd_local ? coop_merge_in_registers<D, true>(a, b, y, split, nsplits, S, tid)
-                             : coop_merge_in_registers<D, false>(a, b, y, split, nsplits, S, tid);
-            if (!ok && lane == 0 && a.status) a.status[FA_DEVSTAT_MERGE_TIMEOUT] = 1u;
+            ok = tl.xcd_local ? coop_merge_in_registers<D, true>(tl, b, y, split, nsplits, S, tid)
+                             : coop_merge_in_registers<D, false>(tl, b, y, split, nsplits, S, tid);
+            if (!ok && lane == 0 && tl.status) tl.status[FA_DEVSTAT_MERGE_TIMEOUT] = 1u;
             FA_TR(10);
             FA_TR_FLUSH();
             return;
         }
         __syncthreads();  // the fold above read the LDS region that the merge reuses
-        if (a.xcd_local) {
-            ok = coop_merge_and_store<D, true>(a, b, y, split, nsplits, S, tid, reinterpret_cast<float *>(smem));
+        if (tl.xcd_local) {
+            ok = coop_merge_and_store<D, true>(tl, b, y, split, nsplits, S, tid, reinterpret_cast<float *>(smem));
         } else {
-            ok = coop_merge_and_store<D, false>(a, b, y, split, nsplits, S, tid, reinterpret_cast<float *>(smem));
+            ok = coop_merge_and_store<D, false>(tl, b, y, split, nsplits, S, tid, reinterpret_cast<float *>(smem));
         }
-        if (!ok && tid == 0 && a.status) a.status[FA_DEVSTAT_MERGE_TIMEOUT] = 1u;
+        if (!ok && tid == 0 && tl.status) tl.status[FA_DEVSTAT_MERGE_TIMEOUT] = 1u;
         return;
     }
 
@@ -1416,15 +1433,15 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     __atomic_signal_fence(__ATOMIC_SEQ_CST);
     __syncthreads();
     if (tid == 0) {
-        const uint32_t ticket = __hip_atomic_fetch_add(&a.counters[(size_t)b * gridDim.y + y], 1u, __ATOMIC_RELAXED,
+        const uint32_t ticket = __hip_atomic_fetch_add(&tl.counters[(size_t)b * GY + y], 1u, __ATOMIC_RELAXED,
                                                        __HIP_MEMORY_SCOPE_AGENT);
         sm_last = (ticket == nsplits - 1) ? 1u : 0u;
     }
     __syncthreads();
     if (!sm_last) return;
-    merge_and_store<D, true, NT>(a, b, y, nsplits, S, tid, reinterpret_cast<float *>(smem), 0, (int)gt);
+    merge_and_store<D, true, NT>(tl, b, y, nsplits, S, tid, reinterpret_cast<float *>(smem), 0, (int)gt);
     if (tid == 0)  // ready for the next launch
-        __hip_atomic_store(&a.counters[(size_t)b * gridDim.y + y], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&tl.counters[(size_t)b * GY + y], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // One small workgroup per head (blockIdx.x): the merge is a launch gap plus the time a CU needs to request the

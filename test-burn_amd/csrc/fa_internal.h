@@ -209,6 +209,7 @@ struct FaDecodeDev {
     uint32_t xcd_local;  // polled merge: a head group's workgroups share an XCD and exchange partials through its L2
     uint32_t rcp_gx, rcp_gy;  // xcd_local: floor(2^32 / d) + 1 for the grid's x and y dimensions (exact quotients of numbers below 2^16 by d < 2^16)
     uint32_t ny_real;    // != 0: the grid's y dimension is padded (to a multiple of 8 head groups) and only y < ny_real exist
+    uint32_t nb_q, nb_r;  // contiguous cache: a partition's 16-row blocks over the streaming waves, quotient and remainder
     unsigned long long poll_ticks;  // polled merge: how long the merging workgroup waits for partials, 100 MHz ticks
     // SAGE + FUSED (the int8 decode step in one launch): q is the raw f16 projection, k the int8 cache (written: the open
     // block's rows), k_scale is written too; the exact rows of the open block, the smoothing mean, the step's quantised query
