@@ -902,7 +902,8 @@ def bench_phase_timeline(f, args, which="decode_8k"):
     FOUNDRY_ATTN_LIB selects it). Every wave stamps the 100 MHz wall clock at the kernel's phase boundaries and leaves the
     stamps in the clock buffer; the workload is replayed as a HIP graph and the phases are reported in microseconds after
     the first workgroup's entry, as min / median / 90th percentile / max over the waves that reached them.
-    which: decode_8k (the fused decode step of the main configuration), sage_32k (the int8 step, wave 0 of every workgroup
+    which: decode_8k (the fused decode step of the main configuration), decode_1k (the same step in its 4-wave form:
+    Qwen2.5-0.5B shape at 1K context, a launch that is all latency), sage_32k (the int8 step, wave 0 of every workgroup
     = the wave that prepares the query and owns the open block), chunk32_8k (the short-chunk prefill kernel)."""
     rng = np.random.default_rng(0xF0DD + 21)
     if which == "decode_8k":
@@ -911,6 +912,26 @@ def bench_phase_timeline(f, args, which="decode_8k"):
         names = ["entry", "start barrier released", "block requests issued", "query operand ready", "first round: S done",
                  "first round: V in LDS", "block loop done", "state in LDS", "fold starts", "records stored", "merge done"]
 
+    elif which == "decode_1k":
+        H, Hkv, D, pos, cap, NL = 14, 2, 64, 1024, 1152, 16
+        cos, sin = fa.rope_tables(1e6, D, cap)
+        dcos, dsin = f.array(cos), f.array(sin)
+        caches = []
+        for i in range(NL):
+            kc, vc = np.zeros((Hkv, cap, D), np.float16), np.zeros((Hkv, cap, D), np.float16)
+            kc[:, :pos] = rng.standard_normal((Hkv, pos, D), dtype=np.float32).astype(np.float16)
+            vc[:, :pos] = rng.standard_normal((Hkv, pos, D), dtype=np.float32).astype(np.float16)
+            caches.append((f.array(kc), f.array(vc)))
+        q, k, v = (rng.standard_normal((1, n * D), dtype=np.float32).astype(np.float16) for n in (H, Hkv, Hkv))
+        dq, dk, dv, dqr, dout = f.array(q), f.array(k), f.array(v), f.zeros((H, 1, D)), f.zeros((1, H * D))
+        p1k = fa.KvPrepFusedParams.make(H, Hkv, D, 1, pos, cap, fa.ROPE_NEOX)
+        per_graph, waves, rows = 2 * NL, 4, 512 * 4
+        names = ["entry", "start barrier released", "block requests issued", "query operand ready", "first round: S done",
+                 "first round: V in LDS", "block loop done", "state in LDS", "fold starts", "records stored", "merge done"]
+
+        def step(i):
+            kc, vc = caches[i % NL]
+            f.decode_step_fused(dq.arg(), dk.arg(), dv.arg(), dqr.arg(), kc.arg(), vc.arg(), dcos.arg(), dsin.arg(), dout.arg(), p1k)
     elif which == "sage_32k":
         H, Hkv, D, N, NL = 16, 4, 128, 32768, 6
         P = N - 1
@@ -1325,7 +1346,7 @@ def bench_floors(f, args):
     emit(out)
 
 
-SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_chunk32_8k": bench_prefill_chunk, "llama3b_prefill_chunk32_32k": lambda f, args: bench_prefill_chunk(f, args, 32, 32736), "llama3b_prefill_chunk64_8k": lambda f, args: bench_prefill_chunk(f, args, 64, 8128), "timeline_decode_8k": bench_phase_timeline, "timeline_sage_32k": lambda f, args: bench_phase_timeline(f, args, "sage_32k"), "timeline_chunk32_8k": lambda f, args: bench_phase_timeline(f, args, "chunk32_8k"), "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_decode_2k": bench_short_decode, "llama3b_decode_512": lambda f, args: bench_short_decode(f, args, 511), "llama3b_prefill_2k": bench_prefill,
+SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_chunk32_8k": bench_prefill_chunk, "llama3b_prefill_chunk32_32k": lambda f, args: bench_prefill_chunk(f, args, 32, 32736), "llama3b_prefill_chunk64_8k": lambda f, args: bench_prefill_chunk(f, args, 64, 8128), "timeline_decode_8k": bench_phase_timeline, "timeline_decode_1k": lambda f, args: bench_phase_timeline(f, args, "decode_1k"), "timeline_sage_32k": lambda f, args: bench_phase_timeline(f, args, "sage_32k"), "timeline_chunk32_8k": lambda f, args: bench_phase_timeline(f, args, "chunk32_8k"), "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_decode_2k": bench_short_decode, "llama3b_decode_512": lambda f, args: bench_short_decode(f, args, 511), "llama3b_prefill_2k": bench_prefill,
              "llama3b_prefill_8k": lambda f, args: bench_prefill(f, args, 8192), "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,

@@ -90,6 +90,7 @@ constexpr int NT = NW * 64;  // threads per workgroup
 constexpr int BK = 16;       // keys per block (MFMA M dimension)
 constexpr int MBX = 3;       // blocks a wave keeps in flight (one round)
 constexpr int MAX_GT = 16;   // query heads served by one workgroup (the MFMA N dimension)
+constexpr int OWN_GT = 8;    // up to this many, the waves' states at the end of the block loop have LDS of their own
 
 using DecodeDev = ::FaDecodeDev;
 
@@ -588,6 +589,13 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         if constexpr (NW == 4)
             asm volatile("" ::"s"(a.d_len), "s"(a.d_len_stride), "s"(a.kv_len_add), "s"(a.kv_len), "s"(a.kv_len_bound));
     }
+    if constexpr (PAGED) {
+        // (a paged launch needs the length, then the page ids, before it can ask for rows: what those take in one trip)
+        asm volatile("" ::"s"(a.k), "s"(a.v), "s"(a.block_table), "s"(a.bt_stride), "s"(a.block_size), "s"(a.block_shift),
+                     "s"(a.n_kv_heads), "s"(a.capacity), "s"(a.chunk), "s"(a.sub_per_kv), "s"(a.gt), "s"(a.xcd_local),
+                     "s"(a.rcp_gx), "s"(a.rcp_gy), "s"(gridDim.x), "s"(gridDim.y), "s"(a.d_len), "s"(a.d_len_stride),
+                     "s"(a.kv_len_add), "s"(a.kv_len), "s"(a.kv_len_bound));
+    }
     if constexpr (EARLY_START) {
         if (tid == 0) sm_q_ready = 0;
         __syncthreads();
@@ -804,6 +812,9 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
         if (wave == 0) {
             // As below: the requests that do not depend on the length go out before any other wave may request anything.
             __builtin_amdgcn_s_setprio(3);
+            // (the arguments of these requests in one trip: the other waves wait at the barrier below until they are out)
+            asm volatile("" ::"s"(a.q), "s"(a.qin_stride_b), "s"(a.k_in), "s"(a.kvin_stride_b), "s"(a.sage_mean), "s"(a.v_in),
+                         "s"(a.sage_tail), "s"(a.d_len), "s"(a.d_len_stride), "s"(a.kv_len_add), "s"(a.kv_len), "s"(a.kv_len_bound));
             constexpr int QV = MAX_GT * D / 8 / 64;  // 16-byte pieces of the group's query rows per lane
             uint4 qv[QV], kv4 = make_uint4(0, 0, 0, 0), mv4 = make_uint4(0, 0, 0, 0);
             const __half *qrow = a.q + (size_t)b * a.qin_stride_b + (size_t)head0 * D;
@@ -949,6 +960,9 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
             // raw K / V row (parked in the block registers that this wave does not otherwise use). All lanes load
             // from valid addresses and select afterwards, so that no divergent branch separates the requests.
             __builtin_amdgcn_s_setprio(3);
+            if constexpr (NW == 4)  // (this wave's own arguments in one trip; the 8-wave form at 8K context loses 0.06 us by it)
+                asm volatile("" ::"s"(a.q), "s"(a.k_in), "s"(a.v_in), "s"(a.qin_stride_b), "s"(a.kvin_stride_b), "s"(a.cos_t),
+                             "s"(a.sin_t), "s"(a.table_rows), "s"(a.apply_rope), "s"(a.rope_normal));
             U4H qx[KSTEPS], qb[KSTEPS];
             const __half *qrow = a.q + (size_t)b * a.qin_stride_b + (size_t)(head0 + (head_ok ? n : 0)) * D;
             const __half *krow = a.k_in + (size_t)b * a.kvin_stride_b + (size_t)kvh * D;
@@ -1325,10 +1339,10 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     l_run += xor32(l_run);
 
     // Fold of the NW waves through LDS: sm_acc[wave][head][D] (+ 8 floats per wave, see below), sm_ml[wave][head][2].
-    // With up to 4 heads the states have a region of their own, so a wave writes its state as soon as it is done (the
+    // With up to OWN_GT heads the states have a region of their own, so a wave writes its state as soon as it is done (the
     // waves finish spread over the streaming time) and only the last wave's write is left before the barrier; with
     // more heads the region would not fit beside the V tiles and reuses them once every wave is done with them.
-    const bool own_region = gt <= 4;
+    const bool own_region = gt <= OWN_GT;
     if (!own_region) __syncthreads();  // every wave is done with its V region
     float *sm_acc = own_region ? reinterpret_cast<float *>(rope_lds + 2 * D) : reinterpret_cast<float *>(smem);
     const uint32_t wstr = gt * D + 8;  // a wave pair is 2 wstr apart: 64 bytes off a multiple of the bank span
@@ -1466,13 +1480,20 @@ enum Mode { MODE_PLAIN = 0, MODE_PAGED = 1, MODE_SAGE = 2, MODE_FUSED = 3, MODE_
 template <int D>
 size_t decode_lds_bytes(uint32_t gt) {
     // the per-wave V blocks + the Q^T operand + one RoPE table row
-    // ... + the waves' states at the end of the block loop, for up to 4 heads (more heads reuse the V tiles)
-    const size_t v_tiles = (size_t)NW * MBX * BK * (D * 2 + 32) + (size_t)(D / 32) * 64 * 16 + 2 * D +
-                           (size_t)NW * (4 * D + 8) * sizeof(float) + (size_t)NW * 4 * 2 * sizeof(float);
+    const size_t tiles = (size_t)NW * MBX * BK * (D * 2 + 32) + (size_t)(D / 32) * 64 * 16 + 2 * D;
+    // the waves' states at the end of the block loop: behind the tiles for up to OWN_GT heads (at 128 dims and 8 waves
+    // that is 145 KB of the compute unit's 160; two 4-wave workgroups need 75 KB each), over them for more
     const size_t fold = ((size_t)NW * (gt * D + 8) + (size_t)NW * gt * 2) * sizeof(float);
     const size_t merge = (size_t)NT * 6 * sizeof(float) * POLL_IPT;  // the cooperative merge holds POLL_IPT records per thread
-    size_t m = v_tiles > fold ? v_tiles : fold;
+    const size_t m = gt <= (uint32_t)OWN_GT ? tiles + fold : (tiles > fold ? tiles : fold);
     return m > merge ? m : merge;
+}
+// (the largest over the head counts a launch can have)
+template <int D>
+size_t decode_lds_cap() {
+    size_t cap = 0;
+    for (uint32_t gt = 1; gt <= (uint32_t)MAX_GT; ++gt) cap = decode_lds_bytes<D>(gt) > cap ? decode_lds_bytes<D>(gt) : cap;
+    return cap;
 }
 
 template <int D>
@@ -1486,7 +1507,7 @@ fa_status launch_d(fa_ctx *ctx, const DecodeDev &a, dim3 grid, int mode) {
         std::lock_guard<std::mutex> lds_lock(lds_mu);
         bool &lds_allowed = lds_allowed_on[ctx->device & 63];
         if (!lds_allowed) {
-            const int cap = (int)decode_lds_bytes<D>(MAX_GT);
+            const int cap = (int)decode_lds_cap<D>();
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, true, false, false>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
             FA_HIP(hipFuncSetAttribute((const void *)flash_decode_mfma_kernel<D, false, true, false>, hipFuncAttributeMaxDynamicSharedMemorySize, cap));
