@@ -270,6 +270,9 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a_by_value
             else if (ahead == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | BLK_DMA);
             else __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * BLK_DMA) & 15) | (((2 * BLK_DMA) >> 4) << 14));
         };
+        // (Tried as well: the whole ring requested at once - at 8K context a partition is just its four rounds - and slots
+        // reused without the producer waiting while it has rounds on their way. No gain, 19.7 against 19.4 us per launch:
+        // the rows do not arrive any sooner, memory delivers the launch's 33.5 MB at its own rate from the first request on.)
         // (Spacing the first rounds' requests in time, one round of the whole launch per interval at the memory's rate,
         // was tried so that round 0 would not share the queues with the later rounds: it lands 4.3 - 4.8 us after the
         // launch either way - 0.9 us until the workgroup knows its partition, 1.1 us until the requests are out, 2.5 us
