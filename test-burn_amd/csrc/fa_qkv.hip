@@ -50,6 +50,14 @@ struct QkvDev {
     const __half *scales[3];
 };
 
+// One of three values by matrix index. (Taken by value on purpose: `mat == 0 ? x0 : mat == 1 ? x1 : x2` written out on
+// variables is a conditional LVALUE - the compiler selects an address and loads through it, per lane, which keeps the three
+// in memory: launch arguments were fetched with a vector load from the argument block, locals went to scratch.)
+template <typename T>
+__device__ __forceinline__ T pick3(int mat, T x0, T x1, T x2) {
+    return mat == 0 ? x0 : mat == 1 ? x1 : x2;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
@@ -58,30 +66,46 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // WB: bits per weight - 16 (f16), 8 (Q8_0) or 4 (Q4_0)
 template <int WB>
-__global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
+__global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value) {
     constexpr bool Q8 = WB != 16;  // block-quantised: integer weights + one f16 scale per 32 of a row
     constexpr bool Q4 = WB == 4;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    // The arguments are read straight from the launch's argument block (the struct is its only member) into locals, those
+    // that the first weight request needs in one trip through the scalar cache. As a by-value struct the per-matrix
+    // pointers were fetched where a row's matrix was known - `mat == 0 ? a.w[0] : ...` became a per-lane VECTOR load
+    // from the argument block, with a wait for it (and for the input row requested before it) ahead of the first
+    // weight request: a trip to memory before the stream could start, and another per tile for bias and output.
+    const QkvDev &a = *(const QkvDev *)__builtin_amdgcn_kernarg_segment_ptr();
+    (void)a_by_value;
+    const unsigned char *const w0 = reinterpret_cast<const unsigned char *>(a.w[0]), *const w1 = reinterpret_cast<const unsigned char *>(a.w[1]),
+                        *const w2 = reinterpret_cast<const unsigned char *>(a.w[2]);
+    const uint32_t rows0 = a.rows[0], rows1 = a.rows[1], rows2 = a.rows[2];
+    const __half *const x_in = a.x;
+    const uint32_t K = a.k_dim, m_rows = a.m, cols_per_pass = a.cols_per_pass, rows_per_wg = a.rows_per_wg, x_stride = a.x_stride;
+    const uint32_t canonical_u = a.canonical;
+    asm volatile("" ::"s"(w0), "s"(w1), "s"(w2), "s"(rows0), "s"(rows1), "s"(rows2), "s"(x_in), "s"(K), "s"(m_rows), "s"(cols_per_pass),
+                 "s"(rows_per_wg), "s"(x_stride), "s"(canonical_u));
+    const bool canonical = canonical_u != 0;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, c = lane >> 4;
-    const uint32_t K = a.k_dim, nkb = K / 32;
-    const uint32_t total_rows = a.rows[0] + a.rows[1] + a.rows[2];
-    const uint32_t row_begin = blockIdx.x * a.rows_per_wg;
-    const uint32_t row_end = min(total_rows, row_begin + a.rows_per_wg);
+    const uint32_t nkb = K / 32;
+    const uint32_t total_rows = rows0 + rows1 + rows2;
+    const uint32_t row_begin = blockIdx.x * rows_per_wg;
+    const uint32_t row_end = min(total_rows, row_begin + rows_per_wg);
     if (row_begin >= row_end) return;
     const uint32_t n_tiles = (row_end - row_begin + 15) / 16;
-    const uint32_t m0 = blockIdx.y * a.cols_per_pass, cols = min(a.cols_per_pass, a.m - m0);
+    const uint32_t m0 = blockIdx.y * cols_per_pass, cols = min(cols_per_pass, m_rows - m0);
     unsigned char *x_lds = smem;
-    float *red = reinterpret_cast<float *>(smem + (size_t)a.cols_per_pass * a.x_stride);  // [QKV_NW][16][17], and scratch
+    float *red = reinterpret_cast<float *>(smem + (size_t)cols_per_pass * x_stride);  // [QKV_NW][16][17], and scratch
     // Q8: the block scales of this workgroup's rows, [tile][feature block][16 rows] f16
     _Float16 *sc_lds = reinterpret_cast<_Float16 *>(red + QKV_NW * 16 * 17);
 
     // Where a row of the concatenated list lives: matrix, row inside it, the matrix's row count.
-    auto locate = [&](uint32_t gr, int &mat, uint32_t &lrow) {
+    auto locate = [&](uint32_t gr, int &mat, uint32_t &lrow) __attribute__((always_inline)) {
         mat = 0, lrow = gr;
-        if (lrow >= a.rows[0]) {
-            lrow -= a.rows[0], mat = 1;
-            if (lrow >= a.rows[1]) lrow -= a.rows[1], mat = 2;
+        if (lrow >= rows0) {
+            lrow -= rows0, mat = 1;
+            if (lrow >= rows1) lrow -= rows1, mat = 2;
         }
     };
     // Weight operand of (tile, feature block kb): lane (n, c) holds features 8c..8c+7 of the block for row n of the
@@ -91,17 +115,17 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     // (Q8: the same element indices, one byte per element.)
     // (Q4: two elements per byte, element 2i in the low nibble of byte i.)
     typedef typename std::conditional<Q4, uint32_t, typename std::conditional<Q8, u2v_t, h8_t>::type>::type wreg_t;
-    auto tile_base = [&](uint32_t tile, const unsigned char *&p0, size_t &kb_stride, bool &ok) {
+    auto tile_base = [&](uint32_t tile, const unsigned char *&p0, size_t &kb_stride, bool &ok) __attribute__((always_inline)) {
         const uint32_t gr = row_begin + tile * 16 + n;
         ok = gr < row_end;
         int mat;
         uint32_t lrow;
         locate(ok ? gr : row_begin, mat, lrow);
-        const unsigned char *base = reinterpret_cast<const unsigned char *>(mat == 0 ? a.w[0] : mat == 1 ? a.w[1] : a.w[2]);
-        const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
+        const unsigned char *base = pick3(mat, w0, w1, w2);
+        const uint32_t N = pick3(mat, rows0, rows1, rows1);
         // canonical (blocked by 32 features): (k % 32) + 32 * (row + (k / 32) * N); row-major: row * K + k
-        p0 = base + (a.canonical ? (size_t)lrow * 32 + c * 8 : (size_t)lrow * K + c * 8) * WB / 8;
-        kb_stride = (a.canonical ? (size_t)N * 32 : 32) * WB / 8;
+        p0 = base + (canonical ? (size_t)lrow * 32 + c * 8 : (size_t)lrow * K + c * 8) * WB / 8;
+        kb_stride = (canonical ? (size_t)N * 32 : 32) * WB / 8;
     };
 
     // A wave takes the feature blocks kb = wave, wave + 8, ... of every tile, in batches of QKV_UNITS; two batches
@@ -110,7 +134,7 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     const uint32_t bpt = (per_tile + QKV_UNITS - 1) / QKV_UNITS;          // batches per tile
     const uint32_t n_batches = n_tiles * bpt;
     wreg_t wbuf[2][QKV_UNITS];
-    auto request = [&](wreg_t(&buf)[QKV_UNITS], uint32_t batch) {
+    auto request = [&](wreg_t(&buf)[QKV_UNITS], uint32_t batch) __attribute__((always_inline)) {
         const uint32_t tile = batch / bpt, j0 = (batch % bpt) * QKV_UNITS;
         const unsigned char *p0;
         size_t kb_stride;
@@ -119,12 +143,13 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
 #pragma unroll
         for (int i = 0; i < QKV_UNITS; ++i) {
             const uint32_t kb = (uint32_t)wave + (j0 + i) * QKV_NW;
-            wreg_t z;
-            if constexpr (Q4) z = 0u;
-            else if constexpr (Q8) z = u2v_t{0u, 0u};
-            else z = h8_t{0, 0, 0, 0, 0, 0, 0, 0};
-            // weights are read once per launch: non-temporal, so that they do not push everything else out of the L2
-            buf[i] = (ok && kb < nkb) ? __builtin_nontemporal_load(reinterpret_cast<const wreg_t *>(p0 + (size_t)kb * kb_stride)) : z;
+            // weights are read once per launch: non-temporal, so that they do not push everything else out of the L2.
+            // Every lane loads (a lane whose row is past the workgroup's last reads the first row's block: its sums
+            // are never written), and a block past the row's last is skipped by the whole wave and never consumed. No
+            // lane-dependent branch and no zero to merge with: with `(ok && kb < nkb) ? load : 0` the compiler
+            // moved a loaded register right behind every other request - a wait for ALL requests so far, one trip to
+            // memory per pair of requests.
+            if (kb < nkb) buf[i] = __builtin_nontemporal_load(reinterpret_cast<const wreg_t *>(p0 + (size_t)kb * kb_stride));
         }
     };
     // The first input row is requested before the weights (a CU's vector loads return in request order), then the
@@ -135,21 +160,23 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     for (int j = 0; j < XPRE; ++j) {
         const uint32_t k8 = tid + j * QKV_NT;
         const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-        x0[j] = k8 < K / 8 ? *reinterpret_cast<const h8_t *>(a.x + (size_t)m0 * K + k8 * 8) : z;
+        x0[j] = k8 < K / 8 ? *reinterpret_cast<const h8_t *>(x_in + (size_t)m0 * K + k8 * 8) : z;
     }
     // Q8: the block scales of this workgroup's rows (scales[row][kb] f16, row-major,
     // tests/gemv_v2_parity.rs:100-102), requested before the weights as well; they go to LDS as [tile][kb][row].
     constexpr int SPRE = 4;
     _Float16 sc0[SPRE];
+    const __half *const sc_p0 = Q8 ? a.scales[0] : nullptr, *const sc_p1 = Q8 ? a.scales[1] : nullptr, *const sc_p2 = Q8 ? a.scales[2] : nullptr;
+    if (Q8) asm volatile("" ::"s"(sc_p0), "s"(sc_p1), "s"(sc_p2));
     const uint32_t n_scales = Q8 ? n_tiles * 16 * nkb : 0u;
-    auto scale_of = [&](uint32_t idx) -> _Float16 {
+    auto scale_of = [&](uint32_t idx) __attribute__((always_inline)) -> _Float16 {
         const uint32_t tr = idx / nkb, kb = idx - tr * nkb;  // tr = tile * 16 + row
         const uint32_t gr = row_begin + tr;
         if (gr >= row_end) return (_Float16)0.0f;
         int mat;
         uint32_t lrow;
         locate(gr, mat, lrow);
-        const __half *sp = mat == 0 ? a.scales[0] : mat == 1 ? a.scales[1] : a.scales[2];
+        const __half *sp = pick3(mat, sc_p0, sc_p1, sc_p2);
         return *reinterpret_cast<const _Float16 *>(sp + (size_t)lrow * nkb + kb);
     };
     if (Q8) {
@@ -161,6 +188,12 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     }
     request(wbuf[0], 0);
     if (n_batches > 1) request(wbuf[1], 1);
+    // (what the normalisation and the write stage take, while the first requests are on their way)
+    const __half *const gamma = a.gamma, *const residual = a.residual;
+    const __half *const bias0 = a.bias[0], *const bias1 = a.bias[1], *const bias2 = a.bias[2];
+    __half *const out0 = a.out[0], *const out1 = a.out[1], *const out2 = a.out[2];
+    const float eps = a.eps, alpha = a.alpha, beta = a.beta;
+    asm volatile("" ::"s"(gamma), "s"(residual), "s"(bias0), "s"(bias1), "s"(bias2), "s"(out0), "s"(out1), "s"(out2), "s"(eps), "s"(alpha), "s"(beta));
 
     // Input rows of this pass into LDS, normalised: x * rsqrt(mean(x^2) + eps) * gamma in f32, rounded to f16.
     // Four rows or more: a wave takes whole rows (row r by wave r % 8) and needs no workgroup barrier for the sum of
@@ -168,8 +201,8 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     const bool rows_by_wave = cols >= 4;  // measured on 5120 x 3072: 2 rows 9.2 us row after row, 10.4 by wave; 4 rows 11.3 / 10.5; 8 rows 15.7 / 11.1
     if (rows_by_wave) {
         for (uint32_t r = wave; r < cols; r += QKV_NW) {
-            const __half *xr = a.x + (size_t)(m0 + r) * K;
-            unsigned char *dst = x_lds + (size_t)r * a.x_stride;
+            const __half *xr = x_in + (size_t)(m0 + r) * K;
+            unsigned char *dst = x_lds + (size_t)r * x_stride;
             float ss = 0.0f;
             for (uint32_t k8 = lane; k8 < K / 8; k8 += 64) {
                 const h8_t v = *reinterpret_cast<const h8_t *>(xr + k8 * 8);
@@ -177,11 +210,11 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) ss += (float)v[i] * (float)v[i];
             }
-            if (a.gamma) {
-                const float inv_rms = rsqrtf(wave_sum(ss) / (float)K + a.eps);
+            if (gamma) {
+                const float inv_rms = rsqrtf(wave_sum(ss) / (float)K + eps);
                 for (uint32_t k8 = lane; k8 < K / 8; k8 += 64) {  // each lane rewrites what it wrote
                     h8_t v = *reinterpret_cast<const h8_t *>(dst + k8 * 16);
-                    const h8_t g = *reinterpret_cast<const h8_t *>(a.gamma + k8 * 8);
+                    const h8_t g = *reinterpret_cast<const h8_t *>(gamma + k8 * 8);
 #pragma unroll
                     for (int i = 0; i < 8; ++i) v[i] = (_Float16)(((float)v[i] * inv_rms) * (float)g[i]);
                     *reinterpret_cast<h8_t *>(dst + k8 * 16) = v;
@@ -190,8 +223,8 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
         }
     }
     for (uint32_t r = 0; r < (rows_by_wave ? 0u : cols); ++r) {
-        const __half *xr = a.x + (size_t)(m0 + r) * K;
-        unsigned char *dst = x_lds + (size_t)r * a.x_stride;
+        const __half *xr = x_in + (size_t)(m0 + r) * K;
+        unsigned char *dst = x_lds + (size_t)r * x_stride;
         float ss = 0.0f;
         for (uint32_t k8 = tid, j = 0; k8 < K / 8; k8 += QKV_NT, ++j) {
             h8_t v;
@@ -201,17 +234,17 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) ss += (float)v[i] * (float)v[i];
         }
-        if (a.gamma) {
+        if (gamma) {
             ss = wave_sum(ss);
             if (lane == 0) red[wave] = ss;
             __syncthreads();
             float tot = 0.0f;
 #pragma unroll
             for (int w = 0; w < QKV_NW; ++w) tot += red[w];
-            const float inv_rms = rsqrtf(tot / (float)K + a.eps);
+            const float inv_rms = rsqrtf(tot / (float)K + eps);
             for (uint32_t k8 = tid; k8 < K / 8; k8 += QKV_NT) {  // each thread rewrites what it wrote
                 h8_t v = *reinterpret_cast<const h8_t *>(dst + k8 * 16);
-                const h8_t g = *reinterpret_cast<const h8_t *>(a.gamma + k8 * 8);
+                const h8_t g = *reinterpret_cast<const h8_t *>(gamma + k8 * 8);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) v[i] = (_Float16)(((float)v[i] * inv_rms) * (float)g[i]);
                 *reinterpret_cast<h8_t *>(dst + k8 * 16) = v;
@@ -229,7 +262,7 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     __syncthreads();
 
     // Sums the 8 waves' partial results of tile t in wave order, adds the bias, rounds once, stores token-major.
-    auto finish_tile = [&](uint32_t t, const f4v_t &mine) {
+    auto finish_tile = [&](uint32_t t, const f4v_t &mine) __attribute__((always_inline)) {
         __syncthreads();  // `red` may still be read for the previous tile
 #pragma unroll
         for (int i = 0; i < 4; ++i) red[((size_t)wave * 16 + c * 4 + i) * 17 + n] = mine[i];
@@ -244,12 +277,12 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
                 int mat;
                 uint32_t lrow;
                 locate(gr, mat, lrow);
-                const __half *bias = mat == 0 ? a.bias[0] : mat == 1 ? a.bias[1] : a.bias[2];
-                __half *out = mat == 0 ? a.out[0] : mat == 1 ? a.out[1] : a.out[2];
-                const uint32_t N = mat == 0 ? a.rows[0] : a.rows[1];
-                s *= a.alpha;
+                const __half *bias = pick3(mat, bias0, bias1, bias2);
+                __half *out = pick3(mat, out0, out1, out2);
+                const uint32_t N = pick3(mat, rows0, rows1, rows1);
+                s *= alpha;
                 if (bias) s += __half2float(bias[lrow]);
-                if (a.residual) s += __half2float(a.residual[(size_t)(m0 + col) * N + lrow]) * a.beta;
+                if (residual) s += __half2float(residual[(size_t)(m0 + col) * N + lrow]) * beta;
                 out[(size_t)(m0 + col) * N + lrow] = __float2half(s);
             }
         }
@@ -259,8 +292,8 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a) {
     // tile after tile and every wave sees the same sequence, so a tile is finished when its last batch is consumed.
     f4v_t d = {0.0f, 0.0f, 0.0f, 0.0f};
     const bool col_ok = (uint32_t)n < cols;
-    const unsigned char *x_lane = x_lds + (size_t)(col_ok ? n : 0) * a.x_stride + c * 16;
-    auto consume = [&](const wreg_t(&buf)[QKV_UNITS], uint32_t batch) {
+    const unsigned char *x_lane = x_lds + (size_t)(col_ok ? n : 0) * x_stride + c * 16;
+    auto consume = [&](const wreg_t(&buf)[QKV_UNITS], uint32_t batch) __attribute__((always_inline)) {
         const uint32_t tile = batch / bpt, j0 = (batch % bpt) * QKV_UNITS;
 #pragma unroll
         for (int i = 0; i < QKV_UNITS; ++i) {
