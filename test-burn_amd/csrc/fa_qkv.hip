@@ -80,10 +80,10 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
     const unsigned char *const w0 = reinterpret_cast<const unsigned char *>(a.w[0]), *const w1 = reinterpret_cast<const unsigned char *>(a.w[1]),
                         *const w2 = reinterpret_cast<const unsigned char *>(a.w[2]);
     const uint32_t rows0 = a.rows[0], rows1 = a.rows[1], rows2 = a.rows[2];
-    const __half *const x_in = a.x;
+    const __half *const x_in = a.x, *const gamma = a.gamma;
     const uint32_t K = a.k_dim, m_rows = a.m, cols_per_pass = a.cols_per_pass, rows_per_wg = a.rows_per_wg, x_stride = a.x_stride;
     const uint32_t canonical_u = a.canonical;
-    asm volatile("" ::"s"(w0), "s"(w1), "s"(w2), "s"(rows0), "s"(rows1), "s"(rows2), "s"(x_in), "s"(K), "s"(m_rows), "s"(cols_per_pass),
+    asm volatile("" ::"s"(w0), "s"(w1), "s"(w2), "s"(rows0), "s"(rows1), "s"(rows2), "s"(x_in), "s"(gamma), "s"(K), "s"(m_rows), "s"(cols_per_pass),
                  "s"(rows_per_wg), "s"(x_stride), "s"(canonical_u));
     const bool canonical = canonical_u != 0;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -134,7 +134,11 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
     const uint32_t bpt = (per_tile + QKV_UNITS - 1) / QKV_UNITS;          // batches per tile
     const uint32_t n_batches = n_tiles * bpt;
     wreg_t wbuf[2][QKV_UNITS];
-    auto request = [&](wreg_t(&buf)[QKV_UNITS], uint32_t batch) __attribute__((always_inline)) {
+    // `every`: all QKV_UNITS requests are made, one past the row's last block re-reads the last block (the first batch of
+    // a workgroup is asked for this way: from 2048 features on none of its blocks is past the end, and with a fixed
+    // number of requests behind the input row's the compiler can wait for that row alone - with a wave-dependent
+    // number it waited for every weight of the first two batches before the normalisation could start).
+    auto request = [&](wreg_t(&buf)[QKV_UNITS], uint32_t batch, bool every) __attribute__((always_inline)) {
         const uint32_t tile = batch / bpt, j0 = (batch % bpt) * QKV_UNITS;
         const unsigned char *p0;
         size_t kb_stride;
@@ -149,7 +153,8 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
             // lane-dependent branch and no zero to merge with: with `(ok && kb < nkb) ? load : 0` the compiler
             // moved a loaded register right behind every other request - a wait for ALL requests so far, one trip to
             // memory per pair of requests.
-            if (kb < nkb) buf[i] = __builtin_nontemporal_load(reinterpret_cast<const wreg_t *>(p0 + (size_t)kb * kb_stride));
+            if (every) buf[i] = __builtin_nontemporal_load(reinterpret_cast<const wreg_t *>(p0 + (size_t)min(kb, nkb - 1) * kb_stride));
+            else if (kb < nkb) buf[i] = __builtin_nontemporal_load(reinterpret_cast<const wreg_t *>(p0 + (size_t)kb * kb_stride));
         }
     };
     // The first input row is requested before the weights (a CU's vector loads return in request order), then the
@@ -161,6 +166,15 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
         const uint32_t k8 = tid + j * QKV_NT;
         const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
         x0[j] = k8 < K / 8 ? *reinterpret_cast<const h8_t *>(x_in + (size_t)m0 * K + k8 * 8) : z;
+    }
+    // ... and with it this thread's pieces of the norm's weights (of the input row again when there is no norm, so that
+    // the number of requests does not depend on it): requested behind the weights they would arrive behind them.
+    h8_t g0[XPRE];
+#pragma unroll
+    for (int j = 0; j < XPRE; ++j) {
+        const uint32_t k8 = tid + j * QKV_NT;
+        const h8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+        g0[j] = k8 < K / 8 ? *reinterpret_cast<const h8_t *>((gamma ? gamma : x_in) + k8 * 8) : z;
     }
     // Q8: the block scales of this workgroup's rows (scales[row][kb] f16, row-major,
     // tests/gemv_v2_parity.rs:100-102), requested before the weights as well; they go to LDS as [tile][kb][row].
@@ -186,14 +200,14 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
             sc0[j] = idx < n_scales ? scale_of(idx) : (_Float16)0.0f;
         }
     }
-    request(wbuf[0], 0);
-    if (n_batches > 1) request(wbuf[1], 1);
+    request(wbuf[0], 0, true);
+    if (n_batches > 1) request(wbuf[1], 1, false);
     // (what the normalisation and the write stage take, while the first requests are on their way)
-    const __half *const gamma = a.gamma, *const residual = a.residual;
+    const __half *const residual = a.residual;
     const __half *const bias0 = a.bias[0], *const bias1 = a.bias[1], *const bias2 = a.bias[2];
     __half *const out0 = a.out[0], *const out1 = a.out[1], *const out2 = a.out[2];
     const float eps = a.eps, alpha = a.alpha, beta = a.beta;
-    asm volatile("" ::"s"(gamma), "s"(residual), "s"(bias0), "s"(bias1), "s"(bias2), "s"(out0), "s"(out1), "s"(out2), "s"(eps), "s"(alpha), "s"(beta));
+    asm volatile("" ::"s"(residual), "s"(bias0), "s"(bias1), "s"(bias2), "s"(out0), "s"(out1), "s"(out2), "s"(eps), "s"(alpha), "s"(beta));
 
     // Input rows of this pass into LDS, normalised: x * rsqrt(mean(x^2) + eps) * gamma in f32, rounded to f16.
     // Four rows or more: a wave takes whole rows (row r by wave r % 8) and needs no workgroup barrier for the sum of
@@ -242,9 +256,11 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
 #pragma unroll
             for (int w = 0; w < QKV_NW; ++w) tot += red[w];
             const float inv_rms = rsqrtf(tot / (float)K + eps);
-            for (uint32_t k8 = tid; k8 < K / 8; k8 += QKV_NT) {  // each thread rewrites what it wrote
+            for (uint32_t k8 = tid, j = 0; k8 < K / 8; k8 += QKV_NT, ++j) {  // each thread rewrites what it wrote
                 h8_t v = *reinterpret_cast<const h8_t *>(dst + k8 * 16);
-                const h8_t g = *reinterpret_cast<const h8_t *>(gamma + k8 * 8);
+                h8_t g;
+                if (j < (uint32_t)XPRE) g = j == 0 ? g0[0] : g0[1];
+                else g = *reinterpret_cast<const h8_t *>(gamma + k8 * 8);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) v[i] = (_Float16)(((float)v[i] * inv_rms) * (float)g[i]);
                 *reinterpret_cast<h8_t *>(dst + k8 * 16) = v;
@@ -345,10 +361,10 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
     };
     for (uint32_t b = 0; b < n_batches; b += 2) {
         consume(wbuf[0], b);
-        if (b + 2 < n_batches) request(wbuf[0], b + 2);
+        if (b + 2 < n_batches) request(wbuf[0], b + 2, false);
         if (b + 1 < n_batches) {
             consume(wbuf[1], b + 1);
-            if (b + 3 < n_batches) request(wbuf[1], b + 3);
+            if (b + 3 < n_batches) request(wbuf[1], b + 3, false);
         }
     }
 }
