@@ -48,6 +48,7 @@ struct QkvDev {
     float alpha, beta;
     // Q8_0 weights: w[i] point at int8 values (same two layouts, in elements), scales[i] at f16 [rows, k_dim / 32]
     const __half *scales[3];
+    uint32_t rcp_nkb;  // floor(2^32 / (k_dim / 32)) + 1: exact quotients of a workgroup's scale indices (below 2^16)
 };
 
 // One of three values by matrix index. (Taken by value on purpose: `mat == 0 ? x0 : mat == 1 ? x1 : x2` written out on
@@ -177,14 +178,17 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
         g0[j] = k8 < K / 8 ? *reinterpret_cast<const h8_t *>((gamma ? gamma : x_in) + k8 * 8) : z;
     }
     // Q8: the block scales of this workgroup's rows (scales[row][kb] f16, row-major,
-    // tests/gemv_v2_parity.rs:100-102), requested before the weights as well; they go to LDS as [tile][kb][row].
+    // tests/gemv_v2_parity.rs:100-102); they go to LDS as [tile][kb][row].
     constexpr int SPRE = 4;
     _Float16 sc0[SPRE];
     const __half *const sc_p0 = Q8 ? a.scales[0] : nullptr, *const sc_p1 = Q8 ? a.scales[1] : nullptr, *const sc_p2 = Q8 ? a.scales[2] : nullptr;
-    if (Q8) asm volatile("" ::"s"(sc_p0), "s"(sc_p1), "s"(sc_p2));
+    const uint32_t rcp_nkb = Q8 ? a.rcp_nkb : 0u;
+    if (Q8) asm volatile("" ::"s"(sc_p0), "s"(sc_p1), "s"(sc_p2), "s"(rcp_nkb));
+    // (index / nkb as a product: four divisions per thread stood between the launch's entry and its first weight request)
+    auto div_nkb = [&](uint32_t idx) __attribute__((always_inline)) -> uint32_t { return nkb == 1 ? idx : __umulhi(idx, rcp_nkb); };
     const uint32_t n_scales = Q8 ? n_tiles * 16 * nkb : 0u;
     auto scale_of = [&](uint32_t idx) __attribute__((always_inline)) -> _Float16 {
-        const uint32_t tr = idx / nkb, kb = idx - tr * nkb;  // tr = tile * 16 + row
+        const uint32_t tr = div_nkb(idx), kb = idx - tr * nkb;  // tr = tile * 16 + row
         const uint32_t gr = row_begin + tr;
         if (gr >= row_end) return (_Float16)0.0f;
         int mat;
@@ -193,6 +197,9 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
         const __half *sp = pick3(mat, sc_p0, sc_p1, sc_p2);
         return *reinterpret_cast<const _Float16 *>(sp + (size_t)lrow * nkb + kb);
     };
+    request(wbuf[0], 0, true);
+    // (the scales behind the first batch: their addresses take a few hundred instructions, which the first weight
+    // requests should not wait for; they are needed when that batch is consumed)
     if (Q8) {
 #pragma unroll
         for (int j = 0; j < SPRE; ++j) {
@@ -200,7 +207,6 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
             sc0[j] = idx < n_scales ? scale_of(idx) : (_Float16)0.0f;
         }
     }
-    request(wbuf[0], 0, true);
     if (n_batches > 1) request(wbuf[1], 1, false);
     // (what the normalisation and the write stage take, while the first requests are on their way)
     const __half *const residual = a.residual;
@@ -271,7 +277,7 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
     if (Q8) {
         for (uint32_t idx = tid, j = 0; idx < n_scales; idx += QKV_NT, ++j) {
             const _Float16 v = j < (uint32_t)SPRE ? (j == 0 ? sc0[0] : j == 1 ? sc0[1] : j == 2 ? sc0[2] : sc0[3]) : scale_of(idx);
-            const uint32_t tr = idx / nkb, kb = idx - tr * nkb;
+            const uint32_t tr = div_nkb(idx), kb = idx - tr * nkb;
             sc_lds[((size_t)(tr >> 4) * nkb + kb) * 16 + (tr & 15)] = v;
         }
     }
@@ -378,6 +384,7 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l, bool weight_
     a.x = l.x, a.gamma = l.gamma, a.k_dim = l.k_dim, a.m = l.m, a.eps = l.eps, a.canonical = l.canonical ? 1u : 0u;
     a.residual = l.residual, a.alpha = l.alpha, a.beta = l.beta;
     for (int i = 0; i < 3; ++i) a.scales[i] = l.scales[i];
+    a.rcp_nkb = l.k_dim / 32 > 1 ? (uint32_t)((1ull << 32) / (l.k_dim / 32)) + 1u : 0u;
     const bool q8 = l.scales[0] != nullptr;
     const bool q4 = l.weight_bits == 4;
     // More than a few input rows: no longer a weight stream but a GEMM (fa_gemm.hip). Measured on 5120 x 3072 with a
