@@ -580,14 +580,15 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // then cleared here, behind a barrier that costs the waves' entry skew only.
     constexpr bool EARLY_START = FUSED && !SAGE && NW == 8;
     if constexpr (!PAGED) {
-        // ... and those on the way to the first request in ONE trip through the scalar cache, not one trip per use.
+        // The arguments on the way to the first request, in ONE trip through the scalar cache (an empty statement that takes
+        // them as scalar inputs makes the compiler fetch them here): read where they are used they were five trips in a row.
         asm volatile("" ::"s"(a.k), "s"(a.v), "s"(a.k_stride_b), "s"(a.k_stride_h), "s"(a.v_stride_b), "s"(a.v_stride_h),
                      "s"(a.capacity), "s"(a.chunk), "s"(a.sub_per_kv), "s"(a.gt), "s"(a.xcd_local), "s"(a.rcp_gx),
                      "s"(a.rcp_gy), "s"(a.nb_q), "s"(a.nb_r), "s"(gridDim.x), "s"(gridDim.y));
         // (In the 4-wave form also what reading the length takes, one more trip later instead of three: 6.28 -> 6.24 us
         // per launch at 512 tokens of context. The 8-wave form loses by it, 10.12 -> 10.19 us at 8K.)
         if constexpr (NW == 4)
-            asm volatile("" ::"s"(a.d_len), "s"(a.d_len_stride), "s"(a.kv_len_add), "s"(a.kv_len), "s"(a.kv_len_bound));
+            asm volatile("" ::"s"(a.d_len), "s"(a.d_len_stride), "s"(a.kv_len_add), "s"(a.kv_len), "s"(a.kv_len_bound), "s"(a.ny_real));
     }
     if constexpr (PAGED) {
         // (a paged launch needs the length, then the page ids, before it can ask for rows: what those take in one trip)
