@@ -665,12 +665,12 @@ def bench_o_proj(f, args, q8=False):
     f.profile_enable(False)
 
 
-def bench_long_decode(f, args):
+def bench_long_decode(f, args, ctx=131072):
     """Llama-3.2-3B-shaped single-layer decode step at 131072 tokens of context (contiguous cache, 537 MB of K and V
     per layer): the decode kernel where one launch is large. Two layers' caches in rotation (more than the last-level
-    cache holds)."""
+    cache holds); at ctx = 65536 / 32768 (llama3b_decode_64k / _32k) four / eight."""
     import orc
-    H, Hkv, D, pos, NL = 24, 8, 128, 131071, 2
+    H, Hkv, D, pos, NL = 24, 8, 128, ctx - 1, 2 * (131072 // ctx)
     cap = pos + 1 + 128
     rng = np.random.default_rng(0xF0DD + 9)
     cos, sin = fa.rope_tables(5e5, D, cap)
@@ -707,9 +707,9 @@ def bench_long_decode(f, args):
     f.synchronize()
     dt = time.perf_counter() - t0
     nbytes = 2.0 * Hkv * (pos + 1) * D * 2 + 2 * Hkv * D * 2 + 2 * H * D * 2 + 2 * Hkv * D * 2 + 2 * D
-    _finish_secondary(f, args, "decode-attn layer-steps/s + achieved HBM GB/s, Llama-3.2-3B shape @128K ctx",
+    _finish_secondary(f, args, "decode-attn layer-steps/s + achieved HBM GB/s, Llama-3.2-3B shape @%dK ctx" % (ctx // 1024),
                       "llama3.2-3b single-layer decode step at long context: RoPE + KV append + flash decode, batch 1, "
-                      "H24/Hkv8/D128, kv_len 131072, eager launches (profiling events on)", "fused_rope_append_decode_kernel",
+                      "H24/Hkv8/D128, kv_len %d, eager launches (profiling events on)" % ctx, "fused_rope_append_decode_kernel",
                       nbytes, dt, {"decode_max_abs_err": err})
     f.profile_enable(False)
 
@@ -1346,7 +1346,7 @@ def bench_floors(f, args):
     emit(out)
 
 
-SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_chunk32_8k": bench_prefill_chunk, "llama3b_prefill_chunk32_32k": lambda f, args: bench_prefill_chunk(f, args, 32, 32736), "llama3b_prefill_chunk64_8k": lambda f, args: bench_prefill_chunk(f, args, 64, 8128), "timeline_decode_8k": bench_phase_timeline, "timeline_decode_1k": lambda f, args: bench_phase_timeline(f, args, "decode_1k"), "timeline_sage_32k": lambda f, args: bench_phase_timeline(f, args, "sage_32k"), "timeline_chunk32_8k": lambda f, args: bench_phase_timeline(f, args, "chunk32_8k"), "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_decode_2k": bench_short_decode, "llama3b_decode_512": lambda f, args: bench_short_decode(f, args, 511), "llama3b_prefill_2k": bench_prefill,
+SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_chunk32_8k": bench_prefill_chunk, "llama3b_prefill_chunk32_32k": lambda f, args: bench_prefill_chunk(f, args, 32, 32736), "llama3b_prefill_chunk64_8k": lambda f, args: bench_prefill_chunk(f, args, 64, 8128), "timeline_decode_8k": bench_phase_timeline, "timeline_decode_1k": lambda f, args: bench_phase_timeline(f, args, "decode_1k"), "timeline_sage_32k": lambda f, args: bench_phase_timeline(f, args, "sage_32k"), "timeline_chunk32_8k": lambda f, args: bench_phase_timeline(f, args, "chunk32_8k"), "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_decode_64k": lambda f, args: bench_long_decode(f, args, 65536), "llama3b_decode_32k": lambda f, args: bench_long_decode(f, args, 32768), "llama3b_decode_2k": bench_short_decode, "llama3b_decode_512": lambda f, args: bench_short_decode(f, args, 511), "llama3b_prefill_2k": bench_prefill,
              "llama3b_prefill_8k": lambda f, args: bench_prefill(f, args, 8192), "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,

@@ -89,7 +89,9 @@ fa_status fa_launch_decode(fa_ctx *ctx, const DecodeLaunch &L) {
         // which 768 keys (393 KB) do not amortise when workgroups run one after the other on a CU
         // (C3, 8 waves: 62.9 us with <= 768 keys, 52.0 us with <= 1536).
         const uint32_t long_chunk = 4u * nw * MBX * BK;  // four rounds of a workgroup: 1536 keys at 8 waves
-        const uint32_t per_slot = ceil_div_u32(ceil_div_u32(bound, s_max), long_chunk);
+        // (One sequence has nothing to balance: its partitions stay whole, one per slot, and with every workgroup
+        // resident the merge runs inside the launch instead of as a second one.)
+        const uint32_t per_slot = L.batch == 1 ? 1u : ceil_div_u32(ceil_div_u32(bound, s_max), long_chunk);
         uint32_t c = ceil_div_u32(ceil_div_u32(bound, s_max * per_slot), (uint32_t)BK) * BK;
         if (c < nw * BK) c = nw * BK;
         return c;
