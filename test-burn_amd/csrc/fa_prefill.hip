@@ -449,7 +449,19 @@ __device__ __forceinline__ void phase_barrier() {
 // Wave w of a group moves rows 16w..16w+15 of every tile of its group (16 rows never straddle a page). Rows past
 // the visible keys come out of the buffer descriptor's bound check as zeros.
 template <int D, bool BF16, bool PAGED>
-__global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a) {
+__global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a_by_value) {
+    // The launch's arguments as a local copy read from its argument block in ONE trip through the scalar cache (an empty
+    // statement that takes the fields as scalar inputs makes the compiler fetch them here). As a by-value struct the
+    // fields were fetched where the program first needs them: thirteen dependent trips, one wait each, between the entry
+    // and the first request of a workgroup's first item.
+    const PrefillDev a = *(const PrefillDev *)__builtin_amdgcn_kernarg_segment_ptr();
+    (void)a_by_value;
+    asm volatile("" ::"s"(a.q), "s"(a.k), "s"(a.v), "s"(a.out), "s"(a.q_stride_h), "s"(a.q_stride_m), "s"(a.k_stride_h), "s"(a.v_stride_h),
+                 "s"(a.out_stride_h), "s"(a.out_stride_m), "s"(a.block_table), "s"(a.n_heads), "s"(a.group_size), "s"(a.q_len),
+                 "s"(a.kv_len), "s"(a.query_offset), "s"(a.causal), "s"(a.block_size), "s"(a.block_shift), "s"(a.n_kv_heads));
+    asm volatile("" ::"s"(a.splits), "s"(a.n_qt), "s"(a.n_items), "s"(a.n_workgroups), "s"(a.pool_bytes32), "s"(a.pack_heads),
+                 "s"(a.pack_nb), "s"(a.pack_blocks), "s"(a.part_rows), "s"(a.part_acc), "s"(a.part_ml), "s"(a.scale_log2e),
+                 "s"(a.out_aligned16), "s"(a.clock_out));
     constexpr int DSTEPS = D / 16, DBLKS = D / 32, ROWB = D * 2, CHK = D / 8;
     constexpr int K_TILE = BN * ROWB, V_TILE = BN * ROWB, GRP_LDS = 2 * K_TILE + 2 * V_TILE;
     constexpr int RB_BYTES = CHK * 256;  // one 16-row block of a K tile
@@ -972,7 +984,6 @@ template <int D, bool BF16>
 __global__ void __launch_bounds__(256) flash_prefill_merge_kernel(PrefillDev a) {
     constexpr int CG = D / 4;           // float4 columns per row
     constexpr int ROWS = 256 / CG;      // rows per workgroup (8 at D = 128, 16 at D = 64)
-    constexpr int PB = 8;               // splits loaded per batch
     const uint32_t S = a.splits, PR = a.part_rows;
     const uint32_t SLABS = PR / ROWS;   // workgroups per query tile
     const uint32_t n_qt = gridDim.x / (a.n_heads * SLABS);
@@ -982,34 +993,46 @@ __global__ void __launch_bounds__(256) flash_prefill_merge_kernel(PrefillDev a) 
     const uint32_t q_row = q_tile * BM + r;
     if (q_row >= a.q_len) return;
     const size_t base = (((size_t)head * n_qt + q_tile) * S) * PR + r;
-    float mstar = -1e30f;
-    for (uint32_t s0 = 0; s0 < S; s0 += PB) {  // PB loads in flight (one after the other they cost a memory latency each)
-        float2 ml[PB];
-#pragma unroll
-        for (int k = 0; k < PB; ++k) ml[k] = *reinterpret_cast<const float2 *>(a.part_ml + (base + (size_t)min(s0 + k, S - 1) * PR) * 2);
-#pragma unroll
-        for (int k = 0; k < PB; ++k)
-            if (s0 + k < S && ml[k].y > 0.0f) mstar = fmaxf(mstar, ml[k].x);
-    }
-    float L = 0.0f;
+    // All of a row's splits in ONE trip to memory when there are at most 32 of them (the usual case): the (max, sum)
+    // pairs and the sums are requested together - the addresses of the sums do not depend on the pairs - and the two passes
+    // of the reference (the row's maximum, then the weighted sums in split order) run on registers. The batch size is the
+    // smallest of 4, 8, 16, 32 that covers the splits (loads past the last split re-read it and carry no weight). More
+    // than 32 splits go in batches of 32 whose results are combined as the batches of a running softmax are.
+    // (Before: 8 pairs per trip for the maximum, then 8 pairs and sums per trip again - eight trips in a row for 32
+    // splits, most of the launch's 5.9 us.)
+    float m_run = -1e30f, L = 0.0f;
     float4 o = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    for (uint32_t s0 = 0; s0 < S; s0 += PB) {
-        float4 v[PB];
-        float2 ml[PB];
+    auto batch = [&](auto pb, uint32_t s0) __attribute__((always_inline)) {
+        constexpr int P = decltype(pb)::value;
+        float4 v[P];
+        float2 ml[P];
 #pragma unroll
-        for (int k = 0; k < PB; ++k) {
+        for (int k = 0; k < P; ++k) {
             const uint32_t s = min(s0 + k, S - 1);  // clamped; masked below
-            v[k] = *reinterpret_cast<const float4 *>(a.part_acc + (base + (size_t)s * PR) * D + c4 * 4);
             ml[k] = *reinterpret_cast<const float2 *>(a.part_ml + (base + (size_t)s * PR) * 2);
+            v[k] = *reinterpret_cast<const float4 *>(a.part_acc + (base + (size_t)s * PR) * D + c4 * 4);
         }
+        float mb = m_run;
 #pragma unroll
-        for (int k = 0; k < PB; ++k) {
-            if (s0 + k >= S || !(ml[k].y > 0.0f)) continue;
-            const float w = fast_exp2(ml[k].x - mstar);
-            L += ml[k].y * w;
-            o.x += v[k].x * w, o.y += v[k].y * w, o.z += v[k].z * w, o.w += v[k].w * w;
+        for (int k = 0; k < P; ++k)
+            if (s0 + k < S && ml[k].y > 0.0f) mb = fmaxf(mb, ml[k].x);
+        const float e0 = fast_exp2(m_run - mb);  // (0 for the first batch: nothing has been summed yet)
+        L *= e0, o.x *= e0, o.y *= e0, o.z *= e0, o.w *= e0;
+#pragma unroll
+        for (int k = 0; k < P; ++k) {
+            const bool counts = s0 + k < S && ml[k].y > 0.0f;
+            const float w = counts ? fast_exp2(ml[k].x - mb) : 0.0f;
+            L += counts ? ml[k].y * w : 0.0f;
+            o.x += counts ? v[k].x * w : 0.0f, o.y += counts ? v[k].y * w : 0.0f;
+            o.z += counts ? v[k].z * w : 0.0f, o.w += counts ? v[k].w * w : 0.0f;
         }
-    }
+        m_run = mb;
+    };
+    if (S <= 4) batch(std::integral_constant<int, 4>{}, 0);
+    else if (S <= 8) batch(std::integral_constant<int, 8>{}, 0);
+    else if (S <= 16) batch(std::integral_constant<int, 16>{}, 0);
+    else
+        for (uint32_t s0 = 0; s0 < S; s0 += 32) batch(std::integral_constant<int, 32>{}, s0);
     const float inv = (isfinite(L) && fabsf(L) > 1e-6f) ? (1.0f / L) : 0.0f;
     h4_t h;
     h[0] = to_elem<BF16>(o.x * inv), h[1] = to_elem<BF16>(o.y * inv), h[2] = to_elem<BF16>(o.z * inv), h[3] = to_elem<BF16>(o.w * inv);
