@@ -35,6 +35,7 @@ def gpu_decode(q, k, v, H, D, N, causal=True, query_offset=None, q_arg_dims=None
     (16, 2, 128, 3000, 3008),   # Qwen2.5-3B shape
     (16, 4, 128, 5000, 5120),   # SmolLM3 shape
     (32, 8, 128, 777, 1024),
+    (24, 8, 128, 70000, 70016),  # a long context at batch 1: whole partitions, one per compute unit, merged inside the launch
     (8, 8, 64, 130, 130), (2, 1, 128, 64, 64), (12, 2, 64, 333, 400), (10, 2, 128, 100, 128), (16, 1, 64, 70, 96),
 ])
 def test_decode_vs_oracle(H, Hkv, D, N, cap):

@@ -55,6 +55,7 @@ class Paged:
     (14, 2, 64, 16, [100, 5, 64]),
     (24, 8, 128, 32, [300, 31]),
     (8, 8, 64, 64, [129]),
+    (24, 8, 128, 16, [40000]),  # one long sequence: whole partitions, one per compute unit, merged inside the launch
 ])
 def test_paged_batched_decode_step(H, Hkv, D, bs, lens):
     """One batched decode step: append one token per sequence at seq_lens[b], then ragged flash decode."""
