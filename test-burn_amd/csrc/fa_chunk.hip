@@ -312,7 +312,8 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a_by_value
         // suspicion was that writing them back at the end of the launch is why launches of a graph follow one another
         // 2 us apart here against 0.4 us after a decode launch. An agent-scope release from every workgroup: 26.8 us per
         // launch instead of 19.3; from one workgroup per XCD: no gain. Device-scope stores for the sums and (m, l), which go
-        // through to memory as they are made: 28.4 us, and 45.6 instead of 26.5 at 64 rows - the wave waits for them.)
+        // through to memory as they are made: 28.4 us, and 45.6 instead of 26.5 at 64 rows - the wave waits for them. Non-temporal
+        // stores: no change at 32 rows, 26.7 - 27.2 us instead of 24.8 - 25.9 at 64.)
         return;  // (a wave that has ended no longer counts at the workgroup's barriers)
     }
 
