@@ -28,6 +28,7 @@
 // device-coherent accesses. Same residency assumption and the same bounded wait as the decode kernel's polled merge.
 #include "fa_internal.h"
 #include "fa_lds_dma.h"
+#include <type_traits>
 
 namespace {
 
@@ -120,6 +121,7 @@ __global__ void __launch_bounds__(NTW, 1) flash_chunk_kernel(ChunkDev a_by_value
     // The arguments are read where the program needs them, straight from the launch's argument block (the struct is its
     // only member): a by-value struct is copied field by field at the kernel's entry, every field the kernel ever uses
     // ahead of the first request. Those that the first request does need come in one trip through the scalar cache.
+    static_assert(std::is_trivially_copyable<ChunkDev>::value, "read as raw bytes from the argument block, where it is the first member");
     const ChunkDev &a = *(const ChunkDev *)__builtin_amdgcn_kernarg_segment_ptr();
     (void)a_by_value;
     asm volatile("" ::"s"(a.k), "s"(a.v), "s"(a.k_stride_h), "s"(a.v_stride_h), "s"(a.part_len), "s"(a.kv_end), "s"(a.nsplits),

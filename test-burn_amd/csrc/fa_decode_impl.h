@@ -518,6 +518,7 @@ __global__ void __launch_bounds__(NT, NW == 8 ? 1 : 2) flash_decode_mfma_kernel(
     // The arguments are read where the program needs them, straight from the launch's argument block (the struct is its
     // first and only member): a by-value struct is copied field by field at the kernel's entry, which puts every field
     // the kernel ever uses - four dozen scalar registers, half of them spilled at once - ahead of the first request.
+    static_assert(std::is_trivially_copyable<DecodeDev>::value, "read as raw bytes from the argument block, where it is the first member");
     const DecodeDev &a = *(const DecodeDev *)__builtin_amdgcn_kernarg_segment_ptr();
     (void)a_by_value;
     constexpr int KSTEPS = SAGE ? D / 64 : D / 32;  // MFMA steps over head_dim for S^T; 16 B per lane each

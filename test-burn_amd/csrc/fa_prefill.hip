@@ -454,6 +454,7 @@ __global__ void __launch_bounds__(512, 1) flash_prefill_dma_kernel(PrefillDev a_
     // statement that takes the fields as scalar inputs makes the compiler fetch them here). As a by-value struct the
     // fields were fetched where the program first needs them: thirteen dependent trips, one wait each, between the entry
     // and the first request of a workgroup's first item.
+    static_assert(std::is_trivially_copyable<PrefillDev>::value, "read as raw bytes from the argument block, where it is the first member");
     const PrefillDev a = *(const PrefillDev *)__builtin_amdgcn_kernarg_segment_ptr();
     (void)a_by_value;
     asm volatile("" ::"s"(a.q), "s"(a.k), "s"(a.v), "s"(a.out), "s"(a.q_stride_h), "s"(a.q_stride_m), "s"(a.k_stride_h), "s"(a.v_stride_h),

@@ -76,6 +76,7 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
     // pointers were fetched where a row's matrix was known - `mat == 0 ? a.w[0] : ...` became a per-lane VECTOR load
     // from the argument block, with a wait for it (and for the input row requested before it) ahead of the first
     // weight request: a trip to memory before the stream could start, and another per tile for bias and output.
+    static_assert(std::is_trivially_copyable<QkvDev>::value, "read as raw bytes from the argument block, where it is the first member");
     const QkvDev &a = *(const QkvDev *)__builtin_amdgcn_kernarg_segment_ptr();
     (void)a_by_value;
     const unsigned char *const w0 = reinterpret_cast<const unsigned char *>(a.w[0]), *const w1 = reinterpret_cast<const unsigned char *>(a.w[1]),
