@@ -482,7 +482,8 @@ fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_ar
  * by fa_kv_prep_fused on the same context: every projection is rounded to f16 as FusedQkv stores it, then rotated and
  * placed as KvPrepFused does. qkv_params->m must equal params->seq_len, n_dim = params->d_model, n_kv = params->kv_dim;
  * head_dim 64 or 128; f16 only; q_rot, caches / pools, biases and tables 16-byte aligned. From fa_set_gemm_min_m() rows
- * on it is the GEMM's write stage (no q / k / v round trip, one launch fewer); with fewer rows the weight-stream
+ * on it is the GEMM's write stage (no q / k / v round trip, one launch fewer); with fewer rows - and for a chunk that
+ * the one-launch weight stream for up to 32 rows takes (see fa_matmul) - the weight-stream
  * kernel writes q, k, v into the context's workspace and the KvPrepFused kernel follows (m = 1 belongs to
  * fa_decode_step_fused, which takes the raw projections). Workspace rule under capture as for fa_fused_qkv. */
 fa_status fa_fused_qkv_kv_prep(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
@@ -509,6 +510,10 @@ fa_status fa_fused_qkv_kv_prep_paged(fa_ctx *ctx, const fa_tensor_arg *w_q, cons
  * (FA_ERR_OPERATION_NOT_SUPPORTED). bias, c: NULL or NULL buffer = absent (the reference's "zero" placeholder).
  * Any m is accepted: up to fa_set_gemm_min_m() - 1 input rows run as passes of 16 over the weight stream; from there
  * on the op is a tiled GEMM on the matrix cores, the counterpart of the reference's GEMM for large m (src/metals/mma).
+ * A chunk of 12 to 32 input rows (the reference's default prefill chunk is 32) against F16 weights of 2048 or 3072
+ * features with at most 32 weight rows per compute unit is one launch of a weight-stream kernel of its own instead of
+ * the GEMM's three, unless fa_set_gemm_min_m() was called with a threshold the chunk reaches (environment
+ * FOUNDRY_ATTN_QKV_ROWS32_MIN_M, read at fa_ctx_create: the fewest rows it takes, 33 = never).
  * Block-quantised weights follow the arithmetic of the path that runs: the weight stream multiplies each 32-block's f32
  * sum by the block scale (the GEMV policies, policy_q8.metal / policy_q4_0.metal), the GEMM works on f16(weight * scale)
  * tiles like the reference's tile loader (src/metals/mma/tile_loader.metal:100-120); the two differ by the f16 rounding

@@ -120,6 +120,7 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     ctx->decode_waves = env_u32("FOUNDRY_ATTN_DECODE_WAVES", 0);
     if (ctx->decode_waves != 4 && ctx->decode_waves != 8) ctx->decode_waves = 0;
     ctx->gemm_min_m = env_u32("FOUNDRY_ATTN_GEMM_MIN_M", 0);
+    ctx->qkv_rows32_min_m = env_u32("FOUNDRY_ATTN_QKV_ROWS32_MIN_M", 0);
     ctx->gemm_variant = env_u32("FOUNDRY_ATTN_GEMM_VARIANT", 0);
     if (ctx->gemm_variant > 3) ctx->gemm_variant = 0;
     ctx->prefill_split_k = env_u32("FOUNDRY_ATTN_PREFILL_SPLIT_K", 0);
@@ -1050,7 +1051,9 @@ static fa_status fused_qkv_kv_prep(fa_ctx *ctx, FusedQkvLaunch &Q, KvPrepLaunch 
                        kp.d_model, kp.kv_dim);
     if (!(kp.head_dim == 64 || kp.head_dim == 128))
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv + KvPrepFused supports head_dim 64 or 128, got %u", kp.head_dim);
-    if (Q.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : FA_GEMM_MIN_M_DEFAULT)) {  // the row count from which fa_launch_fused_qkv takes the GEMM
+    // (a chunk that the one-launch weight stream for up to 32 rows takes goes the way of the few rows below: two launches
+    // where the GEMM with its norm and finish launches takes three)
+    if (Q.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : FA_GEMM_MIN_M_DEFAULT) && !fa_qkv_rows32_takes(ctx, Q)) {  // the row count from which fa_launch_fused_qkv takes the GEMM
         QkvRopeLaunch R;
         R.cos_t = K.cos_t, R.sin_t = K.sin_t, R.q_rot = K.q_rot, R.k_cache = K.k_cache, R.v_cache = K.v_cache;
         R.block_table = K.mode == 1 ? K.block_table : nullptr;

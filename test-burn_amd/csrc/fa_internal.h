@@ -63,6 +63,7 @@ struct fa_ctx {
     uint32_t decode_waves = 0;     // waves per decode workgroup: 0 = by launch size, 4 or 8
     uint32_t gemm_variant = 0;     // GEMM kernel: 0 = auto, 1 = tiles through registers, 2 / 3 = straight into LDS in steps of 64 / 32 features
     uint32_t gemm_min_m = 0;       // FusedQkv / MatMul: input rows from which the GEMM runs (0 = default)
+    uint32_t qkv_rows32_min_m = 0;  // FusedQkv / MatMul: from this many input rows (up to 32) the one-launch weight stream for 32 rows; 0 = default, 33 = never
     uint32_t prefill_split_k = 0;  // 0 = auto
     uint32_t sage_fused_step = 1;  // the int8 decode step as one launch (env FOUNDRY_ATTN_SAGE_FUSED=0: append kernel + decode kernel)
     bool prefill_chunk_off = false;  // a wait inside the short-chunk prefill kernel (or the polled decode merge) has run out: not routed to until fa_set_prefill_variant
@@ -277,6 +278,7 @@ struct FusedQkvLaunch {
 // weight_stream_only: never the GEMM (whose scratch is the context's workspace), whatever the number of input rows
 fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l, bool weight_stream_only = false);
 fa_status fa_launch_fused_qkv_gemm(fa_ctx *ctx, const FusedQkvLaunch &l);  // fa_gemm.hip: many input rows
+bool fa_qkv_rows32_takes(const fa_ctx *ctx, const FusedQkvLaunch &l);       // fa_qkv.hip: 12 to 32 input rows in one weight-stream launch
 
 fa_status fa_launch_sage_k_mean(fa_ctx *ctx, const void *k, uint32_t n_kv_heads, uint32_t capacity, uint32_t head_dim,
                                 uint32_t kv_len, float *mean_out);

@@ -376,7 +376,195 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
     }
 }
 
+// The same weight stream for 12 to 32 input rows (the reference's default prefill chunk is 32 rows): one launch where the
+// GEMM route takes three (norm, split GEMM, finish) for a launch that is still all weight stream. Differences from the
+// kernel above:
+//   * the input rows do not fit a compute unit's LDS (32 x 3072 f16 = 196 KB), and no wave needs them all: wave w
+//     multiplies its own feature blocks only (an eighth of them), so it keeps just those features of all 32 rows in registers, in
+//     the layout of the matrix instruction's second operand (XJ blocks x 2 row halves x 16 bytes per lane);
+//   * RMSNorm: every wave sums the squares of its slice per row, the eight partial sums meet in LDS, and the wave scales
+//     its slice (the norm's weights are staged in LDS once); the same roundings as above;
+//   * one workgroup per compute unit takes up to 32 weight rows as two 16-row tiles against the two 16-row halves of the
+//     input: four accumulators, and every weight of the workgroup is requested before the first is used - a fixed
+//     number of requests per wave, so that the compiler's waits are exact.
+// XJ = feature blocks per wave = k_dim / 256 (8 or 12: k_dim 2048, 3072; 16 spills); F16 weights.
+template <int XJ>
+__global__ void __launch_bounds__(QKV_NT, 1) fused_qkv_rows32_kernel(QkvDev a_by_value) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    static_assert(std::is_trivially_copyable<QkvDev>::value, "read as raw bytes from the argument block, where it is the first member");
+    const QkvDev &a = *(const QkvDev *)__builtin_amdgcn_kernarg_segment_ptr();
+    (void)a_by_value;
+    const unsigned char *const w0 = reinterpret_cast<const unsigned char *>(a.w[0]), *const w1 = reinterpret_cast<const unsigned char *>(a.w[1]),
+                        *const w2 = reinterpret_cast<const unsigned char *>(a.w[2]);
+    const uint32_t rows0 = a.rows[0], rows1 = a.rows[1], rows2 = a.rows[2];
+    const __half *const x_in = a.x, *const gamma = a.gamma;
+    const uint32_t K = a.k_dim, m_rows = a.m, rows_per_wg = a.rows_per_wg, canonical_u = a.canonical;
+    asm volatile("" ::"s"(w0), "s"(w1), "s"(w2), "s"(rows0), "s"(rows1), "s"(rows2), "s"(x_in), "s"(gamma), "s"(K), "s"(m_rows),
+                 "s"(rows_per_wg), "s"(canonical_u));
+    const bool canonical = canonical_u != 0;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, c = lane >> 4;
+    const uint32_t total_rows = rows0 + rows1 + rows2;
+    const uint32_t row_begin = blockIdx.x * rows_per_wg;
+    const uint32_t row_end = min(total_rows, row_begin + rows_per_wg);
+    if (row_begin >= row_end) return;
+    const uint32_t m0 = blockIdx.y * 32u, cols = min(32u, m_rows - m0);
+    _Float16 *g_lds = reinterpret_cast<_Float16 *>(smem);                   // [K] the norm's weights
+    float *ss_lds = reinterpret_cast<float *>(smem + (size_t)K * 2);        // [QKV_NW][32] sums of squares of the waves' slices
+    float *red = ss_lds + QKV_NW * 32;                                      // [QKV_NW][2 tiles][2 halves][16][17]
+
+    // The norm's weights (one 16-byte piece per thread and pass) and this wave's slice of the input rows, before any weight
+    // is requested: a compute unit's requests return in order.
+    constexpr int GPRE = 2;  // pieces per thread: k_dim up to 8192
+    h8_t g0[GPRE];
+#pragma unroll
+    for (int j = 0; j < GPRE; ++j) {
+        const uint32_t k8 = min((uint32_t)tid + j * QKV_NT, K / 8 - 1);
+        g0[j] = *reinterpret_cast<const h8_t *>((gamma ? gamma : x_in) + k8 * 8);
+    }
+    // Wave w takes the feature blocks 2w, 2w + 1, 2w + 16, 2w + 17, ...: adjacent pairs, so that the two requests for a
+    // pair touch the same 16 cache lines one after the other (a request of the operand's shape covers 64 bytes of each of
+    // 16 rows - half a line; with blocks w, w + 8, ... the other halves belonged to the next wave and every line came from
+    // L2 twice).
+    auto kb_of = [&](int j) __attribute__((always_inline)) -> uint32_t { return 2u * (uint32_t)wave + 16u * (uint32_t)(j >> 1) + (uint32_t)(j & 1); };
+    h8_t xs[XJ][2];
+#pragma unroll
+    for (int j = 0; j < XJ; ++j)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t row = min(m0 + 16u * h + (uint32_t)n, m_rows - 1);  // (rows past the last are zeroed below)
+            xs[j][h] = *reinterpret_cast<const h8_t *>(x_in + (size_t)row * K + kb_of(j) * 32u + c * 8);
+        }
+    // Every weight of the workgroup: tile t is the weight rows row_begin + 16 t .., lane (n, c) takes features 8c .. 8c + 7
+    // of block kb for row n of the tile (a row past the workgroup's last reads the first row's block: never written).
+    h8_t wv[2][XJ];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+        const uint32_t gr = row_begin + 16u * t + (uint32_t)n;
+        uint32_t lrow = gr < row_end ? gr : row_begin;
+        int mat = 0;
+        if (lrow >= rows0) {
+            lrow -= rows0, mat = 1;
+            if (lrow >= rows1) lrow -= rows1, mat = 2;
+        }
+        const unsigned char *base = pick3(mat, w0, w1, w2);
+        const uint32_t N = pick3(mat, rows0, rows1, rows1);
+        // canonical (blocked by 32 features): (k % 32) + 32 * (row + (k / 32) * N); row-major: row * K + k
+        const unsigned char *p0 = base + (canonical ? (size_t)lrow * 32 + c * 8 : (size_t)lrow * K + c * 8) * 2;
+        const size_t kb_stride = (canonical ? (size_t)N * 32 : 32) * 2;
+#pragma unroll
+        for (int j = 0; j < XJ; ++j)
+            wv[t][j] = __builtin_nontemporal_load(reinterpret_cast<const h8_t *>(p0 + (size_t)kb_of(j) * kb_stride));
+    }
+    const float eps = a.eps;
+    if (gamma) {
+#pragma unroll
+        for (int j = 0; j < GPRE; ++j) {
+            const uint32_t k8 = (uint32_t)tid + j * QKV_NT;
+            if (k8 < K / 8) *reinterpret_cast<h8_t *>(g_lds + k8 * 8) = g0[j];
+        }
+        // sums of squares of the slice, per input row: over the blocks, then over the four lanes that share a row
+        float ss[2] = {0.0f, 0.0f};
+#pragma unroll
+        for (int j = 0; j < XJ; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) ss[h] += (float)xs[j][h][i] * (float)xs[j][h][i];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            ss[h] += __shfl_xor(ss[h], 16, 64);
+            ss[h] += __shfl_xor(ss[h], 32, 64);
+            if (c == 0) ss_lds[wave * 32 + 16 * h + n] = ss[h];
+        }
+        __syncthreads();
+        float inv_rms[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            float tot = 0.0f;
+#pragma unroll
+            for (int w = 0; w < QKV_NW; ++w) tot += ss_lds[w * 32 + 16 * h + n];
+            inv_rms[h] = rsqrtf(tot / (float)K + eps);
+        }
+#pragma unroll
+        for (int j = 0; j < XJ; ++j) {
+            const h8_t g = *reinterpret_cast<const h8_t *>(g_lds + kb_of(j) * 32u + c * 8);
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) xs[j][h][i] = (_Float16)(((float)xs[j][h][i] * inv_rms[h]) * (float)g[i]);
+        }
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+        if (16u * h + (uint32_t)n >= cols) {
+#pragma unroll
+            for (int j = 0; j < XJ; ++j) xs[j][h] = h8_t{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    // what the write stage takes, while the weights are on their way
+    const __half *const residual = a.residual;
+    const __half *const bias0 = a.bias[0], *const bias1 = a.bias[1], *const bias2 = a.bias[2];
+    __half *const out0 = a.out[0], *const out1 = a.out[1], *const out2 = a.out[2];
+    const float alpha = a.alpha, beta = a.beta;
+    asm volatile("" ::"s"(residual), "s"(bias0), "s"(bias1), "s"(bias2), "s"(out0), "s"(out1), "s"(out2), "s"(alpha), "s"(beta));
+
+    f4v_t d[2][2] = {{{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}}, {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}}};
+#pragma unroll
+    for (int j = 0; j < XJ; ++j)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) d[t][h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv[t][j], xs[j][h], d[t][h], 0, 0, 0);
+    // The eight waves' partial tiles are summed in wave order, the write stage applied, rows rounded once.
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) red[((((size_t)wave * 2 + t) * 2 + h) * 16 + c * 4 + i) * 17 + n] = d[t][h][i];
+    __syncthreads();
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+        const int o = tid + pass * QKV_NT;  // (tile, weight row of the tile, input row)
+        const int t = o >> 9, row = (o >> 5) & 15, col = o & 31, h = col >> 4, cn = col & 15;
+        const uint32_t gr = row_begin + 16u * t + (uint32_t)row;
+        if (gr < row_end && (uint32_t)col < cols) {
+            float s = 0.0f;
+#pragma unroll
+            for (int w = 0; w < QKV_NW; ++w) s += red[((((size_t)w * 2 + t) * 2 + h) * 16 + row) * 17 + cn];
+            uint32_t lrow = gr;
+            int mat = 0;
+            if (lrow >= rows0) {
+                lrow -= rows0, mat = 1;
+                if (lrow >= rows1) lrow -= rows1, mat = 2;
+            }
+            const __half *bias = pick3(mat, bias0, bias1, bias2);
+            __half *out = pick3(mat, out0, out1, out2);
+            const uint32_t N = pick3(mat, rows0, rows1, rows1);
+            s *= alpha;
+            if (bias) s += __half2float(bias[lrow]);
+            if (residual) s += __half2float(residual[(size_t)(m0 + col) * N + lrow]) * beta;
+            out[(size_t)(m0 + col) * N + lrow] = __float2half(s);
+        }
+    }
+}
+
 }  // namespace
+
+// Whether a FusedQkv / MatMul launch goes to the one-launch kernel for 12 to 32 input rows: F16 weights, k_dim 2048 or 3072
+// (at 4096 a wave's slice and its weights no longer fit the registers), at most 32 weight rows per compute unit; an explicit
+// GEMM threshold (fa_set_gemm_min_m) wins.
+bool fa_qkv_rows32_takes(const fa_ctx *ctx, const FusedQkvLaunch &l) {
+    constexpr uint32_t ROWS32_MIN_M_DEFAULT = 12;
+    auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
+    const uint32_t total_rows = l.n_dim + 2 * l.n_kv;
+    const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
+    const uint32_t xj = l.k_dim / 256, rpw = ceil_div_u32(total_rows, n_cus);
+    const uint32_t min_m = ctx->qkv_rows32_min_m ? ctx->qkv_rows32_min_m : ROWS32_MIN_M_DEFAULT;
+    return l.scales[0] == nullptr && l.weight_bits == 16 && l.k_dim % 256 == 0 && (xj == 8 || xj == 12) && rpw <= 32 && l.m >= min_m &&
+           l.m <= 32 && !(ctx->gemm_min_m && l.m >= ctx->gemm_min_m) && aligned16(l.x) && aligned16(l.w[0]) && aligned16(l.w[1]) &&
+           aligned16(l.w[2]) && aligned16(l.gamma);
+}
 
 fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l, bool weight_stream_only) {
     QkvDev a;
@@ -396,9 +584,24 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l, bool weight_
     auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
     const bool gemm_ok = l.k_dim % (q8 ? 32 : 8) == 0 && aligned16(l.x) && aligned16(l.w[0]) && aligned16(l.w[1]) &&
                          aligned16(l.w[2]) && aligned16(l.gamma);
-    if (!weight_stream_only && gemm_ok && l.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : GEMM_MIN_M_DEFAULT)) return fa_launch_fused_qkv_gemm(ctx, l);
     const uint32_t total_rows = l.n_dim + 2 * l.n_kv;
     const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
+    // A chunk of up to 32 input rows (the reference's default prefill chunk) is still a weight stream: one launch of the
+    // kernel that keeps each wave's slice of the input rows in registers, where the GEMM route takes three launches.
+    {
+        const uint32_t xj = l.k_dim / 256, rpw = ceil_div_u32(total_rows, n_cus);
+        const bool ok = fa_qkv_rows32_takes(ctx, l);
+        if (ok) {
+            a.rows_per_wg = rpw, a.cols_per_pass = 32, a.x_stride = 0;
+            const size_t lds = (size_t)l.k_dim * 2 + (size_t)QKV_NW * 32 * sizeof(float) + (size_t)QKV_NW * 2 * 2 * 16 * 17 * sizeof(float);
+            const dim3 grid(ceil_div_u32(total_rows, rpw), 1);
+            FaLaunchScope scope(ctx, l.n_kv ? "fused_qkv_rows32_kernel" : "matmul_rows32_kernel", true);
+            if (xj == 8) scope.launch(fused_qkv_rows32_kernel<8>, grid, dim3(QKV_NT), lds, a);
+            else scope.launch(fused_qkv_rows32_kernel<12>, grid, dim3(QKV_NT), lds, a);
+            return scope.finish();
+        }
+    }
+    if (!weight_stream_only && gemm_ok && l.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : GEMM_MIN_M_DEFAULT)) return fa_launch_fused_qkv_gemm(ctx, l);
     // Workgroups: a multiple of the CU count, enough of them that a workgroup's rows fit one 16-row tile where the
     // matrix allows (5120 rows, 256 CUs: 512 workgroups of 10 rows, two resident per CU - every CU requests the same
     // bytes, and all of a wave's blocks are in flight at once); at most 64 rows (4 tiles) per workgroup. Measured on

@@ -185,6 +185,84 @@ def test_fused_qkv_errors():
         z.free()
 
 
+@pytest.mark.parametrize("K,N,NK,m,norm,bias,layout", [
+    (3072, 3072, 1024, 32, True, False, 1),   # Llama-3.2-3B, the reference's default prefill chunk
+    (3072, 3072, 1024, 17, True, True, 0),    # row-major weights, a ragged second half of the input rows
+    (2048, 2048, 256, 12, False, True, 1),    # no RMSNorm, the fewest rows the kernel takes by default
+    (2048, 3000, 40, 31, True, True, 1),      # weight rows that do not fill the workgroups' tiles, tiles across the matrices
+])
+def test_fused_qkv_chunk_of_up_to_32_rows_in_one_launch(K, N, NK, m, norm, bias, layout):
+    """12 to 32 input rows against F16 weights of 2048 or 3072 features run as ONE weight-stream launch (each wave keeps
+    its slice of the input rows in registers); an explicit GEMM threshold sends the same call through the GEMM. Both
+    against the oracle, and the profiler's launch counts say which kernel ran."""
+    announce("fused qkv, chunk in one launch", K, N, NK, m, norm, bias, layout)
+    f = ctx()
+    rng = np.random.default_rng(K + N + m + 7)
+    x, g, ws, bs = _data(rng, K, N, NK, m)
+    want = orc.fused_qkv(x, *ws, gamma=g if norm else None, biases=bs if bias else None, layout=0)
+    dev_w = [f.array(orc.to_canonical(w) if layout == 1 else w.reshape(-1)) for w in ws]
+    dx, dg = f.array(x), f.array(g)
+    db = [f.array(b) for b in bs]
+    outs = [f.zeros((m, n)) for n in (N, NK, NK)]
+    try:
+        for min_m, kernel in ((0, "fused_qkv_rows32_kernel"), (12, "fused_qkv_gemm_kernel")):
+            f.set_gemm_min_m(min_m)
+            for o in outs:
+                o.upload(np.zeros(o.shape, np.float16))
+            f.profile_reset()
+            f.profile_enable(True)
+            f.fused_qkv(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), outs[0].arg(), outs[1].arg(), outs[2].arg(),
+                        K, N, NK, m, gamma=dg.arg() if norm else None, biases=[b.arg() for b in db] if bias else None, layout=layout)
+            f.synchronize()
+            assert f.profile_query(kernel)[0] == 1, (kernel, min_m)
+            f.profile_enable(False)
+            for o, w, name in zip(outs, want, "qkv"):
+                got = o.download()
+                assert np.all(np.isfinite(got)), (name, min_m)
+                assert _close(got, w, K), (name, min_m, float(np.max(np.abs(got.astype(np.float64) - w.astype(np.float64)))))
+    finally:
+        f.profile_enable(False)
+        f.set_gemm_min_m()
+    for b in dev_w + [dx, dg] + db + outs:
+        b.free()
+
+
+@pytest.mark.parametrize("m,n,k,canonical,bias,resid,alpha,beta", [
+    (32, 3072, 3072, True, False, True, 1.0, 1.0),    # Llama-3.2-3B o_proj of a default prefill chunk
+    (20, 2048, 2048, False, True, True, 0.25, 0.75),  # row-major weights, bias, scaled residual
+])
+def test_matmul_chunk_of_up_to_32_rows_in_one_launch(m, n, k, canonical, bias, resid, alpha, beta):
+    announce("matmul, chunk in one launch", m, n, k, canonical, bias, resid, alpha, beta)
+    f = ctx()
+    rng = np.random.default_rng(m + n + k + 7)
+    x = rng.uniform(-1, 1, (m, k)).astype(np.float16)
+    w = rng.uniform(-0.1, 0.1, (n, k)).astype(np.float16)
+    b = rng.uniform(-0.1, 0.1, n).astype(np.float16)
+    c = rng.uniform(-1, 1, (m, n)).astype(np.float16)
+    want = orc.matmul_gemv(x, w, b if bias else None, c if resid else None, 0, 32, alpha, beta)
+    dx, dw = f.array(x), f.array(orc.to_canonical(w) if canonical else w.reshape(-1))
+    db, dc, out = f.array(b), f.array(c), f.zeros((m, n))
+    try:
+        for min_m, kernel in ((0, "matmul_rows32_kernel"), (12, None)):
+            f.set_gemm_min_m(min_m)
+            out.upload(np.zeros((m, n), np.float16))
+            f.profile_reset()
+            f.profile_enable(True)
+            f.matmul(dx.arg(), dw.arg(), out.arg(), m, n, k, bias=db.arg() if bias else None, c=dc.arg() if resid else None,
+                     transpose_b=not canonical, alpha=alpha, beta=beta)
+            f.synchronize()
+            assert f.profile_query("matmul_rows32_kernel")[0] == (1 if kernel else 0), min_m
+            f.profile_enable(False)
+            got = out.download()
+            g, wv = got.astype(np.float64), want.astype(np.float64)
+            assert np.all(np.abs(g - wv) <= 2 * np.maximum(np.abs(wv), 2.0 ** -10) * 2.0 ** -10 + 1e-4), (min_m, float(np.max(np.abs(g - wv))))
+    finally:
+        f.profile_enable(False)
+        f.set_gemm_min_m()
+    for z in (dx, dw, db, dc, out):
+        z.free()
+
+
 # ---------------------------------------------------------------- MatMul (the o_proj consumer of attn_out)
 
 @pytest.mark.parametrize("m,n,k,canonical,bias,resid,alpha,beta", [

@@ -21,7 +21,10 @@ def _paths(m):
     if m < 12:
         return [(0, 0), (1, 0), (1, 1)]
     if m <= 64:
-        return [(0, 0), (0, 1), (0, 2), (0, 3), (1 << 30, 0)]
+        paths = [(0, 0), (0, 1), (0, 2), (0, 3), (1 << 30, 0)]
+        if 12 <= m <= 32:  # an explicit threshold: the GEMM also where the one-launch kernel for up to 32 rows takes the chunk
+            paths += [(12, 0), (12, 1), (12, 2), (12, 3)]
+        return paths
     return [(0, 0), (0, 1), (0, 2), (0, 3)]
 
 
