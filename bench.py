@@ -827,6 +827,69 @@ def bench_attn_block(f, args):
         "parity": {"outputs_finite": finite, "note": "stage-by-stage parity of this chain: tests/test_gpu_block.py"}}))
 
 
+def bench_chunk_block(f, args, m=32, prefix=8160):
+    """The attention block of the reference's default prefill mode: a chunk of m = 32 rows (src/model/executor.rs:232-250)
+    after `prefix` cached tokens goes through all 28 layers of a Llama-3.2-3B-shaped model - FusedQkv + KvPrepFused (one
+    op: RMSNorm, projections, RoPE, append of the chunk's rows), causal FlashAttention of the chunk against the prefix and
+    itself, o_proj MatMul with residual - as ONE HIP graph per step; F16 canonical weights, distinct buffers per layer.
+    The MLP between the blocks is not part of this path. HBM-bound: a layer reads its weights and the prefix once."""
+    L, H, Hkv, D = 28, 24, 8, 128
+    dm, kvd = H * D, Hkv * D
+    N, cap = prefix + m, prefix + 512
+    rng = np.random.default_rng(0xF0DD + 16)
+    cos, sin = fa.rope_tables(5e5, D, cap)
+    dcos, dsin = f.array(cos), f.array(sin)
+    base_kv = rng.standard_normal((Hkv, cap, D), dtype=np.float32).astype(np.float16)
+    wq = fa.canonical_layout(rng.uniform(-0.05, 0.05, (dm, dm)).astype(np.float16))
+    wk = fa.canonical_layout(rng.uniform(-0.05, 0.05, (kvd, dm)).astype(np.float16))
+    layers = []
+    for i in range(L):  # distinct device buffers per layer (contents rolled copies: only the addresses matter for timing)
+        layers.append(dict(kc=f.array(np.roll(base_kv, i, axis=1)), vc=f.array(np.roll(base_kv, i + 3, axis=1)),
+                           wq=f.array(np.roll(wq, i)), wk=f.array(np.roll(wk, i)), wv=f.array(np.roll(wk, i + 5)),
+                           wo=f.array(np.roll(wq, i + 9)), g=f.array(rng.uniform(0.5, 1.5, dm).astype(np.float16))))
+    hid = [f.array(rng.uniform(-1, 1, (m, dm)).astype(np.float16)), f.zeros((m, dm))]
+    dqr, dattn = f.zeros((H, m, D)), f.zeros((m, dm))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, m, prefix, cap, fa.ROPE_NORMAL)
+
+    def enqueue():
+        for i, ly in enumerate(layers):
+            src, dst = hid[i % 2], hid[(i + 1) % 2]
+            f.fused_qkv_kv_prep(src.arg(), ly["wq"].arg(), ly["wk"].arg(), ly["wv"].arg(), dm, dqr.arg(), dcos.arg(), dsin.arg(), p,
+                                k_cache=ly["kc"].arg(), v_cache=ly["vc"].arg(), gamma=ly["g"].arg())
+            f.flash_attention(dqr.arg(), ly["kc"].arg(), ly["vc"].arg(), dattn.arg(), True, prefix, H, D, N, m)
+            f.matmul(dattn.arg(), ly["wo"].arg(), dst.arg(), m, dm, dm, c=src.arg(), transpose_b=False, alpha=1.0, beta=1.0)
+
+    enqueue()  # (workspaces reach their size before the capture)
+    f.synchronize()
+    f.start_capture()
+    enqueue()
+    graph = f.end_capture()
+    for _ in range(max(args.warmup, 1)):
+        graph.launch()
+    f.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graph.launch()
+    f.synchronize()
+    dt = time.perf_counter() - t0
+    graph.destroy()
+    finite = bool(np.all(np.isfinite(hid[0].download())))
+    nbytes = L * (2.0 * (dm + 2 * kvd) * dm + 2.0 * dm * dm + 2.0 * 2 * Hkv * N * D + 4.0 * 2 * m * dm)
+    per_step = dt / args.steps
+    emit(({
+        "metric": "prefill-chunk attention-block steps/s + achieved HBM GB/s, Llama-3.2-3B, %d rows after %d tokens" % (m, prefix),
+        "value": 1.0 / per_step, "unit": "steps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": per_step * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "llama3.2-3b attention block x 28 layers per step on a prefill chunk of %d rows after %d tokens: "
+                               "FusedQkv + KvPrepFused (one op), causal FlashAttention, o_proj with residual; one HIP graph per step"
+                               % (m, prefix)},
+        "roofline": {"bound": "hbm", "achieved": nbytes / per_step / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": nbytes / per_step / 1e9 / HBM_PEAK_GBPS, "traffic": None, "kernel": "whole step (the launches of 28 layers)",
+                     "bytes_per_step": nbytes, "us_per_layer": per_step * 1e6 / L},
+        "parity": {"outputs_finite": finite, "note": "stage-by-stage parity of these ops: tests/test_gpu_qkv_kv_prep.py, tests/test_gpu_prefill.py, tests/test_gpu_qkv.py"}}))
+
+
 def bench_prefill_chunk(f, args, m=32, prefix=8160):
     """One prefill chunk of m rows (32 = the reference's default chunk, src/model/executor.rs:232-250) attending a contiguous
     Llama-3.2-3B-shaped cache that already holds `prefix` tokens: the short-chunk kernel (partitions merged inside the
@@ -1346,7 +1409,7 @@ def bench_floors(f, args):
     emit(out)
 
 
-SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_chunk32_8k": bench_prefill_chunk, "llama3b_prefill_chunk32_32k": lambda f, args: bench_prefill_chunk(f, args, 32, 32736), "llama3b_prefill_chunk64_8k": lambda f, args: bench_prefill_chunk(f, args, 64, 8128), "timeline_decode_8k": bench_phase_timeline, "timeline_decode_1k": lambda f, args: bench_phase_timeline(f, args, "decode_1k"), "timeline_sage_32k": lambda f, args: bench_phase_timeline(f, args, "sage_32k"), "timeline_chunk32_8k": lambda f, args: bench_phase_timeline(f, args, "chunk32_8k"), "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_decode_64k": lambda f, args: bench_long_decode(f, args, 65536), "llama3b_decode_32k": lambda f, args: bench_long_decode(f, args, 32768), "llama3b_decode_2k": bench_short_decode, "llama3b_decode_512": lambda f, args: bench_short_decode(f, args, 511), "llama3b_prefill_2k": bench_prefill,
+SECONDARY = {"floors": bench_floors, "llama3b_attn_block": bench_attn_block, "llama3b_chunk_block": bench_chunk_block, "llama3b_prefill_block": bench_prefill_block, "llama3b_prefill_chunk32_8k": bench_prefill_chunk, "llama3b_prefill_chunk32_32k": lambda f, args: bench_prefill_chunk(f, args, 32, 32736), "llama3b_prefill_chunk64_8k": lambda f, args: bench_prefill_chunk(f, args, 64, 8128), "timeline_decode_8k": bench_phase_timeline, "timeline_decode_1k": lambda f, args: bench_phase_timeline(f, args, "decode_1k"), "timeline_sage_32k": lambda f, args: bench_phase_timeline(f, args, "sage_32k"), "timeline_chunk32_8k": lambda f, args: bench_phase_timeline(f, args, "chunk32_8k"), "llama3b_prefill_block_fused": lambda f, args: bench_prefill_block(f, args, fused=True), "llama3b_decode_128k": bench_long_decode, "llama3b_decode_64k": lambda f, args: bench_long_decode(f, args, 65536), "llama3b_decode_32k": lambda f, args: bench_long_decode(f, args, 32768), "llama3b_decode_2k": bench_short_decode, "llama3b_decode_512": lambda f, args: bench_short_decode(f, args, 511), "llama3b_prefill_2k": bench_prefill,
              "llama3b_prefill_8k": lambda f, args: bench_prefill(f, args, 8192), "qwen05b_decode_1k": bench_small_decode,
              "qwen3b_paged_decode": bench_paged_decode, "smollm3_sage_decode_32k": bench_sage_decode,
              "llama3b_kv_growth": bench_kv_growth, "llama3b_fused_qkv": bench_fused_qkv,

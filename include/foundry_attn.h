@@ -482,10 +482,12 @@ fa_status fa_fused_qkv(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_ar
  * by fa_kv_prep_fused on the same context: every projection is rounded to f16 as FusedQkv stores it, then rotated and
  * placed as KvPrepFused does. qkv_params->m must equal params->seq_len, n_dim = params->d_model, n_kv = params->kv_dim;
  * head_dim 64 or 128; f16 only; q_rot, caches / pools, biases and tables 16-byte aligned. From fa_set_gemm_min_m() rows
- * on it is the GEMM's write stage (no q / k / v round trip, one launch fewer); with fewer rows - and for a chunk that
- * the one-launch weight stream for up to 32 rows takes (see fa_matmul) - the weight-stream
- * kernel writes q, k, v into the context's workspace and the KvPrepFused kernel follows (m = 1 belongs to
- * fa_decode_step_fused, which takes the raw projections). Workspace rule under capture as for fa_fused_qkv. */
+ * on it is the GEMM's write stage (no q / k / v round trip, one launch fewer); a chunk that the one-launch weight stream
+ * for up to 32 rows takes (see fa_matmul; the reference's default prefill chunk) has it as that kernel's write stage: the
+ * whole op is ONE launch (environment FOUNDRY_ATTN_QKV_ROWS32_ROPE=0, read at fa_ctx_create: two launches as below); with
+ * fewer rows the weight-stream kernel writes q, k, v into the context's workspace and the KvPrepFused kernel follows
+ * (m = 1 belongs to fa_decode_step_fused, which takes the raw projections). Workspace rule under capture as for
+ * fa_fused_qkv. */
 fa_status fa_fused_qkv_kv_prep(fa_ctx *ctx, const fa_tensor_arg *w_q, const fa_tensor_arg *s_q, const fa_tensor_arg *w_k,
                                const fa_tensor_arg *s_k, const fa_tensor_arg *w_v, const fa_tensor_arg *s_v,
                                const fa_tensor_arg *input, const fa_tensor_arg *bias_q, const fa_tensor_arg *bias_k,

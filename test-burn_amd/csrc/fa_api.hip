@@ -121,6 +121,7 @@ extern "C" fa_status fa_ctx_create(int device, fa_ctx **out) {
     if (ctx->decode_waves != 4 && ctx->decode_waves != 8) ctx->decode_waves = 0;
     ctx->gemm_min_m = env_u32("FOUNDRY_ATTN_GEMM_MIN_M", 0);
     ctx->qkv_rows32_min_m = env_u32("FOUNDRY_ATTN_QKV_ROWS32_MIN_M", 0);
+    ctx->qkv_rows32_rope = env_u32("FOUNDRY_ATTN_QKV_ROWS32_ROPE", 1) != 0;
     ctx->gemm_variant = env_u32("FOUNDRY_ATTN_GEMM_VARIANT", 0);
     if (ctx->gemm_variant > 3) ctx->gemm_variant = 0;
     ctx->prefill_split_k = env_u32("FOUNDRY_ATTN_PREFILL_SPLIT_K", 0);
@@ -1051,9 +1052,10 @@ static fa_status fused_qkv_kv_prep(fa_ctx *ctx, FusedQkvLaunch &Q, KvPrepLaunch 
                        kp.d_model, kp.kv_dim);
     if (!(kp.head_dim == 64 || kp.head_dim == 128))
         return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv + KvPrepFused supports head_dim 64 or 128, got %u", kp.head_dim);
-    // (a chunk that the one-launch weight stream for up to 32 rows takes goes the way of the few rows below: two launches
-    // where the GEMM with its norm and finish launches takes three)
-    if (Q.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : FA_GEMM_MIN_M_DEFAULT) && !fa_qkv_rows32_takes(ctx, Q)) {  // the row count from which fa_launch_fused_qkv takes the GEMM
+    // A chunk that the one-launch weight stream for up to 32 rows takes does the KvPrepFused work in that kernel's write
+    // stage (FOUNDRY_ATTN_QKV_ROWS32_ROPE=0: as two launches, like the few rows below); from gemm_min_m rows on, the GEMM's.
+    const bool rows32 = fa_qkv_rows32_takes(ctx, Q);
+    if ((rows32 && ctx->qkv_rows32_rope) || (!rows32 && Q.m >= (ctx->gemm_min_m ? ctx->gemm_min_m : FA_GEMM_MIN_M_DEFAULT))) {
         QkvRopeLaunch R;
         R.cos_t = K.cos_t, R.sin_t = K.sin_t, R.q_rot = K.q_rot, R.k_cache = K.k_cache, R.v_cache = K.v_cache;
         R.block_table = K.mode == 1 ? K.block_table : nullptr;
@@ -1061,7 +1063,7 @@ static fa_status fused_qkv_kv_prep(fa_ctx *ctx, FusedQkvLaunch &Q, KvPrepLaunch 
         R.max_seq_len = kp.max_seq_len, R.block_size = K.block_size, R.capacity = K.capacity, R.table_rows = K.table_rows;
         R.rope_normal = kp.rope_mode == FA_ROPE_MODE_NORMAL;
         R.apply_rope = kp.no_rope_layer_step == 0 || ((kp.layer_idx + 1u) % kp.no_rope_layer_step) != 0u;
-        return fa_launch_fused_qkv_gemm_rope(ctx, Q, R);
+        return rows32 ? fa_launch_fused_qkv_rows32_rope(ctx, Q, R) : fa_launch_fused_qkv_gemm_rope(ctx, Q, R);
     }
     const size_t nq = ((size_t)Q.m * Q.n_dim * sizeof(__half) + 255) & ~(size_t)255;
     const size_t nkv = ((size_t)Q.m * Q.n_kv * sizeof(__half) + 255) & ~(size_t)255;

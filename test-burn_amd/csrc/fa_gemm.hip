@@ -47,13 +47,6 @@ typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef float f4v_t __attribute__((ext_vector_type(4)));
 typedef float f16v_t __attribute__((ext_vector_type(16)));
 
-// KvPrepFused as the write stage (kv_prep_fused.metal:45-122): out[0] is q_rot [H, m, D], out[1] / out[2] the K / V cache.
-struct RopeDev {
-    const __half *cos_t, *sin_t;
-    const int32_t *block_table;  // paged: the sequence's table row
-    uint32_t on, head_dim, n_kv_heads, position_offset, max_seq_len, block_size, capacity, table_rows, normal, apply;
-};
-
 struct GemmDev {
     const void *w[3];       // f16, or int8 (Q8_0) / nibbles (Q4_0) in the same element order
     const __half *scales[3];  // Q8_0: f16 [rows, k_dim / 32] per matrix
@@ -71,13 +64,6 @@ struct GemmDev {
     float *partial;
     RopeDev rope;
 };
-
-// Rotation of one element: products and sum rounded separately (kv_prep_fused.metal:74-82), as fa_kvprep.hip.
-__device__ __forceinline__ float rope_one(float x, float mate, float c, float s, bool first) {
-#pragma clang fp contract(off)
-    const float p0 = x * c, p1 = mate * s;
-    return first ? p0 - p1 : p0 + p1;
-}
 
 // Write stage of one piece: y = the projections of token gm, columns gn .. gn + 7 of matrix mat (0 Q, 1 K, 2 V),
 // already rounded to f16 as FusedQkv stores them; mate = the piece half a head away (NeoX pairing; unused otherwise).

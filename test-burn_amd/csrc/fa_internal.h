@@ -64,6 +64,7 @@ struct fa_ctx {
     uint32_t gemm_variant = 0;     // GEMM kernel: 0 = auto, 1 = tiles through registers, 2 / 3 = straight into LDS in steps of 64 / 32 features
     uint32_t gemm_min_m = 0;       // FusedQkv / MatMul: input rows from which the GEMM runs (0 = default)
     uint32_t qkv_rows32_min_m = 0;  // FusedQkv / MatMul: from this many input rows (up to 32) the one-launch weight stream for 32 rows; 0 = default, 33 = never
+    bool qkv_rows32_rope = true;    // FusedQkv + KvPrepFused of such a chunk: the KvPrepFused work in that launch's write stage (false: a second launch)
     uint32_t prefill_split_k = 0;  // 0 = auto
     uint32_t sage_fused_step = 1;  // the int8 decode step as one launch (env FOUNDRY_ATTN_SAGE_FUSED=0: append kernel + decode kernel)
     bool prefill_chunk_off = false;  // a wait inside the short-chunk prefill kernel (or the polled decode merge) has run out: not routed to until fa_set_prefill_variant

@@ -388,11 +388,20 @@ __global__ void __launch_bounds__(QKV_NT, 2) fused_qkv_kernel(QkvDev a_by_value)
 //     input: four accumulators, and every weight of the workgroup is requested before the first is used - a fixed
 //     number of requests per wave, so that the compiler's waits are exact.
 // XJ = feature blocks per wave = k_dim / 256 (8 or 12: k_dim 2048, 3072; 16 spills); F16 weights.
-template <int XJ>
-__global__ void __launch_bounds__(QKV_NT, 1) fused_qkv_rows32_kernel(QkvDev a_by_value) {
+// ROPE: the write stage is KvPrepFused (kv_prep_fused.metal:45-122) on the f16 values FusedQkv would store - rotation of Q
+// and K, Q to q_rot [H, m, D], K and V to their cache rows. A workgroup then takes whole rotation pairs: adjacent weight
+// rows (2i, 2i + 1), or - NeoX pairing - tile 0 = the rows of up to 16 pairs in the first half of a head and tile 1 = their
+// mates half a head on, so that the thread that stores an element finds its mate in the workgroup's own partial sums.
+struct Rows32Dev {
+    QkvDev q;
+    RopeDev r;
+};
+template <int XJ, bool ROPE>
+__global__ void __launch_bounds__(QKV_NT, 1) fused_qkv_rows32_kernel(Rows32Dev a_by_value) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    static_assert(std::is_trivially_copyable<QkvDev>::value, "read as raw bytes from the argument block, where it is the first member");
-    const QkvDev &a = *(const QkvDev *)__builtin_amdgcn_kernarg_segment_ptr();
+    static_assert(std::is_trivially_copyable<Rows32Dev>::value, "read as raw bytes from the argument block, where it is the first member");
+    const Rows32Dev &args = *(const Rows32Dev *)__builtin_amdgcn_kernarg_segment_ptr();
+    const QkvDev &a = args.q;
     (void)a_by_value;
     const unsigned char *const w0 = reinterpret_cast<const unsigned char *>(a.w[0]), *const w1 = reinterpret_cast<const unsigned char *>(a.w[1]),
                         *const w2 = reinterpret_cast<const unsigned char *>(a.w[2]);
@@ -409,6 +418,26 @@ __global__ void __launch_bounds__(QKV_NT, 1) fused_qkv_rows32_kernel(QkvDev a_by
     const uint32_t row_end = min(total_rows, row_begin + rows_per_wg);
     if (row_begin >= row_end) return;
     const uint32_t m0 = blockIdx.y * 32u, cols = min(32u, m_rows - m0);
+    // ROPE (rows_per_wg is even, the matrices hold whole heads): the pairing and the head size
+    uint32_t neox = 0, half_shift = 0, pair_begin = 0, pair_end = 0;
+    if constexpr (ROPE) {
+        const uint32_t normal = args.r.normal, head_dim = args.r.head_dim;
+        asm volatile("" ::"s"(normal), "s"(head_dim));
+        neox = normal ? 0u : 1u, half_shift = head_dim == 128 ? 6u : 5u;
+        pair_begin = row_begin >> 1, pair_end = row_end >> 1;
+    }
+    // Weight row of slot (tile t, row n of the tile) across the three matrices laid end to end; a slot past the workgroup's
+    // last row gives the workgroup's first row with valid = false.
+    auto slot_row = [&](uint32_t t, uint32_t n_, bool &valid) __attribute__((always_inline)) -> uint32_t {
+        if (ROPE && neox) {
+            const uint32_t p = pair_begin + n_, pv = p < pair_end ? p : pair_begin;
+            valid = p < pair_end;
+            return ((pv >> half_shift) << (half_shift + 1)) + (pv & ((1u << half_shift) - 1u)) + (t << half_shift);
+        }
+        const uint32_t gr = row_begin + 16u * t + n_;
+        valid = gr < row_end;
+        return valid ? gr : row_begin;
+    };
     _Float16 *g_lds = reinterpret_cast<_Float16 *>(smem);                   // [K] the norm's weights
     float *ss_lds = reinterpret_cast<float *>(smem + (size_t)K * 2);        // [QKV_NW][32] sums of squares of the waves' slices
     float *red = ss_lds + QKV_NW * 32;                                      // [QKV_NW][2 tiles][2 halves][16][17]
@@ -440,8 +469,8 @@ __global__ void __launch_bounds__(QKV_NT, 1) fused_qkv_rows32_kernel(QkvDev a_by
     h8_t wv[2][XJ];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-        const uint32_t gr = row_begin + 16u * t + (uint32_t)n;
-        uint32_t lrow = gr < row_end ? gr : row_begin;
+        bool slot_valid;
+        uint32_t lrow = slot_row((uint32_t)t, (uint32_t)n, slot_valid);
         int mat = 0;
         if (lrow >= rows0) {
             lrow -= rows0, mat = 1;
@@ -507,6 +536,36 @@ __global__ void __launch_bounds__(QKV_NT, 1) fused_qkv_rows32_kernel(QkvDev a_by
     __half *const out0 = a.out[0], *const out1 = a.out[1], *const out2 = a.out[2];
     const float alpha = a.alpha, beta = a.beta;
     asm volatile("" ::"s"(residual), "s"(bias0), "s"(bias1), "s"(bias2), "s"(out0), "s"(out1), "s"(out2), "s"(alpha), "s"(beta));
+    // ROPE: thread (row = tid % 16, col = tid / 16) stores the elements of slot row of both tiles for input row col, rows
+    // fastest (the lanes of a store cover consecutive elements of a head). Its two table entries and, in a paged cache, its
+    // block are requested here, behind the weights, from addresses that are valid whatever the slot.
+    const uint32_t w_row = (uint32_t)tid & 15u, w_col = (uint32_t)tid >> 4;
+    _Float16 rc[2] = {(_Float16)0.0f, (_Float16)0.0f}, rs[2] = {(_Float16)0.0f, (_Float16)0.0f};
+    uint32_t r_pos = 0, r_blk = 0;
+    uint32_t n_kv_heads = 0, max_seq_len = 0, block_size = 1, capacity = 0, apply = 0;
+    bool paged = false;
+    if constexpr (ROPE) {
+        const __half *const cos_t = args.r.cos_t, *const sin_t = args.r.sin_t;
+        const int32_t *const block_table = args.r.block_table;
+        const uint32_t position_offset = args.r.position_offset, table_rows = args.r.table_rows;
+        block_size = args.r.block_size, n_kv_heads = args.r.n_kv_heads, max_seq_len = args.r.max_seq_len, capacity = args.r.capacity;
+        apply = args.r.apply;
+        asm volatile("" ::"s"(cos_t), "s"(sin_t), "s"(block_table), "s"(position_offset), "s"(table_rows), "s"(block_size), "s"(n_kv_heads),
+                     "s"(max_seq_len), "s"(capacity), "s"(apply));
+        paged = block_table != nullptr;
+        r_pos = position_offset + m0 + min(w_col, cols - 1u);
+        const uint32_t tp = min(r_pos, table_rows - 1u);  // stay inside the tables
+        const uint32_t hmask = (1u << half_shift) - 1u;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            bool v_;
+            const uint32_t hd = slot_row((uint32_t)t, w_row, v_) & (2u * hmask + 1u);
+            const uint32_t tc = neox ? (hd & hmask) : (hd >> 1);
+            rc[t] = *reinterpret_cast<const _Float16 *>(cos_t + ((size_t)tp << half_shift) + tc);
+            rs[t] = *reinterpret_cast<const _Float16 *>(sin_t + ((size_t)tp << half_shift) + tc);
+        }
+        if (block_table) r_blk = (uint32_t)block_table[r_pos / block_size];
+    }
 
     f4v_t d[2][2] = {{{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}}, {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}}};
 #pragma unroll
@@ -523,10 +582,63 @@ __global__ void __launch_bounds__(QKV_NT, 1) fused_qkv_rows32_kernel(QkvDev a_by
 #pragma unroll
             for (int i = 0; i < 4; ++i) red[((((size_t)wave * 2 + t) * 2 + h) * 16 + c * 4 + i) * 17 + n] = d[t][h][i];
     __syncthreads();
+    if constexpr (ROPE) {
+        const uint32_t D = 2u << half_shift, half = 1u << half_shift;
+        const int h = (int)(w_col >> 4), cn = (int)(w_col & 15u);
+        auto tile_sum = [&](uint32_t t, uint32_t row) __attribute__((always_inline)) -> float {
+            float s = 0.0f;
+#pragma unroll
+            for (int w = 0; w < QKV_NW; ++w) s += red[((((size_t)w * 2 + t) * 2 + h) * 16 + row) * 17 + cn];
+            return s;
+        };
+        // the f16 values FusedQkv stores, of the thread's slot in both tiles (of the workgroup's first row where the slot is
+        // past its last: every lane takes part in the exchange below)
+        _Float16 y2[2];
+        uint32_t lrow2[2];
+        int mat2[2];
+        bool valid2[2];
+#pragma unroll
+        for (uint32_t t = 0; t < 2; ++t) {
+            uint32_t lrow = slot_row(t, w_row, valid2[t]);
+            int mat = 0;
+            if (lrow >= rows0) {
+                lrow -= rows0, mat = 1;
+                if (lrow >= rows1) lrow -= rows1, mat = 2;
+            }
+            const __half *bias = pick3(mat, bias0, bias1, bias2);
+            float s = tile_sum(t, w_row) * alpha;
+            if (bias) s += __half2float(bias[lrow]);
+            y2[t] = (_Float16)s, lrow2[t] = lrow, mat2[t] = mat;
+        }
+#pragma unroll
+        for (uint32_t t = 0; t < 2; ++t) {
+            // the mate: the same slot of the other tile (NeoX), or the neighbouring slot = the neighbouring lane
+            const _Float16 y_adj = (_Float16)__shfl_xor((float)y2[t], 1, 64);
+            const _Float16 ym = neox ? y2[t ^ 1u] : y_adj;
+            if (!valid2[t] || w_col >= cols) continue;
+            const uint32_t lrow = lrow2[t];
+            const int mat = mat2[t];
+            const uint32_t hd = lrow & (D - 1u), head = lrow >> (half_shift + 1);
+            const bool first = neox ? hd < half : (hd & 1u) == 0;
+            _Float16 y = y2[t];
+            if (mat != 2 && apply) y = (_Float16)rope_one((float)y, (float)ym, (float)rc[t], (float)rs[t], first);
+            _Float16 *dst;
+            if (mat == 0) {
+                dst = reinterpret_cast<_Float16 *>(out0) + ((size_t)head * m_rows + (m0 + w_col)) * D + hd;
+            } else {
+                if (r_pos >= capacity) continue;  // never outside the cache
+                const size_t crow = paged ? (((size_t)r_blk * n_kv_heads + head) * block_size + r_pos % block_size) * D
+                                          : ((size_t)head * max_seq_len + r_pos) * D;
+                dst = reinterpret_cast<_Float16 *>(mat == 1 ? out1 : out2) + crow + hd;
+            }
+            *dst = y;
+        }
+        return;
+    }
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
-        const int o = tid + pass * QKV_NT;  // (tile, weight row of the tile, input row)
-        const int t = o >> 9, row = (o >> 5) & 15, col = o & 31, h = col >> 4, cn = col & 15;
+        // (tile, input row, weight row of the tile), weight rows fastest: the lanes of a store cover consecutive outputs
+        const int t = pass, row = tid & 15, col = tid >> 4, h = col >> 4, cn = col & 15;
         const uint32_t gr = row_begin + 16u * t + (uint32_t)row;
         if (gr < row_end && (uint32_t)col < cols) {
             float s = 0.0f;
@@ -566,6 +678,47 @@ bool fa_qkv_rows32_takes(const fa_ctx *ctx, const FusedQkvLaunch &l) {
            aligned16(l.w[2]) && aligned16(l.gamma);
 }
 
+static size_t rows32_lds_bytes(uint32_t k_dim) {
+    return (size_t)k_dim * 2 + (size_t)QKV_NW * 32 * sizeof(float) + (size_t)QKV_NW * 2 * 2 * 16 * 17 * sizeof(float);
+}
+
+// FusedQkv + KvPrepFused of a chunk of 12 to 32 rows as one launch.
+fa_status fa_launch_fused_qkv_rows32_rope(fa_ctx *ctx, const FusedQkvLaunch &l, const QkvRopeLaunch &r) {
+    if (!fa_qkv_rows32_takes(ctx, l)) return fa_fail(FA_ERR_INVALID_OPERATION, "fa_launch_fused_qkv_rows32_rope: not a launch of the 32-row weight stream");
+    if (!(r.head_dim == 64 || r.head_dim == 128))
+        return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "FusedQkv with the KvPrepFused write stage supports head_dim 64 or 128, got %u", r.head_dim);
+    if (l.n_dim != r.n_heads * r.head_dim || l.n_kv != r.n_kv_heads * r.head_dim)
+        return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: n_dim %u / n_kv %u are not n_heads %u / n_kv_heads %u x head_dim %u", l.n_dim,
+                       l.n_kv, r.n_heads, r.n_kv_heads, r.head_dim);
+    if (l.residual) return fa_fail(FA_ERR_OPERATION_NOT_SUPPORTED, "the KvPrepFused write stage takes no residual");
+    if (r.table_rows == 0) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: empty RoPE tables");
+    Rows32Dev args;
+    memset(&args, 0, sizeof(args));
+    QkvDev &a = args.q;
+    for (int i = 0; i < 3; ++i) a.w[i] = l.w[i], a.bias[i] = l.bias[i];
+    a.out[0] = r.q_rot, a.out[1] = r.k_cache, a.out[2] = r.v_cache;
+    a.rows[0] = l.n_dim, a.rows[1] = l.n_kv, a.rows[2] = l.n_kv;
+    a.x = l.x, a.gamma = l.gamma, a.k_dim = l.k_dim, a.m = l.m, a.eps = l.eps, a.canonical = l.canonical ? 1u : 0u;
+    a.alpha = l.alpha, a.beta = l.beta;
+    RopeDev &d = args.r;
+    d.cos_t = r.cos_t, d.sin_t = r.sin_t, d.block_table = r.block_table;
+    d.on = 1, d.head_dim = r.head_dim, d.n_kv_heads = r.n_kv_heads, d.position_offset = r.position_offset;
+    d.max_seq_len = r.max_seq_len, d.block_size = r.block_size ? r.block_size : 1, d.capacity = r.capacity;
+    d.table_rows = r.table_rows, d.normal = r.rope_normal ? 1u : 0u, d.apply = r.apply_rope ? 1u : 0u;
+    // whole pairs per workgroup: an even number of weight rows, at most 32 (the matrices hold whole heads, so the total is even)
+    const uint32_t total_rows = l.n_dim + 2 * l.n_kv;
+    const uint32_t n_cus = ctx->n_cus > 0 ? (uint32_t)ctx->n_cus : 256u;
+    const uint32_t rpw = 2 * ceil_div_u32(total_rows / 2, n_cus);
+    if (rpw > 32) return fa_fail(FA_ERR_INVALID_OPERATION, "fa_launch_fused_qkv_rows32_rope: %u weight rows per workgroup", rpw);
+    a.rows_per_wg = rpw, a.cols_per_pass = 32, a.x_stride = 0;
+    const uint32_t xj = l.k_dim / 256;
+    const dim3 grid(ceil_div_u32(total_rows, rpw), 1);
+    FaLaunchScope scope(ctx, "fused_qkv_rows32_rope_kernel", true);
+    if (xj == 8) scope.launch(fused_qkv_rows32_kernel<8, true>, grid, dim3(QKV_NT), rows32_lds_bytes(l.k_dim), args);
+    else scope.launch(fused_qkv_rows32_kernel<12, true>, grid, dim3(QKV_NT), rows32_lds_bytes(l.k_dim), args);
+    return scope.finish();
+}
+
 fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l, bool weight_stream_only) {
     QkvDev a;
     for (int i = 0; i < 3; ++i) a.w[i] = l.w[i], a.bias[i] = l.bias[i], a.out[i] = l.out[i];
@@ -593,11 +746,13 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l, bool weight_
         const bool ok = fa_qkv_rows32_takes(ctx, l);
         if (ok) {
             a.rows_per_wg = rpw, a.cols_per_pass = 32, a.x_stride = 0;
-            const size_t lds = (size_t)l.k_dim * 2 + (size_t)QKV_NW * 32 * sizeof(float) + (size_t)QKV_NW * 2 * 2 * 16 * 17 * sizeof(float);
+            Rows32Dev args;
+            memset(&args, 0, sizeof(args));
+            args.q = a;
             const dim3 grid(ceil_div_u32(total_rows, rpw), 1);
             FaLaunchScope scope(ctx, l.n_kv ? "fused_qkv_rows32_kernel" : "matmul_rows32_kernel", true);
-            if (xj == 8) scope.launch(fused_qkv_rows32_kernel<8>, grid, dim3(QKV_NT), lds, a);
-            else scope.launch(fused_qkv_rows32_kernel<12>, grid, dim3(QKV_NT), lds, a);
+            if (xj == 8) scope.launch(fused_qkv_rows32_kernel<8, false>, grid, dim3(QKV_NT), rows32_lds_bytes(l.k_dim), args);
+            else scope.launch(fused_qkv_rows32_kernel<12, false>, grid, dim3(QKV_NT), rows32_lds_bytes(l.k_dim), args);
             return scope.finish();
         }
     }

@@ -37,6 +37,13 @@ def _paths(m):
     (16, 4, 128, 1024, 130, 3, 256, fa.ROPE_NEOX, False, True, 1, 2, 4),       # ... layer 2 is
     (8, 8, 64, 512, 5, 100, 128, fa.ROPE_NORMAL, True, True, 1, 0, 0),         # a few rows: weight stream, then KvPrepFused, inside the op
     (3, 1, 64, 256, 17, 0, 32, fa.ROPE_NEOX, True, False, 0, 0, 0),            # 192 weight rows: a tile and a half
+    # chunks of 12 to 32 rows against 2048 or 3072 features: KvPrepFused as the write stage of the one-launch weight stream
+    (16, 2, 128, 2048, 17, 40, 128, fa.ROPE_NEOX, True, True, 1, 0, 0),        # NeoX pairs (a workgroup takes both halves), biases, ragged rows
+    (14, 2, 128, 2048, 32, 5, 64, fa.ROPE_NEOX, False, False, 0, 0, 0),        # row-major weights, a last workgroup with two pairs
+    (32, 8, 64, 2048, 24, 3, 64, fa.ROPE_NEOX, True, True, 1, 0, 0),           # 64-wide heads: pairs of one workgroup across two heads
+    (32, 8, 64, 3072, 12, 50, 64, fa.ROPE_NORMAL, True, True, 1, 0, 0),        # adjacent pairs, 64-wide heads, biases
+    (16, 4, 128, 2048, 20, 3, 64, fa.ROPE_NEOX, True, False, 1, 3, 4),         # a layer that is not rotated
+    (16, 4, 128, 2048, 20, 3, 64, fa.ROPE_NEOX, True, False, 1, 2, 4),         # ... and one that is
 ])
 def test_fused_op_equals_the_two_ops(H, Hkv, D, K, m, pos, cap, mode, norm, bias, layout, layer, step):
     announce("fused qkv + kv prep", H, Hkv, D, K, m, pos, cap, mode, norm, bias, layout, layer, step)
@@ -96,6 +103,8 @@ def test_fused_op_equals_the_two_ops(H, Hkv, D, K, m, pos, cap, mode, norm, bias
     (24, 8, 128, 3072, 150, 0, 16, fa.ROPE_NORMAL),   # an empty sequence of a batch of three
     (16, 2, 128, 2048, 64, 40, 16, fa.ROPE_NEOX),     # after a prefix that ends inside a block
     (14, 2, 64, 896, 7, 9, 32, fa.ROPE_NEOX),         # a few rows (the weight-stream form)
+    (16, 2, 128, 2048, 30, 40, 16, fa.ROPE_NEOX),     # a chunk of the one-launch weight stream: rows across three blocks
+    (24, 8, 128, 3072, 32, 37, 16, fa.ROPE_NORMAL),
 ])
 def test_fused_op_into_a_paged_cache(H, Hkv, D, K, m, pos, bs, mode):
     announce("fused qkv + kv prep, paged", H, Hkv, D, K, m, pos, bs, mode)
@@ -132,6 +141,37 @@ def test_fused_op_into_a_paged_cache(H, Hkv, D, K, m, pos, bs, mode):
     for pg in pgs:
         pg.free()
     for b in dev_w + [dx, dg, dcos, dsin, dq, dk, dv] + dqr:
+        b.free()
+
+
+def test_fused_op_of_a_short_chunk_is_one_launch():
+    """A chunk of 12 to 32 rows (the reference's default prefill chunk, src/model/executor.rs:232-250) against 2048 or 3072
+    features: RMSNorm, projections, RoPE and the cache append leave ONE kernel (the profiler's launch counts)."""
+    announce("fused qkv + kv prep, launches of a short chunk")
+    f = ctx()
+    H, Hkv, D, K, m, pos, cap = 24, 8, 128, 3072, 32, 100, 256
+    rng = np.random.default_rng(11)
+    x, g, ws, _ = _data(rng, K, H * D, Hkv * D, m)
+    cos, sin = fa.rope_tables(5e5, D, cap)
+    dev_w = [f.array(orc.to_canonical(w)) for w in ws]
+    dx, dg, dcos, dsin = f.array(x), f.array(g), f.array(cos), f.array(sin)
+    dqr, dkc, dvc = f.zeros((H, m, D)), f.zeros((Hkv, cap, D)), f.zeros((Hkv, cap, D))
+    p = fa.KvPrepFusedParams.make(H, Hkv, D, m, pos, cap, fa.ROPE_NORMAL)
+    f.profile_reset()
+    f.profile_enable(True)
+    try:
+        f.fused_qkv_kv_prep(dx.arg(), dev_w[0].arg(), dev_w[1].arg(), dev_w[2].arg(), K, dqr.arg(), dcos.arg(), dsin.arg(), p,
+                            k_cache=dkc.arg(), v_cache=dvc.arg(), gamma=dg.arg())
+        f.synchronize()
+        assert f.profile_query("fused_qkv_rows32_rope_kernel")[0] == 1
+        for other in ("fused_qkv_rows32_kernel", "kv_prep_fused_elem_kernel", "kv_prep_fused_vec_kernel", "fused_qkv_gemm_kernel"):
+            assert f.profile_query(other)[0] == 0, other
+    finally:
+        f.profile_enable(False)
+    kc, vc = dkc.download(), dvc.download()
+    assert not kc[:, :pos].any() and not kc[:, pos + m:].any() and kc[:, pos:pos + m].any()  # only the chunk's rows are written
+    assert not vc[:, :pos].any() and not vc[:, pos + m:].any() and vc[:, pos:pos + m].any()
+    for b in dev_w + [dx, dg, dcos, dsin, dqr, dkc, dvc]:
         b.free()
 
 
