@@ -1554,9 +1554,11 @@ def main():
         result["configs"], result["floors"] = {}, None
         for tag, fn in (("C1_qwen05b_decode_1k", bench_small_decode), ("C3_qwen3b_paged_decode", bench_paged_decode),
                         ("C4_llama3b_prefill_2k", bench_prefill), ("C5_smollm3_sage_decode_32k", bench_sage_decode),
-                        ("llama3b_prefill_chunk32_8k", bench_prefill_chunk), ("floors", bench_floors)):
+                        ("llama3b_prefill_chunk32_8k", bench_prefill_chunk), ("llama3b_attn_block", bench_attn_block),
+                        ("llama3b_chunk_block", bench_chunk_block), ("floors", bench_floors)):
             _COLLECT = []
             g = fa.Foundry(0)
+            sub.steps, sub.warmup = (20, 3) if fn in (bench_attn_block, bench_chunk_block) else (100, 10)  # (28 layers per step)
             try:
                 fn(g, sub)
             finally:
