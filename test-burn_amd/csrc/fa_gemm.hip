@@ -23,6 +23,7 @@
 // several workgroups (split-K: f32 partial tiles in the workspace, added in split order by gemm_finish_kernel).
 #include "fa_internal.h"
 #include "fa_qkv_rope.h"
+#include <atomic>
 #include <type_traits>
 
 namespace {
@@ -911,16 +912,16 @@ static fa_status launch_gemm(fa_ctx *ctx, const FusedQkvLaunch &l, const QkvRope
         FA_TRY(norm.finish());
         a.x = (const __half *)ctx->workspace;
     }
-    static bool lds_allowed_on[64] = {};  // per device
-    bool &lds_allowed = lds_allowed_on[ctx->device & 63];
-    if (!lds_allowed) {
+    static std::atomic<bool> lds_allowed_on[64];  // per device (contexts of several threads may get here together: the calls are idempotent)
+    std::atomic<bool> &lds_allowed = lds_allowed_on[ctx->device & 63];
+    if (!lds_allowed.load(std::memory_order_acquire)) {
         FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
         FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true, 16>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
         FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
         FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
         FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<false, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
         FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_kernel<true, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
-        lds_allowed = true;
+        lds_allowed.store(true, std::memory_order_release);
     }
     FaLaunchScope scope(ctx, l.n_kv ? "fused_qkv_gemm_kernel" : "matmul_gemm_kernel", true);
     const uint32_t grid = (uint32_t)n_wg * a.k_splits;
@@ -936,12 +937,12 @@ static fa_status launch_gemm(fa_ctx *ctx, const FusedQkvLaunch &l, const QkvRope
         if (l.canonical) scope.launch(qkv_gemm_dma32_kernel<true>, dim3(grid), dim3(GM_NT), GR_LDS_BYTES, a);
         else scope.launch(qkv_gemm_dma32_kernel<false>, dim3(grid), dim3(GM_NT), GR_LDS_BYTES, a);
     } else if (dma_ok && ctx->gemm_variant != 1) {
-        static bool dma_lds_allowed_on[64] = {};  // per device
-        bool &dma_lds_allowed = dma_lds_allowed_on[ctx->device & 63];
-        if (!dma_lds_allowed) {
+        static std::atomic<bool> dma_lds_allowed_on[64];  // per device (contexts of several threads may get here together: the calls are idempotent)
+        std::atomic<bool> &dma_lds_allowed = dma_lds_allowed_on[ctx->device & 63];
+        if (!dma_lds_allowed.load(std::memory_order_acquire)) {
             FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_dma_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
             FA_HIP(hipFuncSetAttribute((const void *)qkv_gemm_dma_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));
-            dma_lds_allowed = true;
+            dma_lds_allowed.store(true, std::memory_order_release);
         }
         if (l.canonical) scope.launch(qkv_gemm_dma_kernel<true>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);
         else scope.launch(qkv_gemm_dma_kernel<false>, dim3(grid), dim3(GM_NT), GM_LDS_BYTES, a);

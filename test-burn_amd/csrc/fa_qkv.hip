@@ -24,6 +24,7 @@
 // consumer of the attention output.
 #include "fa_internal.h"
 #include "fa_qkv_rope.h"
+#include <atomic>
 #include <type_traits>
 
 namespace {
@@ -776,16 +777,16 @@ fa_status fa_launch_fused_qkv(fa_ctx *ctx, const FusedQkvLaunch &l, bool weight_
     const uint32_t tiles_per_wg = ceil_div_u32(rows_per_wg, 16);
     const size_t lds = (size_t)cols * a.x_stride + (size_t)QKV_NW * 16 * 17 * sizeof(float) +
                        (q8 ? (size_t)tiles_per_wg * 16 * (l.k_dim / 32) * 2 : 0);
-    static bool lds_allowed_on[64] = {};  // per device
-    bool &lds_allowed = lds_allowed_on[ctx->device & 63];
-    if (!lds_allowed) {
+    static std::atomic<bool> lds_allowed_on[64];  // per device (contexts of several threads may get here together: the calls are idempotent)
+    std::atomic<bool> &lds_allowed = lds_allowed_on[ctx->device & 63];
+    if (!lds_allowed.load(std::memory_order_acquire)) {
         FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)(lds_budget + 16 * 1024)));
         FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)(lds_budget + 16 * 1024)));
         FA_HIP(hipFuncSetAttribute((const void *)fused_qkv_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                    (int)(lds_budget + 16 * 1024)));
-        lds_allowed = true;
+        lds_allowed.store(true, std::memory_order_release);
     }
     const dim3 grid(ceil_div_u32(total_rows, rows_per_wg), ceil_div_u32(l.m, cols));
     if (grid.y > 65535u) return fa_fail(FA_ERR_INVALID_SHAPE, "Invalid shape: FusedQkv m %u needs %u passes", l.m, grid.y);
