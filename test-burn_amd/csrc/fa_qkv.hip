@@ -516,13 +516,30 @@ __global__ void __launch_bounds__(QKV_NT, 1) fused_qkv_rows32_kernel(Rows32Dev a
             for (int w = 0; w < QKV_NW; ++w) tot += ss_lds[w * 32 + 16 * h + n];
             inv_rms[h] = rsqrtf(tot / (float)K + eps);
         }
+        // (x * inv_rms) * gamma, each product rounded to f32, the result to f16: two instructions per element that take the
+        // f16 halves as they lie in the registers (the plain form converts both factors and the result separately, five per
+        // element, and with all 32 rows to scale in every workgroup that was a quarter of the launch)
+        typedef uint32_t u4v_t __attribute__((ext_vector_type(4)));
+        const float neg_zero = -0.0f;  // (a sum with -0 keeps the sign of a zero product)
 #pragma unroll
         for (int j = 0; j < XJ; ++j) {
-            const h8_t g = *reinterpret_cast<const h8_t *>(g_lds + kb_of(j) * 32u + c * 8);
+            const u4v_t g2 = *reinterpret_cast<const u4v_t *>(g_lds + kb_of(j) * 32u + c * 8);
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
+            for (int h = 0; h < 2; ++h) {
+                const u4v_t x2 = __builtin_bit_cast(u4v_t, xs[j][h]);
+                u4v_t y2;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) xs[j][h][i] = (_Float16)(((float)xs[j][h][i] * inv_rms[h]) * (float)g[i]);
+                for (int e = 0; e < 4; ++e) {
+                    float t0, t1;
+                    uint32_t y;
+                    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(t0) : "v"(x2[e]), "v"(inv_rms[h]), "v"(neg_zero));
+                    asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(t1) : "v"(x2[e]), "v"(inv_rms[h]), "v"(neg_zero));
+                    asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[0,1,0]" : "=v"(y) : "v"(t0), "v"(g2[e]), "v"(neg_zero));
+                    asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[0,1,0] op_sel_hi:[0,1,0]" : "+v"(y) : "v"(t1), "v"(g2[e]), "v"(neg_zero));
+                    y2[e] = y;
+                }
+                xs[j][h] = __builtin_bit_cast(h8_t, y2);
+            }
         }
     }
 #pragma unroll
